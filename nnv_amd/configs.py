@@ -1,0 +1,122 @@
+"""Synthetic benchmark configurations for the relax-star reach path.
+
+Five seeded network + input-set definitions.  All draws come from
+``numpy.random.RandomState(1000 + k)`` (the frozen legacy MT19937 stream), in this order:
+the input point ``x`` first (uniform), then for every affine layer in network order its
+weight tensor (standard normal, filled in MATLAB column-major order, scaled by
+sqrt(2 / fan_in)) followed by its bias (standard normal scaled by 0.1, i.e. variance 0.01).
+
+Layer dictionaries use NNV's own array layouts:
+  fc:   W is Out x In, b is Out                       (FullyConnectedLayer.Weights / .Bias)
+  conv: W is FH x FW x Cin x Cout, b is Cout,
+        padding [t b l r], stride [sh sw], dilation [dh dw]   (Conv2DLayer properties,
+        code/nnv/engine/nn/layers/Conv2DLayer.m:15-33)
+  relu: no parameters
+"""
+from __future__ import annotations
+
+import numpy as np
+
+BIAS_SIGMA = 0.1
+
+
+def _fc(rs, n_out, n_in):
+    W = rs.randn(n_out * n_in).reshape((n_out, n_in), order="F") * np.sqrt(2.0 / n_in)
+    b = rs.randn(n_out) * BIAS_SIGMA
+    return {"type": "fc", "W": W, "b": b}
+
+
+def _conv(rs, fh, fw, cin, cout, stride, pad):
+    fan_in = fh * fw * cin
+    W = rs.randn(fh * fw * cin * cout).reshape((fh, fw, cin, cout), order="F") * np.sqrt(2.0 / fan_in)
+    b = rs.randn(cout) * BIAS_SIGMA
+    return {"type": "conv", "W": W, "b": b, "padding": [pad, pad, pad, pad],
+            "stride": [stride, stride], "dilation": [1, 1]}
+
+
+def _relu():
+    return {"type": "relu"}
+
+
+def conv_out_hw(h, w, layer):
+    """Feature-map size, code/nnv/engine/nn/layers/Conv2DLayer.m:1134-1135."""
+    fh, fw = layer["W"].shape[:2]
+    t, b, l, r = layer["padding"]
+    sh, sw = layer["stride"]
+    dh, dw = layer["dilation"]
+    ho = (h + t + b - (fh - 1) * dh - 1) // sh + 1
+    wo = (w + l + r - (fw - 1) * dw - 1) // sw + 1
+    return ho, wo
+
+
+def fc_net(rs, widths):
+    layers = []
+    for i in range(len(widths) - 1):
+        layers.append(_fc(rs, widths[i + 1], widths[i]))
+        if i < len(widths) - 2:
+            layers.append(_relu())
+    return layers
+
+
+def make_config(k: int, shrink: int = 1):
+    """Return a dict {name, layers, kind, lb, ub[, image_shape][, partition]} for config k (1..5).
+
+    ``shrink`` > 1 divides hidden widths / channel counts (and for k = 5 the number of
+    bisected dimensions) so the CPU checker finishes in seconds; shrink = 1 is the full size.
+    """
+    rs = np.random.RandomState(1000 + k)
+    if k == 1:
+        c = rs.rand(5) - 0.5
+        layers = fc_net(rs, [5] + [max(50 // shrink, 4)] * 6 + [5])
+        return {"name": "cfg1_fc_5x50x6x5", "kind": "star", "layers": layers,
+                "lb": c - 0.02, "ub": c + 0.02}
+    if k in (2, 5):
+        # config 5 reuses config 2's network and box (seed 1002)
+        rs = np.random.RandomState(1002)
+        n_in = 784 if shrink == 1 else max(784 // shrink, 16)
+        hid = max(1024 // shrink, 8)
+        x = rs.rand(n_in)
+        layers = fc_net(rs, [n_in, hid, hid, hid, 10])
+        cfg = {"name": "cfg2_fc_784_1024x3_10", "kind": "star", "layers": layers,
+               "lb": x - 0.02, "ub": x + 0.02}
+        if k == 5:
+            ndim = 10 if shrink == 1 else max(2, 10 // shrink)
+            cfg["name"] = "cfg5_bab_%d_boxes" % (2 ** ndim)
+            # all widths are equal, so the "widest" dimensions are the first ones (stable order);
+            # Box.partition order: first listed index varies slowest
+            cfg["partition"] = {"indexes": list(range(ndim)), "numbers": [2] * ndim}
+        return cfg
+    if k == 3:
+        hw = 28 if shrink == 1 else max(28 // shrink, 6)
+        c1, c2, f = max(16 // shrink, 2), max(32 // shrink, 2), max(100 // shrink, 4)
+        x = rs.rand(hw * hw)
+        conv1 = _conv(rs, 3, 3, 1, c1, 1, 1)
+        conv2 = _conv(rs, 3, 3, c1, c2, 2, 1)
+        h1, w1 = conv_out_hw(hw, hw, conv1)
+        h2, w2 = conv_out_hw(h1, w1, conv2)
+        layers = [conv1, _relu(), conv2, _relu(), _fc(rs, f, h2 * w2 * c2), _relu(), _fc(rs, 10, f)]
+        eps = 1.0 / 255.0
+        return {"name": "cfg3_cnn_28x28x1", "kind": "image", "image_shape": (hw, hw, 1),
+                "layers": layers, "lb": x - eps, "ub": x + eps}
+    if k == 4:
+        hw = 32 if shrink == 1 else max(32 // shrink, 10)
+        ca, cb, f = max(32 // shrink, 2), max(64 // shrink, 2), max(512 // shrink, 4)
+        x = rs.rand(hw * hw * 3)
+        conv1 = _conv(rs, 3, 3, 3, ca, 1, 1)
+        conv2 = _conv(rs, 3, 3, ca, ca, 2, 0)
+        conv3 = _conv(rs, 3, 3, ca, cb, 1, 1)
+        conv4 = _conv(rs, 3, 3, cb, cb, 2, 0)
+        h, w = hw, hw
+        for L in (conv1, conv2, conv3, conv4):
+            h, w = conv_out_hw(h, w, L)
+        layers = [conv1, _relu(), conv2, _relu(), conv3, _relu(), conv4, _relu(),
+                  _fc(rs, f, h * w * cb), _relu(), _fc(rs, 10, f)]
+        eps = 2.0 / 255.0
+        return {"name": "cfg4_cnn_32x32x3", "kind": "image", "image_shape": (hw, hw, 3),
+                "layers": layers, "lb": x - eps, "ub": x + eps}
+    raise ValueError("config index must be 1..5")
+
+
+def count_updates(layer_shapes):
+    """Generator-neuron updates of one reach: sum over layer steps of N_out * (n_out + 1)."""
+    return int(sum(int(N) * (int(n) + 1) for (N, n) in layer_shapes))

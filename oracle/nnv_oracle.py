@@ -1,0 +1,571 @@
+"""CPU restatement of NNV's relax-star reachability path (TEST INFRASTRUCTURE ONLY).
+
+This module is the *checker* for the HIP implementation.  It restates, statement by
+statement and in fp64 numpy, what the MATLAB reference does on the path
+
+    NN.reach -> {FullyConnectedLayer, Conv2DLayer, ReluLayer}.reach
+             -> Star.affineMap / dlconv / PosLin.reach_relaxed_star_* (relaxFactor = 1)
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import it.  The
+product (nnv_amd) never imports it and has no CPU fallback.
+
+Conventions
+-----------
+* Matrices are numpy arrays; ``V`` is ``N x (n+1)`` with column 0 the centre, exactly as
+  the reference's ``Star.V``.  Image tensors are ``H x W x C x (n+1)`` like ``ImageStar.V``
+  and are flattened in MATLAB (column-major, ``order='F'``) order.
+* Index vectors are 0-based here (the reference's are 1-based doubles).
+* Every function cites the reference file:line (relative to code/nnv/engine/) it follows.
+
+Parity pinning (what checks each function; see tests/test_oracle_*.py)
+----------------------------------------------------------------------
+* box_generators / star_from_box / affine_map / estimate_ranges: the reference's own
+  golden file results/tests/baselines/set/test_star_affineMap_results.mat (S1_V, S4_lb,
+  S4_ub), star_test_results.mat, the ImageStar getRange known answer ([-2, 2]) and the
+  interval-arithmetic closed form.
+* conv2d_feature_map / conv2d_reach: the reference's known-answer test
+  tests/nn/layers/Conv2DLayer/test_layers_Conv2D.m:14-28, and torch's fp64 conv2d as an
+  independent library routine.  Bit-level parity with MathWorks' closed ``dlconv``:
+  PARITY UNPINNED (summation order unknowable here; values agree to rounding).
+* box_partition: closed form (Cartesian grid, first listed index slowest).
+* reach_relaxed_star / multiple_step_reach_star_approx_at_one: no reference test runs a
+  relax-star method, so PARITY UNPINNED by golden vectors; pinned by the source text plus
+  hand-computed scalar triangle, brute-force corner enumeration, the containment
+  (soundness) invariant the reference's own soundness tests use, structural invariants
+  and permutation-equivalence of the six variants.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+RELAX_METHODS = (
+    "relax-star-range",
+    "relax-star-area",
+    "relax-star-bound",
+    "relax-star-ub",
+    "relax-star-random",
+    "relax-star-static",
+)
+
+
+# --------------------------------------------------------------------------------------
+# sets
+# --------------------------------------------------------------------------------------
+class OStar:
+    """Field-for-field mirror of the reference's Star value class (set/Star.m:13-24)."""
+
+    def __init__(self, V, C, d, predicate_lb=None, predicate_ub=None,
+                 state_lb=None, state_ub=None, Z=None):
+        # set/Star.m:153-189 (5-argument constructor and its size checks)
+        V = np.asarray(V, dtype=np.float64)
+        C = np.asarray(C, dtype=np.float64)
+        d = np.asarray(d, dtype=np.float64).reshape(-1)
+        if C.ndim != 2:
+            C = C.reshape(-1, V.shape[1] - 1)
+        if V.shape[1] != C.shape[1] + 1:
+            raise ValueError("Inconsistency between basic matrix and constraint matrix")
+        if C.shape[0] != d.shape[0]:
+            raise ValueError("Inconsistency between constraint matrix and constraint vector")
+        if predicate_lb is not None and predicate_ub is not None:
+            predicate_lb = np.asarray(predicate_lb, dtype=np.float64).reshape(-1)
+            predicate_ub = np.asarray(predicate_ub, dtype=np.float64).reshape(-1)
+            if predicate_lb.size and predicate_ub.size and (
+                    predicate_lb.size != predicate_ub.size or predicate_lb.size != C.shape[1]):
+                raise ValueError("Inconsistency between number of predicate variables and "
+                                 "predicate lower- or upper-bounds vector")
+        self.V = V
+        self.C = C
+        self.d = d
+        self.dim = V.shape[0]
+        self.nVar = C.shape[1]
+        self.predicate_lb = predicate_lb
+        self.predicate_ub = predicate_ub
+        self.state_lb = state_lb
+        self.state_ub = state_ub
+        self.Z = Z  # (c, V) of the outer zonotope or None
+
+
+class OImageStar:
+    """Mirror of the reference's ImageStar (set/ImageStar.m:47-94): V is H x W x C x (n+1)."""
+
+    def __init__(self, V, C, d, pred_lb, pred_ub, im_lb=None, im_ub=None):
+        # set/ImageStar.m:172-227 (5-argument constructor)
+        V = np.asarray(V, dtype=np.float64)
+        C = np.asarray(C, dtype=np.float64)
+        d = np.asarray(d, dtype=np.float64).reshape(-1)
+        if C.shape[0] != d.shape[0]:
+            raise ValueError("Inconsistent dimension between constraint matrix and constraint vector")
+        pred_lb = np.asarray(pred_lb, dtype=np.float64).reshape(-1)
+        pred_ub = np.asarray(pred_ub, dtype=np.float64).reshape(-1)
+        if C.shape[1] != pred_lb.size or C.shape[1] != pred_ub.size:
+            raise ValueError("Number of predicates is different from the size of the lower "
+                             "bound or upper bound predicate vector")
+        if V.ndim != 4 or V.shape[3] != C.shape[1] + 1:
+            raise ValueError("Inconsistency between the basis matrix and the number of predicate variables")
+        self.V = V
+        self.C = C
+        self.d = d
+        self.numPred = C.shape[1]
+        self.pred_lb = pred_lb
+        self.pred_ub = pred_ub
+        self.height, self.width, self.numChannel = V.shape[:3]
+        self.im_lb = im_lb
+        self.im_ub = im_ub
+
+    def to_star(self) -> OStar:
+        # set/ImageStar.m:569-592: column j of the Star is reshape(V(:,:,:,j), N, 1)
+        N = self.height * self.width * self.numChannel
+        V1 = self.V.reshape(N, self.numPred + 1, order="F")
+        if self.im_lb is not None and self.im_ub is not None:
+            return OStar(V1, self.C, self.d, self.pred_lb, self.pred_ub,
+                         np.asarray(self.im_lb).reshape(N, order="F"),
+                         np.asarray(self.im_ub).reshape(N, order="F"))
+        return OStar(V1, self.C, self.d, self.pred_lb, self.pred_ub)
+
+
+def box_generators(lb, ub):
+    """Box constructor arithmetic, set/Box.m:16-58.
+
+    center = 0.5*(lb+ub); vec = 0.5*(ub-lb); generators = diag(vec) with all-zero columns
+    removed (only when numel(gens) > 1, Box.m:41-43).
+    """
+    lb = np.asarray(lb, dtype=np.float64).reshape(-1)
+    ub = np.asarray(ub, dtype=np.float64).reshape(-1)
+    if lb.size != ub.size:
+        raise ValueError("Inconsistent dimensions between lb and ub")
+    center = 0.5 * (lb + ub)
+    vec = 0.5 * (ub - lb)
+    gens = np.diag(vec)
+    if gens.size > 1:
+        gens = gens[:, ~np.all(gens == 0, axis=0)]
+    return center, gens
+
+
+def box_single_partition(lb, ub, part_id, part_num):
+    """set/Box.m:61-91 (part_id is 0-based here)."""
+    if part_num == 1:
+        return [(lb.copy(), ub.copy())]
+    delta = (ub[part_id] - lb[part_id]) / part_num
+    out = []
+    for i in range(1, part_num + 1):
+        new_lb = lb.copy()
+        new_ub = ub.copy()
+        new_lb[part_id] = lb[part_id] + (i - 1) * delta
+        new_ub[part_id] = new_lb[part_id] + delta
+        out.append((new_lb, new_ub))
+    return out
+
+
+def box_partition(lb, ub, part_indexes, part_numbers):
+    """set/Box.m:96-139: successive single partitions; first listed index varies slowest."""
+    lb = np.asarray(lb, dtype=np.float64).reshape(-1)
+    ub = np.asarray(ub, dtype=np.float64).reshape(-1)
+    boxes = [(lb, ub)]
+    for idx, num in zip(part_indexes, part_numbers):
+        nxt = []
+        for (l, u) in boxes:
+            nxt.extend(box_single_partition(l, u, idx, num))
+        boxes = nxt
+    return boxes
+
+
+def star_from_box(lb, ub) -> OStar:
+    """Star(lb, ub), set/Star.m:220-237 (+ Box.toStar -> Zono.toStar, set/Zono.m:301-309).
+
+    V = [center gens]; C = zeros(1, n); d = 0; predicate bounds -1/+1; state bounds = lb/ub;
+    Z = Zono(center, gens).
+    """
+    lb = np.asarray(lb, dtype=np.float64).reshape(-1)
+    ub = np.asarray(ub, dtype=np.float64).reshape(-1)
+    center, gens = box_generators(lb, ub)
+    n = gens.shape[1]
+    V = np.concatenate([center[:, None], gens], axis=1)
+    return OStar(V, np.zeros((1, n)), np.zeros(1), -np.ones(n), np.ones(n),
+                 lb.copy(), ub.copy(), Z=(center.copy(), gens.copy()))
+
+
+def image_star_from_bounds(lb_im, ub_im) -> OImageStar:
+    """ImageStar(lb_im, ub_im), set/ImageStar.m:302-343: Star(lb,ub).toImageStar(h,w,c)."""
+    lb_im = np.asarray(lb_im, dtype=np.float64)
+    ub_im = np.asarray(ub_im, dtype=np.float64)
+    if lb_im.shape != ub_im.shape:
+        raise ValueError("Inconsistency between lower bound image and upper bound image")
+    if lb_im.ndim == 2:
+        lb_im = lb_im[:, :, None]
+        ub_im = ub_im[:, :, None]
+    h, w, c = lb_im.shape
+    S = star_from_box(lb_im.reshape(-1, order="F"), ub_im.reshape(-1, order="F"))
+    IS = star_to_image_star(S, h, w, c)
+    IS.im_lb = lb_im
+    IS.im_ub = ub_im
+    return IS
+
+
+def star_to_image_star(S: OStar, height, width, num_channel) -> OImageStar:
+    """Star.toImageStar, set/Star.m:1398-1418: plain column-major reshape of V."""
+    if S.dim != height * width * num_channel:
+        raise ValueError("Inconsistent dimension in the ImageStar and the original Star set")
+    V = S.V.reshape(height, width, num_channel, S.nVar + 1, order="F")
+    if S.state_lb is not None and S.state_ub is not None:
+        return OImageStar(V, S.C, S.d, S.predicate_lb, S.predicate_ub,
+                          np.asarray(S.state_lb).reshape(height, width, num_channel, order="F"),
+                          np.asarray(S.state_ub).reshape(height, width, num_channel, order="F"))
+    return OImageStar(V, S.C, S.d, S.predicate_lb, S.predicate_ub)
+
+
+# --------------------------------------------------------------------------------------
+# affine maps
+# --------------------------------------------------------------------------------------
+def affine_map(S: OStar, W, b=None) -> OStar:
+    """Star.affineMap, set/Star.m:313-343.
+
+    newV = W*V; newV(:,1) = newV(:,1) + b; C, d, predicate bounds pass through; the outer
+    zonotope is mapped as well (set/Zono.m:47-74).  State bounds are dropped (6-arg ctor).
+    """
+    W = np.asarray(W, dtype=np.float64)
+    if W.shape[1] != S.dim:
+        raise ValueError("Inconsistency between the affine mapping matrix and dimension of the star set")
+    newV = W @ S.V
+    if b is not None and np.size(b):
+        b = np.asarray(b, dtype=np.float64)
+        if b.ndim == 2 and b.shape[1] != 1:
+            raise ValueError("Mapping vector should have one column")
+        b = b.reshape(-1)
+        if b.shape[0] != W.shape[0]:
+            raise ValueError("Inconsistency between the mapping vec and mapping matrix")
+        newV[:, 0] = newV[:, 0] + b
+    newZ = None
+    if S.Z is not None:
+        zc, zV = S.Z
+        nc = W @ zc
+        if b is not None and np.size(b):
+            nc = nc + b
+        newZ = (nc, W @ zV)
+    return OStar(newV, S.C, S.d, S.predicate_lb, S.predicate_ub, Z=newZ)
+
+
+def fc_reach(I, W, b):
+    """FullyConnectedLayer.reach_star_single_input, nn/layers/FullyConnectedLayer.m:295-316, 467-481.
+
+    ImageStar: V(1,1,:,:) = W*reshape(V, N, n+1); V(1,1,:,1) += Bias -> ImageStar 1x1xOutx(n+1).
+    Star: affineMap(W, b).
+    """
+    W = np.asarray(W, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64).reshape(-1)
+    if isinstance(I, OImageStar):
+        N = I.height * I.width * I.numChannel
+        if N != W.shape[1]:
+            raise ValueError("Inconsistency between the size of the input image and the InputSize of the network")
+        n = I.numPred
+        newV = W @ I.V.reshape(N, n + 1, order="F")
+        newV[:, 0] = newV[:, 0] + b
+        return OImageStar(newV.reshape(1, 1, W.shape[0], n + 1, order="F"),
+                          I.C, I.d, I.pred_lb, I.pred_ub)
+    if isinstance(I, OStar):
+        return affine_map(I, W, b)
+    raise TypeError("Input set is not an ImageStar or Star")
+
+
+def conv2d_output_size(H, W, FH, FW, padding, stride, dilation):
+    """Feature-map size, nn/layers/Conv2DLayer.m:1134-1135 (padding = [t b l r])."""
+    t, b, l, r = padding
+    ho = int(np.floor((H + t + b - (FH - 1) * dilation[0] - 1) / stride[0] + 1))
+    wo = int(np.floor((W + l + r - (FW - 1) * dilation[1] - 1) / stride[1] + 1))
+    return ho, wo
+
+
+def conv2d_feature_map(inp, Wf, padding, stride, dilation):
+    """Conv2DLayer.compute_featureMap, nn/layers/Conv2DLayer.m:1111-1204 (single channel, 2-D).
+
+    Zero padding [t b l r] (get_zero_padding_input, :1064-1108), then for every output cell
+    val = sum_{i,j} I(i0 + (i-1)*dil, j0 + (j-1)*dil) * W(i,j): cross-correlation, no flip.
+    Pure-python loops: used for small known-answer checks only.
+    """
+    inp = np.asarray(inp, dtype=np.float64)
+    Wf = np.asarray(Wf, dtype=np.float64)
+    t, b, l, r = padding
+    h, w = inp.shape
+    I = np.zeros((t + h + b, l + w + r))
+    I[t:t + h, l:l + w] = inp
+    ho, wo = conv2d_output_size(h, w, Wf.shape[0], Wf.shape[1], padding, stride, dilation)
+    out = np.zeros((ho, wo))
+    for i in range(ho):
+        for j in range(wo):
+            val = 0.0
+            for fi in range(Wf.shape[0]):
+                for fj in range(Wf.shape[1]):
+                    ie = i * stride[0] + fi * dilation[0]
+                    je = j * stride[1] + fj * dilation[1]
+                    if ie < I.shape[0] and je < I.shape[1]:
+                        val = val + I[ie, je] * Wf[fi, fj]
+            out[i, j] = val
+    return out
+
+
+def conv2d_tensor(X, Wt, bias, padding, stride, dilation):
+    """dlconv semantics used at nn/layers/Conv2DLayer.m:591-592 on an H x W x Cin x B tensor.
+
+    Wt is FH x FW x Cin x Cout, cross-correlation (same definition as compute_featureMap
+    summed over input channels), zero padding [t b l r].  bias (Cout,) or None is added after
+    the sum.  Taps are accumulated in (fh fastest, fw, then the channel contraction) order.
+    """
+    X = np.asarray(X, dtype=np.float64)
+    Wt = np.asarray(Wt, dtype=np.float64)
+    H, W_, Cin, B = X.shape
+    FH, FW, Cin2, Cout = Wt.shape
+    if Cin != Cin2:
+        raise ValueError("Input set contains %d channels while the convolutional layers has %d channels"
+                         % (Cin, Cin2))
+    t, b, l, r = padding
+    ho, wo = conv2d_output_size(H, W_, FH, FW, padding, stride, dilation)
+    Xp = np.zeros((t + H + b, l + W_ + r, Cin, B))
+    Xp[t:t + H, l:l + W_] = X
+    out = np.zeros((ho, wo, Cout, B))
+    for fw in range(FW):
+        for fh in range(FH):
+            h0 = fh * dilation[0]
+            w0 = fw * dilation[1]
+            patch = Xp[h0:h0 + (ho - 1) * stride[0] + 1:stride[0],
+                       w0:w0 + (wo - 1) * stride[1] + 1:stride[1]]  # ho x wo x Cin x B
+            # contract the channel axis: (ho,wo,Cin,B) x (Cin,Cout) -> (ho,wo,Cout,B)
+            out += np.einsum("hwcb,co->hwob", patch, Wt[fh, fw], optimize=True)
+    if bias is not None:
+        out += np.asarray(bias, dtype=np.float64).reshape(1, 1, Cout, 1)
+    return out
+
+
+def conv2d_reach(I: OImageStar, Wt, bias, padding=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1)) -> OImageStar:
+    """Conv2DLayer.reach_star_single_input, nn/layers/Conv2DLayer.m:559-601, 780.
+
+    c = dlconv(V(:,:,:,1), W, Bias); G = dlconv(V(:,:,:,2:end), W, 0); V' = cat(4, c, G);
+    C, d, predicate bounds pass through; the result is a 5-argument ImageStar (no im_lb/ub).
+    """
+    if not isinstance(I, OImageStar):
+        raise TypeError("The input is not an ImageStar object")
+    Wt = np.asarray(Wt, dtype=np.float64)
+    if I.numChannel != Wt.shape[2]:
+        raise ValueError("Input set contains %d channels while the convolutional layers has %d channels"
+                         % (I.numChannel, Wt.shape[2]))
+    bias = np.zeros(Wt.shape[3]) if bias is None else np.asarray(bias, dtype=np.float64).reshape(-1)
+    c = conv2d_tensor(I.V[:, :, :, :1], Wt, bias, padding, stride, dilation)
+    G = conv2d_tensor(I.V[:, :, :, 1:], Wt, None, padding, stride, dilation)
+    return OImageStar(np.concatenate([c, G], axis=3), I.C, I.d, I.pred_lb, I.pred_ub)
+
+
+# --------------------------------------------------------------------------------------
+# ranges and the relaxed ReLU
+# --------------------------------------------------------------------------------------
+def estimate_ranges(S: OStar):
+    """Star.estimateRanges, set/Star.m:1078-1106.
+
+    pos = max(V,0); neg = min(V,0) (whole matrix, centre column included); the four products
+    use [0; predicate bounds] so the centre column cancels;
+    lb = V(:,1) + xmin1 + xmin2, ub = V(:,1) + xmax1 + xmax2 (left to right).
+    Empty predicate bounds default to -1/+1 (:1091-1096).
+    """
+    pos_mat = S.V.copy()
+    neg_mat = S.V.copy()
+    pos_mat[pos_mat < 0] = 0
+    neg_mat[neg_mat > 0] = 0
+    plb = S.predicate_lb
+    pub = S.predicate_ub
+    if plb is None or np.size(plb) == 0:
+        plb = -np.ones(S.nVar)
+    if pub is None or np.size(pub) == 0:
+        pub = np.ones(S.nVar)
+    lbv = np.concatenate([[0.0], plb])
+    ubv = np.concatenate([[0.0], pub])
+    xmin1 = pos_mat @ lbv
+    xmax1 = pos_mat @ ubv
+    xmin2 = neg_mat @ ubv
+    xmax2 = neg_mat @ lbv
+    lb = S.V[:, 0] + xmin1 + xmin2
+    ub = S.V[:, 0] + xmax1 + xmax2
+    return lb, ub
+
+
+def image_star_estimate_ranges(I: OImageStar):
+    """ImageStar.estimateRanges, set/ImageStar.m:836-885 (same formula on the tensor form)."""
+    if I.im_lb is not None and I.im_ub is not None:
+        return I.im_lb, I.im_ub
+    gens = I.V[:, :, :, 1:]
+    pos = np.where(gens < 0, 0.0, gens)
+    neg = np.where(gens > 0, 0.0, gens)
+    lb = I.V[:, :, :, 0] + np.tensordot(pos, I.pred_lb, axes=(3, 0)) + np.tensordot(neg, I.pred_ub, axes=(3, 0))
+    ub = I.V[:, :, :, 0] + np.tensordot(pos, I.pred_ub, axes=(3, 0)) + np.tensordot(neg, I.pred_lb, axes=(3, 0))
+    return lb, ub
+
+
+def reset_row(S: OStar, rows) -> OStar:
+    """Star.resetRow, set/Star.m:1442-1461: V(map,:) = 0 (and the same on Z)."""
+    V1 = S.V.copy()
+    V1[rows, :] = 0
+    newZ = None
+    if S.Z is not None:
+        c2 = S.Z[0].copy()
+        c2[rows] = 0
+        V2 = S.Z[1].copy()
+        V2[rows, :] = 0
+        newZ = (c2, V2)
+    return OStar(V1, S.C, S.d, S.predicate_lb, S.predicate_ub, Z=newZ)
+
+
+def multiple_step_reach_star_approx_at_one(I: OStar, index, lb, ub) -> OStar:
+    """PosLin.multipleStepReachStarApprox_at_one, nn/funcs/PosLin.m:685-742.
+
+    index: crossing neurons (0-based) in the order the new predicate columns get; lb/ub their
+    bounds.  Returns Star(new_V, new_C, new_d, new_pred_lb, new_pred_ub): no Z, no state bounds.
+    """
+    index = np.asarray(index, dtype=np.int64).reshape(-1)
+    lb = np.asarray(lb, dtype=np.float64).reshape(-1)
+    ub = np.asarray(ub, dtype=np.float64).reshape(-1)
+    N = I.dim
+    m = index.size
+    V1 = I.V.copy()
+    V1[index, :] = 0
+    V2 = np.zeros((N, m))
+    for i in range(m):
+        V2[index[i], i] = 1
+    new_V = np.concatenate([V1, V2], axis=1)
+
+    n = I.nVar
+    C0 = np.concatenate([I.C, np.zeros((I.C.shape[0], m))], axis=1)
+    d0 = I.d
+    C1 = np.concatenate([np.zeros((m, n)), -np.eye(m)], axis=1)
+    d1 = np.zeros(m)
+    C2 = np.concatenate([I.V[index, 1:n + 1], -V2[index, :m]], axis=1)
+    d2 = -I.V[index, 0]
+    a = ub / (ub - lb)
+    b = a * lb
+    C3 = np.concatenate([(-a)[:, None] * I.V[index, 1:n + 1], V2[index, :m]], axis=1)
+    d3 = a * I.V[index, 0] - b
+    new_C = np.concatenate([C0, C1, C2, C3], axis=0)
+    new_d = np.concatenate([d0, d1, d2, d3])
+    new_pred_lb = np.concatenate([I.predicate_lb, np.zeros(m)])
+    new_pred_ub = np.concatenate([I.predicate_ub, ub])
+    return OStar(new_V, new_C, new_d, new_pred_lb, new_pred_ub)
+
+
+def relax_classify(lb, ub, method):
+    """Classification and crossing order shared by the six variants at relaxFactor = 1.
+
+    map1 = find(ub <= 0); map2 = find(lb < 0 & ub > 0) (ascending);
+    range: sort(ub-lb,'descend') (nn/funcs/PosLin.m:934-936);
+    area:  sort(0.5*(abs(ub).*abs(lb)),'descend') (:1049-1052);
+    bound/ub/random/static keep ascending order (:1167-1174,1232; :1326-1329,1397;
+    :1488-1492; :1604-1605).  MATLAB's sort is stable.
+    """
+    map1 = np.flatnonzero(ub <= 0)
+    map2 = np.flatnonzero((lb < 0) & (ub > 0))
+    if method == "relax-star-range":
+        key = ub[map2] - lb[map2]
+        order = np.argsort(-key, kind="stable")
+        map2 = map2[order]
+    elif method == "relax-star-area":
+        key = 0.5 * (np.abs(ub[map2]) * np.abs(lb[map2]))
+        order = np.argsort(-key, kind="stable")
+        map2 = map2[order]
+    elif method not in RELAX_METHODS:
+        raise ValueError("This reachability method does not exist")
+    return map1, map2
+
+
+def reach_relaxed_star(I: OStar, method: str, relax_factor: float = 1.0) -> OStar:
+    """PosLin.reach_relaxed_star_{range,area,bound,ub,random,static} at relaxFactor = 1
+    (nn/funcs/PosLin.m:863-1650).  n1 = round((1-rf)*numel(map2)) = 0, so no LP is solved:
+    In = I.resetRow(map1); S = multipleStepReachStarApprox_at_one(In, map, lb(map), ub(map)).
+    """
+    if not isinstance(I, OStar):
+        raise TypeError("Input is not a star")
+    if relax_factor < 0 or relax_factor > 1:
+        raise ValueError("Invalid relax factor")
+    if relax_factor != 1:
+        raise NotImplementedError("oracle restates the relaxFactor = 1 path only")
+    lb, ub = estimate_ranges(I)
+    map1, mp = relax_classify(lb, ub, method)
+    In = reset_row(I, map1)
+    return multiple_step_reach_star_approx_at_one(In, mp, lb[mp], ub[mp])
+
+
+def poslin_reach(I, method, option=None, relax_factor=0.0, dis_opt=None, lp_solver="linprog"):
+    """PosLin.reach dispatcher, nn/funcs/PosLin.m:2073-2169 (relax-star branches only)."""
+    if method in RELAX_METHODS:
+        return reach_relaxed_star(I, method, relax_factor)
+    raise ValueError("This reachability method does not exist")
+
+
+def relu_reach(I, method, relax_factor=1.0):
+    """ReluLayer.reach_star_single_input, nn/layers/ReluLayer.m:72-150.
+
+    ImageStar: toStar -> PosLin.reach -> toImageStar(h, w, c); Star: PosLin.reach.
+    """
+    if isinstance(I, OImageStar):
+        Y = poslin_reach(I.to_star(), method, None, relax_factor)
+        return star_to_image_star(Y, I.height, I.width, I.numChannel)
+    if isinstance(I, OStar):
+        return poslin_reach(I, method, None, relax_factor)
+    raise TypeError("input is not an ImageStar, Star or VolumeStar")
+
+
+# --------------------------------------------------------------------------------------
+# network loop
+# --------------------------------------------------------------------------------------
+def nn_reach(layers, input_set, reach_method="relax-star-area", relax_factor=1.0, keep=False):
+    """NN.reach -> reach_noConns, nn/NN.m:189-278, 1529-1551, for a list of layer dicts:
+
+    {"type": "fc", "W": (Out x In), "b": (Out,)}
+    {"type": "conv", "W": (FH x FW x Cin x Cout), "b": (Cout,), "padding": [t b l r],
+     "stride": [sh sw], "dilation": [dh dw]}
+    {"type": "relu"}
+
+    input_set may be a set or a list of sets (the reference loops serially over arrays,
+    nn/layers/FullyConnectedLayer.m:504-507).  Returns the output set(s); with keep=True also
+    the per-layer sets (NN.reachSet).
+    """
+    if "relax-star" in reach_method and not (0 <= relax_factor <= 1):
+        raise ValueError("Invalid relaxFactor. The value of relax factor must be between 0 and 1")
+    single = not isinstance(input_set, (list, tuple))
+    sets = [input_set] if single else list(input_set)
+    reach_set = []
+    for L in layers:
+        out = []
+        for S in sets:
+            if L["type"] == "fc":
+                out.append(fc_reach(S, L["W"], L["b"]))
+            elif L["type"] == "conv":
+                out.append(conv2d_reach(S, L["W"], L.get("b"), L.get("padding", (0, 0, 0, 0)),
+                                        L.get("stride", (1, 1)), L.get("dilation", (1, 1))))
+            elif L["type"] == "relu":
+                out.append(relu_reach(S, reach_method, relax_factor))
+            else:
+                raise ValueError("unknown layer type " + str(L["type"]))
+        sets = out
+        if keep:
+            reach_set.append(out[0] if single else out)
+    res = sets[0] if single else sets
+    return (res, reach_set) if keep else res
+
+
+def output_ranges(S):
+    """Reported output bounds: estimateRanges of the last layer's set (set/Star.m:1078-1106)."""
+    if isinstance(S, OImageStar):
+        S = S.to_star() if S.im_lb is None else OStar(
+            S.V.reshape(-1, S.numPred + 1, order="F"), S.C, S.d, S.pred_lb, S.pred_ub)
+    return estimate_ranges(S)
+
+
+def evaluate(layers, x):
+    """Concrete forward pass (layer.evaluate) used by the containment checks:
+    FC y = W*x + b (nn/layers/FullyConnectedLayer.m:159), conv = cross-correlation + bias,
+    ReLU = max(x, 0)."""
+    x = np.asarray(x, dtype=np.float64)
+    for L in layers:
+        if L["type"] == "fc":
+            x = np.asarray(L["W"]) @ x.reshape(-1, order="F") + np.asarray(L["b"]).reshape(-1)
+        elif L["type"] == "conv":
+            x = conv2d_tensor(x.reshape(x.shape + (1,) * (4 - x.ndim)) if x.ndim == 3 else x[:, :, None, None],
+                              L["W"], L.get("b"), L.get("padding", (0, 0, 0, 0)),
+                              L.get("stride", (1, 1)), L.get("dilation", (1, 1)))[:, :, :, 0]
+        elif L["type"] == "relu":
+            x = np.maximum(x, 0)
+    return x

@@ -1,0 +1,91 @@
+"""Pin the CPU oracle against the reference's own golden vectors and known-answer tests."""
+import numpy as np
+import pytest
+
+from oracle import nnv_oracle as o
+
+
+def test_affine_map_known_answer(golden):
+    # results/tests/baselines/set/test_star_affineMap_results.mat: S1 = S.affineMap(W, b)
+    g = golden["star_affineMap"]
+    S = o.OStar(g["S_V"], g["S_C"], g["S_d"])
+    S1 = o.affine_map(S, g["W"], g["b"])
+    assert np.array_equal(S1.V, g["S1_V"])
+    assert np.array_equal(S1.C, g["S1_C"])           # constraints pass through untouched
+    assert np.array_equal(S1.d, g["S1_d"].reshape(-1))
+
+
+def test_affine_map_rejects_bad_shapes(golden):
+    g = golden["star_affineMap"]
+    S = o.OStar(g["S_V"], g["S_C"], g["S_d"])
+    with pytest.raises(ValueError, match="affine mapping matrix"):
+        o.affine_map(S, np.ones((2, 3)), None)
+    with pytest.raises(ValueError, match="mapping vec"):
+        o.affine_map(S, np.ones((2, 2)), np.ones(3))
+
+
+def test_box_star_affine_ranges_known_answer(golden):
+    # Star(lb, ub).affineMap(W2, []) then ranges: S4_lb / S4_ub.  The reference stored LP
+    # ranges (getRanges); on a star whose only constraints are the predicate box the LP optimum
+    # is the interval closed form estimateRanges computes, so they agree to rounding.
+    g = golden["star_affineMap"]
+    S3 = o.star_from_box(g["box_lb"].reshape(-1), g["box_ub"].reshape(-1))
+    assert S3.V.shape == (3, 4) and S3.nVar == 3
+    assert np.array_equal(S3.C, np.zeros((1, 3))) and np.array_equal(S3.d, np.zeros(1))
+    assert np.array_equal(S3.predicate_lb, -np.ones(3)) and np.array_equal(S3.predicate_ub, np.ones(3))
+    S4 = o.affine_map(S3, g["W2"], None)
+    lb, ub = o.estimate_ranges(S4)
+    np.testing.assert_allclose(lb, g["S4_lb"].reshape(-1), rtol=0, atol=1e-14)
+    np.testing.assert_allclose(ub, g["S4_ub"].reshape(-1), rtol=0, atol=1e-14)
+    # W2 is MATLAB rng(42); rand(3,3) == numpy RandomState(42) filled column-major
+    W2 = np.random.RandomState(42).rand(9).reshape(3, 3, order="F")
+    assert np.array_equal(W2, g["W2"])
+
+
+def test_star_box_values(golden):
+    # star_test.m stores B2 = box of a star; a box star built from those bounds has
+    # centre 0.5*(lb+ub) and one generator per non-degenerate dimension (Box.m:35-45).
+    g = golden["star_test"]
+    lb, ub = g["B2_lb"].reshape(-1), g["B2_ub"].reshape(-1)
+    S = o.star_from_box(lb, ub)
+    assert S.nVar == 2                       # dimension 0 has lb == ub -> zero column removed
+    assert np.array_equal(S.V[:, 0], 0.5 * (lb + ub))
+    assert np.array_equal(S.V[:, 1:], np.array([[0, 0], [0.5, 0], [0, 0.5]]))
+    l2, u2 = o.estimate_ranges(S)
+    assert np.array_equal(l2, lb) and np.array_equal(u2, ub)
+
+
+def test_conv_feature_map_known_answer(golden):
+    # tests/nn/layers/Conv2DLayer/test_layers_Conv2D.m:14-28
+    g = golden["conv2d_featureMap"]
+    fm = o.conv2d_feature_map(g["I"], g["W"], g["padding"], g["stride"], g["dilation"])
+    assert np.array_equal(fm, g["expected"])
+    assert np.array_equal(fm, np.array([[4, 3, 4], [2, 4, 3], [2, 3, 4]], dtype=float))
+    # the tensor routine used for reach agrees with the in-tree definition
+    t = o.conv2d_tensor(g["I"][:, :, None, None], g["W"][:, :, None, None], None,
+                        g["padding"], g["stride"], g["dilation"])
+    assert np.array_equal(t[:, :, 0, 0], g["expected"])
+
+
+def test_conv_not_flipped():
+    # an asymmetric filter distinguishes cross-correlation from true convolution
+    I = np.arange(16, dtype=float).reshape(4, 4)
+    W = np.array([[1.0, 2.0], [3.0, 4.0]])
+    fm = o.conv2d_feature_map(I, W, [0, 0, 0, 0], [1, 1], [1, 1])
+    assert fm[0, 0] == I[0, 0] * 1 + I[0, 1] * 2 + I[1, 0] * 3 + I[1, 1] * 4
+
+
+def test_imagestar_estimate_ranges_known_answer(golden):
+    # tests/set/image_star/test_ImageStar_getRange.m:45-62: V = [0,-1,1], pred in [-1,1]^2
+    g = golden["imagestar_getRange_issue"]
+    I = o.OImageStar(g["V"], np.zeros((1, 2)), np.zeros(1), g["pred_lb"].reshape(-1), g["pred_ub"].reshape(-1))
+    lb, ub = o.image_star_estimate_ranges(I)
+    assert lb.reshape(-1)[0] == -2.0 and ub.reshape(-1)[0] == 2.0
+    l2, u2 = o.estimate_ranges(I.to_star())
+    assert l2[0] == -2.0 and u2[0] == 2.0
+
+
+def test_relu_evaluate_known_answer(golden):
+    # tests/nn/layers/ReluLayer/test_layers_relu.m:19-33
+    g = golden["relu_evaluate"]
+    assert np.array_equal(o.evaluate([{"type": "relu"}], g["IM"]), g["IM_out"])
