@@ -1,0 +1,180 @@
+#!/usr/bin/env python3
+"""Benchmark of the relax-star reach path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--method relax-star-area]
+
+A step is one full ``NN.reach`` of the benchmark configuration (default: config 2, the fully
+connected 784-1024-1024-1024-10 net with a 784-generator input box) with the input set and the
+weights already resident in HBM; it ends with the output set and its estimated output bounds
+resident in HBM.  Prints ONE JSON line:
+
+  metric/value   generator-neuron updates per second = sum over layer steps of N_out*(n_out+1),
+                 divided by reach wall-time (ms_per_step is the reach wall-time itself)
+  roofline       the dominant kernel (the fp64 MFMA GEMM of the hidden FC layers): dense flop
+                 2*M*K*(n+1) per launch over its HIP-event duration, against 78.6 TFLOP/s
+  cpu_baseline   the CPU oracle (numpy/OpenBLAS restatement of NNV's path, "port") timed on this
+                 host on a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+FP64_MFMA_PEAK_TFLOPS = 78.6
+HBM_PEAK_GBS = 8000.0
+
+
+def layer_shapes(reach_set):
+    out = []
+    for s in reach_set:
+        sets = s if isinstance(s, list) else [s]
+        for t in sets:
+            N, n, _ = t._h.dims()
+            out.append((N, n))
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2)
+    ap.add_argument("--method", default="relax-star-area")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (sets shard across GPUs without communication; "
+                 "that path is not built) - use --gpus 1")
+
+    import nnv_amd
+    from nnv_amd.configs import count_updates, make_config
+    from tests.gpu_util import input_sets
+
+    cfg = make_config(args.config)
+    ctx = nnv_amd.default_context()
+    net = nnv_amd.NN.from_config(cfg["layers"], cfg["name"])
+    opts = {"reachMethod": args.method, "relaxFactor": 1}
+    dev_in, ora_in = input_sets(cfg)
+    lib, h = ctx.lib, ctx.handle
+
+    def step():
+        out = net.reach(dev_in, opts)
+        outs = out if isinstance(out, list) else [out]
+        for o_ in outs:  # output bounds, left on the device
+            nnv_amd._lib.check(lib.nnvhip_estimate_ranges(h, o_._h.h, None, None))
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    ctx.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = 1e3 * wall / args.steps
+    shapes = layer_shapes(net.reachSet)
+    updates = count_updates(shapes)
+    value = updates / (wall / args.steps)
+
+    # ---- per-kernel timing with HIP events on the library's stream ------------------------------
+    ctx.set_timing(True)
+    per_layer = np.zeros(len(net.Layers))
+    reps = max(5, min(args.steps, 20))
+    for _ in range(reps):
+        rs = dev_in
+        for i, L in enumerate(net.Layers):
+            rs = L.reach(rs, args.method, [], 1, None, "linprog")
+            per_layer[i] += ctx.last_op_time_ms()
+    per_layer /= reps
+    ctx.set_timing(False)
+
+    # dominant kernel: the GEMM of the FC layers with more than 32 output rows (one launch per layer)
+    gemm_flop, gemm_ms, gemm_launches = 0.0, 0.0, 0
+    relu_bytes, relu_ms = 0.0, 0.0
+    layer_report = []
+    prev_sets = dev_in if isinstance(dev_in, list) else [dev_in]
+    for i, (Ld, L) in enumerate(zip(cfg["layers"], net.Layers)):
+        outs = net.reachSet[i] if isinstance(net.reachSet[i], list) else [net.reachSet[i]]
+        entry = {"layer": i + 1, "type": Ld["type"], "ms": round(float(per_layer[i]), 4)}
+        if Ld["type"] == "fc":
+            M, K = Ld["W"].shape
+            cols = sum(s._h.dims()[1] + 1 for s in outs)
+            flop = 2.0 * M * K * cols
+            entry["dense_tflops"] = round(flop / (per_layer[i] * 1e-3) / 1e12, 3)
+            if M > 32:
+                gemm_flop += flop
+                gemm_ms += per_layer[i]
+                gemm_launches += 1
+        elif Ld["type"] == "conv":
+            fh, fw, cin, cout = Ld["W"].shape
+            flop = 0.0
+            for s in outs:
+                N, n, _ = s._h.dims()
+                flop += 2.0 * (N // cout) * cout * fh * fw * cin * (n + 1)
+            entry["dense_tflops"] = round(flop / (per_layer[i] * 1e-3) / 1e12, 3)
+        else:
+            b = 0.0
+            for sp, so in zip(prev_sets, outs):
+                N, n, _ = sp._h.dims()
+                m = so._h.dims()[1] - n
+                # estimateRanges read of V + masked copy read of V + write of the N x (n+1+m) output
+                b += 8.0 * N * (n + 1) * 2 + 8.0 * N * (n + 1 + m) + 8.0 * m * (n + 1)
+            entry["algo_GBps"] = round(b / (per_layer[i] * 1e-3) / 1e9, 1)
+            relu_bytes += b
+            relu_ms += per_layer[i]
+        layer_report.append(entry)
+        prev_sets = outs
+
+    if gemm_launches:
+        achieved = gemm_flop / (gemm_ms * 1e-3) / 1e12
+        roofline = {"kernel": "gemm_f64_kernel", "bound": "mfma", "achieved": round(achieved, 3),
+                    "peak": FP64_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / FP64_MFMA_PEAK_TFLOPS, 4),
+                    "traffic": None, "launches_per_step": gemm_launches,
+                    "avg_launch_ms": round(gemm_ms / gemm_launches, 4),
+                    "flop_per_launch": gemm_flop / gemm_launches}
+    else:
+        achieved = relu_bytes / (relu_ms * 1e-3) / 1e9
+        roofline = {"kernel": "relu step", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None}
+    if relu_ms > 0:
+        roofline["relu_step_algo_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
+
+    # ---- CPU baseline: the oracle on this host -------------------------------------------------
+    cpu = None
+    if not args.no_cpu:
+        from oracle import nnv_oracle as o
+        n_cpu, t_cpu = 0, 0.0
+        while t_cpu < args.cpu_seconds and n_cpu < 50:
+            t1 = time.perf_counter()
+            o.nn_reach(cfg["layers"], ora_in, args.method, 1.0)
+            t_cpu += time.perf_counter() - t1
+            n_cpu += 1
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cpu = {"value": updates / (t_cpu / n_cpu), "unit": "updates/s", "cores": threads, "kind": "port",
+               "ms_per_reach": round(1e3 * t_cpu / n_cpu, 2),
+               "sample": "%d full %s reach(es) by the numpy/OpenBLAS oracle (dense C built at every ReLU, as NNV does)"
+                         % (n_cpu, cfg["name"])}
+
+    print(json.dumps({
+        "metric": "generator_neuron_updates_per_s", "value": value, "unit": "updates/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": cfg["name"], "reach_method": args.method, "relax_factor": 1,
+                   "sets": len(dev_in) if isinstance(dev_in, list) else 1,
+                   "updates_per_step": updates,
+                   "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, list) else None},
+        "roofline": roofline, "cpu_baseline": cpu, "layers": layer_report,
+    }))
+
+
+if __name__ == "__main__":
+    main()

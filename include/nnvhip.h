@@ -1,0 +1,151 @@
+/*
+ * nnvhip.h - C ABI of libnnvhip.so: NNV's relax-star reachability path on one MI355X.
+ *
+ * The library keeps star sets resident in HBM behind opaque handles and runs, entirely on the
+ * device, the three layer operations NNV's NN.reach loop calls (relaxFactor = 1, fp64):
+ *
+ *   FullyConnectedLayer.reach  -> nnvhip_affine_fc        (Star.affineMap, W*[c V] + b)
+ *   Conv2DLayer.reach          -> nnvhip_affine_conv2d    (dlconv over the generator axis)
+ *   ReluLayer.reach            -> nnvhip_relu_relax       (PosLin.reach_relaxed_star_*)
+ *   Star.estimateRanges        -> nnvhip_estimate_ranges
+ *
+ * "file:line" citations are relative to code/nnv/engine/ of the NNV reference tree.
+ *
+ * Conventions: all matrices are fp64, column-major, exactly MATLAB's memory layout, so a MEX
+ * gateway passes mxGetDoubles() pointers straight through.  V is N x (n+1) with column 0 the
+ * centre.  An ImageStar's H x W x C x (n+1) tensor is the same memory as an (H*W*C) x (n+1)
+ * matrix (set/ImageStar.m:569-592, set/Star.m:1398-1418), so one handle type serves both.
+ * Index vectors are 0-based int32 here (NNV's are 1-based doubles; the gateway adds 1).
+ * Every function returns an nnvhip_status; on failure nnvhip_last_error() holds the message,
+ * which for NNV's own argument checks is NNV's error text.
+ *
+ * Threading: one host thread per context (NNV's relax-star reach is single-core,
+ * nn/NN.m:1227-1231).  Handles are reference counted; an operation never modifies its input.
+ */
+#ifndef NNVHIP_H
+#define NNVHIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct nnvhip_ctx nnvhip_ctx;       /* device context: stream, memory pool, timers   */
+typedef struct nnvhip_star nnvhip_star;     /* a Star / ImageStar resident in HBM            */
+typedef struct nnvhip_fc nnvhip_fc;         /* FullyConnectedLayer weights resident in HBM   */
+typedef struct nnvhip_conv2d nnvhip_conv2d; /* Conv2DLayer weights resident in HBM           */
+
+typedef enum {
+  NNVHIP_OK = 0,
+  NNVHIP_ERR_SHAPE = 1,        /* a size check of the reference failed                      */
+  NNVHIP_ERR_METHOD = 2,       /* unknown reachability method / crossing order              */
+  NNVHIP_ERR_RELAX_FACTOR = 3, /* relaxFactor outside [0,1], or != 1 (LP path not built)    */
+  NNVHIP_ERR_OOM = 4,          /* device allocation failed                                  */
+  NNVHIP_ERR_HIP = 5,          /* a HIP runtime call failed                                 */
+  NNVHIP_ERR_ARG = 6           /* null pointer / invalid handle / invalid argument          */
+} nnvhip_status;
+
+/* Order of the crossing neurons = order of the new predicate columns (nn/funcs/PosLin.m):
+ * INDEX  ascending neuron index: relax-star-bound/-ub/-random/-static (:1167-1232, :1326-1397,
+ *        :1488-1492, :1604-1605);
+ * AREA   sort(0.5*|ub|.*|lb|, 'descend'), stable: relax-star-area (:1049-1052);
+ * RANGE  sort(ub-lb, 'descend'), stable: relax-star-range (:934-936). */
+typedef enum { NNVHIP_ORDER_INDEX = 0, NNVHIP_ORDER_AREA = 1, NNVHIP_ORDER_RANGE = 2 } nnvhip_order;
+
+/* ---- context -------------------------------------------------------------------------- */
+/* Replaces NN.reach's reachOptions.device hook (nn/NN.m:216-222): selects the GPU, creates the
+ * stream and the device memory pool. */
+int nnvhip_create(int device, nnvhip_ctx** ctx);
+int nnvhip_destroy(nnvhip_ctx* ctx);
+/* Message of the last failing call on this thread. */
+const char* nnvhip_last_error(void);
+/* Waits for all queued device work of the context (wait(gpuDevice) in the reference's GPU path). */
+int nnvhip_synchronize(nnvhip_ctx* ctx);
+/* Device time in ms of the most recent layer call (NN.reachTime(i) = toc, nn/NN.m:1542-1545).
+ * Timing is off by default; enabling it makes this call wait for the layer to finish. */
+int nnvhip_set_timing(nnvhip_ctx* ctx, int enabled);
+int nnvhip_last_op_time_ms(nnvhip_ctx* ctx, double* ms);
+/* Returns every cached device block of the pool to the driver (hipFree). */
+int nnvhip_trim_pool(nnvhip_ctx* ctx);
+/* Bytes currently handed out by / cached in the pool. */
+int nnvhip_pool_stats(nnvhip_ctx* ctx, int64_t* bytes_in_use, int64_t* bytes_cached);
+
+/* ---- sets ----------------------------------------------------------------------------- */
+/* Star(V, C, d, pred_lb, pred_ub), set/Star.m:153-189: uploads host arrays.  V is N x (n+1),
+ * C is p x n, d has p entries; pred_lb/pred_ub may be NULL (both) for the -1/+1 default of
+ * Star.estimateRanges (set/Star.m:1091-1096).  C/d may be NULL with p = 0. */
+int nnvhip_star_create(nnvhip_ctx* ctx, int64_t N, int64_t n, const double* V, const double* pred_lb,
+                       const double* pred_ub, const double* C, const double* d, int64_t p,
+                       nnvhip_star** out);
+/* Star(lb, ub), set/Star.m:220-237 with Box (set/Box.m:16-58): centre 0.5*(lb+ub), one
+ * generator 0.5*(ub-lb)(i)*e_i per dimension with non-zero half-width, C = zeros(1,n), d = 0,
+ * predicate bounds -1/+1.  Built on the device from the two N-vectors.  `count` boxes are given
+ * as the columns of N x count matrices; out[] receives `count` handles laid out back to back in
+ * one device arena (the array of Stars NN.reach accepts, nn/NN.m:204-207). */
+int nnvhip_star_from_box(nnvhip_ctx* ctx, int64_t N, int64_t count, const double* lb, const double* ub,
+                         nnvhip_star** out);
+int nnvhip_star_retain(nnvhip_star* s);
+int nnvhip_star_release(nnvhip_star* s);
+/* dim, nVar and the number of constraint rows size(C,1). */
+int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p);
+/* Property reads: dense MATLAB arrays.  V: N x (n+1).  Bounds: n each.  C: p x n, d: p, laid out
+ * exactly as PosLin.multipleStepReachStarApprox_at_one builds them, [C0;C1;C2;C3]
+ * (nn/funcs/PosLin.m:711-735), materialised from the device's structured store. */
+int nnvhip_star_fetch_V(const nnvhip_star* s, double* V);
+int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* pred_lb, double* pred_ub);
+int nnvhip_star_fetch_constraints(const nnvhip_star* s, double* C, double* d);
+/* For a set returned by nnvhip_relu_relax: counts of inactive (ub <= 0) and crossing
+ * (lb < 0 & ub > 0) neurons, and the crossing list in new-predicate order with its bounds
+ * (map1/map2 and lb(map), ub(map) of nn/funcs/PosLin.m:921-925, 1094-1096).  Any output pointer
+ * may be NULL. */
+int nnvhip_star_relu_counts(const nnvhip_star* s, int64_t* n_inactive, int64_t* n_crossing);
+int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb, double* ub);
+
+/* ---- Star.estimateRanges, set/Star.m:1078-1106 ------------------------------------------ */
+/* lb = c + max(V,0)*[0;pred_lb] + min(V,0)*[0;pred_ub]; ub likewise.  One pass over V; the
+ * result is cached on the handle (nnvhip_relu_relax reuses it).  lb/ub: host, N entries each,
+ * may be NULL to only compute and cache on the device. */
+int nnvhip_estimate_ranges(nnvhip_ctx* ctx, nnvhip_star* s, double* lb, double* ub);
+/* Array form: lb/ub are N x count (all sets must have the same dim). */
+int nnvhip_estimate_ranges_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, double* lb,
+                                 double* ub);
+
+/* ---- layers ---------------------------------------------------------------------------- */
+/* FullyConnectedLayer(W, b), nn/layers/FullyConnectedLayer.m:39-99: W is M x K, b has M entries
+ * (NULL = no bias, the affineMap(W, []) form). */
+int nnvhip_fc_create(nnvhip_ctx* ctx, const double* W, const double* b, int64_t M, int64_t K,
+                     nnvhip_fc** out);
+int nnvhip_fc_destroy(nnvhip_fc* fc);
+/* Conv2DLayer(W, b, padding, stride, dilation), nn/layers/Conv2DLayer.m:15-33: W is
+ * FH x FW x Cin x Cout, bias has Cout entries (NULL = 0), padding [t b l r], stride [sh sw],
+ * dilation [dh dw]. */
+int nnvhip_conv2d_create(nnvhip_ctx* ctx, const double* W, const double* bias, int64_t FH, int64_t FW,
+                         int64_t Cin, int64_t Cout, const int64_t padding[4], const int64_t stride[2],
+                         const int64_t dilation[2], nnvhip_conv2d** out);
+int nnvhip_conv2d_destroy(nnvhip_conv2d* conv);
+/* Output feature-map size for an H x W input, nn/layers/Conv2DLayer.m:1134-1135. */
+int nnvhip_conv2d_output_size(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t* Ho, int64_t* Wo);
+
+/* FullyConnectedLayer.reach_star_single_input / Star.affineMap,
+ * nn/layers/FullyConnectedLayer.m:295-316, 476-481; set/Star.m:313-343:
+ * V' = W*V; V'(:,1) += b; constraints and predicate bounds are shared with the input.
+ * `count` sets are mapped in one pass (reach_star_multipleInputs, :486-512). */
+int nnvhip_affine_fc(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, nnvhip_star* const* in,
+                     nnvhip_star** out);
+/* Conv2DLayer.reach_star_single_input, nn/layers/Conv2DLayer.m:559-601, 780: the input set is
+ * read as an H x W x Cin x (n+1) ImageStar; centre gets conv + bias, generators conv only;
+ * cross-correlation (no kernel flip), zero padding.  Output dim is Ho*Wo*Cout. */
+int nnvhip_affine_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t count,
+                         nnvhip_star* const* in, nnvhip_star** out);
+/* ReluLayer.reach -> PosLin.reach(I, 'relax-star-*', [], relaxFactor, ...),
+ * nn/layers/ReluLayer.m:72-150, nn/funcs/PosLin.m:863-1650, 685-742, set/Star.m:1442-1461.
+ * estimateRanges; inactive rows -> 0; every crossing neuron gets a new predicate column, the
+ * three triangle constraints and predicate bounds [0, ub].  relax_factor must be 1 (no LP). */
+int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor, int64_t count,
+                      nnvhip_star* const* in, nnvhip_star** out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NNVHIP_H */

@@ -1,1 +1,9 @@
-"""nnv_amd: MI355X-native star-set reachability (relax-star, relaxFactor = 1) behind NNV's API."""
+"""nnv_amd: MI355X-native star-set reachability (relax-star, relaxFactor = 1) behind NNV's API.
+
+The compute path is the HIP library nnv_amd/libnnvhip.so (C ABI in include/nnvhip.h); these Python
+classes mirror NNV's MATLAB classes for the path and call it through ctypes.
+"""
+from ._lib import Context, NNVHipError, NNVHipOutOfMemory, default_context  # noqa: F401
+from .layers import Conv2DLayer, FullyConnectedLayer, PosLin, ReluLayer  # noqa: F401
+from .nn import NN  # noqa: F401
+from .sets import Box, ImageStar, Star  # noqa: F401

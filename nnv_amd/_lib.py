@@ -1,0 +1,149 @@
+"""ctypes binding of libnnvhip.so.  There is no CPU fallback: a missing library is an error."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libnnvhip.so")
+
+OK, ERR_SHAPE, ERR_METHOD, ERR_RELAX_FACTOR, ERR_OOM, ERR_HIP, ERR_ARG = range(7)
+ORDER_INDEX, ORDER_AREA, ORDER_RANGE = 0, 1, 2
+
+# every entry point declared in include/nnvhip.h
+SYMBOLS = [
+    "nnvhip_create", "nnvhip_destroy", "nnvhip_last_error", "nnvhip_synchronize", "nnvhip_set_timing",
+    "nnvhip_last_op_time_ms", "nnvhip_trim_pool", "nnvhip_pool_stats", "nnvhip_star_create",
+    "nnvhip_star_from_box", "nnvhip_star_retain", "nnvhip_star_release", "nnvhip_star_dims",
+    "nnvhip_star_fetch_V", "nnvhip_star_fetch_pred_bounds", "nnvhip_star_fetch_constraints",
+    "nnvhip_star_relu_counts", "nnvhip_star_fetch_crossing", "nnvhip_estimate_ranges",
+    "nnvhip_estimate_ranges_batch", "nnvhip_fc_create", "nnvhip_fc_destroy", "nnvhip_conv2d_create",
+    "nnvhip_conv2d_destroy", "nnvhip_conv2d_output_size", "nnvhip_affine_fc", "nnvhip_affine_conv2d",
+    "nnvhip_relu_relax",
+]
+
+
+class NNVHipError(RuntimeError):
+    """A HIP runtime failure or an invalid handle."""
+
+
+class NNVHipOutOfMemory(MemoryError):
+    pass
+
+
+_lib = None
+
+
+def load():
+    """Load the in-tree HIP library; raises if it has not been built (python -m nnv_amd.build)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("nnv_amd/libnnvhip.so is missing: build it with `python -m nnv_amd.build` "
+                          "(there is no CPU fallback)")
+    lib = C.CDLL(LIB_PATH)
+    p, i64, dbl = C.c_void_p, C.c_int64, C.c_double
+    pp = C.POINTER(C.c_void_p)
+    pi64 = C.POINTER(C.c_int64)
+    sig = {
+        "nnvhip_create": [C.c_int, pp],
+        "nnvhip_destroy": [p],
+        "nnvhip_synchronize": [p],
+        "nnvhip_set_timing": [p, C.c_int],
+        "nnvhip_last_op_time_ms": [p, C.POINTER(dbl)],
+        "nnvhip_trim_pool": [p],
+        "nnvhip_pool_stats": [p, pi64, pi64],
+        "nnvhip_star_create": [p, i64, i64, p, p, p, p, p, i64, pp],
+        "nnvhip_star_from_box": [p, i64, i64, p, p, pp],
+        "nnvhip_star_retain": [p],
+        "nnvhip_star_release": [p],
+        "nnvhip_star_dims": [p, pi64, pi64, pi64],
+        "nnvhip_star_fetch_V": [p, p],
+        "nnvhip_star_fetch_pred_bounds": [p, p, p],
+        "nnvhip_star_fetch_constraints": [p, p, p],
+        "nnvhip_star_relu_counts": [p, pi64, pi64],
+        "nnvhip_star_fetch_crossing": [p, p, p, p],
+        "nnvhip_estimate_ranges": [p, p, p, p],
+        "nnvhip_estimate_ranges_batch": [p, i64, pp, p, p],
+        "nnvhip_fc_create": [p, p, p, i64, i64, pp],
+        "nnvhip_fc_destroy": [p],
+        "nnvhip_conv2d_create": [p, p, p, i64, i64, i64, i64, pi64, pi64, pi64, pp],
+        "nnvhip_conv2d_destroy": [p],
+        "nnvhip_conv2d_output_size": [p, i64, i64, pi64, pi64],
+        "nnvhip_affine_fc": [p, p, i64, pp, pp],
+        "nnvhip_affine_conv2d": [p, p, i64, i64, i64, pp, pp],
+        "nnvhip_relu_relax": [p, C.c_int, dbl, i64, pp, pp],
+    }
+    for name, args in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = C.c_int
+    lib.nnvhip_last_error.argtypes = []
+    lib.nnvhip_last_error.restype = C.c_char_p
+    _lib = lib
+    return lib
+
+
+def check(status: int):
+    """Turn a non-zero status into the exception NNV's error() call corresponds to."""
+    if status == OK:
+        return
+    msg = load().nnvhip_last_error().decode("utf-8", "replace")
+    if status in (ERR_SHAPE, ERR_METHOD, ERR_RELAX_FACTOR):
+        raise ValueError(msg)
+    if status == ERR_OOM:
+        raise NNVHipOutOfMemory(msg)
+    raise NNVHipError(msg)
+
+
+def f64(a, order="F"):
+    """Contiguous column-major fp64 copy/view of a host array (MATLAB memory layout)."""
+    return np.require(np.asarray(a, dtype=np.float64), dtype=np.float64, requirements=["F" if order == "F" else "C", "A"])
+
+
+def ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+_default_ctx = None
+
+
+class Context:
+    """One GPU context: stream, device memory pool, per-layer timer."""
+
+    def __init__(self, device: int = 0):
+        lib = load()
+        h = C.c_void_p()
+        check(lib.nnvhip_create(int(device), C.byref(h)))
+        self.handle = h
+        self.lib = lib
+        self.device = device
+
+    def synchronize(self):
+        check(self.lib.nnvhip_synchronize(self.handle))
+
+    def set_timing(self, enabled: bool):
+        check(self.lib.nnvhip_set_timing(self.handle, 1 if enabled else 0))
+
+    def last_op_time_ms(self) -> float:
+        ms = C.c_double()
+        check(self.lib.nnvhip_last_op_time_ms(self.handle, C.byref(ms)))
+        return ms.value
+
+    def pool_stats(self):
+        a, b = C.c_int64(), C.c_int64()
+        check(self.lib.nnvhip_pool_stats(self.handle, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def trim_pool(self):
+        check(self.lib.nnvhip_trim_pool(self.handle))
+
+
+def default_context() -> Context:
+    global _default_ctx
+    if _default_ctx is None:
+        _default_ctx = Context(int(os.environ.get("NNVHIP_DEVICE", "0")))
+    return _default_ctx

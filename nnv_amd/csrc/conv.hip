@@ -1,0 +1,228 @@
+// affineMap of a Conv2DLayer on an ImageStar (nn/layers/Conv2DLayer.m:559-601): the same
+// cross-correlation applied to the centre image (plus bias) and to every generator image.
+//
+// Implicit GEMM on fp64 MFMA.  With P = Ho*Wo output positions per image and G = n+1 images the
+// output, in MATLAB's H x W x C x (n+1) layout, is a (P*G) x Cout matrix whose rows are contiguous in
+// memory per (channel, image); the reduction runs over the K = FH*FW*Cin filter taps, which is
+// exactly the row order of MATLAB's FH x FW x Cin x Cout weight array.  The im2col operand is never
+// materialised: each block gathers its 128-position x 16-tap tile straight from the input images
+// (zero for padding taps) into LDS; the weight tile is loaded like the generator tile of the dense
+// GEMM.  MFMA operand "b" carries positions (the memory-contiguous direction of the output), "a"
+// carries output channels.
+#include <algorithm>
+
+#include "internal.h"
+#include "mfma_tile.h"
+
+namespace nnvhip {
+
+struct ConvGeom {
+  int H, W, Cin, Ho, Wo, Cout;
+  int FH, FW, sh, sw, dh, dw, pt, pl;
+  int K, Kp;
+  int P;   // Ho * Wo
+  int HW;  // H * W
+};
+
+constexpr int kMaxTaps = 4096;  // tap table held in LDS: 8 bytes per (padded) tap
+
+// Tap k = fh + FH*(fw + FW*ci) -> packed (input offset ci*H*W : 32 | fh*dh : 16 | fw*dw : 16).
+__device__ __forceinline__ unsigned long long pack_tap(const ConvGeom& g, int k) {
+  if (k >= g.K) return ~0ull;  // padded tap: never valid
+  const int fh = k % g.FH;
+  const int t = k / g.FH;
+  const int fw = t % g.FW;
+  const int ci = t / g.FW;
+  return ((unsigned long long)(unsigned)(ci * g.HW) << 32) | ((unsigned long long)(fh * g.dh) << 16) |
+         (unsigned long long)(fw * g.dw);
+}
+
+template <int TP, int TC, int WR, int WC>
+__global__ __launch_bounds__(256) void conv2d_f64_kernel(const double* __restrict__ in, int64_t ldin,
+                                                          double* __restrict__ out, int64_t ldout,
+                                                          const double* __restrict__ Wt,
+                                                          const double* __restrict__ bias, ConvGeom g,
+                                                          int64_t total_rows, int tiles_c) {
+  static_assert(WR * WC == 4, "four waves per block");
+  constexpr int FM = TP / WR / 16;
+  constexpr int FN = TC / WC / 16;
+  constexpr int LDP_S = TP + kPadRow;  // Ps[k][position]
+  constexpr int LDW_S = kKt + kPadK;   // Wts[cout][k]
+  __shared__ double Ps[2][kKt * LDP_S];
+  __shared__ double Wts[2][TC * LDW_S];
+  extern __shared__ unsigned long long taps[];  // Kp entries
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wr = wave % WR;
+  const int wc = wave / WR;
+  const int64_t bid = blockIdx.x;
+  const int c0 = (int)(bid % tiles_c) * TC;
+  const int64_t R0 = (bid / tiles_c) * TP;
+
+  for (int k = tid; k < g.Kp; k += 256) taps[k] = pack_tap(g, k);
+
+  // this thread's gather position (fixed for the whole K loop)
+  constexpr int P_PASS = TP * kKt / 256;  // gathered elements per thread per K-tile
+  constexpr int K_STEP = 256 / TP;        // taps covered by one pass
+  const int p_local = tid % TP;
+  const int k_first = tid / TP;
+  const int64_t R = R0 + p_local;
+  const bool rvalid = R < total_rows;
+  int h0 = 0, w0 = 0;
+  const double* img = in;
+  if (rvalid) {
+    const int64_t gi = R / g.P;
+    const int p = (int)(R - gi * g.P);
+    const int wo = p / g.Ho;
+    const int ho = p - wo * g.Ho;
+    h0 = ho * g.sh - g.pt;
+    w0 = wo * g.sw - g.pl;
+    img = in + gi * ldin;
+  }
+
+  constexpr int W_VEC = TC * kKt / 2;
+  constexpr int W_PASS = (W_VEC + 255) / 256;
+  double rp[P_PASS];
+  double2 rw[W_PASS];
+
+  auto load_tiles = [&](int k0) {
+#pragma unroll
+    for (int q = 0; q < P_PASS; ++q) {
+      const unsigned long long t = taps[k0 + k_first + q * K_STEP];
+      const int h = h0 + (int)((t >> 16) & 0xffffu);
+      const int w = w0 + (int)(t & 0xffffu);
+      const bool ok = rvalid && t != ~0ull && (unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W;
+      rp[q] = ok ? img[(int64_t)(unsigned)(t >> 32) + h + (int64_t)w * g.H] : 0.0;
+    }
+#pragma unroll
+    for (int q = 0; q < W_PASS; ++q) {
+      const int idx = tid + q * 256;
+      const int k2 = idx % (kKt / 2);
+      const int j = idx / (kKt / 2);
+      double2 v = make_double2(0.0, 0.0);
+      if (idx < W_VEC && c0 + j < g.Cout) v = *reinterpret_cast<const double2*>(Wt + (k0 + 2 * k2) + (int64_t)(c0 + j) * g.Kp);
+      rw[q] = v;
+    }
+  };
+  auto store_tiles = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < P_PASS; ++q) Ps[buf][(k_first + q * K_STEP) * LDP_S + p_local] = rp[q];
+#pragma unroll
+    for (int q = 0; q < W_PASS; ++q) {
+      const int idx = tid + q * 256;
+      const int k2 = idx % (kKt / 2);
+      const int j = idx / (kKt / 2);
+      if (idx < W_VEC) *reinterpret_cast<double2*>(&Wts[buf][j * LDW_S + 2 * k2]) = rw[q];
+    }
+  };
+
+  double4_t acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j) acc[i][j] = double4_t{0.0, 0.0, 0.0, 0.0};
+
+  __syncthreads();  // tap table ready
+  const int nk = g.Kp / kKt;
+  load_tiles(0);
+  store_tiles(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) load_tiles((kt + 1) * kKt);
+    mfma_tile_k16<FM, FN>(&Ps[cur][wr * (TP / WR)], LDP_S, &Wts[cur][(wc * (TC / WC)) * LDW_S], LDW_S, lane, acc);
+    if (kt + 1 < nk) store_tiles(cur ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: lane l, register r holds out[position R0 + ... + l%16][channel c0 + ... + l/16 + 4r]
+  const int lrow = lane & 15;
+  const int lcol = lane >> 4;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int64_t Rr = R0 + wr * (TP / WR) + i * 16 + lrow;
+    if (Rr >= total_rows) continue;
+    const int64_t gi = Rr / g.P;
+    const int p = (int)(Rr - gi * g.P);
+    double* o = out + gi * ldout + p;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int co = c0 + wc * (TC / WC) + j * 16 + lcol + 4 * r;
+        if (co < g.Cout) {
+          double v = acc[i][j][r];
+          if (bias != nullptr && gi == 0) v = v + bias[co];  // centre image only
+          o[(int64_t)co * g.P] = v;
+        }
+      }
+    }
+  }
+}
+
+__global__ void zero_pad_rows_kernel(double* __restrict__ V, int64_t ld, int64_t N, int64_t ncols) {
+  const int64_t pad = ld - N;
+  const int64_t total = pad * ncols;
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x)
+    V[N + t % pad + (t / pad) * ld] = 0.0;
+}
+
+template <int TP, int TC, int WR, int WC>
+static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGeom& g, const double* in, int64_t ldin,
+                           double* out, int64_t ldout, int64_t ncols) {
+  const int64_t total_rows = (int64_t)g.P * ncols;
+  const int64_t tiles_c = ceil_div(g.Cout, TC);
+  const int64_t blocks = ceil_div(total_rows, TP) * tiles_c;
+  if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
+  const size_t dyn = sizeof(unsigned long long) * g.Kp;
+  hipLaunchKernelGGL((conv2d_f64_kernel<TP, TC, WR, WC>), dim3((unsigned)blocks), dim3(256), dyn, ctx->stream, in, ldin,
+                     out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows,
+                     (int)tiles_c);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                  const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
+                  const int32_t* /*centre_flags*/) {
+  if (cv->Kp > kMaxTaps) NNV_FAIL(NNVHIP_ERR_SHAPE, "filters with more than %d taps (FH*FW*Cin) are not supported", kMaxTaps);
+  if ((cv->FH - 1) * cv->dil[0] > 0xffff || (cv->FW - 1) * cv->dil[1] > 0xffff)
+    NNV_FAIL(NNVHIP_ERR_SHAPE, "dilated filter extent too large");
+  ConvGeom g;
+  g.H = (int)H;
+  g.W = (int)W;
+  g.Cin = (int)cv->Cin;
+  g.Ho = (int)Ho;
+  g.Wo = (int)Wo;
+  g.Cout = (int)cv->Cout;
+  g.FH = (int)cv->FH;
+  g.FW = (int)cv->FW;
+  g.sh = (int)cv->stride[0];
+  g.sw = (int)cv->stride[1];
+  g.dh = (int)cv->dil[0];
+  g.dw = (int)cv->dil[1];
+  g.pt = (int)cv->pad[0];
+  g.pl = (int)cv->pad[2];
+  g.K = (int)cv->K;
+  g.Kp = (int)cv->Kp;
+  g.P = (int)(Ho * Wo);
+  g.HW = (int)(H * W);
+  const int64_t Nout = Ho * Wo * cv->Cout;
+  int st;
+  if (cv->Cout <= 16)
+    st = launch_conv_cfg<128, 16, 4, 1>(ctx, cv, g, in, ldin, out, ldout, ncols);
+  else if (cv->Cout <= 32)
+    st = launch_conv_cfg<128, 32, 2, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
+  else
+    st = launch_conv_cfg<128, 64, 2, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
+  NNV_TRY(st);
+  if (ldout != Nout) {  // keep the padding rows of the output at zero
+    hipLaunchKernelGGL(zero_pad_rows_kernel, dim3(256), dim3(256), 0, ctx->stream, out, ldout, Nout, ncols);
+    NNV_HIP_TRY(hipGetLastError());
+  }
+  return NNVHIP_OK;
+}
+
+}  // namespace nnvhip

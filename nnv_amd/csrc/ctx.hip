@@ -1,0 +1,710 @@
+// Context, device memory pool, set handles and the host-side orchestration of the affine layers.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "internal.h"
+
+namespace nnvhip {
+
+static thread_local char g_err[1024] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+}
+
+Buffer::~Buffer() {
+  if (ctx && ptr) ctx->release_block(ptr, bytes);
+}
+
+// Size classes: multiples of 256 B up to 64 KiB, then 1/8-octave steps (<= 12.5 % slack), so a
+// repeated reach over the same network re-uses every block without calling hipMalloc again.
+static size_t size_class(size_t bytes) {
+  if (bytes < 256) return 256;
+  if (bytes <= (64u << 10)) return (bytes + 255) & ~size_t(255);
+  size_t p = size_t(1) << (63 - __builtin_clzll((unsigned long long)bytes));
+  size_t step = p >> 3;
+  return (bytes + step - 1) / step * step;
+}
+
+nnvhip_star* new_star(nnvhip_ctx* ctx) {
+  nnvhip_star* s = new nnvhip_star();
+  s->ctx = ctx;
+  ctx->live_handles++;
+  return s;
+}
+
+}  // namespace nnvhip
+
+using namespace nnvhip;
+
+int nnvhip_ctx::alloc(size_t bytes, BufRef* out) {
+  size_t cls = size_class(bytes ? bytes : 1);
+  void* p = nullptr;
+  auto it = free_blocks.find(cls);
+  if (it != free_blocks.end()) {
+    p = it->second;
+    free_blocks.erase(it);
+    bytes_cached -= (int64_t)cls;
+  } else {
+    hipError_t e = hipMalloc(&p, cls);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      trim();  // give cached blocks back and retry once
+      e = hipMalloc(&p, cls);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        NNV_FAIL(NNVHIP_ERR_OOM, "out of device memory allocating %zu bytes", cls);
+      }
+    }
+  }
+  bytes_in_use += (int64_t)cls;
+  auto b = std::make_shared<Buffer>();
+  b->ctx = this;
+  b->ptr = p;
+  b->bytes = cls;
+  *out = std::move(b);
+  return NNVHIP_OK;
+}
+
+void nnvhip_ctx::release_block(void* p, size_t bytes) {
+  // Blocks are recycled without waiting: every consumer runs on the context's single stream, so
+  // a later user of the block is ordered after the earlier one.
+  free_blocks.emplace(bytes, p);
+  bytes_in_use -= (int64_t)bytes;
+  bytes_cached += (int64_t)bytes;
+}
+
+int nnvhip_ctx::trim() {
+  if (stream) (void)hipStreamSynchronize(stream);
+  for (auto& kv : free_blocks) (void)hipFree(kv.second);
+  free_blocks.clear();
+  bytes_cached = 0;
+  return NNVHIP_OK;
+}
+
+int nnvhip_ctx::stage(size_t bytes, void** host) {
+  bytes = (bytes + 255) & ~size_t(255);
+  if (bytes > pinned_bytes) {
+    NNV_HIP_TRY(hipStreamSynchronize(stream));
+    if (pinned) NNV_HIP_TRY(hipHostFree(pinned));
+    pinned = nullptr;
+    pinned_bytes = std::max(bytes * 2, size_t(4) << 20);
+    NNV_HIP_TRY(hipHostMalloc((void**)&pinned, pinned_bytes, hipHostMallocDefault));
+    pinned_off = 0;
+  }
+  if (pinned_off + bytes > pinned_bytes) {
+    NNV_HIP_TRY(hipStreamSynchronize(stream));  // earlier async copies out of the ring are done
+    pinned_off = 0;
+  }
+  *host = pinned + pinned_off;
+  pinned_off += bytes;
+  return NNVHIP_OK;
+}
+
+int nnvhip_ctx::upload(const void* host, size_t bytes, BufRef* out) {
+  void* st = nullptr;
+  NNV_TRY(stage(bytes, &st));
+  memcpy(st, host, bytes);
+  NNV_TRY(alloc(bytes, out));
+  NNV_HIP_TRY(hipMemcpyAsync((*out)->ptr, st, bytes, hipMemcpyHostToDevice, stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_ctx::begin_op() {
+  if (timing) NNV_HIP_TRY(hipEventRecord(ev0, stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_ctx::end_op() {
+  if (timing) {
+    NNV_HIP_TRY(hipEventRecord(ev1, stream));
+    NNV_HIP_TRY(hipEventSynchronize(ev1));
+    float ms = 0.f;
+    NNV_HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
+    last_ms = ms;
+  }
+  return NNVHIP_OK;
+}
+
+#define CHECK_CTX(c)                                                  \
+  do {                                                                \
+    if (!(c)) NNV_FAIL(NNVHIP_ERR_ARG, "null context");               \
+    NNV_HIP_TRY(hipSetDevice((c)->device));                           \
+  } while (0)
+
+extern "C" {
+
+const char* nnvhip_last_error(void) { return g_err; }
+
+int nnvhip_create(int device, nnvhip_ctx** out) {
+  if (!out) NNV_FAIL(NNVHIP_ERR_ARG, "null output pointer");
+  int ndev = 0;
+  NNV_HIP_TRY(hipGetDeviceCount(&ndev));
+  if (device < 0 || device >= ndev) NNV_FAIL(NNVHIP_ERR_ARG, "device %d not present (%d visible)", device, ndev);
+  NNV_HIP_TRY(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  NNV_HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    NNV_FAIL(NNVHIP_ERR_ARG, "libnnvhip is built for gfx950 (MI355X); device %d is %s", device, prop.gcnArchName);
+  nnvhip_ctx* c = new nnvhip_ctx();
+  c->device = device;
+  NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+  NNV_HIP_TRY(hipEventCreate(&c->ev0));
+  NNV_HIP_TRY(hipEventCreate(&c->ev1));
+  *out = c;
+  return NNVHIP_OK;
+}
+
+int nnvhip_destroy(nnvhip_ctx* c) {
+  if (!c) return NNVHIP_OK;
+  if (c->live_handles != 0)
+    NNV_FAIL(NNVHIP_ERR_ARG, "context still has %lld live handles", (long long)c->live_handles);
+  NNV_HIP_TRY(hipSetDevice(c->device));
+  c->trim();
+  if (c->pinned) (void)hipHostFree(c->pinned);
+  (void)hipEventDestroy(c->ev0);
+  (void)hipEventDestroy(c->ev1);
+  (void)hipStreamDestroy(c->stream);
+  delete c;
+  return NNVHIP_OK;
+}
+
+int nnvhip_synchronize(nnvhip_ctx* c) {
+  CHECK_CTX(c);
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_set_timing(nnvhip_ctx* c, int enabled) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  c->timing = enabled != 0;
+  return NNVHIP_OK;
+}
+
+int nnvhip_last_op_time_ms(nnvhip_ctx* c, double* ms) {
+  if (!c || !ms) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  *ms = c->last_ms;
+  return NNVHIP_OK;
+}
+
+int nnvhip_trim_pool(nnvhip_ctx* c) {
+  CHECK_CTX(c);
+  return c->trim();
+}
+
+int nnvhip_pool_stats(nnvhip_ctx* c, int64_t* in_use, int64_t* cached) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  if (in_use) *in_use = c->bytes_in_use;
+  if (cached) *cached = c->bytes_cached;
+  return NNVHIP_OK;
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* sets                                                                                        */
+/* ------------------------------------------------------------------------------------------ */
+
+// Uploads a host column-major rows x cols matrix into a zero-padded device matrix with leading
+// dimension ld.
+static int upload_matrix(nnvhip_ctx* c, const double* host, int64_t rows, int64_t cols, int64_t ld,
+                         double* dev) {
+  if (rows == 0 || cols == 0) return NNVHIP_OK;
+  if (ld != rows) NNV_HIP_TRY(hipMemsetAsync(dev, 0, sizeof(double) * ld * cols, c->stream));
+  NNV_HIP_TRY(hipMemcpy2DAsync(dev, sizeof(double) * ld, host, sizeof(double) * rows, sizeof(double) * rows,
+                               cols, hipMemcpyHostToDevice, c->stream));
+  // the source is pageable caller memory: finish before returning
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_create(nnvhip_ctx* c, int64_t N, int64_t n, const double* V, const double* pred_lb,
+                       const double* pred_ub, const double* C, const double* d, int64_t p,
+                       nnvhip_star** out) {
+  CHECK_CTX(c);
+  if (!out || !V) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  if (N <= 0 || n < 0 || p < 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "invalid set size N=%lld n=%lld p=%lld", (long long)N, (long long)n, (long long)p);
+  if ((pred_lb == nullptr) != (pred_ub == nullptr))
+    NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistency between number of predicate variables and predicate lower- or upper-bounds vector");
+  if (p > 0 && (!C || !d)) NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistency between constraint matrix and constraint vector");
+  nnvhip_star* s = new_star(c);
+  std::unique_ptr<nnvhip_star, int (*)(nnvhip_star*)> guard(s, nnvhip_star_release);
+  s->N = N;
+  s->n = n;
+  s->ld = round_up(N, kLdAlign);
+  NNV_TRY(c->alloc(sizeof(double) * s->ld * (n + 1), &s->Vbuf));
+  s->V = s->Vbuf->as<double>();
+  NNV_TRY(upload_matrix(c, V, N, n + 1, s->ld, s->V));
+  int64_t npad = round_up(std::max<int64_t>(n, 1), kLdAlign);
+  NNV_TRY(c->alloc(sizeof(double) * 2 * npad, &s->pbuf));
+  s->plb = s->pbuf->as<double>();
+  s->pub = s->plb + npad;
+  if (n > 0) {
+    std::vector<double> tmp(2 * npad, 0.0);
+    for (int64_t i = 0; i < n; ++i) {
+      tmp[i] = pred_lb ? pred_lb[i] : -1.0;  // default of Star.estimateRanges, set/Star.m:1091-1096
+      tmp[npad + i] = pred_ub ? pred_ub[i] : 1.0;
+    }
+    NNV_HIP_TRY(hipMemcpyAsync(s->plb, tmp.data(), sizeof(double) * 2 * npad, hipMemcpyHostToDevice, c->stream));
+    NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  }
+  auto base = std::make_shared<ConsNode>();
+  base->p_total = p;
+  base->n_total = n;
+  if (p > 0 && n > 0) {
+    base->ldc = round_up(p, kLdAlign);
+    NNV_TRY(c->alloc(sizeof(double) * base->ldc * n, &base->C0));
+    NNV_TRY(upload_matrix(c, C, p, n, base->ldc, base->C0->as<double>()));
+  }
+  if (p > 0) {
+    NNV_TRY(c->alloc(sizeof(double) * p, &base->d0));
+    NNV_HIP_TRY(hipMemcpyAsync(base->d0->ptr, d, sizeof(double) * p, hipMemcpyHostToDevice, c->stream));
+    NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  }
+  s->cons = base;
+  *out = guard.release();
+  return NNVHIP_OK;
+}
+
+__global__ void box_fill_kernel(double* __restrict__ V, int64_t ld, int N, const double* __restrict__ center,
+                                const double* __restrict__ vec, const int32_t* __restrict__ gen_dim,
+                                const int64_t* __restrict__ col_off, const int64_t* __restrict__ gen_off) {
+  // one block column per (set, column); rows across threads.  Column 0 is the centre; column
+  // 1+g holds vec(dim_g) at row dim_g and zeros elsewhere (diag(vec) with empty columns removed).
+  int set = blockIdx.z;
+  int64_t ncols = col_off[set + 1] - col_off[set];
+  for (int64_t j = blockIdx.y; j < ncols; j += gridDim.y) {
+    double* col = V + (col_off[set] + j) * ld;
+    int dim = j == 0 ? -1 : gen_dim[gen_off[set] + j - 1];
+    for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < ld; r += gridDim.x * blockDim.x) {
+      double v = 0.0;
+      if (r < N) {
+        if (j == 0) v = center[(int64_t)set * N + r];
+        else if (r == dim) v = vec[(int64_t)set * N + r];
+      }
+      col[r] = v;
+    }
+  }
+}
+
+__global__ void fill_pm_one_kernel(double* __restrict__ plb, double* __restrict__ pub, int64_t n) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i < n) {
+    plb[i] = -1.0;
+    pub[i] = 1.0;
+  }
+}
+
+int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* lb, const double* ub,
+                         nnvhip_star** out) {
+  CHECK_CTX(c);
+  if (!lb || !ub || !out) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  if (N <= 0 || count <= 0 || count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistent dimensions between lb and ub");
+  // Box constructor arithmetic on the host (set/Box.m:35-45): it decides the column count.
+  std::vector<double> center(N * count), vec(N * count);
+  std::vector<int32_t> gen_dim;
+  std::vector<int64_t> col_off(count + 1, 0), gen_off(count + 1, 0);
+  for (int64_t s = 0; s < count; ++s) {
+    int64_t n = 0;
+    for (int64_t i = 0; i < N; ++i) {
+      double l = lb[s * N + i], u = ub[s * N + i];
+      center[s * N + i] = 0.5 * (l + u);
+      double v = 0.5 * (u - l);
+      vec[s * N + i] = v;
+      // zero columns are deleted only when the generator matrix has more than one element
+      if (v != 0.0 || N == 1) {
+        gen_dim.push_back((int32_t)i);
+        ++n;
+      }
+    }
+    gen_off[s + 1] = gen_off[s] + n;
+    col_off[s + 1] = col_off[s] + n + 1;
+  }
+  int64_t ld = round_up(N, kLdAlign);
+  int64_t total_cols = col_off[count];
+  BufRef arena, dcenter, dvec, dgen, dcol, dgoff;
+  NNV_TRY(c->alloc(sizeof(double) * ld * total_cols, &arena));
+  NNV_TRY(c->upload(center.data(), sizeof(double) * center.size(), &dcenter));
+  NNV_TRY(c->upload(vec.data(), sizeof(double) * vec.size(), &dvec));
+  if (gen_dim.empty()) gen_dim.push_back(0);
+  NNV_TRY(c->upload(gen_dim.data(), sizeof(int32_t) * gen_dim.size(), &dgen));
+  NNV_TRY(c->upload(col_off.data(), sizeof(int64_t) * col_off.size(), &dcol));
+  NNV_TRY(c->upload(gen_off.data(), sizeof(int64_t) * gen_off.size(), &dgoff));
+  int64_t max_cols = 0;
+  for (int64_t s = 0; s < count; ++s) max_cols = std::max(max_cols, col_off[s + 1] - col_off[s]);
+  dim3 grid((unsigned)std::min<int64_t>(ceil_div(ld, 256), 64), (unsigned)std::min<int64_t>(max_cols, 4096),
+            (unsigned)count);
+  hipLaunchKernelGGL(box_fill_kernel, grid, dim3(256), 0, c->stream, arena->as<double>(), ld, (int)N,
+                     dcenter->as<double>(), dvec->as<double>(), dgen->as<int32_t>(), dcol->as<int64_t>(),
+                     dgoff->as<int64_t>());
+  NNV_HIP_TRY(hipGetLastError());
+  // predicate bounds -1/+1 for all sets in one buffer
+  int64_t npad_total = 0;
+  std::vector<int64_t> poff(count);
+  for (int64_t s = 0; s < count; ++s) {
+    poff[s] = npad_total;
+    npad_total += 2 * round_up(std::max<int64_t>(gen_off[s + 1] - gen_off[s], 1), kLdAlign);
+  }
+  BufRef pb;
+  NNV_TRY(c->alloc(sizeof(double) * npad_total, &pb));
+  for (int64_t s = 0; s < count; ++s) {
+    nnvhip_star* st = new_star(c);
+    st->N = N;
+    st->n = gen_off[s + 1] - gen_off[s];
+    st->ld = ld;
+    st->Vbuf = arena;
+    st->V = arena->as<double>() + col_off[s] * ld;
+    st->pbuf = pb;
+    int64_t npad = round_up(std::max<int64_t>(st->n, 1), kLdAlign);
+    st->plb = pb->as<double>() + poff[s];
+    st->pub = st->plb + npad;
+    // C = zeros(1, n), d = 0 (set/Star.m:226-227): a base node with one all-zero row
+    auto base = std::make_shared<ConsNode>();
+    base->p_total = 1;
+    base->n_total = st->n;
+    st->cons = base;  // C0/d0 left null = all zeros
+    out[s] = st;
+  }
+  // one launch fills every set's bounds: lb half gets -1, ub half +1
+  for (int64_t s = 0; s < count; ++s) {
+    int64_t npad = round_up(std::max<int64_t>(out[s]->n, 1), kLdAlign);
+    hipLaunchKernelGGL(fill_pm_one_kernel, dim3((unsigned)ceil_div(npad, 256)), dim3(256), 0, c->stream,
+                       out[s]->plb, out[s]->pub, npad);
+  }
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_retain(nnvhip_star* s) {
+  if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
+  s->refs.fetch_add(1);
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_release(nnvhip_star* s) {
+  if (!s) return NNVHIP_OK;
+  if (s->refs.fetch_sub(1) == 1) {
+    nnvhip_ctx* c = s->ctx;
+    delete s;
+    c->live_handles--;
+  }
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p) {
+  if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
+  if (N) *N = s->N;
+  if (n) *n = s->n;
+  if (p) *p = s->cons ? s->cons->p_total : 0;
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_fetch_V(const nnvhip_star* s, double* V) {
+  if (!s || !V) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  nnvhip_ctx* c = s->ctx;
+  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_HIP_TRY(hipMemcpy2DAsync(V, sizeof(double) * s->N, s->V, sizeof(double) * s->ld, sizeof(double) * s->N,
+                               s->n + 1, hipMemcpyDeviceToHost, c->stream));
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* lb, double* ub) {
+  if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
+  nnvhip_ctx* c = s->ctx;
+  NNV_HIP_TRY(hipSetDevice(c->device));
+  if (s->n > 0) {
+    if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb, s->plb, sizeof(double) * s->n, hipMemcpyDeviceToHost, c->stream));
+    if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub, s->pub, sizeof(double) * s->n, hipMemcpyDeviceToHost, c->stream));
+  }
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_fetch_constraints(const nnvhip_star* s, double* C, double* d) {
+  if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
+  NNV_HIP_TRY(hipSetDevice(s->ctx->device));
+  return materialize_constraints(s, C, d);
+}
+
+int nnvhip_star_relu_counts(const nnvhip_star* s, int64_t* n_inactive, int64_t* n_crossing) {
+  if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
+  if (s->n_crossing < 0) NNV_FAIL(NNVHIP_ERR_ARG, "set was not produced by the ReLU step");
+  if (n_inactive) *n_inactive = s->n_inactive;
+  if (n_crossing) *n_crossing = s->n_crossing;
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb, double* ub) {
+  if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
+  if (s->n_crossing < 0) NNV_FAIL(NNVHIP_ERR_ARG, "set was not produced by the ReLU step");
+  nnvhip_ctx* c = s->ctx;
+  NNV_HIP_TRY(hipSetDevice(c->device));
+  const ConsNode* node = s->cons.get();
+  int64_t m = s->n_crossing;
+  if (m > 0) {
+    if (index) NNV_HIP_TRY(hipMemcpyAsync(index, node->index->ptr, sizeof(int32_t) * m, hipMemcpyDeviceToHost, c->stream));
+    const double* lbub = node->lbub->as<double>() + node->lbub_off;
+    if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb, lbub, sizeof(double) * m, hipMemcpyDeviceToHost, c->stream));
+    if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub, lbub + node->ld_rows, sizeof(double) * m, hipMemcpyDeviceToHost, c->stream));
+  }
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_estimate_ranges(nnvhip_ctx* c, nnvhip_star* s, double* lb, double* ub) {
+  return nnvhip_estimate_ranges_batch(c, 1, &s, lb, ub);
+}
+
+int nnvhip_estimate_ranges_batch(nnvhip_ctx* c, int64_t count, nnvhip_star* const* s, double* lb, double* ub) {
+  CHECK_CTX(c);
+  if (!s || count <= 0) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  for (int64_t i = 0; i < count; ++i) {
+    if (!s[i] || s[i]->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid set handle %lld", (long long)i);
+    if (s[i]->N != s[0]->N) NNV_FAIL(NNVHIP_ERR_SHAPE, "sets of one array must have the same dimension");
+  }
+  NNV_TRY(c->begin_op());
+  NNV_TRY(compute_ranges(c, count, s));
+  NNV_TRY(c->end_op());
+  if (lb || ub) {
+    int64_t N = s[0]->N;
+    for (int64_t i = 0; i < count; ++i) {
+      if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb + i * N, s[i]->lb, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
+      if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub + i * N, s[i]->ub, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
+    }
+    NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  }
+  return NNVHIP_OK;
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* layers                                                                                      */
+/* ------------------------------------------------------------------------------------------ */
+
+int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M, int64_t K, nnvhip_fc** out) {
+  CHECK_CTX(c);
+  if (!W || !out) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  if (M <= 0 || K <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistent dimension between the weight matrix and bias vector");
+  std::unique_ptr<nnvhip_fc> fc(new nnvhip_fc());
+  fc->ctx = c;
+  fc->M = M;
+  fc->K = K;
+  fc->Mp = round_up(M, kLdAlign);
+  fc->Kp = round_up(K, kLdAlign);
+  NNV_TRY(c->alloc(sizeof(double) * fc->Mp * fc->Kp, &fc->W));
+  NNV_HIP_TRY(hipMemsetAsync(fc->W->ptr, 0, sizeof(double) * fc->Mp * fc->Kp, c->stream));
+  NNV_HIP_TRY(hipMemcpy2DAsync(fc->W->ptr, sizeof(double) * fc->Mp, W, sizeof(double) * M, sizeof(double) * M, K,
+                               hipMemcpyHostToDevice, c->stream));
+  if (b) {
+    NNV_TRY(c->alloc(sizeof(double) * fc->Mp, &fc->bias));
+    NNV_HIP_TRY(hipMemsetAsync(fc->bias->ptr, 0, sizeof(double) * fc->Mp, c->stream));
+    NNV_HIP_TRY(hipMemcpyAsync(fc->bias->ptr, b, sizeof(double) * M, hipMemcpyHostToDevice, c->stream));
+  }
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  c->live_handles++;
+  *out = fc.release();
+  return NNVHIP_OK;
+}
+
+int nnvhip_fc_destroy(nnvhip_fc* fc) {
+  if (!fc) return NNVHIP_OK;
+  nnvhip_ctx* c = fc->ctx;
+  delete fc;
+  c->live_handles--;
+  return NNVHIP_OK;
+}
+
+int nnvhip_conv2d_create(nnvhip_ctx* c, const double* W, const double* bias, int64_t FH, int64_t FW, int64_t Cin,
+                         int64_t Cout, const int64_t padding[4], const int64_t stride[2], const int64_t dilation[2],
+                         nnvhip_conv2d** out) {
+  CHECK_CTX(c);
+  if (!W || !out || !padding || !stride || !dilation) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  if (FH <= 0 || FW <= 0 || Cin <= 0 || Cout <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Invalid weights array");
+  for (int i = 0; i < 4; ++i)
+    if (padding[i] < 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Invalid padding matrix");
+  if (stride[0] <= 0 || stride[1] <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Invalid stride matrix");
+  if (dilation[0] <= 0 || dilation[1] <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Invalid dilation matrix");
+  std::unique_ptr<nnvhip_conv2d> cv(new nnvhip_conv2d());
+  cv->ctx = c;
+  cv->FH = FH;
+  cv->FW = FW;
+  cv->Cin = Cin;
+  cv->Cout = Cout;
+  for (int i = 0; i < 4; ++i) cv->pad[i] = padding[i];
+  for (int i = 0; i < 2; ++i) {
+    cv->stride[i] = stride[i];
+    cv->dil[i] = dilation[i];
+  }
+  cv->K = FH * FW * Cin;
+  cv->Kp = round_up(cv->K, kLdAlign);
+  // MATLAB's FH x FW x Cin x Cout array is a (FH*FW*Cin) x Cout column-major matrix already
+  NNV_TRY(c->alloc(sizeof(double) * cv->Kp * Cout, &cv->W));
+  NNV_HIP_TRY(hipMemsetAsync(cv->W->ptr, 0, sizeof(double) * cv->Kp * Cout, c->stream));
+  NNV_HIP_TRY(hipMemcpy2DAsync(cv->W->ptr, sizeof(double) * cv->Kp, W, sizeof(double) * cv->K, sizeof(double) * cv->K,
+                               Cout, hipMemcpyHostToDevice, c->stream));
+  if (bias) {
+    NNV_TRY(c->alloc(sizeof(double) * Cout, &cv->bias));
+    NNV_HIP_TRY(hipMemcpyAsync(cv->bias->ptr, bias, sizeof(double) * Cout, hipMemcpyHostToDevice, c->stream));
+  }
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  c->live_handles++;
+  *out = cv.release();
+  return NNVHIP_OK;
+}
+
+int nnvhip_conv2d_destroy(nnvhip_conv2d* cv) {
+  if (!cv) return NNVHIP_OK;
+  nnvhip_ctx* c = cv->ctx;
+  delete cv;
+  c->live_handles--;
+  return NNVHIP_OK;
+}
+
+int nnvhip_conv2d_output_size(const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t* Ho, int64_t* Wo) {
+  if (!cv) NNV_FAIL(NNVHIP_ERR_ARG, "null layer handle");
+  // floor((H + t + b - (FH-1)*dh - 1)/sh + 1), nn/layers/Conv2DLayer.m:1134-1135
+  int64_t eh = H + cv->pad[0] + cv->pad[1] - (cv->FH - 1) * cv->dil[0] - 1;
+  int64_t ew = W + cv->pad[2] + cv->pad[3] - (cv->FW - 1) * cv->dil[1] - 1;
+  if (eh < 0 || ew < 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "filter does not fit the padded input");
+  if (Ho) *Ho = eh / cv->stride[0] + 1;
+  if (Wo) *Wo = ew / cv->stride[1] + 1;
+  return NNVHIP_OK;
+}
+
+// Shared set-up of the affine layers: validates the input array, allocates one output arena with
+// the sets back to back, and creates output handles that share constraints and predicate bounds
+// with their inputs.
+static int make_affine_outputs(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, int64_t Nout,
+                               std::vector<nnvhip_star*>* outs, bool* contiguous, int64_t* total_cols) {
+  int64_t ldout = round_up(Nout, kLdAlign);
+  int64_t cols = 0;
+  bool contig = true;
+  for (int64_t i = 0; i < count; ++i) {
+    if (i > 0 && (in[i]->ld != in[0]->ld || in[i]->V != in[i - 1]->V + (in[i - 1]->n + 1) * in[i - 1]->ld)) contig = false;
+    cols += in[i]->n + 1;
+  }
+  BufRef arena;
+  NNV_TRY(c->alloc(sizeof(double) * ldout * cols, &arena));
+  int64_t off = 0;
+  for (int64_t i = 0; i < count; ++i) {
+    nnvhip_star* o = new_star(c);
+    o->N = Nout;
+    o->n = in[i]->n;
+    o->ld = ldout;
+    o->Vbuf = arena;
+    o->V = arena->as<double>() + off * ldout;
+    o->pbuf = in[i]->pbuf;
+    o->plb = in[i]->plb;
+    o->pub = in[i]->pub;
+    o->cons = in[i]->cons;
+    off += in[i]->n + 1;
+    outs->push_back(o);
+  }
+  *contiguous = contig;
+  *total_cols = cols;
+  return NNVHIP_OK;
+}
+
+static void release_all(std::vector<nnvhip_star*>& v) {
+  for (auto* s : v) nnvhip_star_release(s);
+  v.clear();
+}
+
+static int check_set_array(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
+  if (!in || !out || count <= 0) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  for (int64_t i = 0; i < count; ++i)
+    if (!in[i] || in[i]->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid set handle %lld", (long long)i);
+  return NNVHIP_OK;
+}
+
+int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
+  CHECK_CTX(c);
+  if (!fc || fc->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid layer handle");
+  NNV_TRY(check_set_array(c, count, in, out));
+  for (int64_t i = 0; i < count; ++i)
+    if (in[i]->N != fc->K)
+      NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistency between the affine mapping matrix and dimension of the star set");
+  std::vector<nnvhip_star*> outs;
+  bool contig = false;
+  int64_t cols = 0;
+  NNV_TRY(c->begin_op());
+  int st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
+  if (st == NNVHIP_OK) {
+    const double* bias = fc->bias ? fc->bias->as<double>() : nullptr;
+    if (contig) {
+      st = launch_gemm(c, fc->W->as<double>(), fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols,
+                       fc->Kp, bias);
+      if (st == NNVHIP_OK && bias && count > 1) {
+        std::vector<double*> centres(count - 1);
+        for (int64_t i = 1; i < count; ++i) centres[i - 1] = outs[i]->V;
+        BufRef tab;
+        st = c->upload(centres.data(), sizeof(double*) * centres.size(), &tab);
+        if (st == NNVHIP_OK) st = launch_bias_columns(c, tab->as<double*>(), count - 1, bias, fc->Mp);
+      }
+    } else {
+      for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+        st = launch_gemm(c, fc->W->as<double>(), fc->Mp, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, fc->Mp,
+                         in[i]->n + 1, fc->Kp, bias);
+    }
+  }
+  if (st == NNVHIP_OK) st = c->end_op();
+  if (st != NNVHIP_OK) {
+    release_all(outs);
+    return st;
+  }
+  for (int64_t i = 0; i < count; ++i) out[i] = outs[i];
+  return NNVHIP_OK;
+}
+
+int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t count,
+                         nnvhip_star* const* in, nnvhip_star** out) {
+  CHECK_CTX(c);
+  if (!cv || cv->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid layer handle");
+  NNV_TRY(check_set_array(c, count, in, out));
+  if (H <= 0 || W <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "The input is not an ImageStar object");
+  for (int64_t i = 0; i < count; ++i) {
+    if (in[i]->N % (H * W) != 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistent dimension in the ImageStar and the original Star set");
+    int64_t ch = in[i]->N / (H * W);
+    if (ch != cv->Cin)
+      NNV_FAIL(NNVHIP_ERR_SHAPE, "Input set contains %lld channels while the convolutional layers has %lld channels",
+               (long long)ch, (long long)cv->Cin);
+  }
+  int64_t Ho = 0, Wo = 0;
+  NNV_TRY(nnvhip_conv2d_output_size(cv, H, W, &Ho, &Wo));
+  int64_t Nout = Ho * Wo * cv->Cout;
+  if (Nout >= (int64_t(1) << 31) || in[0]->N >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "image too large");
+  std::vector<nnvhip_star*> outs;
+  bool contig = false;
+  int64_t cols = 0;
+  NNV_TRY(c->begin_op());
+  int st = make_affine_outputs(c, count, in, Nout, &outs, &contig, &cols);
+  for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+    st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, in[i]->n + 1, nullptr);
+  if (st == NNVHIP_OK) st = c->end_op();
+  if (st != NNVHIP_OK) {
+    release_all(outs);
+    return st;
+  }
+  for (int64_t i = 0; i < count; ++i) out[i] = outs[i];
+  return NNVHIP_OK;
+}
+
+int nnvhip_relu_relax(nnvhip_ctx* c, int order, double relax_factor, int64_t count, nnvhip_star* const* in,
+                      nnvhip_star** out) {
+  CHECK_CTX(c);
+  NNV_TRY(check_set_array(c, count, in, out));
+  if (order != NNVHIP_ORDER_INDEX && order != NNVHIP_ORDER_AREA && order != NNVHIP_ORDER_RANGE)
+    NNV_FAIL(NNVHIP_ERR_METHOD, "This reachability method does not exist");
+  if (!(relax_factor >= 0.0 && relax_factor <= 1.0)) NNV_FAIL(NNVHIP_ERR_RELAX_FACTOR, "Invalid relax factor");
+  if (relax_factor != 1.0)
+    NNV_FAIL(NNVHIP_ERR_RELAX_FACTOR, "relaxFactor < 1 needs the LP-based range optimisation, which this library does not provide");
+  for (int64_t i = 0; i < count; ++i)
+    if (in[i]->N != in[0]->N) NNV_FAIL(NNVHIP_ERR_SHAPE, "sets of one array must have the same dimension");
+  NNV_TRY(c->begin_op());
+  NNV_TRY(relu_relax(c, order, count, in, out));
+  return c->end_op();
+}
+
+}  // extern "C"

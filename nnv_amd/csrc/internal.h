@@ -1,0 +1,175 @@
+// Internal definitions shared by the translation units of libnnvhip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "nnvhip.h"
+
+namespace nnvhip {
+
+// Leading dimensions of every device matrix are multiples of 16 doubles (one 128-byte line), and
+// the padding rows [N, ld) of every generator matrix are kept at exactly zero, so kernels may
+// read whole 16-row groups and the GEMM K loop needs no tail handling.
+constexpr int64_t kLdAlign = 16;
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+inline int64_t ceil_div(int64_t x, int64_t m) { return (x + m - 1) / m; }
+
+void set_error(const char* fmt, ...);
+
+#define NNV_HIP_TRY(expr)                                                                       \
+  do {                                                                                          \
+    hipError_t e_ = (expr);                                                                     \
+    if (e_ != hipSuccess) {                                                                     \
+      ::nnvhip::set_error("HIP error '%s' at %s:%d in %s", hipGetErrorString(e_), __FILE__,     \
+                          __LINE__, #expr);                                                     \
+      return e_ == hipErrorOutOfMemory ? NNVHIP_ERR_OOM : NNVHIP_ERR_HIP;                       \
+    }                                                                                           \
+  } while (0)
+
+#define NNV_TRY(expr)                 \
+  do {                                \
+    int s_ = (expr);                  \
+    if (s_ != NNVHIP_OK) return s_;   \
+  } while (0)
+
+#define NNV_FAIL(code, ...)             \
+  do {                                  \
+    ::nnvhip::set_error(__VA_ARGS__);   \
+    return (code);                      \
+  } while (0)
+
+struct Buffer {
+  nnvhip_ctx* ctx = nullptr;
+  void* ptr = nullptr;
+  size_t bytes = 0;  // size class the block belongs to
+  ~Buffer();
+  template <class T>
+  T* as() const { return static_cast<T*>(ptr); }
+};
+using BufRef = std::shared_ptr<Buffer>;
+
+// One node per ReLU layer of the structured constraint store.  The dense NNV matrix
+// [C0; C1; C2; C3] (nn/funcs/PosLin.m:711-735) is only materialised when the host reads it.
+struct ConsNode {
+  std::shared_ptr<ConsNode> prev;  // null for the base node
+  int64_t p_total = 0;             // constraint rows up to and including this node
+  int64_t n_total = 0;             // predicate variables up to and including this node
+  // base node: dense C0 (p_total x n_total, ld = ldc) and d0
+  BufRef C0;
+  int64_t ldc = 0;
+  BufRef d0;
+  // ReLU node: the m crossing rows of the pre-ReLU [c V] (m x (n_before+1), ld = ld_rows), in
+  // new-predicate order, their bounds and neuron indices
+  int64_t m = 0;
+  int64_t n_before = 0;
+  BufRef rows;            // possibly shared by the sets of one array: data starts at rows_off
+  int64_t rows_off = 0;   // element offset into rows
+  int64_t ld_rows = 0;
+  BufRef lbub;            // lb[0..m), then ub[0..m) at offset ld_rows; data starts at lbub_off
+  int64_t lbub_off = 0;
+  BufRef index;           // int32[m]
+};
+using ConsRef = std::shared_ptr<ConsNode>;
+
+}  // namespace nnvhip
+
+struct nnvhip_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  // size-class caching pool
+  std::multimap<size_t, void*> free_blocks;
+  int64_t bytes_in_use = 0;
+  int64_t bytes_cached = 0;
+  int64_t live_handles = 0;
+  // pinned staging ring for descriptor tables and small read-backs
+  char* pinned = nullptr;
+  size_t pinned_bytes = 0;
+  size_t pinned_off = 0;
+  // per-layer timing
+  bool timing = false;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  double last_ms = 0.0;
+
+  int alloc(size_t bytes, nnvhip::BufRef* out);
+  void release_block(void* p, size_t bytes);
+  int trim();
+  // Returns host-pinned scratch of `bytes`; waits for the stream when the ring wraps.
+  int stage(size_t bytes, void** host);
+  // Copies a host table to a fresh device buffer through the pinned ring (async on the stream).
+  int upload(const void* host, size_t bytes, nnvhip::BufRef* out);
+  int begin_op();
+  int end_op();
+};
+
+struct nnvhip_star {
+  std::atomic<int> refs{1};
+  nnvhip_ctx* ctx = nullptr;
+  int64_t N = 0;   // dim
+  int64_t n = 0;   // nVar
+  int64_t ld = 0;  // leading dimension of V (multiple of 16, >= N)
+  nnvhip::BufRef Vbuf;
+  double* V = nullptr;  // N x (n+1), may point inside a shared arena
+  nnvhip::BufRef pbuf;
+  double* plb = nullptr;
+  double* pub = nullptr;
+  nnvhip::ConsRef cons;
+  // cached estimateRanges result
+  nnvhip::BufRef rbuf;
+  double* lb = nullptr;
+  double* ub = nullptr;
+  // filled for sets produced by the ReLU step
+  int64_t n_inactive = -1;
+  int64_t n_crossing = -1;
+};
+
+struct nnvhip_fc {
+  nnvhip_ctx* ctx = nullptr;
+  int64_t M = 0, K = 0, Mp = 0, Kp = 0;
+  nnvhip::BufRef W;     // Mp x Kp, zero padded, ld = Mp
+  nnvhip::BufRef bias;  // Mp entries (zero padded) or null
+};
+
+struct nnvhip_conv2d {
+  nnvhip_ctx* ctx = nullptr;
+  int64_t FH = 0, FW = 0, Cin = 0, Cout = 0;
+  int64_t pad[4] = {0, 0, 0, 0}, stride[2] = {1, 1}, dil[2] = {1, 1};
+  int64_t K = 0, Kp = 0;  // K = FH*FW*Cin taps, Kp = padded
+  nnvhip::BufRef W;       // Kp x Cout, zero padded rows, ld = Kp (MATLAB layout is already K x Cout)
+  nnvhip::BufRef bias;    // Cout entries or null
+};
+
+namespace nnvhip {
+
+nnvhip_star* new_star(nnvhip_ctx* ctx);
+
+// gemm.hip: C(Mp x ncols, ldc) = A(Mp x Kp, lda) * B(Kp x ncols, ldb); bias (Mp) is added to
+// column 0 when non-null.  Mp, Kp multiples of 16; padding rows of A and B are zero.
+int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
+                int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias);
+// Adds bias to the centre columns of sets 1..count-1 of an arena (set 0 is fused in the GEMM).
+int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t count, const double* bias,
+                        int64_t Mp);
+
+// conv.hip
+int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                  const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
+                  const int32_t* centre_flags /* per column: 1 = add bias */);
+
+// ranges.hip
+int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s);
+
+// relu.hip
+int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out);
+int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host);
+
+}  // namespace nnvhip

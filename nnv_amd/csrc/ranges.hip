@@ -1,0 +1,176 @@
+// Star.estimateRanges (set/Star.m:1078-1106) as one coalesced pass over V.
+//
+// V is column-major, so consecutive lanes own consecutive rows: every wave reads 1 KiB lines down a
+// column (two rows per lane).  The four waves of a block interleave the columns of the block's
+// column chunk; partial sums of the chunks are combined in a fixed order by a second tiny kernel,
+// so results are bit-reproducible from run to run (no floating-point atomics).
+#include <algorithm>
+
+#include "internal.h"
+
+namespace nnvhip {
+
+struct RangeDesc {
+  const double* V;    // N x (n+1), column 0 = centre
+  const double* plb;  // n
+  const double* pub;  // n
+  double* part;       // [chunks][4][ld] partial sums (unused when chunks == 1)
+  double* lb;         // ld
+  double* ub;         // ld
+  int64_t ld;
+  int32_t n;
+  int32_t chunks;
+  int32_t cols_per_chunk;
+  int32_t pad_;
+};
+
+constexpr int kRowsPerBlock = 128;  // 64 lanes x 2 rows
+
+__global__ __launch_bounds__(256) void ranges_partial_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
+  const RangeDesc d = table ? table[blockIdx.z] : one;
+  const int chunk = blockIdx.y;
+  if (chunk >= d.chunks) return;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t r0 = (int64_t)blockIdx.x * kRowsPerBlock + 2 * lane;
+  const bool active = r0 < d.ld;
+  // generator columns are 1..n; chunk c owns [1 + c*cpc, min(n, (c+1)*cpc) + 1)
+  const int j0 = 1 + chunk * d.cols_per_chunk;
+  const int j1 = min(d.n, (chunk + 1) * d.cols_per_chunk) + 1;
+  double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
+  if (active) {
+    const double* col = d.V + r0;
+#pragma unroll 4
+    for (int j = j0 + wave; j < j1; j += 4) {
+      const double2 v = *reinterpret_cast<const double2*>(col + (int64_t)j * d.ld);
+      const double pl = d.plb[j - 1];
+      const double pu = d.pub[j - 1];
+      const double px = fmax(v.x, 0.0), nx = fmin(v.x, 0.0);
+      const double py = fmax(v.y, 0.0), ny = fmin(v.y, 0.0);
+      xmin1.x = fma(px, pl, xmin1.x);
+      xmin1.y = fma(py, pl, xmin1.y);
+      xmax1.x = fma(px, pu, xmax1.x);
+      xmax1.y = fma(py, pu, xmax1.y);
+      xmin2.x = fma(nx, pu, xmin2.x);
+      xmin2.y = fma(ny, pu, xmin2.y);
+      xmax2.x = fma(nx, pl, xmax2.x);
+      xmax2.y = fma(ny, pl, xmax2.y);
+    }
+  }
+  __shared__ double2 red[3][4][64];
+  if (wave > 0) {
+    red[wave - 1][0][lane] = xmin1;
+    red[wave - 1][1][lane] = xmin2;
+    red[wave - 1][2][lane] = xmax1;
+    red[wave - 1][3][lane] = xmax2;
+  }
+  __syncthreads();
+  if (wave == 0 && active) {
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+      xmin1.x += red[w][0][lane].x;
+      xmin1.y += red[w][0][lane].y;
+      xmin2.x += red[w][1][lane].x;
+      xmin2.y += red[w][1][lane].y;
+      xmax1.x += red[w][2][lane].x;
+      xmax1.y += red[w][2][lane].y;
+      xmax2.x += red[w][3][lane].x;
+      xmax2.y += red[w][3][lane].y;
+    }
+    if (d.chunks == 1) {
+      // lb = (c + xmin1) + xmin2, the reference's left-to-right order
+      const double2 c = *reinterpret_cast<const double2*>(d.V + r0);
+      *reinterpret_cast<double2*>(d.lb + r0) = make_double2((c.x + xmin1.x) + xmin2.x, (c.y + xmin1.y) + xmin2.y);
+      *reinterpret_cast<double2*>(d.ub + r0) = make_double2((c.x + xmax1.x) + xmax2.x, (c.y + xmax1.y) + xmax2.y);
+    } else {
+      double* p = d.part + ((int64_t)chunk * 4) * d.ld + r0;
+      *reinterpret_cast<double2*>(p) = xmin1;
+      *reinterpret_cast<double2*>(p + d.ld) = xmin2;
+      *reinterpret_cast<double2*>(p + 2 * d.ld) = xmax1;
+      *reinterpret_cast<double2*>(p + 3 * d.ld) = xmax2;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
+  const RangeDesc d = table ? table[blockIdx.z] : one;
+  if (d.chunks == 1) return;
+  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= d.ld) return;
+  double s[4] = {0, 0, 0, 0};
+  for (int c = 0; c < d.chunks; ++c) {
+    const double* p = d.part + ((int64_t)c * 4) * d.ld + r;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) s[q] += p[q * d.ld];
+  }
+  const double c0 = d.V[r];
+  d.lb[r] = (c0 + s[0]) + s[1];
+  d.ub[r] = (c0 + s[2]) + s[3];
+}
+
+int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
+  // sets that already carry ranges are skipped
+  std::vector<nnvhip_star*> todo;
+  for (int64_t i = 0; i < count; ++i)
+    if (!s[i]->lb) {
+      bool dup = false;
+      for (auto* t : todo) dup = dup || t == s[i];
+      if (!dup) todo.push_back(s[i]);
+    }
+  if (todo.empty()) return NNVHIP_OK;
+  const int64_t nset = (int64_t)todo.size();
+  if (nset > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  int64_t ld = todo[0]->ld;
+  int64_t nmax = 0;
+  for (auto* t : todo) {
+    if (t->ld != ld) NNV_FAIL(NNVHIP_ERR_SHAPE, "sets of one array must have the same dimension");
+    nmax = std::max(nmax, t->n);
+  }
+  // Column chunking: enough blocks to cover the chip a few times over, at least 64 columns per
+  // chunk so the partial-sum traffic stays below ~6 % of V.
+  const int64_t row_blocks = ceil_div(ld, kRowsPerBlock);
+  const int64_t want_blocks = 2048;
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * nset), ceil_div(nmax, 64)));
+  chunks = std::min<int64_t>(chunks, 1024);
+  // one buffer for all lb/ub, one for all partials
+  BufRef rb, pb;
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * ld * nset, &rb));
+  if (chunks > 1) NNV_TRY(ctx->alloc(sizeof(double) * 4 * ld * chunks * nset, &pb));
+  std::vector<RangeDesc> descs(nset);
+  for (int64_t i = 0; i < nset; ++i) {
+    nnvhip_star* t = todo[i];
+    RangeDesc& d = descs[i];
+    d.V = t->V;
+    d.plb = t->plb;
+    d.pub = t->pub;
+    d.ld = ld;
+    d.n = (int32_t)t->n;
+    int64_t ch = std::max<int64_t>(1, std::min<int64_t>(chunks, ceil_div(t->n, 64)));
+    d.chunks = (int32_t)ch;
+    d.cols_per_chunk = (int32_t)std::max<int64_t>(1, ceil_div(t->n, ch));
+    d.part = pb ? pb->as<double>() + 4 * ld * chunks * i : nullptr;
+    d.lb = rb->as<double>() + 2 * ld * i;
+    d.ub = d.lb + ld;
+    d.pad_ = 0;
+  }
+  const RangeDesc* table = nullptr;
+  BufRef tab;
+  if (nset > 1) {
+    NNV_TRY(ctx->upload(descs.data(), sizeof(RangeDesc) * nset, &tab));
+    table = tab->as<RangeDesc>();
+  }
+  dim3 grid((unsigned)row_blocks, (unsigned)chunks, (unsigned)nset);
+  hipLaunchKernelGGL(ranges_partial_kernel, grid, dim3(256), 0, ctx->stream, table, descs[0]);
+  if (chunks > 1)
+    hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 256), 1, (unsigned)nset), dim3(256), 0,
+                       ctx->stream, table, descs[0]);
+  NNV_HIP_TRY(hipGetLastError());
+  for (int64_t i = 0; i < nset; ++i) {
+    todo[i]->rbuf = rb;
+    todo[i]->lb = descs[i].lb;
+    todo[i]->ub = descs[i].ub;
+  }
+  return NNVHIP_OK;
+}
+
+}  // namespace nnvhip

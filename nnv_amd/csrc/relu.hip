@@ -1,0 +1,403 @@
+// The relax-star ReLU step at relaxFactor = 1 (nn/funcs/PosLin.m:863-1650, 685-742;
+// set/Star.m:1442-1461), entirely on the device:
+//   1. classify every neuron from its estimated range (inactive / crossing / active) and compact
+//      the crossing indices in ascending order with wavefront ballots + prefix sums;
+//   2. (area / range orders) rank the crossing neurons by a stable descending key sort;
+//   3. one pass over V: zero the inactive and crossing rows, save the crossing rows for the
+//      constraint store, append the one-hot columns and the new predicate bounds.
+// The dense constraint matrix is never built on this path; materialize_constraints() lays it out
+// exactly as the reference does when the host asks for it.
+#include <algorithm>
+
+#include "internal.h"
+
+namespace nnvhip {
+
+constexpr int kKeep = -1;  // active neuron (lb >= 0, ub > 0): row untouched
+constexpr int kZero = -2;  // inactive neuron (ub <= 0): row reset to 0
+
+struct ReluDesc {
+  const double* Vin;
+  double* Vout;
+  const double* lb;  // estimated ranges of the input set
+  const double* ub;
+  const double* plb_in;
+  const double* pub_in;
+  double* plb_out;
+  double* pub_out;
+  int32_t* cls;        // per row: kKeep, kZero or the crossing position (= new predicate number)
+  int32_t* cross_idx;  // crossing neuron indices in new-predicate order
+  int32_t* asc_idx;    // crossing neuron indices in ascending order (sort orders only)
+  double* key;         // sort keys, ascending-index order
+  int32_t* counts;     // [0] = m (crossing), [1] = inactive
+  double* rows;        // saved crossing rows of the pre-ReLU [c V]: m x ncols_in, ld = ld_rows
+  double* lbub;        // lb then ub (offset ld_rows) of the crossing neurons, new-predicate order
+  int64_t ld;
+  int64_t ld_rows;
+  int32_t N;
+  int32_t ncols_in;  // n + 1
+  int32_t m;
+  int32_t order;
+  int32_t cols_per_chunk;
+  int32_t pad_;
+};
+
+// One 1024-thread block per set.
+__global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.x] : one;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  __shared__ int wcross[16];
+  __shared__ int winact[16];
+  int base = 0, inact_total = 0;
+  int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
+  for (int r0 = 0; r0 < d.N; r0 += 1024) {
+    const int r = r0 + tid;
+    const bool valid = r < d.N;
+    const double l = valid ? d.lb[r] : 0.0;
+    const double u = valid ? d.ub[r] : 1.0;
+    const bool inactive = valid && (u <= 0.0);           // map1 = find(ub <= 0)
+    const bool crossing = valid && (l < 0.0) && (u > 0.0);  // map2 = find(lb < 0 & ub > 0)
+    const unsigned long long bc = __ballot(crossing);
+    const unsigned long long bi = __ballot(inactive);
+    if (lane == 0) {
+      wcross[wave] = __popcll(bc);
+      winact[wave] = __popcll(bi);
+    }
+    __syncthreads();
+    int woff = 0, tot = 0, itot = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int c = wcross[w];
+      woff += w < wave ? c : 0;
+      tot += c;
+      itot += winact[w];
+    }
+    if (crossing) {
+      const int pos = base + woff + __popcll(bc & ((1ull << lane) - 1ull));
+      idx_out[pos] = r;
+      if (d.order == NNVHIP_ORDER_INDEX) {
+        d.cls[r] = pos;
+      } else if (d.order == NNVHIP_ORDER_AREA) {
+        d.key[pos] = 0.5 * (fabs(u) * fabs(l));  // areas = 0.5*(abs(ub).*abs(lb))
+      } else {
+        d.key[pos] = u - l;  // ub - lb
+      }
+    } else if (valid) {
+      d.cls[r] = inactive ? kZero : kKeep;
+    }
+    base += tot;
+    inact_total += itot;
+    __syncthreads();
+  }
+  for (int64_t r = d.N + tid; r < d.ld; r += 1024) d.cls[r] = kKeep;  // padding rows stay zero
+  if (tid == 0) {
+    d.counts[0] = base;
+    d.counts[1] = inact_total;
+  }
+}
+
+// Stable descending sort by counting: rank(i) = #{j : key_j > key_i or (key_j == key_i and j < i)}.
+// j < i in the ascending list is "smaller neuron index", which is what MATLAB's stable sort keeps.
+__global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.z] : one;
+  const int m = d.m;
+  if ((int)(blockIdx.x * 256) >= m) return;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const double ki = i < m ? d.key[i] : 0.0;
+  __shared__ double tile[256];
+  int rank = 0;
+  for (int j0 = 0; j0 < m; j0 += 256) {
+    const int j = j0 + threadIdx.x;
+    tile[threadIdx.x] = j < m ? d.key[j] : 0.0;
+    __syncthreads();
+    const int lim = min(256, m - j0);
+    for (int t = 0; t < lim; ++t) {
+      const double kj = tile[t];
+      rank += (kj > ki || (kj == ki && (j0 + t) < i)) ? 1 : 0;
+    }
+    __syncthreads();
+  }
+  if (i < m) {
+    const int neuron = d.asc_idx[i];
+    d.cross_idx[rank] = neuron;
+    d.cls[neuron] = rank;
+  }
+}
+
+constexpr int kApplyRows = 128;  // 64 lanes x 2 rows, the four waves interleave columns
+
+__global__ __launch_bounds__(256) void relu_apply_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.z] : one;
+  const int ncols_out = d.ncols_in + d.m;
+  const int j0 = blockIdx.y * d.cols_per_chunk;
+  if (j0 >= ncols_out) return;
+  const int j1 = min(ncols_out, j0 + d.cols_per_chunk);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t r0 = (int64_t)blockIdx.x * kApplyRows + 2 * lane;
+  const bool active = r0 < d.ld;
+  int cx = kKeep, cy = kKeep;
+  if (active) {
+    const int2 c = *reinterpret_cast<const int2*>(d.cls + r0);
+    cx = c.x;
+    cy = c.y;
+  }
+  const int n_in = d.ncols_in - 1;
+#pragma unroll 2
+  for (int j = j0 + wave; j < j1; j += 4) {
+    double2 o;
+    if (j < d.ncols_in) {
+      if (active) {
+        const double2 v = *reinterpret_cast<const double2*>(d.Vin + r0 + (int64_t)j * d.ld);
+        o.x = cx == kKeep ? v.x : 0.0;  // V1(map,:) = 0
+        o.y = cy == kKeep ? v.y : 0.0;
+        if (cx >= 0) d.rows[cx + (int64_t)j * d.ld_rows] = v.x;  // I.V(index, :) before zeroing
+        if (cy >= 0) d.rows[cy + (int64_t)j * d.ld_rows] = v.y;
+      }
+      if (blockIdx.x == 0 && lane == 0 && j >= 1) {
+        d.plb_out[j - 1] = d.plb_in[j - 1];
+        d.pub_out[j - 1] = d.pub_in[j - 1];
+      }
+    } else {
+      const int i = j - d.ncols_in;
+      const int neuron = d.cross_idx[i];
+      o.x = r0 == neuron ? 1.0 : 0.0;  // V2(index(i), i) = 1
+      o.y = r0 + 1 == neuron ? 1.0 : 0.0;
+      if (blockIdx.x == 0 && lane == 0) {
+        const double u = d.ub[neuron];
+        d.plb_out[n_in + i] = 0.0;  // new_pred_lb = [plb; zeros(m,1)]
+        d.pub_out[n_in + i] = u;    // new_pred_ub = [pub; ub]
+        d.lbub[i] = d.lb[neuron];
+        d.lbub[d.ld_rows + i] = u;
+      }
+    }
+    if (active) *reinterpret_cast<double2*>(d.Vout + r0 + (int64_t)j * d.ld) = o;
+  }
+}
+
+int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
+  if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  NNV_TRY(compute_ranges(ctx, count, in));
+  const int64_t N = in[0]->N;
+  const int64_t ld = in[0]->ld;
+  if (N >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "set dimension too large");
+  const bool sorted = order != NNVHIP_ORDER_INDEX;
+
+  // scratch shared by all sets: cls | counts ; cross_idx is kept (it becomes the node's index list)
+  BufRef cls_buf, cnt_buf, asc_buf, key_buf;
+  NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &cls_buf));
+  NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * count, &cnt_buf));
+  if (sorted) {
+    NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &asc_buf));
+    NNV_TRY(ctx->alloc(sizeof(double) * ld * count, &key_buf));
+  }
+  std::vector<BufRef> idx_bufs(count);
+  std::vector<ReluDesc> descs(count);
+  for (int64_t i = 0; i < count; ++i) {
+    NNV_TRY(ctx->alloc(sizeof(int32_t) * ld, &idx_bufs[i]));
+    ReluDesc& d = descs[i];
+    d = ReluDesc{};
+    d.Vin = in[i]->V;
+    d.lb = in[i]->lb;
+    d.ub = in[i]->ub;
+    d.plb_in = in[i]->plb;
+    d.pub_in = in[i]->pub;
+    d.cls = cls_buf->as<int32_t>() + ld * i;
+    d.cross_idx = idx_bufs[i]->as<int32_t>();
+    d.asc_idx = sorted ? asc_buf->as<int32_t>() + ld * i : nullptr;
+    d.key = sorted ? key_buf->as<double>() + ld * i : nullptr;
+    d.counts = cnt_buf->as<int32_t>() + 2 * i;
+    d.ld = ld;
+    d.N = (int32_t)N;
+    d.ncols_in = (int32_t)(in[i]->n + 1);
+    d.order = order;
+  }
+  const ReluDesc* table = nullptr;
+  BufRef tab;
+  if (count > 1) {
+    NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
+    table = tab->as<ReluDesc>();
+  }
+  hipLaunchKernelGGL(relu_classify_kernel, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+  NNV_HIP_TRY(hipGetLastError());
+
+  // the column count of the output depends on m: read the counts back
+  void* hc = nullptr;
+  NNV_TRY(ctx->stage(sizeof(int32_t) * 2 * count, &hc));
+  NNV_HIP_TRY(hipMemcpyAsync(hc, cnt_buf->ptr, sizeof(int32_t) * 2 * count, hipMemcpyDeviceToHost, ctx->stream));
+  NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));
+  const std::vector<int32_t> counts(static_cast<const int32_t*>(hc), static_cast<const int32_t*>(hc) + 2 * count);
+
+  // outputs: one V arena, one predicate-bound buffer, one buffer for all saved rows / bounds
+  int64_t total_cols = 0, total_pred = 0, total_rows = 0, total_lbub = 0, max_cols = 0, max_m = 0;
+  std::vector<int64_t> col_off(count), pred_off(count), rows_off(count), lbub_off(count);
+  for (int64_t i = 0; i < count; ++i) {
+    const int64_t m = counts[2 * i];
+    const int64_t ncols_out = in[i]->n + 1 + m;
+    const int64_t ldr = round_up(std::max<int64_t>(m, 1), kLdAlign);
+    col_off[i] = total_cols;
+    pred_off[i] = total_pred;
+    rows_off[i] = total_rows;
+    lbub_off[i] = total_lbub;
+    total_cols += ncols_out;
+    total_pred += 2 * round_up(std::max<int64_t>(in[i]->n + m, 1), kLdAlign);
+    total_rows += m > 0 ? ldr * (in[i]->n + 1) : 0;
+    total_lbub += m > 0 ? 2 * ldr : 0;
+    max_cols = std::max(max_cols, ncols_out);
+    max_m = std::max(max_m, m);
+  }
+  BufRef arena, pred_buf, rows_buf, lbub_buf;
+  NNV_TRY(ctx->alloc(sizeof(double) * ld * total_cols, &arena));
+  NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
+  if (total_rows > 0) {
+    NNV_TRY(ctx->alloc(sizeof(double) * total_rows, &rows_buf));
+    NNV_TRY(ctx->alloc(sizeof(double) * total_lbub, &lbub_buf));
+  }
+  // Column chunking of the apply pass: a few thousand blocks, at least 16 columns each.
+  const int64_t row_blocks = ceil_div(ld, kApplyRows);
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(4096, row_blocks * count), ceil_div(max_cols, 16)));
+  const int64_t cpc = ceil_div(max_cols, chunks);
+  chunks = ceil_div(max_cols, cpc);
+  for (int64_t i = 0; i < count; ++i) {
+    ReluDesc& d = descs[i];
+    const int64_t m = counts[2 * i];
+    const int64_t ldr = round_up(std::max<int64_t>(m, 1), kLdAlign);
+    const int64_t npad = round_up(std::max<int64_t>(in[i]->n + m, 1), kLdAlign);
+    d.m = (int32_t)m;
+    d.Vout = arena->as<double>() + col_off[i] * ld;
+    d.plb_out = pred_buf->as<double>() + pred_off[i];
+    d.pub_out = d.plb_out + npad;
+    d.rows = m > 0 ? rows_buf->as<double>() + rows_off[i] : nullptr;
+    d.lbub = m > 0 ? lbub_buf->as<double>() + lbub_off[i] : nullptr;
+    d.ld_rows = ldr;
+    d.cols_per_chunk = (int32_t)cpc;
+  }
+  if (count > 1) {
+    NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
+    table = tab->as<ReluDesc>();
+  }
+  if (sorted && max_m > 0)
+    hipLaunchKernelGGL(relu_rank_kernel, dim3((unsigned)ceil_div(max_m, 256), 1, (unsigned)count), dim3(256), 0,
+                       ctx->stream, table, descs[0]);
+  hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(256), 0,
+                     ctx->stream, table, descs[0]);
+  NNV_HIP_TRY(hipGetLastError());
+
+  for (int64_t i = 0; i < count; ++i) {
+    const ReluDesc& d = descs[i];
+    nnvhip_star* o = new_star(ctx);
+    o->N = N;
+    o->n = in[i]->n + d.m;
+    o->ld = ld;
+    o->Vbuf = arena;
+    o->V = d.Vout;
+    o->pbuf = pred_buf;
+    o->plb = d.plb_out;
+    o->pub = d.pub_out;
+    o->n_inactive = counts[2 * i + 1];
+    o->n_crossing = d.m;
+    if (d.m > 0) {
+      auto node = std::make_shared<ConsNode>();
+      node->prev = in[i]->cons;
+      node->m = d.m;
+      node->n_before = in[i]->n;
+      node->p_total = in[i]->cons->p_total + 3 * (int64_t)d.m;
+      node->n_total = o->n;
+      node->rows = rows_buf;
+      node->ld_rows = d.ld_rows;
+      node->lbub = lbub_buf;
+      node->index = idx_bufs[i];
+      // views into shared buffers: keep element offsets
+      node->rows_off = rows_off[i];
+      node->lbub_off = lbub_off[i];
+      o->cons = node;
+    } else {
+      o->cons = in[i]->cons;  // no crossing neuron: C, d unchanged
+    }
+    out[i] = o;
+  }
+  return NNVHIP_OK;
+}
+
+// ---- dense constraint materialisation -----------------------------------------------------------
+
+__global__ void cons_copy_kernel(double* __restrict__ C, int64_t ldC, const double* __restrict__ C0, int64_t ldc0,
+                                 int64_t p0, int64_t n0) {
+  const int64_t total = p0 * n0;
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = t % p0, c = t / p0;
+    C[r + c * ldC] = C0[r + c * ldc0];
+  }
+}
+
+// Rows of one ReLU node (nn/funcs/PosLin.m:711-735), r0 = rows before it, nb = n_before:
+//   C1 = [0 -I], d1 = 0;  C2 = [V(index,2:n+1) -I], d2 = -V(index,1);
+//   a = ub./(ub-lb); b = a.*lb;  C3 = [-a.*V(index,2:n+1) I], d3 = a.*V(index,1) - b.
+__global__ void cons_relu_kernel(double* __restrict__ C, int64_t ldC, double* __restrict__ dvec, int64_t r0, int m,
+                                 int nb, const double* __restrict__ rows, int64_t ld_rows,
+                                 const double* __restrict__ lb, const double* __restrict__ ub) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= m) return;
+  const double a = ub[i] / (ub[i] - lb[i]);
+  const int64_t row1 = r0 + i, row2 = r0 + m + i, row3 = r0 + 2 * (int64_t)m + i;
+  for (int j = blockIdx.y; j <= nb; j += gridDim.y) {
+    const double v = rows[i + (int64_t)j * ld_rows];
+    if (j == 0) {
+      dvec[row1] = 0.0;
+      dvec[row2] = -v;
+      dvec[row3] = __dsub_rn(__dmul_rn(a, v), __dmul_rn(a, lb[i]));
+      C[row1 + (int64_t)(nb + i) * ldC] = -1.0;
+      C[row2 + (int64_t)(nb + i) * ldC] = -1.0;
+      C[row3 + (int64_t)(nb + i) * ldC] = 1.0;
+    } else {
+      C[row2 + (int64_t)(j - 1) * ldC] = v;
+      C[row3 + (int64_t)(j - 1) * ldC] = __dmul_rn(-a, v);
+    }
+  }
+}
+
+int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host) {
+  nnvhip_ctx* ctx = s->ctx;
+  const int64_t p = s->cons->p_total, n = s->n;
+  if (p == 0) return NNVHIP_OK;
+  std::vector<const ConsNode*> chain;
+  for (const ConsNode* nd = s->cons.get(); nd; nd = nd->prev.get()) chain.push_back(nd);
+  std::reverse(chain.begin(), chain.end());
+  BufRef Cd, dd;
+  if (n > 0) {
+    NNV_TRY(ctx->alloc(sizeof(double) * p * n, &Cd));
+    NNV_HIP_TRY(hipMemsetAsync(Cd->ptr, 0, sizeof(double) * p * n, ctx->stream));
+  }
+  NNV_TRY(ctx->alloc(sizeof(double) * p, &dd));
+  NNV_HIP_TRY(hipMemsetAsync(dd->ptr, 0, sizeof(double) * p, ctx->stream));
+  double* Cp = Cd ? Cd->as<double>() : nullptr;
+  int64_t r0 = 0;
+  for (const ConsNode* nd : chain) {
+    if (!nd->prev) {  // base node
+      if (nd->C0 && Cp && nd->n_total > 0)
+        hipLaunchKernelGGL(cons_copy_kernel, dim3(1024), dim3(256), 0, ctx->stream, Cp, p, nd->C0->as<double>(), nd->ldc,
+                           nd->p_total, nd->n_total);
+      if (nd->d0)
+        NNV_HIP_TRY(hipMemcpyAsync(dd->ptr, nd->d0->ptr, sizeof(double) * nd->p_total, hipMemcpyDeviceToDevice, ctx->stream));
+      r0 = nd->p_total;
+    } else {
+      double* Cuse = Cp;
+      const int64_t ldC = p;
+      const double* rows = nd->rows->as<double>() + nd->rows_off;
+      const double* lbp = nd->lbub->as<double>() + nd->lbub_off;
+      dim3 grid((unsigned)ceil_div(nd->m, 128), (unsigned)std::min<int64_t>(nd->n_before + 1, 1024));
+      hipLaunchKernelGGL(cons_relu_kernel, grid, dim3(128), 0, ctx->stream, Cuse, ldC, dd->as<double>(), r0, (int)nd->m,
+                         (int)nd->n_before, rows, nd->ld_rows, lbp, lbp + nd->ld_rows);
+      r0 += 3 * nd->m;
+    }
+  }
+  NNV_HIP_TRY(hipGetLastError());
+  if (Cp && C_host) NNV_HIP_TRY(hipMemcpyAsync(C_host, Cp, sizeof(double) * p * n, hipMemcpyDeviceToHost, ctx->stream));
+  if (d_host) NNV_HIP_TRY(hipMemcpyAsync(d_host, dd->ptr, sizeof(double) * p, hipMemcpyDeviceToHost, ctx->stream));
+  NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));
+  return NNVHIP_OK;
+}
+
+}  // namespace nnvhip

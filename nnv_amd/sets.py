@@ -1,0 +1,412 @@
+"""Star / ImageStar / Box: NNV's set classes with the generator matrix resident in HBM.
+
+The classes mirror the fields and methods of the reference that the relax-star reach path and its
+callers touch (code/nnv/engine/set/Star.m:13-24, set/ImageStar.m:47-94, set/Box.m).  A set holds an
+opaque device handle; property reads (``V``, ``C``, ``d``, ``predicate_lb`` ...) fetch dense arrays
+in MATLAB layout on demand.  Index vectors returned to Python are 0-based.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import check, f64, ptr
+
+
+class _Handle:
+    """Owns one reference of a device set handle."""
+
+    __slots__ = ("h", "ctx", "_cache")
+
+    def __init__(self, h, ctx):
+        self.h = h
+        self.ctx = ctx
+        self._cache = {}
+
+    def __del__(self):
+        try:
+            if self.h:
+                self.ctx.lib.nnvhip_star_release(self.h)
+                self.h = None
+        except Exception:
+            pass
+
+    def dims(self):
+        if "dims" not in self._cache:
+            N, n, p = C.c_int64(), C.c_int64(), C.c_int64()
+            check(self.ctx.lib.nnvhip_star_dims(self.h, C.byref(N), C.byref(n), C.byref(p)))
+            self._cache["dims"] = (N.value, n.value, p.value)
+        return self._cache["dims"]
+
+    def fetch_V(self):
+        N, n, _ = self.dims()
+        V = np.empty((N, n + 1), dtype=np.float64, order="F")
+        check(self.ctx.lib.nnvhip_star_fetch_V(self.h, ptr(V)))
+        return V
+
+    def fetch_pred(self):
+        _, n, _ = self.dims()
+        lb = np.empty(n)
+        ub = np.empty(n)
+        check(self.ctx.lib.nnvhip_star_fetch_pred_bounds(self.h, ptr(lb), ptr(ub)))
+        return lb, ub
+
+    def fetch_constraints(self):
+        _, n, p = self.dims()
+        Cm = np.empty((p, n), dtype=np.float64, order="F")
+        d = np.empty(p)
+        check(self.ctx.lib.nnvhip_star_fetch_constraints(self.h, ptr(Cm), ptr(d)))
+        return Cm, d
+
+    def ranges(self):
+        N, _, _ = self.dims()
+        lb = np.empty(N)
+        ub = np.empty(N)
+        check(self.ctx.lib.nnvhip_estimate_ranges(self.ctx.handle, self.h, ptr(lb), ptr(ub)))
+        return lb, ub
+
+    def relu_info(self):
+        ni, nc = C.c_int64(), C.c_int64()
+        check(self.ctx.lib.nnvhip_star_relu_counts(self.h, C.byref(ni), C.byref(nc)))
+        m = nc.value
+        idx = np.empty(m, dtype=np.int32)
+        lb = np.empty(m)
+        ub = np.empty(m)
+        check(self.ctx.lib.nnvhip_star_fetch_crossing(self.h, ptr(idx), ptr(lb), ptr(ub)))
+        return ni.value, idx, lb, ub
+
+
+def _make_handles(ctx, raw):
+    return [_Handle(C.c_void_p(h), ctx) for h in raw]
+
+
+class Box:
+    """set/Box.m: hyper-rectangle with centre/generator form and uniform partitioning."""
+
+    def __init__(self, lb, ub):
+        lb = np.asarray(lb, dtype=np.float64)
+        ub = np.asarray(ub, dtype=np.float64)
+        if (lb.ndim == 2 and lb.shape[1] != 1) or (ub.ndim == 2 and ub.shape[1] != 1):
+            raise ValueError("lb and ub should be a vector")
+        lb = lb.reshape(-1)
+        ub = ub.reshape(-1)
+        if lb.size != ub.size:
+            raise ValueError("Inconsistent dimensions between lb and ub")
+        self.lb = lb
+        self.ub = ub
+        self.dim = lb.size
+        self.center = 0.5 * (lb + ub)            # Box.m:35
+        vec = 0.5 * (ub - lb)                    # Box.m:36
+        gens = np.diag(vec)
+        if gens.size > 1:
+            gens = gens[:, ~np.all(gens == 0, axis=0)]   # Box.m:41-43
+        self.generators = gens
+
+    def singlePartition(self, part_id, part_num):
+        """Box.m:61-91; part_id is 0-based."""
+        if part_id < 0 or part_id >= self.dim:
+            raise ValueError("Invalid partition index")
+        if part_num < 1:
+            raise ValueError("Invalid partition number")
+        if part_num == 1:
+            return [self]
+        delta = (self.ub[part_id] - self.lb[part_id]) / part_num
+        out = []
+        for i in range(1, part_num + 1):
+            new_lb = self.lb.copy()
+            new_ub = self.ub.copy()
+            new_lb[part_id] = self.lb[part_id] + (i - 1) * delta
+            new_ub[part_id] = new_lb[part_id] + delta
+            out.append(Box(new_lb, new_ub))
+        return out
+
+    def partition(self, part_indexes, part_numbers):
+        """Box.m:96-139: first listed index varies slowest."""
+        part_indexes = list(part_indexes)
+        part_numbers = list(part_numbers)
+        if len(part_indexes) != len(part_numbers):
+            raise ValueError("Inconsistent between part_indexes and part_number array, should have the same number of elements")
+        for i, (ix, num) in enumerate(zip(part_indexes, part_numbers)):
+            if ix < 0 or ix >= self.dim:
+                raise ValueError("The %d^th index in part_indexes array is invalid" % (i + 1))
+            if num < 1:
+                raise ValueError("The %d^th number in part_numbers array is invalid" % (i + 1))
+        boxes = [self]
+        for ix, num in zip(part_indexes, part_numbers):
+            nxt = []
+            for b in boxes:
+                nxt.extend(b.singlePartition(ix, num))
+            boxes = nxt
+        return boxes
+
+    def toStar(self, ctx=None):
+        return Star(self.lb, self.ub, ctx=ctx)
+
+
+class Star:
+    """Device-resident Star: x = c + V*a, C*a <= d, predicate_lb <= a <= predicate_ub.
+
+    Constructors (set/Star.m:29-275): ``Star(V, C, d, pred_lb, pred_ub)``, ``Star(V, C, d)``,
+    ``Star(lb, ub)``.  The outer zonotope ``Z`` of the reference is not carried (only the
+    approx-zono method reads it).
+    """
+
+    def __init__(self, *args, ctx=None, _handle=None):
+        self.state_lb = None
+        self.state_ub = None
+        self.Z = None
+        if _handle is not None:
+            self._h = _handle
+            return
+        ctx = ctx or _lib.default_context()
+        lib = ctx.lib
+        if len(args) == 2:
+            lb = np.asarray(args[0], dtype=np.float64)
+            ub = np.asarray(args[1], dtype=np.float64)
+            b = Box(lb, ub)  # size checks
+            out = (C.c_void_p * 1)()
+            check(lib.nnvhip_star_from_box(ctx.handle, b.dim, 1, ptr(f64(b.lb)), ptr(f64(b.ub)), out))
+            self._h = _Handle(C.c_void_p(out[0]), ctx)
+            self.state_lb = b.lb.copy()
+            self.state_ub = b.ub.copy()
+            return
+        if len(args) in (3, 5):
+            V = f64(args[0])
+            Cm = np.asarray(args[1], dtype=np.float64)
+            d = np.asarray(args[2], dtype=np.float64)
+            if V.ndim != 2:
+                raise ValueError("Inconsistency between basic matrix and constraint matrix")
+            if Cm.ndim == 1:
+                Cm = Cm.reshape(1, -1)
+            if d.ndim == 2 and d.shape[1] != 1:
+                raise ValueError("constraint vector should have one column")
+            d = d.reshape(-1)
+            if V.shape[1] != Cm.shape[1] + 1:
+                raise ValueError("Inconsistency between basic matrix and constraint matrix")
+            if Cm.shape[0] != d.shape[0]:
+                raise ValueError("Inconsistency between constraint matrix and constraint vector")
+            plb = pub = None
+            if len(args) == 5 and args[3] is not None and args[4] is not None and np.size(args[3]) and np.size(args[4]):
+                plb = np.asarray(args[3], dtype=np.float64)
+                pub = np.asarray(args[4], dtype=np.float64)
+                if (plb.ndim == 2 and plb.shape[1] != 1) or (pub.ndim == 2 and pub.shape[1] != 1):
+                    raise ValueError("predicate lower- or upper-bounds vector should have one column")
+                plb = f64(plb.reshape(-1))
+                pub = f64(pub.reshape(-1))
+                if plb.size != pub.size or plb.size != Cm.shape[1]:
+                    raise ValueError("Inconsistency between number of predicate variables and predicate lower- or upper-bounds vector")
+            Cm = f64(Cm)
+            d = f64(d)
+            out = C.c_void_p()
+            check(lib.nnvhip_star_create(ctx.handle, V.shape[0], Cm.shape[1], ptr(V), ptr(plb), ptr(pub),
+                                         ptr(Cm) if Cm.size else None, ptr(d) if d.size else None, Cm.shape[0],
+                                         C.byref(out)))
+            self._h = _Handle(out, ctx)
+            return
+        raise ValueError("Invalid number of input arguments (should be 0, 1, 2, 3, 5, 6 or 7)")
+
+    # ---- array construction --------------------------------------------------------------
+    @staticmethod
+    def from_boxes(lbs, ubs, ctx=None):
+        """Array of Star(lb, ub) for the columns of two N x count matrices, built in one device
+        arena (the Star array NN.reach accepts, nn/NN.m:204-207)."""
+        ctx = ctx or _lib.default_context()
+        lbs = f64(lbs)
+        ubs = f64(ubs)
+        if lbs.shape != ubs.shape or lbs.ndim != 2:
+            raise ValueError("Inconsistent dimensions between lb and ub")
+        N, count = lbs.shape
+        out = (C.c_void_p * count)()
+        check(ctx.lib.nnvhip_star_from_box(ctx.handle, N, count, ptr(lbs), ptr(ubs), out))
+        stars = []
+        for i, h in enumerate(_make_handles(ctx, out)):
+            s = Star(_handle=h)
+            s.state_lb = lbs[:, i].copy()
+            s.state_ub = ubs[:, i].copy()
+            stars.append(s)
+        return stars
+
+    # ---- NNV properties ------------------------------------------------------------------
+    @property
+    def ctx(self):
+        return self._h.ctx
+
+    @property
+    def dim(self):
+        return self._h.dims()[0]
+
+    @property
+    def nVar(self):
+        return self._h.dims()[1]
+
+    @property
+    def V(self):
+        return self._h.fetch_V()
+
+    @property
+    def C(self):
+        return self._h.fetch_constraints()[0]
+
+    @property
+    def d(self):
+        return self._h.fetch_constraints()[1]
+
+    @property
+    def predicate_lb(self):
+        return self._h.fetch_pred()[0]
+
+    @property
+    def predicate_ub(self):
+        return self._h.fetch_pred()[1]
+
+    # ---- methods on the path -------------------------------------------------------------
+    def affineMap(self, W, b=None):
+        """Star.affineMap, set/Star.m:313-343."""
+        from .layers import FullyConnectedLayer
+        W = np.asarray(W, dtype=np.float64)
+        if W.ndim != 2 or W.shape[1] != self.dim:
+            raise ValueError("Inconsistency between the affine mapping matrix and dimension of the star set")
+        if b is not None and np.size(b):
+            b = np.asarray(b, dtype=np.float64)
+            if b.ndim == 2 and b.shape[1] != 1:
+                raise ValueError("Mapping vector should have one column")
+            if b.reshape(-1).shape[0] != W.shape[0]:
+                raise ValueError("Inconsistency between the mapping vec and mapping matrix")
+        else:
+            b = None
+        return FullyConnectedLayer._map(self.ctx, W, b, [self])[0]
+
+    def estimateRanges(self):
+        """Star.estimateRanges, set/Star.m:1078-1106 -> (lb, ub)."""
+        return self._h.ranges()
+
+    def toImageStar(self, height, width, numChannel):
+        """Star.toImageStar, set/Star.m:1398-1418: a reshape; the device data is shared."""
+        if self.dim != height * width * numChannel:
+            raise ValueError("Inconsistent dimension in the ImageStar and the original Star set")
+        im = ImageStar(_handle=self._h, shape=(height, width, numChannel))
+        if self.state_lb is not None and self.state_ub is not None:
+            im.im_lb = np.asarray(self.state_lb).reshape((height, width, numChannel), order="F")
+            im.im_ub = np.asarray(self.state_ub).reshape((height, width, numChannel), order="F")
+        return im
+
+    def relu_info(self):
+        """For a set returned by the ReLU step: (n_inactive, crossing index (0-based, new-predicate
+        order), lb(crossing), ub(crossing))."""
+        return self._h.relu_info()
+
+
+class ImageStar:
+    """Device-resident ImageStar (set/ImageStar.m:47-94): V is H x W x C x (numPred+1).
+
+    Constructors: ``ImageStar(V, C, d, pred_lb, pred_ub)`` (:172-227) and
+    ``ImageStar(lb_image, ub_image)`` (:302-343).
+    """
+
+    def __init__(self, *args, ctx=None, _handle=None, shape=None):
+        self.im_lb = None
+        self.im_ub = None
+        if _handle is not None:
+            self._h = _handle
+            self.height, self.width, self.numChannel = shape
+            return
+        if len(args) == 2:
+            lb_im = np.asarray(args[0], dtype=np.float64)
+            ub_im = np.asarray(args[1], dtype=np.float64)
+            if lb_im.size == 0:
+                raise ValueError("Invalid lower bound image")
+            if ub_im.size == 0:
+                raise ValueError("Invalid upper bound image")
+            if lb_im.shape != ub_im.shape:
+                raise ValueError("Inconsistency between lower bound image and upper bound image")
+            if lb_im.ndim == 2:
+                lb_im = lb_im[:, :, None]
+                ub_im = ub_im[:, :, None]
+            if lb_im.ndim != 3:
+                raise ValueError("Inconsistency between lower bound image and upper bound image")
+            h, w, c = lb_im.shape
+            S = Star(lb_im.reshape(-1, order="F"), ub_im.reshape(-1, order="F"), ctx=ctx)
+            self._h = S._h
+            self.height, self.width, self.numChannel = h, w, c
+            self.im_lb = lb_im
+            self.im_ub = ub_im
+            return
+        if len(args) == 5:
+            V = np.asarray(args[0], dtype=np.float64)
+            Cm = np.asarray(args[1], dtype=np.float64)
+            d = np.asarray(args[2], dtype=np.float64)
+            if Cm.ndim == 1:
+                Cm = Cm.reshape(1, -1)
+            if d.ndim == 2 and d.shape[1] != 1:
+                raise ValueError("Invalid constraint vector, vector should have one column")
+            if Cm.shape[0] != d.reshape(-1).shape[0]:
+                raise ValueError("Inconsistent dimension between constraint matrix and constraint vector")
+            plb = np.asarray(args[3], dtype=np.float64).reshape(-1)
+            pub = np.asarray(args[4], dtype=np.float64).reshape(-1)
+            if Cm.shape[1] != plb.size or Cm.shape[1] != pub.size:
+                raise ValueError("Number of predicates is different from the size of the lower bound or upper bound predicate vector")
+            if V.ndim == 2:
+                V = V[:, :, None, None]
+            elif V.ndim == 3:
+                V = V[:, :, :, None]
+            if V.ndim != 4:
+                raise ValueError("Invalid basis matrix")
+            if V.shape[3] != Cm.shape[1] + 1:
+                raise ValueError("Inconsistency between the basis matrix and the number of predicate variables")
+            h, w, c, g = V.shape
+            S = Star(V.reshape(h * w * c, g, order="F"), Cm, d, plb, pub, ctx=ctx)
+            self._h = S._h
+            self.height, self.width, self.numChannel = h, w, c
+            return
+        raise ValueError("Invalid number of input arguments")
+
+    @property
+    def ctx(self):
+        return self._h.ctx
+
+    @property
+    def numPred(self):
+        return self._h.dims()[1]
+
+    @property
+    def V(self):
+        V = self._h.fetch_V()
+        return V.reshape((self.height, self.width, self.numChannel, V.shape[1]), order="F")
+
+    @property
+    def C(self):
+        return self._h.fetch_constraints()[0]
+
+    @property
+    def d(self):
+        return self._h.fetch_constraints()[1]
+
+    @property
+    def pred_lb(self):
+        return self._h.fetch_pred()[0]
+
+    @property
+    def pred_ub(self):
+        return self._h.fetch_pred()[1]
+
+    def toStar(self):
+        """ImageStar.toStar, set/ImageStar.m:569-592: flatten in column-major order (shared data)."""
+        S = Star(_handle=self._h)
+        if self.im_lb is not None and self.im_ub is not None:
+            S.state_lb = np.asarray(self.im_lb).reshape(-1, order="F")
+            S.state_ub = np.asarray(self.im_ub).reshape(-1, order="F")
+        return S
+
+    def estimateRanges(self):
+        """ImageStar.estimateRanges, set/ImageStar.m:836-885 -> (image_lb, image_ub); cached."""
+        if self.im_lb is None or self.im_ub is None:
+            lb, ub = self._h.ranges()
+            shp = (self.height, self.width, self.numChannel)
+            self.im_lb = lb.reshape(shp, order="F")
+            self.im_ub = ub.reshape(shp, order="F")
+        return self.im_lb, self.im_ub
+
+    def relu_info(self):
+        return self._h.relu_info()

@@ -1,0 +1,214 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs."""
+import numpy as np
+import pytest
+
+from tests.gpu_util import RTOL, assert_close, compare_sets, flat_V, input_sets, run_both
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nnv():
+    import nnv_amd
+    nnv_amd.default_context()
+    return nnv_amd
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    from oracle import nnv_oracle
+    return nnv_oracle
+
+
+def _rand_star_arrays(rs, N, n, p=3):
+    V = rs.randn(N, n + 1)
+    C = rs.randn(p, n)
+    d = np.abs(rs.randn(p)) + 5.0
+    lb = -np.abs(rs.rand(n)) - 0.1
+    ub = np.abs(rs.rand(n)) + 0.1
+    return V, C, d, lb, ub
+
+
+def test_golden_affine_map_and_ranges(nnv, oracle, golden):
+    g = golden["star_affineMap"]
+    S = nnv.Star(g["S_V"], g["S_C"], g["S_d"])
+    S1 = S.affineMap(g["W"], g["b"])
+    assert np.array_equal(S1.V, g["S1_V"])
+    assert np.array_equal(S1.C, g["S1_C"]) and np.array_equal(S1.d, g["S1_d"].reshape(-1))
+    S3 = nnv.Star(g["box_lb"].reshape(-1), g["box_ub"].reshape(-1))
+    assert np.array_equal(S3.V, oracle.star_from_box(g["box_lb"].reshape(-1), g["box_ub"].reshape(-1)).V)
+    assert np.array_equal(S3.C, np.zeros((1, 3))) and np.array_equal(S3.d, np.zeros(1))
+    lb, ub = S3.affineMap(g["W2"], None).estimateRanges()
+    np.testing.assert_allclose(lb, g["S4_lb"].reshape(-1), rtol=0, atol=1e-14)
+    np.testing.assert_allclose(ub, g["S4_ub"].reshape(-1), rtol=0, atol=1e-14)
+    gi = golden["imagestar_getRange_issue"]
+    I = nnv.ImageStar(gi["V"], np.zeros((1, 2)), np.zeros(1), gi["pred_lb"], gi["pred_ub"])
+    l, u = I.estimateRanges()
+    assert l.reshape(-1)[0] == -2.0 and u.reshape(-1)[0] == 2.0
+
+
+def test_golden_conv_known_answer(nnv, golden):
+    g = golden["conv2d_featureMap"]
+    I = nnv.ImageStar(g["I"][:, :, None, None].repeat(2, axis=3) * np.array([1.0, 0.0]), np.zeros((1, 1)),
+                      np.zeros(1), [-1.0], [1.0])
+    L = nnv.Conv2DLayer(g["W"][:, :, None, None], np.zeros(1), g["padding"], g["stride"], g["dilation"])
+    R = L.reach(I, "relax-star-area")
+    assert np.array_equal(R.V[:, :, 0, 0], g["expected"])
+    assert not R.V[:, :, 0, 1].any()
+
+
+@pytest.mark.parametrize("N,n", [(1, 1), (5, 3), (16, 16), (50, 7), (129, 300), (1024, 2500), (3000, 65), (10, 4000)])
+def test_star_roundtrip_and_ranges(nnv, oracle, N, n):
+    rs = np.random.RandomState(N * 7 + n)
+    V, C, d, lb, ub = _rand_star_arrays(rs, N, n)
+    S = nnv.Star(V, C, d, lb, ub)
+    assert (S.dim, S.nVar) == (N, n)
+    assert np.array_equal(S.V, V) and np.array_equal(S.C, C) and np.array_equal(S.d, d)
+    assert np.array_equal(S.predicate_lb, lb) and np.array_equal(S.predicate_ub, ub)
+    glb, gub = S.estimateRanges()
+    elb, eub = oracle.estimate_ranges(oracle.OStar(V, C, d, lb, ub))
+    assert_close(glb, elb, "lb", 1e-12)
+    assert_close(gub, eub, "ub", 1e-12)
+    # default predicate bounds (-1/+1) when none are given
+    S2 = nnv.Star(V, C, d)
+    g2l, g2u = S2.estimateRanges()
+    e2l, e2u = oracle.estimate_ranges(oracle.OStar(V, C, d))
+    assert_close(g2l, e2l, "lb default", 1e-12)
+    assert_close(g2u, e2u, "ub default", 1e-12)
+
+
+@pytest.mark.parametrize("M,K,n", [(1, 1, 1), (5, 5, 5), (50, 5, 5), (10, 100, 1045), (64, 64, 63), (100, 784, 20),
+                                   (130, 70, 257), (256, 300, 1000), (1024, 784, 785), (33, 1000, 129)])
+def test_affine_fc(nnv, oracle, M, K, n):
+    rs = np.random.RandomState(M + 3 * K + n)
+    V, C, d, lb, ub = _rand_star_arrays(rs, K, n)
+    W = rs.randn(M, K)
+    b = rs.randn(M)
+    S = nnv.Star(V, C, d, lb, ub)
+    R = S.affineMap(W, b)
+    E = oracle.affine_map(oracle.OStar(V, C, d, lb, ub), W, b)
+    compare_sets(R, E, "affineMap %dx%dx%d" % (M, K, n))
+    R2 = S.affineMap(W, None)
+    assert_close(R2.V[:, 0], (W @ V)[:, 0], "no-bias centre")
+    L = nnv.FullyConnectedLayer(W, b)
+    R3 = L.reach(S, "relax-star-area", [], 1, None, "linprog")
+    assert np.array_equal(R3.V, R.V)
+    with pytest.raises(ValueError, match="affine mapping matrix"):
+        S.affineMap(rs.randn(3, K + 1), None)
+    with pytest.raises(ValueError, match="Unknown reachability method"):
+        L.reach(S, "bogus")
+
+
+@pytest.mark.parametrize("H,W,Cin,Cout,FH,FW,s,p,dil,n", [
+    (5, 5, 1, 1, 3, 3, 1, 0, 1, 1), (7, 6, 3, 4, 3, 3, 1, 1, 1, 9), (9, 9, 2, 5, 3, 3, 2, 0, 1, 30),
+    (8, 10, 1, 2, 3, 2, 2, 1, 1, 17), (11, 9, 2, 3, 3, 3, 1, 2, 2, 5), (28, 28, 1, 16, 3, 3, 1, 1, 1, 40),
+    (14, 14, 16, 32, 3, 3, 2, 1, 1, 33), (15, 15, 32, 64, 3, 3, 1, 1, 1, 20), (12, 12, 40, 70, 5, 5, 2, 2, 1, 7)])
+def test_affine_conv2d(nnv, oracle, H, W, Cin, Cout, FH, FW, s, p, dil, n):
+    rs = np.random.RandomState(H * 31 + Cout)
+    V = rs.randn(H, W, Cin, n + 1)
+    C = rs.randn(2, n)
+    d = np.ones(2)
+    lb, ub = -np.ones(n), np.ones(n)
+    Wt = rs.randn(FH, FW, Cin, Cout)
+    b = rs.randn(Cout)
+    I = nnv.ImageStar(V, C, d, lb, ub)
+    L = nnv.Conv2DLayer(Wt, b, [p, p, p, p], [s, s], [dil, dil])
+    R = L.reach(I, "relax-star-area", "single")
+    E = oracle.conv2d_reach(oracle.OImageStar(V, C, d, lb, ub), Wt, b, [p, p, p, p], [s, s], [dil, dil])
+    assert R.V.shape == E.V.shape
+    compare_sets(R, E, "conv")
+    with pytest.raises(ValueError, match="channels"):
+        nnv.Conv2DLayer(rs.randn(3, 3, Cin + 1, 2), np.zeros(2)).reach(I, "relax-star-area")
+
+
+def test_conv_asymmetric_padding(nnv, oracle):
+    rs = np.random.RandomState(11)
+    V = rs.randn(6, 7, 2, 4)
+    Wt = rs.randn(2, 3, 2, 3)
+    b = rs.randn(3)
+    I = nnv.ImageStar(V, np.zeros((1, 3)), np.zeros(1), -np.ones(3), np.ones(3))
+    R = nnv.Conv2DLayer(Wt, b, [1, 0, 2, 1], [1, 2], [1, 1]).reach(I, "relax-star-area")
+    E = oracle.conv2d_reach(oracle.OImageStar(V, np.zeros((1, 3)), np.zeros(1), -np.ones(3), np.ones(3)), Wt, b,
+                            [1, 0, 2, 1], [1, 2], [1, 1])
+    compare_sets(R, E, "conv asym")
+
+
+@pytest.mark.parametrize("method", ["relax-star-area", "relax-star-range", "relax-star-random", "relax-star-static",
+                                    "relax-star-bound", "relax-star-ub"])
+@pytest.mark.parametrize("N,n", [(7, 3), (64, 10), (1000, 50), (2500, 300)])
+def test_relu_step(nnv, oracle, method, N, n):
+    rs = np.random.RandomState(N + n)
+    V, C, d, lb, ub = _rand_star_arrays(rs, N, n)
+    V[:, 0] *= 3.0
+    S = nnv.Star(V, C, d, lb, ub)
+    R = nnv.PosLin.reach(S, method, [], 1, None, "linprog")
+    O = oracle.OStar(V, C, d, lb, ub)
+    E = oracle.reach_relaxed_star(O, method, 1.0)
+    elb, eub = oracle.estimate_ranges(O)
+    m1, m2 = oracle.relax_classify(elb, eub, method)
+    ni, idx, clb, cub = R.relu_info()
+    assert ni == m1.size and np.array_equal(idx, m2)           # classification + new-predicate order: exact
+    assert np.array_equal(R.V, E.V)                            # zeroing / one-hot columns: exact
+    compare_sets(R, E, "relu " + method)
+    assert np.array_equal(R.C[:3 + 2 * m2.size], E.C[:3 + 2 * m2.size])   # C0, C1, C2 rows are copies: exact
+    assert R.C.shape == (3 + 3 * m2.size, n + m2.size)
+
+
+def test_relu_ties_and_degenerate(nnv, oracle):
+    # hand-built bounds: ub == 0 -> inactive, lb == 0 -> active; equal sort keys keep index order
+    V = np.array([[-0.5, 0.5], [0.5, 0.5], [1.0, -3.0], [-1.0, 2.0], [2.0, 0.0], [-1.0, 0.0], [1.0, 3.0], [-1.0, -2.0]])
+    S = nnv.Star(V, np.zeros((1, 1)), np.zeros(1), [-1.0], [1.0])
+    for method in ("relax-star-area", "relax-star-range", "relax-star-static"):
+        R = nnv.PosLin.reach(S, method, [], 1)
+        E = oracle.reach_relaxed_star(oracle.OStar(V, np.zeros((1, 1)), np.zeros(1), [-1.0], [1.0]), method, 1.0)
+        ni, idx, _, _ = R.relu_info()
+        assert ni == 2
+        assert np.array_equal(R.V, E.V) and np.array_equal(R.C, E.C) and np.array_equal(R.d, E.d), method
+    # all active: identity, no new predicate; all inactive: zero set
+    G = 0.1 * np.random.RandomState(1).randn(20, 4)
+    for c, chk in ((5.0, lambda R, V: np.array_equal(R.V, V)), (-5.0, lambda R, V: not R.V.any())):
+        Vc = np.c_[np.full(20, c), G]
+        R = nnv.PosLin.reach(nnv.Star(Vc, np.zeros((1, 4)), np.zeros(1), -np.ones(4), np.ones(4)), "relax-star-area", [], 1)
+        assert R.nVar == 4 and R.C.shape == (1, 4) and chk(R, Vc)
+    with pytest.raises(ValueError, match="Invalid relax factor"):
+        nnv.PosLin.reach(S, "relax-star-area", [], 1.5)
+    with pytest.raises(ValueError, match="does not exist"):
+        nnv.PosLin.reach(S, "relax-star", [], 1)
+    with pytest.raises(ValueError):
+        nnv.PosLin.reach(S, "relax-star-area", [], 0.5)
+
+
+@pytest.mark.parametrize("method", ["relax-star-area", "relax-star-random"])
+def test_config1_full(nnv, method):
+    margins = []
+    run_both(1, method, margins=margins)
+    assert min(margins) > 1e-12
+
+
+def test_config2_full(nnv, oracle):
+    dev, ora, net = run_both(2, "relax-star-area")
+    dl, du = dev.estimateRanges()
+    ol, ou = oracle.output_ranges(ora)
+    assert_close(dl, ol, "output lb")
+    assert_close(du, ou, "output ub")
+
+
+def test_config3_full(nnv, oracle):
+    dev, ora, net = run_both(3, "relax-star-area")
+    dl, du = dev.estimateRanges()
+    ol, ou = oracle.output_ranges(ora)
+    assert_close(dl.reshape(-1), ol, "output lb")
+    assert_close(du.reshape(-1), ou, "output ub")
+
+
+def test_config4_shrunk(nnv):
+    run_both(4, "relax-star-area", shrink=4)
+    run_both(4, "relax-star-random", shrink=8)
+    # ub-lb has exact mathematical ties across positions of a conv channel: order checked up to ties
+    run_both(4, "relax-star-range", shrink=8, tie_tolerant=True)
+
+
+def test_config5_shrunk_batched(nnv, oracle):
+    dev, ora, net = run_both(5, "relax-star-area", shrink=4, check_constraints=False)
+    assert len(dev) == len(ora) == 4
+    run_both(5, "relax-star-random", shrink=8)
