@@ -114,7 +114,10 @@ __global__ __launch_bounds__(256) void conv2d_f64_kernel(const double* __restric
       const int idx = tid + q * 256;
       const int k2 = idx % (kKt / 2);
       const int j = idx / (kKt / 2);
-      if (idx < W_VEC) *reinterpret_cast<double2*>(&Wts[buf][j * LDW_S + 2 * k2]) = rw[q];
+      if (idx < W_VEC) {  // odd column stride: two 64-bit stores
+        Wts[buf][j * LDW_S + 2 * k2] = rw[q].x;
+        Wts[buf][j * LDW_S + 2 * k2 + 1] = rw[q].y;
+      }
     }
   };
 

@@ -4,24 +4,29 @@
 // column-major stores: the instruction's "b" operand carries 16 consecutive ROWS of W (the
 // memory-contiguous direction of C), its "a" operand 16 columns of V, so lane l, register r of
 // an accumulator holds C[row0 + l%16][col0 + l/16 + 4r] and lanes 0..15 store one 128-byte line.
+#include <algorithm>
+#include <cstdlib>
+#include <string>
+
 #include "internal.h"
 #include "mfma_tile.h"
 
 namespace nnvhip {
 
-// TM x TN output tile per 256-thread block, waves arranged WR x WC, each wave owning
+// TM x TN output tile per block of WR x WC waves, each wave owning
 // (TM/WR) x (TN/WC) = (16*FM) x (16*FN).
-template <int TM, int TN, int WR, int WC>
-__global__ __launch_bounds__(256) void gemm_f64_kernel(const double* __restrict__ A, int64_t lda,
+template <int TM, int TN, int WR, int WC, int KT>
+__global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __restrict__ A, int64_t lda,
                                                         const double* __restrict__ B, int64_t ldb,
                                                         double* __restrict__ C, int64_t ldc, int Mp, int64_t ncols,
-                                                        int Kp, const double* __restrict__ bias, int tiles_m) {
-  static_assert(WR * WC == 4, "four waves per block");
+                                                        int Kp, const double* __restrict__ bias, int tiles_m,
+                                                        int ksplit, double* __restrict__ part) {
+  constexpr int NT = 64 * WR * WC;  // threads per block
   constexpr int FM = TM / WR / 16;
   constexpr int FN = TN / WC / 16;
   constexpr int LDA_S = TM + kPadRow;  // Ws[k][row]
-  constexpr int LDB_S = kKt + kPadK;   // Vs[col][k]
-  __shared__ double Ws[2][kKt * LDA_S];
+  constexpr int LDB_S = KT + kPadK;    // Vs[col][k]
+  __shared__ double Ws[2][KT * LDA_S];
   __shared__ double Vs[2][TN * LDB_S];
 
   const int tid = threadIdx.x;
@@ -35,16 +40,16 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(const double* __restrict_
   const int64_t n0 = (bid / tiles_m) * TN;
 
   // ---- global -> register staging ----------------------------------------------------------
-  constexpr int A_VEC = TM * kKt / 2;          // double2 elements in a W tile
-  constexpr int A_PASS = (A_VEC + 255) / 256;
-  constexpr int B_VEC = TN * kKt / 2;
-  constexpr int B_PASS = (B_VEC + 255) / 256;
+  constexpr int A_VEC = TM * KT / 2;           // double2 elements in a W tile
+  constexpr int A_PASS = (A_VEC + NT - 1) / NT;
+  constexpr int B_VEC = TN * KT / 2;
+  constexpr int B_PASS = (B_VEC + NT - 1) / NT;
   double2 ra[A_PASS], rb[B_PASS];
 
   auto load_tiles = [&](int k0) {
 #pragma unroll
     for (int p = 0; p < A_PASS; ++p) {
-      int idx = tid + p * 256;
+      int idx = tid + p * NT;
       int i2 = idx % (TM / 2);
       int k = idx / (TM / 2);
       int row = m0 + 2 * i2;
@@ -54,9 +59,9 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(const double* __restrict_
     }
 #pragma unroll
     for (int p = 0; p < B_PASS; ++p) {
-      int idx = tid + p * 256;
-      int k2 = idx % (kKt / 2);
-      int j = idx / (kKt / 2);
+      int idx = tid + p * NT;
+      int k2 = idx % (KT / 2);
+      int j = idx / (KT / 2);
       int64_t col = n0 + j;
       double2 v = make_double2(0.0, 0.0);
       if (idx < B_VEC && col < ncols) v = *reinterpret_cast<const double2*>(B + (k0 + 2 * k2) + col * ldb);
@@ -66,17 +71,20 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(const double* __restrict_
   auto store_tiles = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < A_PASS; ++p) {
-      int idx = tid + p * 256;
+      int idx = tid + p * NT;
       int i2 = idx % (TM / 2);
       int k = idx / (TM / 2);
       if (idx < A_VEC) *reinterpret_cast<double2*>(&Ws[buf][k * LDA_S + 2 * i2]) = ra[p];
     }
 #pragma unroll
     for (int p = 0; p < B_PASS; ++p) {
-      int idx = tid + p * 256;
-      int k2 = idx % (kKt / 2);
-      int j = idx / (kKt / 2);
-      if (idx < B_VEC) *reinterpret_cast<double2*>(&Vs[buf][j * LDB_S + 2 * k2]) = rb[p];
+      int idx = tid + p * NT;
+      int k2 = idx % (KT / 2);
+      int j = idx / (KT / 2);
+      if (idx < B_VEC) {  // odd column stride: two 64-bit stores
+        Vs[buf][j * LDB_S + 2 * k2] = rb[p].x;
+        Vs[buf][j * LDB_S + 2 * k2 + 1] = rb[p].y;
+      }
     }
   };
 
@@ -86,16 +94,24 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(const double* __restrict_
 #pragma unroll
     for (int j = 0; j < FN; ++j) acc[i][j] = double4_t{0.0, 0.0, 0.0, 0.0};
 
-  const int nk = Kp / kKt;
-  load_tiles(0);
+  // split-K: block row blockIdx.y owns the K-tiles [kt0, kt1) and writes a partial product
+  const int nk_all = Kp / KT;
+  const int kt0 = (int)((int64_t)nk_all * blockIdx.y / ksplit);
+  const int kt1 = (int)((int64_t)nk_all * (blockIdx.y + 1) / ksplit);
+  load_tiles(kt0 * KT);
   store_tiles(0);
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) load_tiles((kt + 1) * kKt);
-    mfma_tile_k16<FM, FN>(&Ws[cur][wr * (TM / WR)], LDA_S, &Vs[cur][(wc * (TN / WC)) * LDB_S], LDB_S, lane, acc);
-    if (kt + 1 < nk) store_tiles(cur ^ 1);
+  for (int kt = kt0; kt < kt1; ++kt) {
+    const int cur = (kt - kt0) & 1;
+    if (kt + 1 < kt1) load_tiles((kt + 1) * KT);
+    mfma_tile_k16<FM, FN, KT>(&Ws[cur][wr * (TM / WR)], LDA_S, &Vs[cur][(wc * (TN / WC)) * LDB_S], LDB_S, lane, acc);
+    if (kt + 1 < kt1) store_tiles(cur ^ 1);
     __syncthreads();
+  }
+  if (ksplit > 1) {  // partial sums go to the workspace (ld = Mp); bias is added by the reduction
+    C = part + (int64_t)blockIdx.y * Mp * ncols;
+    ldc = Mp;
+    bias = nullptr;
   }
 
   // ---- epilogue: bias on column 0, 128-byte line stores --------------------------------------
@@ -120,15 +136,45 @@ __global__ __launch_bounds__(256) void gemm_f64_kernel(const double* __restrict_
   }
 }
 
-template <int TM, int TN, int WR, int WC>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __restrict__ part, int ksplit, int Mp,
+                                                             int64_t ncols, double* __restrict__ C, int64_t ldc,
+                                                             const double* __restrict__ bias) {
+  const int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t total = (int64_t)Mp * ncols;
+  if (t >= total) return;
+  double s = 0.0;
+  for (int k = 0; k < ksplit; ++k) s += part[(int64_t)k * total + t];
+  const int64_t col = t / Mp;
+  const int row = (int)(t - col * Mp);
+  if (bias != nullptr && col == 0) s = s + bias[row];
+  C[row + col * ldc] = s;
+}
+
+template <int TM, int TN, int WR, int WC, int KT>
 static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
                       int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias) {
   int64_t tiles_m = ceil_div(Mp, TM);
   int64_t tiles_n = ceil_div(ncols, TN);
   int64_t blocks = tiles_m * tiles_n;
   if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large for one launch");
-  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, A, lda, B,
-                     ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m);
+  // Split-K when the output has too few tiles to occupy the chip: partial products into a workspace,
+  // summed in split order by a second kernel (deterministic, no floating-point atomics).
+  const int64_t nk = Kp / KT;
+  int64_t ksplit = 1;
+  if (blocks < 448 && nk >= 8) ksplit = std::min<int64_t>(std::min<int64_t>(16, nk / 4), ceil_div(640, blocks));
+  if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
+  BufRef ws;
+  if (ksplit > 1) NNV_TRY(ctx->alloc(sizeof(double) * ksplit * Mp * ncols, &ws));
+  size_t dyn = 0;
+  if (const char* e = getenv("NNVHIP_GEMM_DYNLDS")) dyn = (size_t)atoi(e);
+  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)blocks, (unsigned)ksplit), dim3(64 * WR * WC), dyn,
+                     ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)ksplit,
+                     ws ? ws->as<double>() : nullptr);
+  if (ksplit > 1) {
+    const int64_t total = Mp * ncols;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream,
+                       ws->as<double>(), (int)ksplit, (int)Mp, ncols, C, ldc, bias);
+  }
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }
@@ -140,16 +186,34 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
   if (Mp >= (int64_t(1) << 31) || Kp >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large");
   if (ncols == 0) return NNVHIP_OK;
   // Tile choice: the largest tile that still yields a few blocks per CU; skinny outputs (the last
-  // layer has 10 rows) get a 16-row tile.
+  // layer has 10 rows) get a 16-row tile.  K must be a multiple of the K-tile (16 or 32).
+#define NNV_GEMM(TM, TN, WR, WC, KT) launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias)
   const int64_t kCUs = 256;
-  if (Mp <= 16) return launch_cfg<16, 256, 1, 4>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias);
-  if (Mp <= 32) return launch_cfg<32, 128, 1, 4>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias);
-  int64_t b128 = ceil_div(Mp, 128) * ceil_div(ncols, 128);
-  if (b128 >= 3 * kCUs) return launch_cfg<128, 128, 2, 2>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias);
-  int64_t b64 = ceil_div(Mp, 64) * ceil_div(ncols, 64);
-  if (b64 >= 2 * kCUs || Mp % 64 == 0 || Mp > 256)
-    return launch_cfg<64, 64, 2, 2>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias);
-  return launch_cfg<32, 128, 1, 4>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias);
+  const bool k32 = Kp % 32 == 0;
+  if (const char* e = getenv("NNVHIP_GEMM_TILE")) {  // tuning knob
+    const std::string t(e);
+    if (t == "128x128x16") return NNV_GEMM(128, 128, 2, 2, 16);
+    if (t == "128x128x16w8") return NNV_GEMM(128, 128, 2, 4, 16);
+    if (t == "128x64x16w8") return NNV_GEMM(128, 64, 4, 2, 16);
+    if (t == "64x64x16w8") return NNV_GEMM(64, 64, 2, 4, 16);
+    if (t == "64x128x16w8") return NNV_GEMM(64, 128, 2, 4, 16);
+    if (k32 && t == "64x64x32w8") return NNV_GEMM(64, 64, 2, 4, 32);
+    if (k32 && t == "128x64x32w8") return NNV_GEMM(128, 64, 4, 2, 32);
+    if (t == "128x64x16") return NNV_GEMM(128, 64, 2, 2, 16);
+    if (t == "64x64x16") return NNV_GEMM(64, 64, 2, 2, 16);
+    if (t == "32x128x16") return NNV_GEMM(32, 128, 1, 4, 16);
+    if (k32 && t == "128x64x32") return NNV_GEMM(128, 64, 2, 2, 32);
+    if (k32 && t == "64x64x32") return NNV_GEMM(64, 64, 2, 2, 32);
+  }
+  if (Mp <= 16) return NNV_GEMM(16, 64, 1, 4, 16);
+  if (Mp <= 32) return NNV_GEMM(32, 128, 1, 4, 16);
+  // eight waves per block keep two waves per SIMD issuing MFMAs even with one block per CU
+  const int64_t b128 = ceil_div(Mp, 128) * ceil_div(ncols, 128);
+  if (b128 >= 2 * kCUs) return NNV_GEMM(128, 128, 2, 4, 16);
+  const int64_t b12864 = ceil_div(Mp, 128) * ceil_div(ncols, 64);
+  if (b12864 >= 4 * kCUs) return NNV_GEMM(128, 64, 4, 2, 16);
+  return NNV_GEMM(64, 64, 2, 4, 16);
+#undef NNV_GEMM
 }
 
 __global__ void bias_columns_kernel(double* const* __restrict__ cols, const double* __restrict__ bias, int Mp) {

@@ -92,20 +92,28 @@ __global__ __launch_bounds__(256) void ranges_partial_kernel(const RangeDesc* __
   }
 }
 
+// Combines the chunk partials in chunk order.  64 rows per block; the four sums of a row are handled
+// by four different waves so that the dependent add chains are short.
 __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
   if (d.chunks == 1) return;
-  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= d.ld) return;
-  double s[4] = {0, 0, 0, 0};
-  for (int c = 0; c < d.chunks; ++c) {
-    const double* p = d.part + ((int64_t)c * 4) * d.ld + r;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) s[q] += p[q * d.ld];
+  const int lane = threadIdx.x & 63;
+  const int q = threadIdx.x >> 6;
+  const int64_t r = (int64_t)blockIdx.x * 64 + lane;
+  __shared__ double sums[4][64];
+  double s = 0.0;
+  if (r < d.ld) {
+    const double* p = d.part + (int64_t)q * d.ld + r;
+#pragma unroll 8
+    for (int c = 0; c < d.chunks; ++c) s += p[(int64_t)c * 4 * d.ld];
   }
-  const double c0 = d.V[r];
-  d.lb[r] = (c0 + s[0]) + s[1];
-  d.ub[r] = (c0 + s[2]) + s[3];
+  sums[q][lane] = s;
+  __syncthreads();
+  if (q == 0 && r < d.ld) {
+    const double c0 = d.V[r];
+    d.lb[r] = (c0 + sums[0][lane]) + sums[1][lane];
+    d.ub[r] = (c0 + sums[2][lane]) + sums[3][lane];
+  }
 }
 
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
@@ -162,7 +170,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   dim3 grid((unsigned)row_blocks, (unsigned)chunks, (unsigned)nset);
   hipLaunchKernelGGL(ranges_partial_kernel, grid, dim3(256), 0, ctx->stream, table, descs[0]);
   if (chunks > 1)
-    hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 256), 1, (unsigned)nset), dim3(256), 0,
+    hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,
                        ctx->stream, table, descs[0]);
   NNV_HIP_TRY(hipGetLastError());
   for (int64_t i = 0; i < nset; ++i) {

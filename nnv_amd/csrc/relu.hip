@@ -29,6 +29,7 @@ struct ReluDesc {
   int32_t* cross_idx;  // crossing neuron indices in new-predicate order
   int32_t* asc_idx;    // crossing neuron indices in ascending order (sort orders only)
   double* key;         // sort keys, ascending-index order
+  int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
   double* rows;        // saved crossing rows of the pre-ReLU [c V]: m x ncols_in, ld = ld_rows
   double* lbub;        // lb then ub (offset ld_rows) of the crossing neurons, new-predicate order
@@ -79,10 +80,10 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
       idx_out[pos] = r;
       if (d.order == NNVHIP_ORDER_INDEX) {
         d.cls[r] = pos;
-      } else if (d.order == NNVHIP_ORDER_AREA) {
-        d.key[pos] = 0.5 * (fabs(u) * fabs(l));  // areas = 0.5*(abs(ub).*abs(lb))
       } else {
-        d.key[pos] = u - l;  // ub - lb
+        // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb
+        d.key[pos] = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : u - l;
+        d.rank[pos] = 0;
       }
     } else if (valid) {
       d.cls[r] = inactive ? kZero : kKeep;
@@ -100,30 +101,44 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
 
 // Stable descending sort by counting: rank(i) = #{j : key_j > key_i or (key_j == key_i and j < i)}.
 // j < i in the ascending list is "smaller neuron index", which is what MATLAB's stable sort keeps.
+// The m x m comparison grid is cut into 256 x 256 tiles, one block each; partial counts are added
+// with integer atomics (exact, order-independent).
 __global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
   const ReluDesc d = table ? table[blockIdx.z] : one;
   const int m = d.m;
-  if ((int)(blockIdx.x * 256) >= m) return;
-  const int i = blockIdx.x * 256 + threadIdx.x;
+  const int i0 = blockIdx.x * 256, j0 = blockIdx.y * 256;
+  if (i0 >= m || j0 >= m) return;
+  const int i = i0 + threadIdx.x;
   const double ki = i < m ? d.key[i] : 0.0;
   __shared__ double tile[256];
-  int rank = 0;
-  for (int j0 = 0; j0 < m; j0 += 256) {
-    const int j = j0 + threadIdx.x;
-    tile[threadIdx.x] = j < m ? d.key[j] : 0.0;
-    __syncthreads();
-    const int lim = min(256, m - j0);
+  const int j = j0 + threadIdx.x;
+  tile[threadIdx.x] = j < m ? d.key[j] : 0.0;
+  __syncthreads();
+  const int lim = min(256, m - j0);
+  int cnt = 0;
+  if (lim == 256) {
+#pragma unroll 8
+    for (int t = 0; t < 256; ++t) {
+      const double kj = tile[t];
+      cnt += (kj > ki || (kj == ki && (j0 + t) < i)) ? 1 : 0;
+    }
+  } else {
     for (int t = 0; t < lim; ++t) {
       const double kj = tile[t];
-      rank += (kj > ki || (kj == ki && (j0 + t) < i)) ? 1 : 0;
+      cnt += (kj > ki || (kj == ki && (j0 + t) < i)) ? 1 : 0;
     }
-    __syncthreads();
   }
-  if (i < m) {
-    const int neuron = d.asc_idx[i];
-    d.cross_idx[rank] = neuron;
-    d.cls[neuron] = rank;
-  }
+  if (i < m && cnt) atomicAdd(&d.rank[i], cnt);
+}
+
+__global__ __launch_bounds__(256) void relu_scatter_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.z] : one;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= d.m) return;
+  const int neuron = d.asc_idx[i];
+  const int r = d.rank[i];
+  d.cross_idx[r] = neuron;
+  d.cls[neuron] = r;
 }
 
 constexpr int kApplyRows = 128;  // 64 lanes x 2 rows, the four waves interleave columns
@@ -186,12 +201,13 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const bool sorted = order != NNVHIP_ORDER_INDEX;
 
   // scratch shared by all sets: cls | counts ; cross_idx is kept (it becomes the node's index list)
-  BufRef cls_buf, cnt_buf, asc_buf, key_buf;
+  BufRef cls_buf, cnt_buf, asc_buf, key_buf, rank_buf;
   NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &cls_buf));
   NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * count, &cnt_buf));
   if (sorted) {
     NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &asc_buf));
     NNV_TRY(ctx->alloc(sizeof(double) * ld * count, &key_buf));
+    NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &rank_buf));
   }
   std::vector<BufRef> idx_bufs(count);
   std::vector<ReluDesc> descs(count);
@@ -208,6 +224,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.cross_idx = idx_bufs[i]->as<int32_t>();
     d.asc_idx = sorted ? asc_buf->as<int32_t>() + ld * i : nullptr;
     d.key = sorted ? key_buf->as<double>() + ld * i : nullptr;
+    d.rank = sorted ? rank_buf->as<int32_t>() + ld * i : nullptr;
     d.counts = cnt_buf->as<int32_t>() + 2 * i;
     d.ld = ld;
     d.N = (int32_t)N;
@@ -278,9 +295,12 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
-  if (sorted && max_m > 0)
-    hipLaunchKernelGGL(relu_rank_kernel, dim3((unsigned)ceil_div(max_m, 256), 1, (unsigned)count), dim3(256), 0,
-                       ctx->stream, table, descs[0]);
+  if (sorted && max_m > 0) {
+    const unsigned t = (unsigned)ceil_div(max_m, 256);
+    if (t > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "too many crossing neurons for the sort kernel");
+    hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
+    hipLaunchKernelGGL(relu_scatter_kernel, dim3(t, 1, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
+  }
   hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(256), 0,
                      ctx->stream, table, descs[0]);
   NNV_HIP_TRY(hipGetLastError());
