@@ -85,8 +85,12 @@ def main():
     updates = count_updates(shapes)
     value = updates / (wall / args.steps)
 
-    # ---- per-kernel timing with HIP events on the library's stream ------------------------------
+    # ---- per-layer and per-kernel timing with HIP events on the library's stream -----------------
+    # set_timing brackets every layer call (NN.reachTime) and, separately, every launch of the two
+    # MFMA kernels with their own event pair, so the kernel's duration excludes host gaps.
     ctx.set_timing(True)
+    ctx.kernel_time(0)
+    ctx.kernel_time(1)
     per_layer = np.zeros(len(net.Layers))
     reps = max(5, min(args.steps, 20))
     for _ in range(reps):
@@ -95,10 +99,12 @@ def main():
             rs = L.reach(rs, args.method, [], 1, None, "linprog")
             per_layer[i] += ctx.last_op_time_ms()
     per_layer /= reps
+    gemm_ms, gemm_launches, _ = ctx.kernel_time(0)
+    conv_ms, conv_launches, _ = ctx.kernel_time(1)
     ctx.set_timing(False)
 
-    # dominant kernel: the GEMM of the FC layers with more than 32 output rows (one launch per layer)
-    gemm_flop, gemm_ms, gemm_launches = 0.0, 0.0, 0
+    # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
+    gemm_flop = conv_flop = 0.0
     relu_bytes, relu_ms = 0.0, 0.0
     layer_report = []
     prev_sets = dev_in if isinstance(dev_in, list) else [dev_in]
@@ -110,10 +116,8 @@ def main():
             cols = sum(s._h.dims()[1] + 1 for s in outs)
             flop = 2.0 * M * K * cols
             entry["dense_tflops"] = round(flop / (per_layer[i] * 1e-3) / 1e12, 3)
-            if M > 32:
+            if M > 32:  # the 64-row-tile kernel; skinnier layers use another instantiation
                 gemm_flop += flop
-                gemm_ms += per_layer[i]
-                gemm_launches += 1
         elif Ld["type"] == "conv":
             fh, fw, cin, cout = Ld["W"].shape
             flop = 0.0
@@ -121,12 +125,14 @@ def main():
                 N, n, _ = s._h.dims()
                 flop += 2.0 * (N // cout) * cout * fh * fw * cin * (n + 1)
             entry["dense_tflops"] = round(flop / (per_layer[i] * 1e-3) / 1e12, 3)
+            conv_flop += flop
         else:
             b = 0.0
             for sp, so in zip(prev_sets, outs):
                 N, n, _ = sp._h.dims()
                 m = so._h.dims()[1] - n
                 # estimateRanges read of V + masked copy read of V + write of the N x (n+1+m) output
+                # + the m saved crossing rows
                 b += 8.0 * N * (n + 1) * 2 + 8.0 * N * (n + 1 + m) + 8.0 * m * (n + 1)
             entry["algo_GBps"] = round(b / (per_layer[i] * 1e-3) / 1e9, 1)
             relu_bytes += b
@@ -134,19 +140,32 @@ def main():
         layer_report.append(entry)
         prev_sets = outs
 
-    if gemm_launches:
-        achieved = gemm_flop / (gemm_ms * 1e-3) / 1e12
-        roofline = {"kernel": "gemm_f64_kernel", "bound": "mfma", "achieved": round(achieved, 3),
-                    "peak": FP64_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / FP64_MFMA_PEAK_TFLOPS, 4),
-                    "traffic": None, "launches_per_step": gemm_launches,
-                    "avg_launch_ms": round(gemm_ms / gemm_launches, 4),
-                    "flop_per_launch": gemm_flop / gemm_launches}
+    def mfma_roofline(name, flop_per_step, ms_total, launches):
+        ach = flop_per_step * reps / (ms_total * 1e-3) / 1e12
+        return {"kernel": name, "bound": "mfma", "achieved": round(ach, 3), "peak": FP64_MFMA_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(ach / FP64_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                "launches_per_step": launches // reps, "avg_launch_ms": round(ms_total / launches, 5),
+                "flop_per_launch": flop_per_step * reps / launches}
+
+    if conv_launches and conv_ms >= gemm_ms:
+        roofline = mfma_roofline("conv2d_f64_kernel", conv_flop, conv_ms, conv_launches)
+        if gemm_launches:
+            roofline["fc_gemm"] = mfma_roofline("gemm_f64_kernel", gemm_flop, gemm_ms, gemm_launches)
+    elif gemm_launches:
+        roofline = mfma_roofline("gemm_f64_kernel", gemm_flop, gemm_ms, gemm_launches)
+        if conv_launches:
+            roofline["conv"] = mfma_roofline("conv2d_f64_kernel", conv_flop, conv_ms, conv_launches)
     else:
         achieved = relu_bytes / (relu_ms * 1e-3) / 1e9
         roofline = {"kernel": "relu step", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None}
     if relu_ms > 0:
         roofline["relu_step_algo_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
+        roofline["relu_step_frac_of_hbm_peak"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+
+    # practical HBM ceiling on this box: a plain copy kernel over 1 GiB (read + write bytes)
+    roofline["measured_copy_GBps"] = round(ctx.probe_copy_bandwidth(1 << 30, 5), 1)
+    ctx.trim_pool()
 
     # ---- CPU baseline: the oracle on this host -------------------------------------------------
     cpu = None

@@ -66,6 +66,19 @@ int nnvhip_synchronize(nnvhip_ctx* ctx);
  * Timing is off by default; enabling it makes this call wait for the layer to finish. */
 int nnvhip_set_timing(nnvhip_ctx* ctx, int enabled);
 int nnvhip_last_op_time_ms(nnvhip_ctx* ctx, double* ms);
+/* Measurement hook (no counterpart in the reference): while timing is enabled, every launch of an
+ * MFMA kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
+ * dense GEMM kernel of the FC layers (tiles of at least 64 rows); which = 1: implicit-GEMM
+ * convolution kernel.  Returns accumulated kernel time, launch count and dense flop executed
+ * (GEMM: 2*Mp*Kp*ncols with M, K padded to 16; conv: 2*Ho*Wo*Cout*FH*FW*Cin*(n+1)) since the last
+ * reset. */
+int nnvhip_kernel_time(nnvhip_ctx* ctx, int which, double* total_ms, int64_t* launches, double* total_flop,
+                       int reset);
+/* Measurement hook (no counterpart in the reference): runs a plain device-to-device copy kernel over
+ * `bytes` (reps + 1 times) and returns the achieved read+write bandwidth of the timed reps in GB/s -
+ * the practical HBM ceiling on this box, and the known-size kernel hardware counters are
+ * calibrated against. */
+int nnvhip_probe_copy_bandwidth(nnvhip_ctx* ctx, int64_t bytes, int reps, double* gbytes_per_s);
 /* Returns every cached device block of the pool to the driver (hipFree). */
 int nnvhip_trim_pool(nnvhip_ctx* ctx);
 /* Bytes currently handed out by / cached in the pool. */

@@ -15,7 +15,8 @@ ORDER_INDEX, ORDER_AREA, ORDER_RANGE = 0, 1, 2
 # every entry point declared in include/nnvhip.h
 SYMBOLS = [
     "nnvhip_create", "nnvhip_destroy", "nnvhip_last_error", "nnvhip_synchronize", "nnvhip_set_timing",
-    "nnvhip_last_op_time_ms", "nnvhip_trim_pool", "nnvhip_pool_stats", "nnvhip_star_create",
+    "nnvhip_last_op_time_ms", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
+    "nnvhip_trim_pool", "nnvhip_pool_stats", "nnvhip_star_create",
     "nnvhip_star_from_box", "nnvhip_star_retain", "nnvhip_star_release", "nnvhip_star_dims",
     "nnvhip_star_fetch_V", "nnvhip_star_fetch_pred_bounds", "nnvhip_star_fetch_constraints",
     "nnvhip_star_relu_counts", "nnvhip_star_fetch_crossing", "nnvhip_estimate_ranges",
@@ -54,6 +55,8 @@ def load():
         "nnvhip_synchronize": [p],
         "nnvhip_set_timing": [p, C.c_int],
         "nnvhip_last_op_time_ms": [p, C.POINTER(dbl)],
+        "nnvhip_kernel_time": [p, C.c_int, C.POINTER(dbl), pi64, C.POINTER(dbl), C.c_int],
+        "nnvhip_probe_copy_bandwidth": [p, i64, C.c_int, C.POINTER(dbl)],
         "nnvhip_trim_pool": [p],
         "nnvhip_pool_stats": [p, pi64, pi64],
         "nnvhip_star_create": [p, i64, i64, p, p, p, p, p, i64, pp],
@@ -132,6 +135,19 @@ class Context:
         ms = C.c_double()
         check(self.lib.nnvhip_last_op_time_ms(self.handle, C.byref(ms)))
         return ms.value
+
+    def kernel_time(self, which, reset=True):
+        """(total ms, launches, dense flop) of an MFMA kernel group (0 = FC GEMM, 1 = convolution)
+        accumulated while timing was enabled."""
+        ms, n, fl = C.c_double(), C.c_int64(), C.c_double()
+        check(self.lib.nnvhip_kernel_time(self.handle, int(which), C.byref(ms), C.byref(n), C.byref(fl), 1 if reset else 0))
+        return ms.value, n.value, fl.value
+
+    def probe_copy_bandwidth(self, nbytes=1 << 30, reps=5) -> float:
+        """Achieved read+write GB/s of a plain copy kernel over nbytes (practical HBM ceiling)."""
+        g = C.c_double()
+        check(self.lib.nnvhip_probe_copy_bandwidth(self.handle, int(nbytes), int(reps), C.byref(g)))
+        return g.value
 
     def pool_stats(self):
         a, b = C.c_int64(), C.c_int64()

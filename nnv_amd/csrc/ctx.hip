@@ -114,6 +114,24 @@ int nnvhip_ctx::upload(const void* host, size_t bytes, BufRef* out) {
   return NNVHIP_OK;
 }
 
+int nnvhip_ctx::kernel_timer_begin(bool on) {
+  if (on) NNV_HIP_TRY(hipEventRecord(kev0, stream));
+  return NNVHIP_OK;
+}
+
+int nnvhip_ctx::kernel_timer_end(bool on, int which, double flop) {
+  if (on) {  // events directly around one kernel: its duration alone, as a profiler reports it
+    NNV_HIP_TRY(hipEventRecord(kev1, stream));
+    NNV_HIP_TRY(hipEventSynchronize(kev1));
+    float ms = 0.f;
+    NNV_HIP_TRY(hipEventElapsedTime(&ms, kev0, kev1));
+    kern_ms[which] += ms;
+    kern_launches[which] += 1;
+    kern_flop[which] += flop;
+  }
+  return NNVHIP_OK;
+}
+
 int nnvhip_ctx::begin_op() {
   if (timing) NNV_HIP_TRY(hipEventRecord(ev0, stream));
   return NNVHIP_OK;
@@ -155,6 +173,8 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
+  NNV_HIP_TRY(hipEventCreate(&c->kev0));
+  NNV_HIP_TRY(hipEventCreate(&c->kev1));
   *out = c;
   return NNVHIP_OK;
 }
@@ -168,6 +188,8 @@ int nnvhip_destroy(nnvhip_ctx* c) {
   if (c->pinned) (void)hipHostFree(c->pinned);
   (void)hipEventDestroy(c->ev0);
   (void)hipEventDestroy(c->ev1);
+  (void)hipEventDestroy(c->kev0);
+  (void)hipEventDestroy(c->kev1);
   (void)hipStreamDestroy(c->stream);
   delete c;
   return NNVHIP_OK;
@@ -188,6 +210,49 @@ int nnvhip_set_timing(nnvhip_ctx* c, int enabled) {
 int nnvhip_last_op_time_ms(nnvhip_ctx* c, double* ms) {
   if (!c || !ms) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   *ms = c->last_ms;
+  return NNVHIP_OK;
+}
+
+int nnvhip_kernel_time(nnvhip_ctx* c, int which, double* total_ms, int64_t* launches, double* total_flop, int reset) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  if (which < 0 || which > 1) NNV_FAIL(NNVHIP_ERR_ARG, "unknown kernel group %d", which);
+  if (total_ms) *total_ms = c->kern_ms[which];
+  if (launches) *launches = c->kern_launches[which];
+  if (total_flop) *total_flop = c->kern_flop[which];
+  if (reset) {
+    c->kern_ms[which] = 0.0;
+    c->kern_launches[which] = 0;
+    c->kern_flop[which] = 0.0;
+  }
+  return NNVHIP_OK;
+}
+
+__global__ __launch_bounds__(256) void probe_copy_kernel(const double2* __restrict__ in, double2* __restrict__ out,
+                                                          int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += stride) out[i] = in[i];
+}
+
+int nnvhip_probe_copy_bandwidth(nnvhip_ctx* c, int64_t bytes, int reps, double* gbytes_per_s) {
+  CHECK_CTX(c);
+  if (bytes < 16 || reps < 1 || !gbytes_per_s) NNV_FAIL(NNVHIP_ERR_ARG, "invalid argument");
+  bytes &= ~int64_t(15);
+  BufRef a, b;
+  NNV_TRY(c->alloc((size_t)bytes, &a));
+  NNV_TRY(c->alloc((size_t)bytes, &b));
+  NNV_HIP_TRY(hipMemsetAsync(a->ptr, 0, (size_t)bytes, c->stream));
+  const int64_t n = bytes / 16;
+  const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(n, 256), 256 * 32);
+  hipLaunchKernelGGL(probe_copy_kernel, dim3(blocks), dim3(256), 0, c->stream, a->as<double2>(), b->as<double2>(), n);
+  NNV_HIP_TRY(hipEventRecord(c->kev0, c->stream));
+  for (int i = 0; i < reps; ++i)
+    hipLaunchKernelGGL(probe_copy_kernel, dim3(blocks), dim3(256), 0, c->stream, a->as<double2>(), b->as<double2>(), n);
+  NNV_HIP_TRY(hipEventRecord(c->kev1, c->stream));
+  NNV_HIP_TRY(hipEventSynchronize(c->kev1));
+  NNV_HIP_TRY(hipGetLastError());
+  float ms = 0.f;
+  NNV_HIP_TRY(hipEventElapsedTime(&ms, c->kev0, c->kev1));
+  *gbytes_per_s = 2.0 * (double)bytes * reps / (ms * 1e-3) / 1e9;  // bytes read + bytes written
   return NNVHIP_OK;
 }
 

@@ -165,11 +165,12 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
   BufRef ws;
   if (ksplit > 1) NNV_TRY(ctx->alloc(sizeof(double) * ksplit * Mp * ncols, &ws));
-  size_t dyn = 0;
-  if (const char* e = getenv("NNVHIP_GEMM_DYNLDS")) dyn = (size_t)atoi(e);
-  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)blocks, (unsigned)ksplit), dim3(64 * WR * WC), dyn,
+  const bool timed = ctx->timing && TM >= 64;
+  NNV_TRY(ctx->kernel_timer_begin(timed));
+  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)blocks, (unsigned)ksplit), dim3(64 * WR * WC), 0,
                      ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)ksplit,
                      ws ? ws->as<double>() : nullptr);
+  NNV_TRY(ctx->kernel_timer_end(timed, 0, 2.0 * (double)Mp * (double)Kp * (double)ncols));
   if (ksplit > 1) {
     const int64_t total = Mp * ncols;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream,

@@ -68,8 +68,8 @@ struct ConsNode {
   BufRef C0;
   int64_t ldc = 0;
   BufRef d0;
-  // ReLU node: the m crossing rows of the pre-ReLU [c V] (m x (n_before+1), ld = ld_rows), in
-  // new-predicate order, their bounds and neuron indices
+  // ReLU node: the m crossing rows of the pre-ReLU [c V] (m x (n_before+1), ld = ld_rows) in
+  // ascending neuron order (coalesced to write), plus bounds and indices in new-predicate order
   int64_t m = 0;
   int64_t n_before = 0;
   BufRef rows;            // possibly shared by the sets of one array: data starts at rows_off
@@ -77,7 +77,8 @@ struct ConsNode {
   int64_t ld_rows = 0;
   BufRef lbub;            // lb[0..m), then ub[0..m) at offset ld_rows; data starts at lbub_off
   int64_t lbub_off = 0;
-  BufRef index;           // int32[m]
+  BufRef index;           // int32[m]: crossing neuron indices in new-predicate order
+  BufRef rowmap;          // int32[m] at element offset lbub_off: new-predicate number -> row of `rows`
 };
 using ConsRef = std::shared_ptr<ConsNode>;
 
@@ -99,6 +100,14 @@ struct nnvhip_ctx {
   bool timing = false;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   double last_ms = 0.0;
+  // timing of the dominant kernel alone (events directly around its launch), per instantiation group
+  hipEvent_t kev0 = nullptr, kev1 = nullptr;
+  // [0] dense MFMA GEMM (tiles of at least 64 rows), [1] implicit-GEMM convolution
+  double kern_ms[2] = {0.0, 0.0};
+  int64_t kern_launches[2] = {0, 0};
+  double kern_flop[2] = {0.0, 0.0};
+  int kernel_timer_begin(bool on);
+  int kernel_timer_end(bool on, int which, double flop);
 
   int alloc(size_t bytes, nnvhip::BufRef* out);
   void release_block(void* p, size_t bytes);

@@ -40,21 +40,31 @@ __global__ __launch_bounds__(256) void ranges_partial_kernel(const RangeDesc* __
   double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
   if (active) {
     const double* col = d.V + r0;
-#pragma unroll 4
-    for (int j = j0 + wave; j < j1; j += 4) {
-      const double2 v = *reinterpret_cast<const double2*>(col + (int64_t)j * d.ld);
-      const double pl = d.plb[j - 1];
-      const double pu = d.pub[j - 1];
-      const double px = fmax(v.x, 0.0), nx = fmin(v.x, 0.0);
-      const double py = fmax(v.y, 0.0), ny = fmin(v.y, 0.0);
-      xmin1.x = fma(px, pl, xmin1.x);
-      xmin1.y = fma(py, pl, xmin1.y);
-      xmax1.x = fma(px, pu, xmax1.x);
-      xmax1.y = fma(py, pu, xmax1.y);
-      xmin2.x = fma(nx, pu, xmin2.x);
-      xmin2.y = fma(ny, pu, xmin2.y);
-      xmax2.x = fma(nx, pl, xmax2.x);
-      xmax2.y = fma(ny, pl, xmax2.y);
+    // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
+    for (int jb = j0 + 4 * wave; jb < j1; jb += 16) {
+      double2 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        v[u] = make_double2(0.0, 0.0);
+        if (jb + u < j1) v[u] = *reinterpret_cast<const double2*>(col + (int64_t)(jb + u) * d.ld);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = jb + u;
+        if (j >= j1) break;
+        const double pl = d.plb[j - 1];
+        const double pu = d.pub[j - 1];
+        const double px = fmax(v[u].x, 0.0), nx = fmin(v[u].x, 0.0);
+        const double py = fmax(v[u].y, 0.0), ny = fmin(v[u].y, 0.0);
+        xmin1.x = fma(px, pl, xmin1.x);
+        xmin1.y = fma(py, pl, xmin1.y);
+        xmax1.x = fma(px, pu, xmax1.x);
+        xmax1.y = fma(py, pu, xmax1.y);
+        xmin2.x = fma(nx, pu, xmin2.x);
+        xmin2.y = fma(ny, pu, xmin2.y);
+        xmax2.x = fma(nx, pl, xmax2.x);
+        xmax2.y = fma(ny, pl, xmax2.y);
+      }
     }
   }
   __shared__ double2 red[3][4][64];

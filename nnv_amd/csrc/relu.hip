@@ -25,13 +25,14 @@ struct ReluDesc {
   const double* pub_in;
   double* plb_out;
   double* pub_out;
-  int32_t* cls;        // per row: kKeep, kZero or the crossing position (= new predicate number)
+  int32_t* cls;        // per row: kKeep, kZero or the crossing neuron's position in ascending order
   int32_t* cross_idx;  // crossing neuron indices in new-predicate order
+  int32_t* rowmap;     // new-predicate number -> row of `rows` (= ascending position of that neuron)
   int32_t* asc_idx;    // crossing neuron indices in ascending order (sort orders only)
   double* key;         // sort keys, ascending-index order
   int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
-  double* rows;        // saved crossing rows of the pre-ReLU [c V]: m x ncols_in, ld = ld_rows
+  double* rows;        // saved crossing rows of the pre-ReLU [c V], ascending neuron order: m x ncols_in
   double* lbub;        // lb then ub (offset ld_rows) of the crossing neurons, new-predicate order
   int64_t ld;
   int64_t ld_rows;
@@ -43,7 +44,15 @@ struct ReluDesc {
   int32_t pad_;
 };
 
-// One 1024-thread block per set.
+// "a sorts before b" under the stable descending key order: larger key first, ties by smaller
+// neuron index (MATLAB's sort(...,'descend') keeps equal keys in their original, ascending order).
+__device__ __forceinline__ bool sorts_before(double ka, int ia, double kb, int ib) {
+  return ka > kb || (ka == kb && ia < ib);
+}
+
+// One 1024-thread block per set.  SORT_CAP > 0: crossing lists of up to SORT_CAP neurons are sorted
+// here by a bitonic network in LDS; longer lists are left to the tiled rank kernels.
+template <int SORT_CAP>
 __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
   const ReluDesc d = table ? table[blockIdx.x] : one;
   const int tid = threadIdx.x;
@@ -51,6 +60,8 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   const int wave = tid >> 6;
   __shared__ int wcross[16];
   __shared__ int winact[16];
+  __shared__ double skey[SORT_CAP > 0 ? SORT_CAP : 1];
+  __shared__ int sidx[SORT_CAP > 0 ? SORT_CAP : 1];
   int base = 0, inact_total = 0;
   int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
   for (int r0 = 0; r0 < d.N; r0 += 1024) {
@@ -58,7 +69,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     const bool valid = r < d.N;
     const double l = valid ? d.lb[r] : 0.0;
     const double u = valid ? d.ub[r] : 1.0;
-    const bool inactive = valid && (u <= 0.0);           // map1 = find(ub <= 0)
+    const bool inactive = valid && (u <= 0.0);              // map1 = find(ub <= 0)
     const bool crossing = valid && (l < 0.0) && (u > 0.0);  // map2 = find(lb < 0 & ub > 0)
     const unsigned long long bc = __ballot(crossing);
     const unsigned long long bi = __ballot(inactive);
@@ -78,12 +89,16 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     if (crossing) {
       const int pos = base + woff + __popcll(bc & ((1ull << lane) - 1ull));
       idx_out[pos] = r;
-      if (d.order == NNVHIP_ORDER_INDEX) {
-        d.cls[r] = pos;
-      } else {
+      d.cls[r] = pos;
+      if (d.order != NNVHIP_ORDER_INDEX) {
         // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb
-        d.key[pos] = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : u - l;
+        const double key = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : u - l;
+        d.key[pos] = key;
         d.rank[pos] = 0;
+        if (SORT_CAP > 0 && pos < SORT_CAP) {
+          skey[pos] = key;
+          sidx[pos] = r;
+        }
       }
     } else if (valid) {
       d.cls[r] = inactive ? kZero : kKeep;
@@ -93,9 +108,78 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     __syncthreads();
   }
   for (int64_t r = d.N + tid; r < d.ld; r += 1024) d.cls[r] = kKeep;  // padding rows stay zero
+  const int m = base;
   if (tid == 0) {
-    d.counts[0] = base;
+    d.counts[0] = m;
     d.counts[1] = inact_total;
+  }
+  if (SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP) {
+    // Bitonic network over P = 2^ceil(log2 m) entries, element i = e*1024 + tid held in registers.
+    // Exchange distance j < 64 stays inside a wave (shuffles), 64 <= j < 1024 goes through LDS,
+    // j >= 1024 pairs two registers of the same thread.
+    constexpr int E = SORT_CAP >= 1024 ? SORT_CAP / 1024 : 1;
+    int P = 1;
+    while (P < m) P <<= 1;
+    __syncthreads();
+    double key[E];
+    int idx[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int i = e * 1024 + tid;
+      key[e] = i < m ? skey[i] : -__builtin_huge_val();  // sentinels sort after every real entry
+      idx[e] = i < m ? sidx[i] : 0x7fffffff;
+    }
+    for (int k = 2; k <= P; k <<= 1) {
+      for (int j = k >> 1; j > 0; j >>= 1) {
+        if (j >= 64 && j < 1024) {
+          __syncthreads();
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            skey[e * 1024 + tid] = key[e];
+            sidx[e * 1024 + tid] = idx[e];
+          }
+          __syncthreads();
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const int i = e * 1024 + tid;
+          if (i >= P) continue;
+          double pk;
+          int pi;
+          if (j >= 1024) {
+            const int pe = e ^ (j >> 10);
+            // both registers of the pair are updated when the lower one is visited
+            if (pe < e) continue;
+            pk = key[pe];
+            pi = idx[pe];
+            const bool want_before = (i & k) == 0;
+            if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
+              key[pe] = key[e];
+              idx[pe] = idx[e];
+              key[e] = pk;
+              idx[e] = pi;
+            }
+            continue;
+          } else if (j >= 64) {
+            pk = skey[i ^ j];
+            pi = sidx[i ^ j];
+          } else {
+            pk = __shfl_xor(key[e], j);
+            pi = __shfl_xor(idx[e], j);
+          }
+          const bool want_before = ((i & j) == 0) == ((i & k) == 0);
+          if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
+            key[e] = pk;
+            idx[e] = pi;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int i = e * 1024 + tid;
+      if (i < m) d.cross_idx[i] = idx[e];
+    }
   }
 }
 
@@ -135,10 +219,7 @@ __global__ __launch_bounds__(256) void relu_scatter_kernel(const ReluDesc* __res
   const ReluDesc d = table ? table[blockIdx.z] : one;
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= d.m) return;
-  const int neuron = d.asc_idx[i];
-  const int r = d.rank[i];
-  d.cross_idx[r] = neuron;
-  d.cls[neuron] = r;
+  d.cross_idx[d.rank[i]] = d.asc_idx[i];
 }
 
 constexpr int kApplyRows = 128;  // 64 lanes x 2 rows, the four waves interleave columns
@@ -160,35 +241,46 @@ __global__ __launch_bounds__(256) void relu_apply_kernel(const ReluDesc* __restr
     cy = c.y;
   }
   const int n_in = d.ncols_in - 1;
-#pragma unroll 2
-  for (int j = j0 + wave; j < j1; j += 4) {
-    double2 o;
-    if (j < d.ncols_in) {
-      if (active) {
-        const double2 v = *reinterpret_cast<const double2*>(d.Vin + r0 + (int64_t)j * d.ld);
-        o.x = cx == kKeep ? v.x : 0.0;  // V1(map,:) = 0
-        o.y = cy == kKeep ? v.y : 0.0;
-        if (cx >= 0) d.rows[cx + (int64_t)j * d.ld_rows] = v.x;  // I.V(index, :) before zeroing
-        if (cy >= 0) d.rows[cy + (int64_t)j * d.ld_rows] = v.y;
-      }
-      if (blockIdx.x == 0 && lane == 0 && j >= 1) {
-        d.plb_out[j - 1] = d.plb_in[j - 1];
-        d.pub_out[j - 1] = d.pub_in[j - 1];
-      }
-    } else {
-      const int i = j - d.ncols_in;
-      const int neuron = d.cross_idx[i];
-      o.x = r0 == neuron ? 1.0 : 0.0;  // V2(index(i), i) = 1
-      o.y = r0 + 1 == neuron ? 1.0 : 0.0;
-      if (blockIdx.x == 0 && lane == 0) {
-        const double u = d.ub[neuron];
-        d.plb_out[n_in + i] = 0.0;  // new_pred_lb = [plb; zeros(m,1)]
-        d.pub_out[n_in + i] = u;    // new_pred_ub = [pub; ub]
-        d.lbub[i] = d.lb[neuron];
-        d.lbub[d.ld_rows + i] = u;
-      }
+  const bool writer = blockIdx.x == 0 && lane == 0;
+  // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
+  for (int jb = j0 + 4 * wave; jb < j1; jb += 16) {
+    double2 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = jb + u;
+      v[u] = make_double2(0.0, 0.0);
+      if (active && j < j1 && j < d.ncols_in) v[u] = *reinterpret_cast<const double2*>(d.Vin + r0 + (int64_t)j * d.ld);
     }
-    if (active) *reinterpret_cast<double2*>(d.Vout + r0 + (int64_t)j * d.ld) = o;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = jb + u;
+      if (j >= j1) break;
+      double2 o;
+      if (j < d.ncols_in) {
+        o.x = cx == kKeep ? v[u].x : 0.0;  // V1(map,:) = 0
+        o.y = cy == kKeep ? v[u].y : 0.0;
+        if (cx >= 0) d.rows[cx + (int64_t)j * d.ld_rows] = v[u].x;  // I.V(index, :) before zeroing
+        if (cy >= 0) d.rows[cy + (int64_t)j * d.ld_rows] = v[u].y;
+        if (writer && j >= 1) {
+          d.plb_out[j - 1] = d.plb_in[j - 1];
+          d.pub_out[j - 1] = d.pub_in[j - 1];
+        }
+      } else {
+        const int i = j - d.ncols_in;
+        const int neuron = d.cross_idx[i];
+        o.x = r0 == neuron ? 1.0 : 0.0;  // V2(index(i), i) = 1
+        o.y = r0 + 1 == neuron ? 1.0 : 0.0;
+        if (writer) {
+          const double ub = d.ub[neuron];
+          d.plb_out[n_in + i] = 0.0;  // new_pred_lb = [plb; zeros(m,1)]
+          d.pub_out[n_in + i] = ub;   // new_pred_ub = [pub; ub]
+          d.lbub[i] = d.lb[neuron];
+          d.lbub[d.ld_rows + i] = ub;
+          d.rowmap[i] = d.cls[neuron];
+        }
+      }
+      if (active) *reinterpret_cast<double2*>(d.Vout + r0 + (int64_t)j * d.ld) = o;
+    }
   }
 }
 
@@ -237,7 +329,15 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
-  hipLaunchKernelGGL(relu_classify_kernel, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+  // crossing lists short enough for LDS are sorted inside the classification kernel
+  int sort_cap = 0;
+  if (sorted) sort_cap = N <= 1024 ? 1024 : 8192;
+  if (sort_cap == 0)
+    hipLaunchKernelGGL(relu_classify_kernel<0>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+  else if (sort_cap == 1024)
+    hipLaunchKernelGGL(relu_classify_kernel<1024>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+  else
+    hipLaunchKernelGGL(relu_classify_kernel<8192>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
   NNV_HIP_TRY(hipGetLastError());
 
   // the column count of the output depends on m: read the counts back
@@ -265,16 +365,17 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     max_cols = std::max(max_cols, ncols_out);
     max_m = std::max(max_m, m);
   }
-  BufRef arena, pred_buf, rows_buf, lbub_buf;
+  BufRef arena, pred_buf, rows_buf, lbub_buf, map_buf;
   NNV_TRY(ctx->alloc(sizeof(double) * ld * total_cols, &arena));
   NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
   if (total_rows > 0) {
     NNV_TRY(ctx->alloc(sizeof(double) * total_rows, &rows_buf));
     NNV_TRY(ctx->alloc(sizeof(double) * total_lbub, &lbub_buf));
+    NNV_TRY(ctx->alloc(sizeof(int32_t) * total_lbub, &map_buf));
   }
-  // Column chunking of the apply pass: a few thousand blocks, at least 16 columns each.
+  // Column chunking of the apply pass: a couple of thousand blocks, at least 32 columns each.
   const int64_t row_blocks = ceil_div(ld, kApplyRows);
-  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(4096, row_blocks * count), ceil_div(max_cols, 16)));
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(2048, row_blocks * count), ceil_div(max_cols, 32)));
   const int64_t cpc = ceil_div(max_cols, chunks);
   chunks = ceil_div(max_cols, cpc);
   for (int64_t i = 0; i < count; ++i) {
@@ -288,6 +389,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.pub_out = d.plb_out + npad;
     d.rows = m > 0 ? rows_buf->as<double>() + rows_off[i] : nullptr;
     d.lbub = m > 0 ? lbub_buf->as<double>() + lbub_off[i] : nullptr;
+    d.rowmap = m > 0 ? map_buf->as<int32_t>() + lbub_off[i] : nullptr;
     d.ld_rows = ldr;
     d.cols_per_chunk = (int32_t)cpc;
   }
@@ -295,7 +397,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
-  if (sorted && max_m > 0) {
+  if (sorted && max_m > sort_cap) {  // some list was too long for the in-LDS sort: rank every list
     const unsigned t = (unsigned)ceil_div(max_m, 256);
     if (t > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "too many crossing neurons for the sort kernel");
     hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
@@ -329,6 +431,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       node->ld_rows = d.ld_rows;
       node->lbub = lbub_buf;
       node->index = idx_bufs[i];
+      node->rowmap = map_buf;
       // views into shared buffers: keep element offsets
       node->rows_off = rows_off[i];
       node->lbub_off = lbub_off[i];
@@ -357,13 +460,15 @@ __global__ void cons_copy_kernel(double* __restrict__ C, int64_t ldC, const doub
 //   a = ub./(ub-lb); b = a.*lb;  C3 = [-a.*V(index,2:n+1) I], d3 = a.*V(index,1) - b.
 __global__ void cons_relu_kernel(double* __restrict__ C, int64_t ldC, double* __restrict__ dvec, int64_t r0, int m,
                                  int nb, const double* __restrict__ rows, int64_t ld_rows,
-                                 const double* __restrict__ lb, const double* __restrict__ ub) {
+                                 const int32_t* __restrict__ rowmap, const double* __restrict__ lb,
+                                 const double* __restrict__ ub) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= m) return;
+  const int src = rowmap[i];
   const double a = ub[i] / (ub[i] - lb[i]);
   const int64_t row1 = r0 + i, row2 = r0 + m + i, row3 = r0 + 2 * (int64_t)m + i;
   for (int j = blockIdx.y; j <= nb; j += gridDim.y) {
-    const double v = rows[i + (int64_t)j * ld_rows];
+    const double v = rows[src + (int64_t)j * ld_rows];
     if (j == 0) {
       dvec[row1] = 0.0;
       dvec[row2] = -v;
@@ -409,7 +514,8 @@ int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host
       const double* lbp = nd->lbub->as<double>() + nd->lbub_off;
       dim3 grid((unsigned)ceil_div(nd->m, 128), (unsigned)std::min<int64_t>(nd->n_before + 1, 1024));
       hipLaunchKernelGGL(cons_relu_kernel, grid, dim3(128), 0, ctx->stream, Cuse, ldC, dd->as<double>(), r0, (int)nd->m,
-                         (int)nd->n_before, rows, nd->ld_rows, lbp, lbp + nd->ld_rows);
+                         (int)nd->n_before, rows, nd->ld_rows, nd->rowmap->as<int32_t>() + nd->lbub_off, lbp,
+                         lbp + nd->ld_rows);
       r0 += 3 * nd->m;
     }
   }
