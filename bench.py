@@ -28,6 +28,9 @@ import numpy as np  # noqa: E402
 
 FP64_MFMA_PEAK_TFLOPS = 78.6
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+# scaled by the 1 GiB copy kernel of the same run (profiles/<workload>_hbm_traffic.md): (read, write) MiB
+MEASURED_TRAFFIC_MIB = {("cfg2_fc_784_1024x3_10", "gemm_f64_kernel"): (64.55, 21.41)}
 
 
 def layer_shapes(reach_set):
@@ -159,6 +162,9 @@ def main():
         achieved = relu_bytes / (relu_ms * 1e-3) / 1e9
         roofline = {"kernel": "relu step", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None}
+    t = MEASURED_TRAFFIC_MIB.get((cfg["name"], roofline["kernel"]))
+    if t is not None and args.method == "relax-star-area":
+        roofline["traffic"] = round((t[0] + t[1]) * 1048576.0)
     if relu_ms > 0:
         roofline["relu_step_algo_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
         roofline["relu_step_frac_of_hbm_peak"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)

@@ -20,7 +20,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
                                                         const double* __restrict__ B, int64_t ldb,
                                                         double* __restrict__ C, int64_t ldc, int Mp, int64_t ncols,
                                                         int Kp, const double* __restrict__ bias, int tiles_m,
-                                                        int ksplit, double* __restrict__ part) {
+                                                        int tiles_n, int xr, int local_m, int ksplit,
+                                                        double* __restrict__ part) {
   constexpr int NT = 64 * WR * WC;  // threads per block
   constexpr int FM = TM / WR / 16;
   constexpr int FN = TN / WC / 16;
@@ -34,10 +35,19 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   const int wave = tid >> 6;
   const int wr = wave % WR;
   const int wc = wave / WR;
-  // consecutive blocks walk down the rows of one column band, so the band's V tile stays hot
-  const int64_t bid = blockIdx.x;
-  const int m0 = (int)(bid % tiles_m) * TM;
-  const int64_t n0 = (bid / tiles_m) * TN;
+  // XCD-aware tile mapping.  Workgroups are dealt round-robin to the 8 XCDs (each with its own
+  // 4 MiB L2) by linear id, so blockIdx.x % 8 names the XCD.  The XCDs form an xr x (8/xr) grid over
+  // the tile matrix: XCD (i, j) owns the row tiles congruent to i mod xr and the column tiles
+  // congruent to j mod 8/xr, i.e. it touches 1/xr of W and xr/8 of V instead of all of V.  Inside
+  // an XCD consecutive blocks walk down the row tiles of one column tile, keeping its V tile hot.
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int xc = 8 / xr;
+  const int mt = (slot % local_m) * xr + (xcd % xr);
+  const int64_t nt = (int64_t)(slot / local_m) * xc + (xcd / xr);
+  if (mt >= tiles_m || nt >= tiles_n) return;
+  const int m0 = mt * TM;
+  const int64_t n0 = nt * TN;
 
   // ---- global -> register staging ----------------------------------------------------------
   constexpr int A_VEC = TM * KT / 2;           // double2 elements in a W tile
@@ -156,7 +166,27 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   int64_t tiles_m = ceil_div(Mp, TM);
   int64_t tiles_n = ceil_div(ncols, TN);
   int64_t blocks = tiles_m * tiles_n;
-  if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large for one launch");
+  if (blocks >= (int64_t(1) << 28)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large for one launch");
+  // XCD grid xr x (8/xr): least HBM/fabric traffic (8/xr)*|W| + xr*|V| among the shapes whose
+  // busiest XCD has (almost) the fewest tiles
+  int64_t best_xr = 8, best_slots = 0;
+  double best_cost = 0.0;
+  for (int64_t xr = 1; xr <= 8; xr *= 2) {
+    const int64_t slots = ceil_div(tiles_m, xr) * ceil_div(tiles_n, 8 / xr);
+    const double traffic = (8.0 / xr) * (double)Mp * Kp + (double)xr * Kp * (double)ncols;
+    const double cost = (double)slots * (1.0 + 0.03 * traffic / ((double)Mp * Kp + (double)Kp * ncols) / 8.0);
+    if (best_slots == 0 || cost < best_cost) {
+      best_cost = cost;
+      best_xr = xr;
+      best_slots = slots;
+    }
+  }
+  if (const char* e = getenv("NNVHIP_GEMM_XR")) {
+    best_xr = std::max(1, std::min(8, atoi(e)));
+    best_slots = ceil_div(tiles_m, best_xr) * ceil_div(tiles_n, 8 / best_xr);
+  }
+  const int64_t local_m = ceil_div(tiles_m, best_xr);
+  const int64_t grid_x = 8 * best_slots;
   // Split-K when the output has too few tiles to occupy the chip: partial products into a workspace,
   // summed in split order by a second kernel (deterministic, no floating-point atomics).
   const int64_t nk = Kp / KT;
@@ -167,9 +197,9 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   if (ksplit > 1) NNV_TRY(ctx->alloc(sizeof(double) * ksplit * Mp * ncols, &ws));
   const bool timed = ctx->timing && TM >= 64;
   NNV_TRY(ctx->kernel_timer_begin(timed));
-  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)blocks, (unsigned)ksplit), dim3(64 * WR * WC), 0,
-                     ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)ksplit,
-                     ws ? ws->as<double>() : nullptr);
+  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)grid_x, (unsigned)ksplit), dim3(64 * WR * WC), 0,
+                     ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)tiles_n,
+                     (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, 2.0 * (double)Mp * (double)Kp * (double)ncols));
   if (ksplit > 1) {
     const int64_t total = Mp * ncols;

@@ -1,0 +1,51 @@
+classdef ImageStar < ImageStar
+    % NNV ImageStar resident in HBM: the H x W x C x (numPred+1) tensor is the same device memory as
+    % the (H*W*C) x (numPred+1) Star matrix (ImageStar.m:569-592, Star.m:1398-1418).
+    properties
+        dev = [];   % nnvhip.DeviceSet
+    end
+    methods
+        function obj = ImageStar(varargin)
+            % nnvhip.ImageStar(dev, h, w, c) | nnvhip.ImageStar(IS) | nnvhip.ImageStar(lb_im, ub_im)
+            obj = obj@ImageStar();
+            if nargin == 4
+                obj.dev = varargin{1};
+                obj.height = varargin{2}; obj.width = varargin{3}; obj.numChannel = varargin{4};
+            elseif nargin == 1
+                IS = varargin{1};
+                S = nnvhip.Star(IS.toStar);
+                obj.dev = S.dev;
+                obj.height = IS.height; obj.width = IS.width; obj.numChannel = IS.numChannel;
+                obj.im_lb = IS.im_lb; obj.im_ub = IS.im_ub;
+            elseif nargin == 2
+                lb = varargin{1}; ub = varargin{2}; n = size(lb);
+                if numel(n) == 2, n(3) = 1; end
+                S = nnvhip.Star(reshape(lb, [], 1), reshape(ub, [], 1));
+                obj.dev = S.dev;
+                obj.height = n(1); obj.width = n(2); obj.numChannel = n(3);
+                obj.im_lb = lb; obj.im_ub = ub;
+            end
+            if ~isempty(obj.dev)
+                dims = nnvhip_mex('star_dims', obj.dev.h);
+                obj.numPred = dims(2);
+            end
+        end
+        function S = toStar(obj)                     % ImageStar.m:569-592
+            S = nnvhip.Star(obj.dev);
+        end
+        function [lb, ub] = estimateRanges(obj, varargin)   % ImageStar.m:836-885
+            if isempty(obj.im_lb) || isempty(obj.im_ub)
+                [l, u] = nnvhip_mex('estimate_ranges', obj.dev.h);
+                obj.im_lb = reshape(l, obj.height, obj.width, obj.numChannel);
+                obj.im_ub = reshape(u, obj.height, obj.width, obj.numChannel);
+            end
+            lb = obj.im_lb; ub = obj.im_ub;
+        end
+        function IS = gather(obj)
+            V = nnvhip_mex('fetch_V', obj.dev.h);
+            [C, d] = nnvhip_mex('fetch_constraints', obj.dev.h);
+            [plb, pub] = nnvhip_mex('fetch_pred', obj.dev.h);
+            IS = ImageStar(reshape(V, obj.height, obj.width, obj.numChannel, []), C, d, plb, pub);
+        end
+    end
+end

@@ -1,0 +1,42 @@
+classdef ReluLayer < ReluLayer
+    % ReluLayer whose relax-star reach (ReluLayer.m:72-150 -> PosLin.reach, PosLin.m:863-1650) runs on
+    % the device.  The override sits at layer level because PosLin.multipleStepReachStarApprox_at_one
+    % reads I.V directly (PosLin.m:702) and would force a device -> host fetch.
+    methods
+        function obj = ReluLayer(varargin)
+            obj = obj@ReluLayer(varargin{:});
+        end
+        function images = reach_star_multipleInputs(obj, in_images, method, option, relaxFactor, dis_opt, lp_solver) %#ok<INUSD>
+            switch char(method)
+                case 'relax-star-range', order = 2;                       % PosLin.m:934-936
+                case 'relax-star-area',  order = 1;                       % PosLin.m:1049-1052
+                case {'relax-star-bound', 'relax-star-ub', 'relax-star-random', 'relax-star-static'}
+                    order = 0;                                            % ascending neuron index
+                otherwise
+                    error("This reachability method does not exist");
+            end
+            if relaxFactor < 0 || relaxFactor > 1
+                error('Invalid relax factor');
+            end
+            n = length(in_images);
+            hs = zeros(1, n, 'uint64');
+            for i = 1:n, hs(i) = in_images(i).dev.h; end
+            out = nnvhip_mex('relu_relax', order, relaxFactor, hs);
+            for i = n:-1:1
+                if isa(in_images(i), 'ImageStar')
+                    images(i) = nnvhip.ImageStar(nnvhip.DeviceSet(out(i)), in_images(i).height, in_images(i).width, in_images(i).numChannel);
+                else
+                    images(i) = nnvhip.Star(nnvhip.DeviceSet(out(i)));
+                end
+                if strcmp(dis_opt, 'display')
+                    [idx, ~, ~, ninact] = nnvhip_mex('fetch_crossing', out(i));
+                    fprintf('\n%d neurons with ub <= 0 are found by estimating ranges', ninact);
+                    fprintf('\nConstruct new star set, %d new predicate variables are introduced', numel(idx));
+                end
+            end
+        end
+        function images = reach_star_single_input(obj, in_image, method, relaxFactor, dis_opt, lp_solver)
+            images = obj.reach_star_multipleInputs(in_image, method, 'single', relaxFactor, dis_opt, lp_solver);
+        end
+    end
+end

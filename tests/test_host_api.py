@@ -1,0 +1,77 @@
+"""CPU checks of the host-side mirror of NNV's classes: argument validation, error strings, option
+parsing and the Box arithmetic - everything that does not need a device call."""
+import numpy as np
+import pytest
+
+from nnv_amd.configs import conv_out_hw, count_updates, make_config
+from nnv_amd.layers import RELAX_ORDER, Conv2DLayer, FullyConnectedLayer
+from nnv_amd.nn import NN
+from nnv_amd.sets import Box
+from oracle import nnv_oracle as o
+
+
+def test_box_matches_oracle_arithmetic():
+    lb = np.array([0.1, -1.0, 2.0, 2.0])
+    ub = np.array([0.4, 1.0, 2.0, 3.5])
+    b = Box(lb, ub)
+    c, g = o.box_generators(lb, ub)
+    assert np.array_equal(b.center, c) and np.array_equal(b.generators, g)
+    assert b.generators.shape == (4, 3)          # the zero-width dimension has no generator
+    parts = b.partition([0, 3], [2, 3])
+    ref = o.box_partition(lb, ub, [0, 3], [2, 3])
+    assert len(parts) == 6
+    for p, (l, u) in zip(parts, ref):
+        assert np.array_equal(p.lb, l) and np.array_equal(p.ub, u)
+    with pytest.raises(ValueError, match="Inconsistent dimensions"):
+        Box([0, 1], [1])
+    with pytest.raises(ValueError, match="index in part_indexes"):
+        b.partition([7], [2])
+
+
+def test_layer_constructors_validate_like_nnv():
+    with pytest.raises(ValueError, match="weight matrix and bias vector"):
+        FullyConnectedLayer(np.ones((3, 2)), np.ones(4))
+    with pytest.raises(ValueError, match="one column"):
+        FullyConnectedLayer(np.ones((3, 2)), np.ones((3, 2)))
+    L = FullyConnectedLayer("fc", np.ones((3, 2)), np.ones((3, 1)))
+    assert (L.InputSize, L.OutputSize, L.Name) == (2, 3, "fc")
+    assert np.array_equal(L.evaluate([1.0, 2.0]), [4.0, 4.0, 4.0])
+    with pytest.raises(ValueError, match="filter weights and filter biases"):
+        Conv2DLayer(np.ones((3, 3, 2, 4)), np.ones(3))
+    C = Conv2DLayer(np.ones((3, 3, 2, 4)), np.ones(4), [1, 1, 1, 1], [2, 2], [1, 1])
+    assert (C.NumChannels, C.NumFilters, C.FilterSize) == (2, 4, [3, 3])
+    assert C.output_size(32, 32) == (16, 16)
+    assert C.output_size(15, 15) == conv_out_hw(15, 15, {"W": np.ones((3, 3, 2, 4)), "padding": [1, 1, 1, 1],
+                                                           "stride": [2, 2], "dilation": [1, 1]})
+
+
+def test_reach_options_validation():
+    net = NN([])
+    with pytest.raises(ValueError, match="specify a relax factor"):
+        net.validate_reach_options({"reachMethod": "relax-star-area"})
+    with pytest.raises(ValueError, match="between 0 and 1"):
+        net.validate_reach_options({"reachMethod": "relax-star-area", "relaxFactor": 1.5})
+    opts = net.validate_reach_options({"reachMethod": "relax-star-area", "relaxFactor": 1, "numCores": 8})
+    assert opts["numCores"] == 1 and opts["reachOption"] == "single"      # nn/NN.m:1227-1231
+    with pytest.raises(TypeError, match="Wrong input set type"):
+        net.reach(np.zeros(3), {"reachMethod": "relax-star-area", "relaxFactor": 1})
+
+
+def test_relax_orders_cover_the_six_variants():
+    assert sorted(RELAX_ORDER) == sorted(o.RELAX_METHODS)
+    assert RELAX_ORDER["relax-star-area"] != RELAX_ORDER["relax-star-range"]
+    assert len({RELAX_ORDER[m] for m in ("relax-star-bound", "relax-star-ub", "relax-star-random", "relax-star-static")}) == 1
+
+
+def test_configs_are_reproducible_and_sized():
+    a, b = make_config(2), make_config(2)
+    assert np.array_equal(a["layers"][0]["W"], b["layers"][0]["W"]) and np.array_equal(a["lb"], b["lb"])
+    assert [L["W"].shape for L in a["layers"] if L["type"] == "fc"] == [(1024, 784), (1024, 1024), (1024, 1024), (10, 1024)]
+    c5 = make_config(5)
+    assert np.array_equal(c5["layers"][0]["W"], a["layers"][0]["W"]) and len(c5["partition"]["indexes"]) == 10
+    c4 = make_config(4)
+    assert c4["image_shape"] == (32, 32, 3) and c4["layers"][8]["W"].shape == (512, 7 * 7 * 64)
+    c3 = make_config(3)
+    assert c3["layers"][4]["W"].shape == (100, 14 * 14 * 32)
+    assert abs(np.std(a["layers"][2]["W"]) - np.sqrt(2.0 / 1024)) < 1e-3
+    assert count_updates([(3, 4), (2, 1)]) == 3 * 5 + 2 * 2
