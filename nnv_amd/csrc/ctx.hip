@@ -513,7 +513,7 @@ int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb,
     if (index) NNV_HIP_TRY(hipMemcpyAsync(index, node->index->ptr, sizeof(int32_t) * m, hipMemcpyDeviceToHost, c->stream));
     const double* lbub = node->lbub->as<double>() + node->lbub_off;
     if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb, lbub, sizeof(double) * m, hipMemcpyDeviceToHost, c->stream));
-    if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub, lbub + node->ld_rows, sizeof(double) * m, hipMemcpyDeviceToHost, c->stream));
+    if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub, lbub + node->ld_lbub, sizeof(double) * m, hipMemcpyDeviceToHost, c->stream));
   }
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   return NNVHIP_OK;

@@ -68,17 +68,18 @@ struct ConsNode {
   BufRef C0;
   int64_t ldc = 0;
   BufRef d0;
-  // ReLU node: the m crossing rows of the pre-ReLU [c V] (m x (n_before+1), ld = ld_rows) in
-  // ascending neuron order (coalesced to write), plus bounds and indices in new-predicate order
+  // ReLU node: the C2/C3 rows are the crossing rows of the pre-ReLU [c V].  They are not copied:
+  // the node keeps the input set's (immutable) generator buffer alive and gathers rows by index
+  // when the dense matrix is materialised.
   int64_t m = 0;
   int64_t n_before = 0;
-  BufRef rows;            // possibly shared by the sets of one array: data starts at rows_off
-  int64_t rows_off = 0;   // element offset into rows
-  int64_t ld_rows = 0;
-  BufRef lbub;            // lb[0..m), then ub[0..m) at offset ld_rows; data starts at lbub_off
+  BufRef src;                    // owner of the pre-ReLU generator matrix
+  const double* src_V = nullptr; // its N x (n_before+1) matrix
+  int64_t src_ld = 0;
+  BufRef lbub;                   // lb[0..m), then ub[0..m) at offset ld_lbub; data starts at lbub_off
   int64_t lbub_off = 0;
-  BufRef index;           // int32[m]: crossing neuron indices in new-predicate order
-  BufRef rowmap;          // int32[m] at element offset lbub_off: new-predicate number -> row of `rows`
+  int64_t ld_lbub = 0;
+  BufRef index;                  // int32[m]: crossing neuron indices in new-predicate order
 };
 using ConsRef = std::shared_ptr<ConsNode>;
 

@@ -3,8 +3,9 @@
 //   1. classify every neuron from its estimated range (inactive / crossing / active) and compact
 //      the crossing indices in ascending order with wavefront ballots + prefix sums;
 //   2. (area / range orders) rank the crossing neurons by a stable descending key sort;
-//   3. one pass over V: zero the inactive and crossing rows, save the crossing rows for the
-//      constraint store, append the one-hot columns and the new predicate bounds.
+//   3. one pass over V: zero the inactive and crossing rows, append the one-hot columns and the new
+//      predicate bounds.  The crossing rows the constraints need are not copied: the constraint node
+//      keeps the (immutable) pre-ReLU generator matrix alive and remembers the row indices.
 // The dense constraint matrix is never built on this path; materialize_constraints() lays it out
 // exactly as the reference does when the host asks for it.
 #include <algorithm>
@@ -27,15 +28,13 @@ struct ReluDesc {
   double* pub_out;
   int32_t* cls;        // per row: kKeep, kZero or the crossing neuron's position in ascending order
   int32_t* cross_idx;  // crossing neuron indices in new-predicate order
-  int32_t* rowmap;     // new-predicate number -> row of `rows` (= ascending position of that neuron)
   int32_t* asc_idx;    // crossing neuron indices in ascending order (sort orders only)
   double* key;         // sort keys, ascending-index order
   int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
-  double* rows;        // saved crossing rows of the pre-ReLU [c V], ascending neuron order: m x ncols_in
-  double* lbub;        // lb then ub (offset ld_rows) of the crossing neurons, new-predicate order
+  double* lbub;        // lb then ub (offset ld_lbub) of the crossing neurons, new-predicate order
   int64_t ld;
-  int64_t ld_rows;
+  int64_t ld_lbub;
   int32_t N;
   int32_t ncols_in;  // n + 1
   int32_t m;
@@ -259,8 +258,6 @@ __global__ __launch_bounds__(256) void relu_apply_kernel(const ReluDesc* __restr
       if (j < d.ncols_in) {
         o.x = cx == kKeep ? v[u].x : 0.0;  // V1(map,:) = 0
         o.y = cy == kKeep ? v[u].y : 0.0;
-        if (cx >= 0) d.rows[cx + (int64_t)j * d.ld_rows] = v[u].x;  // I.V(index, :) before zeroing
-        if (cy >= 0) d.rows[cy + (int64_t)j * d.ld_rows] = v[u].y;
         if (writer && j >= 1) {
           d.plb_out[j - 1] = d.plb_in[j - 1];
           d.pub_out[j - 1] = d.pub_in[j - 1];
@@ -275,8 +272,7 @@ __global__ __launch_bounds__(256) void relu_apply_kernel(const ReluDesc* __restr
           d.plb_out[n_in + i] = 0.0;  // new_pred_lb = [plb; zeros(m,1)]
           d.pub_out[n_in + i] = ub;   // new_pred_ub = [pub; ub]
           d.lbub[i] = d.lb[neuron];
-          d.lbub[d.ld_rows + i] = ub;
-          d.rowmap[i] = d.cls[neuron];
+          d.lbub[d.ld_lbub + i] = ub;
         }
       }
       if (active) *reinterpret_cast<double2*>(d.Vout + r0 + (int64_t)j * d.ld) = o;
@@ -347,32 +343,26 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));
   const std::vector<int32_t> counts(static_cast<const int32_t*>(hc), static_cast<const int32_t*>(hc) + 2 * count);
 
-  // outputs: one V arena, one predicate-bound buffer, one buffer for all saved rows / bounds
-  int64_t total_cols = 0, total_pred = 0, total_rows = 0, total_lbub = 0, max_cols = 0, max_m = 0;
-  std::vector<int64_t> col_off(count), pred_off(count), rows_off(count), lbub_off(count);
+  // outputs: one V arena, one predicate-bound buffer, one buffer for the crossing bounds
+  int64_t total_cols = 0, total_pred = 0, total_lbub = 0, max_cols = 0, max_m = 0;
+  std::vector<int64_t> col_off(count), pred_off(count), lbub_off(count);
   for (int64_t i = 0; i < count; ++i) {
     const int64_t m = counts[2 * i];
     const int64_t ncols_out = in[i]->n + 1 + m;
     const int64_t ldr = round_up(std::max<int64_t>(m, 1), kLdAlign);
     col_off[i] = total_cols;
     pred_off[i] = total_pred;
-    rows_off[i] = total_rows;
     lbub_off[i] = total_lbub;
     total_cols += ncols_out;
     total_pred += 2 * round_up(std::max<int64_t>(in[i]->n + m, 1), kLdAlign);
-    total_rows += m > 0 ? ldr * (in[i]->n + 1) : 0;
     total_lbub += m > 0 ? 2 * ldr : 0;
     max_cols = std::max(max_cols, ncols_out);
     max_m = std::max(max_m, m);
   }
-  BufRef arena, pred_buf, rows_buf, lbub_buf, map_buf;
+  BufRef arena, pred_buf, lbub_buf;
   NNV_TRY(ctx->alloc(sizeof(double) * ld * total_cols, &arena));
   NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
-  if (total_rows > 0) {
-    NNV_TRY(ctx->alloc(sizeof(double) * total_rows, &rows_buf));
-    NNV_TRY(ctx->alloc(sizeof(double) * total_lbub, &lbub_buf));
-    NNV_TRY(ctx->alloc(sizeof(int32_t) * total_lbub, &map_buf));
-  }
+  if (total_lbub > 0) NNV_TRY(ctx->alloc(sizeof(double) * total_lbub, &lbub_buf));
   // Column chunking of the apply pass: a couple of thousand blocks, at least 32 columns each.
   const int64_t row_blocks = ceil_div(ld, kApplyRows);
   int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(2048, row_blocks * count), ceil_div(max_cols, 32)));
@@ -387,10 +377,8 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.Vout = arena->as<double>() + col_off[i] * ld;
     d.plb_out = pred_buf->as<double>() + pred_off[i];
     d.pub_out = d.plb_out + npad;
-    d.rows = m > 0 ? rows_buf->as<double>() + rows_off[i] : nullptr;
     d.lbub = m > 0 ? lbub_buf->as<double>() + lbub_off[i] : nullptr;
-    d.rowmap = m > 0 ? map_buf->as<int32_t>() + lbub_off[i] : nullptr;
-    d.ld_rows = ldr;
+    d.ld_lbub = ldr;
     d.cols_per_chunk = (int32_t)cpc;
   }
   if (count > 1) {
@@ -427,13 +415,13 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       node->n_before = in[i]->n;
       node->p_total = in[i]->cons->p_total + 3 * (int64_t)d.m;
       node->n_total = o->n;
-      node->rows = rows_buf;
-      node->ld_rows = d.ld_rows;
+      node->src = in[i]->Vbuf;  // zero-copy: C2/C3 rows are rows of the input's immutable [c V]
+      node->src_V = in[i]->V;
+      node->src_ld = in[i]->ld;
+      node->ld_lbub = d.ld_lbub;
       node->lbub = lbub_buf;
       node->index = idx_bufs[i];
-      node->rowmap = map_buf;
       // views into shared buffers: keep element offsets
-      node->rows_off = rows_off[i];
       node->lbub_off = lbub_off[i];
       o->cons = node;
     } else {
@@ -460,11 +448,11 @@ __global__ void cons_copy_kernel(double* __restrict__ C, int64_t ldC, const doub
 //   a = ub./(ub-lb); b = a.*lb;  C3 = [-a.*V(index,2:n+1) I], d3 = a.*V(index,1) - b.
 __global__ void cons_relu_kernel(double* __restrict__ C, int64_t ldC, double* __restrict__ dvec, int64_t r0, int m,
                                  int nb, const double* __restrict__ rows, int64_t ld_rows,
-                                 const int32_t* __restrict__ rowmap, const double* __restrict__ lb,
+                                 const int32_t* __restrict__ index, const double* __restrict__ lb,
                                  const double* __restrict__ ub) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= m) return;
-  const int src = rowmap[i];
+  const int src = index[i];  // I.V(index(i), :)
   const double a = ub[i] / (ub[i] - lb[i]);
   const int64_t row1 = r0 + i, row2 = r0 + m + i, row3 = r0 + 2 * (int64_t)m + i;
   for (int j = blockIdx.y; j <= nb; j += gridDim.y) {
@@ -510,12 +498,11 @@ int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host
     } else {
       double* Cuse = Cp;
       const int64_t ldC = p;
-      const double* rows = nd->rows->as<double>() + nd->rows_off;
+      const double* rows = nd->src_V;
       const double* lbp = nd->lbub->as<double>() + nd->lbub_off;
       dim3 grid((unsigned)ceil_div(nd->m, 128), (unsigned)std::min<int64_t>(nd->n_before + 1, 1024));
       hipLaunchKernelGGL(cons_relu_kernel, grid, dim3(128), 0, ctx->stream, Cuse, ldC, dd->as<double>(), r0, (int)nd->m,
-                         (int)nd->n_before, rows, nd->ld_rows, nd->rowmap->as<int32_t>() + nd->lbub_off, lbp,
-                         lbp + nd->ld_rows);
+                         (int)nd->n_before, rows, nd->src_ld, nd->index->as<int32_t>(), lbp, lbp + nd->ld_lbub);
       r0 += 3 * nd->m;
     }
   }
