@@ -38,12 +38,13 @@ __device__ __forceinline__ unsigned long long pack_tap(const ConvGeom& g, int k)
 }
 
 template <int TP, int TC, int WR, int WC>
-__global__ __launch_bounds__(256) void conv2d_f64_kernel(const double* __restrict__ in, int64_t ldin,
+__global__ __launch_bounds__(64 * WR * WC) void conv2d_f64_kernel(const double* __restrict__ in, int64_t ldin,
                                                           double* __restrict__ out, int64_t ldout,
                                                           const double* __restrict__ Wt,
                                                           const double* __restrict__ bias, ConvGeom g,
                                                           int64_t total_rows, int tiles_c) {
-  static_assert(WR * WC == 4, "four waves per block");
+  constexpr int NT = 64 * WR * WC;  // threads per block
+  static_assert(NT % TP == 0 && (TP * kKt) % NT == 0, "gather mapping needs NT = TP * (taps per pass)");
   constexpr int FM = TP / WR / 16;
   constexpr int FN = TC / WC / 16;
   constexpr int LDP_S = TP + kPadRow;  // Ps[k][position]
@@ -61,11 +62,11 @@ __global__ __launch_bounds__(256) void conv2d_f64_kernel(const double* __restric
   const int c0 = (int)(bid % tiles_c) * TC;
   const int64_t R0 = (bid / tiles_c) * TP;
 
-  for (int k = tid; k < g.Kp; k += 256) taps[k] = pack_tap(g, k);
+  for (int k = tid; k < g.Kp; k += NT) taps[k] = pack_tap(g, k);
 
   // this thread's gather position (fixed for the whole K loop)
-  constexpr int P_PASS = TP * kKt / 256;  // gathered elements per thread per K-tile
-  constexpr int K_STEP = 256 / TP;        // taps covered by one pass
+  constexpr int P_PASS = TP * kKt / NT;  // gathered elements per thread per K-tile
+  constexpr int K_STEP = NT / TP;        // taps covered by one pass
   const int p_local = tid % TP;
   const int k_first = tid / TP;
   const int64_t R = R0 + p_local;
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(256) void conv2d_f64_kernel(const double* __restric
   }
 
   constexpr int W_VEC = TC * kKt / 2;
-  constexpr int W_PASS = (W_VEC + 255) / 256;
+  constexpr int W_PASS = (W_VEC + NT - 1) / NT;
   double rp[P_PASS];
   double2 rw[W_PASS];
 
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(256) void conv2d_f64_kernel(const double* __restric
     }
 #pragma unroll
     for (int q = 0; q < W_PASS; ++q) {
-      const int idx = tid + q * 256;
+      const int idx = tid + q * NT;
       const int k2 = idx % (kKt / 2);
       const int j = idx / (kKt / 2);
       double2 v = make_double2(0.0, 0.0);
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(256) void conv2d_f64_kernel(const double* __restric
     for (int q = 0; q < P_PASS; ++q) Ps[buf][(k_first + q * K_STEP) * LDP_S + p_local] = rp[q];
 #pragma unroll
     for (int q = 0; q < W_PASS; ++q) {
-      const int idx = tid + q * 256;
+      const int idx = tid + q * NT;
       const int k2 = idx % (kKt / 2);
       const int j = idx / (kKt / 2);
       if (idx < W_VEC) {  // odd column stride: two 64-bit stores
@@ -181,7 +182,7 @@ static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvG
   if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
   const size_t dyn = sizeof(unsigned long long) * g.Kp;
   NNV_TRY(ctx->kernel_timer_begin(ctx->timing));
-  hipLaunchKernelGGL((conv2d_f64_kernel<TP, TC, WR, WC>), dim3((unsigned)blocks), dim3(256), dyn, ctx->stream, in, ldin,
+  hipLaunchKernelGGL((conv2d_f64_kernel<TP, TC, WR, WC>), dim3((unsigned)blocks), dim3(64 * WR * WC), dyn, ctx->stream, in, ldin,
                      out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows,
                      (int)tiles_c);
   NNV_TRY(ctx->kernel_timer_end(ctx->timing, 1, 2.0 * (double)total_rows * g.Cout * g.K));
@@ -215,13 +216,15 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W
   g.P = (int)(Ho * Wo);
   g.HW = (int)(H * W);
   const int64_t Nout = Ho * Wo * cv->Cout;
+  // 128 positions x Cout tile, eight waves per block (two per SIMD keep the MFMA pipe fed while
+  // the other wave gathers)
   int st;
   if (cv->Cout <= 16)
-    st = launch_conv_cfg<128, 16, 4, 1>(ctx, cv, g, in, ldin, out, ldout, ncols);
+    st = launch_conv_cfg<128, 16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols);
   else if (cv->Cout <= 32)
-    st = launch_conv_cfg<128, 32, 2, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
+    st = launch_conv_cfg<128, 32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
   else
-    st = launch_conv_cfg<128, 64, 2, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
+    st = launch_conv_cfg<128, 64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
   NNV_TRY(st);
   if (ldout != Nout) {  // keep the padding rows of the output at zero
     hipLaunchKernelGGL(zero_pad_rows_kernel, dim3(256), dim3(256), 0, ctx->stream, out, ldout, Nout, ncols);

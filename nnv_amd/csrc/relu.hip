@@ -32,6 +32,7 @@ struct ReluDesc {
   double* key;         // sort keys, ascending-index order
   int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
+  int32_t* blk_counts; // multi-block classification: per 1024-row block {crossing, inactive}
   double* lbub;        // lb then ub (offset ld_lbub) of the crossing neurons, new-predicate order
   int64_t ld;
   int64_t ld_lbub;
@@ -47,6 +48,75 @@ struct ReluDesc {
 // neuron index (MATLAB's sort(...,'descend') keeps equal keys in their original, ascending order).
 __device__ __forceinline__ bool sorts_before(double ka, int ia, double kb, int ib) {
   return ka > kb || (ka == kb && ia < ib);
+}
+
+// Bitonic network over P = 2^ceil(log2 m) entries staged in skey/sidx (m <= CAP), element
+// i = e*1024 + tid held in registers.  Exchange distance j < 64 stays inside a wave (shuffles),
+// 64 <= j < 1024 goes through LDS, j >= 1024 pairs two registers of the same thread.  Writes the
+// neuron indices in sorted order to out[0..m).  All 1024 threads of the block must call it.
+template <int CAP>
+__device__ __forceinline__ void bitonic_sort_desc(double* skey, int* sidx, int m, int tid, int32_t* __restrict__ out) {
+  constexpr int E = CAP >= 1024 ? CAP / 1024 : 1;
+  int P = 1;
+  while (P < m) P <<= 1;
+  double key[E];
+  int idx[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = e * 1024 + tid;
+    key[e] = i < m ? skey[i] : -__builtin_huge_val();  // sentinels sort after every real entry
+    idx[e] = i < m ? sidx[i] : 0x7fffffff;
+  }
+  for (int k = 2; k <= P; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      if (j >= 64 && j < 1024) {
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          skey[e * 1024 + tid] = key[e];
+          sidx[e * 1024 + tid] = idx[e];
+        }
+        __syncthreads();
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const int i = e * 1024 + tid;
+        if (i >= P) continue;
+        double pk;
+        int pi;
+        if (j >= 1024) {
+          const int pe = e ^ (j >> 10);
+          if (pe < e) continue;  // both registers of the pair are updated when the lower one is visited
+          pk = key[pe];
+          pi = idx[pe];
+          const bool want_before = (i & k) == 0;
+          if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
+            key[pe] = key[e];
+            idx[pe] = idx[e];
+            key[e] = pk;
+            idx[e] = pi;
+          }
+          continue;
+        } else if (j >= 64) {
+          pk = skey[i ^ j];
+          pi = sidx[i ^ j];
+        } else {
+          pk = __shfl_xor(key[e], j);
+          pi = __shfl_xor(idx[e], j);
+        }
+        const bool want_before = ((i & j) == 0) == ((i & k) == 0);
+        if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
+          key[e] = pk;
+          idx[e] = pi;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int i = e * 1024 + tid;
+    if (i < m) out[i] = idx[e];
+  }
 }
 
 // One 1024-thread block per set.  SORT_CAP > 0: crossing lists of up to SORT_CAP neurons are sorted
@@ -113,71 +183,113 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     d.counts[1] = inact_total;
   }
   if (SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP) {
-    // Bitonic network over P = 2^ceil(log2 m) entries, element i = e*1024 + tid held in registers.
-    // Exchange distance j < 64 stays inside a wave (shuffles), 64 <= j < 1024 goes through LDS,
-    // j >= 1024 pairs two registers of the same thread.
-    constexpr int E = SORT_CAP >= 1024 ? SORT_CAP / 1024 : 1;
-    int P = 1;
-    while (P < m) P <<= 1;
     __syncthreads();
-    double key[E];
-    int idx[E];
-#pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const int i = e * 1024 + tid;
-      key[e] = i < m ? skey[i] : -__builtin_huge_val();  // sentinels sort after every real entry
-      idx[e] = i < m ? sidx[i] : 0x7fffffff;
+    bitonic_sort_desc<SORT_CAP>(skey, sidx, m, tid, d.cross_idx);
+  }
+}
+
+// Sorts a crossing list of at most 1024 entries that the multi-block classification left in
+// ascending order (keys in d.key, neurons in d.asc_idx).  One block per set.
+__global__ __launch_bounds__(1024) void relu_sort_small_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.x] : one;
+  const int m = d.m;
+  if (m <= 0 || m > 1024) return;
+  __shared__ double skey[1024];
+  __shared__ int sidx[1024];
+  const int tid = threadIdx.x;
+  if (tid < m) {
+    skey[tid] = d.key[tid];
+    sidx[tid] = d.asc_idx[tid];
+  }
+  __syncthreads();
+  bitonic_sort_desc<1024>(skey, sidx, m, tid, d.cross_idx);
+}
+
+// Multi-block classification for sets with more than 1024 neurons: pass 1 counts the crossing and
+// inactive neurons of every 1024-row block, pass 2 turns the block counts into offsets (at most a
+// few dozen values) and writes the ascending crossing list.  Grid: (row blocks, 1, sets).
+__global__ __launch_bounds__(1024) void relu_count_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.z] : one;
+  const int r = blockIdx.x * 1024 + threadIdx.x;
+  const bool valid = r < d.N;
+  const double l = valid ? d.lb[r] : 0.0;
+  const double u = valid ? d.ub[r] : 1.0;
+  const bool inactive = valid && (u <= 0.0);
+  const bool crossing = valid && (l < 0.0) && (u > 0.0);
+  const unsigned long long bc = __ballot(crossing);
+  const unsigned long long bi = __ballot(inactive);
+  __shared__ int wc[16], wi[16];
+  if ((threadIdx.x & 63) == 0) {
+    wc[threadIdx.x >> 6] = __popcll(bc);
+    wi[threadIdx.x >> 6] = __popcll(bi);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int c = 0, i = 0;
+    for (int w = 0; w < 16; ++w) {
+      c += wc[w];
+      i += wi[w];
     }
-    for (int k = 2; k <= P; k <<= 1) {
-      for (int j = k >> 1; j > 0; j >>= 1) {
-        if (j >= 64 && j < 1024) {
-          __syncthreads();
-#pragma unroll
-          for (int e = 0; e < E; ++e) {
-            skey[e * 1024 + tid] = key[e];
-            sidx[e * 1024 + tid] = idx[e];
-          }
-          __syncthreads();
-        }
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          const int i = e * 1024 + tid;
-          if (i >= P) continue;
-          double pk;
-          int pi;
-          if (j >= 1024) {
-            const int pe = e ^ (j >> 10);
-            // both registers of the pair are updated when the lower one is visited
-            if (pe < e) continue;
-            pk = key[pe];
-            pi = idx[pe];
-            const bool want_before = (i & k) == 0;
-            if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
-              key[pe] = key[e];
-              idx[pe] = idx[e];
-              key[e] = pk;
-              idx[e] = pi;
-            }
-            continue;
-          } else if (j >= 64) {
-            pk = skey[i ^ j];
-            pi = sidx[i ^ j];
-          } else {
-            pk = __shfl_xor(key[e], j);
-            pi = __shfl_xor(idx[e], j);
-          }
-          const bool want_before = ((i & j) == 0) == ((i & k) == 0);
-          if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
-            key[e] = pk;
-            idx[e] = pi;
-          }
-        }
-      }
+    d.blk_counts[2 * blockIdx.x] = c;
+    d.blk_counts[2 * blockIdx.x + 1] = i;
+  }
+}
+
+__global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.z] : one;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  __shared__ int wcross[16];
+  __shared__ int sbase, stot, sinact;
+  if (wave == 0) {  // offset of this block = crossing counts of the blocks before it
+    int before = 0, tot = 0, inact = 0;
+    for (int b = lane; b < (int)gridDim.x; b += 64) {
+      const int c = d.blk_counts[2 * b];
+      before += b < (int)blockIdx.x ? c : 0;
+      tot += c;
+      inact += d.blk_counts[2 * b + 1];
     }
+    for (int off = 32; off > 0; off >>= 1) {
+      before += __shfl_xor(before, off);
+      tot += __shfl_xor(tot, off);
+      inact += __shfl_xor(inact, off);
+    }
+    if (lane == 0) {
+      sbase = before;
+      stot = tot;
+      sinact = inact;
+    }
+  }
+  const int r = blockIdx.x * 1024 + tid;
+  const bool valid = r < d.N;
+  const double l = valid ? d.lb[r] : 0.0;
+  const double u = valid ? d.ub[r] : 1.0;
+  const bool inactive = valid && (u <= 0.0);
+  const bool crossing = valid && (l < 0.0) && (u > 0.0);
+  const unsigned long long bc = __ballot(crossing);
+  if (lane == 0) wcross[wave] = __popcll(bc);
+  __syncthreads();
+  int woff = 0;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const int i = e * 1024 + tid;
-      if (i < m) d.cross_idx[i] = idx[e];
+  for (int w = 0; w < 16; ++w) woff += w < wave ? wcross[w] : 0;
+  int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
+  if (crossing) {
+    const int pos = sbase + woff + __popcll(bc & ((1ull << lane) - 1ull));
+    idx_out[pos] = r;
+    d.cls[r] = pos;
+    if (d.order != NNVHIP_ORDER_INDEX) {
+      d.key[pos] = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : u - l;
+      d.rank[pos] = 0;
+    }
+  } else if (valid) {
+    d.cls[r] = inactive ? kZero : kKeep;
+  }
+  if (blockIdx.x == gridDim.x - 1) {
+    for (int64_t p = d.N + tid; p < d.ld; p += 1024) d.cls[p] = kKeep;  // padding rows stay zero
+    if (tid == 0) {
+      d.counts[0] = stot;
+      d.counts[1] = sinact;
     }
   }
 }
@@ -289,9 +401,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const bool sorted = order != NNVHIP_ORDER_INDEX;
 
   // scratch shared by all sets: cls | counts ; cross_idx is kept (it becomes the node's index list)
-  BufRef cls_buf, cnt_buf, asc_buf, key_buf, rank_buf;
+  BufRef cls_buf, cnt_buf, asc_buf, key_buf, rank_buf, blk_buf;
+  const int64_t nblk = ceil_div(N, 1024);
   NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &cls_buf));
   NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * count, &cnt_buf));
+  if (N > 8192) NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * nblk * count, &blk_buf));
   if (sorted) {
     NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &asc_buf));
     NNV_TRY(ctx->alloc(sizeof(double) * ld * count, &key_buf));
@@ -314,6 +428,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.key = sorted ? key_buf->as<double>() + ld * i : nullptr;
     d.rank = sorted ? rank_buf->as<int32_t>() + ld * i : nullptr;
     d.counts = cnt_buf->as<int32_t>() + 2 * i;
+    d.blk_counts = blk_buf ? blk_buf->as<int32_t>() + 2 * nblk * i : nullptr;
     d.ld = ld;
     d.N = (int32_t)N;
     d.ncols_in = (int32_t)(in[i]->n + 1);
@@ -325,15 +440,21 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
-  // crossing lists short enough for LDS are sorted inside the classification kernel
-  int sort_cap = 0;
-  if (sorted) sort_cap = N <= 1024 ? 1024 : 8192;
-  if (sort_cap == 0)
-    hipLaunchKernelGGL(relu_classify_kernel<0>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
-  else if (sort_cap == 1024)
-    hipLaunchKernelGGL(relu_classify_kernel<1024>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
-  else
-    hipLaunchKernelGGL(relu_classify_kernel<8192>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+  // Up to 8192 neurons: one block per set classifies, compacts and sorts (bitonic network).  Larger
+  // sets: two multi-block passes; their sort, if any, follows the read-back of the counts.
+  const int sort_cap = !sorted ? 0 : N <= 1024 ? 1024 : N <= 8192 ? 8192 : 0;
+  if (N <= 8192) {
+    if (!sorted)
+      hipLaunchKernelGGL(relu_classify_kernel<0>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+    else if (N <= 1024)
+      hipLaunchKernelGGL(relu_classify_kernel<1024>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+    else
+      hipLaunchKernelGGL(relu_classify_kernel<8192>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+  } else {
+    const dim3 grid((unsigned)ceil_div(N, 1024), 1, (unsigned)count);
+    hipLaunchKernelGGL(relu_count_kernel, grid, dim3(1024), 0, ctx->stream, table, descs[0]);
+    hipLaunchKernelGGL(relu_compact_kernel, grid, dim3(1024), 0, ctx->stream, table, descs[0]);
+  }
   NNV_HIP_TRY(hipGetLastError());
 
   // the column count of the output depends on m: read the counts back
@@ -385,7 +506,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
-  if (sorted && max_m > sort_cap) {  // some list was too long for the in-LDS sort: rank every list
+  if (sorted && sort_cap == 0 && max_m > 0 && max_m <= 1024) {
+    hipLaunchKernelGGL(relu_sort_small_kernel, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+  } else if (sorted && max_m > sort_cap) {  // lists too long for the in-LDS sort: rank every list
     const unsigned t = (unsigned)ceil_div(max_m, 256);
     if (t > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "too many crossing neurons for the sort kernel");
     hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
