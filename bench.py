@@ -93,20 +93,27 @@ def main():
     # ---- per-layer and per-kernel timing with HIP events on the library's stream -----------------
     # set_timing brackets every layer call (NN.reachTime) and, separately, every launch of the two
     # MFMA kernels with their own event pair, so the kernel's duration excludes host gaps.
-    ctx.set_timing(True)
-    ctx.kernel_time(0)
-    ctx.kernel_time(1)
-    per_layer = np.zeros(len(net.Layers))
     reps = max(5, min(args.steps, 20))
-    for _ in range(reps):
-        rs = dev_in
-        for i, L in enumerate(net.Layers):
-            rs = L.reach(rs, args.method, [], 1, None, "linprog")
-            per_layer[i] += ctx.last_op_time_ms()
-    per_layer /= reps
+
+    def timed_pass(level):
+        ctx.set_timing(level)
+        acc = np.zeros(len(net.Layers))
+        for _ in range(reps):
+            rs = dev_in
+            for i, L in enumerate(net.Layers):
+                rs = L.reach(rs, args.method, [], 1, None, "linprog")
+                acc[i] += ctx.last_op_time_ms()
+        ctx.set_timing(0)
+        return acc / reps
+
+    per_layer = timed_pass(1)          # NN.reachTime-style device time per layer
+    for grp in range(4):
+        ctx.kernel_time(grp)
+    timed_pass(2)                      # per-kernel event pairs
     gemm_ms, gemm_launches, _ = ctx.kernel_time(0)
     conv_ms, conv_launches, _ = ctx.kernel_time(1)
-    ctx.set_timing(False)
+    rng_ms, rng_launches, rng_bytes = ctx.kernel_time(2)
+    app_ms, app_launches, app_bytes = ctx.kernel_time(3)
 
     # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
     gemm_flop = conv_flop = 0.0
@@ -163,6 +170,16 @@ def main():
         achieved = relu_bytes / (relu_ms * 1e-3) / 1e9
         roofline = {"kernel": "relu step", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None}
+    # the HBM-bound kernels: algorithmic bytes over their own HIP-event durations
+    hbm = {}
+    for name, ms_, n_, b_ in (("ranges_partial_kernel", rng_ms, rng_launches, rng_bytes),
+                              ("relu_apply_kernel", app_ms, app_launches, app_bytes)):
+        if n_:
+            g = b_ / (ms_ * 1e-3) / 1e9
+            hbm[name] = {"bound": "hbm", "achieved": round(g, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(g / HBM_PEAK_GBS, 4), "launches_per_step": n_ // reps,
+                         "avg_launch_ms": round(ms_ / n_, 5)}
+    roofline["hbm_kernels"] = hbm
     t = MEASURED_TRAFFIC_MIB.get((cfg["name"], roofline["kernel"]))
     if t is not None and args.method == "relax-star-area":
         roofline["traffic"] = round((t[0] + t[1]) * 1048576.0)

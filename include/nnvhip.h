@@ -27,6 +27,12 @@
 
 #include <stdint.h>
 
+#if defined(__GNUC__)
+#define NNVHIP_API __attribute__((visibility("default")))
+#else
+#define NNVHIP_API
+#endif
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -56,39 +62,41 @@ typedef enum { NNVHIP_ORDER_INDEX = 0, NNVHIP_ORDER_AREA = 1, NNVHIP_ORDER_RANGE
 /* ---- context -------------------------------------------------------------------------- */
 /* Replaces NN.reach's reachOptions.device hook (nn/NN.m:216-222): selects the GPU, creates the
  * stream and the device memory pool. */
-int nnvhip_create(int device, nnvhip_ctx** ctx);
-int nnvhip_destroy(nnvhip_ctx* ctx);
+NNVHIP_API int nnvhip_create(int device, nnvhip_ctx** ctx);
+NNVHIP_API int nnvhip_destroy(nnvhip_ctx* ctx);
 /* Message of the last failing call on this thread. */
-const char* nnvhip_last_error(void);
+NNVHIP_API const char* nnvhip_last_error(void);
 /* Waits for all queued device work of the context (wait(gpuDevice) in the reference's GPU path). */
-int nnvhip_synchronize(nnvhip_ctx* ctx);
+NNVHIP_API int nnvhip_synchronize(nnvhip_ctx* ctx);
 /* Device time in ms of the most recent layer call (NN.reachTime(i) = toc, nn/NN.m:1542-1545).
- * Timing is off by default; enabling it makes this call wait for the layer to finish. */
-int nnvhip_set_timing(nnvhip_ctx* ctx, int enabled);
-int nnvhip_last_op_time_ms(nnvhip_ctx* ctx, double* ms);
-/* Measurement hook (no counterpart in the reference): while timing is enabled, every launch of an
- * MFMA kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
- * dense GEMM kernel of the FC layers (tiles of at least 64 rows); which = 1: implicit-GEMM
- * convolution kernel.  Returns accumulated kernel time, launch count and dense flop executed
- * (GEMM: 2*Mp*Kp*ncols with M, K padded to 16; conv: 2*Ho*Wo*Cout*FH*FW*Cin*(n+1)) since the last
- * reset. */
-int nnvhip_kernel_time(nnvhip_ctx* ctx, int which, double* total_ms, int64_t* launches, double* total_flop,
+ * Timing is off by default (enabled = 0); 1 brackets every layer call with HIP events and makes the
+ * call wait for the layer to finish; 2 additionally brackets single kernels (nnvhip_kernel_time). */
+NNVHIP_API int nnvhip_set_timing(nnvhip_ctx* ctx, int enabled);
+NNVHIP_API int nnvhip_last_op_time_ms(nnvhip_ctx* ctx, double* ms);
+/* Measurement hook (no counterpart in the reference): while timing level 2 is set, every launch of a
+ * kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
+ * dense GEMM kernel of the FC layers (tiles of at least 64 rows); 1: implicit-GEMM convolution
+ * kernel; 2: estimateRanges column pass; 3: ReLU apply pass.  Returns accumulated kernel time,
+ * launch count and work since the last reset.  Work is dense flop for 0 and 1 (GEMM:
+ * 2*Mp*Kp*ncols with M, K padded to 16; conv: 2*Ho*Wo*Cout*FH*FW*Cin*(n+1)) and algorithmic bytes for
+ * 2 (8*N*(n+1) + 16*n + 16*N per set) and 3 (8*N*(n+1) read + 8*N*(n+1+m) written per set). */
+NNVHIP_API int nnvhip_kernel_time(nnvhip_ctx* ctx, int which, double* total_ms, int64_t* launches, double* total_work,
                        int reset);
 /* Measurement hook (no counterpart in the reference): runs a plain device-to-device copy kernel over
  * `bytes` (reps + 1 times) and returns the achieved read+write bandwidth of the timed reps in GB/s -
  * the practical HBM ceiling on this box, and the known-size kernel hardware counters are
  * calibrated against. */
-int nnvhip_probe_copy_bandwidth(nnvhip_ctx* ctx, int64_t bytes, int reps, double* gbytes_per_s);
+NNVHIP_API int nnvhip_probe_copy_bandwidth(nnvhip_ctx* ctx, int64_t bytes, int reps, double* gbytes_per_s);
 /* Returns every cached device block of the pool to the driver (hipFree). */
-int nnvhip_trim_pool(nnvhip_ctx* ctx);
+NNVHIP_API int nnvhip_trim_pool(nnvhip_ctx* ctx);
 /* Bytes currently handed out by / cached in the pool. */
-int nnvhip_pool_stats(nnvhip_ctx* ctx, int64_t* bytes_in_use, int64_t* bytes_cached);
+NNVHIP_API int nnvhip_pool_stats(nnvhip_ctx* ctx, int64_t* bytes_in_use, int64_t* bytes_cached);
 
 /* ---- sets ----------------------------------------------------------------------------- */
 /* Star(V, C, d, pred_lb, pred_ub), set/Star.m:153-189: uploads host arrays.  V is N x (n+1),
  * C is p x n, d has p entries; pred_lb/pred_ub may be NULL (both) for the -1/+1 default of
  * Star.estimateRanges (set/Star.m:1091-1096).  C/d may be NULL with p = 0. */
-int nnvhip_star_create(nnvhip_ctx* ctx, int64_t N, int64_t n, const double* V, const double* pred_lb,
+NNVHIP_API int nnvhip_star_create(nnvhip_ctx* ctx, int64_t N, int64_t n, const double* V, const double* pred_lb,
                        const double* pred_ub, const double* C, const double* d, int64_t p,
                        nnvhip_star** out);
 /* Star(lb, ub), set/Star.m:220-237 with Box (set/Box.m:16-58): centre 0.5*(lb+ub), one
@@ -96,66 +104,66 @@ int nnvhip_star_create(nnvhip_ctx* ctx, int64_t N, int64_t n, const double* V, c
  * predicate bounds -1/+1.  Built on the device from the two N-vectors.  `count` boxes are given
  * as the columns of N x count matrices; out[] receives `count` handles laid out back to back in
  * one device arena (the array of Stars NN.reach accepts, nn/NN.m:204-207). */
-int nnvhip_star_from_box(nnvhip_ctx* ctx, int64_t N, int64_t count, const double* lb, const double* ub,
+NNVHIP_API int nnvhip_star_from_box(nnvhip_ctx* ctx, int64_t N, int64_t count, const double* lb, const double* ub,
                          nnvhip_star** out);
-int nnvhip_star_retain(nnvhip_star* s);
-int nnvhip_star_release(nnvhip_star* s);
+NNVHIP_API int nnvhip_star_retain(nnvhip_star* s);
+NNVHIP_API int nnvhip_star_release(nnvhip_star* s);
 /* dim, nVar and the number of constraint rows size(C,1). */
-int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p);
+NNVHIP_API int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p);
 /* Property reads: dense MATLAB arrays.  V: N x (n+1).  Bounds: n each.  C: p x n, d: p, laid out
  * exactly as PosLin.multipleStepReachStarApprox_at_one builds them, [C0;C1;C2;C3]
  * (nn/funcs/PosLin.m:711-735), materialised from the device's structured store. */
-int nnvhip_star_fetch_V(const nnvhip_star* s, double* V);
-int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* pred_lb, double* pred_ub);
-int nnvhip_star_fetch_constraints(const nnvhip_star* s, double* C, double* d);
+NNVHIP_API int nnvhip_star_fetch_V(const nnvhip_star* s, double* V);
+NNVHIP_API int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* pred_lb, double* pred_ub);
+NNVHIP_API int nnvhip_star_fetch_constraints(const nnvhip_star* s, double* C, double* d);
 /* For a set returned by nnvhip_relu_relax: counts of inactive (ub <= 0) and crossing
  * (lb < 0 & ub > 0) neurons, and the crossing list in new-predicate order with its bounds
  * (map1/map2 and lb(map), ub(map) of nn/funcs/PosLin.m:921-925, 1094-1096).  Any output pointer
  * may be NULL. */
-int nnvhip_star_relu_counts(const nnvhip_star* s, int64_t* n_inactive, int64_t* n_crossing);
-int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb, double* ub);
+NNVHIP_API int nnvhip_star_relu_counts(const nnvhip_star* s, int64_t* n_inactive, int64_t* n_crossing);
+NNVHIP_API int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb, double* ub);
 
 /* ---- Star.estimateRanges, set/Star.m:1078-1106 ------------------------------------------ */
 /* lb = c + max(V,0)*[0;pred_lb] + min(V,0)*[0;pred_ub]; ub likewise.  One pass over V; the
  * result is cached on the handle (nnvhip_relu_relax reuses it).  lb/ub: host, N entries each,
  * may be NULL to only compute and cache on the device. */
-int nnvhip_estimate_ranges(nnvhip_ctx* ctx, nnvhip_star* s, double* lb, double* ub);
+NNVHIP_API int nnvhip_estimate_ranges(nnvhip_ctx* ctx, nnvhip_star* s, double* lb, double* ub);
 /* Array form: lb/ub are N x count (all sets must have the same dim). */
-int nnvhip_estimate_ranges_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, double* lb,
+NNVHIP_API int nnvhip_estimate_ranges_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, double* lb,
                                  double* ub);
 
 /* ---- layers ---------------------------------------------------------------------------- */
 /* FullyConnectedLayer(W, b), nn/layers/FullyConnectedLayer.m:39-99: W is M x K, b has M entries
  * (NULL = no bias, the affineMap(W, []) form). */
-int nnvhip_fc_create(nnvhip_ctx* ctx, const double* W, const double* b, int64_t M, int64_t K,
+NNVHIP_API int nnvhip_fc_create(nnvhip_ctx* ctx, const double* W, const double* b, int64_t M, int64_t K,
                      nnvhip_fc** out);
-int nnvhip_fc_destroy(nnvhip_fc* fc);
+NNVHIP_API int nnvhip_fc_destroy(nnvhip_fc* fc);
 /* Conv2DLayer(W, b, padding, stride, dilation), nn/layers/Conv2DLayer.m:15-33: W is
  * FH x FW x Cin x Cout, bias has Cout entries (NULL = 0), padding [t b l r], stride [sh sw],
  * dilation [dh dw]. */
-int nnvhip_conv2d_create(nnvhip_ctx* ctx, const double* W, const double* bias, int64_t FH, int64_t FW,
+NNVHIP_API int nnvhip_conv2d_create(nnvhip_ctx* ctx, const double* W, const double* bias, int64_t FH, int64_t FW,
                          int64_t Cin, int64_t Cout, const int64_t padding[4], const int64_t stride[2],
                          const int64_t dilation[2], nnvhip_conv2d** out);
-int nnvhip_conv2d_destroy(nnvhip_conv2d* conv);
+NNVHIP_API int nnvhip_conv2d_destroy(nnvhip_conv2d* conv);
 /* Output feature-map size for an H x W input, nn/layers/Conv2DLayer.m:1134-1135. */
-int nnvhip_conv2d_output_size(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t* Ho, int64_t* Wo);
+NNVHIP_API int nnvhip_conv2d_output_size(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t* Ho, int64_t* Wo);
 
 /* FullyConnectedLayer.reach_star_single_input / Star.affineMap,
  * nn/layers/FullyConnectedLayer.m:295-316, 476-481; set/Star.m:313-343:
  * V' = W*V; V'(:,1) += b; constraints and predicate bounds are shared with the input.
  * `count` sets are mapped in one pass (reach_star_multipleInputs, :486-512). */
-int nnvhip_affine_fc(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, nnvhip_star* const* in,
+NNVHIP_API int nnvhip_affine_fc(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, nnvhip_star* const* in,
                      nnvhip_star** out);
 /* Conv2DLayer.reach_star_single_input, nn/layers/Conv2DLayer.m:559-601, 780: the input set is
  * read as an H x W x Cin x (n+1) ImageStar; centre gets conv + bias, generators conv only;
  * cross-correlation (no kernel flip), zero padding.  Output dim is Ho*Wo*Cout. */
-int nnvhip_affine_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t count,
+NNVHIP_API int nnvhip_affine_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t count,
                          nnvhip_star* const* in, nnvhip_star** out);
 /* ReluLayer.reach -> PosLin.reach(I, 'relax-star-*', [], relaxFactor, ...),
  * nn/layers/ReluLayer.m:72-150, nn/funcs/PosLin.m:863-1650, 685-742, set/Star.m:1442-1461.
  * estimateRanges; inactive rows -> 0; every crossing neuron gets a new predicate column, the
  * three triangle constraints and predicate bounds [0, ub].  relax_factor must be 1 (no LP). */
-int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor, int64_t count,
+NNVHIP_API int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor, int64_t count,
                       nnvhip_star* const* in, nnvhip_star** out);
 
 #ifdef __cplusplus

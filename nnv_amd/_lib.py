@@ -128,8 +128,9 @@ class Context:
     def synchronize(self):
         check(self.lib.nnvhip_synchronize(self.handle))
 
-    def set_timing(self, enabled: bool):
-        check(self.lib.nnvhip_set_timing(self.handle, 1 if enabled else 0))
+    def set_timing(self, level):
+        """0/False: off; 1/True: per-layer device times; 2: also per-kernel timers (kernel_time)."""
+        check(self.lib.nnvhip_set_timing(self.handle, int(level)))
 
     def last_op_time_ms(self) -> float:
         ms = C.c_double()
@@ -137,8 +138,9 @@ class Context:
         return ms.value
 
     def kernel_time(self, which, reset=True):
-        """(total ms, launches, dense flop) of an MFMA kernel group (0 = FC GEMM, 1 = convolution)
-        accumulated while timing was enabled."""
+        """(total ms, launches, work) of a kernel group accumulated while timing was enabled:
+        0 = FC GEMM, 1 = convolution (work = dense flop); 2 = estimateRanges pass, 3 = ReLU apply pass
+        (work = algorithmic bytes)."""
         ms, n, fl = C.c_double(), C.c_int64(), C.c_double()
         check(self.lib.nnvhip_kernel_time(self.handle, int(which), C.byref(ms), C.byref(n), C.byref(fl), 1 if reset else 0))
         return ms.value, n.value, fl.value

@@ -17,7 +17,7 @@ LIB = os.path.join(HERE, "libnnvhip.so")
 SOURCES = ["ctx.hip", "gemm.hip", "conv.hip", "ranges.hip", "relu.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-unknown-warning-option",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,

@@ -181,11 +181,11 @@ static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvG
   const int64_t blocks = ceil_div(total_rows, TP) * tiles_c;
   if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
   const size_t dyn = sizeof(unsigned long long) * g.Kp;
-  NNV_TRY(ctx->kernel_timer_begin(ctx->timing));
+  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL((conv2d_f64_kernel<TP, TC, WR, WC>), dim3((unsigned)blocks), dim3(64 * WR * WC), dyn, ctx->stream, in, ldin,
                      out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows,
                      (int)tiles_c);
-  NNV_TRY(ctx->kernel_timer_end(ctx->timing, 1, 2.0 * (double)total_rows * g.Cout * g.K));
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 1, 2.0 * (double)total_rows * g.Cout * g.K));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }

@@ -204,6 +204,7 @@ int nnvhip_synchronize(nnvhip_ctx* c) {
 int nnvhip_set_timing(nnvhip_ctx* c, int enabled) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
   c->timing = enabled != 0;
+  c->kernel_timing = enabled >= 2;
   return NNVHIP_OK;
 }
 
@@ -215,7 +216,7 @@ int nnvhip_last_op_time_ms(nnvhip_ctx* c, double* ms) {
 
 int nnvhip_kernel_time(nnvhip_ctx* c, int which, double* total_ms, int64_t* launches, double* total_flop, int reset) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
-  if (which < 0 || which > 1) NNV_FAIL(NNVHIP_ERR_ARG, "unknown kernel group %d", which);
+  if (which < 0 || which >= nnvhip_ctx::kKernelGroups) NNV_FAIL(NNVHIP_ERR_ARG, "unknown kernel group %d", which);
   if (total_ms) *total_ms = c->kern_ms[which];
   if (launches) *launches = c->kern_launches[which];
   if (total_flop) *total_flop = c->kern_flop[which];

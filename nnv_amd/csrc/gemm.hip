@@ -15,7 +15,7 @@ namespace nnvhip {
 
 // TM x TN output tile per block of WR x WC waves, each wave owning
 // (TM/WR) x (TN/WC) = (16*FM) x (16*FN).
-template <int TM, int TN, int WR, int WC, int KT, int NS>
+template <int TM, int TN, int WR, int WC, int KT>
 __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __restrict__ A, int64_t lda,
                                                         const double* __restrict__ B, int64_t ldb,
                                                         double* __restrict__ C, int64_t ldc, int Mp, int64_t ncols,
@@ -27,9 +27,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   constexpr int FN = TN / WC / 16;
   constexpr int LDA_S = TM + kPadRow;  // Ws[k][row]
   constexpr int LDB_S = KT + kPadK;    // Vs[col][k]
-  static_assert(NS == 2 || NS == 3, "two or three LDS stages");
-  __shared__ double Ws[NS][KT * LDA_S];
-  __shared__ double Vs[NS][TN * LDB_S];
+  __shared__ double Ws[2][KT * LDA_S];
+  __shared__ double Vs[2][TN * LDB_S];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -109,45 +108,19 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   const int nk_all = Kp / KT;
   const int kt0 = (int)((int64_t)nk_all * blockIdx.y / ksplit);
   const int kt1 = (int)((int64_t)nk_all * (blockIdx.y + 1) / ksplit);
+  // two LDS stages: tile t+1 travels global -> registers while tile t is multiplied, then goes to the
+  // other stage; one barrier per K-tile.  (A three-stage variant with the barrier hidden behind the
+  // first MFMA step measured no faster: the limit is the per-wave MFMA issue cadence, not the barrier.)
   const int nk = kt1 - kt0;
-  if (NS == 2) {
-    // two LDS stages: tile t+1 travels global -> registers while tile t is multiplied, then goes to
-    // the other stage; one barrier per K-tile between the two
-    load_tiles(kt0 * KT);
-    store_tiles(0);
+  load_tiles(kt0 * KT);
+  store_tiles(0);
+  __syncthreads();
+  for (int t = 0; t < nk; ++t) {
+    const int cur = t & 1;
+    if (t + 1 < nk) load_tiles((kt0 + t + 1) * KT);
+    mfma_tile_k16<FM, FN, KT>(&Ws[cur][wr * (TM / WR)], LDA_S, &Vs[cur][(wc * (TN / WC)) * LDB_S], LDB_S, lane, acc);
+    if (t + 1 < nk) store_tiles(cur ^ 1);
     __syncthreads();
-    for (int t = 0; t < nk; ++t) {
-      const int cur = t & 1;
-      if (t + 1 < nk) load_tiles((kt0 + t + 1) * KT);
-      mfma_tile_k16<FM, FN, KT>(&Ws[cur][wr * (TM / WR)], LDA_S, &Vs[cur][(wc * (TN / WC)) * LDB_S], LDB_S, lane, acc);
-      if (t + 1 < nk) store_tiles(cur ^ 1);
-      __syncthreads();
-    }
-  } else {
-    // three LDS stages: tile t+1 is already complete in LDS when tile t is multiplied, so the one
-    // barrier per K-tile sits behind the first MFMA step of the tile (the MFMA pipe keeps working
-    // while waves meet) and only guards the stage that tile t+2 overwrites.
-    load_tiles(kt0 * KT);
-    store_tiles(0);
-    if (nk > 1) {
-      load_tiles((kt0 + 1) * KT);
-      store_tiles(1);
-    }
-    __syncthreads();
-    if (nk > 2) load_tiles((kt0 + 2) * KT);
-    int cur = 0;
-    for (int t = 0; t < nk; ++t) {
-      const double* ws = &Ws[cur][wr * (TM / WR)];
-      const double* vs = &Vs[cur][(wc * (TN / WC)) * LDB_S];
-      mfma_tile_k16<FM, FN, KT, 0, 1>(ws, LDA_S, vs, LDB_S, lane, acc);
-      __syncthreads();
-      if (t + 2 < nk) {
-        store_tiles(cur == 0 ? 2 : cur - 1);  // stage of tile t-1
-        if (t + 3 < nk) load_tiles((kt0 + t + 3) * KT);
-      }
-      mfma_tile_k16<FM, FN, KT, 1, KT / 4>(ws, LDA_S, vs, LDB_S, lane, acc);
-      cur = cur == 2 ? 0 : cur + 1;
-    }
   }
   if (ksplit > 1) {  // partial sums go to the workspace (ld = Mp); bias is added by the reduction
     C = part + (int64_t)blockIdx.y * Mp * ncols;
@@ -191,7 +164,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __rest
   C[row + col * ldc] = s;
 }
 
-template <int TM, int TN, int WR, int WC, int KT, int NS = 2>
+template <int TM, int TN, int WR, int WC, int KT>
 static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
                       int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias) {
   int64_t tiles_m = ceil_div(Mp, TM);
@@ -226,9 +199,9 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
   BufRef ws;
   if (ksplit > 1) NNV_TRY(ctx->alloc(sizeof(double) * ksplit * Mp * ncols, &ws));
-  const bool timed = ctx->timing && TM >= 64;
+  const bool timed = ctx->kernel_timing && TM >= 64;
   NNV_TRY(ctx->kernel_timer_begin(timed));
-  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT, NS>), dim3((unsigned)grid_x, (unsigned)ksplit), dim3(64 * WR * WC), 0,
+  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)grid_x, (unsigned)ksplit), dim3(64 * WR * WC), 0,
                      ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)tiles_n,
                      (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, 2.0 * (double)Mp * (double)Kp * (double)ncols));
@@ -250,39 +223,7 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
   // Tile choice: the largest tile that still yields a few blocks per CU; skinny outputs (the last
   // layer has 10 rows) get a 16-row tile.  K must be a multiple of the K-tile (16 or 32).
 #define NNV_GEMM(TM, TN, WR, WC, KT) launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias)
-#define NNV_GEMM3(TM, TN, WR, WC) launch_cfg<TM, TN, WR, WC, 16, 3>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias)
   const int64_t kCUs = 256;
-  const bool k32 = Kp % 32 == 0;
-  if (const char* e = getenv("NNVHIP_GEMM_TILE")) {  // tuning knob
-    const std::string t(e);
-    if (t == "s3:64x64") return NNV_GEMM3(64, 64, 2, 4);
-    if (t == "s3:128x64") return NNV_GEMM3(128, 64, 4, 2);
-    if (t == "s3:128x80") return NNV_GEMM3(128, 80, 8, 1);
-    if (t == "s3:64x96") return NNV_GEMM3(64, 96, 4, 2);
-    if (t == "s3:128x128") return NNV_GEMM3(128, 128, 2, 4);
-    if (t == "s3:128x32") return NNV_GEMM3(128, 32, 8, 1);
-    if (t == "128x32") return NNV_GEMM(128, 32, 8, 1, 16);
-    if (t == "128x48") return NNV_GEMM(128, 48, 8, 1, 16);
-    if (t == "128x64") return NNV_GEMM(128, 64, 8, 1, 16);
-    if (t == "128x80") return NNV_GEMM(128, 80, 8, 1, 16);
-    if (t == "128x96") return NNV_GEMM(128, 96, 8, 1, 16);
-    if (t == "128x112") return NNV_GEMM(128, 112, 8, 1, 16);
-    if (t == "64x96") return NNV_GEMM(64, 96, 4, 2, 16);
-    if (t == "64x128") return NNV_GEMM(64, 128, 4, 2, 16);
-    if (t == "64x32") return NNV_GEMM(64, 32, 4, 2, 16);
-    if (t == "128x128x16") return NNV_GEMM(128, 128, 2, 2, 16);
-    if (t == "128x128x16w8") return NNV_GEMM(128, 128, 2, 4, 16);
-    if (t == "128x64x16w8") return NNV_GEMM(128, 64, 4, 2, 16);
-    if (t == "64x64x16w8") return NNV_GEMM(64, 64, 2, 4, 16);
-    if (t == "64x128x16w8") return NNV_GEMM(64, 128, 2, 4, 16);
-    if (k32 && t == "64x64x32w8") return NNV_GEMM(64, 64, 2, 4, 32);
-    if (k32 && t == "128x64x32w8") return NNV_GEMM(128, 64, 4, 2, 32);
-    if (t == "128x64x16") return NNV_GEMM(128, 64, 2, 2, 16);
-    if (t == "64x64x16") return NNV_GEMM(64, 64, 2, 2, 16);
-    if (t == "32x128x16") return NNV_GEMM(32, 128, 1, 4, 16);
-    if (k32 && t == "128x64x32") return NNV_GEMM(128, 64, 2, 2, 32);
-    if (k32 && t == "64x64x32") return NNV_GEMM(64, 64, 2, 2, 32);
-  }
   if (Mp <= 16) return NNV_GEMM(16, 64, 1, 4, 16);
   if (Mp <= 32) return NNV_GEMM(32, 128, 1, 4, 16);
   // Eight-wave tiles (two waves per SIMD issue MFMAs even with one block per CU).  The shape is
@@ -306,6 +247,10 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
       best_cost = cost;
     }
   }
+  if (const char* e = getenv("NNVHIP_GEMM_TILE")) {  // tuning knob: "TMxTN" of one of the shapes above
+    for (int i = 0; i < (int)(sizeof(shapes) / sizeof(shapes[0])); ++i)
+      if (std::to_string(shapes[i].tm) + "x" + std::to_string(shapes[i].tn) == e) best = i;
+  }
   switch (shapes[best].tm * 1000 + shapes[best].tn) {
     case 64064: return NNV_GEMM(64, 64, 2, 4, 16);
     case 64096: return NNV_GEMM(64, 96, 4, 2, 16);
@@ -318,7 +263,6 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
     default: return NNV_GEMM(128, 128, 2, 4, 16);
   }
 #undef NNV_GEMM
-#undef NNV_GEMM3
 }
 
 __global__ void bias_columns_kernel(double* const* __restrict__ cols, const double* __restrict__ bias, int Mp) {

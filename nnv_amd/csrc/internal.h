@@ -98,15 +98,18 @@ struct nnvhip_ctx {
   size_t pinned_bytes = 0;
   size_t pinned_off = 0;
   // per-layer timing
-  bool timing = false;
+  bool timing = false;         // per-layer events (nnvhip_last_op_time_ms)
+  bool kernel_timing = false;  // additionally one event pair per launch of the timed kernel groups
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   double last_ms = 0.0;
   // timing of the dominant kernel alone (events directly around its launch), per instantiation group
   hipEvent_t kev0 = nullptr, kev1 = nullptr;
-  // [0] dense MFMA GEMM (tiles of at least 64 rows), [1] implicit-GEMM convolution
-  double kern_ms[2] = {0.0, 0.0};
-  int64_t kern_launches[2] = {0, 0};
-  double kern_flop[2] = {0.0, 0.0};
+  // [0] dense MFMA GEMM (tiles of at least 64 rows), [1] implicit-GEMM convolution (work = flop),
+  // [2] estimateRanges column pass, [3] ReLU apply pass (work = algorithmic bytes)
+  static constexpr int kKernelGroups = 4;
+  double kern_ms[kKernelGroups] = {0.0, 0.0, 0.0, 0.0};
+  int64_t kern_launches[kKernelGroups] = {0, 0, 0, 0};
+  double kern_flop[kKernelGroups] = {0.0, 0.0, 0.0, 0.0};
   int kernel_timer_begin(bool on);
   int kernel_timer_end(bool on, int which, double flop);
 

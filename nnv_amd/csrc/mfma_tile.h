@@ -12,19 +12,19 @@ constexpr int kKt = 16;      // K-tile of the convolution kernel
 constexpr int kPadRow = 0;  // [k][row] array: a lane group reads 16 consecutive doubles - always distinct
 constexpr int kPadK = 1;    // [col][k] array: odd column stride -> 16 columns hit 16 distinct bank pairs
 
-// MFMA steps [KK0, KK1) (4 deep each; default: the whole KT-deep K-tile) of a (16*FM) x (16*FN) wave tile.
+// One K-tile (KT deep = KT/4 16x16x4 MFMA steps) of a (16*FM) x (16*FN) wave tile.
 //   rows_s: LDS, element (k, row) at rows_s[k * ld_rows + row]   -> MFMA operand "b"
 //   cols_s: LDS, element (col, k) at cols_s[col * ld_cols + k]   -> MFMA operand "a"
 // v_mfma_f64_16x16x4_f64 operand layout on gfx950 (measured): lane l supplies a[i = l%16][k = l/16]
 // and b[k = l/16][j = l%16]; result register r of lane l is D[i = l/16 + 4r][j = l%16].
-template <int FM, int FN, int KT = kKt, int KK0 = 0, int KK1 = KT / 4>
+template <int FM, int FN, int KT = kKt>
 __device__ __forceinline__ void mfma_tile_k16(const double* __restrict__ rows_s, int ld_rows,
                                               const double* __restrict__ cols_s, int ld_cols, int lane,
                                               double4_t (&acc)[FM][FN]) {
   const int l16 = lane & 15;
   const int kq = lane >> 4;
 #pragma unroll
-  for (int kk = KK0; kk < KK1; ++kk) {
+  for (int kk = 0; kk < KT / 4; ++kk) {
     const int k = kk * 4 + kq;
     double b[FM], a[FN];
 #pragma unroll

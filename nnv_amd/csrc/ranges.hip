@@ -178,7 +178,11 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     table = tab->as<RangeDesc>();
   }
   dim3 grid((unsigned)row_blocks, (unsigned)chunks, (unsigned)nset);
+  double bytes = 0.0;  // algorithmic: V once, the predicate bounds, lb/ub out
+  for (auto* t : todo) bytes += 8.0 * (double)t->N * (double)(t->n + 1) + 16.0 * (double)t->n + 16.0 * (double)t->N;
+  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL(ranges_partial_kernel, grid, dim3(256), 0, ctx->stream, table, descs[0]);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
   if (chunks > 1)
     hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,
                        ctx->stream, table, descs[0]);

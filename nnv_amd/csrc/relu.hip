@@ -514,8 +514,13 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
     hipLaunchKernelGGL(relu_scatter_kernel, dim3(t, 1, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
   }
+  double bytes = 0.0;  // algorithmic: read N x (n+1), write N x (n+1+m)
+  for (int64_t i = 0; i < count; ++i)
+    bytes += 8.0 * (double)N * (double)(in[i]->n + 1) + 8.0 * (double)N * (double)(in[i]->n + 1 + descs[i].m);
+  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(256), 0,
                      ctx->stream, table, descs[0]);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 3, bytes));
   NNV_HIP_TRY(hipGetLastError());
 
   for (int64_t i = 0; i < count; ++i) {

@@ -212,3 +212,29 @@ def test_config5_shrunk_batched(nnv, oracle):
     dev, ora, net = run_both(5, "relax-star-area", shrink=4, check_constraints=False)
     assert len(dev) == len(ora) == 4
     run_both(5, "relax-star-random", shrink=8)
+
+
+def test_out_of_memory_is_an_error_code_not_a_crash(nnv):
+    # Star(lb, ub) with 2^20 free dimensions needs an 8.8 TB generator matrix: the library must
+    # report NNVHIP_ERR_OOM (MemoryError here) and stay usable
+    N = 1 << 20
+    with pytest.raises(MemoryError):
+        nnv.Star(np.zeros(N), np.ones(N))
+    S = nnv.Star(np.zeros(4), np.ones(4))
+    assert S.nVar == 4 and np.array_equal(S.estimateRanges()[1], np.ones(4))
+
+
+def test_zero_width_dimensions_and_scalar_box(nnv, oracle):
+    lb = np.array([0.5, -1.0, 2.0, 2.0])
+    ub = np.array([0.5, 1.0, 2.0, 3.0])
+    S = nnv.Star(lb, ub)
+    E = oracle.star_from_box(lb, ub)
+    assert S.nVar == 2 and np.array_equal(S.V, E.V)
+    one = nnv.Star(np.array([1.0]), np.array([1.0]))         # numel(gens) == 1: the zero column stays
+    assert one.nVar == 1 and np.array_equal(one.V, oracle.star_from_box([1.0], [1.0]).V)
+    allfix = nnv.Star(np.array([1.0, 2.0]), np.array([1.0, 2.0]))
+    assert allfix.nVar == 0 and np.array_equal(allfix.V, np.array([[1.0], [2.0]]))
+    l, u = allfix.estimateRanges()
+    assert np.array_equal(l, [1.0, 2.0]) and np.array_equal(u, [1.0, 2.0])
+    R = nnv.PosLin.reach(allfix, "relax-star-area", [], 1)
+    assert R.nVar == 0 and np.array_equal(R.V, allfix.V)
