@@ -5,6 +5,7 @@
 // column chunk; partial sums of the chunks are combined in a fixed order by a second tiny kernel,
 // so results are bit-reproducible from run to run (no floating-point atomics).
 #include <algorithm>
+#include <cstdlib>
 
 #include "internal.h"
 
@@ -21,18 +22,23 @@ struct RangeDesc {
   int32_t n;
   int32_t chunks;
   int32_t cols_per_chunk;
-  int32_t pad_;
+  int32_t row_waves;  // waves of a block laid along rows (1, 2, 4 or 8); the others interleave columns
 };
 
-constexpr int kRowsPerBlock = 128;  // 64 lanes x 2 rows
+constexpr int kRowsPerWave = 128;  // 64 lanes x 2 rows
+constexpr int kRangeWaves = 8;     // waves per block
 
-__global__ __launch_bounds__(256) void ranges_partial_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
+__global__ __launch_bounds__(64 * kRangeWaves) void ranges_partial_kernel(const RangeDesc* __restrict__ table,
+                                                                          RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
   const int chunk = blockIdx.y;
   if (chunk >= d.chunks) return;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t r0 = (int64_t)blockIdx.x * kRowsPerBlock + 2 * lane;
+  const int wrow = wave % d.row_waves;
+  const int wcol = wave / d.row_waves;
+  const int col_waves = kRangeWaves / d.row_waves;
+  const int64_t r0 = ((int64_t)blockIdx.x * d.row_waves + wrow) * kRowsPerWave + 2 * lane;
   const bool active = r0 < d.ld;
   // generator columns are 1..n; chunk c owns [1 + c*cpc, min(n, (c+1)*cpc) + 1)
   const int j0 = 1 + chunk * d.cols_per_chunk;
@@ -41,7 +47,7 @@ __global__ __launch_bounds__(256) void ranges_partial_kernel(const RangeDesc* __
   if (active) {
     const double* col = d.V + r0;
     // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
-    for (int jb = j0 + 4 * wave; jb < j1; jb += 16) {
+    for (int jb = j0 + 4 * wcol; jb < j1; jb += 4 * col_waves) {
       double2 v[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -67,25 +73,26 @@ __global__ __launch_bounds__(256) void ranges_partial_kernel(const RangeDesc* __
       }
     }
   }
-  __shared__ double2 red[3][4][64];
-  if (wave > 0) {
-    red[wave - 1][0][lane] = xmin1;
-    red[wave - 1][1][lane] = xmin2;
-    red[wave - 1][2][lane] = xmax1;
-    red[wave - 1][3][lane] = xmax2;
+  // waves that share rows (same wrow) are combined in wave order by the wcol == 0 wave
+  __shared__ double2 red[kRangeWaves][4][64];
+  if (wcol > 0) {
+    red[wave][0][lane] = xmin1;
+    red[wave][1][lane] = xmin2;
+    red[wave][2][lane] = xmax1;
+    red[wave][3][lane] = xmax2;
   }
   __syncthreads();
-  if (wave == 0 && active) {
-#pragma unroll
-    for (int w = 0; w < 3; ++w) {
-      xmin1.x += red[w][0][lane].x;
-      xmin1.y += red[w][0][lane].y;
-      xmin2.x += red[w][1][lane].x;
-      xmin2.y += red[w][1][lane].y;
-      xmax1.x += red[w][2][lane].x;
-      xmax1.y += red[w][2][lane].y;
-      xmax2.x += red[w][3][lane].x;
-      xmax2.y += red[w][3][lane].y;
+  if (wcol == 0 && active) {
+    for (int w = 1; w < col_waves; ++w) {
+      const int src = w * d.row_waves + wrow;
+      xmin1.x += red[src][0][lane].x;
+      xmin1.y += red[src][0][lane].y;
+      xmin2.x += red[src][1][lane].x;
+      xmin2.y += red[src][1][lane].y;
+      xmax1.x += red[src][2][lane].x;
+      xmax1.y += red[src][2][lane].y;
+      xmax2.x += red[src][3][lane].x;
+      xmax2.y += red[src][3][lane].y;
     }
     if (d.chunks == 1) {
       // lb = (c + xmin1) + xmin2, the reference's left-to-right order
@@ -146,7 +153,12 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   }
   // Column chunking: enough blocks to cover the chip a few times over, at least 64 columns per
   // chunk so the partial-sum traffic stays below ~6 % of V.
-  const int64_t row_blocks = ceil_div(ld, kRowsPerBlock);
+  int row_waves = 1;  // measured best: all eight waves on the same 128 rows, interleaving columns
+  if (const char* e = getenv("NNVHIP_RANGES_ROW_WAVES")) {
+    const int v = atoi(e);
+    row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
+  }
+  const int64_t row_blocks = ceil_div(ld, kRowsPerWave * row_waves);
   const int64_t want_blocks = 2048;
   int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * nset), ceil_div(nmax, 64)));
   chunks = std::min<int64_t>(chunks, 1024);
@@ -169,7 +181,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     d.part = pb ? pb->as<double>() + 4 * ld * chunks * i : nullptr;
     d.lb = rb->as<double>() + 2 * ld * i;
     d.ub = d.lb + ld;
-    d.pad_ = 0;
+    d.row_waves = row_waves;
   }
   const RangeDesc* table = nullptr;
   BufRef tab;
@@ -181,7 +193,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   double bytes = 0.0;  // algorithmic: V once, the predicate bounds, lb/ub out
   for (auto* t : todo) bytes += 8.0 * (double)t->N * (double)(t->n + 1) + 16.0 * (double)t->n + 16.0 * (double)t->N;
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL(ranges_partial_kernel, grid, dim3(256), 0, ctx->stream, table, descs[0]);
+  hipLaunchKernelGGL(ranges_partial_kernel, grid, dim3(64 * kRangeWaves), 0, ctx->stream, table, descs[0]);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
   if (chunks > 1)
     hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,

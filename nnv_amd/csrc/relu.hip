@@ -9,6 +9,7 @@
 // The dense constraint matrix is never built on this path; materialize_constraints() lays it out
 // exactly as the reference does when the host asks for it.
 #include <algorithm>
+#include <cstdlib>
 
 #include "internal.h"
 
@@ -41,7 +42,7 @@ struct ReluDesc {
   int32_t m;
   int32_t order;
   int32_t cols_per_chunk;
-  int32_t pad_;
+  int32_t row_waves;  // apply pass: waves of a block laid along rows (1, 2, 4 or 8); the rest along columns
 };
 
 // "a sorts before b" under the stable descending key order: larger key first, ties by smaller
@@ -335,7 +336,9 @@ __global__ __launch_bounds__(256) void relu_scatter_kernel(const ReluDesc* __res
 
 constexpr int kApplyRows = 128;  // 64 lanes x 2 rows, the four waves interleave columns
 
-__global__ __launch_bounds__(256) void relu_apply_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+constexpr int kApplyWaves = 8;  // waves per block of the apply pass
+
+__global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
   const ReluDesc d = table ? table[blockIdx.z] : one;
   const int ncols_out = d.ncols_in + d.m;
   const int j0 = blockIdx.y * d.cols_per_chunk;
@@ -343,7 +346,12 @@ __global__ __launch_bounds__(256) void relu_apply_kernel(const ReluDesc* __restr
   const int j1 = min(ncols_out, j0 + d.cols_per_chunk);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t r0 = (int64_t)blockIdx.x * kApplyRows + 2 * lane;
+  // row_waves waves of the block sit next to each other along the rows (contiguous memory of one
+  // column), the others take different columns
+  const int wrow = wave % d.row_waves;
+  const int wcol = wave / d.row_waves;
+  const int col_waves = kApplyWaves / d.row_waves;
+  const int64_t r0 = ((int64_t)blockIdx.x * d.row_waves + wrow) * kApplyRows + 2 * lane;
   const bool active = r0 < d.ld;
   int cx = kKeep, cy = kKeep;
   if (active) {
@@ -352,9 +360,9 @@ __global__ __launch_bounds__(256) void relu_apply_kernel(const ReluDesc* __restr
     cy = c.y;
   }
   const int n_in = d.ncols_in - 1;
-  const bool writer = blockIdx.x == 0 && lane == 0;
+  const bool writer = blockIdx.x == 0 && wrow == 0 && lane == 0;
   // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
-  for (int jb = j0 + 4 * wave; jb < j1; jb += 16) {
+  for (int jb = j0 + 4 * wcol; jb < j1; jb += 4 * col_waves) {
     double2 v[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -484,9 +492,15 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   NNV_TRY(ctx->alloc(sizeof(double) * ld * total_cols, &arena));
   NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
   if (total_lbub > 0) NNV_TRY(ctx->alloc(sizeof(double) * total_lbub, &lbub_buf));
-  // Column chunking of the apply pass: a couple of thousand blocks, at least 32 columns each.
-  const int64_t row_blocks = ceil_div(ld, kApplyRows);
-  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(2048, row_blocks * count), ceil_div(max_cols, 32)));
+  // Column chunking of the apply pass: a couple of thousand blocks, at least two steps per wave.
+  int row_waves = ld >= 8 * kApplyRows ? 8 : ld >= 4 * kApplyRows ? 4 : ld >= 2 * kApplyRows ? 2 : 1;
+  if (const char* e = getenv("NNVHIP_APPLY_ROW_WAVES")) {
+    const int v = atoi(e);
+    row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
+  }
+  const int64_t row_blocks = ceil_div(ld, kApplyRows * row_waves);
+  const int64_t min_cpc = (const int64_t)8 * (kApplyWaves / row_waves);  // two 4-column steps per wave
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(2048, row_blocks * count), ceil_div(max_cols, min_cpc)));
   const int64_t cpc = ceil_div(max_cols, chunks);
   chunks = ceil_div(max_cols, cpc);
   for (int64_t i = 0; i < count; ++i) {
@@ -501,6 +515,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.lbub = m > 0 ? lbub_buf->as<double>() + lbub_off[i] : nullptr;
     d.ld_lbub = ldr;
     d.cols_per_chunk = (int32_t)cpc;
+    d.row_waves = row_waves;
   }
   if (count > 1) {
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
@@ -518,7 +533,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   for (int64_t i = 0; i < count; ++i)
     bytes += 8.0 * (double)N * (double)(in[i]->n + 1) + 8.0 * (double)N * (double)(in[i]->n + 1 + descs[i].m);
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(256), 0,
+  hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(64 * kApplyWaves), 0,
                      ctx->stream, table, descs[0]);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 3, bytes));
   NNV_HIP_TRY(hipGetLastError());
