@@ -173,6 +173,8 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
+  NNV_HIP_TRY(hipHostMalloc((void**)&c->mailbox, 64, hipHostMallocDefault));
+  for (int i = 0; i < 16; ++i) c->mailbox[i] = 0;
   NNV_HIP_TRY(hipEventCreate(&c->kev0));
   NNV_HIP_TRY(hipEventCreate(&c->kev1));
   *out = c;
@@ -186,6 +188,7 @@ int nnvhip_destroy(nnvhip_ctx* c) {
   NNV_HIP_TRY(hipSetDevice(c->device));
   c->trim();
   if (c->pinned) (void)hipHostFree(c->pinned);
+  if (c->mailbox) (void)hipHostFree((void*)c->mailbox);
   (void)hipEventDestroy(c->ev0);
   (void)hipEventDestroy(c->ev1);
   (void)hipEventDestroy(c->kev0);

@@ -97,6 +97,10 @@ struct nnvhip_ctx {
   char* pinned = nullptr;
   size_t pinned_bytes = 0;
   size_t pinned_off = 0;
+  // mailbox in pinned host memory: a kernel posts {m, inactive, sequence number} there and the host
+  // spins on it, which is quicker than a device-to-host copy plus stream synchronisation
+  volatile int32_t* mailbox = nullptr;
+  int32_t mailbox_seq = 0;
   // per-layer timing
   bool timing = false;         // per-layer events (nnvhip_last_op_time_ms)
   bool kernel_timing = false;  // additionally one event pair per launch of the timed kernel groups

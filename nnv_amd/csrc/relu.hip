@@ -9,7 +9,9 @@
 // The dense constraint matrix is never built on this path; materialize_constraints() lays it out
 // exactly as the reference does when the host asks for it.
 #include <algorithm>
+#include <chrono>
 #include <cstdlib>
+#include <cstring>
 
 #include "internal.h"
 
@@ -34,6 +36,9 @@ struct ReluDesc {
   int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
   int32_t* blk_counts; // multi-block classification: per 1024-row block {crossing, inactive}
+  int32_t* mailbox;    // host-pinned {m, inactive, seq}; null = counts are fetched by a copy instead
+  int32_t mailbox_seq;
+  int32_t pad2_;
   double* lbub;        // lb then ub (offset ld_lbub) of the crossing neurons, new-predicate order
   int64_t ld;
   int64_t ld_lbub;
@@ -44,6 +49,16 @@ struct ReluDesc {
   int32_t cols_per_chunk;
   int32_t row_waves;  // apply pass: waves of a block laid along rows (1, 2, 4 or 8); the rest along columns
 };
+
+// Posts the counts to the host mailbox: payload first, system-scope fence, then the sequence number
+// the host is spinning on.
+__device__ __forceinline__ void post_counts(int32_t* mailbox, int m, int inactive, int seq) {
+  if (mailbox == nullptr) return;
+  mailbox[0] = m;
+  mailbox[1] = inactive;
+  __threadfence_system();
+  __hip_atomic_store(&mailbox[2], seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // "a sorts before b" under the stable descending key order: larger key first, ties by smaller
 // neuron index (MATLAB's sort(...,'descend') keeps equal keys in their original, ascending order).
@@ -182,6 +197,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   if (tid == 0) {
     d.counts[0] = m;
     d.counts[1] = inact_total;
+    post_counts(d.mailbox, m, inact_total, d.mailbox_seq);  // the host can size the output while we sort
   }
   if (SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP) {
     __syncthreads();
@@ -291,6 +307,7 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
     if (tid == 0) {
       d.counts[0] = stot;
       d.counts[1] = sinact;
+      post_counts(d.mailbox, stot, sinact, d.mailbox_seq);
     }
   }
 }
@@ -437,10 +454,16 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.rank = sorted ? rank_buf->as<int32_t>() + ld * i : nullptr;
     d.counts = cnt_buf->as<int32_t>() + 2 * i;
     d.blk_counts = blk_buf ? blk_buf->as<int32_t>() + 2 * nblk * i : nullptr;
+    d.mailbox = nullptr;
     d.ld = ld;
     d.N = (int32_t)N;
     d.ncols_in = (int32_t)(in[i]->n + 1);
     d.order = order;
+  }
+  const bool use_mailbox = count == 1 && ctx->mailbox != nullptr;
+  if (use_mailbox) {
+    descs[0].mailbox = const_cast<int32_t*>(ctx->mailbox);
+    descs[0].mailbox_seq = ++ctx->mailbox_seq;
   }
   const ReluDesc* table = nullptr;
   BufRef tab;
@@ -465,12 +488,29 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   }
   NNV_HIP_TRY(hipGetLastError());
 
-  // the column count of the output depends on m: read the counts back
-  void* hc = nullptr;
-  NNV_TRY(ctx->stage(sizeof(int32_t) * 2 * count, &hc));
-  NNV_HIP_TRY(hipMemcpyAsync(hc, cnt_buf->ptr, sizeof(int32_t) * 2 * count, hipMemcpyDeviceToHost, ctx->stream));
-  NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));
-  const std::vector<int32_t> counts(static_cast<const int32_t*>(hc), static_cast<const int32_t*>(hc) + 2 * count);
+  // the column count of the output depends on m: fetch the counts
+  std::vector<int32_t> counts(2 * count);
+  if (use_mailbox) {
+    // one set: the kernel posts the counts to pinned host memory; spin on the sequence number
+    const auto t0 = std::chrono::steady_clock::now();
+    long spins = 0;
+    while (ctx->mailbox[2] != ctx->mailbox_seq) {
+      if ((++spins & 0xfff) == 0 &&
+          std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 10.0) {
+        NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));  // surfaces a launch failure, if any
+        if (ctx->mailbox[2] != ctx->mailbox_seq) NNV_FAIL(NNVHIP_ERR_HIP, "classification kernel did not report its counts");
+      }
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
+    counts[0] = ctx->mailbox[0];
+    counts[1] = ctx->mailbox[1];
+  } else {
+    void* hc = nullptr;
+    NNV_TRY(ctx->stage(sizeof(int32_t) * 2 * count, &hc));
+    NNV_HIP_TRY(hipMemcpyAsync(hc, cnt_buf->ptr, sizeof(int32_t) * 2 * count, hipMemcpyDeviceToHost, ctx->stream));
+    NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    memcpy(counts.data(), hc, sizeof(int32_t) * 2 * count);
+  }
 
   // outputs: one V arena, one predicate-bound buffer, one buffer for the crossing bounds
   int64_t total_cols = 0, total_pred = 0, total_lbub = 0, max_cols = 0, max_m = 0;
