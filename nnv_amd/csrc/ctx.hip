@@ -702,7 +702,16 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
   int st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
   if (st == NNVHIP_OK) {
     const double* bias = fc->bias ? fc->bias->as<double>() : nullptr;
-    if (contig) {
+    if (count == 1) {
+      // one set: the GEMM epilogue also leaves the partial sums of Star.estimateRanges, so the
+      // output set carries its ranges without another pass over V
+      RangeFuse fuse;
+      fuse.plb = outs[0]->plb;
+      fuse.pub = outs[0]->pub;
+      st = launch_gemm(c, fc->W->as<double>(), fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols,
+                       fc->Kp, bias, &fuse);
+      if (st == NNVHIP_OK && fuse.chunks > 0) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks);
+    } else if (contig) {
       st = launch_gemm(c, fc->W->as<double>(), fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols,
                        fc->Kp, bias);
       if (st == NNVHIP_OK && bias && count > 1) {

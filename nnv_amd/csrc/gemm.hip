@@ -21,7 +21,10 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
                                                         double* __restrict__ C, int64_t ldc, int Mp, int64_t ncols,
                                                         int Kp, const double* __restrict__ bias, int tiles_m,
                                                         int tiles_n, int xr, int local_m, int ksplit,
-                                                        double* __restrict__ part) {
+                                                        double* __restrict__ part,
+                                                        const double* __restrict__ plb,
+                                                        const double* __restrict__ pub,
+                                                        double* __restrict__ rpart) {
   constexpr int NT = 64 * WR * WC;  // threads per block
   constexpr int FM = TM / WR / 16;
   constexpr int FN = TN / WC / 16;
@@ -128,9 +131,60 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
     bias = nullptr;
   }
 
-  // ---- epilogue: bias on column 0, 128-byte line stores --------------------------------------
   const int lrow = lane & 15;
   const int lcol = lane >> 4;
+  // ---- fused estimateRanges: partial sums of this column tile ----------------------------------
+  // xmin1 = sum max(v,0)*plb, xmin2 = sum min(v,0)*pub, xmax1 = sum max(v,0)*pub, xmax2 = sum min(v,0)*plb
+  // over the tile's generator columns (column 0, the centre, is skipped), per output row.
+  if (rpart != nullptr) {
+    double* red = &Ws[0][0];  // the K loop is over (last barrier passed): reuse the W stage
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+      double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int64_t col = n0 + wc * (TN / WC) + j * 16 + lcol + 4 * r;
+          if (col >= 1 && col < ncols) {
+            const double v = acc[i][j][r];
+            const double pl = plb[col - 1], pu = pub[col - 1];
+            const double p = fmax(v, 0.0), q = fmin(v, 0.0);
+            s0 = fma(p, pl, s0);
+            s1 = fma(q, pu, s1);
+            s2 = fma(p, pu, s2);
+            s3 = fma(q, pl, s3);
+          }
+        }
+      }
+      // the four lane groups (lcol) hold different columns of the same rows
+      s0 += __shfl_xor(s0, 16);
+      s1 += __shfl_xor(s1, 16);
+      s2 += __shfl_xor(s2, 16);
+      s3 += __shfl_xor(s3, 16);
+      s0 += __shfl_xor(s0, 32);
+      s1 += __shfl_xor(s1, 32);
+      s2 += __shfl_xor(s2, 32);
+      s3 += __shfl_xor(s3, 32);
+      if (lcol == 0) {
+        double* dst = red + ((wc * TM) + wr * (TM / WR) + i * 16 + lrow) * 4;
+        dst[0] = s0;
+        dst[1] = s1;
+        dst[2] = s2;
+        dst[3] = s3;
+      }
+    }
+    __syncthreads();
+    for (int t = tid; t < TM * 4; t += NT) {  // waves along the columns are combined in order
+      const int row = t >> 2, q = t & 3;
+      double s = 0.0;
+#pragma unroll
+      for (int w = 0; w < WC; ++w) s += red[(w * TM + row) * 4 + q];
+      if (m0 + row < Mp) rpart[((int64_t)nt * 4 + q) * ldc + m0 + row] = s;
+    }
+  }
+
+  // ---- epilogue: bias on column 0, 128-byte line stores --------------------------------------
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
     int row = m0 + wr * (TM / WR) + i * 16 + lrow;
@@ -166,7 +220,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __rest
 
 template <int TM, int TN, int WR, int WC, int KT>
 static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
-                      int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias) {
+                      int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse) {
   int64_t tiles_m = ceil_div(Mp, TM);
   int64_t tiles_n = ceil_div(ncols, TN);
   int64_t blocks = tiles_m * tiles_n;
@@ -199,11 +253,18 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
   BufRef ws;
   if (ksplit > 1) NNV_TRY(ctx->alloc(sizeof(double) * ksplit * Mp * ncols, &ws));
+  double* rpart = nullptr;
+  if (fuse != nullptr && ksplit == 1) {  // the epilogue sees final values: fuse the range sums
+    NNV_TRY(ctx->alloc(sizeof(double) * 4 * ldc * tiles_n, &fuse->part));
+    fuse->chunks = tiles_n;
+    rpart = fuse->part->as<double>();
+  }
   const bool timed = ctx->kernel_timing && TM >= 64;
   NNV_TRY(ctx->kernel_timer_begin(timed));
   hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)grid_x, (unsigned)ksplit), dim3(64 * WR * WC), 0,
                      ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)tiles_n,
-                     (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr);
+                     (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
+                     fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, 2.0 * (double)Mp * (double)Kp * (double)ncols));
   if (ksplit > 1) {
     const int64_t total = Mp * ncols;
@@ -215,14 +276,14 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
 }
 
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C, int64_t ldc,
-                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias) {
+                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse) {
   if (Mp % 16 || Kp % 16 || lda % 2 || ldb % 2 || Mp > lda || Kp > ldb || Mp > ldc)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: GEMM operands violate the padding contract");
   if (Mp >= (int64_t(1) << 31) || Kp >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large");
   if (ncols == 0) return NNVHIP_OK;
   // Tile choice: the largest tile that still yields a few blocks per CU; skinny outputs (the last
   // layer has 10 rows) get a 16-row tile.  K must be a multiple of the K-tile (16 or 32).
-#define NNV_GEMM(TM, TN, WR, WC, KT) launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias)
+#define NNV_GEMM(TM, TN, WR, WC, KT) launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias, fuse)
   const int64_t kCUs = 256;
   if (Mp <= 16) return NNV_GEMM(16, 64, 1, 4, 16);
   if (Mp <= 32) return NNV_GEMM(32, 128, 1, 4, 16);

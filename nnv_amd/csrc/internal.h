@@ -169,10 +169,20 @@ namespace nnvhip {
 
 nnvhip_star* new_star(nnvhip_ctx* ctx);
 
+// Optional fusion of Star.estimateRanges into the GEMM epilogue (one set per launch): every column
+// tile leaves the four partial range sums of its rows in `part` ([chunks][4][ldc]); the caller then
+// runs the range reduction over the chunks instead of a separate pass over the output.
+struct RangeFuse {
+  const double* plb = nullptr;  // predicate bounds of the set's n = ncols - 1 generator columns
+  const double* pub = nullptr;
+  BufRef part;                  // out: partial sums (allocated by the launcher)
+  int64_t chunks = 0;           // out: number of column tiles; 0 = not fused (split-K was used)
+};
+
 // gemm.hip: C(Mp x ncols, ldc) = A(Mp x Kp, lda) * B(Kp x ncols, ldb); bias (Mp) is added to
 // column 0 when non-null.  Mp, Kp multiples of 16; padding rows of A and B are zero.
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
-                int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias);
+                int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse = nullptr);
 // Adds bias to the centre columns of sets 1..count-1 of an arena (set 0 is fused in the GEMM).
 int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t count, const double* bias,
                         int64_t Mp);
@@ -184,6 +194,8 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t
 
 // ranges.hip
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s);
+// Turns the per-column-tile partial sums a fused GEMM left behind into the set's cached lb/ub.
+int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks);
 
 // relu.hip
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out);

@@ -113,7 +113,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void ranges_partial_kernel(const 
 // by four different waves so that the dependent add chains are short.
 __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
-  if (d.chunks == 1) return;
+  if (d.chunks == 1 && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
   const int lane = threadIdx.x & 63;
   const int q = threadIdx.x >> 6;
   const int64_t r = (int64_t)blockIdx.x * 64 + lane;
@@ -204,6 +204,30 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     todo[i]->lb = descs[i].lb;
     todo[i]->ub = descs[i].ub;
   }
+  return NNVHIP_OK;
+}
+
+int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks) {
+  if (s->lb || chunks < 1) return NNVHIP_OK;
+  BufRef rb;
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * s->ld, &rb));
+  RangeDesc d{};
+  d.V = s->V;
+  d.plb = s->plb;
+  d.pub = s->pub;
+  d.part = part->as<double>();
+  d.lb = rb->as<double>();
+  d.ub = d.lb + s->ld;
+  d.ld = s->ld;
+  d.n = (int32_t)s->n;
+  d.chunks = (int32_t)chunks;
+  d.cols_per_chunk = 0;
+  d.row_waves = 1;
+  hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(s->ld, 64), 1, 1), dim3(256), 0, ctx->stream, nullptr, d);
+  NNV_HIP_TRY(hipGetLastError());
+  s->rbuf = rb;
+  s->lb = d.lb;
+  s->ub = d.ub;
   return NNVHIP_OK;
 }
 
