@@ -232,7 +232,9 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   for (int64_t xr = 1; xr <= 8; xr *= 2) {
     const int64_t slots = ceil_div(tiles_m, xr) * ceil_div(tiles_n, 8 / xr);
     const double traffic = (8.0 / xr) * (double)Mp * Kp + (double)xr * Kp * (double)ncols;
-    const double cost = (double)slots * (1.0 + 0.03 * traffic / ((double)Mp * Kp + (double)Kp * ncols) / 8.0);
+    // an XCD has 32 CUs: up to 32 tiles per XCD still run in one round, so small imbalances are free
+    const int64_t eff_slots = slots < 128 ? ceil_div(slots, 32) * 32 : slots;
+    const double cost = (double)eff_slots * (1.0 + 0.03 * traffic / ((double)Mp * Kp + (double)Kp * ncols) / 8.0);
     if (best_slots == 0 || cost < best_cost) {
       best_cost = cost;
       best_xr = xr;
