@@ -60,14 +60,13 @@ def main():
                  "that path is not built) - use --gpus 1")
 
     import nnv_amd
-    from nnv_amd.configs import count_updates, make_config
-    from tests.gpu_util import input_sets
+    from nnv_amd.configs import count_updates, device_input_sets, make_config
 
     cfg = make_config(args.config)
     ctx = nnv_amd.default_context()
     net = nnv_amd.NN.from_config(cfg["layers"], cfg["name"])
     opts = {"reachMethod": args.method, "relaxFactor": 1}
-    dev_in, ora_in = input_sets(cfg)
+    dev_in = device_input_sets(cfg, ctx)
     lib, h = ctx.lib, ctx.handle
 
     def step():
@@ -144,10 +143,13 @@ def main():
             for sp, so in zip(prev_sets, outs):
                 N, n, _ = sp._h.dims()
                 m = so._h.dims()[1] - n
-                # masked-copy read of V + write of the N x (n+1+m) output, plus the estimateRanges read
-                # of V unless the producing FC layer already left the range sums (single-set FC)
+                # read of the rows the step keeps + write of the N x (n+1+m) output, plus the
+                # estimateRanges read of V unless the producing FC layer already left the range sums
                 fused = i > 0 and cfg["layers"][i - 1]["type"] == "fc" and len(outs) == 1
-                b += 8.0 * N * (n + 1) * (1 if fused else 2) + 8.0 * N * (n + 1 + m)
+                ni, nc = ctypes.c_int64(), ctypes.c_int64()
+                nnv_amd._lib.check(ctx.lib.nnvhip_star_relu_counts(so._h.h, ctypes.byref(ni), ctypes.byref(nc)))
+                kept = N - ni.value - nc.value
+                b += 8.0 * N * (n + 1) * (0 if fused else 1) + 8.0 * kept * (n + 1) + 8.0 * N * (n + 1 + m)
             entry["algo_GBps"] = round(b / (per_layer[i] * 1e-3) / 1e9, 1)
             relu_bytes += b
             relu_ms += per_layer[i]
@@ -198,6 +200,14 @@ def main():
     cpu = None
     if not args.no_cpu:
         from oracle import nnv_oracle as o
+        if "partition" in cfg:
+            ora_in = [o.star_from_box(l, u) for (l, u) in o.box_partition(
+                cfg["lb"], cfg["ub"], cfg["partition"]["indexes"], cfg["partition"]["numbers"])]
+        elif cfg["kind"] == "image":
+            sh = cfg["image_shape"]
+            ora_in = o.image_star_from_bounds(cfg["lb"].reshape(sh, order="F"), cfg["ub"].reshape(sh, order="F"))
+        else:
+            ora_in = o.star_from_box(cfg["lb"], cfg["ub"])
         n_cpu, t_cpu = 0, 0.0
         while t_cpu < args.cpu_seconds and n_cpu < 50:
             t1 = time.perf_counter()

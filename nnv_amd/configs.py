@@ -120,3 +120,19 @@ def make_config(k: int, shrink: int = 1):
 def count_updates(layer_shapes):
     """Generator-neuron updates of one reach: sum over layer steps of N_out * (n_out + 1)."""
     return int(sum(int(N) * (int(n) + 1) for (N, n) in layer_shapes))
+
+
+def device_input_sets(cfg, ctx=None):
+    """Input set(s) of a config on the device, built as NNV builds them: Star(lb, ub) /
+    ImageStar(lb, ub) (set/Star.m:220-237, set/ImageStar.m:302-343), and for the partitioned
+    config Box.partition (set/Box.m:96-139) followed by one Star per sub-box."""
+    from .sets import Box, ImageStar, Star
+    if "partition" in cfg:
+        boxes = Box(cfg["lb"], cfg["ub"]).partition(cfg["partition"]["indexes"], cfg["partition"]["numbers"])
+        lbs = np.stack([b.lb for b in boxes], axis=1)
+        ubs = np.stack([b.ub for b in boxes], axis=1)
+        return Star.from_boxes(lbs, ubs, ctx=ctx)
+    if cfg["kind"] == "image":
+        sh = cfg["image_shape"]
+        return ImageStar(cfg["lb"].reshape(sh, order="F"), cfg["ub"].reshape(sh, order="F"), ctx=ctx)
+    return Star(cfg["lb"], cfg["ub"], ctx=ctx)

@@ -1,8 +1,8 @@
 // Star.estimateRanges (set/Star.m:1078-1106) as one coalesced pass over V.
 //
 // V is column-major, so consecutive lanes own consecutive rows: every wave reads 1 KiB lines down a
-// column (two rows per lane).  The four waves of a block interleave the columns of the block's
-// column chunk; partial sums of the chunks are combined in a fixed order by a second tiny kernel,
+// column (two rows per lane).  The eight waves of a block interleave the columns of the block's
+// column chunk, eight loads in flight per wave; partial sums of the chunks are combined in a fixed order by a second tiny kernel,
 // so results are bit-reproducible from run to run (no floating-point atomics).
 #include <algorithm>
 #include <cstdlib>
@@ -28,8 +28,9 @@ struct RangeDesc {
 constexpr int kRowsPerWave = 128;  // 64 lanes x 2 rows
 constexpr int kRangeWaves = 8;     // waves per block
 
-__global__ __launch_bounds__(64 * kRangeWaves) void ranges_partial_kernel(const RangeDesc* __restrict__ table,
-                                                                          RangeDesc one) {
+template <int U, int OCC>
+__global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(const RangeDesc* __restrict__ table,
+                                                                               RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
   const int chunk = blockIdx.y;
   if (chunk >= d.chunks) return;
@@ -46,16 +47,17 @@ __global__ __launch_bounds__(64 * kRangeWaves) void ranges_partial_kernel(const 
   double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
   if (active) {
     const double* col = d.V + r0;
-    // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
-    for (int jb = j0 + 4 * wcol; jb < j1; jb += 4 * col_waves) {
-      double2 v[4];
+    // each wave takes U consecutive columns per step; the U loads are issued before any is used
+#pragma unroll 1
+    for (int jb = j0 + U * wcol; jb < j1; jb += U * col_waves) {
+      double2 v[U];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < U; ++u) {
         v[u] = make_double2(0.0, 0.0);
         if (jb + u < j1) v[u] = *reinterpret_cast<const double2*>(col + (int64_t)(jb + u) * d.ld);
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < U; ++u) {
         const int j = jb + u;
         if (j >= j1) break;
         const double pl = d.plb[j - 1];
@@ -159,7 +161,8 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
   }
   const int64_t row_blocks = ceil_div(ld, kRowsPerWave * row_waves);
-  const int64_t want_blocks = 2048;
+  int64_t want_blocks = 2048;
+  if (const char* e = getenv("NNVHIP_RANGES_BLOCKS")) want_blocks = std::max(1, atoi(e));
   int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * nset), ceil_div(nmax, 64)));
   chunks = std::min<int64_t>(chunks, 1024);
   // one buffer for all lb/ub, one for all partials
@@ -193,7 +196,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   double bytes = 0.0;  // algorithmic: V once, the predicate bounds, lb/ub out
   for (auto* t : todo) bytes += 8.0 * (double)t->N * (double)(t->n + 1) + 16.0 * (double)t->n + 16.0 * (double)t->N;
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL(ranges_partial_kernel, grid, dim3(64 * kRangeWaves), 0, ctx->stream, table, descs[0]);
+  hipLaunchKernelGGL((ranges_partial_kernel<8, 4>), grid, dim3(64 * kRangeWaves), 0, ctx->stream, table, descs[0]);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
   if (chunks > 1)
     hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,

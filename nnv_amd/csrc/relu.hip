@@ -376,8 +376,30 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
     cx = c.x;
     cy = c.y;
   }
+  // rows that are zeroed anyway are not read: lines whose 16 rows are all inactive or crossing never
+  // leave HBM
+  const bool need = active && (cx == kKeep || cy == kKeep);
   const int n_in = d.ncols_in - 1;
-  const bool writer = blockIdx.x == 0 && wrow == 0 && lane == 0;
+  // predicate bounds and the (lb, ub) of the crossing neurons: one thread per column of this block's
+  // chunk, done by the first row block only
+  if (blockIdx.x == 0) {
+    for (int j = j0 + (int)threadIdx.x; j < j1; j += 64 * kApplyWaves) {
+      if (j < d.ncols_in) {
+        if (j >= 1) {
+          d.plb_out[j - 1] = d.plb_in[j - 1];
+          d.pub_out[j - 1] = d.pub_in[j - 1];
+        }
+      } else {
+        const int i = j - d.ncols_in;
+        const int neuron = d.cross_idx[i];
+        const double ub = d.ub[neuron];
+        d.plb_out[n_in + i] = 0.0;  // new_pred_lb = [plb; zeros(m,1)]
+        d.pub_out[n_in + i] = ub;   // new_pred_ub = [pub; ub]
+        d.lbub[i] = d.lb[neuron];
+        d.lbub[d.ld_lbub + i] = ub;
+      }
+    }
+  }
   // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
   for (int jb = j0 + 4 * wcol; jb < j1; jb += 4 * col_waves) {
     double2 v[4];
@@ -385,8 +407,9 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
     for (int u = 0; u < 4; ++u) {
       const int j = jb + u;
       v[u] = make_double2(0.0, 0.0);
-      if (active && j < j1 && j < d.ncols_in) v[u] = *reinterpret_cast<const double2*>(d.Vin + r0 + (int64_t)j * d.ld);
+      if (need && j < j1 && j < d.ncols_in) v[u] = *reinterpret_cast<const double2*>(d.Vin + r0 + (int64_t)j * d.ld);
     }
+    if (!active) continue;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = jb + u;
@@ -395,24 +418,12 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
       if (j < d.ncols_in) {
         o.x = cx == kKeep ? v[u].x : 0.0;  // V1(map,:) = 0
         o.y = cy == kKeep ? v[u].y : 0.0;
-        if (writer && j >= 1) {
-          d.plb_out[j - 1] = d.plb_in[j - 1];
-          d.pub_out[j - 1] = d.pub_in[j - 1];
-        }
       } else {
-        const int i = j - d.ncols_in;
-        const int neuron = d.cross_idx[i];
+        const int neuron = d.cross_idx[j - d.ncols_in];
         o.x = r0 == neuron ? 1.0 : 0.0;  // V2(index(i), i) = 1
         o.y = r0 + 1 == neuron ? 1.0 : 0.0;
-        if (writer) {
-          const double ub = d.ub[neuron];
-          d.plb_out[n_in + i] = 0.0;  // new_pred_lb = [plb; zeros(m,1)]
-          d.pub_out[n_in + i] = ub;   // new_pred_ub = [pub; ub]
-          d.lbub[i] = d.lb[neuron];
-          d.lbub[d.ld_lbub + i] = ub;
-        }
       }
-      if (active) *reinterpret_cast<double2*>(d.Vout + r0 + (int64_t)j * d.ld) = o;
+      *reinterpret_cast<double2*>(d.Vout + r0 + (int64_t)j * d.ld) = o;
     }
   }
 }
@@ -540,7 +551,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   }
   const int64_t row_blocks = ceil_div(ld, kApplyRows * row_waves);
   const int64_t min_cpc = (const int64_t)8 * (kApplyWaves / row_waves);  // two 4-column steps per wave
-  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(2048, row_blocks * count), ceil_div(max_cols, min_cpc)));
+  int64_t want_blocks = 8192;
+  if (const char* e = getenv("NNVHIP_APPLY_BLOCKS")) want_blocks = std::max(1, atoi(e));
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * count), ceil_div(max_cols, min_cpc)));
   const int64_t cpc = ceil_div(max_cols, chunks);
   chunks = ceil_div(max_cols, cpc);
   for (int64_t i = 0; i < count; ++i) {
@@ -569,9 +582,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
     hipLaunchKernelGGL(relu_scatter_kernel, dim3(t, 1, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
   }
-  double bytes = 0.0;  // algorithmic: read N x (n+1), write N x (n+1+m)
-  for (int64_t i = 0; i < count; ++i)
-    bytes += 8.0 * (double)N * (double)(in[i]->n + 1) + 8.0 * (double)N * (double)(in[i]->n + 1 + descs[i].m);
+  double bytes = 0.0;  // algorithmic: read the rows that are kept, write N x (n+1+m)
+  for (int64_t i = 0; i < count; ++i) {
+    const double kept = (double)(N - counts[2 * i] - counts[2 * i + 1]);
+    bytes += 8.0 * kept * (double)(in[i]->n + 1) + 8.0 * (double)N * (double)(in[i]->n + 1 + descs[i].m);
+  }
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(64 * kApplyWaves), 0,
                      ctx->stream, table, descs[0]);
