@@ -122,6 +122,22 @@ def test_config5_full_batched_equals_single(nnv):
         l1, u1 = one.estimateRanges()
         assert_close(l1, lb[:, i], "set %d lb" % i)
         assert_close(u1, ub[:, i], "set %d ub" % i)
+    # full-size oracle parity of two slots of the batched pass: classification and new-predicate
+    # order bit-exact at every ReLU, generators and per-set output bounds within RTOL
+    for i in (3, 900):
+        ora_out, ora_sets = o.nn_reach(cfg["layers"], o.star_from_box(*boxes[i]), "relax-star-area", 1.0, keep=True)
+        prev = o.star_from_box(*boxes[i])
+        for li, L in enumerate(cfg["layers"]):
+            if L["type"] == "relu":
+                plb, pub = o.estimate_ranges(prev)
+                m1, m2 = o.relax_classify(plb, pub, "relax-star-area")
+                ni, idx, _, _ = net.reachSet[li][i].relu_info()
+                assert ni == m1.size and np.array_equal(idx, m2), "set %d layer %d vs oracle" % (i, li + 1)
+            prev = ora_sets[li]
+        assert_close(outs[i].V, ora_out.V, "set %d output V vs oracle" % i)
+        ol, ou = o.estimate_ranges(ora_out)
+        assert_close(lb[:, i], ol, "set %d lb vs oracle" % i)
+        assert_close(ub[:, i], ou, "set %d ub vs oracle" % i)
     # concrete corner of sub-box 517 lands inside its bounds
     l517, u517 = boxes[517]
     y = o.evaluate(cfg["layers"], u517)
