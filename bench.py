@@ -192,6 +192,24 @@ def main():
         roofline["relu_step_algo_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
         roofline["relu_step_frac_of_hbm_peak"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
 
+    # ---- specification check on the resident output sets (not part of `value`) -----------------
+    spec = None
+    last = net.Layers[-1]
+    if hasattr(last, "Bias") and len(last.Bias) > 1:
+        from nnv_amd import verify
+        out_sets = net.reachSet[-1]
+        hs = net.robustness_set(0, "max")
+        verify.halfspace_check(out_sets, hs)
+        ctx.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(10):
+            verdict, _, _ = verify.halfspace_check(out_sets, hs)
+        ctx.synchronize()
+        spec = {"ms": round((time.perf_counter() - t1) / 10 * 1e3, 4), "sets": int(verdict.shape[0]),
+                "halfspaces": int(verdict.shape[1]),
+                "decided_without_lp": int(np.sum(verdict != verify.HS_UNDECIDED)), "pairs": int(verdict.size),
+                "what": "LP-free pass of verify_specification for robustness_set(target=0): G*[c V], row bounds, verdicts"}
+
     # practical HBM ceiling on this box: a plain copy kernel over 1 GiB (read + write bytes)
     roofline["measured_copy_GBps"] = round(ctx.probe_copy_bandwidth(1 << 30, 5), 1)
     ctx.trim_pool()
@@ -228,7 +246,7 @@ def main():
                    "sets": len(dev_in) if isinstance(dev_in, list) else 1,
                    "updates_per_step": updates,
                    "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, list) else None},
-        "roofline": roofline, "cpu_baseline": cpu, "layers": layer_report,
+        "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec, "layers": layer_report,
     }))
 
 

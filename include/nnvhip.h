@@ -166,6 +166,30 @@ NNVHIP_API int nnvhip_affine_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, 
 NNVHIP_API int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor, int64_t count,
                       nnvhip_star* const* in, nnvhip_star** out);
 
+/* ---- specification check, utils/verify_specification.m:36-80 ----------------------------- */
+/* verify_specification intersects every output set with every half-space {x | G x <= g} of the
+ * unsafe region (Star.intersectHalfSpace, set/Star.m:555-589) and asks whether the result is empty
+ * (Star.isEmptySet, set/Star.m:1216-1232, one LP over the dense C, d).  This call answers most of
+ * those questions without C: for each set and each half-space it maps the set through G
+ * (Y = G*[c V], the C1/d1 rows of set/Star.m:577-578) and bounds every row of Y over the predicate
+ * box exactly as Star.estimateRanges does (set/Star.m:1078-1106).
+ *   some row has lo > g          -> NNVHIP_HS_DISJOINT: the LP is infeasible, the intersection is empty
+ *   every row has hi <= g        -> NNVHIP_HS_INSIDE: the whole set satisfies the half-space, so the
+ *                                   intersection is the set itself
+ *   otherwise                    -> NNVHIP_HS_UNDECIDED: only the LP over (C, d) can tell; the host
+ *                                   builds it from nnvhip_star_fetch_constraints + nnvhip_halfspace_rows
+ * The half-spaces are stacked: half-space h owns rows [row_ptr[h], row_ptr[h+1]) of G (R x N,
+ * column-major, R = row_ptr[n_hs]) and of g.  Outputs (host, any may be NULL): verdict is
+ * count x n_hs (set index fastest), lo and hi are R x count. */
+enum { NNVHIP_HS_DISJOINT = 1, NNVHIP_HS_UNDECIDED = 2, NNVHIP_HS_INSIDE = 3 };
+NNVHIP_API int nnvhip_halfspace_check(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, int64_t n_hs,
+                           const int64_t* row_ptr, const double* G, const double* g, int64_t N,
+                           int32_t* verdict, double* lo, double* hi);
+/* The rows Star.intersectHalfSpace appends for one set (set/Star.m:577-581):
+ * C1 = G*V(:,2:n+1) (R x n, column-major) and d1 = g - G*V(:,1). */
+NNVHIP_API int nnvhip_halfspace_rows(nnvhip_ctx* ctx, nnvhip_star* s, int64_t R, const double* G, const double* g,
+                          int64_t N, double* C1, double* d1);
+
 #ifdef __cplusplus
 }
 #endif

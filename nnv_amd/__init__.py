@@ -7,3 +7,4 @@ from ._lib import Context, NNVHipError, NNVHipOutOfMemory, default_context  # no
 from .layers import Conv2DLayer, FullyConnectedLayer, PosLin, ReluLayer  # noqa: F401
 from .nn import NN  # noqa: F401
 from .sets import Box, ImageStar, Star  # noqa: F401
+from .verify import HalfSpace, verify_specification  # noqa: F401

@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "libnnvhip.so")
 
 OK, ERR_SHAPE, ERR_METHOD, ERR_RELAX_FACTOR, ERR_OOM, ERR_HIP, ERR_ARG = range(7)
 ORDER_INDEX, ORDER_AREA, ORDER_RANGE = 0, 1, 2
+HS_DISJOINT, HS_UNDECIDED, HS_INSIDE = 1, 2, 3
 
 # every entry point declared in include/nnvhip.h
 SYMBOLS = [
@@ -22,7 +23,7 @@ SYMBOLS = [
     "nnvhip_star_relu_counts", "nnvhip_star_fetch_crossing", "nnvhip_estimate_ranges",
     "nnvhip_estimate_ranges_batch", "nnvhip_fc_create", "nnvhip_fc_destroy", "nnvhip_conv2d_create",
     "nnvhip_conv2d_destroy", "nnvhip_conv2d_output_size", "nnvhip_affine_fc", "nnvhip_affine_conv2d",
-    "nnvhip_relu_relax",
+    "nnvhip_relu_relax", "nnvhip_halfspace_check", "nnvhip_halfspace_rows",
 ]
 
 
@@ -79,6 +80,8 @@ def load():
         "nnvhip_affine_fc": [p, p, i64, pp, pp],
         "nnvhip_affine_conv2d": [p, p, i64, i64, i64, pp, pp],
         "nnvhip_relu_relax": [p, C.c_int, dbl, i64, pp, pp],
+        "nnvhip_halfspace_check": [p, i64, pp, i64, p, p, p, i64, p, p, p],
+        "nnvhip_halfspace_rows": [p, p, i64, p, p, i64, p, p],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)

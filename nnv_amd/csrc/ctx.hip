@@ -539,9 +539,28 @@ int nnvhip_estimate_ranges_batch(nnvhip_ctx* c, int64_t count, nnvhip_star* cons
   NNV_TRY(c->end_op());
   if (lb || ub) {
     int64_t N = s[0]->N;
-    for (int64_t i = 0; i < count; ++i) {
-      if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb + i * N, s[i]->lb, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
-      if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub + i * N, s[i]->ub, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
+    // ranges computed by one call sit at a fixed stride in one buffer
+    const int64_t stride = count > 1 ? s[1]->lb - s[0]->lb : 0;
+    bool regular = count > 1 && stride >= N;
+    for (int64_t i = 1; i < count && regular; ++i)
+      regular = s[i]->rbuf == s[0]->rbuf && s[i]->lb == s[0]->lb + i * stride && s[i]->ub == s[0]->ub + i * stride;
+    if (regular && stride <= 4 * N + 64) {
+      // one contiguous copy of the whole range buffer, unpacked on the host (strided 2-D copies of
+      // short rows are issued row by row by the runtime)
+      const int64_t off_ub = s[0]->ub - s[0]->lb;
+      std::vector<double> tmp((size_t)(stride * (count - 1) + std::max<int64_t>(N, off_ub + N)));
+      NNV_HIP_TRY(hipMemcpyAsync(tmp.data(), s[0]->lb, sizeof(double) * tmp.size(), hipMemcpyDeviceToHost, c->stream));
+      NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+      for (int64_t i = 0; i < count; ++i) {
+        if (lb) std::copy(tmp.begin() + i * stride, tmp.begin() + i * stride + N, lb + i * N);
+        if (ub) std::copy(tmp.begin() + i * stride + off_ub, tmp.begin() + i * stride + off_ub + N, ub + i * N);
+      }
+      return NNVHIP_OK;
+    } else {
+      for (int64_t i = 0; i < count; ++i) {
+        if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb + i * N, s[i]->lb, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
+        if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub + i * N, s[i]->ub, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
+      }
     }
     NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   }

@@ -198,6 +198,41 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
     std::vector<nnvhip_star*> in = handles_of(prhs[3]), out(in.size());
     check(nnvhip_relu_relax(ctx(), (int)mxGetScalar(prhs[1]), mxGetScalar(prhs[2]), (int64_t)in.size(), in.data(), out.data()));
     plhs[0] = to_mx(out);
+  } else if (cmd == "halfspace_check") {  // (handles, G (R x dim), g (R x 1), rows_per_halfspace) -> [verdict (count x n_hs), lo, hi]
+    // LP-free part of utils/verify_specification.m:36-80; 1 = disjoint, 2 = undecided (LP), 3 = inside
+    need(nrhs, 4, "halfspace_check");
+    std::vector<nnvhip_star*> in = handles_of(prhs[1]);
+    const mwSize R = mxGetM(prhs[2]), N = mxGetN(prhs[2]);
+    if (mxGetNumberOfElements(prhs[3]) != R)
+      mexErrMsgIdAndTxt("nnvhip:error", "Inconsistent dimension between Halfspace matrix and halfspace vector");
+    const mwSize n_hs = mxGetNumberOfElements(prhs[4]);
+    const double* rows = dbl(prhs[4], "rows_per_halfspace");
+    std::vector<int64_t> row_ptr(n_hs + 1, 0);
+    for (mwSize h = 0; h < n_hs; ++h) row_ptr[h + 1] = row_ptr[h] + (int64_t)rows[h];
+    if (row_ptr[n_hs] != (int64_t)R)
+      mexErrMsgIdAndTxt("nnvhip:error", "Inconsistent dimension between Halfspace matrix and halfspace vector");
+    std::vector<int32_t> verdict(in.size() * n_hs);
+    mxArray* lo = mxCreateDoubleMatrix(R, in.size(), mxREAL);
+    mxArray* hi = mxCreateDoubleMatrix(R, in.size(), mxREAL);
+    check(nnvhip_halfspace_check(ctx(), (int64_t)in.size(), in.data(), (int64_t)n_hs, row_ptr.data(), dbl(prhs[2], "G"),
+                                 dbl(prhs[3], "g"), (int64_t)N, verdict.data(), mxGetDoubles(lo), mxGetDoubles(hi)));
+    plhs[0] = mxCreateDoubleMatrix(in.size(), n_hs, mxREAL);
+    for (size_t i = 0; i < verdict.size(); ++i) mxGetDoubles(plhs[0])[i] = (double)verdict[i];
+    if (nlhs > 1) plhs[1] = lo; else mxDestroyArray(lo);
+    if (nlhs > 2) plhs[2] = hi; else mxDestroyArray(hi);
+  } else if (cmd == "halfspace_rows") {  // (handle, G, g) -> [C1, d1]      Star.intersectHalfSpace, set/Star.m:577-578
+    need(nrhs, 3, "halfspace_rows");
+    nnvhip_star* s = handle_of<nnvhip_star>(prhs[1]);
+    int64_t N, n, p;
+    check(nnvhip_star_dims(s, &N, &n, &p));
+    const mwSize R = mxGetM(prhs[2]);
+    if (mxGetNumberOfElements(prhs[3]) != R)
+      mexErrMsgIdAndTxt("nnvhip:error", "Inconsistent dimension between Halfspace matrix and halfspace vector");
+    plhs[0] = mxCreateDoubleMatrix(R, (mwSize)n, mxREAL);
+    mxArray* d1 = mxCreateDoubleMatrix(R, 1, mxREAL);
+    check(nnvhip_halfspace_rows(ctx(), s, (int64_t)R, dbl(prhs[2], "G"), dbl(prhs[3], "g"), (int64_t)mxGetN(prhs[2]),
+                                mxGetDoubles(plhs[0]), mxGetDoubles(d1)));
+    if (nlhs > 1) plhs[1] = d1; else mxDestroyArray(d1);
   } else if (cmd == "sync") {
     check(nnvhip_synchronize(ctx()));
   } else if (cmd == "set_timing") {

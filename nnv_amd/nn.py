@@ -3,8 +3,11 @@ from __future__ import annotations
 
 import time
 
+import numpy as np
+
 from .layers import Conv2DLayer, FullyConnectedLayer, ReluLayer
 from .sets import ImageStar, Star
+from .verify import HalfSpace, verify_specification
 
 
 class NN:
@@ -90,3 +93,36 @@ class NN:
             self.reachTime[i] = time.perf_counter() - t0
             self.reachSet[i] = rs
         return rs
+
+    # ---- robustness check (the consumer of the reach set) ---------------------------------
+    def robustness_set(self, target, class_type="max"):
+        """NN.robustness_set, nn/NN.m:1334-1368 (target is 0-based): one single-row HalfSpace per
+        other class, the unsafe region "some other class scores at least as high"."""
+        layer = self.Layers[-1]
+        if not isinstance(layer, FullyConnectedLayer):
+            raise ValueError("Output size is set to 0, but it must be >= 1")
+        outSize = len(layer.Bias)
+        if target >= outSize:
+            raise ValueError("Target idx must be less than or equal to the output size of the NN.")
+        G = np.delete(np.eye(outSize), target, axis=0)
+        if class_type == "max":
+            G = -G
+            G[:, target] = 1.0
+        elif class_type == "min":
+            G[:, target] = -1.0
+        return [HalfSpace(G[i:i + 1, :], [0.0]) for i in range(G.shape[0])]
+
+    def checkRobust(self, outputSet, target):
+        """NN.checkRobust, nn/NN.m:608-636: 1 robust, 2 unknown."""
+        if not isinstance(target, (HalfSpace, list, tuple)):
+            if isinstance(target, (int, np.integer)) or getattr(target, "ndim", 1) == 0:
+                target = self.robustness_set(int(target), "max")
+            else:
+                raise ValueError("Target must be a HalfSpace (unsafe/not robust region) or as a scalar determining the output label target.")
+        return verify_specification(outputSet, target)
+
+    def verify_robustness(self, inputSet, reachOptions, target):
+        """NN.verify_robustness, nn/NN.m:639-655.  The relax-star methods over-approximate, so an
+        "unknown" (2) is never promoted to "not robust" (0)."""
+        R = self.reach(inputSet, reachOptions)
+        return self.checkRobust(R, target)

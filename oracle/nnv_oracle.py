@@ -33,6 +33,15 @@ Parity pinning (what checks each function; see tests/test_oracle_*.py)
   hand-computed scalar triangle, brute-force corner enumeration, the containment
   (soundness) invariant the reference's own soundness tests use, structural invariants
   and permutation-equivalence of the six variants.
+* halfspace_contains / is_empty_set / intersect_half_space: the reference's known answers
+  (tests/set/halfspace/test_half_space_contain.m, tests/set/star/test_star_isEmptySet.m:17-23,
+  tests/soundness/test_set_conversion.m:60-68) and closed forms on boxes.  The LP itself is
+  MATLAB's linprog in the reference and scipy's HiGHS here: feasibility verdicts agree except
+  within solver tolerance of the boundary.
+* robustness_set / verify_specification: no reference test holds a value for them (the
+  regression tests only check that the methods exist): PARITY UNPINNED by vectors; pinned by
+  the source text, hand-built cases and the point-wise meaning of the verdict (a sampled
+  output inside the unsafe region forces "unknown").
 """
 from __future__ import annotations
 
@@ -569,3 +578,115 @@ def evaluate(layers, x):
         elif L["type"] == "relu":
             x = np.maximum(x, 0)
     return x
+
+
+# --------------------------------------------------------------------------------------
+# specification check (the consumer of the reach set)
+# --------------------------------------------------------------------------------------
+class OHalfSpace:
+    """HalfSpace {x | G x <= g}, set/HalfSpace.m:1-33."""
+
+    def __init__(self, G, g):
+        G = np.asarray(G, dtype=np.float64)
+        if G.ndim == 1:
+            G = G.reshape(1, -1)
+        g = np.asarray(g, dtype=np.float64)
+        if g.ndim == 2 and g.shape[1] != 1:
+            raise ValueError("Half-space vector should have one column")
+        g = g.reshape(-1)
+        if G.shape[0] != g.shape[0]:
+            raise ValueError("Inconsistent dimension between half-space matrix and half-space vector")
+        self.G = G
+        self.g = g
+        self.dim = G.shape[1]
+
+
+def halfspace_contains(H: OHalfSpace, x) -> bool:
+    """HalfSpace.contains, set/HalfSpace.m:36-57: no entry of g - G*x is negative."""
+    x = np.asarray(x, dtype=np.float64).reshape(-1)
+    if x.size != H.dim:
+        raise ValueError("Inconsistent dimension between the vector x and the half-space object")
+    return not np.any(H.g - H.G @ x < 0)
+
+
+def is_empty_set(S: OStar) -> bool:
+    """Star.isEmptySet, set/Star.m:1216-1232: feasibility LP with a zero objective over
+    C*a <= d, predicate_lb <= a <= predicate_ub (utils/lpsolver.m; its box-only shortcut
+    :36-50 is restated first).  MATLAB's linprog is replaced by scipy's HiGHS."""
+    from scipy.optimize import linprog
+    n = S.nVar
+    lb = S.predicate_lb if S.predicate_lb is not None and np.size(S.predicate_lb) else None
+    ub = S.predicate_ub if S.predicate_ub is not None and np.size(S.predicate_ub) else None
+    A, b = S.C, S.d
+    if (A.size == 0 or not np.any(A)) and lb is not None and ub is not None \
+            and np.all(np.isfinite(lb)) and np.all(np.isfinite(ub)) and (b.size == 0 or np.all(b >= 0)):
+        return False  # lpsolver.m:36-50: closed-form optimum over the box, exit flag "l1"
+    bounds = [(None if lb is None else lb[i], None if ub is None else ub[i]) for i in range(n)]
+    res = linprog(np.zeros(n), A_ub=A if A.size else None, b_ub=b if A.size else None, bounds=bounds, method="highs")
+    if res.status == 0:
+        return False
+    if res.status == 2:
+        return True
+    raise RuntimeError("LP solver error, status %d: %s" % (res.status, res.message))
+
+
+def intersect_half_space(S: OStar, H, g):
+    """Star.intersectHalfSpace, set/Star.m:555-589: appends C1 = H*V(:,2:end),
+    d1 = g - H*V(:,1); returns None when the result is empty."""
+    H = np.asarray(H, dtype=np.float64)
+    if H.ndim == 1:
+        H = H.reshape(1, -1)
+    g = np.asarray(g, dtype=np.float64)
+    if g.ndim == 2 and g.shape[1] != 1:
+        raise ValueError("Halfspace vector should have one column")
+    g = g.reshape(-1)
+    if H.shape[0] != g.shape[0]:
+        raise ValueError("Inconsistent dimension between Halfspace matrix and halfspace vector")
+    if H.shape[1] != S.dim:
+        raise ValueError("Inconsistent dimension between halfspace and star set")
+    C1 = H @ S.V[:, 1:]
+    d1 = g - H @ S.V[:, 0]
+    out = OStar(S.V, np.vstack([S.C, C1]), np.concatenate([S.d, d1]), S.predicate_lb, S.predicate_ub)
+    return None if is_empty_set(out) else out
+
+
+def verify_specification(reach_set, halfspaces) -> int:
+    """utils/verify_specification.m:36-80.  reach_set: a set or a list of sets; halfspaces: one
+    OHalfSpace or a list (an OR of unsafe regions).  1 = no set meets any half-space (property
+    holds), 2 = some intersection is non-empty (unknown for an over-approximation)."""
+    R = reach_set if isinstance(reach_set, (list, tuple)) else [reach_set]
+    prop = halfspaces if isinstance(halfspaces, (list, tuple)) else [halfspaces]
+    result = 1
+    for H in prop:
+        for S in R:
+            if isinstance(S, OImageStar):
+                S = S.to_star()
+            if intersect_half_space(S, H.G, H.g) is not None:
+                return 2
+    return result
+
+
+def robustness_set(out_size: int, target: int, class_type: str = "max"):
+    """NN.robustness_set, nn/NN.m:1334-1368 (target is 0-based here): one single-row half-space
+    per other class; for 'max' the row is x_target - x_j <= 0 written as [-e_j + e_target]."""
+    if target >= out_size:
+        raise ValueError("Target idx must be less than or equal to the output size of the NN.")
+    G = np.eye(out_size)
+    G = np.delete(G, target, axis=0)
+    if class_type == "max":
+        G = -G
+        G[:, target] = 1.0
+    elif class_type == "min":
+        G[:, target] = -1.0
+    return [OHalfSpace(G[i:i + 1, :], np.zeros(1)) for i in range(G.shape[0])]
+
+
+def verify_robustness(layers, input_set, reach_method, target, relax_factor=1.0) -> int:
+    """NN.verify_robustness -> checkRobust, nn/NN.m:590-640: reach, then the specification check
+    against robustness_set(target, 'max') (or the given half-spaces).  An over-approximate method
+    never turns 2 into 0."""
+    out = nn_reach(layers, input_set, reach_method, relax_factor)
+    if isinstance(target, (int, np.integer)):
+        layer = [L for L in layers if L["type"] == "fc"][-1]
+        target = robustness_set(layer["W"].shape[0], int(target), "max")
+    return verify_specification(out, target)
