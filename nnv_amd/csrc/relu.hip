@@ -135,6 +135,97 @@ __device__ __forceinline__ void bitonic_sort_desc(double* skey, int* sidx, int m
   }
 }
 
+// ---- sorting network for lists of at most 1024 entries, one entry per thread -------------------
+// Keys are non-negative doubles, so their bit patterns order like signed 64-bit integers; the
+// sentinel (minimum integer) sorts after every real entry.  The network is the "flip" form of the
+// bitonic sort: for k = 2, 4, ..., P every block of k entries first exchanges i <-> i ^ (k-1), then
+// i <-> i ^ j for j = k/4, ..., 1, always leaving the entry that sorts first in the lower slot.
+// All exchange distances are compile-time constants, so distances inside a row of 16 lanes use DPP
+// moves, distances inside 32 lanes ds_swizzle, 32..63 ds_bpermute, and only the 10 widest of the 55
+// stages go through LDS with block barriers.
+template <int MASK>
+__device__ __forceinline__ int lane_xor(int v) {
+  static_assert(MASK >= 1 && MASK < 64, "exchange inside one wave");
+  if constexpr (MASK == 1) {
+    return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+  } else if constexpr (MASK == 2) {
+    return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+  } else if constexpr (MASK == 3) {
+    return __builtin_amdgcn_update_dpp(v, v, 0x1B, 0xF, 0xF, false);  // quad_perm [3,2,1,0]
+  } else if constexpr (MASK == 7) {
+    return __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false);  // row_half_mirror
+  } else if constexpr (MASK == 15) {
+    return __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false);  // row_mirror
+  } else if constexpr (MASK == 8) {
+    return __builtin_amdgcn_update_dpp(v, v, 0x128, 0xF, 0xF, false);  // row_ror:8
+  } else if constexpr (MASK == 4) {
+    // banks 0 and 2 (lanes 0-3, 8-11 of a row) read lane+4, banks 1 and 3 read lane-4
+    const int r = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xF, 0x5, false);  // row_shl:4
+    return __builtin_amdgcn_update_dpp(r, v, 0x114, 0xF, 0xA, false);         // row_shr:4
+  } else if constexpr (MASK < 32) {
+    return __builtin_amdgcn_ds_swizzle(v, 0x1F | (MASK << 10));  // bit-mask mode: lane ^ MASK within 32
+  } else {
+    return __shfl_xor(v, MASK);
+  }
+}
+
+// One compare-exchange stage: partner = tid ^ MASK; the slot whose LOWBIT bit of tid is clear keeps
+// the entry that sorts first (larger key; equal keys: smaller neuron index).
+template <int MASK, int LOWBIT>
+__device__ __forceinline__ void sort_stage(long long& key, int& idx, long long* skey, int* sidx, int tid) {
+  long long pk;
+  int pi;
+  if constexpr (MASK >= 64) {
+    __syncthreads();
+    skey[tid] = key;
+    sidx[tid] = idx;
+    __syncthreads();
+    pk = skey[tid ^ MASK];
+    pi = sidx[tid ^ MASK];
+  } else {
+    const int lo = lane_xor<MASK>((int)(unsigned)(key & 0xffffffffll));
+    const int hi = lane_xor<MASK>((int)(key >> 32));
+    pk = ((long long)hi << 32) | (unsigned)lo;
+    pi = lane_xor<MASK>(idx);
+  }
+  const bool mine_first = key > pk || (key == pk && idx < pi);
+  const bool lower = (tid & LOWBIT) == 0;
+  if (mine_first != lower) {
+    key = pk;
+    idx = pi;
+  }
+}
+
+template <int K, int J>
+__device__ __forceinline__ void sort_steps(long long& key, int& idx, long long* skey, int* sidx, int tid) {
+  if constexpr (J >= 1) {
+    sort_stage<J, J>(key, idx, skey, sidx, tid);
+    sort_steps<K, J / 2>(key, idx, skey, sidx, tid);
+  }
+}
+
+template <int P, int K>
+__device__ __forceinline__ void sort_merges(long long& key, int& idx, long long* skey, int* sidx, int tid) {
+  if constexpr (K <= P) {
+    sort_stage<K - 1, K / 2>(key, idx, skey, sidx, tid);  // flip: i <-> i ^ (k-1)
+    sort_steps<K, K / 4>(key, idx, skey, sidx, tid);
+    sort_merges<P, 2 * K>(key, idx, skey, sidx, tid);
+  }
+}
+
+// Sorts m <= 1024 (key bits, neuron) pairs staged in skey/sidx[0..m) and writes the neuron indices
+// in sorted order to out[0..m).  All 1024 threads of the block must call it.
+__device__ __forceinline__ void sort_small_desc(long long* skey, int* sidx, int m, int tid, int32_t* __restrict__ out) {
+  long long key = tid < m ? skey[tid] : (long long)0x8000000000000000ull;
+  int idx = tid < m ? sidx[tid] : 0x7fffffff;
+  if (m <= 64) sort_merges<64, 2>(key, idx, skey, sidx, tid);
+  else if (m <= 128) sort_merges<128, 2>(key, idx, skey, sidx, tid);
+  else if (m <= 256) sort_merges<256, 2>(key, idx, skey, sidx, tid);
+  else if (m <= 512) sort_merges<512, 2>(key, idx, skey, sidx, tid);
+  else sort_merges<1024, 2>(key, idx, skey, sidx, tid);
+  if (tid < m) out[tid] = idx;
+}
+
 // One 1024-thread block per set.  SORT_CAP > 0: crossing lists of up to SORT_CAP neurons are sorted
 // here by a bitonic network in LDS; longer lists are left to the tiled rank kernels.
 template <int SORT_CAP>
@@ -147,6 +238,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   __shared__ int winact[16];
   __shared__ double skey[SORT_CAP > 0 ? SORT_CAP : 1];
   __shared__ int sidx[SORT_CAP > 0 ? SORT_CAP : 1];
+  static_assert(sizeof(double) == sizeof(long long), "keys are sorted through their bit patterns");
   int base = 0, inact_total = 0;
   int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
   for (int r0 = 0; r0 < d.N; r0 += 1024) {
@@ -201,7 +293,10 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   }
   if (SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP) {
     __syncthreads();
-    bitonic_sort_desc<SORT_CAP>(skey, sidx, m, tid, d.cross_idx);
+    if constexpr (SORT_CAP == 1024)  // the staged doubles are read back as their bit patterns
+      sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
+    else
+      bitonic_sort_desc<SORT_CAP>(skey, sidx, m, tid, d.cross_idx);
   }
 }
 
@@ -219,7 +314,7 @@ __global__ __launch_bounds__(1024) void relu_sort_small_kernel(const ReluDesc* _
     sidx[tid] = d.asc_idx[tid];
   }
   __syncthreads();
-  bitonic_sort_desc<1024>(skey, sidx, m, tid, d.cross_idx);
+  sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
 }
 
 // Multi-block classification for sets with more than 1024 neurons: pass 1 counts the crossing and

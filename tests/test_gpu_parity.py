@@ -154,6 +154,29 @@ def test_relu_step(nnv, oracle, method, N, n):
     assert R.C.shape == (3 + 3 * m2.size, n + m2.size)
 
 
+@pytest.mark.parametrize("method", ["relax-star-area", "relax-star-range"])
+@pytest.mark.parametrize("N", [2, 3, 33, 64, 65, 127, 128, 129, 255, 257, 511, 513, 777, 1023, 1024, 1025, 2047, 4100, 8192, 9000])
+def test_crossing_order_all_list_lengths_with_ties(nnv, oracle, method, N):
+    # every neuron crosses; keys come from a handful of values so that most of them tie and the stable
+    # rule (equal keys keep ascending neuron order) decides the order.  Bounds are exact in fp64:
+    # one generator, centre 0, |V| in {1/8, 1/4, 1/2, 1}  ->  lb = -|v|, ub = |v|.
+    rs = np.random.RandomState(N)
+    mag = rs.choice([0.125, 0.25, 0.5, 1.0], size=N) * rs.choice([-1.0, 1.0], size=N)
+    V = np.c_[np.zeros(N), mag]
+    if N > 3:
+        V[rs.choice(N, size=N // 7, replace=False), 0] = 4.0      # some active neurons in between
+        V[rs.choice(N, size=N // 9, replace=False), 0] = -4.0     # and some inactive ones
+    args = (V, np.zeros((1, 1)), np.zeros(1), [-1.0], [1.0])
+    R = nnv.PosLin.reach(nnv.Star(*args), method, [], 1)
+    O = oracle.OStar(*args)
+    elb, eub = oracle.estimate_ranges(O)
+    m1, m2 = oracle.relax_classify(elb, eub, method)
+    ni, idx, clb, cub = R.relu_info()
+    assert ni == m1.size
+    assert np.array_equal(idx, m2)
+    assert np.array_equal(clb, elb[m2]) and np.array_equal(cub, eub[m2])
+
+
 def test_relu_ties_and_degenerate(nnv, oracle):
     # hand-built bounds: ub == 0 -> inactive, lb == 0 -> active; equal sort keys keep index order
     V = np.array([[-0.5, 0.5], [0.5, 0.5], [1.0, -3.0], [-1.0, 2.0], [2.0, 0.0], [-1.0, 0.0], [1.0, 3.0], [-1.0, -2.0]])
