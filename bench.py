@@ -60,9 +60,9 @@ def main():
                  "that path is not built) - use --gpus 1")
 
     import nnv_amd
-    from nnv_amd.configs import count_updates, device_input_sets, make_config
+    from nnv_amd.configs import count_updates, device_input_sets, make_config, make_extended_cnn
 
-    cfg = make_config(args.config)
+    cfg = make_extended_cnn(32, 3) if args.config == 6 else make_config(args.config)
     ctx = nnv_amd.default_context()
     net = nnv_amd.NN.from_config(cfg["layers"], cfg["name"])
     opts = {"reachMethod": args.method, "relaxFactor": 1}
@@ -107,13 +107,14 @@ def main():
         return acc / reps
 
     per_layer = timed_pass(1)          # NN.reachTime-style device time per layer
-    for grp in range(4):
+    for grp in range(5):
         ctx.kernel_time(grp)
     timed_pass(2)                      # per-kernel event pairs
     gemm_ms, gemm_launches, _ = ctx.kernel_time(0)
     conv_ms, conv_launches, _ = ctx.kernel_time(1)
     rng_ms, rng_launches, rng_bytes = ctx.kernel_time(2)
     app_ms, app_launches, app_bytes = ctx.kernel_time(3)
+    row_ms, row_launches, row_bytes = ctx.kernel_time(4)
 
     # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
     gemm_flop = conv_flop = 0.0
@@ -138,7 +139,11 @@ def main():
                 flop += 2.0 * (N // cout) * cout * fh * fw * cin * (n + 1)
             entry["dense_tflops"] = round(flop / (per_layer[i] * 1e-3) / 1e12, 3)
             conv_flop += flop
-        else:
+        elif Ld["type"] in ("batchnorm", "avgpool", "flatten", "imageinput"):
+            b = sum(8.0 * (sp._h.dims()[0] + so._h.dims()[0]) * (sp._h.dims()[1] + 1) for sp, so in zip(prev_sets, outs))
+            if per_layer[i] > 0:
+                entry["algo_GBps"] = round(b / (per_layer[i] * 1e-3) / 1e9, 1)
+        elif Ld["type"] == "relu":
             b = 0.0
             for sp, so in zip(prev_sets, outs):
                 N, n, _ = sp._h.dims()
@@ -178,7 +183,8 @@ def main():
     # the HBM-bound kernels: algorithmic bytes over their own HIP-event durations
     hbm = {}
     for name, ms_, n_, b_ in (("ranges_partial_kernel", rng_ms, rng_launches, rng_bytes),
-                              ("relu_apply_kernel", app_ms, app_launches, app_bytes)):
+                              ("relu_apply_kernel", app_ms, app_launches, app_bytes),
+                              ("row-wise affine layers (rowmap/avgpool/permute kernels)", row_ms, row_launches, row_bytes)):
         if n_:
             g = b_ / (ms_ * 1e-3) / 1e9
             hbm[name] = {"bound": "hbm", "achieved": round(g, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

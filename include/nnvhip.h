@@ -76,10 +76,12 @@ NNVHIP_API int nnvhip_last_op_time_ms(nnvhip_ctx* ctx, double* ms);
 /* Measurement hook (no counterpart in the reference): while timing level 2 is set, every launch of a
  * kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
  * dense GEMM kernel of the FC layers (tiles of at least 64 rows); 1: implicit-GEMM convolution
- * kernel; 2: estimateRanges column pass; 3: ReLU apply pass.  Returns accumulated kernel time,
+ * kernel; 2: estimateRanges column pass; 3: ReLU apply pass; 4: row-wise affine layers (row map,
+ * average pooling, row permutation).  Returns accumulated kernel time,
  * launch count and work since the last reset.  Work is dense flop for 0 and 1 (GEMM:
  * 2*Mp*Kp*ncols with M, K padded to 16; conv: 2*Ho*Wo*Cout*FH*FW*Cin*(n+1)) and algorithmic bytes for
- * 2 (8*N*(n+1) + 16*n + 16*N per set) and 3 (8*N*(n+1) read + 8*N*(n+1+m) written per set). */
+ * 2 (8*N*(n+1) + 16*n + 16*N per set), 3 (8*kept*(n+1) read + 8*N*(n+1+m) written per set, kept =
+ * rows that are neither inactive nor crossing) and 4 (8*(Nin + Nout)*(n+1) per set). */
 NNVHIP_API int nnvhip_kernel_time(nnvhip_ctx* ctx, int which, double* total_ms, int64_t* launches, double* total_work,
                        int reset);
 /* Measurement hook (no counterpart in the reference): runs a plain device-to-device copy kernel over
@@ -189,6 +191,44 @@ NNVHIP_API int nnvhip_halfspace_check(nnvhip_ctx* ctx, int64_t count, nnvhip_sta
  * C1 = G*V(:,2:n+1) (R x n, column-major) and d1 = g - G*V(:,1). */
 NNVHIP_API int nnvhip_halfspace_rows(nnvhip_ctx* ctx, nnvhip_star* s, int64_t R, const double* G, const double* g,
                           int64_t N, double* C1, double* d1);
+
+/* ---- row-wise affine layers -------------------------------------------------------------- */
+/* A per-row affine program: up to 8 steps, step s applies `v = v <op> params[:, s]` to the centre
+ * column only (NNVHIP_SCOPE_CENTRE) or to the centre and every generator (NNVHIP_SCOPE_ALL), in
+ * order.  It carries, with the reference's own order of operations,
+ *   BatchNormalizationLayer.reach_star_single_input, nn/layers/BatchNormalizationLayer.m:247-351
+ *     (ImageStar: c - mean; all / sqrt(var + eps); all * scale; c + offset.  Star: all * l; c + b),
+ *   ImageInputLayer.reach_star_single_input, nn/layers/ImageInputLayer.m:121-166
+ *     (zerocenter, zscore, rescale-zero-one, rescale-symmetric),
+ *   ImageStar.affineMap(scale, offset), set/ImageStar.m:431-460.
+ * params is N x n_steps, column-major (per-channel values are expanded to rows by the caller). */
+typedef struct nnvhip_rowmap nnvhip_rowmap;
+enum { NNVHIP_OP_ADD = 0, NNVHIP_OP_SUB = 1, NNVHIP_OP_MUL = 2, NNVHIP_OP_DIV = 3 };
+enum { NNVHIP_SCOPE_CENTRE = 0, NNVHIP_SCOPE_ALL = 1 };
+NNVHIP_API int nnvhip_rowmap_create(nnvhip_ctx* ctx, int64_t N, int32_t n_steps, const int32_t* op,
+                         const int32_t* scope, const double* params, nnvhip_rowmap** out);
+NNVHIP_API int nnvhip_rowmap_destroy(nnvhip_rowmap* map);
+NNVHIP_API int nnvhip_affine_rowmap(nnvhip_ctx* ctx, const nnvhip_rowmap* map, int64_t count,
+                         nnvhip_star* const* in, nnvhip_star** out);
+
+/* AveragePooling2DLayer(poolSize [h w], stride [sh sw], padding [t b l r]),
+ * nn/layers/AveragePooling2DLayer.m:35-147; reach_star_single_input :424-436 applies evaluate
+ * (:229-247, MatConvNet's vl_nnpool 'avg') to every H x W x C image of V: the mean over the part
+ * of each window that lies inside the image.  Output dim is Ho*Wo*C. */
+typedef struct nnvhip_avgpool2d nnvhip_avgpool2d;
+NNVHIP_API int nnvhip_avgpool2d_create(nnvhip_ctx* ctx, const int64_t pool[2], const int64_t stride[2],
+                            const int64_t padding[4], nnvhip_avgpool2d** out);
+NNVHIP_API int nnvhip_avgpool2d_destroy(nnvhip_avgpool2d* layer);
+NNVHIP_API int nnvhip_avgpool2d_output_size(const nnvhip_avgpool2d* layer, int64_t H, int64_t W, int64_t* Ho,
+                                 int64_t* Wo);
+NNVHIP_API int nnvhip_affine_avgpool2d(nnvhip_ctx* ctx, const nnvhip_avgpool2d* layer, int64_t H, int64_t W,
+                            int64_t count, nnvhip_star* const* in, nnvhip_star** out);
+
+/* Row permutation out(r, :) = in(src_row[r], :): the C-style variants of FlattenLayer.evaluate
+ * applied to every image of V (nn/layers/FlattenLayer.m:118-170, 178-199).  The MATLAB-style
+ * flatten is a plain reshape and needs no call.  src_row: N entries, 0-based, a permutation. */
+NNVHIP_API int nnvhip_permute_rows(nnvhip_ctx* ctx, int64_t N, const int32_t* src_row, int64_t count,
+                        nnvhip_star* const* in, nnvhip_star** out);
 
 #ifdef __cplusplus
 }

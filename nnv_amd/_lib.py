@@ -23,7 +23,9 @@ SYMBOLS = [
     "nnvhip_star_relu_counts", "nnvhip_star_fetch_crossing", "nnvhip_estimate_ranges",
     "nnvhip_estimate_ranges_batch", "nnvhip_fc_create", "nnvhip_fc_destroy", "nnvhip_conv2d_create",
     "nnvhip_conv2d_destroy", "nnvhip_conv2d_output_size", "nnvhip_affine_fc", "nnvhip_affine_conv2d",
-    "nnvhip_relu_relax", "nnvhip_halfspace_check", "nnvhip_halfspace_rows",
+    "nnvhip_relu_relax", "nnvhip_halfspace_check", "nnvhip_halfspace_rows", "nnvhip_rowmap_create",
+    "nnvhip_rowmap_destroy", "nnvhip_affine_rowmap", "nnvhip_avgpool2d_create", "nnvhip_avgpool2d_destroy",
+    "nnvhip_avgpool2d_output_size", "nnvhip_affine_avgpool2d", "nnvhip_permute_rows",
 ]
 
 
@@ -82,6 +84,14 @@ def load():
         "nnvhip_relu_relax": [p, C.c_int, dbl, i64, pp, pp],
         "nnvhip_halfspace_check": [p, i64, pp, i64, p, p, p, i64, p, p, p],
         "nnvhip_halfspace_rows": [p, p, i64, p, p, i64, p, p],
+        "nnvhip_rowmap_create": [p, i64, C.c_int32, p, p, p, pp],
+        "nnvhip_rowmap_destroy": [p],
+        "nnvhip_affine_rowmap": [p, p, i64, pp, pp],
+        "nnvhip_avgpool2d_create": [p, pi64, pi64, pi64, pp],
+        "nnvhip_avgpool2d_destroy": [p],
+        "nnvhip_avgpool2d_output_size": [p, i64, i64, pi64, pi64],
+        "nnvhip_affine_avgpool2d": [p, p, i64, i64, i64, pp, pp],
+        "nnvhip_permute_rows": [p, i64, p, i64, pp, pp],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)

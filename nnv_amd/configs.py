@@ -117,6 +117,31 @@ def make_config(k: int, shrink: int = 1):
     raise ValueError("config index must be 1..5")
 
 
+def make_extended_cnn(hw=16, cin=3, seed=2001):
+    """A CNN that strings together the further affine layers around the relax-star ReLU:
+    ImageInputLayer (zscore) -> conv 3x3x8 -> BatchNormalization -> ReLU -> AveragePooling 2x2/2 ->
+    conv 3x3x16 -> ReLU -> AveragePooling 3x3/2 pad 1 -> Flatten (Keras C-style) -> FC 32 -> ReLU -> FC 10."""
+    rs = np.random.RandomState(seed)
+    x = rs.rand(hw * hw * cin)
+    c1, c2 = 8, 16
+    conv1 = _conv(rs, 3, 3, cin, c1, 1, 1)
+    bn = {"type": "batchnorm", "mean": 0.1 * rs.randn(c1), "var": rs.rand(c1) + 0.5, "eps": 1e-5,
+          "scale": 1.0 + 0.1 * rs.randn(c1), "offset": 0.1 * rs.randn(c1)}
+    pool1 = {"type": "avgpool", "pool": [2, 2], "stride": [2, 2], "padding": [0, 0, 0, 0]}
+    conv2 = _conv(rs, 3, 3, c1, c2, 1, 1)
+    pool2 = {"type": "avgpool", "pool": [3, 3], "stride": [2, 2], "padding": [1, 1, 1, 1]}
+    h = hw // 2
+    h2 = (h + 2 - 3) // 2 + 1
+    flat = {"type": "flatten", "flatten_type": "nnet.keras.layer.FlattenCStyleLayer"}
+    inp = {"type": "imageinput", "normalization": "zscore", "input_size": [hw, hw, cin],
+           "mean": rs.rand(1, 1, cin), "std": 0.5 + rs.rand(cin)}
+    layers = [inp, conv1, bn, _relu(), pool1, conv2, _relu(), pool2, flat,
+              _fc(rs, 32, h2 * h2 * c2), _relu(), _fc(rs, 10, 32)]
+    eps = 1.0 / 255.0
+    return {"name": "cnn_with_norm_pool_flatten_%dx%dx%d" % (hw, hw, cin), "kind": "image", "image_shape": (hw, hw, cin),
+            "layers": layers, "lb": x - eps, "ub": x + eps}
+
+
 def count_updates(layer_shapes):
     """Generator-neuron updates of one reach: sum over layer steps of N_out * (n_out + 1)."""
     return int(sum(int(N) * (int(n) + 1) for (N, n) in layer_shapes))

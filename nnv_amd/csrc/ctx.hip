@@ -661,11 +661,13 @@ int nnvhip_conv2d_output_size(const nnvhip_conv2d* cv, int64_t H, int64_t W, int
   return NNVHIP_OK;
 }
 
+}  // extern "C"
+
 // Shared set-up of the affine layers: validates the input array, allocates one output arena with
 // the sets back to back, and creates output handles that share constraints and predicate bounds
 // with their inputs.
-static int make_affine_outputs(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, int64_t Nout,
-                               std::vector<nnvhip_star*>* outs, bool* contiguous, int64_t* total_cols) {
+int nnvhip::make_affine_outputs(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, int64_t Nout,
+                                std::vector<nnvhip_star*>* outs, bool* contiguous, int64_t* total_cols) {
   int64_t ldout = round_up(Nout, kLdAlign);
   int64_t cols = 0;
   bool contig = true;
@@ -695,17 +697,19 @@ static int make_affine_outputs(nnvhip_ctx* c, int64_t count, nnvhip_star* const*
   return NNVHIP_OK;
 }
 
-static void release_all(std::vector<nnvhip_star*>& v) {
+void nnvhip::release_all(std::vector<nnvhip_star*>& v) {
   for (auto* s : v) nnvhip_star_release(s);
   v.clear();
 }
 
-static int check_set_array(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
+int nnvhip::check_set_array(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
   if (!in || !out || count <= 0) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   for (int64_t i = 0; i < count; ++i)
     if (!in[i] || in[i]->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid set handle %lld", (long long)i);
   return NNVHIP_OK;
 }
+
+extern "C" {
 
 int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
   CHECK_CTX(c);

@@ -109,11 +109,12 @@ struct nnvhip_ctx {
   // timing of the dominant kernel alone (events directly around its launch), per instantiation group
   hipEvent_t kev0 = nullptr, kev1 = nullptr;
   // [0] dense MFMA GEMM (tiles of at least 64 rows), [1] implicit-GEMM convolution (work = flop),
-  // [2] estimateRanges column pass, [3] ReLU apply pass (work = algorithmic bytes)
-  static constexpr int kKernelGroups = 4;
-  double kern_ms[kKernelGroups] = {0.0, 0.0, 0.0, 0.0};
-  int64_t kern_launches[kKernelGroups] = {0, 0, 0, 0};
-  double kern_flop[kKernelGroups] = {0.0, 0.0, 0.0, 0.0};
+  // [2] estimateRanges column pass, [3] ReLU apply pass, [4] row-wise affine layers (batch
+  // normalisation, input normalisation, average pooling, flatten) (work = algorithmic bytes)
+  static constexpr int kKernelGroups = 5;
+  double kern_ms[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0};
+  int64_t kern_launches[kKernelGroups] = {0, 0, 0, 0, 0};
+  double kern_flop[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0};
   int kernel_timer_begin(bool on);
   int kernel_timer_end(bool on, int which, double flop);
 
@@ -168,6 +169,14 @@ struct nnvhip_conv2d {
 namespace nnvhip {
 
 nnvhip_star* new_star(nnvhip_ctx* ctx);
+
+// Shared set-up of the affine layers (ctx.hip): validates the handle array; allocates one output arena
+// with the sets back to back and creates output handles that share constraints and predicate bounds
+// with their inputs; releases a vector of handles after a failure.
+int check_set_array(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, nnvhip_star** out);
+int make_affine_outputs(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, int64_t Nout,
+                        std::vector<nnvhip_star*>* outs, bool* contiguous, int64_t* total_cols);
+void release_all(std::vector<nnvhip_star*>& v);
 
 // Optional fusion of Star.estimateRanges into the GEMM epilogue (one set per launch): every column
 // tile leaves the four partial range sums of its rows in `part` ([chunks][4][ldc]); the caller then

@@ -233,6 +233,64 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
     check(nnvhip_halfspace_rows(ctx(), s, (int64_t)R, dbl(prhs[2], "G"), dbl(prhs[3], "g"), (int64_t)mxGetN(prhs[2]),
                                 mxGetDoubles(plhs[0]), mxGetDoubles(d1)));
     if (nlhs > 1) plhs[1] = d1; else mxDestroyArray(d1);
+  } else if (cmd == "rowmap_create") {  // (ops (1 x S), scopes (1 x S), params (N x S)) -> layer handle
+    // per-row affine programme: ops 0 add | 1 sub | 2 mul | 3 div; scopes 0 centre column | 1 all columns
+    need(nrhs, 3, "rowmap_create");
+    const mwSize S = mxGetN(prhs[3]), N = mxGetM(prhs[3]);
+    if (mxGetNumberOfElements(prhs[1]) != S || mxGetNumberOfElements(prhs[2]) != S)
+      mexErrMsgIdAndTxt("nnvhip:error", "one op and one scope per parameter column");
+    std::vector<int32_t> op(S), sc(S);
+    for (mwSize i = 0; i < S; ++i) {
+      op[i] = (int32_t)dbl(prhs[1], "ops")[i];
+      sc[i] = (int32_t)dbl(prhs[2], "scopes")[i];
+    }
+    nnvhip_rowmap* m = nullptr;
+    check(nnvhip_rowmap_create(ctx(), (int64_t)N, (int32_t)S, op.data(), sc.data(), dbl(prhs[3], "params"), &m));
+    plhs[0] = to_mx(m);
+  } else if (cmd == "rowmap_destroy") {
+    need(nrhs, 1, "rowmap_destroy");
+    check(nnvhip_rowmap_destroy(handle_of<nnvhip_rowmap>(prhs[1])));
+  } else if (cmd == "affine_rowmap") {  // (layer, handles) -> handles      BatchNormalizationLayer / ImageInputLayer reach
+    need(nrhs, 2, "affine_rowmap");
+    std::vector<nnvhip_star*> in = handles_of(prhs[2]), out(in.size());
+    check(nnvhip_affine_rowmap(ctx(), handle_of<nnvhip_rowmap>(prhs[1]), (int64_t)in.size(), in.data(), out.data()));
+    plhs[0] = to_mx(out);
+  } else if (cmd == "avgpool2d_create") {  // (poolSize [h w], stride [sh sw], padding [t b l r]) -> layer handle
+    need(nrhs, 3, "avgpool2d_create");
+    if (mxGetNumberOfElements(prhs[1]) != 2) mexErrMsgIdAndTxt("nnvhip:error", "Invalid pool size");
+    if (mxGetNumberOfElements(prhs[2]) != 2) mexErrMsgIdAndTxt("nnvhip:error", "Invalid stride");
+    if (mxGetNumberOfElements(prhs[3]) != 4) mexErrMsgIdAndTxt("nnvhip:error", "Invalide padding size");
+    int64_t pool[2], st[2], pad[4];
+    for (int i = 0; i < 2; ++i) {
+      pool[i] = (int64_t)dbl(prhs[1], "poolSize")[i];
+      st[i] = (int64_t)dbl(prhs[2], "stride")[i];
+    }
+    for (int i = 0; i < 4; ++i) pad[i] = (int64_t)dbl(prhs[3], "padding")[i];
+    nnvhip_avgpool2d* l = nullptr;
+    check(nnvhip_avgpool2d_create(ctx(), pool, st, pad, &l));
+    plhs[0] = to_mx(l);
+  } else if (cmd == "avgpool2d_destroy") {
+    need(nrhs, 1, "avgpool2d_destroy");
+    check(nnvhip_avgpool2d_destroy(handle_of<nnvhip_avgpool2d>(prhs[1])));
+  } else if (cmd == "affine_avgpool2d") {  // (layer, H, W, handles) -> [handles, Ho, Wo]      AveragePooling2DLayer.reach
+    need(nrhs, 4, "affine_avgpool2d");
+    std::vector<nnvhip_star*> in = handles_of(prhs[4]), out(in.size());
+    nnvhip_avgpool2d* l = handle_of<nnvhip_avgpool2d>(prhs[1]);
+    const int64_t H = (int64_t)mxGetScalar(prhs[2]), W = (int64_t)mxGetScalar(prhs[3]);
+    int64_t Ho = 0, Wo = 0;
+    check(nnvhip_avgpool2d_output_size(l, H, W, &Ho, &Wo));
+    check(nnvhip_affine_avgpool2d(ctx(), l, H, W, (int64_t)in.size(), in.data(), out.data()));
+    plhs[0] = to_mx(out);
+    if (nlhs > 1) plhs[1] = mxCreateDoubleScalar((double)Ho);
+    if (nlhs > 2) plhs[2] = mxCreateDoubleScalar((double)Wo);
+  } else if (cmd == "permute_rows") {  // (src_row (1-based, N x 1), handles) -> handles      C-style FlattenLayer.reach
+    need(nrhs, 2, "permute_rows");
+    const mwSize N = mxGetNumberOfElements(prhs[1]);
+    std::vector<int32_t> src(N);
+    for (mwSize i = 0; i < N; ++i) src[i] = (int32_t)dbl(prhs[1], "src_row")[i] - 1;
+    std::vector<nnvhip_star*> in = handles_of(prhs[2]), out(in.size());
+    check(nnvhip_permute_rows(ctx(), (int64_t)N, src.data(), (int64_t)in.size(), in.data(), out.data()));
+    plhs[0] = to_mx(out);
   } else if (cmd == "sync") {
     check(nnvhip_synchronize(ctx()));
   } else if (cmd == "set_timing") {

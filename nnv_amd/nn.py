@@ -6,6 +6,8 @@ import time
 import numpy as np
 
 from .layers import Conv2DLayer, FullyConnectedLayer, ReluLayer
+from .layers_affine import (AveragePooling2DLayer, BatchNormalizationLayer, FlattenLayer, ImageInputLayer,
+                            LayerS)
 from .sets import ImageStar, Star
 from .verify import HalfSpace, verify_specification
 
@@ -36,6 +38,19 @@ class NN:
                                           L.get("dilation", [1, 1])))
             elif L["type"] == "relu":
                 layers.append(ReluLayer())
+            elif L["type"] == "batchnorm":
+                layers.append(BatchNormalizationLayer(NumChannels=np.size(L["mean"]), TrainedMean=L["mean"],
+                                                      TrainedVariance=L["var"], Epsilon=L["eps"], Scale=L["scale"],
+                                                      Offset=L["offset"]))
+            elif L["type"] == "avgpool":
+                layers.append(AveragePooling2DLayer(L["pool"], L["stride"], L["padding"]))
+            elif L["type"] == "flatten":
+                layers.append(FlattenLayer("FlattenLayer", L["flatten_type"]))
+            elif L["type"] == "imageinput":
+                layers.append(ImageInputLayer("ImageInputLayer", L.get("input_size", []), L["normalization"], "auto",
+                                              L.get("mean"), L.get("std"), L.get("min"), L.get("max")))
+            elif L["type"] == "layers":
+                layers.append(LayerS(L["W"], L["b"], L["f"]))
             else:
                 raise ValueError("unknown layer type %r" % (L["type"],))
         return NN(layers, name)

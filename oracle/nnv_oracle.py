@@ -42,6 +42,15 @@ Parity pinning (what checks each function; see tests/test_oracle_*.py)
   regression tests only check that the methods exist): PARITY UNPINNED by vectors; pinned by
   the source text, hand-built cases and the point-wise meaning of the verdict (a sampled
   output inside the unsafe region forces "unknown").
+* avgpool2d_tensor: the reference's known answers without padding
+  (tests/nn/layers/AveragePooling2DLayer/test_layers_averagePooling.m:14-23, 41-56) and, for the
+  padded border, MatConvNet's published rule (mean over the cells inside the image) against torch's
+  avg_pool2d(count_include_pad=False).  MatConvNet ships only as binaries in the reference:
+  last-ulp summation order PARITY UNPINNED.
+* batchnorm_*, image_input_*, image_star_affine_map, flatten_*: no reference test holds a value
+  (PARITY UNPINNED by vectors); pinned by the textbook formulas, hand-computed permutations and by
+  the affine-consistency identity reach(I).c = evaluate(c), reach(I).v_j = evaluate(c + v_j) -
+  evaluate(c), which ties every reach restatement to its evaluate.
 """
 from __future__ import annotations
 
@@ -546,6 +555,16 @@ def nn_reach(layers, input_set, reach_method="relax-star-area", relax_factor=1.0
                                         L.get("stride", (1, 1)), L.get("dilation", (1, 1))))
             elif L["type"] == "relu":
                 out.append(relu_reach(S, reach_method, relax_factor))
+            elif L["type"] == "batchnorm":
+                out.append(batchnorm_reach(S, L["mean"], L["var"], L["eps"], L["scale"], L["offset"]))
+            elif L["type"] == "avgpool":
+                out.append(avgpool2d_reach(S, L["pool"], L["stride"], L["padding"]))
+            elif L["type"] == "flatten":
+                out.append(flatten_reach(S, L["flatten_type"]))
+            elif L["type"] == "imageinput":
+                out.append(image_input_reach(S, L["normalization"], L.get("mean"), L.get("std"), L.get("min"), L.get("max")))
+            elif L["type"] == "layers":
+                out.append(layers_reach(S, L["W"], L["b"], L["f"], reach_method, relax_factor))
             else:
                 raise ValueError("unknown layer type " + str(L["type"]))
         sets = out
@@ -577,7 +596,223 @@ def evaluate(layers, x):
                               L.get("stride", (1, 1)), L.get("dilation", (1, 1)))[:, :, :, 0]
         elif L["type"] == "relu":
             x = np.maximum(x, 0)
+        elif L["type"] == "batchnorm":
+            x = batchnorm_evaluate(x, L["mean"], L["var"], L["eps"], L["scale"], L["offset"])
+        elif L["type"] == "avgpool":
+            x = avgpool2d_tensor(x[:, :, :, None], L["pool"], L["stride"], L["padding"])[:, :, :, 0]
+        elif L["type"] == "flatten":
+            x = flatten_evaluate(x, L["flatten_type"]) if x.ndim == 3 else x
+        elif L["type"] == "imageinput":
+            x = image_input_evaluate(x, L["normalization"], L.get("mean"), L.get("std"), L.get("min"), L.get("max"))
+        elif L["type"] == "layers":
+            x = np.asarray(L["W"]) @ x.reshape(-1, order="F") + np.asarray(L["b"]).reshape(-1)
+            if L["f"] == "poslin":
+                x = np.maximum(x, 0)
     return x
+
+
+# --------------------------------------------------------------------------------------
+# further affine layers: batch normalisation, average pooling, flatten, input normalisation
+# --------------------------------------------------------------------------------------
+def _chan(a, C):
+    """A per-channel parameter (1x1xC array, vector or scalar) as a length-C vector."""
+    a = np.asarray(a, dtype=np.float64).reshape(-1)
+    if a.size == 1:
+        a = np.repeat(a, C)
+    if a.size != C:
+        raise ValueError("Inconsistent number of channels between scale array and the ImageStar")
+    return a
+
+
+def batchnorm_evaluate(x, mean, var, eps, scale, offset):
+    """BatchNormalizationLayer.evaluate, nn/layers/BatchNormalizationLayer.m:118-229: per channel
+    (third axis of an image, entries of a vector) ((x - mean)/sqrt(var + eps))*scale + offset."""
+    x = np.asarray(x, dtype=np.float64)
+    if x.ndim == 3:
+        C = x.shape[2]
+        m, v, s, o = (_chan(a, C)[None, None, :] for a in (mean, var, scale, offset))
+    else:
+        C = x.size
+        m, v, s, o = (_chan(a, C).reshape(x.shape) for a in (mean, var, scale, offset))
+    return s * ((x - m) / np.sqrt(v + eps)) + o
+
+
+def batchnorm_reach(I, mean, var, eps, scale, offset):
+    """BatchNormalizationLayer.reach_star_single_input, nn/layers/BatchNormalizationLayer.m:247-351.
+
+    ImageStar (:286-330), per channel i:  V(:,:,i,1) -= mean_i;  V(:,:,i,:) = V(:,:,i,:) .* 1 / sqrt(var_i + eps)
+    (MATLAB evaluates `x .* 1 / s` left to right: a division by s);  V(:,:,i,:) .*= scale_i;
+    V(:,:,i,1) += offset_i.   Star (:332-349):  l = scale ./ sqrt(var + eps);  b = offset - mean .* l;
+    V = V .* l;  V(:,1) += b."""
+    if isinstance(I, OImageStar):
+        C = I.numChannel
+        m, v, s, o = (_chan(a, C) for a in (mean, var, scale, offset))
+        V = I.V.copy()
+        for i in range(C):
+            V[:, :, i, 0] = V[:, :, i, 0] - m[i]
+            V[:, :, i, :] = (V[:, :, i, :] * 1.0) / np.sqrt(v[i] + eps)
+            V[:, :, i, :] = V[:, :, i, :] * s[i]
+            V[:, :, i, 0] = V[:, :, i, 0] + o[i]
+        return OImageStar(V, I.C, I.d, I.pred_lb, I.pred_ub)
+    if isinstance(I, OStar):
+        N = I.dim
+        m, v, s, o = (_chan(a, N) for a in (mean, var, scale, offset))
+        l = s / np.sqrt(v + eps)
+        b = o - m * l
+        V = I.V * l[:, None]
+        V[:, 0] = V[:, 0] + b
+        return OStar(V, I.C, I.d, I.predicate_lb, I.predicate_ub)
+    raise TypeError("Input is not a Star, ImageStar or VolumeStar")
+
+
+def avgpool2d_output_size(H, W, pool, padding, stride):
+    """AveragePooling2DLayer.get_size_averageMap, nn/layers/AveragePooling2DLayer.m:396-418."""
+    t, b, l, r = padding
+    return ((H + t + b - pool[0]) // stride[0] + 1, (W + l + r - pool[1]) // stride[1] + 1)
+
+
+def avgpool2d_tensor(X, pool, stride, padding):
+    """AveragePooling2DLayer.evaluate, nn/layers/AveragePooling2DLayer.m:229-247 = MatConvNet's
+    vl_nnpool(..., 'Method', 'avg') (third-party, vendored only as binaries; restated from its
+    published CPU source): for every output cell the window is clipped to the image and the mean is
+    taken over the cells that remain (padding does not count), as sum * (1 / count); the sum runs
+    over window columns (outer) and rows (inner).  X: H x W x C x B."""
+    X = np.asarray(X, dtype=np.float64)
+    H, W, C, B = X.shape
+    ph, pw = pool
+    sh, sw = stride
+    t, b, l, r = padding
+    Ho, Wo = avgpool2d_output_size(H, W, pool, padding, stride)
+    Y = np.zeros((Ho, Wo, C, B))
+    for wo in range(Wo):
+        x1 = wo * sw - l
+        x2 = min(x1 + pw, W)
+        x1 = max(x1, 0)
+        for ho in range(Ho):
+            y1 = ho * sh - t
+            y2 = min(y1 + ph, H)
+            y1 = max(y1, 0)
+            acc = np.zeros((C, B))
+            for x in range(x1, x2):
+                for y in range(y1, y2):
+                    acc = acc + X[y, x, :, :]
+            Y[ho, wo, :, :] = acc * (1.0 / ((y2 - y1) * (x2 - x1)))
+    return Y
+
+
+def avgpool2d_reach(I: OImageStar, pool, stride, padding) -> OImageStar:
+    """AveragePooling2DLayer.reach_star_single_input, nn/layers/AveragePooling2DLayer.m:424-436:
+    Y = evaluate(V) on all n+1 images; constraints and predicate bounds unchanged."""
+    if not isinstance(I, OImageStar):
+        raise TypeError("The input is not an ImageStar object")
+    return OImageStar(avgpool2d_tensor(I.V, pool, stride, padding), I.C, I.d, I.pred_lb, I.pred_ub)
+
+
+def flatten_evaluate(image, layer_type):
+    """FlattenLayer.evaluate for an H x W x C image, nn/layers/FlattenLayer.m:118-170: MATLAB style is
+    a column-major reshape; Keras C-style permutes [3 2 1] first; the ONNX variants permute [2 1 3]."""
+    image = np.asarray(image, dtype=np.float64)
+    if image.ndim != 3:
+        raise ValueError("Invalid input.")
+    if layer_type == "nnet.keras.layer.FlattenCStyleLayer":
+        image = np.transpose(image, (2, 1, 0))
+    elif layer_type == "nnet.cnn.layer.FlattenLayer":
+        pass
+    elif layer_type in ("nnet.onnx.layer.FlattenLayer", "nnet.onnx.layer.FlattenInto2dLayer",
+                        "nnet.onnx.layer.Flatten3dInto2dLayer"):
+        image = np.transpose(image, (1, 0, 2))
+    else:
+        raise ValueError("Unknown type of flatten layer")
+    return image.reshape(1, 1, -1, order="F")
+
+
+def flatten_reach(I, layer_type):
+    """FlattenLayer.reach_single_input, nn/layers/FlattenLayer.m:178-199: evaluate on each of the n+1
+    images -> ImageStar 1 x 1 x N x (n+1).  Stars pass through (:218-221)."""
+    if isinstance(I, OStar):
+        return I
+    if not isinstance(I, OImageStar):
+        raise TypeError("Invalid input set (ImageStar, ImageZono or VolumeStar)")
+    N = I.height * I.width * I.numChannel
+    V = np.zeros((1, 1, N, I.numPred + 1))
+    for i in range(I.numPred + 1):
+        V[0, 0, :, i] = flatten_evaluate(I.V[:, :, :, i], layer_type).reshape(-1)
+    return OImageStar(V, I.C, I.d, I.pred_lb, I.pred_ub)
+
+
+def image_star_affine_map(I: OImageStar, scale, offset) -> OImageStar:
+    """ImageStar.affineMap(scale, offset), set/ImageStar.m:431-460: new_V = scale .* V (scalar or
+    1x1xC scale broadcast over the image), new_V(:,:,:,1) += offset (scalar, 1x1xC or H x W x C)."""
+    V = I.V
+    if scale is not None and np.size(scale):
+        sc = np.asarray(scale, dtype=np.float64)
+        if sc.size != 1 and sc.size != I.numChannel:
+            raise ValueError("Inconsistent number of channels between scale array and the ImageStar")
+        V = (sc.reshape(-1)[0] if sc.size == 1 else sc.reshape(1, 1, -1, 1)) * V
+    else:
+        V = V.copy()
+    if offset is not None and np.size(offset):
+        off = np.asarray(offset, dtype=np.float64)
+        if off.size == I.numChannel and off.ndim <= 1:
+            off = off.reshape(1, 1, -1)
+        V[:, :, :, 0] = V[:, :, :, 0] + off
+    return OImageStar(V, I.C, I.d, I.pred_lb, I.pred_ub)
+
+
+def image_input_evaluate(x, normalization, mean=None, std=None, mn=None, mx=None):
+    """ImageInputLayer.evaluate, nn/layers/ImageInputLayer.m:60-117."""
+    x = np.asarray(x, dtype=np.float64)
+    if normalization == "none":
+        return x
+    if normalization == "zerocenter":
+        return x - np.asarray(mean, dtype=np.float64)
+    if normalization == "zscore":
+        return (x - np.asarray(mean, dtype=np.float64)) / np.asarray(std, dtype=np.float64).reshape(1, 1, -1)
+    if normalization == "rescale-zero-one":
+        return (x - mn) / (mx - mn) if mn is not None and mx is not None else x / 255
+    if normalization == "rescale-symmetric":
+        return 2 * (x - mn) / (mx - mn) - 1 if mn is not None and mx is not None else 2 * x / 255 - 1
+    raise ValueError("The normalization method is not supported yet.")
+
+
+def image_input_reach(I: OImageStar, normalization, mean=None, std=None, mn=None, mx=None) -> OImageStar:
+    """ImageInputLayer.reach_star_single_input, nn/layers/ImageInputLayer.m:121-166."""
+    if not isinstance(I, OImageStar):
+        raise TypeError("Input is not an ImageStar")
+    if normalization == "none":
+        return I
+    if normalization == "zerocenter":
+        return image_star_affine_map(I, None, -np.asarray(mean, dtype=np.float64))
+    if normalization == "zscore":
+        out = image_star_affine_map(I, None, -np.asarray(mean, dtype=np.float64))
+        sd = np.asarray(std, dtype=np.float64).reshape(-1)
+        for nc in range(out.numChannel):
+            out.V[:, :, nc, :] = out.V[:, :, nc, :] / sd[nc]
+        return out
+    if normalization == "rescale-zero-one":
+        if mn is not None and mx is not None:
+            out = image_star_affine_map(I, None, -np.asarray(mn, dtype=np.float64))
+            out.V = out.V * (1.0 / (mx - mn))
+            return out
+        return image_star_affine_map(I, 1 / 255, None)
+    if normalization == "rescale-symmetric":
+        if mn is not None and mx is not None:
+            out = image_star_affine_map(I, None, -np.asarray(mn, dtype=np.float64))
+            out.V = out.V * (2.0 / (mx - mn))
+            return image_star_affine_map(out, None, -1.0)
+        return image_star_affine_map(I, 2 / 255, -1.0)
+    raise ValueError("The normalization method is not supported yet.")
+
+
+def layers_reach(I, W, b, f, reach_method, relax_factor=1.0):
+    """LayerS.reach, nn/layers/LayerS.m:120-262: affineMap(W, b), then the activation
+    ('purelin' and 'softmax' leave the set, 'poslin' -> PosLin.reach)."""
+    I1 = affine_map(I, W, b)
+    if f in ("purelin", "softmax"):
+        return I1
+    if f == "poslin":
+        return reach_relaxed_star(I1, reach_method, relax_factor)
+    raise ValueError("Unsupported activation function, currently support purelin, poslin(ReLU), satlin, satlins, logsig, tansig, softmax")
 
 
 # --------------------------------------------------------------------------------------
