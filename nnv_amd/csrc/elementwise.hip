@@ -134,15 +134,31 @@ __global__ __launch_bounds__(64 * kEwWaves) void avgpool_kernel(const SetDesc* _
     base = (int64_t)c * a.H * a.W;
     scale = 1.0 / (double)((y2 - y1) * (x2 - x1));
   }
-  for (int j = j0 + wave; j < j1; j += kEwWaves) {
-    double acc = 0.0;
+  // each wave takes 4 consecutive columns per step: four independent sums keep more loads in flight
+  for (int jb = j0 + 4 * wave; jb < j1; jb += 4 * kEwWaves) {
+    const int nu = min(4, j1 - jb);
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
     if (real) {
-      const double* col = d.in + (int64_t)j * a.ldin + base;
-      for (int x = x1; x < x2; ++x)
-        for (int y = y1; y < y2; ++y) acc = __dadd_rn(acc, col[y + (int64_t)x * a.H]);
-      acc = __dmul_rn(acc, scale);
+      const double* col = d.in + (int64_t)jb * a.ldin + base;
+      if (nu == 4) {
+        for (int x = x1; x < x2; ++x)
+          for (int y = y1; y < y2; ++y) {
+            const double* p = col + y + (int64_t)x * a.H;
+            const double v0 = p[0], v1 = p[a.ldin], v2 = p[2 * a.ldin], v3 = p[3 * a.ldin];
+            acc[0] = __dadd_rn(acc[0], v0);
+            acc[1] = __dadd_rn(acc[1], v1);
+            acc[2] = __dadd_rn(acc[2], v2);
+            acc[3] = __dadd_rn(acc[3], v3);
+          }
+      } else {
+        for (int u = 0; u < nu; ++u)
+          for (int x = x1; x < x2; ++x)
+            for (int y = y1; y < y2; ++y) acc[u] = __dadd_rn(acc[u], col[y + (int64_t)x * a.H + (int64_t)u * a.ldin]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc[u] = __dmul_rn(acc[u], scale);
     }
-    d.out[r + (int64_t)j * a.ldout] = acc;  // padding rows of the output stay zero
+    for (int u = 0; u < nu; ++u) d.out[r + (int64_t)(jb + u) * a.ldout] = acc[u];  // padding rows stay zero
   }
 }
 
@@ -177,6 +193,36 @@ __global__ __launch_bounds__(64 * kEwWaves) void permute_rows_kernel(const SetDe
 #pragma unroll
     for (int u = 0; u < 4; ++u)
       if (jb + u < j1) *reinterpret_cast<double2*>(d.out + r0 + (int64_t)(jb + u) * a.ldout) = v[u];
+  }
+}
+
+// Short columns (N <= kPermLdsRows): a block stages whole columns in LDS with coalesced loads and
+// gathers from there, so global memory sees only contiguous traffic.  Grid: (1, column chunks, sets).
+constexpr int kPermLdsRows = 4096;
+constexpr int kPermCols = 2;  // columns staged per step
+
+__global__ __launch_bounds__(64 * kEwWaves) void permute_rows_lds_kernel(const SetDesc* __restrict__ table, SetDesc one,
+                                                                         PermArgs a, int n_rows) {
+  const SetDesc d = table ? table[blockIdx.z] : one;
+  const int j0 = blockIdx.y * a.cols_per_chunk;
+  if (j0 >= d.ncols) return;
+  const int j1 = min(d.ncols, j0 + a.cols_per_chunk);
+  __shared__ double stage[kPermCols][kPermLdsRows];
+  const int tid = threadIdx.x;
+  for (int jb = j0; jb < j1; jb += kPermCols) {
+#pragma unroll
+    for (int u = 0; u < kPermCols; ++u)
+      if (jb + u < j1)
+        for (int r = tid; r < n_rows; r += 64 * kEwWaves) stage[u][r] = d.in[r + (int64_t)(jb + u) * a.ldin];
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < kPermCols; ++u)
+      if (jb + u < j1)
+        for (int64_t r = tid; r < a.ldout; r += 64 * kEwWaves) {
+          const int src = a.src_row[r];
+          d.out[r + (int64_t)(jb + u) * a.ldout] = src >= 0 ? stage[u][src] : 0.0;
+        }
+    __syncthreads();
   }
 }
 
@@ -366,7 +412,7 @@ int nnvhip_affine_avgpool2d(nnvhip_ctx* c, const nnvhip_avgpool2d* p, int64_t H,
   a.sw = (int32_t)p->stride[1];
   a.pt = (int32_t)p->pad[0];
   a.pl = (int32_t)p->pad[2];
-  return run_row_layer(c, count, in, out, Ho * Wo * C, 64, kEwWaves,
+  return run_row_layer(c, count, in, out, Ho * Wo * C, 64, 4 * kEwWaves,
                        [&](dim3 grid, const SetDesc* table, const SetDesc& one, int32_t cpc, int64_t ldout) {
                          a.cols_per_chunk = cpc;
                          a.ldout = ldout;
@@ -396,6 +442,14 @@ int nnvhip_permute_rows(nnvhip_ctx* c, int64_t N, const int32_t* src_row, int64_
   PermArgs a{};
   a.src_row = perm->as<int32_t>();
   a.ldin = in[0]->ld;
+  if (ld <= kPermLdsRows)
+    return run_row_layer(c, count, in, out, N, int64_t(1) << 30, 4 * kPermCols,
+                         [&](dim3 grid, const SetDesc* table, const SetDesc& one, int32_t cpc, int64_t ldout) {
+                           a.cols_per_chunk = cpc;
+                           a.ldout = ldout;
+                           hipLaunchKernelGGL(permute_rows_lds_kernel, grid, dim3(64 * kEwWaves), 0, c->stream, table, one,
+                                              a, (int)N);
+                         });
   return run_row_layer(c, count, in, out, N, kEwRows, 4 * kEwWaves,
                        [&](dim3 grid, const SetDesc* table, const SetDesc& one, int32_t cpc, int64_t ldout) {
                          a.cols_per_chunk = cpc;
