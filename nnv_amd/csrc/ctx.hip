@@ -358,11 +358,13 @@ __global__ void box_fill_kernel(double* __restrict__ V, int64_t ld, int N, const
   }
 }
 
-__global__ void fill_pm_one_kernel(double* __restrict__ plb, double* __restrict__ pub, int64_t n) {
+// info[2s] = offset of set s in the bounds buffer, info[2s+1] = its padded predicate count
+__global__ void fill_pm_one_kernel(double* __restrict__ bounds, const int64_t* __restrict__ info) {
+  const int64_t off = info[2 * blockIdx.y], n = info[2 * blockIdx.y + 1];
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   if (i < n) {
-    plb[i] = -1.0;
-    pub[i] = 1.0;
+    bounds[off + i] = -1.0;
+    bounds[off + n + i] = 1.0;
   }
 }
 
@@ -434,13 +436,28 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
     base->p_total = 1;
     base->n_total = st->n;
     st->cons = base;  // C0/d0 left null = all zeros
+    if (st->n > 0) {  // every generator column is vec(dim) * e_dim
+      st->oh_from = 1;
+      st->oh_idx_buf = dgen;
+      st->oh_idx = dgen->as<int32_t>() + gen_off[s];
+      st->oh_scale_buf = dvec;
+      st->oh_scale = dvec->as<double>() + s * N;
+    }
     out[s] = st;
   }
   // one launch fills every set's bounds: lb half gets -1, ub half +1
-  for (int64_t s = 0; s < count; ++s) {
-    int64_t npad = round_up(std::max<int64_t>(out[s]->n, 1), kLdAlign);
-    hipLaunchKernelGGL(fill_pm_one_kernel, dim3((unsigned)ceil_div(npad, 256)), dim3(256), 0, c->stream,
-                       out[s]->plb, out[s]->pub, npad);
+  {
+    std::vector<int64_t> pinfo((size_t)(2 * count));
+    int64_t max_npad = 0;
+    for (int64_t s = 0; s < count; ++s) {
+      pinfo[2 * s] = poff[s];
+      pinfo[2 * s + 1] = round_up(std::max<int64_t>(out[s]->n, 1), kLdAlign);
+      max_npad = std::max(max_npad, pinfo[2 * s + 1]);
+    }
+    BufRef dinfo;
+    NNV_TRY(c->upload(pinfo.data(), sizeof(int64_t) * pinfo.size(), &dinfo));
+    hipLaunchKernelGGL(fill_pm_one_kernel, dim3((unsigned)ceil_div(max_npad, 256), (unsigned)count), dim3(256), 0, c->stream,
+                       pb->as<double>(), dinfo->as<int64_t>());
   }
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
@@ -725,18 +742,60 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
   int st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
   if (st == NNVHIP_OK) {
     const double* bias = fc->bias ? fc->bias->as<double>() : nullptr;
+    const double* Wd = fc->W->as<double>();
+    // Columns of V that are scaled unit vectors (all generators of a box star, the columns a ReLU
+    // appended) need no contraction: W * (s * e_r) = s * W(:, r).  dense[i] = leading columns that do.
+    static const bool dense_only = getenv("NNVHIP_DENSE_AFFINE") != nullptr;
+    std::vector<int64_t> dense((size_t)count);
+    std::vector<GatherSet> gs((size_t)count);
+    int64_t total_dense = 0;
+    bool any_onehot = false;
+    for (int64_t i = 0; i < count; ++i) {
+      const int64_t nc = in[i]->n + 1;
+      dense[i] = (!dense_only && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
+      total_dense += dense[i];
+      any_onehot = any_onehot || dense[i] < nc;
+      GatherSet& g = gs[i];
+      g.idx = in[i]->oh_idx;
+      g.scale = in[i]->oh_scale;
+      g.out = outs[i]->V + dense[i] * outs[i]->ld;
+      g.plb = outs[i]->plb + (dense[i] - 1);
+      g.pub = outs[i]->pub + (dense[i] - 1);
+      g.m = (int32_t)(nc - dense[i]);
+      g.pad_ = 0;
+    }
     if (count == 1) {
       // one set: the GEMM epilogue also leaves the partial sums of Star.estimateRanges, so the
       // output set carries its ranges without another pass over V
       RangeFuse fuse;
       fuse.plb = outs[0]->plb;
       fuse.pub = outs[0]->pub;
-      st = launch_gemm(c, fc->W->as<double>(), fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols,
-                       fc->Kp, bias, &fuse);
-      if (st == NNVHIP_OK && fuse.chunks > 0) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks);
+      const int64_t gch = gather_chunks(fc->Mp, gs[0].m);
+      fuse.extra_chunks = gch;
+      st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], fc->Kp, bias, &fuse);
+      const bool fused = st == NNVHIP_OK && fuse.chunks > 0;
+      if (st == NNVHIP_OK && gs[0].m > 0)
+        st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? fuse.part->as<double>() : nullptr,
+                                   fuse.chunks, gch);
+      if (st == NNVHIP_OK && fused) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0));
     } else if (contig) {
-      st = launch_gemm(c, fc->W->as<double>(), fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols,
-                       fc->Kp, bias);
+      BufRef cmap;
+      const int32_t* colmap = nullptr;
+      if (any_onehot) {  // the dense columns of the sets, as positions in the (shared) arena layout
+        if (cols >= (int64_t(1) << 31)) st = NNVHIP_ERR_SHAPE;
+        std::vector<int32_t> map;
+        map.reserve((size_t)total_dense);
+        int64_t off = 0;
+        for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
+          for (int64_t j = 0; j < dense[i]; ++j) map.push_back((int32_t)(off + j));
+          off += in[i]->n + 1;
+        }
+        if (st == NNVHIP_OK) st = c->upload(map.data(), sizeof(int32_t) * map.size(), &cmap);
+        if (st == NNVHIP_OK) colmap = cmap->as<int32_t>();
+      }
+      if (st == NNVHIP_OK)
+        st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, any_onehot ? total_dense : cols,
+                         fc->Kp, bias, nullptr, colmap);
       if (st == NNVHIP_OK && bias && count > 1) {
         std::vector<double*> centres(count - 1);
         for (int64_t i = 1; i < count; ++i) centres[i - 1] = outs[i]->V;
@@ -744,10 +803,14 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         st = c->upload(centres.data(), sizeof(double*) * centres.size(), &tab);
         if (st == NNVHIP_OK) st = launch_bias_columns(c, tab->as<double*>(), count - 1, bias, fc->Mp);
       }
+      if (st == NNVHIP_OK && any_onehot)
+        st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, count, gs.data(), nullptr, 0, 0);
     } else {
-      for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
-        st = launch_gemm(c, fc->W->as<double>(), fc->Mp, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, fc->Mp,
-                         in[i]->n + 1, fc->Kp, bias);
+      for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
+        st = launch_gemm(c, Wd, fc->Mp, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, fc->Mp, dense[i], fc->Kp, bias);
+        if (st == NNVHIP_OK && gs[i].m > 0)
+          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[i]->ld, 1, &gs[i], nullptr, 0, 0);
+      }
     }
   }
   if (st == NNVHIP_OK) st = c->end_op();

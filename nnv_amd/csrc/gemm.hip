@@ -24,7 +24,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
                                                         double* __restrict__ part,
                                                         const double* __restrict__ plb,
                                                         const double* __restrict__ pub,
-                                                        double* __restrict__ rpart) {
+                                                        double* __restrict__ rpart,
+                                                        const int32_t* __restrict__ colmap) {
   constexpr int NT = 64 * WR * WC;  // threads per block
   constexpr int FM = TM / WR / 16;
   constexpr int FN = TN / WC / 16;
@@ -58,6 +59,13 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   constexpr int B_VEC = TN * KT / 2;
   constexpr int B_PASS = (B_VEC + NT - 1) / NT;
   double2 ra[A_PASS], rb[B_PASS];
+  // column of B behind each staged element (identity unless the dense columns sit scattered in an arena)
+  int64_t bcol[B_PASS];
+#pragma unroll
+  for (int p = 0; p < B_PASS; ++p) {
+    const int64_t col = n0 + (tid + p * NT) / (KT / 2);
+    bcol[p] = (colmap != nullptr && col < ncols) ? (int64_t)colmap[col] : col;
+  }
 
   auto load_tiles = [&](int k0) {
 #pragma unroll
@@ -77,7 +85,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
       int j = idx / (KT / 2);
       int64_t col = n0 + j;
       double2 v = make_double2(0.0, 0.0);
-      if (idx < B_VEC && col < ncols) v = *reinterpret_cast<const double2*>(B + (k0 + 2 * k2) + col * ldb);
+      if (idx < B_VEC && col < ncols) v = *reinterpret_cast<const double2*>(B + (k0 + 2 * k2) + bcol[p] * ldb);
       rb[p] = v;
     }
   };
@@ -197,7 +205,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
         if (col < ncols) {
           double v = acc[i][j][r];
           if (bias != nullptr && col == 0) v = v + bias[row];
-          C[row + col * ldc] = v;
+          const int64_t ccol = (colmap != nullptr && ksplit == 1) ? (int64_t)colmap[col] : col;
+          C[row + ccol * ldc] = v;
         }
       }
     }
@@ -220,7 +229,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __rest
 
 template <int TM, int TN, int WR, int WC, int KT>
 static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
-                      int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse) {
+                      int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse,
+                      const int32_t* colmap) {
   int64_t tiles_m = ceil_div(Mp, TM);
   int64_t tiles_n = ceil_div(ncols, TN);
   int64_t blocks = tiles_m * tiles_n;
@@ -253,11 +263,12 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   int64_t ksplit = 1;
   if (blocks < 128 && nk >= 8) ksplit = std::min<int64_t>(std::min<int64_t>(16, nk / 4), ceil_div(512, blocks));
   if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
+  if (colmap != nullptr) ksplit = 1;  // the split-K workspace is compact; mapped launches are large anyway
   BufRef ws;
   if (ksplit > 1) NNV_TRY(ctx->alloc(sizeof(double) * ksplit * Mp * ncols, &ws));
   double* rpart = nullptr;
   if (fuse != nullptr && ksplit == 1) {  // the epilogue sees final values: fuse the range sums
-    NNV_TRY(ctx->alloc(sizeof(double) * 4 * ldc * tiles_n, &fuse->part));
+    NNV_TRY(ctx->alloc(sizeof(double) * 4 * ldc * (tiles_n + fuse->extra_chunks), &fuse->part));
     fuse->chunks = tiles_n;
     rpart = fuse->part->as<double>();
   }
@@ -266,7 +277,7 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)grid_x, (unsigned)ksplit), dim3(64 * WR * WC), 0,
                      ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)tiles_n,
                      (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
-                     fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart);
+                     fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, colmap);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, 2.0 * (double)Mp * (double)Kp * (double)ncols));
   if (ksplit > 1) {
     const int64_t total = Mp * ncols;
@@ -278,14 +289,15 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
 }
 
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C, int64_t ldc,
-                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse) {
+                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse, const int32_t* colmap) {
   if (Mp % 16 || Kp % 16 || lda % 2 || ldb % 2 || Mp > lda || Kp > ldb || Mp > ldc)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: GEMM operands violate the padding contract");
   if (Mp >= (int64_t(1) << 31) || Kp >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large");
   if (ncols == 0) return NNVHIP_OK;
   // Tile choice: the largest tile that still yields a few blocks per CU; skinny outputs (the last
   // layer has 10 rows) get a 16-row tile.  K must be a multiple of the K-tile (16 or 32).
-#define NNV_GEMM(TM, TN, WR, WC, KT) launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias, fuse)
+#define NNV_GEMM(TM, TN, WR, WC, KT) \
+  launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias, fuse, colmap)
   const int64_t kCUs = 256;
   if (Mp <= 16) return NNV_GEMM(16, 64, 1, 4, 16);
   if (Mp <= 32) return NNV_GEMM(32, 128, 1, 4, 16);

@@ -148,6 +148,14 @@ struct nnvhip_star {
   // filled for sets produced by the ReLU step
   int64_t n_inactive = -1;
   int64_t n_crossing = -1;
+  // Structure hint for the FC affine map: columns [oh_from, n] of V are scaled unit vectors,
+  // column j = oh_scale[r] * e_r with r = oh_idx[j - oh_from] (oh_scale == null: scale 1).  Box stars
+  // (all generators) and ReLU outputs (the appended columns) carry it; 0 = no such block.  V itself is
+  // always fully materialised, the hint only lets W*V skip products with structural zeros.
+  int64_t oh_from = 0;
+  const int32_t* oh_idx = nullptr;
+  const double* oh_scale = nullptr;
+  nnvhip::BufRef oh_idx_buf, oh_scale_buf;
 };
 
 struct nnvhip_fc {
@@ -184,14 +192,18 @@ void release_all(std::vector<nnvhip_star*>& v);
 struct RangeFuse {
   const double* plb = nullptr;  // predicate bounds of the set's n = ncols - 1 generator columns
   const double* pub = nullptr;
+  int64_t extra_chunks = 0;     // in: room to leave behind the GEMM's chunks (for launch_gather_columns)
   BufRef part;                  // out: partial sums (allocated by the launcher)
   int64_t chunks = 0;           // out: number of column tiles; 0 = not fused (split-K was used)
 };
 
 // gemm.hip: C(Mp x ncols, ldc) = A(Mp x Kp, lda) * B(Kp x ncols, ldb); bias (Mp) is added to
 // column 0 when non-null.  Mp, Kp multiples of 16; padding rows of A and B are zero.
+// colmap (optional): compact column t of the product reads column colmap[t] of B and writes column
+// colmap[t] of C (dense columns scattered through an arena of sets); not combined with fuse.
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
-                int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse = nullptr);
+                int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse = nullptr,
+                const int32_t* colmap = nullptr);
 // Adds bias to the centre columns of sets 1..count-1 of an arena (set 0 is fused in the GEMM).
 int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t count, const double* bias,
                         int64_t Mp);
@@ -203,6 +215,21 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t
 
 // ranges.hip
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s);
+// W * (scaled unit vectors): out(:, j) = W(:, idx[j]) * scale[idx[j]] for the one-hot column block of
+// every set (ranges.hip).  With part != null (one set) the four range sums of these columns are left
+// as `chunks` further chunks at part + part_chunk0, in the layout finalize_fused_ranges reads.
+struct GatherSet {
+  const int32_t* idx;
+  const double* scale;  // by row index, or null
+  double* out;          // first one-hot column of the output set
+  const double* plb;    // predicate bounds of these columns (fused range sums only)
+  const double* pub;
+  int32_t m;
+  int32_t pad_;
+};
+int64_t gather_chunks(int64_t Mp, int64_t m);
+int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t Mp, int64_t ldout, int64_t count,
+                          const GatherSet* sets, double* part, int64_t part_chunk0, int64_t chunks);
 // Turns the per-column-tile partial sums a fused GEMM left behind into the set's cached lb/ub.
 int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks);
 

@@ -135,6 +135,133 @@ __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __re
   }
 }
 
+
+// ---- W * (block of scaled unit vectors) -------------------------------------------------------
+// Column j of the block is scale * e_r, so the product column is W(:, r) * scale: a gather of W's
+// columns.  0 + w*scale reproduces what the dense accumulation (starting from +0) leaves, bit for bit.
+// Same geometry as the range pass, and with part != null it also leaves that pass's four partial
+// sums for its columns.
+struct GatherArgs {
+  const double* W;
+  int64_t ldw, ldout;
+  double* part;  // [chunks][4][ldout] or null
+  int32_t cols_per_chunk;
+  int32_t pad_;
+};
+
+__global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const GatherSet* __restrict__ table, GatherSet one,
+                                                                         GatherArgs a) {
+  const GatherSet d = table ? table[blockIdx.z] : one;
+  const int chunk = blockIdx.y;
+  const int j0 = chunk * a.cols_per_chunk;
+  if (j0 >= d.m && a.part == nullptr) return;
+  const int j1 = min(d.m, j0 + a.cols_per_chunk);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t r0 = (int64_t)blockIdx.x * kRowsPerWave + 2 * lane;
+  const bool active = r0 < a.ldout;
+  double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
+  if (active) {
+    for (int jb = j0 + 4 * wave; jb < j1; jb += 4 * kRangeWaves) {
+      double2 v[4];
+      double sc[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        v[u] = make_double2(0.0, 0.0);
+        sc[u] = 1.0;
+        if (jb + u < j1) {
+          const int src = d.idx[jb + u];
+          if (d.scale != nullptr) sc[u] = d.scale[src];
+          v[u] = *reinterpret_cast<const double2*>(a.W + r0 + (int64_t)src * a.ldw);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = jb + u;
+        if (j >= j1) break;
+        double2 o;
+        o.x = __dadd_rn(0.0, __dmul_rn(v[u].x, sc[u]));
+        o.y = __dadd_rn(0.0, __dmul_rn(v[u].y, sc[u]));
+        *reinterpret_cast<double2*>(d.out + r0 + (int64_t)j * a.ldout) = o;
+        if (a.part != nullptr) {
+          const double pl = d.plb[j], pu = d.pub[j];
+          const double px = fmax(o.x, 0.0), nx = fmin(o.x, 0.0);
+          const double py = fmax(o.y, 0.0), ny = fmin(o.y, 0.0);
+          xmin1.x = fma(px, pl, xmin1.x);
+          xmin1.y = fma(py, pl, xmin1.y);
+          xmax1.x = fma(px, pu, xmax1.x);
+          xmax1.y = fma(py, pu, xmax1.y);
+          xmin2.x = fma(nx, pu, xmin2.x);
+          xmin2.y = fma(ny, pu, xmin2.y);
+          xmax2.x = fma(nx, pl, xmax2.x);
+          xmax2.y = fma(ny, pl, xmax2.y);
+        }
+      }
+    }
+  }
+  if (a.part == nullptr) return;
+  __shared__ double2 red[kRangeWaves][4][64];
+  if (wave > 0) {
+    red[wave][0][lane] = xmin1;
+    red[wave][1][lane] = xmin2;
+    red[wave][2][lane] = xmax1;
+    red[wave][3][lane] = xmax2;
+  }
+  __syncthreads();
+  if (wave == 0 && active) {
+    for (int w = 1; w < kRangeWaves; ++w) {
+      xmin1.x += red[w][0][lane].x;
+      xmin1.y += red[w][0][lane].y;
+      xmin2.x += red[w][1][lane].x;
+      xmin2.y += red[w][1][lane].y;
+      xmax1.x += red[w][2][lane].x;
+      xmax1.y += red[w][2][lane].y;
+      xmax2.x += red[w][3][lane].x;
+      xmax2.y += red[w][3][lane].y;
+    }
+    double* p = a.part + ((int64_t)chunk * 4) * a.ldout + r0;
+    *reinterpret_cast<double2*>(p) = xmin1;
+    *reinterpret_cast<double2*>(p + a.ldout) = xmin2;
+    *reinterpret_cast<double2*>(p + 2 * a.ldout) = xmax1;
+    *reinterpret_cast<double2*>(p + 3 * a.ldout) = xmax2;
+  }
+}
+
+// Column chunks of the gather for one set of m one-hot columns: enough blocks to cover the chip.
+int64_t gather_chunks(int64_t Mp, int64_t m) {
+  if (m <= 0) return 0;
+  const int64_t row_blocks = ceil_div(Mp, kRowsPerWave);
+  return std::max<int64_t>(1, std::min<int64_t>(ceil_div(1024, row_blocks), ceil_div(m, 4 * kRangeWaves)));
+}
+
+int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t Mp, int64_t ldout, int64_t count,
+                          const GatherSet* sets, double* part, int64_t part_chunk0, int64_t chunks) {
+  if (count <= 0) return NNVHIP_OK;
+  if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  int64_t max_m = 0;
+  for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, sets[i].m);
+  if (max_m == 0) return NNVHIP_OK;
+  const int64_t row_blocks = ceil_div(ldout, kRowsPerWave);
+  if (part == nullptr) chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(max_m, 4 * kRangeWaves)));
+  GatherArgs a{};
+  a.W = W;
+  a.ldw = ldw;
+  a.ldout = ldout;
+  a.part = part ? part + part_chunk0 * 4 * ldout : nullptr;
+  a.cols_per_chunk = (int32_t)ceil_div(max_m, chunks);
+  const GatherSet* table = nullptr;
+  BufRef tab;
+  if (count > 1) {
+    NNV_TRY(ctx->upload(sets, sizeof(GatherSet) * count, &tab));
+    table = tab->as<GatherSet>();
+  }
+  (void)Mp;
+  hipLaunchKernelGGL(gather_columns_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
+                     dim3(64 * kRangeWaves), 0, ctx->stream, table, sets[0], a);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   // sets that already carry ranges are skipped
   std::vector<nnvhip_star*> todo;

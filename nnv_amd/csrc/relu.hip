@@ -701,6 +701,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     o->pub = d.pub_out;
     o->n_inactive = counts[2 * i + 1];
     o->n_crossing = d.m;
+    if (d.m > 0) {  // the appended columns are the unit vectors of the crossing neurons
+      o->oh_from = in[i]->n + 1;
+      o->oh_idx_buf = idx_bufs[i];
+      o->oh_idx = idx_bufs[i]->as<int32_t>();
+    }
     if (d.m > 0) {
       auto node = std::make_shared<ConsNode>();
       node->prev = in[i]->cons;
