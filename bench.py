@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by the 1 GiB copy kernel of the same run (profiles/<workload>_hbm_traffic.md): (read, write) MiB
 # averaged over the three launches of a step (the 64x64, 64x96 and 128x80 tile instantiations)
-MEASURED_TRAFFIC_MIB = {("cfg2_fc_784_1024x3_10", "gemm_f64_kernel"): (51.30, 12.36)}
+MEASURED_TRAFFIC_MIB = {("cfg2_fc_784_1024x3_10", "gemm_f64_kernel", "dense"): (51.30, 12.36)}
 
 
 def layer_shapes(reach_set):
@@ -53,12 +53,16 @@ def main():
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--method", default="relax-star-area")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--dense", action="store_true",
+                    help="run every FC layer as the full dense contraction (no skipping of structural zeros)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (sets shard across GPUs without communication; "
                  "that path is not built) - use --gpus 1")
 
+    if args.dense:
+        os.environ["NNVHIP_DENSE_AFFINE"] = "1"  # read once by the library
     import nnv_amd
     from nnv_amd.configs import count_updates, device_input_sets, make_config, make_extended_cnn
 
@@ -107,14 +111,15 @@ def main():
         return acc / reps
 
     per_layer = timed_pass(1)          # NN.reachTime-style device time per layer
-    for grp in range(5):
+    for grp in range(6):
         ctx.kernel_time(grp)
     timed_pass(2)                      # per-kernel event pairs
-    gemm_ms, gemm_launches, _ = ctx.kernel_time(0)
-    conv_ms, conv_launches, _ = ctx.kernel_time(1)
+    gemm_ms, gemm_launches, gemm_work = ctx.kernel_time(0)
+    conv_ms, conv_launches, conv_work = ctx.kernel_time(1)
     rng_ms, rng_launches, rng_bytes = ctx.kernel_time(2)
     app_ms, app_launches, app_bytes = ctx.kernel_time(3)
     row_ms, row_launches, row_bytes = ctx.kernel_time(4)
+    gat_ms, gat_launches, gat_bytes = ctx.kernel_time(5)
 
     # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
     gemm_flop = conv_flop = 0.0
@@ -161,37 +166,42 @@ def main():
         layer_report.append(entry)
         prev_sets = outs
 
-    def mfma_roofline(name, flop_per_step, ms_total, launches):
-        ach = flop_per_step * reps / (ms_total * 1e-3) / 1e12
+    # MFMA kernels: flop the kernel executed (the library's own count for its launches: products with
+    # structural zeros that the FC map skips are not counted) over the kernels' HIP-event durations;
+    # dense_equivalent = the dense count of the same layers, 2*M*K*(n+1), as the reference executes them
+    def mfma_roofline(name, work_total, dense_flop_per_step, ms_total, launches):
+        ach = work_total / (ms_total * 1e-3) / 1e12
         return {"kernel": name, "bound": "mfma", "achieved": round(ach, 3), "peak": FP64_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(ach / FP64_MFMA_PEAK_TFLOPS, 4), "traffic": None,
                 "launches_per_step": launches // reps, "avg_launch_ms": round(ms_total / launches, 5),
-                "flop_per_launch": flop_per_step * reps / launches}
+                "flop_per_launch": work_total / launches,
+                "dense_equivalent_flop_per_step": dense_flop_per_step,
+                "ms_per_step": round(ms_total / reps, 5)}
 
-    if conv_launches and conv_ms >= gemm_ms:
-        roofline = mfma_roofline("conv2d_f64_kernel", conv_flop, conv_ms, conv_launches)
-        if gemm_launches:
-            roofline["fc_gemm"] = mfma_roofline("gemm_f64_kernel", gemm_flop, gemm_ms, gemm_launches)
-    elif gemm_launches:
-        roofline = mfma_roofline("gemm_f64_kernel", gemm_flop, gemm_ms, gemm_launches)
-        if conv_launches:
-            roofline["conv"] = mfma_roofline("conv2d_f64_kernel", conv_flop, conv_ms, conv_launches)
-    else:
-        achieved = relu_bytes / (relu_ms * 1e-3) / 1e9
-        roofline = {"kernel": "relu step", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None}
-    # the HBM-bound kernels: algorithmic bytes over their own HIP-event durations
-    hbm = {}
-    for name, ms_, n_, b_ in (("ranges_partial_kernel", rng_ms, rng_launches, rng_bytes),
-                              ("relu_apply_kernel", app_ms, app_launches, app_bytes),
-                              ("row-wise affine layers (rowmap/avgpool/permute kernels)", row_ms, row_launches, row_bytes)):
-        if n_:
-            g = b_ / (ms_ * 1e-3) / 1e9
-            hbm[name] = {"bound": "hbm", "achieved": round(g, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(g / HBM_PEAK_GBS, 4), "launches_per_step": n_ // reps,
-                         "avg_launch_ms": round(ms_ / n_, 5)}
-    roofline["hbm_kernels"] = hbm
-    t = MEASURED_TRAFFIC_MIB.get((cfg["name"], roofline["kernel"]))
+    def hbm_roofline(name, ms_, n_, b_):
+        g = b_ / (ms_ * 1e-3) / 1e9
+        return {"kernel": name, "bound": "hbm", "achieved": round(g, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(g / HBM_PEAK_GBS, 4), "traffic": None, "launches_per_step": n_ // reps,
+                "avg_launch_ms": round(ms_ / n_, 5), "bytes_per_launch": b_ / n_, "ms_per_step": round(ms_ / reps, 5)}
+
+    # the dominant kernel group of a reach, by summed kernel time
+    groups = []
+    if gemm_launches:
+        groups.append((gemm_ms, mfma_roofline("gemm_f64_kernel", gemm_work, gemm_flop, gemm_ms, gemm_launches)))
+    if conv_launches:
+        groups.append((conv_ms, mfma_roofline("conv2d_f64_kernel", conv_work, conv_flop, conv_ms, conv_launches)))
+    if rng_launches:
+        groups.append((rng_ms, hbm_roofline("ranges_partial_kernel", rng_ms, rng_launches, rng_bytes)))
+    if app_launches:
+        groups.append((app_ms, hbm_roofline("relu_apply_kernel", app_ms, app_launches, app_bytes)))
+    if row_launches:
+        groups.append((row_ms, hbm_roofline("row-wise affine layers (rowmap/avgpool/permute kernels)", row_ms, row_launches, row_bytes)))
+    if gat_launches:
+        groups.append((gat_ms, hbm_roofline("gather_columns_kernel", gat_ms, gat_launches, gat_bytes)))
+    groups.sort(key=lambda g: -g[0])
+    roofline = dict(groups[0][1])
+    roofline["other_kernels"] = [g[1] for g in groups[1:]]
+    t = MEASURED_TRAFFIC_MIB.get((cfg["name"], roofline["kernel"], "dense" if args.dense else "structured"))
     if t is not None and args.method == "relax-star-area":
         roofline["traffic"] = round((t[0] + t[1]) * 1048576.0)
     if relu_ms > 0:
@@ -249,6 +259,7 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": cfg["name"], "reach_method": args.method, "relax_factor": 1,
+                   "fc_affine_map": "dense" if args.dense else "structural zeros skipped (one-hot generator columns, reset rows); exact",
                    "sets": len(dev_in) if isinstance(dev_in, list) else 1,
                    "updates_per_step": updates,
                    "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, list) else None},

@@ -764,6 +764,18 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.m = (int32_t)(nc - dense[i]);
       g.pad_ = 0;
     }
+    // Rows of the dense columns that the ReLU step reset to zero need no contraction either: the
+    // GEMM then runs over the kept rows only (used when that at least halves K).
+    auto rows_of = [&](int64_t i, GemmRows* r, int64_t* kp) {
+      *kp = fc->Kp;
+      if (dense_only || in[i]->n_kept < 0 || in[i]->kept_idx == nullptr) return false;
+      const int64_t k = std::max<int64_t>(round_up(in[i]->n_kept, kLdAlign), kLdAlign);
+      if (2 * k > fc->Kp) return false;
+      r->kmap = in[i]->kept_idx;
+      r->flop = 2.0 * (double)fc->Mp * (double)k * (double)dense[i];
+      *kp = k;
+      return true;
+    };
     if (count == 1) {
       // one set: the GEMM epilogue also leaves the partial sums of Star.estimateRanges, so the
       // output set carries its ranges without another pass over V
@@ -772,30 +784,70 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       fuse.pub = outs[0]->pub;
       const int64_t gch = gather_chunks(fc->Mp, gs[0].m);
       fuse.extra_chunks = gch;
-      st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], fc->Kp, bias, &fuse);
+      GemmRows rows;
+      int64_t kp = fc->Kp;
+      const bool compact = rows_of(0, &rows, &kp);
+      st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
+                       compact ? &rows : nullptr);
       const bool fused = st == NNVHIP_OK && fuse.chunks > 0;
       if (st == NNVHIP_OK && gs[0].m > 0)
         st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? fuse.part->as<double>() : nullptr,
                                    fuse.chunks, gch);
       if (st == NNVHIP_OK && fused) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0));
     } else if (contig) {
-      BufRef cmap;
-      const int32_t* colmap = nullptr;
-      if (any_onehot) {  // the dense columns of the sets, as positions in the (shared) arena layout
+      // one launch for the whole array.  With structure to exploit, every set's dense columns are cut
+      // into tiles of 128 that carry their own description (row list, position in the arena).
+      bool any_rows = false;
+      std::vector<GemmRows> rws((size_t)count);
+      std::vector<int64_t> kps((size_t)count);
+      for (int64_t i = 0; i < count; ++i) any_rows = rows_of(i, &rws[i], &kps[i]) || any_rows;
+      if (any_onehot && !any_rows) {
+        // all sets contract over every row: their dense columns are simply listed (tiles may span sets)
         if (cols >= (int64_t(1) << 31)) st = NNVHIP_ERR_SHAPE;
         std::vector<int32_t> map;
         map.reserve((size_t)total_dense);
         int64_t off = 0;
-        for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
+        for (int64_t i = 0; i < count; ++i) {
           for (int64_t j = 0; j < dense[i]; ++j) map.push_back((int32_t)(off + j));
           off += in[i]->n + 1;
         }
+        BufRef cmap;
         if (st == NNVHIP_OK) st = c->upload(map.data(), sizeof(int32_t) * map.size(), &cmap);
-        if (st == NNVHIP_OK) colmap = cmap->as<int32_t>();
+        if (st == NNVHIP_OK) {
+          GemmRows rows;
+          rows.colmap = cmap->as<int32_t>();
+          st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, total_dense, fc->Kp, bias,
+                           nullptr, &rows);
+        }
+      } else if (any_rows) {
+        std::vector<GemmSeg> segs;
+        GemmRows rows;
+        const int64_t tn = gemm_seg_cols(fc->Mp);
+        rows.seg_cols = (int32_t)tn;
+        int64_t off = 0, kp_max = kLdAlign;
+        for (int64_t i = 0; i < count; ++i) {
+          for (int64_t j = 0; j < dense[i]; j += tn) {
+            GemmSeg sg;
+            sg.kmap = rws[i].kmap;
+            sg.col_base = off + j;
+            sg.kp = (int32_t)kps[i];
+            sg.valid = (int32_t)std::min<int64_t>(tn, dense[i] - j);
+            segs.push_back(sg);
+          }
+          rows.flop += 2.0 * (double)fc->Mp * (double)kps[i] * (double)dense[i];
+          kp_max = std::max(kp_max, kps[i]);
+          off += in[i]->n + 1;
+        }
+        BufRef dsegs;
+        st = c->upload(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
+        if (st == NNVHIP_OK) {
+          rows.segs = dsegs->as<GemmSeg>();
+          st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, tn * (int64_t)segs.size(),
+                           kp_max, bias, nullptr, &rows);
+        }
+      } else {
+        st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols, fc->Kp, bias);
       }
-      if (st == NNVHIP_OK)
-        st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, any_onehot ? total_dense : cols,
-                         fc->Kp, bias, nullptr, colmap);
       if (st == NNVHIP_OK && bias && count > 1) {
         std::vector<double*> centres(count - 1);
         for (int64_t i = 1; i < count; ++i) centres[i - 1] = outs[i]->V;
@@ -807,7 +859,11 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, count, gs.data(), nullptr, 0, 0);
     } else {
       for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
-        st = launch_gemm(c, Wd, fc->Mp, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, fc->Mp, dense[i], fc->Kp, bias);
+        GemmRows rows;
+        int64_t kp = fc->Kp;
+        const bool compact = rows_of(i, &rows, &kp);
+        st = launch_gemm(c, Wd, fc->Mp, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, fc->Mp, dense[i], kp, bias, nullptr,
+                         compact ? &rows : nullptr);
         if (st == NNVHIP_OK && gs[i].m > 0)
           st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[i]->ld, 1, &gs[i], nullptr, 0, 0);
       }

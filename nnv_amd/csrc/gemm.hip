@@ -15,7 +15,9 @@ namespace nnvhip {
 
 // TM x TN output tile per block of WR x WC waves, each wave owning
 // (TM/WR) x (TN/WC) = (16*FM) x (16*FN).
-template <int TM, int TN, int WR, int WC, int KT>
+// MAPPED = false: the plain product.  MAPPED = true additionally honours a row list (kmap), a per-tile
+// segment table (segs) and a column map (colmap); kept apart so that the plain kernel pays nothing.
+template <int TM, int TN, int WR, int WC, int KT, bool MAPPED>
 __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __restrict__ A, int64_t lda,
                                                         const double* __restrict__ B, int64_t ldb,
                                                         double* __restrict__ C, int64_t ldc, int Mp, int64_t ncols,
@@ -25,6 +27,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
                                                         const double* __restrict__ plb,
                                                         const double* __restrict__ pub,
                                                         double* __restrict__ rpart,
+                                                        const int32_t* __restrict__ kmap,
+                                                        const GemmSeg* __restrict__ segs,
                                                         const int32_t* __restrict__ colmap) {
   constexpr int NT = 64 * WR * WC;  // threads per block
   constexpr int FM = TM / WR / 16;
@@ -52,6 +56,17 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   if (mt >= tiles_m || nt >= tiles_n) return;
   const int m0 = mt * TM;
   const int64_t n0 = nt * TN;
+  // Row-compacted contraction: kmap lists the rows of B (= columns of A) that can be non-zero, padded
+  // to whole K-tiles with -1; with a segment table every column tile has its own list (one per set).
+  int64_t col_base = n0;       // column of B and C behind the tile's first column
+  int64_t col_end = ncols;     // first column past the valid ones, in the same numbering as col_base
+  if (MAPPED && segs != nullptr) {
+    const GemmSeg sg = segs[nt];
+    kmap = sg.kmap;
+    Kp = sg.kp;
+    col_base = sg.col_base;
+    col_end = sg.col_base + sg.valid;
+  }
 
   // ---- global -> register staging ----------------------------------------------------------
   constexpr int A_VEC = TM * KT / 2;           // double2 elements in a W tile
@@ -59,12 +74,12 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   constexpr int B_VEC = TN * KT / 2;
   constexpr int B_PASS = (B_VEC + NT - 1) / NT;
   double2 ra[A_PASS], rb[B_PASS];
-  // column of B behind each staged element (identity unless the dense columns sit scattered in an arena)
+  // column of B behind each staged element (-1: none)
   int64_t bcol[B_PASS];
 #pragma unroll
   for (int p = 0; p < B_PASS; ++p) {
-    const int64_t col = n0 + (tid + p * NT) / (KT / 2);
-    bcol[p] = (colmap != nullptr && col < ncols) ? (int64_t)colmap[col] : col;
+    const int64_t col = col_base + (tid + p * NT) / (KT / 2);
+    bcol[p] = col < col_end ? ((MAPPED && colmap != nullptr) ? (int64_t)colmap[col] : col) : -1;
   }
 
   auto load_tiles = [&](int k0) {
@@ -75,7 +90,10 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
       int k = idx / (TM / 2);
       int row = m0 + 2 * i2;
       double2 v = make_double2(0.0, 0.0);
-      if (idx < A_VEC && row < Mp) v = *reinterpret_cast<const double2*>(A + row + (int64_t)(k0 + k) * lda);
+      if (idx < A_VEC && row < Mp) {
+        const int kk = (MAPPED && kmap != nullptr) ? kmap[k0 + k] : k0 + k;
+        if (kk >= 0) v = *reinterpret_cast<const double2*>(A + row + (int64_t)kk * lda);
+      }
       ra[p] = v;
     }
 #pragma unroll
@@ -83,9 +101,16 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
       int idx = tid + p * NT;
       int k2 = idx % (KT / 2);
       int j = idx / (KT / 2);
-      int64_t col = n0 + j;
       double2 v = make_double2(0.0, 0.0);
-      if (idx < B_VEC && col < ncols) v = *reinterpret_cast<const double2*>(B + (k0 + 2 * k2) + bcol[p] * ldb);
+      if (idx < B_VEC && bcol[p] >= 0) {
+        if (MAPPED && kmap != nullptr) {
+          const int ka = kmap[k0 + 2 * k2], kb = kmap[k0 + 2 * k2 + 1];
+          if (ka >= 0) v.x = B[ka + bcol[p] * ldb];
+          if (kb >= 0) v.y = B[kb + bcol[p] * ldb];
+        } else {
+          v = *reinterpret_cast<const double2*>(B + (k0 + 2 * k2) + bcol[p] * ldb);
+        }
+      }
       rb[p] = v;
     }
   };
@@ -202,11 +227,11 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         int64_t col = n0 + wc * (TN / WC) + j * 16 + lcol + 4 * r;
-        if (col < ncols) {
+        const int64_t ccol = col_base + (col - n0);
+        if (ccol < col_end) {
           double v = acc[i][j][r];
-          if (bias != nullptr && col == 0) v = v + bias[row];
-          const int64_t ccol = (colmap != nullptr && ksplit == 1) ? (int64_t)colmap[col] : col;
-          C[row + ccol * ldc] = v;
+          if (bias != nullptr && ccol == 0) v = v + bias[row];
+          C[row + ((MAPPED && colmap != nullptr) ? (int64_t)colmap[ccol] : ccol) * ldc] = v;
         }
       }
     }
@@ -230,7 +255,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __rest
 template <int TM, int TN, int WR, int WC, int KT>
 static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
                       int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse,
-                      const int32_t* colmap) {
+                      const GemmRows* rows) {
   int64_t tiles_m = ceil_div(Mp, TM);
   int64_t tiles_n = ceil_div(ncols, TN);
   int64_t blocks = tiles_m * tiles_n;
@@ -263,7 +288,9 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   int64_t ksplit = 1;
   if (blocks < 128 && nk >= 8) ksplit = std::min<int64_t>(std::min<int64_t>(16, nk / 4), ceil_div(512, blocks));
   if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
-  if (colmap != nullptr) ksplit = 1;  // the split-K workspace is compact; mapped launches are large anyway
+  if (rows != nullptr) ksplit = 1;  // the split-K reduction knows nothing of row or column maps
+  if (rows != nullptr && rows->segs != nullptr && rows->seg_cols != TN)
+    NNV_FAIL(NNVHIP_ERR_ARG, "internal: segment table built for another tile width");
   BufRef ws;
   if (ksplit > 1) NNV_TRY(ctx->alloc(sizeof(double) * ksplit * Mp * ncols, &ws));
   double* rpart = nullptr;
@@ -274,11 +301,17 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   }
   const bool timed = ctx->kernel_timing && TM >= 64;
   NNV_TRY(ctx->kernel_timer_begin(timed));
-  hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT>), dim3((unsigned)grid_x, (unsigned)ksplit), dim3(64 * WR * WC), 0,
-                     ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m, (int)tiles_n,
-                     (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
-                     fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, colmap);
-  NNV_TRY(ctx->kernel_timer_end(timed, 0, 2.0 * (double)Mp * (double)Kp * (double)ncols));
+  if (rows != nullptr)
+    hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT, true>), dim3((unsigned)grid_x, (unsigned)ksplit),
+                       dim3(64 * WR * WC), 0, ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
+                       (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
+                       fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, rows->kmap, rows->segs, rows->colmap);
+  else
+    hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT, false>), dim3((unsigned)grid_x, (unsigned)ksplit),
+                       dim3(64 * WR * WC), 0, ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
+                       (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
+                       fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, nullptr, nullptr, nullptr);
+  NNV_TRY(ctx->kernel_timer_end(timed, 0, rows && rows->flop > 0.0 ? rows->flop : 2.0 * (double)Mp * (double)Kp * (double)ncols));
   if (ksplit > 1) {
     const int64_t total = Mp * ncols;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream,
@@ -288,8 +321,10 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   return NNVHIP_OK;
 }
 
+int gemm_seg_cols(int64_t Mp) { return Mp <= 16 ? 64 : 128; }
+
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C, int64_t ldc,
-                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse, const int32_t* colmap) {
+                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse, const GemmRows* rows) {
   if (Mp % 16 || Kp % 16 || lda % 2 || ldb % 2 || Mp > lda || Kp > ldb || Mp > ldc)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: GEMM operands violate the padding contract");
   if (Mp >= (int64_t(1) << 31) || Kp >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large");
@@ -297,7 +332,7 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
   // Tile choice: the largest tile that still yields a few blocks per CU; skinny outputs (the last
   // layer has 10 rows) get a 16-row tile.  K must be a multiple of the K-tile (16 or 32).
 #define NNV_GEMM(TM, TN, WR, WC, KT) \
-  launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias, fuse, colmap)
+  launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias, fuse, rows)
   const int64_t kCUs = 256;
   if (Mp <= 16) return NNV_GEMM(16, 64, 1, 4, 16);
   if (Mp <= 32) return NNV_GEMM(32, 128, 1, 4, 16);
@@ -322,6 +357,7 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
       best_cost = cost;
     }
   }
+  if (rows != nullptr && rows->segs != nullptr) return NNV_GEMM(128, 128, 2, 4, 16);  // see gemm_seg_cols
   if (const char* e = getenv("NNVHIP_GEMM_TILE")) {  // tuning knob: "TMxTN" of one of the shapes above
     for (int i = 0; i < (int)(sizeof(shapes) / sizeof(shapes[0])); ++i)
       if (std::to_string(shapes[i].tm) + "x" + std::to_string(shapes[i].tn) == e) best = i;

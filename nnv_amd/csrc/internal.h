@@ -110,11 +110,12 @@ struct nnvhip_ctx {
   hipEvent_t kev0 = nullptr, kev1 = nullptr;
   // [0] dense MFMA GEMM (tiles of at least 64 rows), [1] implicit-GEMM convolution (work = flop),
   // [2] estimateRanges column pass, [3] ReLU apply pass, [4] row-wise affine layers (batch
-  // normalisation, input normalisation, average pooling, flatten) (work = algorithmic bytes)
-  static constexpr int kKernelGroups = 5;
-  double kern_ms[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0};
-  int64_t kern_launches[kKernelGroups] = {0, 0, 0, 0, 0};
-  double kern_flop[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0};
+  // normalisation, input normalisation, average pooling, flatten), [5] gather of W's columns for the
+  // one-hot generator columns of an FC layer (work = algorithmic bytes)
+  static constexpr int kKernelGroups = 6;
+  double kern_ms[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+  int64_t kern_launches[kKernelGroups] = {0, 0, 0, 0, 0, 0};
+  double kern_flop[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
   int kernel_timer_begin(bool on);
   int kernel_timer_end(bool on, int which, double flop);
 
@@ -156,6 +157,12 @@ struct nnvhip_star {
   const int32_t* oh_idx = nullptr;
   const double* oh_scale = nullptr;
   nnvhip::BufRef oh_idx_buf, oh_scale_buf;
+  // Second hint, set by the ReLU step: only the rows kept_idx[0..n_kept) (ascending; the list is padded
+  // with -1 up to a multiple of 16 and at least 16 entries) of the columns before the one-hot block can
+  // be non-zero -- every other row was reset.  n_kept < 0 = no such knowledge.
+  int64_t n_kept = -1;
+  const int32_t* kept_idx = nullptr;
+  nnvhip::BufRef kept_buf;
 };
 
 struct nnvhip_fc {
@@ -199,11 +206,30 @@ struct RangeFuse {
 
 // gemm.hip: C(Mp x ncols, ldc) = A(Mp x Kp, lda) * B(Kp x ncols, ldb); bias (Mp) is added to
 // column 0 when non-null.  Mp, Kp multiples of 16; padding rows of A and B are zero.
-// colmap (optional): compact column t of the product reads column colmap[t] of B and writes column
-// colmap[t] of C (dense columns scattered through an arena of sets); not combined with fuse.
+// rows (optional): contraction over a subset of the K rows.  kmap lists the rows of B (= columns of A)
+// that can be non-zero, padded with -1 to a multiple of 16; Kp passed to launch_gemm is then the padded
+// length of that list.  With segs (arrays of sets), column tile t of seg_cols = 128 columns has its own
+// description: its row list (null = all rows), the arena column of its first column and how many of
+// its columns exist; ncols is then seg_cols * (number of tiles), seg_cols = gemm_seg_cols(Mp).
+struct GemmSeg {
+  const int32_t* kmap;
+  int64_t col_base;
+  int32_t kp;
+  int32_t valid;
+};
+struct GemmRows {
+  const int32_t* kmap = nullptr;
+  const GemmSeg* segs = nullptr;
+  // without segs: product column t reads column colmap[t] of B and writes column colmap[t] of C
+  // (columns picked from an arena of sets that share the row list)
+  const int32_t* colmap = nullptr;
+  int32_t seg_cols = 128;
+  double flop = 0.0;  // flop actually executed (for the kernel timers)
+};
+int gemm_seg_cols(int64_t Mp);
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
                 int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse = nullptr,
-                const int32_t* colmap = nullptr);
+                const GemmRows* rows = nullptr);
 // Adds bias to the centre columns of sets 1..count-1 of an arena (set 0 is fused in the GEMM).
 int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t count, const double* bias,
                         int64_t Mp);

@@ -255,9 +255,14 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
     NNV_TRY(ctx->upload(sets, sizeof(GatherSet) * count, &tab));
     table = tab->as<GatherSet>();
   }
-  (void)Mp;
+  // algorithmic HBM bytes: every output column written once, W read once (its columns are re-read
+  // from cache)
+  double bytes = 8.0 * (double)Mp * (double)ldw;
+  for (int64_t i = 0; i < count; ++i) bytes += 8.0 * (double)Mp * (double)sets[i].m;
+  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL(gather_columns_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
                      dim3(64 * kRangeWaves), 0, ctx->stream, table, sets[0], a);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }

@@ -35,7 +35,8 @@ struct ReluDesc {
   double* key;         // sort keys, ascending-index order
   int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
-  int32_t* blk_counts; // multi-block classification: per 1024-row block {crossing, inactive}
+  int32_t* keep_idx;   // rows left untouched (active neurons), ascending, then -1 up to a multiple of 16
+  int32_t* blk_counts; // multi-block classification: per 1024-row block {crossing, inactive, kept}
   int32_t* mailbox;    // host-pinned {m, inactive, seq}; null = counts are fetched by a copy instead
   int32_t mailbox_seq;
   int32_t pad2_;
@@ -236,10 +237,11 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   const int wave = tid >> 6;
   __shared__ int wcross[16];
   __shared__ int winact[16];
+  __shared__ int wkeep[16];
   __shared__ double skey[SORT_CAP > 0 ? SORT_CAP : 1];
   __shared__ int sidx[SORT_CAP > 0 ? SORT_CAP : 1];
   static_assert(sizeof(double) == sizeof(long long), "keys are sorted through their bit patterns");
-  int base = 0, inact_total = 0;
+  int base = 0, inact_total = 0, keep_base = 0;
   int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
   for (int r0 = 0; r0 < d.N; r0 += 1024) {
     const int r = r0 + tid;
@@ -248,21 +250,29 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     const double u = valid ? d.ub[r] : 1.0;
     const bool inactive = valid && (u <= 0.0);              // map1 = find(ub <= 0)
     const bool crossing = valid && (l < 0.0) && (u > 0.0);  // map2 = find(lb < 0 & ub > 0)
+    const bool kept = valid && !inactive && !crossing;
     const unsigned long long bc = __ballot(crossing);
     const unsigned long long bi = __ballot(inactive);
+    const unsigned long long bk = __ballot(kept);
     if (lane == 0) {
       wcross[wave] = __popcll(bc);
       winact[wave] = __popcll(bi);
+      wkeep[wave] = __popcll(bk);
     }
     __syncthreads();
-    int woff = 0, tot = 0, itot = 0;
+    int woff = 0, tot = 0, itot = 0, koff = 0, ktot = 0;
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
       const int c = wcross[w];
       woff += w < wave ? c : 0;
       tot += c;
       itot += winact[w];
+      const int k = wkeep[w];
+      koff += w < wave ? k : 0;
+      ktot += k;
     }
+    if (kept) d.keep_idx[keep_base + koff + __popcll(bk & ((1ull << lane) - 1ull))] = r;
+    keep_base += ktot;
     if (crossing) {
       const int pos = base + woff + __popcll(bc & ((1ull << lane) - 1ull));
       idx_out[pos] = r;
@@ -285,6 +295,10 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     __syncthreads();
   }
   for (int64_t r = d.N + tid; r < d.ld; r += 1024) d.cls[r] = kKeep;  // padding rows stay zero
+  if (tid < 2 * (int)kLdAlign) {  // -1 up to the next multiple of 16 past the list (at least 16 entries in all)
+    const int end = max((keep_base + (int)kLdAlign - 1) / (int)kLdAlign * (int)kLdAlign, (int)kLdAlign);
+    if (keep_base + tid < end) d.keep_idx[keep_base + tid] = -1;
+  }
   const int m = base;
   if (tid == 0) {
     d.counts[0] = m;
@@ -342,8 +356,9 @@ __global__ __launch_bounds__(1024) void relu_count_kernel(const ReluDesc* __rest
       c += wc[w];
       i += wi[w];
     }
-    d.blk_counts[2 * blockIdx.x] = c;
-    d.blk_counts[2 * blockIdx.x + 1] = i;
+    d.blk_counts[3 * blockIdx.x] = c;
+    d.blk_counts[3 * blockIdx.x + 1] = i;
+    d.blk_counts[3 * blockIdx.x + 2] = min(1024, d.N - (int)blockIdx.x * 1024) - c - i;  // kept rows of the block
   }
 }
 
@@ -352,25 +367,28 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  __shared__ int wcross[16];
-  __shared__ int sbase, stot, sinact;
-  if (wave == 0) {  // offset of this block = crossing counts of the blocks before it
-    int before = 0, tot = 0, inact = 0;
+  __shared__ int wcross[16], wkeep[16];
+  __shared__ int sbase, stot, sinact, skbase;
+  if (wave == 0) {  // offset of this block = crossing (kept) counts of the blocks before it
+    int before = 0, tot = 0, inact = 0, kbefore = 0;
     for (int b = lane; b < (int)gridDim.x; b += 64) {
-      const int c = d.blk_counts[2 * b];
+      const int c = d.blk_counts[3 * b];
       before += b < (int)blockIdx.x ? c : 0;
       tot += c;
-      inact += d.blk_counts[2 * b + 1];
+      inact += d.blk_counts[3 * b + 1];
+      kbefore += b < (int)blockIdx.x ? d.blk_counts[3 * b + 2] : 0;
     }
     for (int off = 32; off > 0; off >>= 1) {
       before += __shfl_xor(before, off);
       tot += __shfl_xor(tot, off);
       inact += __shfl_xor(inact, off);
+      kbefore += __shfl_xor(kbefore, off);
     }
     if (lane == 0) {
       sbase = before;
       stot = tot;
       sinact = inact;
+      skbase = kbefore;
     }
   }
   const int r = blockIdx.x * 1024 + tid;
@@ -379,12 +397,21 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
   const double u = valid ? d.ub[r] : 1.0;
   const bool inactive = valid && (u <= 0.0);
   const bool crossing = valid && (l < 0.0) && (u > 0.0);
+  const bool kept = valid && !inactive && !crossing;
   const unsigned long long bc = __ballot(crossing);
-  if (lane == 0) wcross[wave] = __popcll(bc);
+  const unsigned long long bk = __ballot(kept);
+  if (lane == 0) {
+    wcross[wave] = __popcll(bc);
+    wkeep[wave] = __popcll(bk);
+  }
   __syncthreads();
-  int woff = 0;
+  int woff = 0, koff = 0;
 #pragma unroll
-  for (int w = 0; w < 16; ++w) woff += w < wave ? wcross[w] : 0;
+  for (int w = 0; w < 16; ++w) {
+    woff += w < wave ? wcross[w] : 0;
+    koff += w < wave ? wkeep[w] : 0;
+  }
+  if (kept) d.keep_idx[skbase + koff + __popcll(bk & ((1ull << lane) - 1ull))] = r;
   int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
   if (crossing) {
     const int pos = sbase + woff + __popcll(bc & ((1ull << lane) - 1ull));
@@ -399,6 +426,11 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
   }
   if (blockIdx.x == gridDim.x - 1) {
     for (int64_t p = d.N + tid; p < d.ld; p += 1024) d.cls[p] = kKeep;  // padding rows stay zero
+    if (tid < 2 * (int)kLdAlign) {  // pad the kept-row list with -1 to a whole K-tile (at least one)
+      const int nkeep = d.N - stot - sinact;
+      const int end = max((nkeep + (int)kLdAlign - 1) / (int)kLdAlign * (int)kLdAlign, (int)kLdAlign);
+      if (nkeep + tid < end) d.keep_idx[nkeep + tid] = -1;
+    }
     if (tid == 0) {
       d.counts[0] = stot;
       d.counts[1] = sinact;
@@ -536,7 +568,12 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const int64_t nblk = ceil_div(N, 1024);
   NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &cls_buf));
   NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * count, &cnt_buf));
-  if (N > 8192) NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * nblk * count, &blk_buf));
+  if (N > 8192) NNV_TRY(ctx->alloc(sizeof(int32_t) * 3 * nblk * count, &blk_buf));
+  // kept-row lists of all sets in one buffer; the classification pads each list with -1 up to a whole
+  // K-tile (at least one), which is what the GEMM's row map expects
+  const int64_t keep_ld = round_up(N, kLdAlign) + kLdAlign;
+  BufRef keep_buf;
+  NNV_TRY(ctx->alloc(sizeof(int32_t) * keep_ld * count, &keep_buf));
   if (sorted) {
     NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &asc_buf));
     NNV_TRY(ctx->alloc(sizeof(double) * ld * count, &key_buf));
@@ -559,7 +596,8 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.key = sorted ? key_buf->as<double>() + ld * i : nullptr;
     d.rank = sorted ? rank_buf->as<int32_t>() + ld * i : nullptr;
     d.counts = cnt_buf->as<int32_t>() + 2 * i;
-    d.blk_counts = blk_buf ? blk_buf->as<int32_t>() + 2 * nblk * i : nullptr;
+    d.blk_counts = blk_buf ? blk_buf->as<int32_t>() + 3 * nblk * i : nullptr;
+    d.keep_idx = keep_buf->as<int32_t>() + keep_ld * i;
     d.mailbox = nullptr;
     d.ld = ld;
     d.N = (int32_t)N;
@@ -706,6 +744,10 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->oh_idx_buf = idx_bufs[i];
       o->oh_idx = idx_bufs[i]->as<int32_t>();
     }
+    // rows of the leading columns that were not reset
+    o->n_kept = N - counts[2 * i] - counts[2 * i + 1];
+    o->kept_buf = keep_buf;
+    o->kept_idx = keep_buf->as<int32_t>() + keep_ld * i;
     if (d.m > 0) {
       auto node = std::make_shared<ConsNode>();
       node->prev = in[i]->cons;

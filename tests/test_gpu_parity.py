@@ -261,3 +261,81 @@ def test_zero_width_dimensions_and_scalar_box(nnv, oracle):
     assert np.array_equal(l, [1.0, 2.0]) and np.array_equal(u, [1.0, 2.0])
     R = nnv.PosLin.reach(allfix, "relax-star-area", [], 1)
     assert R.nVar == 0 and np.array_equal(R.V, allfix.V)
+
+
+def _reach_in_subprocess(dense, k, method, shrink):
+    """Output V / bounds of config k from a fresh process, with or without the structural-zero skipping
+    of the FC map (the switch is read once per process)."""
+    import json
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import json, sys, numpy as np, nnv_amd\n"
+        "from nnv_amd.configs import make_config, device_input_sets\n"
+        "cfg = make_config(%d, %d)\n"
+        "net = nnv_amd.NN.from_config(cfg['layers'])\n"
+        "out = net.reach(device_input_sets(cfg), {'reachMethod': '%s', 'relaxFactor': 1})\n"
+        "outs = out if isinstance(out, list) else [out]\n"
+        "res = []\n"
+        "for o_ in outs:\n"
+        "    V = np.asarray(o_.V); lb, ub = o_.estimateRanges()\n"
+        "    res.append([V.reshape(-1, order='F').tolist(), np.asarray(lb).reshape(-1).tolist(), np.asarray(ub).reshape(-1).tolist()])\n"
+        "json.dump(res, sys.stdout)\n" % (k, shrink, method))
+    env = dict(os.environ)
+    env.pop("NNVHIP_DENSE_AFFINE", None)
+    if dense:
+        env["NNVHIP_DENSE_AFFINE"] = "1"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=200)
+    assert p.returncode == 0, p.stderr.decode()[-2000:]
+    return json.loads(p.stdout.decode())
+
+
+@pytest.mark.parametrize("k,shrink", [(1, 1), (2, 1), (5, 64)])
+def test_structural_zero_skipping_equals_dense_contraction(k, shrink):
+    # W*[c V] with the one-hot columns gathered and the reset rows left out must give what the full
+    # dense contraction gives: same columns bit for bit where only a gather is involved, and the
+    # contracted columns up to the summation order of the kept rows
+    a = _reach_in_subprocess(False, k, "relax-star-area", shrink)
+    b = _reach_in_subprocess(True, k, "relax-star-area", shrink)
+    assert len(a) == len(b)
+    for (Va, la, ua), (Vb, lb_, ub_) in zip(a, b):
+        Va, Vb = np.asarray(Va), np.asarray(Vb)
+        assert Va.shape == Vb.shape
+        scale = np.max(np.abs(Vb))
+        assert np.max(np.abs(Va - Vb)) <= 1e-13 * scale
+        assert np.array_equal(Va == 0, Vb == 0)
+        assert np.allclose(la, lb_, rtol=0, atol=1e-12 * max(1.0, np.max(np.abs(lb_))))
+        assert np.allclose(ua, ub_, rtol=0, atol=1e-12 * max(1.0, np.max(np.abs(ub_))))
+
+
+def test_fc_on_sets_with_and_without_structure_hints(nnv, oracle):
+    # the same matrices as a hand-built Star (no hints), as a box star (all generators one-hot) and as a
+    # ReLU output (appended one-hot columns, reset rows), alone and mixed in one array
+    rs = np.random.RandomState(77)
+    N, M = 96, 40
+    W, b = rs.randn(M, N), rs.randn(M)
+    L = nnv.FullyConnectedLayer(W, b)
+    lbv = -rs.rand(N)
+    ubv = rs.rand(N)
+    lbv[5] = ubv[5] = 0.25          # zero-width dimension: its generator column is dropped
+    box_d, box_o = nnv.Star(lbv, ubv), oracle.star_from_box(lbv, ubv)
+    Vh = rs.randn(N, 9)
+    args = (Vh, np.zeros((1, 8)), np.zeros(1), -np.ones(8), np.ones(8))
+    hand_d, hand_o = nnv.Star(*args), oracle.OStar(*args)
+    W0, b0 = rs.randn(N, N), rs.randn(N)
+    pre_d = nnv.FullyConnectedLayer(W0, b0).reach(box_d, "approx-star")
+    relu_d = nnv.PosLin.reach(pre_d, "relax-star-area", [], 1)
+    relu_o = oracle.reach_relaxed_star(oracle.affine_map(box_o, W0, b0), "relax-star-area", 1.0)
+    for dset, oset, tag in ((box_d, box_o, "box"), (hand_d, hand_o, "hand"), (relu_d, relu_o, "relu")):
+        R = L.reach(dset, "approx-star")
+        E = oracle.affine_map(oset, W, b)
+        assert_close(R.V, E.V, "fc on %s star" % tag)
+        lb, ub = R.estimateRanges()
+        elb, eub = oracle.estimate_ranges(E)
+        assert_close(lb, elb, tag + " lb")
+        assert_close(ub, eub, tag + " ub")
+    outs = L.reach([relu_d, box_d, relu_d], "approx-star")     # array: not one arena, per-set launches
+    for R, oset in zip(outs, (relu_o, box_o, relu_o)):
+        assert_close(R.V, oracle.affine_map(oset, W, b).V, "fc on mixed array")
