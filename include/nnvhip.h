@@ -73,6 +73,13 @@ NNVHIP_API int nnvhip_synchronize(nnvhip_ctx* ctx);
  * call wait for the layer to finish; 2 additionally brackets single kernels (nnvhip_kernel_time). */
 NNVHIP_API int nnvhip_set_timing(nnvhip_ctx* ctx, int enabled);
 NNVHIP_API int nnvhip_last_op_time_ms(nnvhip_ctx* ctx, double* ms);
+/* Measurement switch (no counterpart in the reference).  By default nnvhip_affine_fc leaves out the
+ * products with structural zeros that the producing step recorded on the set handle (one-hot
+ * generator columns of box stars and of ReLU outputs, rows the ReLU step reset); the result is the
+ * same.  enabled = 1 runs every FC layer as the full dense contraction W*[c V], which is how the
+ * reference's Star.affineMap (set/Star.m:313-343) executes it.  Initial value: 1 if the environment
+ * variable NNVHIP_DENSE_AFFINE is set, else 0. */
+NNVHIP_API int nnvhip_set_dense_affine(nnvhip_ctx* ctx, int enabled);
 /* Measurement hook (no counterpart in the reference): while timing level 2 is set, every launch of a
  * kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
  * dense GEMM kernel of the FC layers (tiles of at least 64 rows); 1: implicit-GEMM convolution

@@ -16,7 +16,7 @@ HS_DISJOINT, HS_UNDECIDED, HS_INSIDE = 1, 2, 3
 # every entry point declared in include/nnvhip.h
 SYMBOLS = [
     "nnvhip_create", "nnvhip_destroy", "nnvhip_last_error", "nnvhip_synchronize", "nnvhip_set_timing",
-    "nnvhip_last_op_time_ms", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
+    "nnvhip_last_op_time_ms", "nnvhip_set_dense_affine", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
     "nnvhip_trim_pool", "nnvhip_pool_stats", "nnvhip_star_create",
     "nnvhip_star_from_box", "nnvhip_star_retain", "nnvhip_star_release", "nnvhip_star_dims",
     "nnvhip_star_fetch_V", "nnvhip_star_fetch_pred_bounds", "nnvhip_star_fetch_constraints",
@@ -57,6 +57,7 @@ def load():
         "nnvhip_destroy": [p],
         "nnvhip_synchronize": [p],
         "nnvhip_set_timing": [p, C.c_int],
+        "nnvhip_set_dense_affine": [p, C.c_int],
         "nnvhip_last_op_time_ms": [p, C.POINTER(dbl)],
         "nnvhip_kernel_time": [p, C.c_int, C.POINTER(dbl), pi64, C.POINTER(dbl), C.c_int],
         "nnvhip_probe_copy_bandwidth": [p, i64, C.c_int, C.POINTER(dbl)],
@@ -144,6 +145,11 @@ class Context:
     def set_timing(self, level):
         """0/False: off; 1/True: per-layer device times; 2: also per-kernel timers (kernel_time)."""
         check(self.lib.nnvhip_set_timing(self.handle, int(level)))
+
+    def set_dense_affine(self, enabled):
+        """True: FC layers run as the full dense contraction; False (default): products with the
+        structural zeros recorded on the set handles are left out (same result)."""
+        check(self.lib.nnvhip_set_dense_affine(self.handle, 1 if enabled else 0))
 
     def last_op_time_ms(self) -> float:
         ms = C.c_double()

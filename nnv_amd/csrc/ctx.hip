@@ -170,6 +170,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
     NNV_FAIL(NNVHIP_ERR_ARG, "libnnvhip is built for gfx950 (MI355X); device %d is %s", device, prop.gcnArchName);
   nnvhip_ctx* c = new nnvhip_ctx();
   c->device = device;
+  c->dense_affine = getenv("NNVHIP_DENSE_AFFINE") != nullptr;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
@@ -208,6 +209,12 @@ int nnvhip_set_timing(nnvhip_ctx* c, int enabled) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
   c->timing = enabled != 0;
   c->kernel_timing = enabled >= 2;
+  return NNVHIP_OK;
+}
+
+int nnvhip_set_dense_affine(nnvhip_ctx* c, int enabled) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  c->dense_affine = enabled != 0;
   return NNVHIP_OK;
 }
 
@@ -745,7 +752,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
     const double* Wd = fc->W->as<double>();
     // Columns of V that are scaled unit vectors (all generators of a box star, the columns a ReLU
     // appended) need no contraction: W * (s * e_r) = s * W(:, r).  dense[i] = leading columns that do.
-    static const bool dense_only = getenv("NNVHIP_DENSE_AFFINE") != nullptr;
+    const bool dense_only = c->dense_affine;
     std::vector<int64_t> dense((size_t)count);
     std::vector<GatherSet> gs((size_t)count);
     int64_t total_dense = 0;

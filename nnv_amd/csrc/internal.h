@@ -101,6 +101,9 @@ struct nnvhip_ctx {
   // spins on it, which is quicker than a device-to-host copy plus stream synchronisation
   volatile int32_t* mailbox = nullptr;
   int32_t mailbox_seq = 0;
+  // FC layers as the full dense contraction (no skipping of structural zeros); default from the
+  // environment variable NNVHIP_DENSE_AFFINE
+  bool dense_affine = false;
   // per-layer timing
   bool timing = false;         // per-layer events (nnvhip_last_op_time_ms)
   bool kernel_timing = false;  // additionally one event pair per launch of the timed kernel groups
