@@ -10,6 +10,7 @@
 // GEMM.  MFMA operand "b" carries positions (the memory-contiguous direction of the output), "a"
 // carries output channels.
 #include <algorithm>
+#include <cstring>
 
 #include "internal.h"
 #include "mfma_tile.h"
@@ -173,6 +174,92 @@ __global__ void zero_pad_rows_kernel(double* __restrict__ V, int64_t ld, int64_t
     V[N + t % pad + (t / pad) * ld] = 0.0;
 }
 
+
+// ---- convolution of one-hot generator images -----------------------------------------------------
+// A generator that is s * e_r (r = pixel (h, w, ci)) maps to the filter "stamped" around that pixel:
+// out(ho, wo, co) = s * W(fh, fw, ci, co) for the one tap with ho*sh - pt + fh*dh = h and
+// wo*sw - pl + fw*dw = w, and zero elsewhere.  The dense accumulation would add exact zeros to that
+// one product, so 0 + w*s is the same value.  One pass that writes the output columns (HBM bound);
+// lane = two adjacent output rows, the waves of a block interleave columns.
+struct StampSet {
+  const int32_t* idx;   // input row of every one-hot column
+  const double* scale;  // by input row, or null (= 1)
+  double* out;          // first of these columns in the output set
+  int32_t m;
+  int32_t pad_;
+};
+
+__global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restrict__ table, StampSet one, ConvGeom g,
+                                                         const double* __restrict__ Wt, int64_t ldout, int cols_per_chunk) {
+  const StampSet d = table ? table[blockIdx.z] : one;
+  const int j0 = blockIdx.y * cols_per_chunk;
+  if (j0 >= d.m) return;
+  const int j1 = min(d.m, j0 + cols_per_chunk);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t r0 = (int64_t)blockIdx.x * 128 + 2 * lane;
+  const int64_t Nout = (int64_t)g.P * g.Cout;
+  // the two output rows of this lane: (ho, wo, co), fixed for all columns
+  int hb[2], wb[2], co[2];
+  bool real[2];
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int64_t r = r0 + e;
+    real[e] = r < Nout;
+    const int p = real[e] ? (int)(r % g.P) : 0;
+    co[e] = real[e] ? (int)(r / g.P) : 0;
+    const int wo = p / g.Ho;
+    const int ho = p - wo * g.Ho;
+    hb[e] = ho * g.sh - g.pt;  // input row reached by tap fh = 0
+    wb[e] = wo * g.sw - g.pl;
+  }
+  // the columns of the chunk are decoded once per block (pixel position, channel offset into the
+  // weights, scale) in batches of kStampBatch and then read back from LDS by all lanes
+  constexpr int kStampBatch = 256;
+  __shared__ int s_h[kStampBatch], s_w[kStampBatch], s_k[kStampBatch];
+  __shared__ double s_s[kStampBatch];
+  const bool unit_dil = g.dh == 1 && g.dw == 1;
+  for (int jb = j0; jb < j1; jb += kStampBatch) {
+    const int nb = min(kStampBatch, j1 - jb);
+    __syncthreads();
+    for (int t = threadIdx.x; t < nb; t += 512) {
+      const int src = d.idx[jb + t];
+      const int ci = src / g.HW;
+      const int q = src - ci * g.HW;
+      const int w = q / g.H;
+      s_h[t] = q - w * g.H;
+      s_w[t] = w;
+      s_k[t] = g.FH * g.FW * ci;
+      s_s[t] = d.scale != nullptr ? d.scale[src] : 1.0;
+    }
+    __syncthreads();
+    for (int t = wave; t < nb; t += 8) {
+      const int h = s_h[t], w = s_w[t], kc = s_k[t];
+      const double s = s_s[t];
+      double v[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        v[e] = 0.0;
+        const int th = h - hb[e], tw = w - wb[e];
+        if (real[e] && th >= 0 && tw >= 0) {
+          int fh = th, fw = tw;
+          bool hit = true;
+          if (!unit_dil) {
+            fh = th / g.dh;
+            fw = tw / g.dw;
+            hit = fh * g.dh == th && fw * g.dw == tw;
+          }
+          if (hit && fh < g.FH && fw < g.FW) {
+            const double wv = Wt[fh + g.FH * fw + kc + (int64_t)co[e] * g.Kp];
+            v[e] = __dadd_rn(0.0, __dmul_rn(wv, s));
+          }
+        }
+      }
+      if (r0 < ldout) *reinterpret_cast<double2*>(d.out + r0 + (int64_t)(jb + t) * ldout) = make_double2(v[0], v[1]);
+    }
+  }
+}
+
 template <int TP, int TC, int WR, int WC>
 static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGeom& g, const double* in, int64_t ldin,
                            double* out, int64_t ldout, int64_t ncols) {
@@ -190,6 +277,8 @@ static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvG
   return NNVHIP_OK;
 }
 
+static void fill_geom(ConvGeom& g, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo);
+
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
                   const int32_t* /*centre_flags*/) {
@@ -197,6 +286,26 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W
   if ((cv->FH - 1) * cv->dil[0] > 0xffff || (cv->FW - 1) * cv->dil[1] > 0xffff)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "dilated filter extent too large");
   ConvGeom g;
+  fill_geom(g, cv, H, W, Ho, Wo);
+  const int64_t Nout = Ho * Wo * cv->Cout;
+  // 128 positions x Cout tile, eight waves per block (two per SIMD keep the MFMA pipe fed while
+  // the other wave gathers)
+  int st;
+  if (cv->Cout <= 16)
+    st = launch_conv_cfg<128, 16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols);
+  else if (cv->Cout <= 32)
+    st = launch_conv_cfg<128, 32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
+  else
+    st = launch_conv_cfg<128, 64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
+  NNV_TRY(st);
+  if (ldout != Nout) {  // keep the padding rows of the output at zero
+    hipLaunchKernelGGL(zero_pad_rows_kernel, dim3(256), dim3(256), 0, ctx->stream, out, ldout, Nout, ncols);
+    NNV_HIP_TRY(hipGetLastError());
+  }
+  return NNVHIP_OK;
+}
+
+static void fill_geom(ConvGeom& g, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo) {
   g.H = (int)H;
   g.W = (int)W;
   g.Cin = (int)cv->Cin;
@@ -215,21 +324,39 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W
   g.Kp = (int)cv->Kp;
   g.P = (int)(Ho * Wo);
   g.HW = (int)(H * W);
-  const int64_t Nout = Ho * Wo * cv->Cout;
-  // 128 positions x Cout tile, eight waves per block (two per SIMD keep the MFMA pipe fed while
-  // the other wave gathers)
-  int st;
-  if (cv->Cout <= 16)
-    st = launch_conv_cfg<128, 16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols);
-  else if (cv->Cout <= 32)
-    st = launch_conv_cfg<128, 32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
-  else
-    st = launch_conv_cfg<128, 64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
-  NNV_TRY(st);
-  if (ldout != Nout) {  // keep the padding rows of the output at zero
-    hipLaunchKernelGGL(zero_pad_rows_kernel, dim3(256), dim3(256), 0, ctx->stream, out, ldout, Nout, ncols);
-    NNV_HIP_TRY(hipGetLastError());
+}
+
+int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                       int64_t ldout, int64_t count, const ConvStampSet* sets) {
+  static_assert(sizeof(ConvStampSet) == sizeof(StampSet), "same layout");
+  if (count <= 0) return NNVHIP_OK;
+  if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  int64_t max_m = 0;
+  double bytes = 0.0;
+  for (int64_t i = 0; i < count; ++i) {
+    max_m = std::max<int64_t>(max_m, sets[i].m);
+    bytes += 8.0 * (double)(Ho * Wo * cv->Cout) * (double)sets[i].m;  // algorithmic: the output columns
   }
+  if (max_m == 0) return NNVHIP_OK;
+  ConvGeom g;
+  fill_geom(g, cv, H, W, Ho, Wo);
+  const int64_t row_blocks = ceil_div(ldout, 128);
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(max_m, 32)));
+  const int64_t cpc = ceil_div(max_m, chunks);
+  chunks = ceil_div(max_m, cpc);
+  const StampSet* table = nullptr;
+  BufRef tab;
+  if (count > 1) {
+    NNV_TRY(ctx->upload(sets, sizeof(StampSet) * count, &tab));
+    table = tab->as<StampSet>();
+  }
+  StampSet one;
+  memcpy(&one, &sets[0], sizeof one);
+  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
+  hipLaunchKernelGGL(conv_stamp_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(512), 0,
+                     ctx->stream, table, one, g, cv->W->as<double>(), ldout, (int)cpc);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
+  NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }
 

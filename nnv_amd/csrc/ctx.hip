@@ -907,8 +907,22 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
   int64_t cols = 0;
   NNV_TRY(c->begin_op());
   int st = make_affine_outputs(c, count, in, Nout, &outs, &contig, &cols);
-  for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
-    st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, in[i]->n + 1, nullptr);
+  // generator images that are scaled unit vectors (box ImageStars, columns appended by a ReLU) turn
+  // into stamps of the filter; the implicit GEMM runs over the leading dense images only
+  std::vector<ConvStampSet> stamps((size_t)count);
+  bool any_stamps = false;
+  for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
+    const int64_t nc = in[i]->n + 1;
+    const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
+    stamps[i].idx = in[i]->oh_idx;
+    stamps[i].scale = in[i]->oh_scale;
+    stamps[i].out = outs[i]->V + dense * outs[i]->ld;
+    stamps[i].m = (int32_t)(nc - dense);
+    stamps[i].pad_ = 0;
+    any_stamps = any_stamps || dense < nc;
+    st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, dense, nullptr);
+  }
+  if (st == NNVHIP_OK && any_stamps) st = launch_conv_stamps(c, cv, H, W, Ho, Wo, outs[0]->ld, count, stamps.data());
   if (st == NNVHIP_OK) st = c->end_op();
   if (st != NNVHIP_OK) {
     release_all(outs);

@@ -242,6 +242,17 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
                   const int32_t* centre_flags /* per column: 1 = add bias */);
 
+// Convolution of the one-hot generator columns of every set ("stamps" of the filter), conv.hip.
+struct ConvStampSet {
+  const int32_t* idx;   // input row of every one-hot column
+  const double* scale;  // by input row, or null
+  double* out;          // first of these columns in the output set
+  int32_t m;
+  int32_t pad_;
+};
+int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                       int64_t ldout, int64_t count, const ConvStampSet* sets);
+
 // ranges.hip
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s);
 // W * (scaled unit vectors): out(:, j) = W(:, idx[j]) * scale[idx[j]] for the one-hot column block of

@@ -307,7 +307,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   }
   if (SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP) {
     __syncthreads();
-    if constexpr (SORT_CAP == 1024)  // the staged doubles are read back as their bit patterns
+    if (SORT_CAP == 1024 || m <= 1024)  // the staged doubles are read back as their bit patterns
       sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
     else
       bitonic_sort_desc<SORT_CAP>(skey, sidx, m, tid, d.cross_idx);
