@@ -185,6 +185,9 @@ struct StampSet {
   const int32_t* idx;   // input row of every one-hot column
   const double* scale;  // by input row, or null (= 1)
   double* out;          // first of these columns in the output set
+  const double* plb;    // predicate bounds of these columns
+  const double* pub;
+  double* part;         // [chunks][4][ldout] range sums of these columns (as the estimateRanges pass leaves them)
   int32_t m;
   int32_t pad_;
 };
@@ -192,9 +195,10 @@ struct StampSet {
 __global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restrict__ table, StampSet one, ConvGeom g,
                                                          const double* __restrict__ Wt, int64_t ldout, int cols_per_chunk) {
   const StampSet d = table ? table[blockIdx.z] : one;
-  const int j0 = blockIdx.y * cols_per_chunk;
-  if (j0 >= d.m) return;
+  const int j0 = min(d.m, (int)blockIdx.y * cols_per_chunk);  // an empty chunk still writes its (zero) sums
   const int j1 = min(d.m, j0 + cols_per_chunk);
+  if (d.m == 0) return;
+  double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t r0 = (int64_t)blockIdx.x * 128 + 2 * lane;
@@ -256,7 +260,45 @@ __global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restr
         }
       }
       if (r0 < ldout) *reinterpret_cast<double2*>(d.out + r0 + (int64_t)(jb + t) * ldout) = make_double2(v[0], v[1]);
+      const double pl = d.plb[jb + t], pu = d.pub[jb + t];
+      const double px = fmax(v[0], 0.0), nx = fmin(v[0], 0.0);
+      const double py = fmax(v[1], 0.0), ny = fmin(v[1], 0.0);
+      xmin1.x = fma(px, pl, xmin1.x);
+      xmin1.y = fma(py, pl, xmin1.y);
+      xmax1.x = fma(px, pu, xmax1.x);
+      xmax1.y = fma(py, pu, xmax1.y);
+      xmin2.x = fma(nx, pu, xmin2.x);
+      xmin2.y = fma(ny, pu, xmin2.y);
+      xmax2.x = fma(nx, pl, xmax2.x);
+      xmax2.y = fma(ny, pl, xmax2.y);
     }
+  }
+  // range sums of this chunk: the eight waves hold different columns of the same rows
+  __shared__ double2 red[8][4][64];
+  __syncthreads();
+  if (wave > 0) {
+    red[wave][0][lane] = xmin1;
+    red[wave][1][lane] = xmin2;
+    red[wave][2][lane] = xmax1;
+    red[wave][3][lane] = xmax2;
+  }
+  __syncthreads();
+  if (wave == 0 && r0 < ldout) {
+    for (int w = 1; w < 8; ++w) {
+      xmin1.x += red[w][0][lane].x;
+      xmin1.y += red[w][0][lane].y;
+      xmin2.x += red[w][1][lane].x;
+      xmin2.y += red[w][1][lane].y;
+      xmax1.x += red[w][2][lane].x;
+      xmax1.y += red[w][2][lane].y;
+      xmax2.x += red[w][3][lane].x;
+      xmax2.y += red[w][3][lane].y;
+    }
+    double* p = d.part + ((int64_t)blockIdx.y * 4) * ldout + r0;
+    *reinterpret_cast<double2*>(p) = xmin1;
+    *reinterpret_cast<double2*>(p + ldout) = xmin2;
+    *reinterpret_cast<double2*>(p + 2 * ldout) = xmax1;
+    *reinterpret_cast<double2*>(p + 3 * ldout) = xmax2;
   }
 }
 
@@ -326,8 +368,15 @@ static void fill_geom(ConvGeom& g, const nnvhip_conv2d* cv, int64_t H, int64_t W
   g.HW = (int)(H * W);
 }
 
+int64_t conv_stamp_chunks(int64_t ldout, int64_t count, int64_t max_m) {
+  const int64_t row_blocks = ceil_div(ldout, 128);
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(std::max<int64_t>(max_m, 1), 32)));
+  const int64_t cpc = ceil_div(std::max<int64_t>(max_m, 1), chunks);
+  return ceil_div(std::max<int64_t>(max_m, 1), cpc);
+}
+
 int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
-                       int64_t ldout, int64_t count, const ConvStampSet* sets) {
+                       int64_t ldout, int64_t count, const ConvStampSet* sets, int64_t chunks) {
   static_assert(sizeof(ConvStampSet) == sizeof(StampSet), "same layout");
   if (count <= 0) return NNVHIP_OK;
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
@@ -341,9 +390,7 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int6
   ConvGeom g;
   fill_geom(g, cv, H, W, Ho, Wo);
   const int64_t row_blocks = ceil_div(ldout, 128);
-  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(max_m, 32)));
   const int64_t cpc = ceil_div(max_m, chunks);
-  chunks = ceil_div(max_m, cpc);
   const StampSet* table = nullptr;
   BufRef tab;
   if (count > 1) {

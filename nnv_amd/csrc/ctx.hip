@@ -768,6 +768,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.out = outs[i]->V + dense[i] * outs[i]->ld;
       g.plb = outs[i]->plb + (dense[i] - 1);
       g.pub = outs[i]->pub + (dense[i] - 1);
+      g.part = nullptr;
       g.m = (int32_t)(nc - dense[i]);
       g.pad_ = 0;
     }
@@ -797,9 +798,10 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
                        compact ? &rows : nullptr);
       const bool fused = st == NNVHIP_OK && fuse.chunks > 0;
-      if (st == NNVHIP_OK && gs[0].m > 0)
-        st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? fuse.part->as<double>() : nullptr,
-                                   fuse.chunks, gch);
+      if (st == NNVHIP_OK && gs[0].m > 0) {
+        gs[0].part = fused ? fuse.part->as<double>() + fuse.chunks * 4 * outs[0]->ld : nullptr;
+        st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? gch : 0);
+      }
       if (st == NNVHIP_OK && fused) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0));
     } else if (contig) {
       // one launch for the whole array.  With structure to exploit, every set's dense columns are cut
@@ -862,8 +864,27 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         st = c->upload(centres.data(), sizeof(double*) * centres.size(), &tab);
         if (st == NNVHIP_OK) st = launch_bias_columns(c, tab->as<double*>(), count - 1, bias, fc->Mp);
       }
-      if (st == NNVHIP_OK && any_onehot)
-        st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, count, gs.data(), nullptr, 0, 0);
+      if (st == NNVHIP_OK && any_onehot) {
+        // the gather also leaves the range sums of its columns on the output handles, so the ReLU
+        // that follows scans only the contracted columns
+        int64_t max_m = 0;
+        for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, gs[i].m);
+        const int64_t gch = gather_chunks_batch(outs[0]->ld, count, max_m);
+        BufRef sums;
+        st = c->alloc(sizeof(double) * 4 * outs[0]->ld * gch * count, &sums);
+        if (st == NNVHIP_OK) {
+          for (int64_t i = 0; i < count; ++i)
+            gs[i].part = gs[i].m > 0 ? sums->as<double>() + 4 * outs[0]->ld * gch * i : nullptr;
+          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, count, gs.data(), gch);
+        }
+        for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+          if (gs[i].m > 0) {
+            outs[i]->rng_buf = sums;
+            outs[i]->rng_part = gs[i].part;
+            outs[i]->rng_chunks = gch;
+            outs[i]->rng_first_col = dense[i];
+          }
+      }
     } else {
       for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
         GemmRows rows;
@@ -871,8 +892,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         const bool compact = rows_of(i, &rows, &kp);
         st = launch_gemm(c, Wd, fc->Mp, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, fc->Mp, dense[i], kp, bias, nullptr,
                          compact ? &rows : nullptr);
-        if (st == NNVHIP_OK && gs[i].m > 0)
-          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[i]->ld, 1, &gs[i], nullptr, 0, 0);
+        if (st == NNVHIP_OK && gs[i].m > 0) st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[i]->ld, 1, &gs[i], 0);
       }
     }
   }
@@ -911,18 +931,39 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
   // into stamps of the filter; the implicit GEMM runs over the leading dense images only
   std::vector<ConvStampSet> stamps((size_t)count);
   bool any_stamps = false;
+  int64_t max_m = 0;
   for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
     const int64_t nc = in[i]->n + 1;
     const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
     stamps[i].idx = in[i]->oh_idx;
     stamps[i].scale = in[i]->oh_scale;
     stamps[i].out = outs[i]->V + dense * outs[i]->ld;
+    stamps[i].plb = outs[i]->plb + (dense - 1);
+    stamps[i].pub = outs[i]->pub + (dense - 1);
+    stamps[i].part = nullptr;
     stamps[i].m = (int32_t)(nc - dense);
     stamps[i].pad_ = 0;
     any_stamps = any_stamps || dense < nc;
+    max_m = std::max<int64_t>(max_m, nc - dense);
     st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, dense, nullptr);
   }
-  if (st == NNVHIP_OK && any_stamps) st = launch_conv_stamps(c, cv, H, W, Ho, Wo, outs[0]->ld, count, stamps.data());
+  if (st == NNVHIP_OK && any_stamps) {
+    // the stamp pass also leaves the range sums of its columns on the output handles
+    const int64_t sch = conv_stamp_chunks(outs[0]->ld, count, max_m);
+    BufRef sums;
+    st = c->alloc(sizeof(double) * 4 * outs[0]->ld * sch * count, &sums);
+    if (st == NNVHIP_OK) {
+      for (int64_t i = 0; i < count; ++i) stamps[i].part = sums->as<double>() + 4 * outs[0]->ld * sch * i;
+      st = launch_conv_stamps(c, cv, H, W, Ho, Wo, outs[0]->ld, count, stamps.data(), sch);
+    }
+    for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+      if (stamps[i].m > 0) {
+        outs[i]->rng_buf = sums;
+        outs[i]->rng_part = stamps[i].part;
+        outs[i]->rng_chunks = sch;
+        outs[i]->rng_first_col = (in[i]->n + 1) - stamps[i].m;
+      }
+  }
   if (st == NNVHIP_OK) st = c->end_op();
   if (st != NNVHIP_OK) {
     release_all(outs);

@@ -166,6 +166,13 @@ struct nnvhip_star {
   int64_t n_kept = -1;
   const int32_t* kept_idx = nullptr;
   nnvhip::BufRef kept_buf;
+  // Range sums left behind by the kernel that produced the trailing columns (filter stamps, gathered
+  // columns): rng_chunks chunks of [4][ld] partial sums at rng_part that cover the generator columns
+  // [rng_first_col, n].  estimateRanges then scans only the columns before rng_first_col.
+  nnvhip::BufRef rng_buf;
+  const double* rng_part = nullptr;
+  int64_t rng_chunks = 0;
+  int64_t rng_first_col = 0;
 };
 
 struct nnvhip_fc {
@@ -247,11 +254,16 @@ struct ConvStampSet {
   const int32_t* idx;   // input row of every one-hot column
   const double* scale;  // by input row, or null
   double* out;          // first of these columns in the output set
+  const double* plb;    // predicate bounds of these columns
+  const double* pub;
+  double* part;         // this set's [chunks][4][ldout] range sums
   int32_t m;
   int32_t pad_;
 };
+// Number of column chunks (= range-sum chunks per set) the stamp launch will use.
+int64_t conv_stamp_chunks(int64_t ldout, int64_t count, int64_t max_m);
 int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
-                       int64_t ldout, int64_t count, const ConvStampSet* sets);
+                       int64_t ldout, int64_t count, const ConvStampSet* sets, int64_t chunks);
 
 // ranges.hip
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s);
@@ -262,14 +274,18 @@ struct GatherSet {
   const int32_t* idx;
   const double* scale;  // by row index, or null
   double* out;          // first one-hot column of the output set
-  const double* plb;    // predicate bounds of these columns (fused range sums only)
+  const double* plb;    // predicate bounds of these columns (range sums only)
   const double* pub;
+  double* part;         // where this set's [chunks][4][ldout] range sums go, or null
   int32_t m;
   int32_t pad_;
 };
 int64_t gather_chunks(int64_t Mp, int64_t m);
+int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m);
+// chunks > 0: every set's `part` receives that many chunks (sets with part == null none); chunks = 0:
+// no range sums, the launcher picks the chunking.
 int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t Mp, int64_t ldout, int64_t count,
-                          const GatherSet* sets, double* part, int64_t part_chunk0, int64_t chunks);
+                          const GatherSet* sets, int64_t chunks);
 // Turns the per-column-tile partial sums a fused GEMM left behind into the set's cached lb/ub.
 int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks);
 

@@ -15,7 +15,10 @@ struct RangeDesc {
   const double* V;    // N x (n+1), column 0 = centre
   const double* plb;  // n
   const double* pub;  // n
-  double* part;       // [chunks][4][ld] partial sums (unused when chunks == 1)
+  double* part;       // [chunks][4][ld] partial sums (unused when chunks == 1 and chunks2 == 0)
+  const double* part2;  // further chunks2 chunks left by the producer of the trailing columns, or null
+  int32_t chunks2;
+  int32_t pad_;
   double* lb;         // ld
   double* ub;         // ld
   int64_t ld;
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(c
       xmax2.x += red[src][3][lane].x;
       xmax2.y += red[src][3][lane].y;
     }
-    if (d.chunks == 1) {
+    if (d.chunks == 1 && d.chunks2 == 0) {
       // lb = (c + xmin1) + xmin2, the reference's left-to-right order
       const double2 c = *reinterpret_cast<const double2*>(d.V + r0);
       *reinterpret_cast<double2*>(d.lb + r0) = make_double2((c.x + xmin1.x) + xmin2.x, (c.y + xmin1.y) + xmin2.y);
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(c
 // by four different waves so that the dependent add chains are short.
 __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
-  if (d.chunks == 1 && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
+  if (d.chunks == 1 && d.chunks2 == 0 && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
   const int lane = threadIdx.x & 63;
   const int q = threadIdx.x >> 6;
   const int64_t r = (int64_t)blockIdx.x * 64 + lane;
@@ -125,6 +128,10 @@ __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __re
     const double* p = d.part + (int64_t)q * d.ld + r;
 #pragma unroll 8
     for (int c = 0; c < d.chunks; ++c) s += p[(int64_t)c * 4 * d.ld];
+    if (d.chunks2 > 0) {
+      const double* p2 = d.part2 + (int64_t)q * d.ld + r;
+      for (int c = 0; c < d.chunks2; ++c) s += p2[(int64_t)c * 4 * d.ld];
+    }
   }
   sums[q][lane] = s;
   __syncthreads();
@@ -144,9 +151,8 @@ __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __re
 struct GatherArgs {
   const double* W;
   int64_t ldw, ldout;
-  double* part;  // [chunks][4][ldout] or null
   int32_t cols_per_chunk;
-  int32_t pad_;
+  int32_t with_sums;  // every chunk of the grid leaves range sums in the set's `part` (if it has one)
 };
 
 __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const GatherSet* __restrict__ table, GatherSet one,
@@ -154,7 +160,8 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   const GatherSet d = table ? table[blockIdx.z] : one;
   const int chunk = blockIdx.y;
   const int j0 = chunk * a.cols_per_chunk;
-  if (j0 >= d.m && a.part == nullptr) return;
+  double* part = a.with_sums ? d.part : nullptr;
+  if (j0 >= d.m && part == nullptr) return;
   const int j1 = min(d.m, j0 + a.cols_per_chunk);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -183,7 +190,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
         o.x = __dadd_rn(0.0, __dmul_rn(v[u].x, sc[u]));
         o.y = __dadd_rn(0.0, __dmul_rn(v[u].y, sc[u]));
         *reinterpret_cast<double2*>(d.out + r0 + (int64_t)j * a.ldout) = o;
-        if (a.part != nullptr) {
+        if (part != nullptr) {
           const double pl = d.plb[j], pu = d.pub[j];
           const double px = fmax(o.x, 0.0), nx = fmin(o.x, 0.0);
           const double py = fmax(o.y, 0.0), ny = fmin(o.y, 0.0);
@@ -199,7 +206,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
       }
     }
   }
-  if (a.part == nullptr) return;
+  if (part == nullptr) return;
   __shared__ double2 red[kRangeWaves][4][64];
   if (wave > 0) {
     red[wave][0][lane] = xmin1;
@@ -219,12 +226,19 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
       xmax2.x += red[w][3][lane].x;
       xmax2.y += red[w][3][lane].y;
     }
-    double* p = a.part + ((int64_t)chunk * 4) * a.ldout + r0;
+    double* p = part + ((int64_t)chunk * 4) * a.ldout + r0;
     *reinterpret_cast<double2*>(p) = xmin1;
     *reinterpret_cast<double2*>(p + a.ldout) = xmin2;
     *reinterpret_cast<double2*>(p + 2 * a.ldout) = xmax1;
     *reinterpret_cast<double2*>(p + 3 * a.ldout) = xmax2;
   }
+}
+
+// Column chunks of a gather over `count` sets with at most max_m one-hot columns each.
+int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m) {
+  if (max_m <= 0) return 0;
+  const int64_t row_blocks = ceil_div(ldout, kRowsPerWave);
+  return std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(max_m, 4 * kRangeWaves)));
 }
 
 // Column chunks of the gather for one set of m one-hot columns: enough blocks to cover the chip.
@@ -235,19 +249,20 @@ int64_t gather_chunks(int64_t Mp, int64_t m) {
 }
 
 int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t Mp, int64_t ldout, int64_t count,
-                          const GatherSet* sets, double* part, int64_t part_chunk0, int64_t chunks) {
+                          const GatherSet* sets, int64_t chunks) {
   if (count <= 0) return NNVHIP_OK;
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
   int64_t max_m = 0;
   for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, sets[i].m);
   if (max_m == 0) return NNVHIP_OK;
   const int64_t row_blocks = ceil_div(ldout, kRowsPerWave);
-  if (part == nullptr) chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(max_m, 4 * kRangeWaves)));
+  const bool with_sums = chunks > 0;
+  if (!with_sums) chunks = gather_chunks_batch(ldout, count, max_m);
   GatherArgs a{};
   a.W = W;
   a.ldw = ldw;
   a.ldout = ldout;
-  a.part = part ? part + part_chunk0 * 4 * ldout : nullptr;
+  a.with_sums = with_sums ? 1 : 0;
   a.cols_per_chunk = (int32_t)ceil_div(max_m, chunks);
   const GatherSet* table = nullptr;
   BufRef tab;
@@ -300,8 +315,11 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   // one buffer for all lb/ub, one for all partials
   BufRef rb, pb;
   NNV_TRY(ctx->alloc(sizeof(double) * 2 * ld * nset, &rb));
-  if (chunks > 1) NNV_TRY(ctx->alloc(sizeof(double) * 4 * ld * chunks * nset, &pb));
+  bool pending = false;
+  for (auto* t : todo) pending = pending || (t->rng_part != nullptr && t->rng_chunks > 0);
+  if (chunks > 1 || pending) NNV_TRY(ctx->alloc(sizeof(double) * 4 * ld * chunks * nset, &pb));
   std::vector<RangeDesc> descs(nset);
+  bool any_pending = false;
   for (int64_t i = 0; i < nset; ++i) {
     nnvhip_star* t = todo[i];
     RangeDesc& d = descs[i];
@@ -317,6 +335,19 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     d.lb = rb->as<double>() + 2 * ld * i;
     d.ub = d.lb + ld;
     d.row_waves = row_waves;
+    d.part2 = nullptr;
+    d.chunks2 = 0;
+    d.pad_ = 0;
+    if (t->rng_part != nullptr && t->rng_chunks > 0 && t->rng_first_col >= 1) {
+      // the producer of the trailing columns left their sums: scan only the columns before them
+      d.part2 = t->rng_part;
+      d.chunks2 = (int32_t)t->rng_chunks;
+      d.n = (int32_t)(t->rng_first_col - 1);
+      ch = std::max<int64_t>(1, std::min<int64_t>(chunks, ceil_div(std::max<int64_t>(d.n, 1), 64)));
+      d.chunks = (int32_t)ch;
+      d.cols_per_chunk = (int32_t)std::max<int64_t>(1, ceil_div(std::max<int64_t>(d.n, 1), ch));
+      any_pending = true;
+    }
   }
   const RangeDesc* table = nullptr;
   BufRef tab;
@@ -326,11 +357,12 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   }
   dim3 grid((unsigned)row_blocks, (unsigned)chunks, (unsigned)nset);
   double bytes = 0.0;  // algorithmic: V once, the predicate bounds, lb/ub out
-  for (auto* t : todo) bytes += 8.0 * (double)t->N * (double)(t->n + 1) + 16.0 * (double)t->n + 16.0 * (double)t->N;
+  for (int64_t i = 0; i < nset; ++i)
+    bytes += 8.0 * (double)todo[i]->N * (double)(descs[i].n + 1) + 16.0 * (double)descs[i].n + 16.0 * (double)todo[i]->N;
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL((ranges_partial_kernel<8, 4>), grid, dim3(64 * kRangeWaves), 0, ctx->stream, table, descs[0]);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
-  if (chunks > 1)
+  if (chunks > 1 || any_pending)
     hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,
                        ctx->stream, table, descs[0]);
   NNV_HIP_TRY(hipGetLastError());
@@ -338,6 +370,9 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     todo[i]->rbuf = rb;
     todo[i]->lb = descs[i].lb;
     todo[i]->ub = descs[i].ub;
+    todo[i]->rng_buf.reset();  // the sums are folded in
+    todo[i]->rng_part = nullptr;
+    todo[i]->rng_chunks = 0;
   }
   return NNVHIP_OK;
 }
@@ -358,6 +393,8 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
   d.chunks = (int32_t)chunks;
   d.cols_per_chunk = 0;
   d.row_waves = 1;
+  d.part2 = nullptr;
+  d.chunks2 = 0;
   hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(s->ld, 64), 1, 1), dim3(256), 0, ctx->stream, nullptr, d);
   NNV_HIP_TRY(hipGetLastError());
   s->rbuf = rb;
