@@ -760,6 +760,8 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
     for (int64_t i = 0; i < count; ++i) {
       const int64_t nc = in[i]->n + 1;
       dense[i] = (!dense_only && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
+      // tiny products are launch bound: one dense launch beats GEMM + gather
+      if ((double)fc->Mp * (double)fc->Kp * (double)(nc - dense[i]) * (double)count < 4.0e6) dense[i] = nc;
       total_dense += dense[i];
       any_onehot = any_onehot || dense[i] < nc;
       GatherSet& g = gs[i];
@@ -777,6 +779,10 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
     auto rows_of = [&](int64_t i, GemmRows* r, int64_t* kp) {
       *kp = fc->Kp;
       if (dense_only || in[i]->n_kept < 0 || in[i]->kept_idx == nullptr) return false;
+      // the kept-row list describes the columns before the one-hot block only (a one-hot column has its
+      // 1 in a reset row): usable only if that block is not part of the contraction
+      if (in[i]->oh_from > 0 && dense[i] > in[i]->oh_from) return false;
+      if ((double)fc->Mp * (double)fc->Kp * (double)dense[i] * (double)count < 4.0e6) return false;
       const int64_t k = std::max<int64_t>(round_up(in[i]->n_kept, kLdAlign), kLdAlign);
       if (2 * k > fc->Kp) return false;
       r->kmap = in[i]->kept_idx;

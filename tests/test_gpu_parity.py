@@ -339,3 +339,14 @@ def test_fc_on_sets_with_and_without_structure_hints(nnv, oracle):
     outs = L.reach([relu_d, box_d, relu_d], "approx-star")     # array: not one arena, per-set launches
     for R, oset in zip(outs, (relu_o, box_o, relu_o)):
         assert_close(R.V, oracle.affine_map(oset, W, b).V, "fc on mixed array")
+
+
+@pytest.mark.parametrize("k,shrink", [(1, 1), (2, 1), (3, 1), (5, 64)])
+def test_configs_with_full_dense_contraction(nnv, k, shrink):
+    # the same oracle parity with every FC / conv layer run as the full dense contraction
+    ctx = nnv.default_context()
+    ctx.set_dense_affine(True)
+    try:
+        run_both(k, "relax-star-area", shrink)
+    finally:
+        ctx.set_dense_affine(False)
