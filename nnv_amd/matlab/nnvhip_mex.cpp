@@ -296,6 +296,9 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
   } else if (cmd == "set_timing") {
     need(nrhs, 1, "set_timing");
     check(nnvhip_set_timing(ctx(), mxGetScalar(prhs[1]) != 0));
+  } else if (cmd == "set_dense_affine") {  // 1: FC / conv layers as the full dense contraction (measurement switch)
+    need(nrhs, 1, "set_dense_affine");
+    check(nnvhip_set_dense_affine(ctx(), mxGetScalar(prhs[1]) != 0));
   } else if (cmd == "last_op_time_ms") {
     double ms = 0;
     check(nnvhip_last_op_time_ms(ctx(), &ms));
