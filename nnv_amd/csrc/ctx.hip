@@ -801,8 +801,19 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       GemmRows rows;
       int64_t kp = fc->Kp;
       const bool compact = rows_of(0, &rows, &kp);
-      st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
-                       compact ? &rows : nullptr);
+      BufRef packed;
+      if (compact && fc->Mp > 128) {  // several row tiles would each gather B: pack the kept rows once instead
+        st = c->alloc(sizeof(double) * kp * dense[0], &packed);
+        if (st == NNVHIP_OK) {
+          PackSet ps{in[0]->V, in[0]->kept_idx, packed->as<double>(), in[0]->ld, (int32_t)kp, (int32_t)dense[0]};
+          st = launch_pack_rows(c, 1, &ps);
+          rows.Bk = packed->as<double>();
+          rows.ldbk = kp;
+        }
+      }
+      if (st == NNVHIP_OK)
+        st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
+                         compact ? &rows : nullptr);
       const bool fused = st == NNVHIP_OK && fuse.chunks > 0;
       if (st == NNVHIP_OK && gs[0].m > 0) {
         gs[0].part = fused ? fuse.part->as<double>() + fuse.chunks * 4 * outs[0]->ld : nullptr;
@@ -839,11 +850,33 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         GemmRows rows;
         const int64_t tn = gemm_seg_cols(fc->Mp);
         rows.seg_cols = (int32_t)tn;
+        // several row tiles would each gather the kept rows of B: pack them once per set instead
+        BufRef packed;
+        std::vector<PackSet> packs;
+        std::vector<const double*> bk((size_t)count, nullptr);
+        if (fc->Mp > 128) {
+          int64_t total = 0;
+          for (int64_t i = 0; i < count; ++i)
+            if (rws[i].kmap != nullptr) total += kps[i] * dense[i];
+          if (total > 0) st = c->alloc(sizeof(double) * total, &packed);
+          int64_t pos = 0;
+          for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+            if (rws[i].kmap != nullptr) {
+              bk[i] = packed->as<double>() + pos;
+              packs.push_back(PackSet{in[i]->V, rws[i].kmap, packed->as<double>() + pos, in[i]->ld, (int32_t)kps[i],
+                                      (int32_t)dense[i]});
+              pos += kps[i] * dense[i];
+            }
+          if (st == NNVHIP_OK && !packs.empty()) st = launch_pack_rows(c, (int64_t)packs.size(), packs.data());
+        }
         int64_t off = 0, kp_max = kLdAlign;
         for (int64_t i = 0; i < count; ++i) {
           for (int64_t j = 0; j < dense[i]; j += tn) {
             GemmSeg sg;
             sg.kmap = rws[i].kmap;
+            sg.Bk = bk[i];
+            sg.ldbk = kps[i];
+            sg.col_local0 = j;
             sg.col_base = off + j;
             sg.kp = (int32_t)kps[i];
             sg.valid = (int32_t)std::min<int64_t>(tn, dense[i] - j);
@@ -854,7 +887,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           off += in[i]->n + 1;
         }
         BufRef dsegs;
-        st = c->upload(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
+        if (st == NNVHIP_OK) st = c->upload(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
         if (st == NNVHIP_OK) {
           rows.segs = dsegs->as<GemmSeg>();
           st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, tn * (int64_t)segs.size(),

@@ -29,7 +29,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
                                                         double* __restrict__ rpart,
                                                         const int32_t* __restrict__ kmap,
                                                         const GemmSeg* __restrict__ segs,
-                                                        const int32_t* __restrict__ colmap) {
+                                                        const int32_t* __restrict__ colmap,
+                                                        const double* __restrict__ Bk, int64_t ldbk) {
   constexpr int NT = 64 * WR * WC;  // threads per block
   constexpr int FM = TM / WR / 16;
   constexpr int FN = TN / WC / 16;
@@ -60,13 +61,20 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   // to whole K-tiles with -1; with a segment table every column tile has its own list (one per set).
   int64_t col_base = n0;       // column of B and C behind the tile's first column
   int64_t col_end = ncols;     // first column past the valid ones, in the same numbering as col_base
+  int64_t bk_col0 = n0;        // column of Bk behind the tile's first column
   if (MAPPED && segs != nullptr) {
     const GemmSeg sg = segs[nt];
     kmap = sg.kmap;
     Kp = sg.kp;
     col_base = sg.col_base;
     col_end = sg.col_base + sg.valid;
+    Bk = sg.Bk;
+    ldbk = sg.ldbk;
+    bk_col0 = sg.col_local0;
   }
+  // Bk: the listed rows of B already packed into a matrix of their own (row t of Bk = row kmap[t] of B);
+  // only A is gathered then
+  const bool b_packed = MAPPED && Bk != nullptr;
 
   // ---- global -> register staging ----------------------------------------------------------
   constexpr int A_VEC = TM * KT / 2;           // double2 elements in a W tile
@@ -103,7 +111,9 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
       int j = idx / (KT / 2);
       double2 v = make_double2(0.0, 0.0);
       if (idx < B_VEC && bcol[p] >= 0) {
-        if (MAPPED && kmap != nullptr) {
+        if (b_packed) {
+          v = *reinterpret_cast<const double2*>(Bk + (k0 + 2 * k2) + (bk_col0 + j) * ldbk);
+        } else if (MAPPED && kmap != nullptr) {
           const int ka = kmap[k0 + 2 * k2], kb = kmap[k0 + 2 * k2 + 1];
           if (ka >= 0) v.x = B[ka + bcol[p] * ldb];
           if (kb >= 0) v.y = B[kb + bcol[p] * ldb];
@@ -305,12 +315,13 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
     hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT, true>), dim3((unsigned)grid_x, (unsigned)ksplit),
                        dim3(64 * WR * WC), 0, ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
                        (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
-                       fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, rows->kmap, rows->segs, rows->colmap);
+                       fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, rows->kmap, rows->segs, rows->colmap,
+                       rows->Bk, rows->ldbk);
   else
     hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT, false>), dim3((unsigned)grid_x, (unsigned)ksplit),
                        dim3(64 * WR * WC), 0, ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
                        (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
-                       fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, nullptr, nullptr, nullptr);
+                       fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, nullptr, nullptr, nullptr, nullptr, 0);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, rows && rows->flop > 0.0 ? rows->flop : 2.0 * (double)Mp * (double)Kp * (double)ncols));
   if (ksplit > 1) {
     const int64_t total = Mp * ncols;
@@ -374,6 +385,61 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
     default: return NNV_GEMM(128, 128, 2, 4, 16);
   }
 #undef NNV_GEMM
+}
+
+// Packs the listed rows of every set's leading columns: Vk(t, j) = V(kept[t], j), zero where kept[t] < 0.
+// Lane = two packed rows, the waves of a block interleave columns.  Grid: (row blocks of 128, column
+// chunks, sets).
+__global__ __launch_bounds__(512) void pack_rows_kernel(const PackSet* __restrict__ table, PackSet one, int cols_per_chunk) {
+  const PackSet d = table ? table[blockIdx.z] : one;
+  const int j0 = blockIdx.y * cols_per_chunk;
+  if (j0 >= d.ncols) return;
+  const int j1 = min(d.ncols, j0 + cols_per_chunk);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int t0 = blockIdx.x * 128 + 2 * lane;
+  if (t0 >= d.kp) return;
+  const int ra = d.kept[t0], rb = d.kept[t0 + 1];
+  for (int jb = j0 + 4 * wave; jb < j1; jb += 32) {
+    double2 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      v[u] = make_double2(0.0, 0.0);
+      if (jb + u < j1) {
+        const double* col = d.V + (int64_t)(jb + u) * d.ld;
+        if (ra >= 0) v[u].x = col[ra];
+        if (rb >= 0) v[u].y = col[rb];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (jb + u < j1) *reinterpret_cast<double2*>(d.Vk + t0 + (int64_t)(jb + u) * d.kp) = v[u];
+  }
+}
+
+int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {
+  if (count <= 0) return NNVHIP_OK;
+  if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  int64_t max_kp = 0, max_cols = 0;
+  for (int64_t i = 0; i < count; ++i) {
+    max_kp = std::max<int64_t>(max_kp, sets[i].kp);
+    max_cols = std::max<int64_t>(max_cols, sets[i].ncols);
+  }
+  if (max_kp == 0 || max_cols == 0) return NNVHIP_OK;
+  const int64_t row_blocks = ceil_div(max_kp, 128);
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(max_cols, 32)));
+  const int64_t cpc = ceil_div(max_cols, chunks);
+  chunks = ceil_div(max_cols, cpc);
+  const PackSet* table = nullptr;
+  BufRef tab;
+  if (count > 1) {
+    NNV_TRY(ctx->upload(sets, sizeof(PackSet) * count, &tab));
+    table = tab->as<PackSet>();
+  }
+  hipLaunchKernelGGL(pack_rows_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(512), 0, ctx->stream,
+                     table, sets[0], (int)cpc);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
 }
 
 __global__ void bias_columns_kernel(double* const* __restrict__ cols, const double* __restrict__ bias, int Mp) {

@@ -223,12 +223,19 @@ struct RangeFuse {
 // its columns exist; ncols is then seg_cols * (number of tiles), seg_cols = gemm_seg_cols(Mp).
 struct GemmSeg {
   const int32_t* kmap;
+  const double* Bk;    // the set's packed rows (see GemmRows::Bk), or null
+  int64_t ldbk;
+  int64_t col_local0;  // column of Bk behind the tile's first column
   int64_t col_base;
   int32_t kp;
   int32_t valid;
 };
 struct GemmRows {
   const int32_t* kmap = nullptr;
+  // the listed rows of B packed into their own matrix (row t = row kmap[t] of B, zero where kmap[t] < 0,
+  // leading dimension ldbk): B is then read from here and only A is gathered
+  const double* Bk = nullptr;
+  int64_t ldbk = 0;
   const GemmSeg* segs = nullptr;
   // without segs: product column t reads column colmap[t] of B and writes column colmap[t] of C
   // (columns picked from an arena of sets that share the row list)
@@ -237,6 +244,17 @@ struct GemmRows {
   double flop = 0.0;  // flop actually executed (for the kernel timers)
 };
 int gemm_seg_cols(int64_t Mp);
+// Vk(t, j) = V(kept[t], j) for t < kp (a multiple of 16; zero where kept[t] < 0), j < ncols; Vk has
+// leading dimension kp.
+struct PackSet {
+  const double* V;
+  const int32_t* kept;
+  double* Vk;
+  int64_t ld;
+  int32_t kp;
+  int32_t ncols;
+};
+int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
                 int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse = nullptr,
                 const GemmRows* rows = nullptr);
