@@ -162,7 +162,8 @@ def main():
                 ni, nc = ctypes.c_int64(), ctypes.c_int64()
                 nnv_amd._lib.check(ctx.lib.nnvhip_star_relu_counts(so._h.h, ctypes.byref(ni), ctypes.byref(nc)))
                 kept = N - ni.value - nc.value
-                b += 8.0 * N * (n + 1) * (0 if fused else 1) + 8.0 * kept * (n + 1) + 8.0 * N * (n + 1 + m)
+                # (the m appended unit-vector columns stay implicit unless a later read asks for them)
+                b += 8.0 * N * (n + 1) * (0 if fused else 1) + 8.0 * kept * (n + 1) + 8.0 * N * (n + 1)
             entry["algo_GBps"] = round(b / (per_layer[i] * 1e-3) / 1e9, 1)
             relu_bytes += b
             relu_ms += per_layer[i]

@@ -171,6 +171,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   nnvhip_ctx* c = new nnvhip_ctx();
   c->device = device;
   c->dense_affine = getenv("NNVHIP_DENSE_AFFINE") != nullptr;
+  c->eager_tail = getenv("NNVHIP_EAGER_TAIL") != nullptr;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
@@ -498,6 +499,7 @@ int nnvhip_star_fetch_V(const nnvhip_star* s, double* V) {
   if (!s || !V) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   nnvhip_ctx* c = s->ctx;
   NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(ensure_dense(c, const_cast<nnvhip_star*>(s)));  // implicit columns are written out on first read
   NNV_HIP_TRY(hipMemcpy2DAsync(V, sizeof(double) * s->N, s->V, sizeof(double) * s->ld, sizeof(double) * s->N,
                                s->n + 1, hipMemcpyDeviceToHost, c->stream));
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
@@ -696,7 +698,7 @@ int nnvhip::make_affine_outputs(nnvhip_ctx* c, int64_t count, nnvhip_star* const
   int64_t cols = 0;
   bool contig = true;
   for (int64_t i = 0; i < count; ++i) {
-    if (i > 0 && (in[i]->ld != in[0]->ld || in[i]->V != in[i - 1]->V + (in[i - 1]->n + 1) * in[i - 1]->ld)) contig = false;
+    if (i > 0 && (in[i]->ld != in[0]->ld || in[i]->V != in[i - 1]->V + in[i - 1]->stored_cols() * in[i - 1]->ld)) contig = false;
     cols += in[i]->n + 1;
   }
   BufRef arena;
@@ -774,6 +776,12 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.m = (int32_t)(nc - dense[i]);
       g.pad_ = 0;
     }
+    // sets whose implicit unit-vector columns take part in the contraction after all get them written out
+    for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+      if (dense[i] > in[i]->stored_cols()) {
+        st = ensure_dense(c, in[i]);
+        contig = false;  // the set left its arena
+      }
     // Rows of the dense columns that the ReLU step reset to zero need no contraction either: the
     // GEMM then runs over the kept rows only (used when that at least halves K).
     auto rows_of = [&](int64_t i, GemmRows* r, int64_t* kp) {
@@ -827,7 +835,9 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       std::vector<GemmRows> rws((size_t)count);
       std::vector<int64_t> kps((size_t)count);
       for (int64_t i = 0; i < count; ++i) any_rows = rows_of(i, &rws[i], &kps[i]) || any_rows;
-      if (any_onehot && !any_rows) {
+      bool all_stored = true;
+      for (int64_t i = 0; i < count; ++i) all_stored = all_stored && in[i]->stored_cols() == in[i]->n + 1;
+      if (any_onehot && !any_rows && all_stored) {
         // all sets contract over every row: their dense columns are simply listed (tiles may span sets)
         if (cols >= (int64_t(1) << 31)) st = NNVHIP_ERR_SHAPE;
         std::vector<int32_t> map;
@@ -835,7 +845,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         int64_t off = 0;
         for (int64_t i = 0; i < count; ++i) {
           for (int64_t j = 0; j < dense[i]; ++j) map.push_back((int32_t)(off + j));
-          off += in[i]->n + 1;
+          off += in[i]->n + 1;  // box stars: all columns stored, input and output arenas laid out alike
         }
         BufRef cmap;
         if (st == NNVHIP_OK) st = c->upload(map.data(), sizeof(int32_t) * map.size(), &cmap);
@@ -845,7 +855,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, total_dense, fc->Kp, bias,
                            nullptr, &rows);
         }
-      } else if (any_rows) {
+      } else if (any_rows || any_onehot) {
         std::vector<GemmSeg> segs;
         GemmRows rows;
         const int64_t tn = gemm_seg_cols(fc->Mp);
@@ -869,7 +879,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             }
           if (st == NNVHIP_OK && !packs.empty()) st = launch_pack_rows(c, (int64_t)packs.size(), packs.data());
         }
-        int64_t off = 0, kp_max = kLdAlign;
+        int64_t off = 0, off_in = 0, kp_max = kLdAlign;
         for (int64_t i = 0; i < count; ++i) {
           for (int64_t j = 0; j < dense[i]; j += tn) {
             GemmSeg sg;
@@ -877,6 +887,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             sg.Bk = bk[i];
             sg.ldbk = kps[i];
             sg.col_local0 = j;
+            sg.b_col_base = off_in + j;
             sg.col_base = off + j;
             sg.kp = (int32_t)kps[i];
             sg.valid = (int32_t)std::min<int64_t>(tn, dense[i] - j);
@@ -885,6 +896,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           rows.flop += 2.0 * (double)fc->Mp * (double)kps[i] * (double)dense[i];
           kp_max = std::max(kp_max, kps[i]);
           off += in[i]->n + 1;
+          off_in += in[i]->stored_cols();
         }
         BufRef dsegs;
         if (st == NNVHIP_OK) st = c->upload(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
@@ -974,6 +986,8 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
   for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
     const int64_t nc = in[i]->n + 1;
     const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
+    if (dense > in[i]->stored_cols()) st = ensure_dense(c, in[i]);
+    if (st != NNVHIP_OK) break;
     stamps[i].idx = in[i]->oh_idx;
     stamps[i].scale = in[i]->oh_scale;
     stamps[i].out = outs[i]->V + dense * outs[i]->ld;

@@ -231,9 +231,11 @@ template <class Launch>
 static int run_row_layer(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, nnvhip_star** out, int64_t Nout,
                          int64_t rows_per_block, int min_cols_per_chunk, Launch launch) {
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
-  for (int64_t i = 0; i < count; ++i)
+  for (int64_t i = 0; i < count; ++i) {
     if (in[i]->N != in[0]->N || in[i]->ld != in[0]->ld)
       NNV_FAIL(NNVHIP_ERR_SHAPE, "sets of one array must have the same dimension");
+    NNV_TRY(ensure_dense(c, in[i]));  // these passes read every column
+  }
   std::vector<nnvhip_star*> outs;
   bool contig = false;
   int64_t cols = 0;

@@ -62,12 +62,14 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   int64_t col_base = n0;       // column of B and C behind the tile's first column
   int64_t col_end = ncols;     // first column past the valid ones, in the same numbering as col_base
   int64_t bk_col0 = n0;        // column of Bk behind the tile's first column
+  int64_t b_col_base = n0;     // column of B behind the tile's first column
   if (MAPPED && segs != nullptr) {
     const GemmSeg sg = segs[nt];
     kmap = sg.kmap;
     Kp = sg.kp;
     col_base = sg.col_base;
     col_end = sg.col_base + sg.valid;
+    b_col_base = sg.b_col_base;
     Bk = sg.Bk;
     ldbk = sg.ldbk;
     bk_col0 = sg.col_local0;
@@ -86,8 +88,9 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   int64_t bcol[B_PASS];
 #pragma unroll
   for (int p = 0; p < B_PASS; ++p) {
-    const int64_t col = col_base + (tid + p * NT) / (KT / 2);
-    bcol[p] = col < col_end ? ((MAPPED && colmap != nullptr) ? (int64_t)colmap[col] : col) : -1;
+    const int64_t jl = (tid + p * NT) / (KT / 2);
+    const int64_t col = col_base + jl;
+    bcol[p] = col < col_end ? ((MAPPED && colmap != nullptr) ? (int64_t)colmap[col] : b_col_base + jl) : -1;
   }
 
   auto load_tiles = [&](int k0) {

@@ -104,6 +104,8 @@ struct nnvhip_ctx {
   // FC layers as the full dense contraction (no skipping of structural zeros); default from the
   // environment variable NNVHIP_DENSE_AFFINE
   bool dense_affine = false;
+  // ReLU outputs always store their appended unit-vector columns (environment NNVHIP_EAGER_TAIL)
+  bool eager_tail = false;
   // per-layer timing
   bool timing = false;         // per-layer events (nnvhip_last_op_time_ms)
   bool kernel_timing = false;  // additionally one event pair per launch of the timed kernel groups
@@ -141,6 +143,11 @@ struct nnvhip_star {
   int64_t ld = 0;  // leading dimension of V (multiple of 16, >= N)
   nnvhip::BufRef Vbuf;
   double* V = nullptr;  // N x (n+1), may point inside a shared arena
+  // Number of columns of V that exist in memory.  A ReLU output keeps its appended unit-vector columns
+  // [oh_from, n] implicit (vcols = oh_from): the FC and conv maps never read them, and whoever needs the
+  // full matrix calls ensure_dense() first.  -1 = all n+1 columns.
+  int64_t vcols = -1;
+  int64_t stored_cols() const { return vcols >= 0 ? vcols : n + 1; }
   nnvhip::BufRef pbuf;
   double* plb = nullptr;
   double* pub = nullptr;
@@ -226,7 +233,8 @@ struct GemmSeg {
   const double* Bk;    // the set's packed rows (see GemmRows::Bk), or null
   int64_t ldbk;
   int64_t col_local0;  // column of Bk behind the tile's first column
-  int64_t col_base;
+  int64_t b_col_base;  // column of B behind the tile's first column (input arena)
+  int64_t col_base;    // column of C behind the tile's first column (output arena)
   int32_t kp;
   int32_t valid;
 };
@@ -308,6 +316,8 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks);
 
 // relu.hip
+// Makes all n+1 columns of V exist (writes the implicit unit-vector columns into a fresh buffer).
+int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s);
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out);
 int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host);
 

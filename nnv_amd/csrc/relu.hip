@@ -49,6 +49,8 @@ struct ReluDesc {
   int32_t order;
   int32_t cols_per_chunk;
   int32_t row_waves;  // apply pass: waves of a block laid along rows (1, 2, 4 or 8); the rest along columns
+  int32_t write_tail; // apply pass: 1 = store the appended unit-vector columns, 0 = leave them implicit
+  int32_t pad3_;
 };
 
 // Posts the counts to the host mailbox: payload first, system-scope fence, then the sequence number
@@ -484,7 +486,7 @@ constexpr int kApplyWaves = 8;  // waves per block of the apply pass
 
 __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
   const ReluDesc d = table ? table[blockIdx.z] : one;
-  const int ncols_out = d.ncols_in + d.m;
+  const int ncols_out = d.ncols_in + (d.write_tail ? d.m : 0);  // columns of V' that are stored
   const int j0 = blockIdx.y * d.cols_per_chunk;
   if (j0 >= ncols_out) return;
   const int j1 = min(ncols_out, j0 + d.cols_per_chunk);
@@ -526,6 +528,16 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
         d.lbub[d.ld_lbub + i] = ub;
       }
     }
+    if (!d.write_tail && blockIdx.y == 0) {  // implicit columns: their predicate bounds all the same
+      for (int i = (int)threadIdx.x; i < d.m; i += 64 * kApplyWaves) {
+        const int neuron = d.cross_idx[i];
+        const double ub = d.ub[neuron];
+        d.plb_out[n_in + i] = 0.0;
+        d.pub_out[n_in + i] = ub;
+        d.lbub[i] = d.lb[neuron];
+        d.lbub[d.ld_lbub + i] = ub;
+      }
+    }
   }
   // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
   for (int jb = j0 + 4 * wcol; jb < j1; jb += 4 * col_waves) {
@@ -555,8 +567,36 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
   }
 }
 
+// unit-vector columns of a set: column j (of ncols) = e_idx[j]
+__global__ void onehot_columns_kernel(double* __restrict__ V, int64_t ld, const int32_t* __restrict__ idx, int ncols) {
+  for (int j = blockIdx.y; j < ncols; j += gridDim.y) {
+    const int hot = idx[j];
+    for (int64_t r = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; r < ld; r += (int64_t)gridDim.x * blockDim.x)
+      V[r + (int64_t)j * ld] = r == hot ? 1.0 : 0.0;
+  }
+}
+
+int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s) {
+  const int64_t have = s->stored_cols();
+  if (have == s->n + 1) return NNVHIP_OK;
+  if (s->oh_idx == nullptr || s->oh_from != have || s->oh_scale != nullptr)
+    NNV_FAIL(NNVHIP_ERR_ARG, "internal: implicit columns without their description");
+  BufRef full;
+  NNV_TRY(ctx->alloc(sizeof(double) * s->ld * (s->n + 1), &full));
+  NNV_HIP_TRY(hipMemcpyAsync(full->ptr, s->V, sizeof(double) * s->ld * have, hipMemcpyDeviceToDevice, ctx->stream));
+  const int m = (int)(s->n + 1 - have);
+  hipLaunchKernelGGL(onehot_columns_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(s->ld, 256), 64), (unsigned)std::min(m, 4096)),
+                     dim3(256), 0, ctx->stream, full->as<double>() + have * s->ld, s->ld, s->oh_idx, m);
+  NNV_HIP_TRY(hipGetLastError());
+  s->Vbuf = full;
+  s->V = full->as<double>();
+  s->vcols = -1;
+  return NNVHIP_OK;
+}
+
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  for (int64_t i = 0; i < count; ++i) NNV_TRY(ensure_dense(ctx, in[i]));
   NNV_TRY(compute_ranges(ctx, count, in));
   const int64_t N = in[0]->N;
   const int64_t ld = in[0]->ld;
@@ -661,7 +701,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   std::vector<int64_t> col_off(count), pred_off(count), lbub_off(count);
   for (int64_t i = 0; i < count; ++i) {
     const int64_t m = counts[2 * i];
-    const int64_t ncols_out = in[i]->n + 1 + m;
+    const int64_t ncols_out = in[i]->n + 1 + (ctx->eager_tail ? m : 0);  // stored columns
     const int64_t ldr = round_up(std::max<int64_t>(m, 1), kLdAlign);
     col_off[i] = total_cols;
     pred_off[i] = total_pred;
@@ -702,6 +742,8 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.ld_lbub = ldr;
     d.cols_per_chunk = (int32_t)cpc;
     d.row_waves = row_waves;
+    d.write_tail = ctx->eager_tail ? 1 : 0;
+    d.pad3_ = 0;
   }
   if (count > 1) {
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
@@ -718,7 +760,8 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   double bytes = 0.0;  // algorithmic: read the rows that are kept, write N x (n+1+m)
   for (int64_t i = 0; i < count; ++i) {
     const double kept = (double)(N - counts[2 * i] - counts[2 * i + 1]);
-    bytes += 8.0 * kept * (double)(in[i]->n + 1) + 8.0 * (double)N * (double)(in[i]->n + 1 + descs[i].m);
+    bytes += 8.0 * kept * (double)(in[i]->n + 1) +
+             8.0 * (double)N * (double)(in[i]->n + 1 + (ctx->eager_tail ? descs[i].m : 0));
   }
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(64 * kApplyWaves), 0,
@@ -743,6 +786,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->oh_from = in[i]->n + 1;
       o->oh_idx_buf = idx_bufs[i];
       o->oh_idx = idx_bufs[i]->as<int32_t>();
+      if (!ctx->eager_tail) o->vcols = in[i]->n + 1;  // ... and exist only as that list
     }
     // rows of the leading columns that were not reset
     o->n_kept = N - counts[2 * i] - counts[2 * i + 1];

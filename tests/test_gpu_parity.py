@@ -350,3 +350,29 @@ def test_configs_with_full_dense_contraction(nnv, k, shrink):
         run_both(k, "relax-star-area", shrink)
     finally:
         ctx.set_dense_affine(False)
+
+
+def test_relu_output_consumers_that_need_every_column(nnv, oracle):
+    # a ReLU output keeps its appended unit-vector columns implicit; ranges, another ReLU, a
+    # row-wise layer and a property read must all see the full matrix
+    rs = np.random.RandomState(91)
+    N, n = 300, 40
+    V, C, d, lb, ub = _rand_star_arrays(rs, N, n)
+    S = nnv.Star(V, C, d, lb, ub)
+    O = oracle.OStar(V, C, d, lb, ub)
+    R = nnv.PosLin.reach(S, "relax-star-area", [], 1)
+    E = oracle.reach_relaxed_star(O, "relax-star-area", 1.0)
+    assert E.nVar > n                                   # some neurons cross
+    rl, ru = R.estimateRanges()                         # before any read of R.V
+    el, eu = oracle.estimate_ranges(E)
+    assert_close(rl, el, "ranges of a ReLU output (lb)")
+    assert_close(ru, eu, "ranges of a ReLU output (ub)")
+    R2 = nnv.PosLin.reach(nnv.PosLin.reach(S, "relax-star-area", [], 1), "relax-star-range", [], 1)
+    E2 = oracle.reach_relaxed_star(E, "relax-star-range", 1.0)
+    assert np.array_equal(R2.V, E2.V)
+    mean, var = rs.randn(N), rs.rand(N) + 0.5
+    BN = nnv.BatchNormalizationLayer(NumChannels=N, TrainedMean=mean, TrainedVariance=var)
+    R3 = BN.reach(nnv.PosLin.reach(S, "relax-star-area", [], 1), "approx-star")
+    E3 = oracle.batchnorm_reach(E, mean, var, 1e-5, np.ones(N), np.zeros(N))
+    assert np.array_equal(R3.V, E3.V)
+    assert np.array_equal(R.V, E.V)                     # property read of the first output, last
