@@ -696,12 +696,15 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     memcpy(counts.data(), hc, sizeof(int32_t) * 2 * count);
   }
 
+  // the appended unit-vector columns are stored only on request or when the FC / conv maps are told to
+  // contract over every column anyway
+  const bool eager_tail = ctx->eager_tail || ctx->dense_affine;
   // outputs: one V arena, one predicate-bound buffer, one buffer for the crossing bounds
   int64_t total_cols = 0, total_pred = 0, total_lbub = 0, max_cols = 0, max_m = 0;
   std::vector<int64_t> col_off(count), pred_off(count), lbub_off(count);
   for (int64_t i = 0; i < count; ++i) {
     const int64_t m = counts[2 * i];
-    const int64_t ncols_out = in[i]->n + 1 + (ctx->eager_tail ? m : 0);  // stored columns
+    const int64_t ncols_out = in[i]->n + 1 + (eager_tail ? m : 0);  // stored columns
     const int64_t ldr = round_up(std::max<int64_t>(m, 1), kLdAlign);
     col_off[i] = total_cols;
     pred_off[i] = total_pred;
@@ -742,7 +745,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.ld_lbub = ldr;
     d.cols_per_chunk = (int32_t)cpc;
     d.row_waves = row_waves;
-    d.write_tail = ctx->eager_tail ? 1 : 0;
+    d.write_tail = eager_tail ? 1 : 0;
     d.pad3_ = 0;
   }
   if (count > 1) {
@@ -761,7 +764,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   for (int64_t i = 0; i < count; ++i) {
     const double kept = (double)(N - counts[2 * i] - counts[2 * i + 1]);
     bytes += 8.0 * kept * (double)(in[i]->n + 1) +
-             8.0 * (double)N * (double)(in[i]->n + 1 + (ctx->eager_tail ? descs[i].m : 0));
+             8.0 * (double)N * (double)(in[i]->n + 1 + (eager_tail ? descs[i].m : 0));
   }
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(64 * kApplyWaves), 0,
@@ -786,7 +789,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->oh_from = in[i]->n + 1;
       o->oh_idx_buf = idx_bufs[i];
       o->oh_idx = idx_bufs[i]->as<int32_t>();
-      if (!ctx->eager_tail) o->vcols = in[i]->n + 1;  // ... and exist only as that list
+      if (!eager_tail) o->vcols = in[i]->n + 1;  // ... and exist only as that list
     }
     // rows of the leading columns that were not reset
     o->n_kept = N - counts[2 * i] - counts[2 * i + 1];
