@@ -172,6 +172,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->device = device;
   c->dense_affine = getenv("NNVHIP_DENSE_AFFINE") != nullptr;
   c->eager_tail = getenv("NNVHIP_EAGER_TAIL") != nullptr;
+  c->eager_rows = getenv("NNVHIP_EAGER_ROWS") != nullptr;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
@@ -777,22 +778,39 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.pad_ = 0;
     }
     // sets whose implicit unit-vector columns take part in the contraction after all get them written out
-    for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
-      if (dense[i] > in[i]->stored_cols()) {
-        st = ensure_dense(c, in[i]);
-        contig = false;  // the set left its arena
-      }
+    // (which also runs a pending row reset)
+    std::vector<nnvhip_star*> full;
+    for (int64_t i = 0; i < count; ++i)
+      if (dense[i] > in[i]->stored_cols() || (dense_only && in[i]->rows_pending)) full.push_back(in[i]);
+    if (!full.empty()) {
+      st = ensure_dense_batch(c, (int64_t)full.size(), full.data());
+      contig = true;  // the sets moved: look again
+      for (int64_t i = 1; i < count; ++i)
+        if (in[i]->ld != in[0]->ld || in[i]->V != in[i - 1]->V + in[i - 1]->stored_cols() * in[i - 1]->ld) contig = false;
+    }
     // Rows of the dense columns that the ReLU step reset to zero need no contraction either: the
     // GEMM then runs over the kept rows only (used when that at least halves K).
-    auto rows_of = [&](int64_t i, GemmRows* r, int64_t* kp) {
+    // *pack: gather the listed rows into a matrix of their own first (several row tiles of W would each
+    // gather them otherwise; and a long list read through the map is slow, so a set that only takes this
+    // route because its reset is pending always packs)
+    auto rows_of = [&](int64_t i, GemmRows* r, int64_t* kp, bool* pack) {
       *kp = fc->Kp;
-      if (dense_only || in[i]->n_kept < 0 || in[i]->kept_idx == nullptr) return false;
+      *pack = fc->Mp > 128;
+      // a set whose row reset is still pending shares its matrix with the ReLU's input: only the listed
+      // rows may be read
+      const bool must = in[i]->rows_pending;
+      if (!must && (dense_only || in[i]->n_kept < 0 || in[i]->kept_idx == nullptr)) return false;
       // the kept-row list describes the columns before the one-hot block only (a one-hot column has its
       // 1 in a reset row): usable only if that block is not part of the contraction
       if (in[i]->oh_from > 0 && dense[i] > in[i]->oh_from) return false;
-      if ((double)fc->Mp * (double)fc->Kp * (double)dense[i] * (double)count < 4.0e6) return false;
+      const bool tiny = (double)fc->Mp * (double)fc->Kp * (double)dense[i] * (double)count < 4.0e6;
+      if (!must && tiny) return false;
       const int64_t k = std::max<int64_t>(round_up(in[i]->n_kept, kLdAlign), kLdAlign);
-      if (2 * k > fc->Kp) return false;
+      if (!must && 2 * k > fc->Kp) return false;
+      if (tiny)
+        *pack = false;  // launch bound: read through the map
+      else if (must && 2 * k > fc->Kp)
+        *pack = true;
       r->kmap = in[i]->kept_idx;
       r->flop = 2.0 * (double)fc->Mp * (double)k * (double)dense[i];
       *kp = k;
@@ -808,9 +826,10 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       fuse.extra_chunks = gch;
       GemmRows rows;
       int64_t kp = fc->Kp;
-      const bool compact = rows_of(0, &rows, &kp);
+      bool pack = false;
+      const bool compact = rows_of(0, &rows, &kp, &pack);
       BufRef packed;
-      if (compact && fc->Mp > 128) {  // several row tiles would each gather B: pack the kept rows once instead
+      if (compact && pack) {
         st = c->alloc(sizeof(double) * kp * dense[0], &packed);
         if (st == NNVHIP_OK) {
           PackSet ps{in[0]->V, in[0]->kept_idx, packed->as<double>(), in[0]->ld, (int32_t)kp, (int32_t)dense[0]};
@@ -834,7 +853,12 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       bool any_rows = false;
       std::vector<GemmRows> rws((size_t)count);
       std::vector<int64_t> kps((size_t)count);
-      for (int64_t i = 0; i < count; ++i) any_rows = rows_of(i, &rws[i], &kps[i]) || any_rows;
+      std::vector<char> pk((size_t)count, 0);
+      for (int64_t i = 0; i < count; ++i) {
+        bool pack = false;
+        any_rows = rows_of(i, &rws[i], &kps[i], &pack) || any_rows;
+        pk[i] = pack && rws[i].kmap != nullptr;
+      }
       bool all_stored = true;
       for (int64_t i = 0; i < count; ++i) all_stored = all_stored && in[i]->stored_cols() == in[i]->n + 1;
       if (any_onehot && !any_rows && all_stored) {
@@ -864,14 +888,14 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         BufRef packed;
         std::vector<PackSet> packs;
         std::vector<const double*> bk((size_t)count, nullptr);
-        if (fc->Mp > 128) {
+        {
           int64_t total = 0;
           for (int64_t i = 0; i < count; ++i)
-            if (rws[i].kmap != nullptr) total += kps[i] * dense[i];
+            if (pk[i]) total += kps[i] * dense[i];
           if (total > 0) st = c->alloc(sizeof(double) * total, &packed);
           int64_t pos = 0;
           for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
-            if (rws[i].kmap != nullptr) {
+            if (pk[i]) {
               bk[i] = packed->as<double>() + pos;
               packs.push_back(PackSet{in[i]->V, rws[i].kmap, packed->as<double>() + pos, in[i]->ld, (int32_t)kps[i],
                                       (int32_t)dense[i]});
@@ -940,7 +964,18 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
         GemmRows rows;
         int64_t kp = fc->Kp;
-        const bool compact = rows_of(i, &rows, &kp);
+        bool pack = false;
+        const bool compact = rows_of(i, &rows, &kp, &pack);
+        BufRef packed;
+        if (compact && pack) {
+          st = c->alloc(sizeof(double) * kp * dense[i], &packed);
+          if (st != NNVHIP_OK) break;
+          PackSet ps{in[i]->V, in[i]->kept_idx, packed->as<double>(), in[i]->ld, (int32_t)kp, (int32_t)dense[i]};
+          st = launch_pack_rows(c, 1, &ps);
+          if (st != NNVHIP_OK) break;
+          rows.Bk = packed->as<double>();
+          rows.ldbk = kp;
+        }
         st = launch_gemm(c, Wd, fc->Mp, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, fc->Mp, dense[i], kp, bias, nullptr,
                          compact ? &rows : nullptr);
         if (st == NNVHIP_OK && gs[i].m > 0) st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[i]->ld, 1, &gs[i], 0);
@@ -983,11 +1018,24 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
   std::vector<ConvStampSet> stamps((size_t)count);
   bool any_stamps = false;
   int64_t max_m = 0;
+  {
+    // the implicit GEMM reads whole images: pending row resets are run first, and sets whose unit-vector
+    // columns take part in the contraction get those written out
+    std::vector<nnvhip_star*> full, prefix;
+    for (int64_t i = 0; i < count; ++i) {
+      const int64_t nc = in[i]->n + 1;
+      const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
+      if (dense > in[i]->stored_cols())
+        full.push_back(in[i]);
+      else if (in[i]->rows_pending)
+        prefix.push_back(in[i]);
+    }
+    if (st == NNVHIP_OK && !full.empty()) st = ensure_dense_batch(c, (int64_t)full.size(), full.data());
+    if (st == NNVHIP_OK && !prefix.empty()) st = ensure_dense_batch(c, (int64_t)prefix.size(), prefix.data(), false);
+  }
   for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
     const int64_t nc = in[i]->n + 1;
     const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
-    if (dense > in[i]->stored_cols()) st = ensure_dense(c, in[i]);
-    if (st != NNVHIP_OK) break;
     stamps[i].idx = in[i]->oh_idx;
     stamps[i].scale = in[i]->oh_scale;
     stamps[i].out = outs[i]->V + dense * outs[i]->ld;

@@ -234,8 +234,8 @@ static int run_row_layer(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, n
   for (int64_t i = 0; i < count; ++i) {
     if (in[i]->N != in[0]->N || in[i]->ld != in[0]->ld)
       NNV_FAIL(NNVHIP_ERR_SHAPE, "sets of one array must have the same dimension");
-    NNV_TRY(ensure_dense(c, in[i]));  // these passes read every column
   }
+  NNV_TRY(ensure_dense_batch(c, count, in));  // these passes read every column
   std::vector<nnvhip_star*> outs;
   bool contig = false;
   int64_t cols = 0;

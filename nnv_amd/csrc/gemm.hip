@@ -301,7 +301,8 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   int64_t ksplit = 1;
   if (blocks < 128 && nk >= 8) ksplit = std::min<int64_t>(std::min<int64_t>(16, nk / 4), ceil_div(512, blocks));
   if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
-  if (rows != nullptr) ksplit = 1;  // the split-K reduction knows nothing of row or column maps
+  // the split-K workspace is laid out for one plain column range: no segment tables, no column maps
+  if (rows != nullptr && (rows->segs != nullptr || rows->colmap != nullptr)) ksplit = 1;
   if (rows != nullptr && rows->segs != nullptr && rows->seg_cols != TN)
     NNV_FAIL(NNVHIP_ERR_ARG, "internal: segment table built for another tile width");
   BufRef ws;

@@ -106,6 +106,9 @@ struct nnvhip_ctx {
   bool dense_affine = false;
   // ReLU outputs always store their appended unit-vector columns (environment NNVHIP_EAGER_TAIL)
   bool eager_tail = false;
+  // ReLU outputs reset their rows at once instead of leaving that to the first reader that needs the
+  // whole matrix (environment NNVHIP_EAGER_ROWS; implied by the two switches above)
+  bool eager_rows = false;
   // per-layer timing
   bool timing = false;         // per-layer events (nnvhip_last_op_time_ms)
   bool kernel_timing = false;  // additionally one event pair per launch of the timed kernel groups
@@ -148,6 +151,13 @@ struct nnvhip_star {
   // full matrix calls ensure_dense() first.  -1 = all n+1 columns.
   int64_t vcols = -1;
   int64_t stored_cols() const { return vcols >= 0 ? vcols : n + 1; }
+  // A ReLU output may also leave the reset of its rows pending: V then still points at the input set's
+  // matrix (shared, never written) and every row that kept_idx does not list counts as zero.  The FC map
+  // contracts over the listed rows only and never notices; everybody else calls ensure_dense(), which
+  // runs the pending pass (it needs the per-row classification cls) into a buffer of the set's own.
+  bool rows_pending = false;
+  nnvhip::BufRef cls_buf;
+  const int32_t* cls = nullptr;
   nnvhip::BufRef pbuf;
   double* plb = nullptr;
   double* pub = nullptr;
@@ -316,8 +326,10 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks);
 
 // relu.hip
-// Makes all n+1 columns of V exist (writes the implicit unit-vector columns into a fresh buffer).
-int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s);
+// Makes V a plain stored matrix: runs a pending row reset and, with need_tail, writes the implicit
+// unit-vector columns, into a fresh buffer.  The batch form keeps the sets of an array back to back.
+int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s, bool need_tail = true);
+int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail = true);
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out);
 int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host);
 

@@ -292,7 +292,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
       if (!dup) todo.push_back(s[i]);
     }
   if (todo.empty()) return NNVHIP_OK;
-  for (auto* t : todo) NNV_TRY(ensure_dense(ctx, t));  // the scan reads every column
+  NNV_TRY(ensure_dense_batch(ctx, (int64_t)todo.size(), todo.data()));  // the scan reads every column
   const int64_t nset = (int64_t)todo.size();
   if (nset > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
   int64_t ld = todo[0]->ld;

@@ -50,7 +50,7 @@ struct ReluDesc {
   int32_t cols_per_chunk;
   int32_t row_waves;  // apply pass: waves of a block laid along rows (1, 2, 4 or 8); the rest along columns
   int32_t write_tail; // apply pass: 1 = store the appended unit-vector columns, 0 = leave them implicit
-  int32_t pad3_;
+  int32_t write_bounds; // apply pass: 1 = also write the predicate bounds and the crossing neurons' (lb, ub)
 };
 
 // Posts the counts to the host mailbox: payload first, system-scope fence, then the sequence number
@@ -229,6 +229,23 @@ __device__ __forceinline__ void sort_small_desc(long long* skey, int* sidx, int 
   if (tid < m) out[tid] = idx;
 }
 
+// Entry j of the output's predicate bounds, new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]
+// (nn/funcs/PosLin.m:737-738), plus the (lb, ub) of crossing neuron j - n_in that the constraint rows need.
+__device__ __forceinline__ void write_pred_bound(const ReluDesc& d, int n_in, int j) {
+  if (j < n_in) {
+    d.plb_out[j] = d.plb_in[j];
+    d.pub_out[j] = d.pub_in[j];
+  } else {
+    const int i = j - n_in;
+    const int neuron = d.cross_idx[i];
+    const double ub = d.ub[neuron];
+    d.plb_out[j] = 0.0;
+    d.pub_out[j] = ub;
+    d.lbub[i] = d.lb[neuron];
+    d.lbub[d.ld_lbub + i] = ub;
+  }
+}
+
 // One 1024-thread block per set.  SORT_CAP > 0: crossing lists of up to SORT_CAP neurons are sorted
 // here by a bitonic network in LDS; longer lists are left to the tiled rank kernels.
 template <int SORT_CAP>
@@ -313,6 +330,11 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
       sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
     else
       bitonic_sort_desc<SORT_CAP>(skey, sidx, m, tid, d.cross_idx);
+  }
+  if (d.write_bounds) {  // the output buffers were sized for the worst case: finish the set here
+    __syncthreads();     // cross_idx is complete
+    const int n_in = d.ncols_in - 1;
+    for (int j = tid; j < n_in + m; j += 1024) write_pred_bound(d, n_in, j);
   }
 }
 
@@ -511,7 +533,7 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
   const int n_in = d.ncols_in - 1;
   // predicate bounds and the (lb, ub) of the crossing neurons: one thread per column of this block's
   // chunk, done by the first row block only
-  if (blockIdx.x == 0) {
+  if (blockIdx.x == 0 && d.write_bounds) {
     for (int j = j0 + (int)threadIdx.x; j < j1; j += 64 * kApplyWaves) {
       if (j < d.ncols_in) {
         if (j >= 1) {
@@ -576,9 +598,56 @@ __global__ void onehot_columns_kernel(double* __restrict__ V, int64_t ld, const 
   }
 }
 
-int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s) {
+// Predicate bounds of the output and (lb, ub) of the crossing neurons, for the ReLU step that leaves
+// the row reset pending: new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)].
+__global__ __launch_bounds__(256) void relu_bounds_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+  const ReluDesc d = table ? table[blockIdx.y] : one;
+  const int n_in = d.ncols_in - 1;
+  for (int j = blockIdx.x * 256 + threadIdx.x; j < n_in + d.m; j += gridDim.x * 256) write_pred_bound(d, n_in, j);
+}
+
+// The apply pass over an array of sets with a common leading dimension.  The descriptors carry Vin,
+// Vout, cls, cross_idx, ncols_in, m, ld, write_tail and write_bounds (plus what the bounds need);
+// the column chunking is chosen here.
+static int launch_apply(nnvhip_ctx* ctx, int64_t count, std::vector<ReluDesc>& descs, double bytes) {
+  const int64_t ld = descs[0].ld;
+  int64_t max_cols = 0;
+  for (int64_t i = 0; i < count; ++i)
+    max_cols = std::max<int64_t>(max_cols, descs[i].ncols_in + (descs[i].write_tail ? descs[i].m : 0));
+  // a couple of thousand blocks, at least two steps per wave
+  int row_waves = ld >= 8 * kApplyRows ? 8 : ld >= 4 * kApplyRows ? 4 : ld >= 2 * kApplyRows ? 2 : 1;
+  if (const char* e = getenv("NNVHIP_APPLY_ROW_WAVES")) {
+    const int v = atoi(e);
+    row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
+  }
+  const int64_t row_blocks = ceil_div(ld, kApplyRows * row_waves);
+  const int64_t min_cpc = (const int64_t)8 * (kApplyWaves / row_waves);  // two 4-column steps per wave
+  int64_t want_blocks = 8192;
+  if (const char* e = getenv("NNVHIP_APPLY_BLOCKS")) want_blocks = std::max(1, atoi(e));
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * count), ceil_div(max_cols, min_cpc)));
+  const int64_t cpc = ceil_div(max_cols, chunks);
+  chunks = ceil_div(max_cols, cpc);
+  for (int64_t i = 0; i < count; ++i) {
+    descs[i].cols_per_chunk = (int32_t)cpc;
+    descs[i].row_waves = row_waves;
+  }
+  const ReluDesc* table = nullptr;
+  BufRef tab;
+  if (count > 1) {
+    NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
+    table = tab->as<ReluDesc>();
+  }
+  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
+  hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(64 * kApplyWaves), 0,
+                     ctx->stream, table, descs[0]);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 3, bytes));
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+// implicit unit-vector columns of a set whose rows are in place: copy and append
+static int write_tail_columns(nnvhip_ctx* ctx, nnvhip_star* s) {
   const int64_t have = s->stored_cols();
-  if (have == s->n + 1) return NNVHIP_OK;
   if (s->oh_idx == nullptr || s->oh_from != have || s->oh_scale != nullptr)
     NNV_FAIL(NNVHIP_ERR_ARG, "internal: implicit columns without their description");
   BufRef full;
@@ -594,9 +663,74 @@ int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s) {
   return NNVHIP_OK;
 }
 
+int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail) {
+  // sets with a pending row reset: one arena and one apply launch per leading dimension
+  std::vector<nnvhip_star*> pend;
+  for (int64_t i = 0; i < count; ++i) {
+    nnvhip_star* s = sets[i];
+    if (s->rows_pending) {
+      if (std::find(pend.begin(), pend.end(), s) == pend.end()) pend.push_back(s);
+    } else if (need_tail && s->stored_cols() != s->n + 1) {
+      NNV_TRY(write_tail_columns(ctx, s));
+    }
+  }
+  while (!pend.empty()) {
+    std::vector<nnvhip_star*> grp, rest;
+    for (auto* s : pend) (s->ld == pend[0]->ld ? grp : rest).push_back(s);
+    const int64_t ld = grp[0]->ld;
+    int64_t total_cols = 0;
+    std::vector<ReluDesc> descs(grp.size());
+    double bytes = 0.0;
+    for (size_t i = 0; i < grp.size(); ++i) {
+      nnvhip_star* s = grp[i];
+      const int64_t have = s->stored_cols();
+      const int64_t m = s->n + 1 - have;
+      if (s->cls == nullptr || (m > 0 && (s->oh_idx == nullptr || s->oh_from != have)) || s->n_kept < 0)
+        NNV_FAIL(NNVHIP_ERR_ARG, "internal: pending row reset without its description");
+      ReluDesc& d = descs[i];
+      d = ReluDesc{};
+      d.Vin = s->V;
+      d.cls = const_cast<int32_t*>(s->cls);
+      d.cross_idx = const_cast<int32_t*>(s->oh_idx);
+      d.ld = ld;
+      d.N = (int32_t)s->N;
+      d.ncols_in = (int32_t)have;
+      d.m = (int32_t)m;
+      d.write_tail = need_tail ? 1 : 0;
+      d.write_bounds = 0;
+      total_cols += have + (need_tail ? m : 0);
+      bytes += 8.0 * (double)s->n_kept * (double)have + 8.0 * (double)s->N * (double)(have + (need_tail ? m : 0));
+    }
+    BufRef arena;
+    NNV_TRY(ctx->alloc(sizeof(double) * ld * total_cols, &arena));
+    int64_t off = 0;
+    for (size_t i = 0; i < grp.size(); ++i) {
+      descs[i].Vout = arena->as<double>() + off * ld;
+      off += descs[i].ncols_in + (need_tail ? descs[i].m : 0);
+    }
+    NNV_TRY(launch_apply(ctx, (int64_t)grp.size(), descs, bytes));
+    for (size_t i = 0; i < grp.size(); ++i) {
+      nnvhip_star* s = grp[i];
+      s->Vbuf = arena;
+      s->V = descs[i].Vout;
+      s->rows_pending = false;
+      s->cls_buf.reset();
+      s->cls = nullptr;
+      if (need_tail) s->vcols = -1;
+    }
+    pend.swap(rest);
+  }
+  return NNVHIP_OK;
+}
+
+int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s, bool need_tail) {
+  if (!s->rows_pending && (!need_tail || s->stored_cols() == s->n + 1)) return NNVHIP_OK;
+  return ensure_dense_batch(ctx, 1, &s, need_tail);
+}
+
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
-  for (int64_t i = 0; i < count; ++i) NNV_TRY(ensure_dense(ctx, in[i]));
+  NNV_TRY(ensure_dense_batch(ctx, count, in));
   NNV_TRY(compute_ranges(ctx, count, in));
   const int64_t N = in[0]->N;
   const int64_t ld = in[0]->ld;
@@ -619,12 +753,40 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->alloc(sizeof(double) * ld * count, &key_buf));
     NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &rank_buf));
   }
+  // the appended unit-vector columns are stored only on request or when the FC / conv maps are told to
+  // contract over every column anyway; the row reset itself is left to whoever needs the whole matrix
+  const bool eager_tail = ctx->eager_tail || ctx->dense_affine;
+  const bool lazy_rows = !eager_tail && !ctx->eager_rows;
+  // With the reset pending, all that is left to write are the predicate bounds and the crossing
+  // neurons' (lb, ub).  The one-block classification does that itself, into buffers sized for the worst
+  // case (every neuron crossing), and the step is a single launch.
+  const bool fold_bounds = lazy_rows && N <= 8192;
+  BufRef pred_buf, lbub_buf;
+  std::vector<int64_t> pred_off(count), lbub_off(count);
+  const int64_t ldr_max = round_up(N, kLdAlign);
+  if (fold_bounds) {
+    int64_t total_pred = 0;
+    for (int64_t i = 0; i < count; ++i) {
+      pred_off[i] = total_pred;
+      lbub_off[i] = 2 * ldr_max * i;
+      total_pred += 2 * round_up(in[i]->n + N, kLdAlign);
+    }
+    NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
+    NNV_TRY(ctx->alloc(sizeof(double) * 2 * ldr_max * count, &lbub_buf));
+  }
   std::vector<BufRef> idx_bufs(count);
   std::vector<ReluDesc> descs(count);
   for (int64_t i = 0; i < count; ++i) {
     NNV_TRY(ctx->alloc(sizeof(int32_t) * ld, &idx_bufs[i]));
     ReluDesc& d = descs[i];
     d = ReluDesc{};
+    if (fold_bounds) {
+      d.plb_out = pred_buf->as<double>() + pred_off[i];
+      d.pub_out = d.plb_out + round_up(in[i]->n + N, kLdAlign);
+      d.lbub = lbub_buf->as<double>() + lbub_off[i];
+      d.ld_lbub = ldr_max;
+      d.write_bounds = 1;
+    }
     d.Vin = in[i]->V;
     d.lb = in[i]->lb;
     d.ub = in[i]->ub;
@@ -696,59 +858,46 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     memcpy(counts.data(), hc, sizeof(int32_t) * 2 * count);
   }
 
-  // the appended unit-vector columns are stored only on request or when the FC / conv maps are told to
-  // contract over every column anyway
-  const bool eager_tail = ctx->eager_tail || ctx->dense_affine;
   // outputs: one V arena, one predicate-bound buffer, one buffer for the crossing bounds
-  int64_t total_cols = 0, total_pred = 0, total_lbub = 0, max_cols = 0, max_m = 0;
-  std::vector<int64_t> col_off(count), pred_off(count), lbub_off(count);
+  int64_t total_cols = 0, total_pred = 0, total_lbub = 0, max_m = 0, max_pred = 0;
+  std::vector<int64_t> col_off(count);
   for (int64_t i = 0; i < count; ++i) {
     const int64_t m = counts[2 * i];
     const int64_t ncols_out = in[i]->n + 1 + (eager_tail ? m : 0);  // stored columns
     const int64_t ldr = round_up(std::max<int64_t>(m, 1), kLdAlign);
     col_off[i] = total_cols;
-    pred_off[i] = total_pred;
-    lbub_off[i] = total_lbub;
     total_cols += ncols_out;
-    total_pred += 2 * round_up(std::max<int64_t>(in[i]->n + m, 1), kLdAlign);
-    total_lbub += m > 0 ? 2 * ldr : 0;
-    max_cols = std::max(max_cols, ncols_out);
+    if (!fold_bounds) {
+      pred_off[i] = total_pred;
+      lbub_off[i] = total_lbub;
+      total_pred += 2 * round_up(std::max<int64_t>(in[i]->n + m, 1), kLdAlign);
+      total_lbub += m > 0 ? 2 * ldr : 0;
+    }
     max_m = std::max(max_m, m);
+    max_pred = std::max(max_pred, in[i]->n + m);
   }
-  BufRef arena, pred_buf, lbub_buf;
-  NNV_TRY(ctx->alloc(sizeof(double) * ld * total_cols, &arena));
-  NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
-  if (total_lbub > 0) NNV_TRY(ctx->alloc(sizeof(double) * total_lbub, &lbub_buf));
-  // Column chunking of the apply pass: a couple of thousand blocks, at least two steps per wave.
-  int row_waves = ld >= 8 * kApplyRows ? 8 : ld >= 4 * kApplyRows ? 4 : ld >= 2 * kApplyRows ? 2 : 1;
-  if (const char* e = getenv("NNVHIP_APPLY_ROW_WAVES")) {
-    const int v = atoi(e);
-    row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
+  BufRef arena;
+  if (!lazy_rows) NNV_TRY(ctx->alloc(sizeof(double) * ld * total_cols, &arena));
+  if (!fold_bounds) {
+    NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
+    if (total_lbub > 0) NNV_TRY(ctx->alloc(sizeof(double) * total_lbub, &lbub_buf));
   }
-  const int64_t row_blocks = ceil_div(ld, kApplyRows * row_waves);
-  const int64_t min_cpc = (const int64_t)8 * (kApplyWaves / row_waves);  // two 4-column steps per wave
-  int64_t want_blocks = 8192;
-  if (const char* e = getenv("NNVHIP_APPLY_BLOCKS")) want_blocks = std::max(1, atoi(e));
-  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * count), ceil_div(max_cols, min_cpc)));
-  const int64_t cpc = ceil_div(max_cols, chunks);
-  chunks = ceil_div(max_cols, cpc);
   for (int64_t i = 0; i < count; ++i) {
     ReluDesc& d = descs[i];
     const int64_t m = counts[2 * i];
+    d.m = (int32_t)m;
+    d.Vout = lazy_rows ? nullptr : arena->as<double>() + col_off[i] * ld;
+    d.write_tail = eager_tail ? 1 : 0;
+    if (fold_bounds) continue;  // bounds are in place already
     const int64_t ldr = round_up(std::max<int64_t>(m, 1), kLdAlign);
     const int64_t npad = round_up(std::max<int64_t>(in[i]->n + m, 1), kLdAlign);
-    d.m = (int32_t)m;
-    d.Vout = arena->as<double>() + col_off[i] * ld;
     d.plb_out = pred_buf->as<double>() + pred_off[i];
     d.pub_out = d.plb_out + npad;
     d.lbub = m > 0 ? lbub_buf->as<double>() + lbub_off[i] : nullptr;
     d.ld_lbub = ldr;
-    d.cols_per_chunk = (int32_t)cpc;
-    d.row_waves = row_waves;
-    d.write_tail = eager_tail ? 1 : 0;
-    d.pad3_ = 0;
+    d.write_bounds = 1;
   }
-  if (count > 1) {
+  if (count > 1 && !fold_bounds) {
     NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
@@ -760,17 +909,23 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
     hipLaunchKernelGGL(relu_scatter_kernel, dim3(t, 1, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
   }
-  double bytes = 0.0;  // algorithmic: read the rows that are kept, write N x (n+1+m)
-  for (int64_t i = 0; i < count; ++i) {
-    const double kept = (double)(N - counts[2 * i] - counts[2 * i + 1]);
-    bytes += 8.0 * kept * (double)(in[i]->n + 1) +
-             8.0 * (double)N * (double)(in[i]->n + 1 + (eager_tail ? descs[i].m : 0));
+  if (fold_bounds) {
+    // nothing left to launch
+  } else if (lazy_rows) {
+    if (max_pred > 0) {
+      hipLaunchKernelGGL(relu_bounds_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(max_pred, 256), 64), (unsigned)count),
+                         dim3(256), 0, ctx->stream, table, descs[0]);
+      NNV_HIP_TRY(hipGetLastError());
+    }
+  } else {
+    double bytes = 0.0;  // algorithmic: read the rows that are kept, write N x (n+1+m)
+    for (int64_t i = 0; i < count; ++i) {
+      const double kept = (double)(N - counts[2 * i] - counts[2 * i + 1]);
+      bytes += 8.0 * kept * (double)(in[i]->n + 1) +
+               8.0 * (double)N * (double)(in[i]->n + 1 + (eager_tail ? descs[i].m : 0));
+    }
+    NNV_TRY(launch_apply(ctx, count, descs, bytes));
   }
-  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(64 * kApplyWaves), 0,
-                     ctx->stream, table, descs[0]);
-  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 3, bytes));
-  NNV_HIP_TRY(hipGetLastError());
 
   for (int64_t i = 0; i < count; ++i) {
     const ReluDesc& d = descs[i];
@@ -778,8 +933,17 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     o->N = N;
     o->n = in[i]->n + d.m;
     o->ld = ld;
-    o->Vbuf = arena;
-    o->V = d.Vout;
+    if (lazy_rows) {  // shares the input's matrix until somebody needs the rows reset in memory
+      o->Vbuf = in[i]->Vbuf;
+      o->V = in[i]->V;
+      o->vcols = in[i]->n + 1;
+      o->rows_pending = true;
+      o->cls_buf = cls_buf;
+      o->cls = cls_buf->as<int32_t>() + ld * i;
+    } else {
+      o->Vbuf = arena;
+      o->V = d.Vout;
+    }
     o->pbuf = pred_buf;
     o->plb = d.plb_out;
     o->pub = d.pub_out;

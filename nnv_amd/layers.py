@@ -40,7 +40,7 @@ def _handles_array(sets):
 def _wrap_like(inputs, ctx, raw, shape_fn=None):
     outs = []
     for s, h in zip(inputs, raw):
-        hd = _Handle(C.c_void_p(h), ctx)
+        hd = _Handle(h, ctx)
         if isinstance(s, ImageStar):
             outs.append(ImageStar(_handle=hd, shape=shape_fn(s)))
         else:
@@ -277,7 +277,7 @@ class PosLin:
             out = (C.c_void_p * len(sets))()
             check(ctx.lib.nnvhip_relu_relax(ctx.handle, RELAX_ORDER[method], float(relaxFactor), len(sets),
                                             _handles_array(sets), out))
-            res = [Star(_handle=_Handle(C.c_void_p(h), ctx)) for h in out]
+            res = [Star(_handle=_Handle(h, ctx)) for h in out]
             if dis_opt == "display":
                 for r in res:
                     ni, idx, _, _ = r.relu_info()

@@ -21,9 +21,9 @@ class _Handle:
     __slots__ = ("h", "ctx", "_cache")
 
     def __init__(self, h, ctx):
-        self.h = h
+        self.h = h          # plain integer address (what a c_void_p argument takes) or a c_void_p
         self.ctx = ctx
-        self._cache = {}
+        self._cache = None  # (N, n, p) once asked for
 
     def __del__(self):
         try:
@@ -34,11 +34,11 @@ class _Handle:
             pass
 
     def dims(self):
-        if "dims" not in self._cache:
+        if self._cache is None:
             N, n, p = C.c_int64(), C.c_int64(), C.c_int64()
             check(self.ctx.lib.nnvhip_star_dims(self.h, C.byref(N), C.byref(n), C.byref(p)))
-            self._cache["dims"] = (N.value, n.value, p.value)
-        return self._cache["dims"]
+            self._cache = (N.value, n.value, p.value)
+        return self._cache
 
     def fetch_V(self):
         N, n, _ = self.dims()

@@ -376,3 +376,40 @@ def test_relu_output_consumers_that_need_every_column(nnv, oracle):
     E3 = oracle.batchnorm_reach(E, mean, var, 1e-5, np.ones(N), np.zeros(N))
     assert np.array_equal(R3.V, E3.V)
     assert np.array_equal(R.V, E.V)                     # property read of the first output, last
+
+
+@pytest.mark.parametrize("N,M", [(96, 40), (700, 300)])
+def test_relu_output_whose_row_reset_is_still_pending(nnv, oracle, N, M):
+    # a ReLU output shares its input's matrix until somebody needs the reset rows in memory: the FC map
+    # must give the same set before and after that, alone and in an array, and the input set is untouched
+    rs = np.random.RandomState(5 + N)
+    W0, b0 = rs.randn(N, N), rs.randn(N)
+    W, b = rs.randn(M, N), rs.randn(M)
+    L = nnv.FullyConnectedLayer(W, b)
+    lbv, ubv = -rs.rand(N), rs.rand(N)
+    box_d, box_o = nnv.Star(lbv, ubv), oracle.star_from_box(lbv, ubv)
+    pre_d = nnv.FullyConnectedLayer(W0, b0).reach(box_d, "approx-star")
+    pre_o = oracle.affine_map(box_o, W0, b0)
+    relu_o = oracle.reach_relaxed_star(pre_o, "relax-star-area", 1.0)
+    E = oracle.affine_map(relu_o, W, b)
+    assert relu_o.nVar > box_o.nVar
+    relu_d = nnv.PosLin.reach(pre_d, "relax-star-area", [], 1)
+    first = L.reach(relu_d, "approx-star")                      # reset pending: contraction over the kept rows
+    assert_close(first.V, E.V, "fc on a ReLU output, reset pending")
+    pair = L.reach([relu_d, nnv.PosLin.reach(pre_d, "relax-star-area", [], 1)], "approx-star")
+    for R in pair:
+        assert_close(R.V, E.V, "fc on an array of ReLU outputs, reset pending")
+    assert np.array_equal(relu_d.V, relu_o.V)                   # the read runs the reset into a new buffer
+    assert_close(pre_d.V, pre_o.V, "input of the ReLU after its output was written out")
+    assert np.count_nonzero(np.asarray(pre_d.V)[:, 0] < 0) > 0  # ... still holds its negative rows
+    second = L.reach(relu_d, "approx-star")
+    assert_close(second.V, E.V, "fc on a ReLU output, rows in memory")
+    el, eu = oracle.estimate_ranges(E)
+    for R in (first, second):
+        lb, ub = R.estimateRanges()
+        assert_close(lb, el, "lb")
+        assert_close(ub, eu, "ub")
+    # a second ReLU directly on a pending output (no layer between)
+    R2 = nnv.PosLin.reach(nnv.PosLin.reach(pre_d, "relax-star-area", [], 1), "relax-star-range", [], 1)
+    E2 = oracle.reach_relaxed_star(relu_o, "relax-star-range", 1.0)
+    assert np.array_equal(R2.V, E2.V)
