@@ -126,6 +126,10 @@ NNVHIP_API int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, in
  * exactly as PosLin.multipleStepReachStarApprox_at_one builds them, [C0;C1;C2;C3]
  * (nn/funcs/PosLin.m:711-735), materialised from the device's structured store. */
 NNVHIP_API int nnvhip_star_fetch_V(const nnvhip_star* s, double* V);
+/* V(rows, :): R x (n+1), column-major, rows 0-based -- the objective rows f = V(index, 2:n+1) and
+ * offsets V(index, 1) that Star.getMin / getMax / getMins / getMaxs hand to the LP solver
+ * (set/Star.m:742-970), gathered on the device so that only those rows cross the bus. */
+NNVHIP_API int nnvhip_star_fetch_rows(const nnvhip_star* s, int64_t R, const int32_t* rows, double* out);
 NNVHIP_API int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* pred_lb, double* pred_ub);
 NNVHIP_API int nnvhip_star_fetch_constraints(const nnvhip_star* s, double* C, double* d);
 /* For a set returned by nnvhip_relu_relax: counts of inactive (ub <= 0) and crossing
@@ -177,6 +181,14 @@ NNVHIP_API int nnvhip_affine_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, 
  * three triangle constraints and predicate bounds [0, ub].  relax_factor must be 1 (no LP). */
 NNVHIP_API int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor, int64_t count,
                       nnvhip_star* const* in, nnvhip_star** out);
+/* PosLin.multipleStepReachStarApprox_at_one(I.resetRow(reset_rows), index, lb, ub),
+ * nn/funcs/PosLin.m:685-742 and set/Star.m:1442-1461: the step with the lists handed in instead of
+ * derived from estimateRanges -- what the relaxFactor < 1 branches call once the host LPs
+ * (Star.getMaxs / getMins) have tightened some bounds (nn/funcs/PosLin.m:1066-1096 and the sibling
+ * heuristics).  reset_rows (n_reset entries) are zeroed; index (m entries, 0-based, with
+ * lb[i] < 0 < ub[i]) get the triangle relaxation, new predicates in the order of the list. */
+NNVHIP_API int nnvhip_relu_apply_lists(nnvhip_ctx* ctx, nnvhip_star* in, int64_t n_reset, const int32_t* reset_rows,
+                            int64_t m, const int32_t* index, const double* lb, const double* ub, nnvhip_star** out);
 
 /* ---- specification check, utils/verify_specification.m:36-80 ----------------------------- */
 /* verify_specification intersects every output set with every half-space {x | G x <= g} of the

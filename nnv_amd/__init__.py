@@ -1,4 +1,4 @@
-"""nnv_amd: MI355X-native star-set reachability (relax-star, relaxFactor = 1) behind NNV's API.
+"""nnv_amd: MI355X-native star-set reachability (the relax-star methods) behind NNV's API.
 
 The compute path is the HIP library nnv_amd/libnnvhip.so (C ABI in include/nnvhip.h); these Python
 classes mirror NNV's MATLAB classes for the path and call it through ctypes.

@@ -26,6 +26,7 @@ SYMBOLS = [
     "nnvhip_relu_relax", "nnvhip_halfspace_check", "nnvhip_halfspace_rows", "nnvhip_rowmap_create",
     "nnvhip_rowmap_destroy", "nnvhip_affine_rowmap", "nnvhip_avgpool2d_create", "nnvhip_avgpool2d_destroy",
     "nnvhip_avgpool2d_output_size", "nnvhip_affine_avgpool2d", "nnvhip_permute_rows",
+    "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists",
 ]
 
 
@@ -69,6 +70,7 @@ def load():
         "nnvhip_star_release": [p],
         "nnvhip_star_dims": [p, pi64, pi64, pi64],
         "nnvhip_star_fetch_V": [p, p],
+        "nnvhip_star_fetch_rows": [p, i64, p, p],
         "nnvhip_star_fetch_pred_bounds": [p, p, p],
         "nnvhip_star_fetch_constraints": [p, p, p],
         "nnvhip_star_relu_counts": [p, pi64, pi64],
@@ -83,6 +85,7 @@ def load():
         "nnvhip_affine_fc": [p, p, i64, pp, pp],
         "nnvhip_affine_conv2d": [p, p, i64, i64, i64, pp, pp],
         "nnvhip_relu_relax": [p, C.c_int, dbl, i64, pp, pp],
+        "nnvhip_relu_apply_lists": [p, p, i64, p, i64, p, p, p, pp],
         "nnvhip_halfspace_check": [p, i64, pp, i64, p, p, p, i64, p, p, p],
         "nnvhip_halfspace_rows": [p, p, i64, p, p, i64, p, p],
         "nnvhip_rowmap_create": [p, i64, C.c_int32, p, p, p, pp],

@@ -507,6 +507,31 @@ int nnvhip_star_fetch_V(const nnvhip_star* s, double* V) {
   return NNVHIP_OK;
 }
 
+int nnvhip_star_fetch_rows(const nnvhip_star* s, int64_t R, const int32_t* rows, double* out) {
+  if (!s || (R > 0 && (!rows || !out)) || R < 0) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  if (R == 0) return NNVHIP_OK;
+  nnvhip_ctx* c = s->ctx;
+  for (int64_t t = 0; t < R; ++t)
+    if (rows[t] < 0 || rows[t] >= s->N) NNV_FAIL(NNVHIP_ERR_ARG, "Invalid index");
+  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(ensure_dense(c, const_cast<nnvhip_star*>(s)));
+  // gather on the device into an Rp x (n+1) matrix (Rp = R rounded up to whole K-tiles, the packing
+  // kernel's granularity), one contiguous copy, then drop the padding rows on the host
+  const int64_t Rp = round_up(R, kLdAlign), nc = s->n + 1;
+  std::vector<int32_t> list((size_t)Rp, -1);
+  std::copy(rows, rows + R, list.begin());
+  BufRef dlist, packed;
+  NNV_TRY(c->upload(list.data(), sizeof(int32_t) * Rp, &dlist));
+  NNV_TRY(c->alloc(sizeof(double) * Rp * nc, &packed));
+  PackSet ps{s->V, dlist->as<int32_t>(), packed->as<double>(), s->ld, (int32_t)Rp, (int32_t)nc};
+  NNV_TRY(launch_pack_rows(c, 1, &ps));
+  std::vector<double> tmp((size_t)(Rp * nc));
+  NNV_HIP_TRY(hipMemcpyAsync(tmp.data(), packed->ptr, sizeof(double) * Rp * nc, hipMemcpyDeviceToHost, c->stream));
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  for (int64_t j = 0; j < nc; ++j) memcpy(out + j * R, tmp.data() + j * Rp, sizeof(double) * R);
+  return NNVHIP_OK;
+}
+
 int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* lb, double* ub) {
   if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
   nnvhip_ctx* c = s->ctx;
@@ -1087,6 +1112,52 @@ int nnvhip_relu_relax(nnvhip_ctx* c, int order, double relax_factor, int64_t cou
     if (in[i]->N != in[0]->N) NNV_FAIL(NNVHIP_ERR_SHAPE, "sets of one array must have the same dimension");
   NNV_TRY(c->begin_op());
   NNV_TRY(relu_relax(c, order, count, in, out));
+  return c->end_op();
+}
+
+int nnvhip_relu_apply_lists(nnvhip_ctx* c, nnvhip_star* in, int64_t n_reset, const int32_t* reset_rows, int64_t m,
+                            const int32_t* index, const double* lb, const double* ub, nnvhip_star** out) {
+  CHECK_CTX(c);
+  if (!in || in->ctx != c || !out) NNV_FAIL(NNVHIP_ERR_ARG, "invalid set handle");
+  if (n_reset < 0 || m < 0 || (n_reset > 0 && !reset_rows) || (m > 0 && (!index || !lb || !ub)))
+    NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  const int64_t N = in->N;
+  // per-row bounds that make the classification reproduce the two lists: a reset row looks inactive
+  // (ub = 0), a listed neuron carries its own (lb, ub), every other row looks active; the keys put the
+  // new predicates in the order of the list
+  std::vector<double> rows((size_t)(3 * N));
+  double* L = rows.data();
+  double* U = L + N;
+  double* K = U + N;
+  std::vector<char> seen((size_t)N, 0);
+  for (int64_t r = 0; r < N; ++r) {
+    L[r] = 0.0;
+    U[r] = 1.0;
+    K[r] = 0.0;
+  }
+  for (int64_t t = 0; t < n_reset; ++t) {
+    const int64_t r = reset_rows[t];
+    if (r < 0 || r >= N) NNV_FAIL(NNVHIP_ERR_ARG, "Invalid index");
+    if (seen[r]) NNV_FAIL(NNVHIP_ERR_ARG, "row %lld is listed twice", (long long)r);
+    seen[r] = 1;
+    L[r] = -1.0;
+    U[r] = 0.0;
+  }
+  for (int64_t t = 0; t < m; ++t) {
+    const int64_t r = index[t];
+    if (r < 0 || r >= N) NNV_FAIL(NNVHIP_ERR_ARG, "Invalid index");
+    if (seen[r]) NNV_FAIL(NNVHIP_ERR_ARG, "row %lld is listed twice", (long long)r);
+    if (!(lb[t] < 0.0 && ub[t] > 0.0)) NNV_FAIL(NNVHIP_ERR_ARG, "neuron %lld: the triangle relaxation needs lb < 0 < ub", (long long)r);
+    seen[r] = 1;
+    L[r] = lb[t];
+    U[r] = ub[t];
+    K[r] = (double)(m - t);
+  }
+  NNV_TRY(c->begin_op());
+  BufRef dev;
+  NNV_TRY(c->upload(rows.data(), sizeof(double) * 3 * N, &dev));
+  ReluGiven g{dev->as<double>(), dev->as<double>() + N, dev->as<double>() + 2 * N};
+  NNV_TRY(relu_relax(c, kOrderGiven, 1, &in, out, &g));
   return c->end_op();
 }
 

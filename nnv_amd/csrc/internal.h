@@ -330,7 +330,17 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
 // unit-vector columns, into a fresh buffer.  The batch form keeps the sets of an array back to back.
 int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s, bool need_tail = true);
 int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail = true);
-int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out);
+// order: NNVHIP_ORDER_* (classification from the sets' estimated ranges), or kOrderGiven with one
+// ReluGiven per set: per-row bounds to classify by (ub <= 0: reset, lb < 0 < ub: crossing, else left
+// alone) and per-row keys whose descending order is the order of the new predicates.
+constexpr int kOrderGiven = 3;
+struct ReluGiven {
+  const double* lb;
+  const double* ub;
+  const double* key;
+};
+int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out,
+               const ReluGiven* given = nullptr);
 int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host);
 
 }  // namespace nnvhip

@@ -33,6 +33,7 @@ struct ReluDesc {
   int32_t* cross_idx;  // crossing neuron indices in new-predicate order
   int32_t* asc_idx;    // crossing neuron indices in ascending order (sort orders only)
   double* key;         // sort keys, ascending-index order
+  const double* given_key;  // order kOrderGiven: the key of every row is handed in (callers with an explicit list)
   int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
   int32_t* keep_idx;   // rows left untouched (active neurons), ascending, then -1 up to a multiple of 16
@@ -298,7 +299,8 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
       d.cls[r] = pos;
       if (d.order != NNVHIP_ORDER_INDEX) {
         // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb
-        const double key = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : u - l;
+        const double key = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l))
+                           : d.order == NNVHIP_ORDER_RANGE ? u - l : d.given_key[r];
         d.key[pos] = key;
         d.rank[pos] = 0;
         if (SORT_CAP > 0 && pos < SORT_CAP) {
@@ -442,7 +444,7 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
     idx_out[pos] = r;
     d.cls[r] = pos;
     if (d.order != NNVHIP_ORDER_INDEX) {
-      d.key[pos] = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : u - l;
+      d.key[pos] = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : d.order == NNVHIP_ORDER_RANGE ? u - l : d.given_key[r];
       d.rank[pos] = 0;
     }
   } else if (valid) {
@@ -728,10 +730,11 @@ int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s, bool need_tail) {
   return ensure_dense_batch(ctx, 1, &s, need_tail);
 }
 
-int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
+int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out, const ReluGiven* given) {
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  if ((order == kOrderGiven) != (given != nullptr)) NNV_FAIL(NNVHIP_ERR_ARG, "internal: explicit lists and their order go together");
   NNV_TRY(ensure_dense_batch(ctx, count, in));
-  NNV_TRY(compute_ranges(ctx, count, in));
+  if (given == nullptr) NNV_TRY(compute_ranges(ctx, count, in));
   const int64_t N = in[0]->N;
   const int64_t ld = in[0]->ld;
   if (N >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "set dimension too large");
@@ -788,8 +791,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       d.write_bounds = 1;
     }
     d.Vin = in[i]->V;
-    d.lb = in[i]->lb;
-    d.ub = in[i]->ub;
+    d.lb = given ? given[i].lb : in[i]->lb;
+    d.ub = given ? given[i].ub : in[i]->ub;
+    d.given_key = given ? given[i].key : nullptr;
     d.plb_in = in[i]->plb;
     d.pub_in = in[i]->pub;
     d.cls = cls_buf->as<int32_t>() + ld * i;

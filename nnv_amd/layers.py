@@ -2,7 +2,8 @@
 
 ``layer.reach(in_sets, method, option, relaxFactor, dis_opt, lp_solver)`` accepts one set or a
 list of sets (NNV's set arrays) and returns the same; the whole array is processed by one batched
-device call.  Only the relax-star methods at relaxFactor = 1 are available for the ReLU.
+device call.  The ReLU offers the relax-star methods: at relaxFactor = 1 entirely on the device,
+below 1 with the LPs of Star.getMaxs / getMins on the host, fed from the resident set.
 """
 from __future__ import annotations
 
@@ -262,6 +263,27 @@ class PosLin:
         return np.maximum(np.asarray(x, dtype=np.float64), 0)
 
     @staticmethod
+    def multipleStepReachStarApprox_at_one(I, index, lb, ub, reset=()):
+        """PosLin.multipleStepReachStarApprox_at_one(I.resetRow(reset), index, lb, ub),
+        nn/funcs/PosLin.m:685-742 with set/Star.m:1442-1461; all indices 0-based."""
+        if not isinstance(I, Star):
+            raise TypeError("Input is not a star")
+        ctx = I.ctx
+        reset = np.ascontiguousarray(np.asarray(reset).reshape(-1), dtype=np.int32)
+        index = np.ascontiguousarray(np.asarray(index).reshape(-1), dtype=np.int32)
+        lb, ub = f64(np.asarray(lb).reshape(-1)), f64(np.asarray(ub).reshape(-1))
+        if lb.size != index.size or ub.size != index.size:
+            raise ValueError("index, lb and ub must have the same length")
+        out = (C.c_void_p * 1)()
+        check(ctx.lib.nnvhip_relu_apply_lists(ctx.handle, I._h.h, reset.size, ptr(reset), index.size, ptr(index),
+                                              ptr(lb), ptr(ub), out))
+        return Star(_handle=_Handle(out[0], ctx))
+
+    @staticmethod
+    def reach_relaxed_star_lp(I, method, relaxFactor, option=None, dis_opt=None, lp_solver="linprog", rng=None):
+        return _relaxed_star_lp(I, method, relaxFactor, option, dis_opt, lp_solver, rng)
+
+    @staticmethod
     def reach(I, method="exact-star", option="parallel", relaxFactor=0, dis_opt=None, lp_solver="linprog"):
         """PosLin.reach, nn/funcs/PosLin.m:2073-2169."""
         sets, single = _as_list(I)
@@ -274,11 +296,15 @@ class PosLin:
             if not sets:
                 return []
             ctx = sets[0].ctx
-            out = (C.c_void_p * len(sets))()
-            check(ctx.lib.nnvhip_relu_relax(ctx.handle, RELAX_ORDER[method], float(relaxFactor), len(sets),
-                                            _handles_array(sets), out))
-            res = [Star(_handle=_Handle(h, ctx)) for h in out]
-            if dis_opt == "display":
+            if relaxFactor == 1:
+                out = (C.c_void_p * len(sets))()
+                check(ctx.lib.nnvhip_relu_relax(ctx.handle, RELAX_ORDER[method], float(relaxFactor), len(sets),
+                                                _handles_array(sets), out))
+                res = [Star(_handle=_Handle(h, ctx)) for h in out]
+            else:
+                # some bounds are tightened by LPs first: host LP solver fed from the resident set
+                res = [PosLin.reach_relaxed_star_lp(s, method, relaxFactor, option, dis_opt, lp_solver) for s in sets]
+            if dis_opt == "display" and relaxFactor == 1:
                 for r in res:
                     ni, idx, _, _ = r.relu_info()
                     print("\n%d neurons with ub <= 0 are found by estimating ranges" % ni)
@@ -288,6 +314,87 @@ class PosLin:
         if method in ("exact-star", "exact-polyhedron", "approx-star", "approx-zono", "abs-dom"):
             raise NotImplementedError("only the relax-star methods are provided by this library (method '%s')" % method)
         raise ValueError("This reachability method does not exist")
+
+
+def _matlab_round(x):
+    return int(np.floor(x + 0.5))      # round(): halves away from zero, x >= 0 here
+
+
+def _sort_descend(key):
+    return np.argsort(-np.asarray(key), kind="stable")   # sort(..., 'descend') keeps ties in order
+
+
+def _setdiff_stable(a, b):
+    return a[~np.isin(a, b)] if len(b) else a
+
+
+def _relaxed_star_lp(I, method, relaxFactor, option=None, dis_opt=None, lp_solver="linprog", rng=None):
+    """The relaxFactor < 1 branches of PosLin.reach_relaxed_star_{range,area,bound,ub,random,static}
+    (nn/funcs/PosLin.m:863-1650): n1 = round((1-relaxFactor)*#crossing) neurons, picked by the method's
+    heuristic, get their upper (then lower) bound from an LP over the set's constraints; neurons whose
+    optimised ub <= 0 are reset, those whose optimised lb >= 0 are left alone, and the rest go through
+    the triangle relaxation with the tighter bounds.  Everything but the LPs runs on the device; the
+    LPs get only the rows of V they need."""
+    lb, ub = I.estimateRanges()
+    map1 = np.flatnonzero(ub <= 0)
+    map2 = np.flatnonzero((lb < 0) & (ub > 0))
+    n1 = _matlab_round((1 - relaxFactor) * map2.size)
+    N = map2.size
+    if method in ("relax-star-range", "relax-star-area", "relax-star-random", "relax-star-static"):
+        if method == "relax-star-range":            # PosLin.m:934-936
+            midx = _sort_descend(ub[map2] - lb[map2])
+            map21, map22 = map2[midx[:n1]], map2[midx[n1:]]
+        elif method == "relax-star-area":           # :1049-1052
+            midx = _sort_descend(0.5 * (np.abs(ub[map2]) * np.abs(lb[map2])))
+            map21, map22 = map2[midx[:n1]], map2[midx[n1:]]
+        elif method == "relax-star-random":         # :1488-1492 (randperm: not reproducible across libraries)
+            rng = rng or np.random
+            map21 = map2[rng.permutation(N)[:n1]]
+            map22 = _setdiff_stable(map2, map21)
+        else:                                       # :1604-1605
+            map21, map22 = map2[:n1], map2[n1:]
+        xmax = I.getMaxs(map21, option, dis_opt, lp_solver)
+        map4 = map21[xmax <= 0]
+        map11 = np.concatenate([map1, map4])
+        map6, xmax1 = map21[xmax > 0], xmax[xmax > 0]
+        xmin = I.getMins(map6, option, dis_opt, lp_solver)
+        keep = xmin < 0
+        index = np.concatenate([map22, map6[keep]])                     # map9
+        lbs = np.concatenate([lb[map22], xmin[keep]])
+        ubs = np.concatenate([ub[map22], xmax1[keep]])
+    else:
+        if method == "relax-star-bound":            # :1167-1176
+            midx1 = _sort_descend(np.concatenate([ub[map2], np.abs(lb[map2])]))[:2 * n1]
+            map21 = map2[midx1[midx1 < N]]
+            map22 = map2[midx1[midx1 >= N] - N]
+        else:                                       # relax-star-ub, :1326-1338
+            midx_u = _sort_descend(ub[map2])
+            midx_l = _sort_descend(np.abs(lb[map2]))
+            if 2 * n1 <= N:
+                map21, map22 = map2[midx_u[:2 * n1]], map2[:0]
+            else:
+                map21, map22 = map2[midx_u[:N]], map2[midx_l[:2 * n1 - N]]
+        lb, ub = lb.copy(), ub.copy()
+        map4 = map2[:0]
+        if map21.size:
+            xmax = I.getMaxs(map21, option, dis_opt, lp_solver)
+            map4 = map21[xmax <= 0]
+            ub[map21[xmax > 0]] = xmax[xmax > 0]
+        map11 = np.concatenate([map1, map4])
+        map23 = _setdiff_stable(map22, map4)
+        map10 = map2[:0]
+        if map23.size:
+            xmin = I.getMins(map23, option, dis_opt, lp_solver)
+            lb[map23[xmin < 0]] = xmin[xmin < 0]
+            map10 = map23[xmin >= 0]
+        index = _setdiff_stable(_setdiff_stable(map2, map4), map10)     # map24
+        lbs, ubs = lb[index], ub[index]
+    if dis_opt == "display":
+        print("\n%d neurons with ub <= 0 are found by estimating ranges" % map1.size)
+        print("(%d+%d =%d)/%d neurons have ub <= 0" % (map1.size, map4.size, map11.size, ub.size))
+        print("%d/%d neurons have lb < 0 & ub > 0" % (index.size, ub.size))
+        print("Construct new star set, %d new predicate variables are introduced" % index.size)
+    return PosLin.multipleStepReachStarApprox_at_one(I, index, lbs, ubs, reset=map11)
 
 
 class ReluLayer:

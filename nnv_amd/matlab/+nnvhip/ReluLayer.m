@@ -6,7 +6,7 @@ classdef ReluLayer < ReluLayer
         function obj = ReluLayer(varargin)
             obj = obj@ReluLayer(varargin{:});
         end
-        function images = reach_star_multipleInputs(obj, in_images, method, option, relaxFactor, dis_opt, lp_solver) %#ok<INUSD>
+        function images = reach_star_multipleInputs(obj, in_images, method, option, relaxFactor, dis_opt, lp_solver) %#ok<INUSL>
             switch char(method)
                 case 'relax-star-range', order = 2;                       % PosLin.m:934-936
                 case 'relax-star-area',  order = 1;                       % PosLin.m:1049-1052
@@ -21,7 +21,12 @@ classdef ReluLayer < ReluLayer
             n = length(in_images);
             hs = zeros(1, n, 'uint64');
             for i = 1:n, hs(i) = in_images(i).dev.h; end
-            out = nnvhip_mex('relu_relax', order, relaxFactor, hs);
+            if relaxFactor == 1
+                out = nnvhip_mex('relu_relax', order, relaxFactor, hs);
+            else    % some bounds come from LPs first (host lpsolver fed from the resident set)
+                out = zeros(1, n, 'uint64');
+                for i = 1:n, out(i) = nnvhip.relaxed_star_lp(hs(i), method, relaxFactor, lp_solver, dis_opt); end
+            end
             for i = n:-1:1
                 if isa(in_images(i), 'ImageStar')
                     images(i) = nnvhip.ImageStar(nnvhip.DeviceSet(out(i)), in_images(i).height, in_images(i).width, in_images(i).numChannel);

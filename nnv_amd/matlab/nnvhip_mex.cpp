@@ -198,6 +198,32 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
     std::vector<nnvhip_star*> in = handles_of(prhs[3]), out(in.size());
     check(nnvhip_relu_relax(ctx(), (int)mxGetScalar(prhs[1]), mxGetScalar(prhs[2]), (int64_t)in.size(), in.data(), out.data()));
     plhs[0] = to_mx(out);
+  } else if (cmd == "fetch_rows") {  // (handle, rows 1-based) -> V(rows, :)      objective rows of Star.getMin/getMax
+    need(nrhs, 2, "fetch_rows");
+    nnvhip_star* s = handle_of<nnvhip_star>(prhs[1]);
+    int64_t N, n, p;
+    check(nnvhip_star_dims(s, &N, &n, &p));
+    const mwSize R = mxGetNumberOfElements(prhs[2]);
+    const double* r1 = dbl(prhs[2], "rows");
+    std::vector<int32_t> rows(R);
+    for (mwSize t = 0; t < R; ++t) rows[t] = (int32_t)r1[t] - 1;
+    plhs[0] = mxCreateDoubleMatrix(R, (mwSize)(n + 1), mxREAL);
+    check(nnvhip_star_fetch_rows(s, (int64_t)R, rows.data(), mxGetDoubles(plhs[0])));
+  } else if (cmd == "relu_apply_lists") {  // (handle, reset rows, index, lb, ub; 1-based) -> handle
+    // PosLin.multipleStepReachStarApprox_at_one(I.resetRow(reset), index, lb, ub), nn/funcs/PosLin.m:685-742
+    need(nrhs, 5, "relu_apply_lists");
+    const mwSize nr = mxGetNumberOfElements(prhs[2]), m = mxGetNumberOfElements(prhs[3]);
+    if (mxGetNumberOfElements(prhs[4]) != m || mxGetNumberOfElements(prhs[5]) != m)
+      mexErrMsgIdAndTxt("nnvhip:error", "index, lb and ub must have the same length");
+    const double* r1 = dbl(prhs[2], "reset");
+    const double* i1 = dbl(prhs[3], "index");
+    std::vector<int32_t> reset(nr), index(m);
+    for (mwSize t = 0; t < nr; ++t) reset[t] = (int32_t)r1[t] - 1;
+    for (mwSize t = 0; t < m; ++t) index[t] = (int32_t)i1[t] - 1;
+    nnvhip_star* out = nullptr;
+    check(nnvhip_relu_apply_lists(ctx(), handle_of<nnvhip_star>(prhs[1]), (int64_t)nr, reset.data(), (int64_t)m, index.data(),
+                                  dbl(prhs[4], "lb"), dbl(prhs[5], "ub"), &out));
+    plhs[0] = to_mx(out);
   } else if (cmd == "halfspace_check") {  // (handles, G (R x dim), g (R x 1), rows_per_halfspace) -> [verdict (count x n_hs), lo, hi]
     // LP-free part of utils/verify_specification.m:36-80; 1 = disjoint, 2 = undecided (LP), 3 = inside
     need(nrhs, 4, "halfspace_check");

@@ -60,6 +60,14 @@ class _Handle:
         check(self.ctx.lib.nnvhip_star_fetch_constraints(self.h, ptr(Cm), ptr(d)))
         return Cm, d
 
+    def fetch_rows(self, rows):
+        """V(rows, :) as an R x (n+1) array; rows 0-based."""
+        rows = np.ascontiguousarray(np.asarray(rows).reshape(-1), dtype=np.int32)
+        _, n, _ = self.dims()
+        out = np.empty((rows.size, n + 1), dtype=np.float64, order="F")
+        check(self.ctx.lib.nnvhip_star_fetch_rows(self.h, rows.size, ptr(rows), ptr(out)))
+        return out
+
     def ranges(self):
         N, _, _ = self.dims()
         lb = np.empty(N)
@@ -204,6 +212,9 @@ class Star:
                                          ptr(Cm) if Cm.size else None, ptr(d) if d.size else None, Cm.shape[0],
                                          C.byref(out)))
             self._h = _Handle(out, ctx)
+            # no bounds given: the device uses estimateRanges' default [-1, 1] (set/Star.m:1091-1096), the LP
+            # methods leave the predicates free as the reference's empty predicate_lb/ub do
+            self._unbounded_predicates = plb is None
             return
         raise ValueError("Invalid number of input arguments (should be 0, 1, 2, 3, 5, 6 or 7)")
 
@@ -281,6 +292,81 @@ class Star:
     def estimateRanges(self):
         """Star.estimateRanges, set/Star.m:1078-1106 -> (lb, ub)."""
         return self._h.ranges()
+
+    # ---- LP-based ranges (host LP fed from the resident set) -------------------------------
+    def _lp_problem(self):
+        """(C as a sparse matrix, d, predicate bounds) of this set, fetched once."""
+        if getattr(self, "_lp", None) is None:
+            from scipy import sparse
+            Cm, d = self._h.fetch_constraints()
+            if getattr(self, "_unbounded_predicates", False):     # Star(V, C, d): predicate_lb/ub are []
+                bounds = np.column_stack([np.full(self.nVar, -np.inf), np.full(self.nVar, np.inf)])
+            else:
+                bounds = np.column_stack(self._h.fetch_pred())
+            self._lp = (sparse.csr_matrix(Cm), d, bounds)
+        return self._lp
+
+    def _lp_min(self, f):
+        """min f'a over C a <= d, pred_lb <= a <= pred_ub (lpsolver's call in set/Star.m:773); scipy's
+        HiGHS stands where the reference calls linprog / glpk."""
+        from scipy.optimize import linprog
+        Cs, d, bounds = self._lp_problem()
+        if Cs.nnz == 0 and np.all(np.isfinite(bounds)) and (d.size == 0 or np.all(d >= 0)):
+            # utils/lpsolver.m:36-50: nothing but the box -> closed form, no solver call
+            return float(np.sum(np.minimum(f * bounds[:, 0], f * bounds[:, 1])))
+        res = linprog(f, A_ub=Cs if Cs.shape[0] else None, b_ub=d if Cs.shape[0] else None, bounds=bounds, method="highs")
+        if res.status != 0:
+            raise RuntimeError("Cannot find an optimal solution, exitflag = %d" % res.status)
+        return res.fun
+
+    def _extremes(self, index, sign):
+        index = np.asarray(index).reshape(-1)
+        if index.size and (index.min() < 0 or index.max() >= self.dim):
+            raise ValueError("Invalid index")
+        out = np.empty(index.size)
+        if index.size == 0:
+            return out
+        rows = self._h.fetch_rows(index)
+        for t in range(index.size):
+            f = rows[t, 1:]
+            if not f.any():
+                out[t] = rows[t, 0]          # all(f(:)==0): the centre entry itself
+            else:
+                out[t] = sign * self._lp_min(sign * f) + rows[t, 0]
+        return out
+
+    def getMin(self, index, lp_solver="linprog"):
+        """Star.getMin, set/Star.m:744-781 (index 0-based)."""
+        return float(self._extremes([index], 1.0)[0])
+
+    def getMax(self, index, lp_solver="linprog"):
+        """Star.getMax, set/Star.m:859-895 (index 0-based)."""
+        return float(self._extremes([index], -1.0)[0])
+
+    def getMins(self, map, par_option="single", dis_option=None, lp_solver="linprog"):
+        """Star.getMins, set/Star.m:784-856: one LP per listed state (0-based list)."""
+        if par_option not in (None, "", "single", "parallel") and not (isinstance(par_option, (list, tuple)) and len(par_option) == 0):
+            raise ValueError("Unknown parallel option")
+        return self._extremes(map, 1.0)
+
+    def getMaxs(self, map, par_option="single", dis_option=None, lp_solver="linprog"):
+        """Star.getMaxs, set/Star.m:898-970."""
+        if par_option not in (None, "", "single", "parallel") and not (isinstance(par_option, (list, tuple)) and len(par_option) == 0):
+            raise ValueError("Unknown parallel option")
+        return self._extremes(map, -1.0)
+
+    def getRange(self, index):
+        """Star.getRange, set/Star.m:710-741 -> (xmin, xmax)."""
+        return self.getMin(index), self.getMax(index)
+
+    def getRanges(self, lp_solver="linprog"):
+        """Star.getRanges, set/Star.m:973-990: 2 LPs per state; empty arrays for an empty set."""
+        from scipy.optimize import linprog
+        Cs, d, bounds = self._lp_problem()
+        if Cs.shape[0] and linprog(np.zeros(self.nVar), A_ub=Cs, b_ub=d, bounds=bounds, method="highs").status == 2:
+            return np.empty(0), np.empty(0)
+        idx = np.arange(self.dim)
+        return self._extremes(idx, 1.0), self._extremes(idx, -1.0)
 
     def toImageStar(self, height, width, numChannel):
         """Star.toImageStar, set/Star.m:1398-1418: a reshape; the device data is shared."""

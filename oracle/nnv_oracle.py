@@ -33,6 +33,15 @@ Parity pinning (what checks each function; see tests/test_oracle_*.py)
   hand-computed scalar triangle, brute-force corner enumeration, the containment
   (soundness) invariant the reference's own soundness tests use, structural invariants
   and permutation-equivalence of the six variants.
+* lpsolver / get_min(s) / get_max(s) / reach_relaxed_star_lp (relaxFactor < 1): the box-only branch of
+  lpsolver is a closed form (checked against interval arithmetic); everything that reaches the LP
+  solver is PARITY UNPINNED (linprog there, HiGHS here: values to solver tolerance, and a neuron whose
+  optimised bound lies within that tolerance of 0 may be classified differently).  Pinned by: LP bounds never looser than estimateRanges, the rf = 1 limit (no LP), the box-star case where every
+  variant reduces to the rf = 1 sets up to the documented order of the new predicates, and the
+  containment invariant of the reference's soundness tests.  get_min / get_max through the solver
+  branch are checked against the reference's stored LP ranges of a star with eleven general
+  constraint rows (results/tests/baselines/set/test_star_intersect_halfSpace_results.mat, S1_lb /
+  S1_ub, written by tests/set/star/test_star_intersect_halfSpace.m:66-79) to 1e-8.
 * halfspace_contains / is_empty_set / intersect_half_space: the reference's known answers
   (tests/set/halfspace/test_half_space_contain.m, tests/set/star/test_star_isEmptySet.m:17-23,
   tests/soundness/test_set_conversion.m:60-68) and closed forms on boxes.  The LP itself is
@@ -488,17 +497,167 @@ def relax_classify(lb, ub, method):
     return map1, map2
 
 
-def reach_relaxed_star(I: OStar, method: str, relax_factor: float = 1.0) -> OStar:
-    """PosLin.reach_relaxed_star_{range,area,bound,ub,random,static} at relaxFactor = 1
-    (nn/funcs/PosLin.m:863-1650).  n1 = round((1-rf)*numel(map2)) = 0, so no LP is solved:
-    In = I.resetRow(map1); S = multipleStepReachStarApprox_at_one(In, map, lb(map), ub(map)).
-    """
+def lpsolver(f, A, b, lb, ub):
+    """utils/lpsolver.m: min f'x s.t. A x <= b, lb <= x <= ub -> fval.
+
+    The box-only shortcut (:36-50: A empty or all-zero, finite bounds, b >= 0) is restated exactly:
+    fval = sum(min(f.*lb, f.*ub)).  Otherwise MATLAB's linprog (glpk as backup) is replaced by
+    scipy's HiGHS, so values agree to solver tolerance only: PARITY UNPINNED beyond that."""
+    f = np.asarray(f, dtype=np.float64).reshape(-1)
+    A = np.asarray(A, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64).reshape(-1)
+    if (A.size == 0 or not np.any(A)) and lb is not None and ub is not None and np.size(lb) and np.size(ub) \
+            and np.all(np.isfinite(lb)) and np.all(np.isfinite(ub)) and (b.size == 0 or np.all(b >= 0)):
+        return float(np.sum(np.minimum(f * lb, f * ub)))
+    from scipy.optimize import linprog
+    n = f.size
+    lo = np.full(n, -np.inf) if lb is None or not np.size(lb) else np.asarray(lb, dtype=np.float64).reshape(-1)
+    hi = np.full(n, np.inf) if ub is None or not np.size(ub) else np.asarray(ub, dtype=np.float64).reshape(-1)
+    res = linprog(f, A_ub=A if A.size else None, b_ub=b if A.size else None,
+                  bounds=np.column_stack([lo, hi]), method="highs")
+    if res.status != 0:
+        raise RuntimeError("Cannot find an optimal solution, exitflag = %d" % res.status)
+    return float(res.fun)
+
+
+def get_min(S: OStar, index) -> float:
+    """Star.getMin, set/Star.m:744-781 (index 0-based): the centre entry if the generator row is all
+    zero, else one LP over (C, d, predicate bounds)."""
+    if index < 0 or index >= S.dim:
+        raise ValueError("Invalid index")
+    f = S.V[index, 1:S.nVar + 1]
+    if not np.any(f):
+        return float(S.V[index, 0])
+    return lpsolver(f, S.C, S.d, S.predicate_lb, S.predicate_ub) + float(S.V[index, 0])
+
+
+def get_max(S: OStar, index) -> float:
+    """Star.getMax, set/Star.m:859-895: -min(-f) + c."""
+    if index < 0 or index >= S.dim:
+        raise ValueError("Invalid index")
+    f = S.V[index, 1:S.nVar + 1]
+    if not np.any(f):
+        return float(S.V[index, 0])
+    return -lpsolver(-f, S.C, S.d, S.predicate_lb, S.predicate_ub) + float(S.V[index, 0])
+
+
+def get_mins(S: OStar, idx):
+    """Star.getMins, set/Star.m:784-856 (single-core branch)."""
+    return np.array([get_min(S, int(i)) for i in np.asarray(idx).reshape(-1)], dtype=np.float64)
+
+
+def get_maxs(S: OStar, idx):
+    """Star.getMaxs, set/Star.m:898-970."""
+    return np.array([get_max(S, int(i)) for i in np.asarray(idx).reshape(-1)], dtype=np.float64)
+
+
+def _round_half_away(x):
+    return int(np.floor(x + 0.5))  # MATLAB round() for x >= 0
+
+
+def _setdiff_stable(a, b):
+    """setdiff(a, b, 'stable') for index vectors."""
+    b = set(int(v) for v in np.asarray(b).reshape(-1))
+    return np.array([v for v in np.asarray(a).reshape(-1) if int(v) not in b], dtype=np.int64)
+
+
+def reach_relaxed_star_lp(I: OStar, method: str, relax_factor: float, rng=None) -> OStar:
+    """PosLin.reach_relaxed_star_{range,area,random,static} (nn/funcs/PosLin.m:863-983, 986-1104,
+    1425-1538, 1541-1650) and _{bound,ub} (:1107-1260, :1263-1422) for any relaxFactor:
+    n1 = round((1-rf)*numel(map2)) neurons get LP bounds.  Statement order follows the source."""
+    lb, ub = estimate_ranges(I)
+    map1 = np.flatnonzero(ub <= 0)
+    map2 = np.flatnonzero((lb < 0) & (ub > 0))
+    n1 = _round_half_away((1 - relax_factor) * map2.size)
+    if method in ("relax-star-range", "relax-star-area", "relax-star-random", "relax-star-static"):
+        if method == "relax-star-range":
+            midx = np.argsort(-(ub[map2] - lb[map2]), kind="stable")
+            map21, map22 = map2[midx[:n1]], map2[midx[n1:]]
+        elif method == "relax-star-area":
+            areas = 0.5 * (np.abs(ub[map2]) * np.abs(lb[map2]))
+            midx = np.argsort(-areas, kind="stable")
+            map21, map22 = map2[midx[:n1]], map2[midx[n1:]]
+        elif method == "relax-star-random":
+            midx = (rng or np.random).permutation(map2.size)[:n1]   # randperm(length(map2), n1)
+            map21 = map2[midx]
+            map22 = _setdiff_stable(map2, map21)
+        else:
+            map21, map22 = map2[:n1], map2[n1:]
+        lb1, ub1 = lb[map22], ub[map22]
+        xmax = get_maxs(I, map21)
+        map3 = np.flatnonzero(xmax <= 0)
+        map4 = map21[map3]
+        map11 = np.concatenate([map1, map4]).astype(np.int64)
+        In = reset_row(I, map11)
+        map5 = np.flatnonzero(xmax > 0)
+        map6 = map21[map5]
+        xmax1 = xmax[map5]
+        xmin = get_mins(I, map6)
+        map7 = np.flatnonzero(xmin < 0)
+        map8 = map6[map7]
+        lb2, ub2 = xmin[map7], xmax1[map7]
+        map9 = np.concatenate([map22, map8]).astype(np.int64)
+        lb3 = np.concatenate([lb1, lb2])
+        ub3 = np.concatenate([ub1, ub2])
+        return multiple_step_reach_star_approx_at_one(In, map9, lb3, ub3)
+    if method not in ("relax-star-bound", "relax-star-ub"):
+        raise ValueError("This reachability method does not exist")
+    N = map2.size
+    if method == "relax-star-bound":
+        lu = np.concatenate([ub[map2], np.abs(lb[map2])])
+        midx = np.argsort(-lu, kind="stable")
+        midx1 = midx[:2 * n1]
+        ub_idx = midx1[midx1 < N]
+        lb_idx = midx1[midx1 >= N] - N
+        map21, map22 = map2[ub_idx], map2[lb_idx]
+    else:
+        midx_u = np.argsort(-ub[map2], kind="stable")
+        midx_l = np.argsort(-np.abs(lb[map2]), kind="stable")
+        if 2 * n1 <= N:
+            map21, map22 = map2[midx_u[:2 * n1]], np.zeros(0, dtype=np.int64)
+        else:
+            map21, map22 = map2[midx_u[:N]], map2[midx_l[:2 * n1 - N]]
+    lb, ub = lb.copy(), ub.copy()
+    if map21.size:
+        xmax = get_maxs(I, map21)
+        map4 = map21[np.flatnonzero(xmax <= 0)]
+        map5 = np.flatnonzero(xmax > 0)
+        map6 = map21[map5]
+        map11 = np.concatenate([map1, map4]).astype(np.int64)
+    else:
+        map11, map5, map6, map4 = map1, np.zeros(0, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0, dtype=np.int64)
+    In = reset_row(I, map11)
+    map23 = _setdiff_stable(map22, map4) if map4.size else map22
+    if map23.size:
+        xmin = get_mins(I, map23)
+        map7 = np.flatnonzero(xmin < 0)
+        map8 = map23[map7]
+        map10 = map23[np.flatnonzero(xmin >= 0)]
+    else:
+        map7, map8, map10 = np.zeros(0, dtype=np.int64), np.zeros(0, dtype=np.int64), np.zeros(0, dtype=np.int64)
+    map24 = _setdiff_stable(map2, map4) if map4.size else map2
+    if map10.size:
+        map24 = _setdiff_stable(map24, map10)
+    if map6.size:
+        ub[map6] = xmax[map5]
+    if map8.size:
+        lb[map8] = xmin[map7]
+    return multiple_step_reach_star_approx_at_one(In, map24, lb[map24], ub[map24])
+
+
+def reach_relaxed_star(I: OStar, method: str, relax_factor: float = 1.0, rng=None) -> OStar:
+    """PosLin.reach_relaxed_star_{range,area,bound,ub,random,static} (nn/funcs/PosLin.m:863-1650).
+    At relaxFactor = 1, n1 = round((1-rf)*numel(map2)) = 0 and no LP is solved:
+    In = I.resetRow(map1); S = multipleStepReachStarApprox_at_one(In, map, lb(map), ub(map));
+    below 1 see reach_relaxed_star_lp."""
     if not isinstance(I, OStar):
         raise TypeError("Input is not a star")
     if relax_factor < 0 or relax_factor > 1:
         raise ValueError("Invalid relax factor")
+    if method not in RELAX_METHODS:
+        raise ValueError("This reachability method does not exist")
     if relax_factor != 1:
-        raise NotImplementedError("oracle restates the relaxFactor = 1 path only")
+        return reach_relaxed_star_lp(I, method, relax_factor, rng)
     lb, ub = estimate_ranges(I)
     map1, mp = relax_classify(lb, ub, method)
     In = reset_row(I, map1)

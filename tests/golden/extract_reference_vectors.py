@@ -11,6 +11,9 @@ Sources (data only; no reference code is imported or executed):
       written by code/nnv/tests/set/star/star_test.m
   * results/tests/baselines/nn/test_layers_relu_results.mat (IM_out) and the literals in
       code/nnv/tests/nn/layers/ReluLayer/test_layers_relu.m:19-33
+  * results/tests/baselines/set/test_star_intersect_halfSpace_results.mat
+      written by code/nnv/tests/set/star/test_star_intersect_halfSpace.m:66-79: a star with eleven
+      general constraint rows and no predicate bounds, and its LP ranges (Star.getRanges)
   * the literal inputs/expected outputs typed in
       code/nnv/tests/nn/layers/Conv2DLayer/test_layers_Conv2D.m:14-28  (conv known answer)
       code/nnv/tests/set/image_star/test_ImageStar_getRange.m:45-62    (ranges known answer)
@@ -42,6 +45,8 @@ def main():
                              ("W", "b", "S_V", "S_C", "S_d", "S1_V", "S1_C", "S1_d", "W2", "S4_lb", "S4_ub")}
     out["star_affineMap"]["box_lb"] = arr([0, -1, 0])   # test_star_affineMap.m:59
     out["star_affineMap"]["box_ub"] = arr([1, 1, 1])    # test_star_affineMap.m:60
+    m = sio.loadmat(os.path.join(base, "set/test_star_intersect_halfSpace_results.mat"))
+    out["star_intersect_halfSpace"] = {k: arr(m[k]) for k in ("H", "g", "S_V", "S1_V", "S1_C", "S1_d", "S1_lb", "S1_ub")}
     m = sio.loadmat(os.path.join(base, "set/star_test_results.mat"))
     out["star_test"] = {k: arr(m[k]) for k in ("S1_V", "S2_V", "S3_V", "B2_lb", "B2_ub")}
     # literal input / expected output of ReluLayer.evaluate typed in test_layers_relu.m:19-33
