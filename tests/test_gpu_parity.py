@@ -197,8 +197,14 @@ def test_relu_ties_and_degenerate(nnv, oracle):
         nnv.PosLin.reach(S, "relax-star-area", [], 1.5)
     with pytest.raises(ValueError, match="does not exist"):
         nnv.PosLin.reach(S, "relax-star", [], 1)
-    with pytest.raises(ValueError):
-        nnv.PosLin.reach(S, "relax-star-area", [], 0.5)
+    # below 1 the host solves LPs first; the all-device entry point says so instead of guessing
+    import ctypes
+    from nnv_amd._lib import ORDER_AREA, check
+    ctx = S.ctx
+    raw_in, raw_out = (ctypes.c_void_p * 1)(S._h.h), (ctypes.c_void_p * 1)()
+    with pytest.raises(ValueError, match="relaxFactor < 1"):
+        check(ctx.lib.nnvhip_relu_relax(ctx.handle, ORDER_AREA, 0.5, 1, raw_in, raw_out))
+    assert nnv.PosLin.reach(S, "relax-star-area", [], 0.5).nVar <= nnv.PosLin.reach(S, "relax-star-area", [], 1).nVar
 
 
 @pytest.mark.parametrize("method", ["relax-star-area", "relax-star-random"])
