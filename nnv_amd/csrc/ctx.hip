@@ -800,7 +800,9 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.pub = outs[i]->pub + (dense[i] - 1);
       g.part = nullptr;
       g.m = (int32_t)(nc - dense[i]);
-      g.pad_ = 0;
+      g.nfill = 0;
+      g.fill = nullptr;
+      g.bias = nullptr;
     }
     // sets whose implicit unit-vector columns take part in the contraction after all get them written out
     // (which also runs a pending row reset)
@@ -832,7 +834,8 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       if (!must && tiny) return false;
       const int64_t k = std::max<int64_t>(round_up(in[i]->n_kept, kLdAlign), kLdAlign);
       if (!must && 2 * k > fc->Kp) return false;
-      if (tiny)
+      static const double pack_min = getenv("NNVHIP_PACK_MIN_FLOP") ? atof(getenv("NNVHIP_PACK_MIN_FLOP")) : 0.0;
+      if (tiny || 2.0 * (double)fc->Mp * (double)k * (double)dense[i] * (double)count < pack_min)
         *pack = false;  // launch bound: read through the map
       else if (must && 2 * k > fc->Kp)
         *pack = true;
@@ -840,6 +843,14 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       r->flop = 2.0 * (double)fc->Mp * (double)k * (double)dense[i];
       *kp = k;
       return true;
+    };
+    // A set whose kept-row list is empty contracts over nothing: its dense columns are the bias and
+    // zeros, which the gather pass writes along with its own columns (no GEMM, no packing).
+    auto nothing_kept = [&](int64_t i, const GemmRows& r) { return r.kmap != nullptr && in[i]->n_kept == 0; };
+    auto fill_by_gather = [&](int64_t i) {
+      gs[i].nfill = (int32_t)dense[i];
+      gs[i].fill = outs[i]->V;
+      gs[i].bias = bias;
     };
     if (count == 1) {
       // one set: the GEMM epilogue also leaves the partial sums of Star.estimateRanges, so the
@@ -853,25 +864,37 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       int64_t kp = fc->Kp;
       bool pack = false;
       const bool compact = rows_of(0, &rows, &kp, &pack);
-      BufRef packed;
-      if (compact && pack) {
-        st = c->alloc(sizeof(double) * kp * dense[0], &packed);
-        if (st == NNVHIP_OK) {
-          PackSet ps{in[0]->V, in[0]->kept_idx, packed->as<double>(), in[0]->ld, (int32_t)kp, (int32_t)dense[0]};
-          st = launch_pack_rows(c, 1, &ps);
-          rows.Bk = packed->as<double>();
-          rows.ldbk = kp;
+      if (compact && nothing_kept(0, rows)) {
+        fill_by_gather(0);
+        const int64_t ch = std::max<int64_t>(1, gather_chunks(fc->Mp, std::max<int64_t>(gs[0].m, gs[0].nfill)));
+        BufRef part;
+        if (gs[0].m > 0) {
+          st = c->alloc(sizeof(double) * 4 * outs[0]->ld * ch, &part);
+          if (st == NNVHIP_OK) gs[0].part = part->as<double>();
         }
+        if (st == NNVHIP_OK) st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), gs[0].m > 0 ? ch : 0);
+        if (st == NNVHIP_OK && gs[0].m > 0) st = finalize_fused_ranges(c, outs[0], part, ch);
+      } else {
+        BufRef packed;
+        if (compact && pack) {
+          st = c->alloc(sizeof(double) * kp * dense[0], &packed);
+          if (st == NNVHIP_OK) {
+            PackSet ps{in[0]->V, in[0]->kept_idx, packed->as<double>(), in[0]->ld, (int32_t)kp, (int32_t)dense[0]};
+            st = launch_pack_rows(c, 1, &ps);
+            rows.Bk = packed->as<double>();
+            rows.ldbk = kp;
+          }
+        }
+        if (st == NNVHIP_OK)
+          st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
+                           compact ? &rows : nullptr);
+        const bool fused = st == NNVHIP_OK && fuse.chunks > 0;
+        if (st == NNVHIP_OK && gs[0].m > 0) {
+          gs[0].part = fused ? fuse.part->as<double>() + fuse.chunks * 4 * outs[0]->ld : nullptr;
+          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? gch : 0);
+        }
+        if (st == NNVHIP_OK && fused) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0));
       }
-      if (st == NNVHIP_OK)
-        st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
-                         compact ? &rows : nullptr);
-      const bool fused = st == NNVHIP_OK && fuse.chunks > 0;
-      if (st == NNVHIP_OK && gs[0].m > 0) {
-        gs[0].part = fused ? fuse.part->as<double>() + fuse.chunks * 4 * outs[0]->ld : nullptr;
-        st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? gch : 0);
-      }
-      if (st == NNVHIP_OK && fused) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0));
     } else if (contig) {
       // one launch for the whole array.  With structure to exploit, every set's dense columns are cut
       // into tiles of 128 that carry their own description (row list, position in the arena).
@@ -879,10 +902,18 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       std::vector<GemmRows> rws((size_t)count);
       std::vector<int64_t> kps((size_t)count);
       std::vector<char> pk((size_t)count, 0);
+      std::vector<char> filled((size_t)count, 0);
+      bool any_fill = false;
       for (int64_t i = 0; i < count; ++i) {
         bool pack = false;
         any_rows = rows_of(i, &rws[i], &kps[i], &pack) || any_rows;
         pk[i] = pack && rws[i].kmap != nullptr;
+        if (nothing_kept(i, rws[i])) {
+          fill_by_gather(i);
+          filled[i] = 1;
+          pk[i] = 0;
+          any_fill = true;
+        }
       }
       bool all_stored = true;
       for (int64_t i = 0; i < count; ++i) all_stored = all_stored && in[i]->stored_cols() == in[i]->n + 1;
@@ -930,7 +961,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         }
         int64_t off = 0, off_in = 0, kp_max = kLdAlign;
         for (int64_t i = 0; i < count; ++i) {
-          for (int64_t j = 0; j < dense[i]; j += tn) {
+          for (int64_t j = 0; j < dense[i] && !filled[i]; j += tn) {
             GemmSeg sg;
             sg.kmap = rws[i].kmap;
             sg.Bk = bk[i];
@@ -942,14 +973,16 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             sg.valid = (int32_t)std::min<int64_t>(tn, dense[i] - j);
             segs.push_back(sg);
           }
-          rows.flop += 2.0 * (double)fc->Mp * (double)kps[i] * (double)dense[i];
-          kp_max = std::max(kp_max, kps[i]);
+          if (!filled[i]) {
+            rows.flop += 2.0 * (double)fc->Mp * (double)kps[i] * (double)dense[i];
+            kp_max = std::max(kp_max, kps[i]);
+          }
           off += in[i]->n + 1;
           off_in += in[i]->stored_cols();
         }
         BufRef dsegs;
-        if (st == NNVHIP_OK) st = c->upload(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
-        if (st == NNVHIP_OK) {
+        if (st == NNVHIP_OK && !segs.empty()) st = c->upload(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
+        if (st == NNVHIP_OK && !segs.empty()) {
           rows.segs = dsegs->as<GemmSeg>();
           st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, tn * (int64_t)segs.size(),
                            kp_max, bias, nullptr, &rows);
@@ -958,23 +991,26 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols, fc->Kp, bias);
       }
       if (st == NNVHIP_OK && bias && count > 1) {
-        std::vector<double*> centres(count - 1);
-        for (int64_t i = 1; i < count; ++i) centres[i - 1] = outs[i]->V;
+        // the GEMM adds the bias to column 0 of the arena (the first set's centre); the other sets'
+        // centres get it here (a set whose dense columns the gather pass fills has it from there)
+        std::vector<double*> centres;
+        for (int64_t i = 1; i < count; ++i)
+          if (!filled[i]) centres.push_back(outs[i]->V);
         BufRef tab;
-        st = c->upload(centres.data(), sizeof(double*) * centres.size(), &tab);
-        if (st == NNVHIP_OK) st = launch_bias_columns(c, tab->as<double*>(), count - 1, bias, fc->Mp);
+        if (!centres.empty()) st = c->upload(centres.data(), sizeof(double*) * centres.size(), &tab);
+        if (st == NNVHIP_OK && !centres.empty()) st = launch_bias_columns(c, tab->as<double*>(), (int64_t)centres.size(), bias, fc->Mp);
       }
-      if (st == NNVHIP_OK && any_onehot) {
+      if (st == NNVHIP_OK && (any_onehot || any_fill)) {
         // the gather also leaves the range sums of its columns on the output handles, so the ReLU
         // that follows scans only the contracted columns
         int64_t max_m = 0;
         for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, gs[i].m);
-        const int64_t gch = gather_chunks_batch(outs[0]->ld, count, max_m);
+        const int64_t gch = gather_chunks_batch(outs[0]->ld, count, max_m);  // 0: nothing to gather, fills only
         BufRef sums;
-        st = c->alloc(sizeof(double) * 4 * outs[0]->ld * gch * count, &sums);
+        if (gch > 0) st = c->alloc(sizeof(double) * 4 * outs[0]->ld * gch * count, &sums);
         if (st == NNVHIP_OK) {
           for (int64_t i = 0; i < count; ++i)
-            gs[i].part = gs[i].m > 0 ? sums->as<double>() + 4 * outs[0]->ld * gch * i : nullptr;
+            gs[i].part = (gch > 0 && gs[i].m > 0) ? sums->as<double>() + 4 * outs[0]->ld * gch * i : nullptr;
           st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, count, gs.data(), gch);
         }
         for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
@@ -982,7 +1018,9 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             outs[i]->rng_buf = sums;
             outs[i]->rng_part = gs[i].part;
             outs[i]->rng_chunks = gch;
-            outs[i]->rng_first_col = dense[i];
+            // the columns before the gathered ones still need a scan -- unless they were filled with zeros,
+            // which add nothing to the sums
+            outs[i]->rng_first_col = filled[i] ? 1 : dense[i];
           }
       }
     } else {
@@ -991,6 +1029,11 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         int64_t kp = fc->Kp;
         bool pack = false;
         const bool compact = rows_of(i, &rows, &kp, &pack);
+        if (compact && nothing_kept(i, rows)) {
+          fill_by_gather(i);
+          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[i]->ld, 1, &gs[i], 0);
+          continue;
+        }
         BufRef packed;
         if (compact && pack) {
           st = c->alloc(sizeof(double) * kp * dense[i], &packed);

@@ -314,7 +314,9 @@ struct GatherSet {
   const double* pub;
   double* part;         // where this set's [chunks][4][ldout] range sums go, or null
   int32_t m;
-  int32_t pad_;
+  int32_t nfill;        // leading output columns that are known to be bias (column 0) and zeros: written here too
+  double* fill;         // column 0 of the output set (nfill > 0)
+  const double* bias;   // or null
 };
 int64_t gather_chunks(int64_t Mp, int64_t m);
 int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m);

@@ -153,6 +153,7 @@ struct GatherArgs {
   int64_t ldw, ldout;
   int32_t cols_per_chunk;
   int32_t with_sums;  // every chunk of the grid leaves range sums in the set's `part` (if it has one)
+  int64_t Mp;         // rows of W (a multiple of 16): the bias has that many entries
 };
 
 __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const GatherSet* __restrict__ table, GatherSet one,
@@ -161,12 +162,26 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   const int chunk = blockIdx.y;
   const int j0 = chunk * a.cols_per_chunk;
   double* part = a.with_sums ? d.part : nullptr;
-  if (j0 >= d.m && part == nullptr) return;
+  if (j0 >= d.m && part == nullptr && d.nfill == 0) return;
   const int j1 = min(d.m, j0 + a.cols_per_chunk);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t r0 = (int64_t)blockIdx.x * kRowsPerWave + 2 * lane;
   const bool active = r0 < a.ldout;
+  // A contraction over no rows at all leaves +0 everywhere and the bias on the centre: this chunk's share
+  // of those columns is written here instead of by a GEMM launch (they add nothing to the range sums).
+  if (d.nfill > 0 && active) {
+    const int fpc = (d.nfill + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int f1 = min(d.nfill, (chunk + 1) * fpc);
+    for (int j = chunk * fpc + wave; j < f1; j += kRangeWaves) {
+      double2 o = make_double2(0.0, 0.0);
+      if (j == 0 && d.bias != nullptr && r0 < a.Mp) {
+        o.x = __dadd_rn(0.0, d.bias[r0]);
+        o.y = __dadd_rn(0.0, d.bias[r0 + 1]);
+      }
+      *reinterpret_cast<double2*>(d.fill + r0 + (int64_t)j * a.ldout) = o;
+    }
+  }
   double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
   if (active) {
     for (int jb = j0 + 4 * wave; jb < j1; jb += 4 * kRangeWaves) {
@@ -252,18 +267,22 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
                           const GatherSet* sets, int64_t chunks) {
   if (count <= 0) return NNVHIP_OK;
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
-  int64_t max_m = 0;
-  for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, sets[i].m);
-  if (max_m == 0) return NNVHIP_OK;
+  int64_t max_m = 0, max_fill = 0;
+  for (int64_t i = 0; i < count; ++i) {
+    max_m = std::max<int64_t>(max_m, sets[i].m);
+    max_fill = std::max<int64_t>(max_fill, sets[i].nfill);
+  }
+  if (max_m == 0 && max_fill == 0) return NNVHIP_OK;
   const int64_t row_blocks = ceil_div(ldout, kRowsPerWave);
   const bool with_sums = chunks > 0;
-  if (!with_sums) chunks = gather_chunks_batch(ldout, count, max_m);
+  if (!with_sums) chunks = std::max<int64_t>(1, gather_chunks_batch(ldout, count, std::max(max_m, max_fill)));
   GatherArgs a{};
   a.W = W;
   a.ldw = ldw;
   a.ldout = ldout;
+  a.Mp = Mp;
   a.with_sums = with_sums ? 1 : 0;
-  a.cols_per_chunk = (int32_t)ceil_div(max_m, chunks);
+  a.cols_per_chunk = (int32_t)ceil_div(std::max<int64_t>(max_m, 1), chunks);
   const GatherSet* table = nullptr;
   BufRef tab;
   if (count > 1) {
@@ -273,7 +292,7 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
   // algorithmic HBM bytes: every output column written once, W read once (its columns are re-read
   // from cache)
   double bytes = 8.0 * (double)Mp * (double)ldw;
-  for (int64_t i = 0; i < count; ++i) bytes += 8.0 * (double)Mp * (double)sets[i].m;
+  for (int64_t i = 0; i < count; ++i) bytes += 8.0 * (double)Mp * (double)(sets[i].m + sets[i].nfill);
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   hipLaunchKernelGGL(gather_columns_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
                      dim3(64 * kRangeWaves), 0, ctx->stream, table, sets[0], a);

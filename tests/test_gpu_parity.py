@@ -419,3 +419,47 @@ def test_relu_output_whose_row_reset_is_still_pending(nnv, oracle, N, M):
     R2 = nnv.PosLin.reach(nnv.PosLin.reach(pre_d, "relax-star-area", [], 1), "relax-star-range", [], 1)
     E2 = oracle.reach_relaxed_star(relu_o, "relax-star-range", 1.0)
     assert np.array_equal(R2.V, E2.V)
+
+
+def test_fc_after_a_relu_that_kept_no_row(nnv, oracle):
+    # every neuron crossing or inactive: the columns the ReLU kept are all zero, so the next FC map has
+    # nothing to contract over -- centre = bias, zeros, gathered columns; alone, in one arena, mixed with a
+    # set that did keep rows, and without a bias
+    rs = np.random.RandomState(12)
+    n, N, M = 20, 400, 300                              # big enough for the structured route
+    W0 = rs.randn(N, n)
+    W1, b1 = rs.randn(M, N), rs.randn(M)
+    wide_lb, wide_ub = -np.ones((n, 3)) * 50, np.ones((n, 3)) * 50
+    wide_lb[:, 1], wide_ub[:, 1] = 0.5, 0.6              # the middle box is narrow: it keeps rows
+    L0 = nnv.FullyConnectedLayer(W0, np.zeros(N))
+    L1 = nnv.FullyConnectedLayer(W1, b1)
+    boxes = nnv.Star.from_boxes(wide_lb, wide_ub)
+    relu = nnv.PosLin.reach(L0.reach(boxes, "approx-star"), "relax-star-area", [], 1)
+    outs = L1.reach(relu, "approx-star")
+    kept = []
+    for i, (R, X) in enumerate(zip(outs, relu)):
+        O = oracle.reach_relaxed_star(oracle.affine_map(oracle.star_from_box(wide_lb[:, i], wide_ub[:, i]), W0, np.zeros(N)),
+                                      "relax-star-area", 1.0)
+        E = oracle.affine_map(O, W1, b1)
+        ni, idx, _, _ = X.relu_info()
+        kept.append(N - ni - idx.size)
+        assert_close(R.V, E.V, "fc after relu, set %d" % i)
+        lb, ub = R.estimateRanges()
+        elb, eub = oracle.estimate_ranges(E)
+        assert_close(lb, elb, "lb %d" % i)
+        assert_close(ub, eub, "ub %d" % i)
+        alone = L1.reach(nnv.PosLin.reach(L0.reach(nnv.Star(wide_lb[:, i], wide_ub[:, i]), "approx-star"),
+                                          "relax-star-area", [], 1), "approx-star")
+        if kept[-1] == 0:
+            assert np.array_equal(alone.V, R.V)      # nothing is summed: bit for bit
+        else:
+            assert_close(alone.V, R.V, "alone against batched")
+        nobias = nnv.PosLin.reach(L0.reach(nnv.Star(wide_lb[:, i], wide_ub[:, i]), "approx-star"),
+                                  "relax-star-area", [], 1).affineMap(W1, None)
+        assert_close(nobias.V, oracle.affine_map(O, W1, None).V, "no bias %d" % i)
+        # a second ReLU on top: its ranges come from the sums the gather pass left
+        R2 = nnv.PosLin.reach(R, "relax-star-range", [], 1)
+        E2 = oracle.reach_relaxed_star(E, "relax-star-range", 1.0)
+        assert R2.nVar == E2.nVar
+        assert_close(R2.V, E2.V, "second relu %d" % i)
+    assert kept[0] == 0 and kept[2] == 0 and kept[1] > 0
