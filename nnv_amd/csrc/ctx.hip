@@ -803,6 +803,10 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.nfill = 0;
       g.fill = nullptr;
       g.bias = nullptr;
+      g.red = nullptr;
+      g.red_k = 0;
+      g.pad_ = 0;
+      g.centre = nullptr;
     }
     // sets whose implicit unit-vector columns take part in the contraction after all get them written out
     // (which also runs a pending row reset)
@@ -885,10 +889,23 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             rows.ldbk = kp;
           }
         }
+        // only the centre is contracted (a box star): the range sums are the gather's alone
+        const bool centre_only = dense[0] == 1 && gs[0].m > 0;
+        SplitKDefer defer;  // ... and the gather pass also sums the centre's split-K partials
         if (st == NNVHIP_OK)
-          st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
-                           compact ? &rows : nullptr);
-        const bool fused = st == NNVHIP_OK && fuse.chunks > 0;
+          st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias,
+                           centre_only ? nullptr : &fuse, compact ? &rows : nullptr, centre_only ? &defer : nullptr);
+        if (st == NNVHIP_OK && centre_only) {
+          st = c->alloc(sizeof(double) * 4 * outs[0]->ld * gch, &fuse.part);
+          fuse.chunks = 0;
+          if (defer.ksplit > 1) {
+            gs[0].red = defer.ws->as<double>();
+            gs[0].red_k = (int32_t)defer.ksplit;
+            gs[0].centre = outs[0]->V;
+            gs[0].bias = bias;
+          }
+        }
+        const bool fused = st == NNVHIP_OK && (fuse.chunks > 0 || centre_only);
         if (st == NNVHIP_OK && gs[0].m > 0) {
           gs[0].part = fused ? fuse.part->as<double>() + fuse.chunks * 4 * outs[0]->ld : nullptr;
           st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? gch : 0);

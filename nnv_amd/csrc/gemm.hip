@@ -268,7 +268,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __rest
 template <int TM, int TN, int WR, int WC, int KT>
 static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
                       int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse,
-                      const GemmRows* rows) {
+                      const GemmRows* rows, SplitKDefer* defer) {
   int64_t tiles_m = ceil_div(Mp, TM);
   int64_t tiles_n = ceil_div(ncols, TN);
   int64_t blocks = tiles_m * tiles_n;
@@ -327,7 +327,10 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
                        (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
                        fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, nullptr, nullptr, nullptr, nullptr, 0);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, rows && rows->flop > 0.0 ? rows->flop : 2.0 * (double)Mp * (double)Kp * (double)ncols));
-  if (ksplit > 1) {
+  if (defer != nullptr) {
+    defer->ws = ws;
+    defer->ksplit = ksplit;
+  } else if (ksplit > 1) {
     const int64_t total = Mp * ncols;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream,
                        ws->as<double>(), (int)ksplit, (int)Mp, ncols, C, ldc, bias);
@@ -339,7 +342,8 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
 int gemm_seg_cols(int64_t Mp) { return Mp <= 16 ? 64 : 128; }
 
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C, int64_t ldc,
-                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse, const GemmRows* rows) {
+                int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse, const GemmRows* rows,
+                SplitKDefer* defer) {
   if (Mp % 16 || Kp % 16 || lda % 2 || ldb % 2 || Mp > lda || Kp > ldb || Mp > ldc)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: GEMM operands violate the padding contract");
   if (Mp >= (int64_t(1) << 31) || Kp >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large");
@@ -347,7 +351,7 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
   // Tile choice: the largest tile that still yields a few blocks per CU; skinny outputs (the last
   // layer has 10 rows) get a 16-row tile.  K must be a multiple of the K-tile (16 or 32).
 #define NNV_GEMM(TM, TN, WR, WC, KT) \
-  launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias, fuse, rows)
+  launch_cfg<TM, TN, WR, WC, KT>(ctx, A, lda, B, ldb, C, ldc, Mp, ncols, Kp, bias, fuse, rows, defer)
   const int64_t kCUs = 256;
   if (Mp <= 16) return NNV_GEMM(16, 64, 1, 4, 16);
   if (Mp <= 32) return NNV_GEMM(32, 128, 1, 4, 16);

@@ -273,9 +273,16 @@ struct PackSet {
   int32_t ncols;
 };
 int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
+// A split-K product leaves `ksplit` partial matrices (Mp x ncols each, ld = Mp) in a workspace; a caller
+// that has a pass over the output coming anyway can take the workspace instead of having the reduction
+// kernel launched (sum in split order, then the bias on column 0).  ksplit = 1: C is final.
+struct SplitKDefer {
+  BufRef ws;
+  int64_t ksplit = 1;
+};
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C,
                 int64_t ldc, int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse = nullptr,
-                const GemmRows* rows = nullptr);
+                const GemmRows* rows = nullptr, SplitKDefer* defer = nullptr);
 // Adds bias to the centre columns of sets 1..count-1 of an arena (set 0 is fused in the GEMM).
 int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t count, const double* bias,
                         int64_t Mp);
@@ -317,6 +324,10 @@ struct GatherSet {
   int32_t nfill;        // leading output columns that are known to be bias (column 0) and zeros: written here too
   double* fill;         // column 0 of the output set (nfill > 0)
   const double* bias;   // or null
+  const double* red;    // split-K partials of the centre column (red_k vectors of Mp entries) to be summed into
+  int32_t red_k;        // `centre`, plus the bias; null / 0 = the centre is final
+  int32_t pad_;
+  double* centre;
 };
 int64_t gather_chunks(int64_t Mp, int64_t m);
 int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m);

@@ -162,12 +162,27 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   const int chunk = blockIdx.y;
   const int j0 = chunk * a.cols_per_chunk;
   double* part = a.with_sums ? d.part : nullptr;
-  if (j0 >= d.m && part == nullptr && d.nfill == 0) return;
+  if (j0 >= d.m && part == nullptr && d.nfill == 0 && d.red == nullptr) return;
   const int j1 = min(d.m, j0 + a.cols_per_chunk);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t r0 = (int64_t)blockIdx.x * kRowsPerWave + 2 * lane;
   const bool active = r0 < a.ldout;
+  // The centre column came out of a split-K product: the first chunk's blocks sum its partial vectors in
+  // split order and add the bias, as the reduction kernel would have.
+  if (d.red != nullptr && chunk == 0 && wave == 0 && active && r0 < a.Mp) {
+    double2 s = make_double2(0.0, 0.0);
+    for (int k = 0; k < d.red_k; ++k) {
+      const double2 p = *reinterpret_cast<const double2*>(d.red + (int64_t)k * a.Mp + r0);
+      s.x += p.x;
+      s.y += p.y;
+    }
+    if (d.bias != nullptr) {
+      s.x = s.x + d.bias[r0];
+      s.y = s.y + d.bias[r0 + 1];
+    }
+    *reinterpret_cast<double2*>(d.centre + r0) = s;
+  }
   // A contraction over no rows at all leaves +0 everywhere and the bias on the centre: this chunk's share
   // of those columns is written here instead of by a GEMM launch (they add nothing to the range sums).
   if (d.nfill > 0 && active) {
