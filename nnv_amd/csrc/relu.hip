@@ -295,14 +295,14 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     keep_base += ktot;
     if (crossing) {
       const int pos = base + woff + __popcll(bc & ((1ull << lane) - 1ull));
-      idx_out[pos] = r;
       d.cls[r] = pos;
-      if (d.order != NNVHIP_ORDER_INDEX) {
-        // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb
+      if (d.order == NNVHIP_ORDER_INDEX) {
+        idx_out[pos] = r;
+      } else {
+        // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb.  The list is sorted below, straight from LDS (a
+        // set of at most SORT_CAP neurons cannot have more crossing ones).
         const double key = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l))
                            : d.order == NNVHIP_ORDER_RANGE ? u - l : d.given_key[r];
-        d.key[pos] = key;
-        d.rank[pos] = 0;
         if (SORT_CAP > 0 && pos < SORT_CAP) {
           skey[pos] = key;
           sidx[pos] = r;
@@ -336,7 +336,35 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   if (d.write_bounds) {  // the output buffers were sized for the worst case: finish the set here
     __syncthreads();     // cross_idx is complete
     const int n_in = d.ncols_in - 1;
-    for (int j = tid; j < n_in + m; j += 1024) write_pred_bound(d, n_in, j);
+    // four entries per thread and step, all loads issued before the first store (the dependent
+    // index -> bound look-ups of the new predicates would otherwise queue up behind one another)
+    for (int jb = tid; jb < n_in + m; jb += 4096) {
+      double a[4], b[4], c[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = jb + u * 1024;
+        a[u] = b[u] = c[u] = 0.0;
+        if (j < n_in) {
+          a[u] = d.plb_in[j];
+          b[u] = d.pub_in[j];
+        } else if (j < n_in + m) {
+          const int neuron = d.cross_idx[j - n_in];
+          b[u] = d.ub[neuron];
+          c[u] = d.lb[neuron];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = jb + u * 1024;
+        if (j >= n_in + m) break;
+        d.plb_out[j] = a[u];  // new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]
+        d.pub_out[j] = b[u];
+        if (j >= n_in) {
+          d.lbub[j - n_in] = c[u];
+          d.lbub[d.ld_lbub + (j - n_in)] = b[u];
+        }
+      }
+    }
   }
 }
 
