@@ -114,7 +114,7 @@ def main():
         return acc / reps
 
     per_layer = timed_pass(1)          # NN.reachTime-style device time per layer
-    for grp in range(6):
+    for grp in range(8):
         ctx.kernel_time(grp)
     timed_pass(2)                      # per-kernel event pairs
     gemm_ms, gemm_launches, gemm_work = ctx.kernel_time(0)
@@ -123,6 +123,8 @@ def main():
     app_ms, app_launches, app_bytes = ctx.kernel_time(3)
     row_ms, row_launches, row_bytes = ctx.kernel_time(4)
     gat_ms, gat_launches, gat_bytes = ctx.kernel_time(5)
+    cls_ms, cls_launches, cls_bytes = ctx.kernel_time(6)
+    fin_ms, fin_launches, fin_bytes = ctx.kernel_time(7)
 
     # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
     gemm_flop = conv_flop = 0.0
@@ -203,9 +205,23 @@ def main():
         groups.append((row_ms, hbm_roofline("row-wise affine layers (rowmap/avgpool/permute kernels)", row_ms, row_launches, row_bytes)))
     if gat_launches:
         groups.append((gat_ms, hbm_roofline("gather_columns_kernel", gat_ms, gat_launches, gat_bytes)))
+    if fin_launches:
+        groups.append((fin_ms, hbm_roofline("ranges_final_kernel", fin_ms, fin_launches, fin_bytes)))
     groups.sort(key=lambda g: -g[0])
     roofline = dict(groups[0][1])
     roofline["other_kernels"] = [g[1] for g in groups[1:]]
+    n_sets = len(dev_in) if isinstance(dev_in, list) else 1
+    if cls_launches:
+        # One block per set (classification, in-block sort of the crossing list, new predicate bounds): a
+        # dependent chain on a single CU, bound by latency and not by a roofline.  It is listed with the
+        # bytes it touches; with a single input set it can be the longest kernel of a reach, and the
+        # roofline object above then describes the longest throughput-bound kernel.
+        c = hbm_roofline("relu_classify_kernel", cls_ms, cls_launches, cls_bytes)
+        c["latency_bound"] = True
+        c["blocks_per_launch"] = n_sets
+        roofline["other_kernels"].append(c)
+        if cls_ms > groups[0][0]:
+            roofline["longest_kernel_by_time"] = "relu_classify_kernel (latency bound, %d block(s) per launch)" % n_sets
     # the MFMA GEMM on the full dense problem of the same reach (what Star.affineMap executes in the
     # reference): a short extra pass with the skipping of structural zeros switched off
     if gemm_launches and not args.dense:

@@ -84,14 +84,17 @@ NNVHIP_API int nnvhip_set_dense_affine(nnvhip_ctx* ctx, int enabled);
  * kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
  * dense GEMM kernel of the FC layers (tiles of at least 64 rows); 1: implicit-GEMM convolution
  * kernel; 2: estimateRanges column pass; 3: ReLU apply pass; 4: row-wise affine layers (row map,
- * average pooling, row permutation); 5: column gather of an FC layer (its one-hot generator columns).
+ * average pooling, row permutation); 5: column gather of an FC layer (its one-hot generator columns);
+ * 6: classification of the ReLU step (incl. the sort of the crossing list and, for sets of up to 8192
+ * neurons, the new predicate bounds); 7: the reduction of range partial sums into lb / ub.
  * Returns accumulated kernel time,
  * launch count and work since the last reset.  Work is the flop executed for 0 and 1 (GEMM:
  * 2*Mp*Kp*ncols over the columns and rows the launch contracts, M and K padded to 16; conv:
  * 2*Ho*Wo*Cout*FH*FW*Cin*(n+1)) and algorithmic bytes for
  * 2 (8*N*(n+1) + 16*n + 16*N per set), 3 (8*kept*(n+1) read + 8*N*(n+1+m) written per set, kept =
- * rows that are neither inactive nor crossing), 4 (8*(Nin + Nout)*(n+1) per set) and 5 (8*M per
- * gathered column written + W read once). */
+ * rows that are neither inactive nor crossing), 4 (8*(Nin + Nout)*(n+1) per set), 5 (8*M per
+ * gathered column written + W read once), 6 (24*N per set, + 32*n when the bounds are written too)
+ * and 7 (8*N*(4*chunks + 3) per set). */
 NNVHIP_API int nnvhip_kernel_time(nnvhip_ctx* ctx, int which, double* total_ms, int64_t* launches, double* total_work,
                        int reset);
 /* Measurement hook (no counterpart in the reference): runs a plain device-to-device copy kernel over

@@ -311,8 +311,8 @@ static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvG
   if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
   const size_t dyn = sizeof(unsigned long long) * g.Kp;
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL((conv2d_f64_kernel<TP, TC, WR, WC>), dim3((unsigned)blocks), dim3(64 * WR * WC), dyn, ctx->stream, in, ldin,
-                     out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows,
+  NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_f64_kernel<TP, TC, WR, WC>), dim3((unsigned)blocks), dim3(64 * WR * WC), dyn, in, ldin,
+             out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows,
                      (int)tiles_c);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 1, 2.0 * (double)total_rows * g.Cout * g.K));
   NNV_HIP_TRY(hipGetLastError());
@@ -400,8 +400,8 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int6
   StampSet one;
   memcpy(&one, &sets[0], sizeof one);
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL(conv_stamp_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(512), 0,
-                     ctx->stream, table, one, g, cv->W->as<double>(), ldout, (int)cpc);
+  NNV_LAUNCH(ctx, ctx->kernel_timing, conv_stamp_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(512), 0,
+             table, one, g, cv->W->as<double>(), ldout, (int)cpc);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;

@@ -114,14 +114,10 @@ int nnvhip_ctx::upload(const void* host, size_t bytes, BufRef* out) {
   return NNVHIP_OK;
 }
 
-int nnvhip_ctx::kernel_timer_begin(bool on) {
-  if (on) NNV_HIP_TRY(hipEventRecord(kev0, stream));
-  return NNVHIP_OK;
-}
+int nnvhip_ctx::kernel_timer_begin(bool) { return NNVHIP_OK; }  // the events travel with the launch (NNV_LAUNCH)
 
 int nnvhip_ctx::kernel_timer_end(bool on, int which, double flop) {
-  if (on) {  // events directly around one kernel: its duration alone, as a profiler reports it
-    NNV_HIP_TRY(hipEventRecord(kev1, stream));
+  if (on) {  // start / stop events of the one kernel just launched
     NNV_HIP_TRY(hipEventSynchronize(kev1));
     float ms = 0.f;
     NNV_HIP_TRY(hipEventElapsedTime(&ms, kev0, kev1));

@@ -345,7 +345,7 @@ int nnvhip_affine_rowmap(nnvhip_ctx* c, const nnvhip_rowmap* m, int64_t count, n
   return run_row_layer(c, count, in, out, m->N, kEwRows, 4 * kEwWaves,
                        [&](dim3 grid, const SetDesc* table, const SetDesc& one, int32_t cpc, int64_t) {
                          a.cols_per_chunk = cpc;
-                         hipLaunchKernelGGL(rowmap_kernel, grid, dim3(64 * kEwWaves), 0, c->stream, table, one, a);
+                         NNV_LAUNCH(c, c->kernel_timing, rowmap_kernel, grid, dim3(64 * kEwWaves), 0, table, one, a);
                        });
 }
 
@@ -418,7 +418,7 @@ int nnvhip_affine_avgpool2d(nnvhip_ctx* c, const nnvhip_avgpool2d* p, int64_t H,
                        [&](dim3 grid, const SetDesc* table, const SetDesc& one, int32_t cpc, int64_t ldout) {
                          a.cols_per_chunk = cpc;
                          a.ldout = ldout;
-                         hipLaunchKernelGGL(avgpool_kernel, grid, dim3(64 * kEwWaves), 0, c->stream, table, one, a);
+                         NNV_LAUNCH(c, c->kernel_timing, avgpool_kernel, grid, dim3(64 * kEwWaves), 0, table, one, a);
                        });
 }
 
@@ -449,14 +449,14 @@ int nnvhip_permute_rows(nnvhip_ctx* c, int64_t N, const int32_t* src_row, int64_
                          [&](dim3 grid, const SetDesc* table, const SetDesc& one, int32_t cpc, int64_t ldout) {
                            a.cols_per_chunk = cpc;
                            a.ldout = ldout;
-                           hipLaunchKernelGGL(permute_rows_lds_kernel, grid, dim3(64 * kEwWaves), 0, c->stream, table, one,
+                           NNV_LAUNCH(c, c->kernel_timing, permute_rows_lds_kernel, grid, dim3(64 * kEwWaves), 0, table, one,
                                               a, (int)N);
                          });
   return run_row_layer(c, count, in, out, N, kEwRows, 4 * kEwWaves,
                        [&](dim3 grid, const SetDesc* table, const SetDesc& one, int32_t cpc, int64_t ldout) {
                          a.cols_per_chunk = cpc;
                          a.ldout = ldout;
-                         hipLaunchKernelGGL(permute_rows_kernel, grid, dim3(64 * kEwWaves), 0, c->stream, table, one, a);
+                         NNV_LAUNCH(c, c->kernel_timing, permute_rows_kernel, grid, dim3(64 * kEwWaves), 0, table, one, a);
                        });
 }
 

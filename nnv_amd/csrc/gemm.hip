@@ -316,14 +316,14 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   const bool timed = ctx->kernel_timing && TM >= 64;
   NNV_TRY(ctx->kernel_timer_begin(timed));
   if (rows != nullptr)
-    hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT, true>), dim3((unsigned)grid_x, (unsigned)ksplit),
-                       dim3(64 * WR * WC), 0, ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
+    NNV_LAUNCH(ctx, timed, (gemm_f64_kernel<TM, TN, WR, WC, KT, true>), dim3((unsigned)grid_x, (unsigned)ksplit),
+                       dim3(64 * WR * WC), 0, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
                        (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
                        fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, rows->kmap, rows->segs, rows->colmap,
                        rows->Bk, rows->ldbk);
   else
-    hipLaunchKernelGGL((gemm_f64_kernel<TM, TN, WR, WC, KT, false>), dim3((unsigned)grid_x, (unsigned)ksplit),
-                       dim3(64 * WR * WC), 0, ctx->stream, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
+    NNV_LAUNCH(ctx, timed, (gemm_f64_kernel<TM, TN, WR, WC, KT, false>), dim3((unsigned)grid_x, (unsigned)ksplit),
+                       dim3(64 * WR * WC), 0, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
                        (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
                        fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, nullptr, nullptr, nullptr, nullptr, 0);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, rows && rows->flop > 0.0 ? rows->flop : 2.0 * (double)Mp * (double)Kp * (double)ncols));

@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <atomic>
 #include <cstdarg>
@@ -120,10 +121,10 @@ struct nnvhip_ctx {
   // [2] estimateRanges column pass, [3] ReLU apply pass, [4] row-wise affine layers (batch
   // normalisation, input normalisation, average pooling, flatten), [5] gather of W's columns for the
   // one-hot generator columns of an FC layer (work = algorithmic bytes)
-  static constexpr int kKernelGroups = 6;
-  double kern_ms[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
-  int64_t kern_launches[kKernelGroups] = {0, 0, 0, 0, 0, 0};
-  double kern_flop[kKernelGroups] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+  static constexpr int kKernelGroups = 8;
+  double kern_ms[kKernelGroups] = {};
+  int64_t kern_launches[kKernelGroups] = {};
+  double kern_flop[kKernelGroups] = {};
   int kernel_timer_begin(bool on);
   int kernel_timer_end(bool on, int which, double flop);
 
@@ -137,6 +138,17 @@ struct nnvhip_ctx {
   int begin_op();
   int end_op();
 };
+
+// Launch on the context's stream.  With `on` the start and stop events ride on the kernel's own
+// dispatch, so kernel_timer_end() reads the duration of the kernel alone (what a profiler reports),
+// not that of an event-launch-event sequence.
+#define NNV_LAUNCH(ctx, on, kernel, grid, block, shmem, ...)                                                       \
+  do {                                                                                                              \
+    if (on)                                                                                                         \
+      hipExtLaunchKernelGGL(kernel, grid, block, shmem, (ctx)->stream, (ctx)->kev0, (ctx)->kev1, 0, __VA_ARGS__); \
+    else                                                                                                            \
+      hipLaunchKernelGGL(kernel, grid, block, shmem, (ctx)->stream, __VA_ARGS__);                                  \
+  } while (0)
 
 struct nnvhip_star {
   std::atomic<int> refs{1};

@@ -309,8 +309,8 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
   double bytes = 8.0 * (double)Mp * (double)ldw;
   for (int64_t i = 0; i < count; ++i) bytes += 8.0 * (double)Mp * (double)(sets[i].m + sets[i].nfill);
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL(gather_columns_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
-                     dim3(64 * kRangeWaves), 0, ctx->stream, table, sets[0], a);
+  NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
+             dim3(64 * kRangeWaves), 0, table, sets[0], a);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
@@ -395,11 +395,15 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   for (int64_t i = 0; i < nset; ++i)
     bytes += 8.0 * (double)todo[i]->N * (double)(descs[i].n + 1) + 16.0 * (double)descs[i].n + 16.0 * (double)todo[i]->N;
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL((ranges_partial_kernel<8, 4>), grid, dim3(64 * kRangeWaves), 0, ctx->stream, table, descs[0]);
+  NNV_LAUNCH(ctx, ctx->kernel_timing, (ranges_partial_kernel<8, 4>), grid, dim3(64 * kRangeWaves), 0, table, descs[0]);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
-  if (chunks > 1 || any_pending)
-    hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,
-                       ctx->stream, table, descs[0]);
+  if (chunks > 1 || any_pending) {
+    double fbytes = 0.0;  // every chunk's four sums read, lb and ub written
+    for (int64_t i = 0; i < nset; ++i) fbytes += 8.0 * (double)ld * (4.0 * (double)(descs[i].chunks + descs[i].chunks2) + 3.0);
+    NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,
+               table, descs[0]);
+    NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 7, fbytes));
+  }
   NNV_HIP_TRY(hipGetLastError());
   for (int64_t i = 0; i < nset; ++i) {
     todo[i]->rbuf = rb;
@@ -430,7 +434,8 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
   d.row_waves = 1;
   d.part2 = nullptr;
   d.chunks2 = 0;
-  hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(s->ld, 64), 1, 1), dim3(256), 0, ctx->stream, nullptr, d);
+  NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel, dim3((unsigned)ceil_div(s->ld, 64), 1, 1), dim3(256), 0, nullptr, d);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 7, 8.0 * (double)s->ld * (4.0 * (double)chunks + 3.0)));
   NNV_HIP_TRY(hipGetLastError());
   s->rbuf = rb;
   s->lb = d.lb;

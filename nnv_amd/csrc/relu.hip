@@ -668,8 +668,8 @@ static int launch_apply(nnvhip_ctx* ctx, int64_t count, std::vector<ReluDesc>& d
     table = tab->as<ReluDesc>();
   }
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  hipLaunchKernelGGL(relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(64 * kApplyWaves), 0,
-                     ctx->stream, table, descs[0]);
+  NNV_LAUNCH(ctx, ctx->kernel_timing, relu_apply_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
+             dim3(64 * kApplyWaves), 0, table, descs[0]);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 3, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
@@ -852,17 +852,25 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // Up to 8192 neurons: one block per set classifies, compacts and sorts (bitonic network).  Larger
   // sets: two multi-block passes; their sort, if any, follows the read-back of the counts.
   const int sort_cap = !sorted ? 0 : N <= 1024 ? 1024 : N <= 8192 ? 8192 : 0;
+  // algorithmic bytes of the classification: lb and ub read, the per-row class and the two index lists
+  // written (plus, when it also writes the predicate bounds, the copy of the input's)
+  double cls_bytes = 0.0;
+  for (int64_t i = 0; i < count; ++i) cls_bytes += 24.0 * (double)N + (fold_bounds ? 32.0 * (double)in[i]->n : 0.0);
+  const bool tk = ctx->kernel_timing;
   if (N <= 8192) {
     if (!sorted)
-      hipLaunchKernelGGL(relu_classify_kernel<0>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+      NNV_LAUNCH(ctx, tk, relu_classify_kernel<0>, dim3((unsigned)count), dim3(1024), 0, table, descs[0]);
     else if (N <= 1024)
-      hipLaunchKernelGGL(relu_classify_kernel<1024>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+      NNV_LAUNCH(ctx, tk, relu_classify_kernel<1024>, dim3((unsigned)count), dim3(1024), 0, table, descs[0]);
     else
-      hipLaunchKernelGGL(relu_classify_kernel<8192>, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+      NNV_LAUNCH(ctx, tk, relu_classify_kernel<8192>, dim3((unsigned)count), dim3(1024), 0, table, descs[0]);
+    NNV_TRY(ctx->kernel_timer_end(tk, 6, cls_bytes));
   } else {
     const dim3 grid((unsigned)ceil_div(N, 1024), 1, (unsigned)count);
-    hipLaunchKernelGGL(relu_count_kernel, grid, dim3(1024), 0, ctx->stream, table, descs[0]);
-    hipLaunchKernelGGL(relu_compact_kernel, grid, dim3(1024), 0, ctx->stream, table, descs[0]);
+    NNV_LAUNCH(ctx, tk, relu_count_kernel, grid, dim3(1024), 0, table, descs[0]);
+    NNV_TRY(ctx->kernel_timer_end(tk, 6, 0.5 * cls_bytes));
+    NNV_LAUNCH(ctx, tk, relu_compact_kernel, grid, dim3(1024), 0, table, descs[0]);
+    NNV_TRY(ctx->kernel_timer_end(tk, 6, 0.5 * cls_bytes));
   }
   NNV_HIP_TRY(hipGetLastError());
 
