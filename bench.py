@@ -31,8 +31,10 @@ FP64_MFMA_PEAK_TFLOPS = 78.6
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by the 1 GiB copy kernel of the same run (profiles/<workload>_hbm_traffic.md): (read, write) MiB
-# averaged over the three launches of a step (the 64x64, 64x96 and 128x80 tile instantiations)
-MEASURED_TRAFFIC_MIB = {("cfg2_fc_784_1024x3_10", "gemm_f64_kernel", "dense"): (51.30, 12.36)}
+# averaged over the launches of a step (dense GEMM: the 64x64, 64x96 and 128x80 tile instantiations; gather:
+# the four FC layers)
+MEASURED_TRAFFIC_MIB = {("cfg2_fc_784_1024x3_10", "gemm_f64_kernel", "dense"): (51.30, 12.36),
+                        ("cfg2_fc_784_1024x3_10", "gather_columns_kernel", "structured"): (4.89, 8.07)}
 
 
 def layer_shapes(reach_set):
