@@ -834,8 +834,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       if (!must && tiny) return false;
       const int64_t k = std::max<int64_t>(round_up(in[i]->n_kept, kLdAlign), kLdAlign);
       if (!must && 2 * k > fc->Kp) return false;
-      static const double pack_min = getenv("NNVHIP_PACK_MIN_FLOP") ? atof(getenv("NNVHIP_PACK_MIN_FLOP")) : 0.0;
-      if (tiny || 2.0 * (double)fc->Mp * (double)k * (double)dense[i] * (double)count < pack_min)
+      if (tiny)
         *pack = false;  // launch bound: read through the map
       else if (must && 2 * k > fc->Kp)
         *pack = true;

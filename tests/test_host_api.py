@@ -75,3 +75,47 @@ def test_configs_are_reproducible_and_sized():
     assert c3["layers"][4]["W"].shape == (100, 14 * 14 * 32)
     assert abs(np.std(a["layers"][2]["W"]) - np.sqrt(2.0 / 1024)) < 1e-3
     assert count_updates([(3, 4), (2, 1)]) == 3 * 5 + 2 * 2
+
+
+class _HostStar:
+    """Stands where a device Star would: ranges and LP bounds of an oracle star, so the host-side
+    bookkeeping of the relaxFactor < 1 heuristics can be checked without a GPU."""
+
+    def __init__(self, S):
+        self.S = S
+
+    def estimateRanges(self):
+        return o.estimate_ranges(self.S)
+
+    def getMaxs(self, idx, *_):
+        return o.get_maxs(self.S, idx)
+
+    def getMins(self, idx, *_):
+        return o.get_mins(self.S, idx)
+
+
+@pytest.mark.parametrize("method", sorted(RELAX_ORDER))
+@pytest.mark.parametrize("rf", [0.0, 0.3, 0.5, 1.0])
+def test_relax_factor_bookkeeping_hands_the_device_the_oracles_lists(monkeypatch, method, rf):
+    # which neurons are reset, which cross with which bounds, and in which order: the lists the host code
+    # passes to the device step must be the ones the restatement of PosLin.reach_relaxed_star_* builds
+    from nnv_amd import layers
+    rs = np.random.RandomState(4)
+    n, N = 5, 30
+    I = o.star_from_box(-rs.rand(n) - 0.2, rs.rand(n) + 0.2)
+    S = o.affine_map(o.reach_relaxed_star(o.affine_map(I, rs.randn(N, n), rs.randn(N) * 0.3), "relax-star-area", 1.0),
+                     rs.randn(N, N) * 0.5, rs.randn(N) * 0.3)
+    seen = {}
+
+    def capture(star, index, lb, ub, reset=()):
+        seen.update(index=np.asarray(index), lb=np.asarray(lb), ub=np.asarray(ub), reset=np.asarray(reset))
+        return o.multiple_step_reach_star_approx_at_one(o.reset_row(star.S, np.asarray(reset, dtype=int)), index, lb, ub)
+
+    monkeypatch.setattr(layers.PosLin, "multipleStepReachStarApprox_at_one", staticmethod(capture))
+    got = layers._relaxed_star_lp(_HostStar(S), method, rf, rng=np.random.RandomState(8))
+    want = o.reach_relaxed_star_lp(S, method, rf, np.random.RandomState(8))
+    assert np.array_equal(got.V, want.V) and np.array_equal(got.C, want.C) and np.array_equal(got.d, want.d)
+    assert np.array_equal(got.predicate_ub, want.predicate_ub)
+    assert np.all(seen["lb"] < 0) and np.all(seen["ub"] > 0)          # what the device step insists on
+    assert len(set(seen["index"]) & set(seen["reset"])) == 0
+    assert len(set(seen["index"])) == seen["index"].size
