@@ -54,14 +54,18 @@ struct ReluDesc {
   int32_t write_bounds; // apply pass: 1 = also write the predicate bounds and the crossing neurons' (lb, ub)
 };
 
-// Posts the counts to the host mailbox: payload first, system-scope fence, then the sequence number
-// the host is spinning on.
+// Posts the counts to the host mailbox.  Payload and sequence number travel in one naturally aligned
+// 64-bit store (sequence number in the top 16 bits, the two counts in 24 bits each), so there is nothing
+// to order and nothing for the posting wave to wait for.
+constexpr int kMailboxCountBits = 24;
+__host__ __device__ __forceinline__ unsigned long long mailbox_word(int m, int inactive, int seq) {
+  return ((unsigned long long)((unsigned)seq & 0xffffu) << (2 * kMailboxCountBits)) |
+         ((unsigned long long)(unsigned)m << kMailboxCountBits) | (unsigned long long)(unsigned)inactive;
+}
 __device__ __forceinline__ void post_counts(int32_t* mailbox, int m, int inactive, int seq) {
   if (mailbox == nullptr) return;
-  mailbox[0] = m;
-  mailbox[1] = inactive;
-  __threadfence_system();
-  __hip_atomic_store(&mailbox[2], seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), mailbox_word(m, inactive, seq), __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // "a sorts before b" under the stable descending key order: larger key first, ties by smaller
@@ -321,13 +325,14 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     if (keep_base + tid < end) d.keep_idx[keep_base + tid] = -1;
   }
   const int m = base;
+  const bool sort_here = SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP;
+  if (sort_here) __syncthreads();  // the keys are staged; nothing of the stores below is in flight yet
   if (tid == 0) {
     d.counts[0] = m;
     d.counts[1] = inact_total;
     post_counts(d.mailbox, m, inact_total, d.mailbox_seq);  // the host can size the output while we sort
   }
-  if (SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP) {
-    __syncthreads();
+  if (sort_here) {
     if (SORT_CAP == 1024 || m <= 1024)  // the staged doubles are read back as their bit patterns
       sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
     else
@@ -838,7 +843,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.ncols_in = (int32_t)(in[i]->n + 1);
     d.order = order;
   }
-  const bool use_mailbox = count == 1 && ctx->mailbox != nullptr;
+  const bool use_mailbox = count == 1 && ctx->mailbox != nullptr && N < (int64_t(1) << kMailboxCountBits);
   if (use_mailbox) {
     descs[0].mailbox = const_cast<int32_t*>(ctx->mailbox);
     descs[0].mailbox_seq = ++ctx->mailbox_seq;
@@ -880,16 +885,19 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     // one set: the kernel posts the counts to pinned host memory; spin on the sequence number
     const auto t0 = std::chrono::steady_clock::now();
     long spins = 0;
-    while (ctx->mailbox[2] != ctx->mailbox_seq) {
+    const volatile unsigned long long* box = reinterpret_cast<const volatile unsigned long long*>(ctx->mailbox);
+    const unsigned long long want = (unsigned long long)((unsigned)ctx->mailbox_seq & 0xffffu);
+    unsigned long long w = *box;
+    while ((w >> (2 * kMailboxCountBits)) != want) {
       if ((++spins & 0xfff) == 0 &&
           std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 10.0) {
         NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));  // surfaces a launch failure, if any
-        if (ctx->mailbox[2] != ctx->mailbox_seq) NNV_FAIL(NNVHIP_ERR_HIP, "classification kernel did not report its counts");
+        if (((*box) >> (2 * kMailboxCountBits)) != want) NNV_FAIL(NNVHIP_ERR_HIP, "classification kernel did not report its counts");
       }
+      w = *box;
     }
-    std::atomic_thread_fence(std::memory_order_acquire);
-    counts[0] = ctx->mailbox[0];
-    counts[1] = ctx->mailbox[1];
+    counts[0] = (int32_t)((w >> kMailboxCountBits) & ((1u << kMailboxCountBits) - 1));
+    counts[1] = (int32_t)(w & ((1u << kMailboxCountBits) - 1));
   } else {
     void* hc = nullptr;
     NNV_TRY(ctx->stage(sizeof(int32_t) * 2 * count, &hc));
