@@ -41,7 +41,9 @@ Parity pinning (what checks each function; see tests/test_oracle_*.py)
   containment invariant of the reference's soundness tests.  get_min / get_max through the solver
   branch are checked against the reference's stored LP ranges of a star with eleven general
   constraint rows (results/tests/baselines/set/test_star_intersect_halfSpace_results.mat, S1_lb /
-  S1_ub, written by tests/set/star/test_star_intersect_halfSpace.m:66-79) to 1e-8.
+  S1_ub, written by tests/set/star/test_star_intersect_halfSpace.m:66-79) and the stored Star.getBox of
+  another (test_star_getBoxFast_results.mat, B1) to 1e-8; the same file's getBoxFast box (B2) is a second
+  known answer for estimate_ranges' interval formula on a general V.
 * halfspace_contains / is_empty_set / intersect_half_space: the reference's known answers
   (tests/set/halfspace/test_half_space_contain.m, tests/set/star/test_star_isEmptySet.m:17-23,
   tests/soundness/test_set_conversion.m:60-68) and closed forms on boxes.  The LP itself is

@@ -163,3 +163,44 @@ def test_network_reach_with_relax_factor(nnv, oracle, method, rf):
     l1, u1 = full.estimateRanges()
     assert np.all(lb >= l1 - 1e-7) and np.all(ub <= u1 + 1e-7)
     assert out.nVar <= full.nVar
+
+
+def test_lp_box_and_interval_box_known_answers(nnv, oracle, golden):
+    # the reference's stored Star.getBox (LP) and Star.getBoxFast (interval arithmetic over the predicates'
+    # bounding box) of one star: host LPs fed from the device, and the device's estimateRanges
+    g = golden["star_getBoxFast"]
+    d = g["I1_d"].reshape(-1)
+    I1 = nnv.Star(g["I1_V"], g["I1_C"], d)
+    lo, hi = I1.getRanges()
+    np.testing.assert_allclose(lo, g["B1_lb"].reshape(-1), rtol=0, atol=1e-8)
+    np.testing.assert_allclose(hi, g["B1_ub"].reshape(-1), rtol=0, atol=1e-8)
+    n = g["I1_C"].shape[1]
+    plb = np.array([oracle.lpsolver(np.eye(n)[j], g["I1_C"], d, None, None) for j in range(n)])
+    pub = np.array([-oracle.lpsolver(-np.eye(n)[j], g["I1_C"], d, None, None) for j in range(n)])
+    lb, ub = nnv.Star(g["I1_V"], g["I1_C"], d, plb, pub).estimateRanges()
+    np.testing.assert_allclose(lb, g["B2_lb"].reshape(-1), rtol=0, atol=1e-8)
+    np.testing.assert_allclose(ub, g["B2_ub"].reshape(-1), rtol=0, atol=1e-8)
+
+
+def test_relu_layer_on_an_image_star_with_relax_factor(nnv, oracle):
+    # ReluLayer.reach of an ImageStar goes toStar -> PosLin.reach -> toImageStar (nn/layers/ReluLayer.m:72-150),
+    # also below relaxFactor 1
+    rs = np.random.RandomState(6)
+    lb = rs.rand(5, 4, 2) - 0.7
+    ub = lb + 0.3 * rs.rand(5, 4, 2)
+    Wt, b = rs.randn(3, 3, 2, 3) * 0.5, rs.randn(3) * 0.1
+    conv = nnv.Conv2DLayer(Wt, b, [1, 1, 1, 1], [1, 1], [1, 1])
+    D = nnv.ReluLayer().reach(conv.reach(nnv.ImageStar(lb, ub), "approx-star"), "relax-star-area", [], 1)
+    W2, b2 = rs.randn(3, 3, 3, 2) * 0.5, rs.randn(2) * 0.1       # a second convolution: genuine constraints
+    D = nnv.Conv2DLayer(W2, b2, [1, 1, 1, 1], [1, 1], [1, 1]).reach(D, "approx-star")
+    O = oracle.relu_reach(oracle.conv2d_reach(oracle.image_star_from_bounds(lb, ub), Wt, b, [1, 1, 1, 1], [1, 1], [1, 1]),
+                          "relax-star-area", 1.0)
+    O = oracle.conv2d_reach(O, W2, b2, [1, 1, 1, 1], [1, 1], [1, 1])
+    for method, rf in (("relax-star-range", 0.0), ("relax-star-area", 0.5)):
+        R = nnv.ReluLayer().reach(D, method, [], rf)
+        E = oracle.relu_reach(O, method, rf)
+        assert isinstance(R, nnv.ImageStar) and (R.height, R.width, R.numChannel) == (E.height, E.width, E.numChannel)
+        assert R.numPred == E.numPred
+        assert_close(R.V.reshape(-1, R.numPred + 1, order="F"), E.V.reshape(-1, E.numPred + 1, order="F"), "V", 1e-7)
+        assert_close(R.C, E.C, "C", 1e-7)
+        assert_close(R.pred_ub, E.pred_ub, "pred_ub", 1e-7)

@@ -171,3 +171,21 @@ def test_lp_step_tightens_and_stays_sound(method):
 def test_round_is_matlabs():
     # n1 = round((1-rf)*numel(map2)): halves go up (numpy's round would send 2.5 to 2)
     assert o._round_half_away(2.5) == 3 and o._round_half_away(3.5) == 4 and o._round_half_away(2.4999) == 2
+
+
+def test_lp_box_and_interval_box_known_answers(golden):
+    # Star.getBox (one LP pair per state, set/Star.m:597-650) and Star.getBoxFast (interval arithmetic over
+    # the bounding box of the predicate polytope, :658-677) of the reference's stored star I1
+    g = golden["star_getBoxFast"]
+    I1 = o.OStar(g["I1_V"], g["I1_C"], g["I1_d"])
+    idx = np.arange(I1.dim)
+    np.testing.assert_allclose(o.get_mins(I1, idx), g["B1_lb"].reshape(-1), rtol=0, atol=1e-8)
+    np.testing.assert_allclose(o.get_maxs(I1, idx), g["B1_ub"].reshape(-1), rtol=0, atol=1e-8)
+    # predicate bounding box by LP (what getPredicateBounds asks the polytope library for), then the same
+    # interval formula estimateRanges uses
+    n = I1.nVar
+    plb = np.array([o.lpsolver(np.eye(n)[j], I1.C, I1.d, None, None) for j in range(n)])
+    pub = np.array([-o.lpsolver(-np.eye(n)[j], I1.C, I1.d, None, None) for j in range(n)])
+    lb, ub = o.estimate_ranges(o.OStar(I1.V, I1.C, I1.d, plb, pub))
+    np.testing.assert_allclose(lb, g["B2_lb"].reshape(-1), rtol=0, atol=1e-8)
+    np.testing.assert_allclose(ub, g["B2_ub"].reshape(-1), rtol=0, atol=1e-8)
