@@ -17,6 +17,9 @@ Sources (data only; no reference code is imported or executed):
   * results/tests/baselines/set/test_star_getBoxFast_results.mat
       written by code/nnv/tests/set/star/test_star_getBoxFast.m:10-63: a star over a random polytope,
       its LP box (Star.getBox, B1) and its interval box over the predicates' bounding box (getBoxFast, B2)
+  * results/tests/baselines/set/test_star_isEmptySet_results.mat
+      written by code/nnv/tests/set/star/test_star_isEmptySet.m:8-37: a feasible star over a random
+      polytope (ten constraint rows) and the verdict Star.isEmptySet gave for it
   * the literal inputs/expected outputs typed in
       code/nnv/tests/nn/layers/Conv2DLayer/test_layers_Conv2D.m:14-28  (conv known answer)
       code/nnv/tests/set/image_star/test_ImageStar_getRange.m:45-62    (ranges known answer)
@@ -52,6 +55,8 @@ def main():
     out["star_intersect_halfSpace"] = {k: arr(m[k]) for k in ("H", "g", "S_V", "S1_V", "S1_C", "S1_d", "S1_lb", "S1_ub")}
     m = sio.loadmat(os.path.join(base, "set/test_star_getBoxFast_results.mat"))
     out["star_getBoxFast"] = {k: arr(m[k]) for k in ("I1_V", "I1_C", "I1_d", "B1_lb", "B1_ub", "B2_lb", "B2_ub")}
+    m = sio.loadmat(os.path.join(base, "set/test_star_isEmptySet_results.mat"))
+    out["star_isEmptySet"] = {k: arr(m[k]) for k in ("S_V", "S_C", "S_d", "S1_V", "S1_C", "S1_d", "b_nonempty", "b_empty")}
     m = sio.loadmat(os.path.join(base, "set/star_test_results.mat"))
     out["star_test"] = {k: arr(m[k]) for k in ("S1_V", "S2_V", "S3_V", "B2_lb", "B2_ub")}
     # literal input / expected output of ReluLayer.evaluate typed in test_layers_relu.m:19-33

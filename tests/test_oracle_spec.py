@@ -39,6 +39,16 @@ def test_is_empty_set_known_answers():
     assert o.is_empty_set(S3) is True
 
 
+def test_is_empty_set_stored_verdicts(golden):
+    # the two stars of tests/set/star/test_star_isEmptySet.m with the verdicts the reference stored for them
+    g = golden["star_isEmptySet"]
+    S = o.OStar(g["S_V"], g["S_C"], g["S_d"])
+    S1 = o.OStar(g["S1_V"], g["S1_C"], g["S1_d"])
+    assert o.is_empty_set(S) is bool(g["b_nonempty"].reshape(-1)[0])
+    assert o.is_empty_set(S1) is bool(g["b_empty"].reshape(-1)[0])
+    assert bool(g["b_empty"].reshape(-1)[0]) and not bool(g["b_nonempty"].reshape(-1)[0])
+
+
 def test_intersect_half_space_rows_and_known_answer():
     # tests/soundness/test_set_conversion.m:60-68: box [-1,1]^2 meets x1 <= 0.5
     S = o.star_from_box([-1.0, -1.0], [1.0, 1.0])
