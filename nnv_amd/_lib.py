@@ -141,6 +141,7 @@ class Context:
         self.handle = h
         self.lib = lib
         self.device = device
+        self.release_set = lib.nnvhip_star_release   # looked up once: every set handle calls it when it dies
 
     def synchronize(self):
         check(self.lib.nnvhip_synchronize(self.handle))

@@ -32,20 +32,20 @@ def _as_list(sets):
 
 
 def _handles_array(sets):
-    arr = (C.c_void_p * len(sets))()
-    for i, s in enumerate(sets):
-        arr[i] = s._h.h
-    return arr
+    return (C.c_void_p * len(sets))(*[s._h.h for s in sets])
 
 
 def _wrap_like(inputs, ctx, raw, shape_fn=None):
+    mk, H = Star._from_handle, _Handle
+    if type(inputs[0]) is Star and all(type(s) is Star for s in inputs):
+        return [mk(H(h, ctx)) for h in raw]          # the common case, kept cheap: arrays of 1000s of sets
     outs = []
     for s, h in zip(inputs, raw):
-        hd = _Handle(h, ctx)
+        hd = H(h, ctx)
         if isinstance(s, ImageStar):
             outs.append(ImageStar(_handle=hd, shape=shape_fn(s)))
         else:
-            outs.append(Star(_handle=hd))
+            outs.append(mk(hd))
     return outs
 
 
@@ -300,7 +300,7 @@ class PosLin:
                 out = (C.c_void_p * len(sets))()
                 check(ctx.lib.nnvhip_relu_relax(ctx.handle, RELAX_ORDER[method], float(relaxFactor), len(sets),
                                                 _handles_array(sets), out))
-                res = [Star(_handle=_Handle(h, ctx)) for h in out]
+                res = [Star._from_handle(_Handle(h, ctx)) for h in out]
             else:
                 # some bounds are tightened by LPs first: host LP solver fed from the resident set
                 res = [PosLin.reach_relaxed_star_lp(s, method, relaxFactor, option, dis_opt, lp_solver) for s in sets]

@@ -28,7 +28,7 @@ class _Handle:
     def __del__(self):
         try:
             if self.h:
-                self.ctx.lib.nnvhip_star_release(self.h)
+                self.ctx.release_set(self.h)
                 self.h = None
         except Exception:
             pass
@@ -161,10 +161,21 @@ class Star:
     approx-zono method reads it).
     """
 
+    # defaults of the fields a constructor may leave alone (instances made by _from_handle set only _h)
+    state_lb = None
+    state_ub = None
+    Z = None
+    _lp = None
+    _unbounded_predicates = False
+
+    @classmethod
+    def _from_handle(cls, handle):
+        """A Star around an existing device handle (the layers wrap whole arrays of outputs this way)."""
+        s = cls.__new__(cls)
+        s._h = handle
+        return s
+
     def __init__(self, *args, ctx=None, _handle=None):
-        self.state_lb = None
-        self.state_ub = None
-        self.Z = None
         if _handle is not None:
             self._h = _handle
             return
@@ -296,10 +307,10 @@ class Star:
     # ---- LP-based ranges (host LP fed from the resident set) -------------------------------
     def _lp_problem(self):
         """(C as a sparse matrix, d, predicate bounds) of this set, fetched once."""
-        if getattr(self, "_lp", None) is None:
+        if self._lp is None:
             from scipy import sparse
             Cm, d = self._h.fetch_constraints()
-            if getattr(self, "_unbounded_predicates", False):     # Star(V, C, d): predicate_lb/ub are []
+            if self._unbounded_predicates:                        # Star(V, C, d): predicate_lb/ub are []
                 bounds = np.column_stack([np.full(self.nVar, -np.inf), np.full(self.nVar, np.inf)])
             else:
                 bounds = np.column_stack(self._h.fetch_pred())
