@@ -289,7 +289,7 @@ def main():
         else:
             ora_in = o.star_from_box(cfg["lb"], cfg["ub"])
         n_cpu, t_cpu = 0, 0.0
-        while t_cpu < args.cpu_seconds and n_cpu < 50:
+        while t_cpu < args.cpu_seconds and n_cpu < 200:
             t1 = time.perf_counter()
             o.nn_reach(cfg["layers"], ora_in, args.method, 1.0)
             t_cpu += time.perf_counter() - t1
