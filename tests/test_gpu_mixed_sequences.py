@@ -124,3 +124,22 @@ def test_random_cnn_sequences(nnv, oracle, seed):
     dev_in = nnv.ImageStar(x - eps, x + eps)
     ora_in = oracle.image_star_from_bounds(x - eps, x + eps)
     _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area")
+
+
+@pytest.mark.parametrize("wide,count,method", [(9000, 1, "relax-star-range"), (8200, 2, "relax-star-static")])
+def test_wide_layers_in_a_sequence(nnv, oracle, wide, count, method):
+    # more than 8192 neurons: classification, sort and bounds run as separate multi-block kernels, and
+    # the sets that come out of them feed batch normalisation, another ReLU and an FC layer
+    rs = np.random.RandomState(wide)
+    n_in = 10
+    layers = [_fc(rs, wide, n_in, 3.0), {"type": "relu"}, _bn(rs, wide), {"type": "relu"}, _fc(rs, 300, wide, 2.0),
+              {"type": "relu"}, _fc(rs, 5, 300)]
+    centre = rs.rand(n_in, count)
+    half = np.abs(rs.randn(n_in, count)) * 0.05
+    lbs, ubs = centre - half, centre + half
+    if count == 1:
+        dev_in, ora_in = nnv.Star(lbs[:, 0], ubs[:, 0]), oracle.star_from_box(lbs[:, 0], ubs[:, 0])
+    else:
+        dev_in = nnv.Star.from_boxes(lbs, ubs)
+        ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
+    _compare(nnv, oracle, layers, dev_in, ora_in, method)
