@@ -273,6 +273,7 @@ def main():
                 "what": "LP-free pass of verify_specification for robustness_set(target=0): G*[c V], row bounds, verdicts"}
 
     # practical HBM ceiling on this box: a plain copy kernel over 1 GiB (read + write bytes)
+    roofline["measured_mfma_TFLOPs"] = round(ctx.probe_mfma_peak(3), 2)     # register-resident MFMA loop
     roofline["measured_copy_GBps"] = round(ctx.probe_copy_bandwidth(1 << 30, 5), 1)
     ctx.trim_pool()
 

@@ -102,6 +102,10 @@ NNVHIP_API int nnvhip_kernel_time(nnvhip_ctx* ctx, int which, double* total_ms, 
  * the practical HBM ceiling on this box, and the known-size kernel hardware counters are
  * calibrated against. */
 NNVHIP_API int nnvhip_probe_copy_bandwidth(nnvhip_ctx* ctx, int64_t bytes, int reps, double* gbytes_per_s);
+/* Measurement hook (no counterpart in the reference): a register-resident loop of fp64 16x16x4 MFMAs on
+ * every CU (no memory traffic); returns the rate of the timed reps in TFLOP/s - the practical ceiling
+ * of the matrix pipes on this box. */
+NNVHIP_API int nnvhip_probe_mfma_peak(nnvhip_ctx* ctx, int reps, double* tflops);
 /* Returns every cached device block of the pool to the driver (hipFree). */
 NNVHIP_API int nnvhip_trim_pool(nnvhip_ctx* ctx);
 /* Bytes currently handed out by / cached in the pool. */

@@ -26,7 +26,7 @@ SYMBOLS = [
     "nnvhip_relu_relax", "nnvhip_halfspace_check", "nnvhip_halfspace_rows", "nnvhip_rowmap_create",
     "nnvhip_rowmap_destroy", "nnvhip_affine_rowmap", "nnvhip_avgpool2d_create", "nnvhip_avgpool2d_destroy",
     "nnvhip_avgpool2d_output_size", "nnvhip_affine_avgpool2d", "nnvhip_permute_rows",
-    "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists",
+    "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists", "nnvhip_probe_mfma_peak",
 ]
 
 
@@ -86,6 +86,7 @@ def load():
         "nnvhip_affine_conv2d": [p, p, i64, i64, i64, pp, pp],
         "nnvhip_relu_relax": [p, C.c_int, dbl, i64, pp, pp],
         "nnvhip_relu_apply_lists": [p, p, i64, p, i64, p, p, p, pp],
+        "nnvhip_probe_mfma_peak": [p, C.c_int, C.POINTER(dbl)],
         "nnvhip_halfspace_check": [p, i64, pp, i64, p, p, p, i64, p, p, p],
         "nnvhip_halfspace_rows": [p, p, i64, p, p, i64, p, p],
         "nnvhip_rowmap_create": [p, i64, C.c_int32, p, p, p, pp],
@@ -167,6 +168,12 @@ class Context:
         ms, n, fl = C.c_double(), C.c_int64(), C.c_double()
         check(self.lib.nnvhip_kernel_time(self.handle, int(which), C.byref(ms), C.byref(n), C.byref(fl), 1 if reset else 0))
         return ms.value, n.value, fl.value
+
+    def probe_mfma_peak(self, reps=3) -> float:
+        """TFLOP/s of a register-resident fp64 MFMA loop on every CU (practical matrix-pipe ceiling)."""
+        t = C.c_double()
+        check(self.lib.nnvhip_probe_mfma_peak(self.handle, int(reps), C.byref(t)))
+        return t.value
 
     def probe_copy_bandwidth(self, nbytes=1 << 30, reps=5) -> float:
         """Achieved read+write GB/s of a plain copy kernel over nbytes (practical HBM ceiling)."""

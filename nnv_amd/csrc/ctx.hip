@@ -4,6 +4,7 @@
 #include <cstring>
 
 #include "internal.h"
+#include "mfma_tile.h"
 
 namespace nnvhip {
 
@@ -262,6 +263,43 @@ int nnvhip_probe_copy_bandwidth(nnvhip_ctx* c, int64_t bytes, int reps, double* 
   float ms = 0.f;
   NNV_HIP_TRY(hipEventElapsedTime(&ms, c->kev0, c->kev1));
   *gbytes_per_s = 2.0 * (double)bytes * reps / (ms * 1e-3) / 1e9;  // bytes read + bytes written
+  return NNVHIP_OK;
+}
+
+// Register-resident fp64 MFMA loop: 8 independent accumulators per wave, 8 waves per block, no memory
+// traffic.  What the matrix pipes deliver on this box when nothing else stands in their way.
+__global__ __launch_bounds__(512) void probe_mfma_kernel(double* __restrict__ out, int iters) {
+  double4_t acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = double4_t{0.0, 0.0, 0.0, 0.0};
+  const double a = threadIdx.x * 1e-3, b = threadIdx.x * 2e-3;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, acc[i], 0, 0, 0);
+  }
+  double s = 0.0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  out[blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+int nnvhip_probe_mfma_peak(nnvhip_ctx* c, int reps, double* tflops) {
+  CHECK_CTX(c);
+  if (reps < 1 || !tflops) NNV_FAIL(NNVHIP_ERR_ARG, "invalid argument");
+  const int blocks = 2048, iters = 2000;
+  BufRef out;
+  NNV_TRY(c->alloc(sizeof(double) * 512 * blocks, &out));
+  hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(512), 0, c->stream, out->as<double>(), iters);
+  NNV_HIP_TRY(hipEventRecord(c->kev0, c->stream));
+  for (int i = 0; i < reps; ++i)
+    hipLaunchKernelGGL(probe_mfma_kernel, dim3(blocks), dim3(512), 0, c->stream, out->as<double>(), iters);
+  NNV_HIP_TRY(hipEventRecord(c->kev1, c->stream));
+  NNV_HIP_TRY(hipEventSynchronize(c->kev1));
+  NNV_HIP_TRY(hipGetLastError());
+  float ms = 0.f;
+  NNV_HIP_TRY(hipEventElapsedTime(&ms, c->kev0, c->kev1));
+  // one 16x16x4 MFMA = 2*16*16*4 flop; 8 per iteration and wave, 8 waves per block
+  *tflops = 2048.0 * 8.0 * iters * 8.0 * blocks * reps / (ms * 1e-3) / 1e12;
   return NNVHIP_OK;
 }
 
