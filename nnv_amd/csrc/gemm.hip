@@ -77,6 +77,15 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
   // Bk: the listed rows of B already packed into a matrix of their own (row t of Bk = row kmap[t] of B);
   // only A is gathered then
   const bool b_packed = MAPPED && Bk != nullptr;
+  // The row list of this tile is copied into LDS first: the staging loads then take their row numbers
+  // from there instead of through a dependent global load ahead of every operand load.
+  constexpr int kMapLds = 2048;
+  __shared__ int kmap_s[MAPPED ? kMapLds : 1];
+  const bool map_lds = MAPPED && kmap != nullptr && Kp <= kMapLds;  // uniform over the block
+  if (map_lds) {
+    for (int k = tid; k < Kp; k += NT) kmap_s[k] = kmap[k];
+    __syncthreads();
+  }
 
   // ---- global -> register staging ----------------------------------------------------------
   constexpr int A_VEC = TM * KT / 2;           // double2 elements in a W tile
@@ -102,7 +111,7 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
       int row = m0 + 2 * i2;
       double2 v = make_double2(0.0, 0.0);
       if (idx < A_VEC && row < Mp) {
-        const int kk = (MAPPED && kmap != nullptr) ? kmap[k0 + k] : k0 + k;
+        const int kk = (MAPPED && kmap != nullptr) ? (map_lds ? kmap_s[k0 + k] : kmap[k0 + k]) : k0 + k;
         if (kk >= 0) v = *reinterpret_cast<const double2*>(A + row + (int64_t)kk * lda);
       }
       ra[p] = v;
@@ -117,7 +126,8 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
         if (b_packed) {
           v = *reinterpret_cast<const double2*>(Bk + (k0 + 2 * k2) + (bk_col0 + j) * ldbk);
         } else if (MAPPED && kmap != nullptr) {
-          const int ka = kmap[k0 + 2 * k2], kb = kmap[k0 + 2 * k2 + 1];
+          const int ka = map_lds ? kmap_s[k0 + 2 * k2] : kmap[k0 + 2 * k2];
+          const int kb = map_lds ? kmap_s[k0 + 2 * k2 + 1] : kmap[k0 + 2 * k2 + 1];
           if (ka >= 0) v.x = B[ka + bcol[p] * ldb];
           if (kb >= 0) v.y = B[kb + bcol[p] * ldb];
         } else {
