@@ -50,8 +50,9 @@ def layer_shapes(reach_set):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default: as many as fill about 0.3 s, between 10 and 1000)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: steps / 10, at least 5)")
     ap.add_argument("--config", type=int, default=2)
     ap.add_argument("--method", default="relax-star-area")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -82,6 +83,19 @@ def main():
         nnv_amd._lib.check(lib.nnvhip_estimate_ranges_batch(h, len(outs), arr, None, None))
         return out
 
+    if args.steps is None:
+        # a reach takes between 0.1 ms and 0.2 s depending on the workload: size the timed region so that
+        # clocks have settled and the timer's granularity does not matter
+        for _ in range(3):
+            step()
+        ctx.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            step()
+        ctx.synchronize()
+        args.steps = int(min(1000, max(10, 0.3 / max((time.perf_counter() - t0) / 3, 1e-6))))
+    if args.warmup is None:
+        args.warmup = max(5, args.steps // 10)
     for _ in range(args.warmup):
         step()
     ctx.synchronize()
