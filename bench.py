@@ -268,6 +268,18 @@ def main():
         roofline["relu_step_algo_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
         roofline["relu_step_frac_of_hbm_peak"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
 
+    # ---- the same step with the host buffers the boundary takes and returns (not `value`) -----------
+    # lb / ub uploaded and the input set built on the device, the reach, the output bounds back on the host
+    n_h2h = max(5, min(args.steps, 50))
+    ctx.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(n_h2h):
+        fresh = device_input_sets(cfg, ctx)
+        res = net.reach(fresh, opts)
+        nnv_amd.Star.estimateRanges_array(res if isinstance(res, list) else [res])
+    host_to_host_ms = 1e3 * (time.perf_counter() - t1) / n_h2h
+    del fresh, res
+
     # ---- specification check on the resident output sets (not part of `value`) -----------------
     spec = None
     last = net.Layers[-1]
@@ -324,7 +336,10 @@ def main():
                    "sets": len(dev_in) if isinstance(dev_in, list) else 1,
                    "updates_per_step": updates,
                    "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, list) else None},
-        "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec, "layers": layer_report,
+        "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec,
+        "host_to_host": {"ms_per_step": round(host_to_host_ms, 4), "steps": n_h2h,
+                         "what": "input bounds uploaded and the set(s) built, reach, output bounds fetched to the host"},
+        "layers": layer_report,
     }))
 
 

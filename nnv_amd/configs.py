@@ -153,9 +153,7 @@ def device_input_sets(cfg, ctx=None):
     config Box.partition (set/Box.m:96-139) followed by one Star per sub-box."""
     from .sets import Box, ImageStar, Star
     if "partition" in cfg:
-        boxes = Box(cfg["lb"], cfg["ub"]).partition(cfg["partition"]["indexes"], cfg["partition"]["numbers"])
-        lbs = np.stack([b.lb for b in boxes], axis=1)
-        ubs = np.stack([b.ub for b in boxes], axis=1)
+        lbs, ubs = Box(cfg["lb"], cfg["ub"]).partition_bounds(cfg["partition"]["indexes"], cfg["partition"]["numbers"])
         return Star.from_boxes(lbs, ubs, ctx=ctx)
     if cfg["kind"] == "image":
         sh = cfg["image_shape"]

@@ -106,11 +106,22 @@ class Box:
         self.ub = ub
         self.dim = lb.size
         self.center = 0.5 * (lb + ub)            # Box.m:35
-        vec = 0.5 * (ub - lb)                    # Box.m:36
-        gens = np.diag(vec)
-        if gens.size > 1:
-            gens = gens[:, ~np.all(gens == 0, axis=0)]   # Box.m:41-43
-        self.generators = gens
+        self._generators = None
+
+    @property
+    def generators(self):
+        """dim x (number of non-degenerate dimensions), built on first use: Star(lb, ub) makes the same
+        matrix on the device and a partition makes thousands of boxes that never show theirs."""
+        if self._generators is None:
+            vec = 0.5 * (self.ub - self.lb)      # Box.m:36
+            if vec.size > 1:
+                keep = np.flatnonzero(vec != 0)  # Box.m:41-43: all-zero columns of diag(vec) are dropped
+                gens = np.zeros((vec.size, keep.size))
+                gens[keep, np.arange(keep.size)] = vec[keep]
+            else:
+                gens = np.diag(vec)
+            self._generators = gens
+        return self._generators
 
     def singlePartition(self, part_id, part_num):
         """Box.m:61-91; part_id is 0-based."""
@@ -148,6 +159,33 @@ class Box:
                 nxt.extend(b.singlePartition(ix, num))
             boxes = nxt
         return boxes
+
+    def partition_bounds(self, part_indexes, part_numbers):
+        """The boxes of partition() as two dim x count matrices (column j = box j), without building
+        the Box objects: same arithmetic, statement by statement (Box.m:79-88, 126-137)."""
+        part_indexes = list(part_indexes)
+        part_numbers = list(part_numbers)
+        if len(part_indexes) != len(part_numbers):
+            raise ValueError("Inconsistent between part_indexes and part_number array, should have the same number of elements")
+        for i, (ix, num) in enumerate(zip(part_indexes, part_numbers)):
+            if ix < 0 or ix >= self.dim:
+                raise ValueError("The %d^th index in part_indexes array is invalid" % (i + 1))
+            if num < 1:
+                raise ValueError("The %d^th number in part_numbers array is invalid" % (i + 1))
+        lbs = self.lb.reshape(-1, 1).copy()
+        ubs = self.ub.reshape(-1, 1).copy()
+        for ix, num in zip(part_indexes, part_numbers):
+            if num == 1:
+                continue
+            delta = (ubs[ix, :] - lbs[ix, :]) / num                        # one delta per current box
+            i = np.arange(1, num + 1, dtype=np.float64)
+            new_lb = lbs[ix, :, None] + (i[None, :] - 1) * delta[:, None]  # box-major, part-minor
+            new_ub = new_lb + delta[:, None]
+            lbs = np.repeat(lbs, num, axis=1)
+            ubs = np.repeat(ubs, num, axis=1)
+            lbs[ix, :] = new_lb.reshape(-1)
+            ubs[ix, :] = new_ub.reshape(-1)
+        return lbs, ubs
 
     def toStar(self, ctx=None):
         return Star(self.lb, self.ub, ctx=ctx)
@@ -393,6 +431,20 @@ class Star:
         """For a set returned by the ReLU step: (n_inactive, crossing index (0-based, new-predicate
         order), lb(crossing), ub(crossing))."""
         return self._h.relu_info()
+
+    @staticmethod
+    def estimateRanges_array(sets):
+        """estimateRanges of every set of an array in one device call -> (lb, ub), dim x count each."""
+        sets = list(sets)
+        if not sets:
+            return np.empty((0, 0)), np.empty((0, 0))
+        ctx = sets[0].ctx
+        N = sets[0].dim
+        lb = np.empty((N, len(sets)), order="F")
+        ub = np.empty((N, len(sets)), order="F")
+        arr = (C.c_void_p * len(sets))(*[s._h.h for s in sets])
+        check(ctx.lib.nnvhip_estimate_ranges_batch(ctx.handle, len(sets), arr, ptr(lb), ptr(ub)))
+        return lb, ub
 
 
 class ImageStar:

@@ -119,3 +119,20 @@ def test_relax_factor_bookkeeping_hands_the_device_the_oracles_lists(monkeypatch
     assert np.all(seen["lb"] < 0) and np.all(seen["ub"] > 0)          # what the device step insists on
     assert len(set(seen["index"]) & set(seen["reset"])) == 0
     assert len(set(seen["index"])) == seen["index"].size
+
+
+def test_partition_bounds_is_the_partition():
+    rs = np.random.RandomState(2)
+    lb = rs.rand(9) - 0.5
+    ub = lb + rs.rand(9) * 0.3 + 0.01
+    b = Box(lb, ub)
+    for idx, nums in (([0, 3, 7], [2, 3, 2]), ([4], [5]), ([1, 2], [1, 4]), ([8, 0], [3, 3])):
+        boxes = b.partition(idx, nums)
+        lbs, ubs = b.partition_bounds(idx, nums)
+        assert lbs.shape == (9, len(boxes))
+        assert np.array_equal(lbs, np.stack([x.lb for x in boxes], axis=1))
+        assert np.array_equal(ubs, np.stack([x.ub for x in boxes], axis=1))
+        ref = o.box_partition(lb, ub, idx, nums)
+        assert np.array_equal(lbs, np.stack([r[0] for r in ref], axis=1))
+    with pytest.raises(ValueError, match="index in part_indexes"):
+        b.partition_bounds([9], [2])
