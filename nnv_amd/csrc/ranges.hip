@@ -125,12 +125,29 @@ __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __re
   __shared__ double sums[4][64];
   double s = 0.0;
   if (r < d.ld) {
+    // the partial sums were written by other CUs moments ago: every load is a trip to memory, so as many
+    // as possible are in flight at once; the additions stay in chunk order
     const double* p = d.part + (int64_t)q * d.ld + r;
-#pragma unroll 8
-    for (int c = 0; c < d.chunks; ++c) s += p[(int64_t)c * 4 * d.ld];
+    int c = 0;
+    for (; c + 32 <= d.chunks; c += 32) {
+      double v[32];
+#pragma unroll
+      for (int u = 0; u < 32; ++u) v[u] = p[(int64_t)(c + u) * 4 * d.ld];
+#pragma unroll
+      for (int u = 0; u < 32; ++u) s += v[u];
+    }
+    {
+      double v[32];
+#pragma unroll
+      for (int u = 0; u < 32; ++u) v[u] = c + u < d.chunks ? p[(int64_t)(c + u) * 4 * d.ld] : 0.0;
+#pragma unroll
+      for (int u = 0; u < 32; ++u)
+        if (c + u < d.chunks) s += v[u];
+    }
     if (d.chunks2 > 0) {
       const double* p2 = d.part2 + (int64_t)q * d.ld + r;
-      for (int c = 0; c < d.chunks2; ++c) s += p2[(int64_t)c * 4 * d.ld];
+#pragma unroll 8
+      for (int c2 = 0; c2 < d.chunks2; ++c2) s += p2[(int64_t)c2 * 4 * d.ld];
     }
   }
   sums[q][lane] = s;

@@ -439,7 +439,7 @@ class Star:
         if not sets:
             return np.empty((0, 0)), np.empty((0, 0))
         ctx = sets[0].ctx
-        N = sets[0].dim
+        N = sets[0]._h.dims()[0]          # Star or ImageStar: the flattened dimension
         lb = np.empty((N, len(sets)), order="F")
         ub = np.empty((N, len(sets)), order="F")
         arr = (C.c_void_p * len(sets))(*[s._h.h for s in sets])

@@ -463,3 +463,24 @@ def test_fc_after_a_relu_that_kept_no_row(nnv, oracle):
         assert R2.nVar == E2.nVar
         assert_close(R2.V, E2.V, "second relu %d" % i)
     assert kept[0] == 0 and kept[2] == 0 and kept[1] > 0
+
+
+def test_ranges_of_an_array_in_one_call(nnv, oracle):
+    rs = np.random.RandomState(3)
+    lbs = rs.rand(30, 4) - 0.5
+    ubs = lbs + rs.rand(30, 4) * 0.2
+    W, b = rs.randn(17, 30), rs.randn(17)
+    outs = nnv.FullyConnectedLayer(W, b).reach(nnv.Star.from_boxes(lbs, ubs), "approx-star")
+    lb, ub = nnv.Star.estimateRanges_array(outs)
+    assert lb.shape == (17, 4)
+    for i, R in enumerate(outs):
+        l, u = R.estimateRanges()
+        assert np.array_equal(lb[:, i], l) and np.array_equal(ub[:, i], u)
+        el, eu = oracle.estimate_ranges(oracle.affine_map(oracle.star_from_box(lbs[:, i], ubs[:, i]), W, b))
+        assert_close(lb[:, i], el, "lb")
+        assert_close(ub[:, i], eu, "ub")
+    im = nnv.ImageStar(lbs[:, 0].reshape(5, 3, 2, order="F"), ubs[:, 0].reshape(5, 3, 2, order="F"))
+    lb, ub = nnv.Star.estimateRanges_array([im])
+    assert_close(lb[:, 0], lbs[:, 0], "image lb")          # centre -/+ half-width: equal up to rounding
+    assert_close(ub[:, 0], ubs[:, 0], "image ub")
+    assert nnv.Star.estimateRanges_array([])[0].size == 0
