@@ -41,6 +41,18 @@ classdef ImageStar < ImageStar
             end
             lb = obj.im_lb; ub = obj.im_ub;
         end
+        function S = changeVarsPrecision(obj, precision)   % Star.m:1539-1560, ImageStar.m:673-695: the device store is fp64 only
+            if ~strcmp(precision, 'double')
+                error('this library keeps sets in double precision only');
+            end
+            S = obj;
+        end
+        function S = changeDevice(obj, deviceTarget)        % Star.m:1563-1585, ImageStar.m:697-720: the data is in HBM either way
+            if ~any(strcmp(deviceTarget, {'cpu', 'gpu'}))
+                error("Device target must be 'cpu' or 'gpu'.");
+            end
+            S = obj;
+        end
         function IS = gather(obj)
             V = nnvhip_mex('fetch_V', obj.dev.h);
             [C, d] = nnvhip_mex('fetch_constraints', obj.dev.h);

@@ -44,6 +44,18 @@ classdef Star < Star
             end
             IS = nnvhip.ImageStar(obj.dev, h, w, c);
         end
+        function S = changeVarsPrecision(obj, precision)   % Star.m:1539-1560: the device store is fp64 only
+            if ~strcmp(precision, 'double')
+                error('this library keeps sets in double precision only');
+            end
+            S = obj;
+        end
+        function S = changeDevice(obj, deviceTarget)        % Star.m:1563-1585: the data is in HBM either way
+            if ~any(strcmp(deviceTarget, {'cpu', 'gpu'}))
+                error("Device target must be 'cpu' or 'gpu'.");
+            end
+            S = obj;
+        end
         function S = gather(obj)
             % plain NNV Star with dense host arrays, C/d in NNV's [C0;C1;C2;C3] layout
             V = nnvhip_mex('fetch_V', obj.dev.h);

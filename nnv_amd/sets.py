@@ -90,6 +90,23 @@ def _make_handles(ctx, raw):
     return [_Handle(C.c_void_p(h), ctx) for h in raw]
 
 
+def _change_precision(obj, precision):
+    """changeVarsPrecision (set/Star.m:1539-1560, set/ImageStar.m): the device store is fp64 only."""
+    if precision == "double":
+        return obj
+    if precision == "single":
+        raise ValueError("this library keeps sets in double precision only")
+    raise ValueError("Only single or double precision arrays allowed. GpuArray/dlarray are coming.")
+
+
+def _change_device(obj, deviceTarget):
+    """changeDevice (set/Star.m:1563-1585): the set lives in HBM either way; property reads hand out
+    host arrays, so both targets return the set itself."""
+    if deviceTarget in ("cpu", "gpu"):
+        return obj
+    raise ValueError("Device target must be 'cpu' or 'gpu'.")
+
+
 class Box:
     """set/Box.m: hyper-rectangle with centre/generator form and uniform partitioning."""
 
@@ -432,6 +449,12 @@ class Star:
         order), lb(crossing), ub(crossing))."""
         return self._h.relu_info()
 
+    def changeVarsPrecision(self, precision):
+        return _change_precision(self, precision)
+
+    def changeDevice(self, deviceTarget):
+        return _change_device(self, deviceTarget)
+
     @staticmethod
     def estimateRanges_array(sets):
         """estimateRanges of every set of an array in one device call -> (lb, ub), dim x count each."""
@@ -556,6 +579,12 @@ class ImageStar:
             self.im_lb = lb.reshape(shp, order="F")
             self.im_ub = ub.reshape(shp, order="F")
         return self.im_lb, self.im_ub
+
+    def changeVarsPrecision(self, precision):
+        return _change_precision(self, precision)
+
+    def changeDevice(self, deviceTarget):
+        return _change_device(self, deviceTarget)
 
     def relu_info(self):
         return self._h.relu_info()

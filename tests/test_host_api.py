@@ -136,3 +136,16 @@ def test_partition_bounds_is_the_partition():
         assert np.array_equal(lbs, np.stack([r[0] for r in ref], axis=1))
     with pytest.raises(ValueError, match="index in part_indexes"):
         b.partition_bounds([9], [2])
+
+
+def test_precision_and_device_switches_of_a_set():
+    from nnv_amd.sets import _change_device, _change_precision
+    marker = object()
+    assert _change_precision(marker, "double") is marker
+    with pytest.raises(ValueError, match="double precision only"):
+        _change_precision(marker, "single")
+    with pytest.raises(ValueError, match="Only single or double"):
+        _change_precision(marker, "half")
+    assert _change_device(marker, "cpu") is marker and _change_device(marker, "gpu") is marker
+    with pytest.raises(ValueError, match="'cpu' or 'gpu'"):
+        _change_device(marker, "tpu")
