@@ -394,7 +394,7 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int6
   const StampSet* table = nullptr;
   BufRef tab;
   if (count > 1) {
-    NNV_TRY(ctx->upload(sets, sizeof(StampSet) * count, &tab));
+    NNV_TRY(ctx->upload_table(sets, sizeof(StampSet) * count, &tab));
     table = tab->as<StampSet>();
   }
   StampSet one;

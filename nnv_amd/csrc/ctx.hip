@@ -91,7 +91,9 @@ int nnvhip_ctx::stage(size_t bytes, void** host) {
   bytes = (bytes + 255) & ~size_t(255);
   if (bytes > pinned_bytes) {
     NNV_HIP_TRY(hipStreamSynchronize(stream));
-    if (pinned) NNV_HIP_TRY(hipHostFree(pinned));
+    // a table handed out from the old ring may still be named by a launch that is about to be issued:
+    // the old ring stays allocated until the context goes (rings only ever grow, by doubling)
+    if (pinned) retired_rings.push_back(pinned);
     pinned = nullptr;
     pinned_bytes = std::max(bytes * 2, size_t(4) << 20);
     NNV_HIP_TRY(hipHostMalloc((void**)&pinned, pinned_bytes, hipHostMallocDefault));
@@ -103,6 +105,18 @@ int nnvhip_ctx::stage(size_t bytes, void** host) {
   }
   *host = pinned + pinned_off;
   pinned_off += bytes;
+  return NNVHIP_OK;
+}
+
+int nnvhip_ctx::upload_table(const void* host, size_t bytes, BufRef* out) {
+  if (bytes > (size_t(64) << 10)) return upload(host, bytes, out);
+  void* st = nullptr;
+  NNV_TRY(stage(bytes, &st));
+  memcpy(st, host, bytes);
+  auto b = std::make_shared<Buffer>();  // no owner: the slot belongs to the ring
+  b->ptr = st;
+  b->bytes = bytes;
+  *out = std::move(b);
   return NNVHIP_OK;
 }
 
@@ -173,8 +187,8 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
-  NNV_HIP_TRY(hipHostMalloc((void**)&c->mailbox, 64, hipHostMallocDefault));
-  for (int i = 0; i < 16; ++i) c->mailbox[i] = 0;
+  NNV_HIP_TRY(hipHostMalloc((void**)&c->mailbox, sizeof(int64_t) * nnvhip_ctx::kMailboxSets, hipHostMallocDefault));
+  memset((void*)c->mailbox, 0, sizeof(int64_t) * nnvhip_ctx::kMailboxSets);
   NNV_HIP_TRY(hipEventCreate(&c->kev0));
   NNV_HIP_TRY(hipEventCreate(&c->kev1));
   *out = c;
@@ -189,6 +203,7 @@ int nnvhip_destroy(nnvhip_ctx* c) {
   c->trim();
   if (c->pinned) (void)hipHostFree(c->pinned);
   if (c->mailbox) (void)hipHostFree((void*)c->mailbox);
+  for (char* r : c->retired_rings) (void)hipHostFree(r);
   (void)hipEventDestroy(c->ev0);
   (void)hipEventDestroy(c->ev1);
   (void)hipEventDestroy(c->kev0);
@@ -978,7 +993,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           off += in[i]->n + 1;  // box stars: all columns stored, input and output arenas laid out alike
         }
         BufRef cmap;
-        if (st == NNVHIP_OK) st = c->upload(map.data(), sizeof(int32_t) * map.size(), &cmap);
+        if (st == NNVHIP_OK) st = c->upload_table(map.data(), sizeof(int32_t) * map.size(), &cmap);
         if (st == NNVHIP_OK) {
           GemmRows rows;
           rows.colmap = cmap->as<int32_t>();
@@ -988,7 +1003,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       } else if (any_rows || any_onehot) {
         std::vector<GemmSeg> segs;
         GemmRows rows;
-        const int64_t tn = gemm_seg_cols(fc->Mp);
+        const int64_t tn = gemm_seg_cols(fc->Mp, count, dense.data());
         rows.seg_cols = (int32_t)tn;
         // several row tiles would each gather the kept rows of B: pack them once per set instead
         BufRef packed;
@@ -1031,7 +1046,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           off_in += in[i]->stored_cols();
         }
         BufRef dsegs;
-        if (st == NNVHIP_OK && !segs.empty()) st = c->upload(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
+        if (st == NNVHIP_OK && !segs.empty()) st = c->upload_table(segs.data(), sizeof(GemmSeg) * segs.size(), &dsegs);
         if (st == NNVHIP_OK && !segs.empty()) {
           rows.segs = dsegs->as<GemmSeg>();
           st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, tn * (int64_t)segs.size(),
@@ -1047,7 +1062,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         for (int64_t i = 1; i < count; ++i)
           if (!filled[i]) centres.push_back(outs[i]->V);
         BufRef tab;
-        if (!centres.empty()) st = c->upload(centres.data(), sizeof(double*) * centres.size(), &tab);
+        if (!centres.empty()) st = c->upload_table(centres.data(), sizeof(double*) * centres.size(), &tab);
         if (st == NNVHIP_OK && !centres.empty()) st = launch_bias_columns(c, tab->as<double*>(), (int64_t)centres.size(), bias, fc->Mp);
       }
       if (st == NNVHIP_OK && (any_onehot || any_fill)) {

@@ -254,7 +254,7 @@ static int run_row_layer(nnvhip_ctx* c, int64_t count, nnvhip_star* const* in, n
     const SetDesc* table = nullptr;
     BufRef tab;
     if (count > 1) {
-      st = c->upload(descs.data(), sizeof(SetDesc) * descs.size(), &tab);
+      st = c->upload_table(descs.data(), sizeof(SetDesc) * descs.size(), &tab);
       if (st == NNVHIP_OK) table = tab->as<SetDesc>();
     }
     if (st == NNVHIP_OK) {

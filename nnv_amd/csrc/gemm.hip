@@ -254,16 +254,19 @@ __global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __
         if (ccol < col_end) {
           double v = acc[i][j][r];
           if (bias != nullptr && ccol == 0) v = v + bias[row];
-          C[row + ((MAPPED && colmap != nullptr) ? (int64_t)colmap[ccol] : ccol) * ldc] = v;
+          // (partial products of a split go to the workspace column by column; the reduction maps them)
+          C[row + ((MAPPED && colmap != nullptr && ksplit == 1) ? (int64_t)colmap[ccol] : ccol) * ldc] = v;
         }
       }
     }
   }
 }
 
+// colmap (or null): column t of the partial products belongs at column colmap[t] of C.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __restrict__ part, int ksplit, int Mp,
                                                              int64_t ncols, double* __restrict__ C, int64_t ldc,
-                                                             const double* __restrict__ bias) {
+                                                             const double* __restrict__ bias,
+                                                             const int32_t* __restrict__ colmap) {
   const int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   const int64_t total = (int64_t)Mp * ncols;
   if (t >= total) return;
@@ -272,7 +275,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __rest
   const int64_t col = t / Mp;
   const int row = (int)(t - col * Mp);
   if (bias != nullptr && col == 0) s = s + bias[row];
-  C[row + col * ldc] = s;
+  C[row + (colmap != nullptr ? (int64_t)colmap[col] : col) * ldc] = s;
 }
 
 template <int TM, int TN, int WR, int WC, int KT>
@@ -311,8 +314,10 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   int64_t ksplit = 1;
   if (blocks < 128 && nk >= 8) ksplit = std::min<int64_t>(std::min<int64_t>(16, nk / 4), ceil_div(512, blocks));
   if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
-  // the split-K workspace is laid out for one plain column range: no segment tables, no column maps
-  if (rows != nullptr && (rows->segs != nullptr || rows->colmap != nullptr)) ksplit = 1;
+  // the split-K workspace is laid out for one plain column range: no segment tables (a column map is
+  // applied by the reduction)
+  if (rows != nullptr && rows->segs != nullptr) ksplit = 1;
+  if (rows != nullptr && rows->colmap != nullptr && defer != nullptr) ksplit = 1;
   if (rows != nullptr && rows->segs != nullptr && rows->seg_cols != TN)
     NNV_FAIL(NNVHIP_ERR_ARG, "internal: segment table built for another tile width");
   BufRef ws;
@@ -343,13 +348,21 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   } else if (ksplit > 1) {
     const int64_t total = Mp * ncols;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, ctx->stream,
-                       ws->as<double>(), (int)ksplit, (int)Mp, ncols, C, ldc, bias);
+                       ws->as<double>(), (int)ksplit, (int)Mp, ncols, C, ldc, bias, rows ? rows->colmap : nullptr);
   }
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }
 
-int gemm_seg_cols(int64_t Mp) { return Mp <= 16 ? 64 : 128; }
+// Tile width of a segmented launch: 128 x 128 tiles when there are enough of them to cover the chip,
+// 64 x 64 for small arrays (and the 16-row tile for skinny outputs).
+int gemm_seg_cols(int64_t Mp, int64_t count, const int64_t* cols) {
+  if (Mp <= 16) return 64;   // the 16 x 64 tile
+  if (Mp <= 32) return 128;  // the 32 x 128 tile
+  int64_t tiles = 0;
+  for (int64_t i = 0; i < count; ++i) tiles += ceil_div(cols[i], 128);
+  return tiles * ceil_div(Mp, 128) < 256 ? 64 : 128;
+}
 
 int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, int64_t ldb, double* C, int64_t ldc,
                 int64_t Mp, int64_t ncols, int64_t Kp, const double* bias, RangeFuse* fuse, const GemmRows* rows,
@@ -386,7 +399,8 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
       best_cost = cost;
     }
   }
-  if (rows != nullptr && rows->segs != nullptr) return NNV_GEMM(128, 128, 2, 4, 16);  // see gemm_seg_cols
+  if (rows != nullptr && rows->segs != nullptr)  // the table was cut for this width: see gemm_seg_cols
+    return rows->seg_cols == 64 ? NNV_GEMM(64, 64, 2, 4, 16) : NNV_GEMM(128, 128, 2, 4, 16);
   if (const char* e = getenv("NNVHIP_GEMM_TILE")) {  // tuning knob: "TMxTN" of one of the shapes above
     for (int i = 0; i < (int)(sizeof(shapes) / sizeof(shapes[0])); ++i)
       if (std::to_string(shapes[i].tm) + "x" + std::to_string(shapes[i].tn) == e) best = i;
@@ -451,7 +465,7 @@ int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {
   const PackSet* table = nullptr;
   BufRef tab;
   if (count > 1) {
-    NNV_TRY(ctx->upload(sets, sizeof(PackSet) * count, &tab));
+    NNV_TRY(ctx->upload_table(sets, sizeof(PackSet) * count, &tab));
     table = tab->as<PackSet>();
   }
   hipLaunchKernelGGL(pack_rows_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count), dim3(512), 0, ctx->stream,

@@ -96,11 +96,13 @@ struct nnvhip_ctx {
   int64_t live_handles = 0;
   // pinned staging ring for descriptor tables and small read-backs
   char* pinned = nullptr;
+  std::vector<char*> retired_rings;
   size_t pinned_bytes = 0;
   size_t pinned_off = 0;
   // mailbox in pinned host memory: a kernel posts {m, inactive, sequence number} there and the host
   // spins on it, which is quicker than a device-to-host copy plus stream synchronisation
-  volatile int32_t* mailbox = nullptr;
+  volatile int32_t* mailbox = nullptr;  // kMailboxSets words of 64 bits, one per set of an array
+  static constexpr int64_t kMailboxSets = 8192;
   int32_t mailbox_seq = 0;
   // FC layers as the full dense contraction (no skipping of structural zeros); default from the
   // environment variable NNVHIP_DENSE_AFFINE
@@ -135,6 +137,10 @@ struct nnvhip_ctx {
   int stage(size_t bytes, void** host);
   // Copies a host table to a fresh device buffer through the pinned ring (async on the stream).
   int upload(const void* host, size_t bytes, nnvhip::BufRef* out);
+  // A descriptor table that only the launches of the current call read.  Small ones stay in the pinned
+  // staging ring and the kernels read them from there (no copy on the stream); the slot is not reused
+  // before the stream has been synchronised.
+  int upload_table(const void* host, size_t bytes, nnvhip::BufRef* out);
   int begin_op();
   int end_op();
 };
@@ -247,9 +253,10 @@ struct RangeFuse {
 // column 0 when non-null.  Mp, Kp multiples of 16; padding rows of A and B are zero.
 // rows (optional): contraction over a subset of the K rows.  kmap lists the rows of B (= columns of A)
 // that can be non-zero, padded with -1 to a multiple of 16; Kp passed to launch_gemm is then the padded
-// length of that list.  With segs (arrays of sets), column tile t of seg_cols = 128 columns has its own
+// length of that list.  With segs (arrays of sets), column tile t of seg_cols columns has its own
 // description: its row list (null = all rows), the arena column of its first column and how many of
-// its columns exist; ncols is then seg_cols * (number of tiles), seg_cols = gemm_seg_cols(Mp).
+// its columns exist; ncols is then seg_cols * (number of tiles), seg_cols = gemm_seg_cols(...) (64 for
+// small arrays and skinny outputs).
 struct GemmSeg {
   const int32_t* kmap;
   const double* Bk;    // the set's packed rows (see GemmRows::Bk), or null
@@ -273,7 +280,7 @@ struct GemmRows {
   int32_t seg_cols = 128;
   double flop = 0.0;  // flop actually executed (for the kernel timers)
 };
-int gemm_seg_cols(int64_t Mp);
+int gemm_seg_cols(int64_t Mp, int64_t count, const int64_t* cols);
 // Vk(t, j) = V(kept[t], j) for t < kp (a multiple of 16; zero where kept[t] < 0), j < ncols; Vk has
 // leading dimension kp.
 struct PackSet {

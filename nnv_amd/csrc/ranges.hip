@@ -318,7 +318,7 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
   const GatherSet* table = nullptr;
   BufRef tab;
   if (count > 1) {
-    NNV_TRY(ctx->upload(sets, sizeof(GatherSet) * count, &tab));
+    NNV_TRY(ctx->upload_table(sets, sizeof(GatherSet) * count, &tab));
     table = tab->as<GatherSet>();
   }
   // algorithmic HBM bytes: every output column written once, W read once (its columns are re-read
@@ -404,7 +404,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   const RangeDesc* table = nullptr;
   BufRef tab;
   if (nset > 1) {
-    NNV_TRY(ctx->upload(descs.data(), sizeof(RangeDesc) * nset, &tab));
+    NNV_TRY(ctx->upload_table(descs.data(), sizeof(RangeDesc) * nset, &tab));
     table = tab->as<RangeDesc>();
   }
   dim3 grid((unsigned)row_blocks, (unsigned)chunks, (unsigned)nset);

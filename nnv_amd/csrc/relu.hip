@@ -669,7 +669,7 @@ static int launch_apply(nnvhip_ctx* ctx, int64_t count, std::vector<ReluDesc>& d
   const ReluDesc* table = nullptr;
   BufRef tab;
   if (count > 1) {
-    NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
+    NNV_TRY(ctx->upload_table(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
@@ -843,15 +843,18 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.ncols_in = (int32_t)(in[i]->n + 1);
     d.order = order;
   }
-  const bool use_mailbox = count == 1 && ctx->mailbox != nullptr && N < (int64_t(1) << kMailboxCountBits);
-  if (use_mailbox) {
-    descs[0].mailbox = const_cast<int32_t*>(ctx->mailbox);
-    descs[0].mailbox_seq = ++ctx->mailbox_seq;
+  const bool use_mailbox = count <= nnvhip_ctx::kMailboxSets && ctx->mailbox != nullptr && N < (int64_t(1) << kMailboxCountBits);
+  if (use_mailbox) {  // every set's block posts into a word of its own
+    ++ctx->mailbox_seq;
+    for (int64_t i = 0; i < count; ++i) {
+      descs[i].mailbox = const_cast<int32_t*>(ctx->mailbox) + 2 * i;
+      descs[i].mailbox_seq = ctx->mailbox_seq;
+    }
   }
   const ReluDesc* table = nullptr;
   BufRef tab;
   if (count > 1) {
-    NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
+    NNV_TRY(ctx->upload_table(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
   // Up to 8192 neurons: one block per set classifies, compacts and sorts (bitonic network).  Larger
@@ -887,17 +890,19 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     long spins = 0;
     const volatile unsigned long long* box = reinterpret_cast<const volatile unsigned long long*>(ctx->mailbox);
     const unsigned long long want = (unsigned long long)((unsigned)ctx->mailbox_seq & 0xffffu);
-    unsigned long long w = *box;
-    while ((w >> (2 * kMailboxCountBits)) != want) {
-      if ((++spins & 0xfff) == 0 &&
-          std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 10.0) {
-        NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));  // surfaces a launch failure, if any
-        if (((*box) >> (2 * kMailboxCountBits)) != want) NNV_FAIL(NNVHIP_ERR_HIP, "classification kernel did not report its counts");
+    for (int64_t i = 0; i < count; ++i) {
+      unsigned long long w = box[i];
+      while ((w >> (2 * kMailboxCountBits)) != want) {
+        if ((++spins & 0xfff) == 0 &&
+            std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 10.0) {
+          NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));  // surfaces a launch failure, if any
+          if ((box[i] >> (2 * kMailboxCountBits)) != want) NNV_FAIL(NNVHIP_ERR_HIP, "classification kernel did not report its counts");
+        }
+        w = box[i];
       }
-      w = *box;
+      counts[2 * i] = (int32_t)((w >> kMailboxCountBits) & ((1u << kMailboxCountBits) - 1));
+      counts[2 * i + 1] = (int32_t)(w & ((1u << kMailboxCountBits) - 1));
     }
-    counts[0] = (int32_t)((w >> kMailboxCountBits) & ((1u << kMailboxCountBits) - 1));
-    counts[1] = (int32_t)(w & ((1u << kMailboxCountBits) - 1));
   } else {
     void* hc = nullptr;
     NNV_TRY(ctx->stage(sizeof(int32_t) * 2 * count, &hc));
@@ -946,7 +951,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.write_bounds = 1;
   }
   if (count > 1 && !fold_bounds) {
-    NNV_TRY(ctx->upload(descs.data(), sizeof(ReluDesc) * count, &tab));
+    NNV_TRY(ctx->upload_table(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
   if (sorted && sort_cap == 0 && max_m > 0 && max_m <= 1024) {
