@@ -265,8 +265,10 @@ def main():
     if t is not None and args.method == "relax-star-area":
         roofline["traffic"] = round((t[0] + t[1]) * 1048576.0)
     if relu_ms > 0:
-        roofline["relu_step_algo_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
-        roofline["relu_step_frac_of_hbm_peak"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        # bytes the dense materialisation of the ReLU steps would move (read V for the ranges, read the kept
+        # rows, write the output) over the time the steps took; the steps leave most of that undone (pending
+        # row reset, range sums from the producing layer), so this can exceed the HBM peak
+        roofline["relu_step_dense_equivalent_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
 
     # ---- the same step with the host buffers the boundary takes and returns (not `value`) -----------
     # lb / ub uploaded and the input set built on the device, the reach, the output bounds back on the host
