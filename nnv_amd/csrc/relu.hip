@@ -74,74 +74,7 @@ __device__ __forceinline__ bool sorts_before(double ka, int ia, double kb, int i
   return ka > kb || (ka == kb && ia < ib);
 }
 
-// Bitonic network over P = 2^ceil(log2 m) entries staged in skey/sidx (m <= CAP), element
-// i = e*1024 + tid held in registers.  Exchange distance j < 64 stays inside a wave (shuffles),
-// 64 <= j < 1024 goes through LDS, j >= 1024 pairs two registers of the same thread.  Writes the
-// neuron indices in sorted order to out[0..m).  All 1024 threads of the block must call it.
-template <int CAP>
-__device__ __forceinline__ void bitonic_sort_desc(double* skey, int* sidx, int m, int tid, int32_t* __restrict__ out) {
-  constexpr int E = CAP >= 1024 ? CAP / 1024 : 1;
-  int P = 1;
-  while (P < m) P <<= 1;
-  double key[E];
-  int idx[E];
-#pragma unroll
-  for (int e = 0; e < E; ++e) {
-    const int i = e * 1024 + tid;
-    key[e] = i < m ? skey[i] : -__builtin_huge_val();  // sentinels sort after every real entry
-    idx[e] = i < m ? sidx[i] : 0x7fffffff;
-  }
-  for (int k = 2; k <= P; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      if (j >= 64 && j < 1024) {
-        __syncthreads();
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          skey[e * 1024 + tid] = key[e];
-          sidx[e * 1024 + tid] = idx[e];
-        }
-        __syncthreads();
-      }
-#pragma unroll
-      for (int e = 0; e < E; ++e) {
-        const int i = e * 1024 + tid;
-        if (i >= P) continue;
-        double pk;
-        int pi;
-        if (j >= 1024) {
-          const int pe = e ^ (j >> 10);
-          if (pe < e) continue;  // both registers of the pair are updated when the lower one is visited
-          pk = key[pe];
-          pi = idx[pe];
-          const bool want_before = (i & k) == 0;
-          if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
-            key[pe] = key[e];
-            idx[pe] = idx[e];
-            key[e] = pk;
-            idx[e] = pi;
-          }
-          continue;
-        } else if (j >= 64) {
-          pk = skey[i ^ j];
-          pi = sidx[i ^ j];
-        } else {
-          pk = __shfl_xor(key[e], j);
-          pi = __shfl_xor(idx[e], j);
-        }
-        const bool want_before = ((i & j) == 0) == ((i & k) == 0);
-        if (sorts_before(key[e], idx[e], pk, pi) != want_before) {
-          key[e] = pk;
-          idx[e] = pi;
-        }
-      }
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < E; ++e) {
-    const int i = e * 1024 + tid;
-    if (i < m) out[i] = idx[e];
-  }
-}
+constexpr int kSortInBlock = 1024;  // longest crossing list the classification block sorts itself
 
 // ---- sorting network for lists of at most 1024 entries, one entry per thread -------------------
 // Keys are non-negative doubles, so their bit patterns order like signed 64-bit integers; the
@@ -262,8 +195,8 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   __shared__ int wcross[16];
   __shared__ int winact[16];
   __shared__ int wkeep[16];
-  __shared__ double skey[SORT_CAP > 0 ? SORT_CAP : 1];
-  __shared__ int sidx[SORT_CAP > 0 ? SORT_CAP : 1];
+  __shared__ double skey[SORT_CAP > 0 ? kSortInBlock : 1];
+  __shared__ int sidx[SORT_CAP > 0 ? kSortInBlock : 1];
   static_assert(sizeof(double) == sizeof(long long), "keys are sorted through their bit patterns");
   int base = 0, inact_total = 0, keep_base = 0;
   int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
@@ -303,11 +236,17 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
       if (d.order == NNVHIP_ORDER_INDEX) {
         idx_out[pos] = r;
       } else {
-        // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb.  The list is sorted below, straight from LDS (a
-        // set of at most SORT_CAP neurons cannot have more crossing ones).
+        // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb.  Lists of up to kSortInBlock entries are sorted
+        // below, straight from LDS; a set with more neurons than that may have a longer list, which the
+        // multi-block rank kernels sort from the copies in global memory.
         const double key = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l))
                            : d.order == NNVHIP_ORDER_RANGE ? u - l : d.given_key[r];
-        if (SORT_CAP > 0 && pos < SORT_CAP) {
+        if (SORT_CAP > kSortInBlock) {
+          idx_out[pos] = r;
+          d.key[pos] = key;
+          d.rank[pos] = 0;
+        }
+        if (SORT_CAP > 0 && pos < kSortInBlock) {
           skey[pos] = key;
           sidx[pos] = r;
         }
@@ -325,20 +264,18 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     if (keep_base + tid < end) d.keep_idx[keep_base + tid] = -1;
   }
   const int m = base;
-  const bool sort_here = SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= SORT_CAP;
+  const bool sort_here = SORT_CAP > 0 && d.order != NNVHIP_ORDER_INDEX && m > 0 && m <= kSortInBlock;
+  // order settled in this block (otherwise the rank kernels settle it and the bounds follow them)
+  const bool order_known = d.order == NNVHIP_ORDER_INDEX || m <= kSortInBlock;
   if (sort_here) __syncthreads();  // the keys are staged; nothing of the stores below is in flight yet
   if (tid == 0) {
     d.counts[0] = m;
     d.counts[1] = inact_total;
     post_counts(d.mailbox, m, inact_total, d.mailbox_seq);  // the host can size the output while we sort
   }
-  if (sort_here) {
-    if (SORT_CAP == 1024 || m <= 1024)  // the staged doubles are read back as their bit patterns
-      sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
-    else
-      bitonic_sort_desc<SORT_CAP>(skey, sidx, m, tid, d.cross_idx);
-  }
-  if (d.write_bounds) {  // the output buffers were sized for the worst case: finish the set here
+  if (sort_here)  // the staged doubles are read back as their bit patterns
+    sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
+  if (d.write_bounds && order_known) {  // the output buffers were sized for the worst case: finish the set here
     __syncthreads();     // cross_idx is complete
     const int n_in = d.ncols_in - 1;
     // four entries per thread and step, all loads issued before the first store (the dependent
@@ -857,9 +794,10 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->upload_table(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
-  // Up to 8192 neurons: one block per set classifies, compacts and sorts (bitonic network).  Larger
-  // sets: two multi-block passes; their sort, if any, follows the read-back of the counts.
-  const int sort_cap = !sorted ? 0 : N <= 1024 ? 1024 : N <= 8192 ? 8192 : 0;
+  // Up to 8192 neurons: one block per set classifies, compacts and sorts crossing lists of up to 1024
+  // entries (sorting network).  Larger sets: two multi-block passes.  Whatever is still unsorted after
+  // the read-back of the counts goes to the multi-block rank kernels.
+  const int sort_cap = !sorted ? 0 : N <= 8192 ? kSortInBlock : 0;
   // algorithmic bytes of the classification: lb and ub read, the per-row class and the two index lists
   // written (plus, when it also writes the predicate bounds, the copy of the input's)
   double cls_bytes = 0.0;
@@ -950,7 +888,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.ld_lbub = ldr;
     d.write_bounds = 1;
   }
-  if (count > 1 && !fold_bounds) {
+  // lists the classification block left unsorted (and, with them, bounds it left unwritten)
+  const bool need_rank = sorted && sort_cap > 0 && max_m > sort_cap;
+  if (count > 1 && (!fold_bounds || need_rank)) {
     NNV_TRY(ctx->upload_table(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
@@ -962,7 +902,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
     hipLaunchKernelGGL(relu_scatter_kernel, dim3(t, 1, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
   }
-  if (fold_bounds) {
+  if (fold_bounds && !need_rank) {
     // nothing left to launch
   } else if (lazy_rows) {
     if (max_pred > 0) {
