@@ -27,6 +27,8 @@ sys.path.insert(0, ROOT)
 
 import numpy as np  # noqa: E402
 
+import nnv_amd  # noqa: E402
+
 FP64_MFMA_PEAK_TFLOPS = 78.6
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
@@ -40,7 +42,7 @@ MEASURED_TRAFFIC_MIB = {("cfg2_fc_784_1024x3_10", "gemm_f64_kernel", "dense"): (
 def layer_shapes(reach_set):
     out = []
     for s in reach_set:
-        sets = s if isinstance(s, list) else [s]
+        sets = s if isinstance(s, (list, nnv_amd.SetArray)) else [s]
         for t in sets:
             N, n, _ = t._h.dims()
             out.append((N, n))
@@ -64,7 +66,6 @@ def main():
         sys.exit("bench.py: this build runs on one GPU only (sets shard across GPUs without communication; "
                  "that path is not built) - use --gpus 1")
 
-    import nnv_amd
     from nnv_amd.configs import count_updates, device_input_sets, make_config, make_extended_cnn
 
     cfg = make_extended_cnn(32, 3) if args.config == 6 else make_config(args.config)
@@ -77,7 +78,7 @@ def main():
 
     def step():
         out = net.reach(dev_in, opts)
-        outs = out if isinstance(out, list) else [out]
+        outs = out if isinstance(out, (list, nnv_amd.SetArray)) else [out]
         arr = (ctypes.c_void_p * len(outs))(*[o_._h.h for o_ in outs])
         # output bounds of all sets in one batched call, left on the device
         nnv_amd._lib.check(lib.nnvhip_estimate_ranges_batch(h, len(outs), arr, None, None))
@@ -146,9 +147,9 @@ def main():
     gemm_flop = conv_flop = 0.0
     relu_bytes, relu_ms = 0.0, 0.0
     layer_report = []
-    prev_sets = dev_in if isinstance(dev_in, list) else [dev_in]
+    prev_sets = dev_in if isinstance(dev_in, (list, nnv_amd.SetArray)) else [dev_in]
     for i, (Ld, L) in enumerate(zip(cfg["layers"], net.Layers)):
-        outs = net.reachSet[i] if isinstance(net.reachSet[i], list) else [net.reachSet[i]]
+        outs = net.reachSet[i] if isinstance(net.reachSet[i], (list, nnv_amd.SetArray)) else [net.reachSet[i]]
         entry = {"layer": i + 1, "type": Ld["type"], "ms": round(float(per_layer[i]), 4)}
         if Ld["type"] == "fc":
             M, K = Ld["W"].shape
@@ -226,7 +227,7 @@ def main():
     groups.sort(key=lambda g: -g[0])
     roofline = dict(groups[0][1])
     roofline["other_kernels"] = [g[1] for g in groups[1:]]
-    n_sets = len(dev_in) if isinstance(dev_in, list) else 1
+    n_sets = len(dev_in) if isinstance(dev_in, (list, nnv_amd.SetArray)) else 1
     if cls_launches:
         # One block per set (classification, in-block sort of the crossing list, new predicate bounds): a
         # dependent chain on a single CU, bound by latency and not by a roofline.  It is listed with the
@@ -278,7 +279,7 @@ def main():
     for _ in range(n_h2h):
         fresh = device_input_sets(cfg, ctx)
         res = net.reach(fresh, opts)
-        nnv_amd.Star.estimateRanges_array(res if isinstance(res, list) else [res])
+        nnv_amd.Star.estimateRanges_array(res if isinstance(res, (list, nnv_amd.SetArray)) else [res])
     host_to_host_ms = 1e3 * (time.perf_counter() - t1) / n_h2h
     del fresh, res
 
@@ -335,9 +336,9 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": cfg["name"], "reach_method": args.method, "relax_factor": 1,
                    "fc_affine_map": "dense" if args.dense else "structural zeros skipped (one-hot generator columns, reset rows); exact",
-                   "sets": len(dev_in) if isinstance(dev_in, list) else 1,
+                   "sets": len(dev_in) if isinstance(dev_in, (list, nnv_amd.SetArray)) else 1,
                    "updates_per_step": updates,
-                   "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, list) else None},
+                   "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, (list, nnv_amd.SetArray)) else None},
         "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec,
         "host_to_host": {"ms_per_step": round(host_to_host_ms, 4), "steps": n_h2h,
                          "what": "input bounds uploaded and the set(s) built, reach, output bounds fetched to the host"},

@@ -127,6 +127,10 @@ NNVHIP_API int nnvhip_star_from_box(nnvhip_ctx* ctx, int64_t N, int64_t count, c
                          nnvhip_star** out);
 NNVHIP_API int nnvhip_star_retain(nnvhip_star* s);
 NNVHIP_API int nnvhip_star_release(nnvhip_star* s);
+/* Releases one reference of each of `count` handles (null entries are skipped): what clearing an
+ * object array of sets does in the reference, e.g. when NN.reach overwrites the per-layer outputs
+ * it keeps in reachSet (nn/NN.m:1531, 1547). */
+NNVHIP_API int nnvhip_star_release_array(int64_t count, nnvhip_star* const* sets);
 /* dim, nVar and the number of constraint rows size(C,1). */
 NNVHIP_API int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p);
 /* Property reads: dense MATLAB arrays.  V: N x (n+1).  Bounds: n each.  C: p x n, d: p, laid out

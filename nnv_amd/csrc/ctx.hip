@@ -537,6 +537,12 @@ int nnvhip_star_release(nnvhip_star* s) {
   return NNVHIP_OK;
 }
 
+int nnvhip_star_release_array(int64_t count, nnvhip_star* const* sets) {
+  if (count < 0 || (count > 0 && !sets)) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  for (int64_t i = 0; i < count; ++i) nnvhip_star_release(sets[i]);
+  return NNVHIP_OK;
+}
+
 int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p) {
   if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
   if (N) *N = s->N;

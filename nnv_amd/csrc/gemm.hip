@@ -17,8 +17,9 @@ namespace nnvhip {
 // (TM/WR) x (TN/WC) = (16*FM) x (16*FN).
 // MAPPED = false: the plain product.  MAPPED = true additionally honours a row list (kmap), a per-tile
 // segment table (segs) and a column map (colmap); kept apart so that the plain kernel pays nothing.
-template <int TM, int TN, int WR, int WC, int KT, bool MAPPED>
-__global__ __launch_bounds__(64 * WR * WC) void gemm_f64_kernel(const double* __restrict__ A, int64_t lda,
+// WPE: waves per SIMD the register allocation is held to (1: whatever the code needs).
+template <int TM, int TN, int WR, int WC, int KT, bool MAPPED, int WPE = 1>
+__global__ __launch_bounds__(64 * WR * WC, WPE) void gemm_f64_kernel(const double* __restrict__ A, int64_t lda,
                                                         const double* __restrict__ B, int64_t ldb,
                                                         double* __restrict__ C, int64_t ldc, int Mp, int64_t ncols,
                                                         int Kp, const double* __restrict__ bias, int tiles_m,
@@ -330,13 +331,20 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   }
   const bool timed = ctx->kernel_timing && TM >= 64;
   NNV_TRY(ctx->kernel_timer_begin(timed));
-  if (rows != nullptr)
-    NNV_LAUNCH(ctx, timed, (gemm_f64_kernel<TM, TN, WR, WC, KT, true>), dim3((unsigned)grid_x, (unsigned)ksplit),
+  if (rows != nullptr) {
+    // The mapped 128 x 128 tile needs a few registers more than let two blocks share a CU.  With a short
+    // contraction (few kept rows) the start and the end of a tile weigh as much as its K loop, and a
+    // second resident block hides them: for launches of many such tiles the allocation is held to 128
+    // registers (at the price of a few reloads per K-tile; measured: 12% quicker at K = 240 over
+    // 57344 tiles, 8% slower over 460 tiles, where two rounds of one block per CU do as well).
+    auto kern = gemm_f64_kernel<TM, TN, WR, WC, KT, true>;
+    if (TM == 128 && TN == 128 && Kp <= 512 && blocks >= 2048) kern = gemm_f64_kernel<TM, TN, WR, WC, KT, true, (TM == 128 && TN == 128 ? 4 : 1)>;
+    NNV_LAUNCH(ctx, timed, kern, dim3((unsigned)grid_x, (unsigned)ksplit),
                        dim3(64 * WR * WC), 0, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
                        (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,
                        fuse ? fuse->plb : nullptr, fuse ? fuse->pub : nullptr, rpart, rows->kmap, rows->segs, rows->colmap,
                        rows->Bk, rows->ldbk);
-  else
+  } else
     NNV_LAUNCH(ctx, timed, (gemm_f64_kernel<TM, TN, WR, WC, KT, false>), dim3((unsigned)grid_x, (unsigned)ksplit),
                        dim3(64 * WR * WC), 0, A, lda, B, ldb, C, ldc, (int)Mp, ncols, (int)Kp, bias, (int)tiles_m,
                        (int)tiles_n, (int)best_xr, (int)local_m, (int)ksplit, ws ? ws->as<double>() : nullptr,

@@ -13,7 +13,7 @@ import numpy as np
 
 from . import _lib
 from ._lib import ORDER_AREA, ORDER_INDEX, ORDER_RANGE, check, f64, ptr
-from .sets import ImageStar, Star, _Handle
+from .sets import ImageStar, SetArray, Star, _Handle
 
 RELAX_ORDER = {
     "relax-star-range": ORDER_RANGE,   # nn/funcs/PosLin.m:934-936
@@ -27,26 +27,45 @@ _AFFINE_STAR_METHODS = ("approx-star", "exact-star", "abs-dom")
 
 
 def _as_list(sets):
+    """(array of sets, whether a single set was given).  An array a layer returned stays as it is: its
+    elements are only made into objects when somebody reads them."""
+    if isinstance(sets, SetArray):
+        return sets, False
     single = not isinstance(sets, (list, tuple))
     return ([sets] if single else list(sets)), single
 
 
 def _handles_array(sets):
+    if isinstance(sets, SetArray):
+        return sets.handles()
     return (C.c_void_p * len(sets))(*[s._h.h for s in sets])
 
 
-def _wrap_like(inputs, ctx, raw, shape_fn=None):
-    mk, H = Star._from_handle, _Handle
-    if type(inputs[0]) is Star and all(type(s) is Star for s in inputs):
-        return [mk(H(h, ctx)) for h in raw]          # the common case, kept cheap: arrays of 1000s of sets
-    outs = []
-    for s, h in zip(inputs, raw):
-        hd = H(h, ctx)
+def _shapes(sets):
+    """None when every set of the array is a Star; else one entry per set, None for a Star and
+    (height, width, numChannel) for an ImageStar.  Anything else in the array is a TypeError."""
+    if isinstance(sets, SetArray):
+        return sets.shapes
+    if all(type(s) is Star for s in sets):
+        return None
+    out = []
+    for s in sets:
         if isinstance(s, ImageStar):
-            outs.append(ImageStar(_handle=hd, shape=shape_fn(s)))
+            out.append((s.height, s.width, s.numChannel))
+        elif isinstance(s, Star):
+            out.append(None)
         else:
-            outs.append(mk(hd))
-    return outs
+            raise TypeError("not a Star or an ImageStar")
+    return out
+
+
+def _wrap_like(inputs, ctx, raw, out_shape=None):
+    """The output array for the handles `raw`: a Star for a Star input, an ImageStar of `out_shape`
+    (default: the input's own shape) for an ImageStar input."""
+    shp = _shapes(inputs)
+    if shp is not None and out_shape is not None:
+        shp = [None if s is None else out_shape for s in shp]
+    return SetArray(ctx, raw, shp)
 
 
 class FullyConnectedLayer:
@@ -99,7 +118,7 @@ class FullyConnectedLayer:
         weights = weights or FullyConnectedLayer._Weights(ctx, W, b)
         out = (C.c_void_p * len(sets))()
         check(ctx.lib.nnvhip_affine_fc(ctx.handle, weights.h, len(sets), _handles_array(sets), out))
-        return _wrap_like(sets, ctx, out, lambda s: (1, 1, W.shape[0]))
+        return _wrap_like(sets, ctx, out, (1, 1, W.shape[0]))
 
     def _weights(self, ctx):
         if ctx not in self._dev:
@@ -113,14 +132,16 @@ class FullyConnectedLayer:
         """nn/layers/FullyConnectedLayer.m:295-316, 476-512."""
         if option not in (None, "", "single", "parallel") and not (isinstance(option, (list, tuple)) and len(option) == 0):
             raise ValueError("Unknown computation option, should be parallel or single")
-        if not inputs:
+        if not len(inputs):
             return []
-        for s in inputs:
-            if not isinstance(s, (Star, ImageStar)):
-                raise TypeError("Input set is not an ImageStar or Star")
-            if isinstance(s, ImageStar) and s.height * s.width * s.numChannel != self.InputSize:
+        try:
+            shapes = _shapes(inputs)
+        except TypeError:
+            raise TypeError("Input set is not an ImageStar or Star") from None
+        for shp in shapes or ():
+            if shp is not None and shp[0] * shp[1] * shp[2] != self.InputSize:
                 raise ValueError("Inconsistency between the size of the input image and the InputSize of the network")
-        ctx = inputs[0].ctx
+        ctx = inputs.ctx if isinstance(inputs, SetArray) else inputs[0].ctx
         return FullyConnectedLayer._map(ctx, self.Weights, self.Bias, inputs, self._weights(ctx))
 
     def reach(self, in_images, method="approx-star", option=None, relaxFactor=0, dis_opt=None, lp_solver="linprog"):
@@ -225,7 +246,7 @@ class Conv2DLayer:
         """nn/layers/Conv2DLayer.m:559-601, 780, 862-886."""
         if option not in (None, "", "single", "parallel") and not (isinstance(option, (list, tuple)) and len(option) == 0):
             raise ValueError("Unknown computation option")
-        if not inputs:
+        if not len(inputs):
             return []
         for s in inputs:
             if not isinstance(s, ImageStar):
@@ -241,7 +262,7 @@ class Conv2DLayer:
         out = (C.c_void_p * len(inputs))()
         check(ctx.lib.nnvhip_affine_conv2d(ctx.handle, self._weights(ctx).h, H, W, len(inputs),
                                            _handles_array(inputs), out))
-        return _wrap_like(inputs, ctx, out, lambda s: (ho, wo, self.NumFilters))
+        return _wrap_like(inputs, ctx, out, (ho, wo, self.NumFilters))
 
     def reach(self, in_images, method="approx-star", option="single", relaxFactor=0, dis_opt=None, lp_solver="linprog"):
         """nn/layers/Conv2DLayer.m:913-973."""
@@ -288,19 +309,21 @@ class PosLin:
         """PosLin.reach, nn/funcs/PosLin.m:2073-2169."""
         sets, single = _as_list(I)
         if method in RELAX_ORDER:
-            for s in sets:
-                if not isinstance(s, Star):
-                    raise TypeError("Input is not a star")
+            lazy = isinstance(sets, SetArray)
+            if not (lazy and sets.shapes is None):
+                for s in sets:
+                    if not isinstance(s, Star):
+                        raise TypeError("Input is not a star")
             if relaxFactor < 0 or relaxFactor > 1:
                 raise ValueError("Invalid relax factor")
-            if not sets:
+            if not len(sets):
                 return []
-            ctx = sets[0].ctx
+            ctx = sets.ctx if lazy else sets[0].ctx
             if relaxFactor == 1:
                 out = (C.c_void_p * len(sets))()
                 check(ctx.lib.nnvhip_relu_relax(ctx.handle, RELAX_ORDER[method], float(relaxFactor), len(sets),
                                                 _handles_array(sets), out))
-                res = [Star._from_handle(_Handle(h, ctx)) for h in out]
+                res = SetArray(ctx, out)
             else:
                 # some bounds are tightened by LPs first: host LP solver fed from the resident set
                 res = [PosLin.reach_relaxed_star_lp(s, method, relaxFactor, option, dis_opt, lp_solver) for s in sets]
@@ -414,11 +437,18 @@ class ReluLayer:
         toStar -> PosLin.reach -> toImageStar, which on the device is the same memory."""
         if option not in (None, "", "single", "parallel") and not (isinstance(option, (list, tuple)) and len(option) == 0):
             raise ValueError("Unknown computation option")
+        if "reduceMem" in method:
+            raise NotImplementedError("the reduceMem variants are outside this library")
+        if isinstance(in_images, SetArray) and method in RELAX_ORDER and relaxFactor == 1 and dis_opt != "display":
+            # an array straight from the previous layer: no object per set is needed
+            ctx, shapes = in_images.ctx, in_images.shapes
+            out = (C.c_void_p * len(in_images))()
+            if len(in_images):
+                check(ctx.lib.nnvhip_relu_relax(ctx.handle, RELAX_ORDER[method], 1.0, len(in_images), in_images.handles(), out))
+            return SetArray(ctx, out, None if shapes is None else list(shapes))
         for s in in_images:
             if not isinstance(s, (Star, ImageStar)):
                 raise TypeError("input is not an ImageStar, Star or VolumeStar")
-        if "reduceMem" in method:
-            raise NotImplementedError("the reduceMem variants are outside this library")
         stars = [s.toStar() if isinstance(s, ImageStar) else s for s in in_images]
         res = PosLin.reach(stars, method, None, relaxFactor, dis_opt, lp_solver) if stars else []
         out = []

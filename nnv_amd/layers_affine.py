@@ -35,10 +35,10 @@ class RowMap:
         except Exception:
             pass
 
-    def apply(self, sets, shape_fn=None):
+    def apply(self, sets, out_shape=None):
         out = (C.c_void_p * len(sets))()
         check(self.ctx.lib.nnvhip_affine_rowmap(self.ctx.handle, self.h, len(sets), _handles_array(sets), out))
-        return _wrap_like(sets, self.ctx, out, shape_fn or (lambda s: (s.height, s.width, s.numChannel)))
+        return _wrap_like(sets, self.ctx, out, out_shape)
 
 
 def _per_row(values, H, W, Cn):
@@ -314,7 +314,7 @@ class AveragePooling2DLayer:
         ho, wo = self.output_size(H, W)
         out = (C.c_void_p * len(inputs))()
         check(ctx.lib.nnvhip_affine_avgpool2d(ctx.handle, self._dev[ctx].h, H, W, len(inputs), _handles_array(inputs), out))
-        return _wrap_like(inputs, ctx, out, lambda s: (ho, wo, Cn))
+        return _wrap_like(inputs, ctx, out, (ho, wo, Cn))
 
     def reach(self, in_images, method="approx-star", option="single", relaxFactor=0, dis_opt=None, lp_solver="linprog"):
         """:550-608."""
@@ -384,7 +384,7 @@ class FlattenLayer:
         src = np.ascontiguousarray(src, dtype=np.int32)
         out = (C.c_void_p * len(inputs))()
         check(ctx.lib.nnvhip_permute_rows(ctx.handle, N, ptr(src), len(inputs), _handles_array(inputs), out))
-        return _wrap_like(inputs, ctx, out, lambda s: (1, 1, N))
+        return _wrap_like(inputs, ctx, out, (1, 1, N))
 
     def reach(self, in_images, method="approx-star", option="single", relaxFactor=0, dis_opt=None, lp_solver="linprog"):
         """:246-300."""

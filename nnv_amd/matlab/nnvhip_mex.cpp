@@ -98,7 +98,8 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
     plhs[0] = to_mx(out);
   } else if (cmd == "star_release") {
     need(nrhs, 1, "star_release");
-    for (auto* s : handles_of(prhs[1])) check(nnvhip_star_release(s));
+    const std::vector<nnvhip_star*> hs = handles_of(prhs[1]);
+    check(nnvhip_star_release_array((int64_t)hs.size(), hs.data()));
   } else if (cmd == "star_dims") {  // handle -> [dim nVar nConstraintRows]
     need(nrhs, 1, "star_dims");
     int64_t N, n, p;

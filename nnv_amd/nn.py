@@ -8,7 +8,7 @@ import numpy as np
 from .layers import Conv2DLayer, FullyConnectedLayer, ReluLayer
 from .layers_affine import (AveragePooling2DLayer, BatchNormalizationLayer, FlattenLayer, ImageInputLayer,
                             LayerS)
-from .sets import ImageStar, Star
+from .sets import ImageStar, SetArray, Star
 from .verify import HalfSpace, verify_specification
 
 
@@ -71,7 +71,7 @@ class NN:
 
     def reach(self, inputSet, reachOptions=None):
         """nn/NN.m:189-278: inputSet is a Star / ImageStar or a list of them."""
-        probe = inputSet[0] if isinstance(inputSet, (list, tuple)) and inputSet else inputSet
+        probe = inputSet[0] if isinstance(inputSet, (list, tuple, SetArray)) and len(inputSet) else inputSet
         if not isinstance(probe, (Star, ImageStar)):
             raise TypeError('Wrong input set type. Input set must be of type "Star", "ImageStar", "VolumeStar", "ImageZono", or "Zono"')
         if reachOptions is not None:
@@ -95,7 +95,7 @@ class NN:
         self.reachSet = [None] * self.numLayers
         self.reachTime = [0.0] * self.numLayers
         rs = inSet
-        ctx = (rs[0] if isinstance(rs, (list, tuple)) else rs).ctx
+        ctx = rs.ctx if isinstance(rs, SetArray) else (rs[0] if isinstance(rs, (list, tuple)) else rs).ctx
         timed = self.dis_opt == "display"
         for i, layer in enumerate(self.Layers):
             if timed:

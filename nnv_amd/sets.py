@@ -7,6 +7,7 @@ in MATLAB layout on demand.  Index vectors returned to Python are 0-based.
 """
 from __future__ import annotations
 
+import collections.abc
 import ctypes as C
 
 import numpy as np
@@ -458,14 +459,15 @@ class Star:
     @staticmethod
     def estimateRanges_array(sets):
         """estimateRanges of every set of an array in one device call -> (lb, ub), dim x count each."""
-        sets = list(sets)
-        if not sets:
+        if not isinstance(sets, SetArray):
+            sets = list(sets)
+        if not len(sets):
             return np.empty((0, 0)), np.empty((0, 0))
         ctx = sets[0].ctx
         N = sets[0]._h.dims()[0]          # Star or ImageStar: the flattened dimension
         lb = np.empty((N, len(sets)), order="F")
         ub = np.empty((N, len(sets)), order="F")
-        arr = (C.c_void_p * len(sets))(*[s._h.h for s in sets])
+        arr = sets.handles() if isinstance(sets, SetArray) else (C.c_void_p * len(sets))(*[s._h.h for s in sets])
         check(ctx.lib.nnvhip_estimate_ranges_batch(ctx.handle, len(sets), arr, ptr(lb), ptr(ub)))
         return lb, ub
 
@@ -588,3 +590,69 @@ class ImageStar:
 
     def relu_info(self):
         return self._h.relu_info()
+
+
+class SetArray(collections.abc.Sequence):
+    """The array of sets a layer returns for an array of input sets (the object arrays NN.reach
+    hands from layer to layer and keeps in reachSet, nn/NN.m:1544-1547).
+
+    It holds the device handles.  The Star / ImageStar object of an element is made when that element
+    is first read, so passing an array of a thousand sets through a network costs no Python work per
+    set; indexing, iteration, ``len`` and slicing (a plain list of the elements) behave as for a list.
+    """
+
+    __slots__ = ("ctx", "_raw", "_shapes", "_items")
+
+    def __init__(self, ctx, raw, shapes=None):
+        self.ctx = ctx
+        self._raw = raw          # ctypes array of handles; this object owns one reference of each
+        self._shapes = shapes    # None: Stars only; else per element None (Star) or (height, width, numChannel)
+        self._items = None       # the elements read so far (each then owns its handle's reference)
+
+    def __len__(self):
+        return len(self._raw)
+
+    def __getitem__(self, i):
+        if isinstance(i, slice):
+            return [self[k] for k in range(*i.indices(len(self._raw)))]
+        n = len(self._raw)
+        if i < 0:
+            i += n
+        if not 0 <= i < n:
+            raise IndexError("set array index out of range")
+        if self._items is None:
+            self._items = [None] * n
+        it = self._items[i]
+        if it is None:
+            hd = _Handle(self._raw[i], self.ctx)
+            shape = None if self._shapes is None else self._shapes[i]
+            it = Star._from_handle(hd) if shape is None else ImageStar(_handle=hd, shape=shape)
+            self._items[i] = it
+        return it
+
+    def __iter__(self):
+        for i in range(len(self._raw)):
+            yield self[i]
+
+    def handles(self):
+        """The handles as the ctypes array a batched entry point takes."""
+        return self._raw
+
+    @property
+    def shapes(self):
+        """None when every element is a Star, else one entry per element: None or the image shape."""
+        return self._shapes
+
+    def __repr__(self):
+        return "<SetArray of %d sets>" % len(self._raw)
+
+    def __del__(self):
+        try:
+            raw = self._raw
+            if self._items is not None:      # elements that were read keep their handle
+                for i, it in enumerate(self._items):
+                    if it is not None:
+                        raw[i] = None
+            self.ctx.release_sets(len(raw), raw)
+        except Exception:
+            pass

@@ -14,7 +14,7 @@ import numpy as np
 
 from . import _lib
 from ._lib import HS_DISJOINT, HS_INSIDE, HS_UNDECIDED, check, f64, ptr
-from .sets import ImageStar, Star
+from .sets import ImageStar, SetArray, Star
 
 
 class HalfSpace:
@@ -60,7 +60,7 @@ last_stats = SpecStats()
 
 
 def _as_star_handles(reachSet):
-    sets = list(reachSet) if isinstance(reachSet, (list, tuple)) else [reachSet]
+    sets = list(reachSet) if isinstance(reachSet, (list, tuple, SetArray)) else [reachSet]
     out = []
     for S in sets:
         if isinstance(S, ImageStar):

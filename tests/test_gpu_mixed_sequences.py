@@ -52,7 +52,7 @@ def _compare(nnv, oracle, layers, dev_in, ora_in, method, tol=1e-9):
     net = nnv.NN.from_config(layers)
     out = net.reach(dev_in, {"reachMethod": method, "relaxFactor": 1})
     exp, exp_sets = oracle.nn_reach(layers, ora_in, method, 1.0, keep=True)
-    outs = out if isinstance(out, list) else [out]
+    outs = out if isinstance(out, (list, nnv.SetArray)) else [out]
     exps = exp if isinstance(exp, list) else [exp]
     assert len(outs) == len(exps)
     for R, E in zip(outs, exps):
@@ -68,7 +68,7 @@ def _compare(nnv, oracle, layers, dev_in, ora_in, method, tol=1e-9):
     # every intermediate set too, read after the whole reach has run (so the reads meet sets whose
     # row reset or appended columns were never needed by the next layer)
     for i, (rset, eset) in enumerate(zip(net.reachSet, exp_sets)):
-        r0 = rset[0] if isinstance(rset, list) else rset
+        r0 = rset[0] if isinstance(rset, (list, nnv.SetArray)) else rset
         e0 = eset[0] if isinstance(eset, list) else eset
         RV, EV = np.asarray(r0.V), e0.V
         if EV.ndim == 4:

@@ -282,7 +282,7 @@ def _reach_in_subprocess(dense, k, method, shrink):
         "cfg = make_config(%d, %d)\n"
         "net = nnv_amd.NN.from_config(cfg['layers'])\n"
         "out = net.reach(device_input_sets(cfg), {'reachMethod': '%s', 'relaxFactor': 1})\n"
-        "outs = out if isinstance(out, list) else [out]\n"
+        "outs = out if isinstance(out, (list, nnv_amd.SetArray)) else [out]\n"
         "res = []\n"
         "for o_ in outs:\n"
         "    V = np.asarray(o_.V); lb, ub = o_.estimateRanges()\n"

@@ -140,7 +140,7 @@ def test_array_of_sets_and_multiple_halfspaces(nnv):
     from nnv_amd import verify
     cfg = make_config(5, 64)
     net, dev, ora = reach_both(nnv, cfg)
-    assert isinstance(dev, list) and len(dev) == len(ora) > 1
+    assert isinstance(dev, (list, nnv.SetArray)) and len(dev) == len(ora) > 1
     n_out = cfg["layers"][-1]["W"].shape[0]
     rs = np.random.RandomState(5)
     hs = [nnv.HalfSpace(rs.randn(2, n_out), rs.randn(2)) for _ in range(4)]

@@ -149,3 +149,51 @@ def test_precision_and_device_switches_of_a_set():
     assert _change_device(marker, "cpu") is marker and _change_device(marker, "gpu") is marker
     with pytest.raises(ValueError, match="'cpu' or 'gpu'"):
         _change_device(marker, "tpu")
+
+
+class _CountingCtx:
+    """Stands where a device context would: records which handles are released and how."""
+
+    def __init__(self):
+        self.single, self.bulk = [], []
+
+    def release_set(self, h):
+        self.single.append(h)
+
+    def release_sets(self, count, raw):
+        self.bulk.append([raw[i] for i in range(count) if raw[i]])
+
+
+def test_set_array_makes_objects_on_demand_and_releases_every_handle_once():
+    import ctypes as C
+    import gc
+    from nnv_amd.sets import ImageStar, SetArray, Star
+    ctx = _CountingCtx()
+    raw = (C.c_void_p * 5)(11, 12, 13, 14, 15)
+    arr = SetArray(ctx, raw, [None, (2, 2, 1), None, None, None])
+    assert len(arr) == 5 and arr._items is None            # nothing wrapped yet
+    assert arr.handles() is raw
+    b = arr[1]
+    assert isinstance(b, ImageStar) and (b.height, b.width, b.numChannel) == (2, 2, 1)
+    assert arr[1] is b and arr[-4] is b                     # one object per element
+    e = arr[-1]
+    assert type(e) is Star and e._h.h == 15
+    with pytest.raises(IndexError):
+        arr[5]
+    assert [s._h.h for s in arr[2:4]] == [13, 14]           # a slice is a plain list of the elements
+    del arr
+    gc.collect()
+    # the array released what nobody read (11), in one call; 13 and 14 died with the slice's list
+    assert ctx.bulk == [[11]]
+    assert sorted(ctx.single) == [13, 14]
+    del b, e
+    gc.collect()
+    assert sorted(ctx.single) == [12, 13, 14, 15]
+    # an array nobody looked into goes in one call
+    ctx2 = _CountingCtx()
+    arr2 = SetArray(ctx2, (C.c_void_p * 3)(1, 2, 3))
+    assert [type(s) for s in arr2] == [Star] * 3 and ctx2.single == []
+    arr3 = SetArray(ctx2, (C.c_void_p * 3)(4, 5, 6))
+    del arr3
+    gc.collect()
+    assert ctx2.bulk == [[4, 5, 6]]
