@@ -621,7 +621,7 @@ int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb,
   const ConsNode* node = s->cons.get();
   int64_t m = s->n_crossing;
   if (m > 0) {
-    if (index) NNV_HIP_TRY(hipMemcpyAsync(index, node->index->ptr, sizeof(int32_t) * m, hipMemcpyDeviceToHost, c->stream));
+    if (index) NNV_HIP_TRY(hipMemcpyAsync(index, node->index->as<int32_t>() + node->index_off, sizeof(int32_t) * m, hipMemcpyDeviceToHost, c->stream));
     const double* lbub = node->lbub->as<double>() + node->lbub_off;
     if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb, lbub, sizeof(double) * m, hipMemcpyDeviceToHost, c->stream));
     if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub, lbub + node->ld_lbub, sizeof(double) * m, hipMemcpyDeviceToHost, c->stream));

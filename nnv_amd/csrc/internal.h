@@ -11,6 +11,7 @@
 #include <map>
 #include <memory>
 #include <string>
+#include <unordered_set>
 #include <vector>
 
 #include "nnvhip.h"
@@ -80,7 +81,8 @@ struct ConsNode {
   BufRef lbub;                   // lb[0..m), then ub[0..m) at offset ld_lbub; data starts at lbub_off
   int64_t lbub_off = 0;
   int64_t ld_lbub = 0;
-  BufRef index;                  // int32[m]: crossing neuron indices in new-predicate order
+  BufRef index;                  // crossing neuron indices in new-predicate order: int32[m] at index_off
+  int64_t index_off = 0;
 };
 using ConsRef = std::shared_ptr<ConsNode>;
 

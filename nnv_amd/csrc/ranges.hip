@@ -336,12 +336,9 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   // sets that already carry ranges are skipped
   std::vector<nnvhip_star*> todo;
+  std::unordered_set<nnvhip_star*> seen;
   for (int64_t i = 0; i < count; ++i)
-    if (!s[i]->lb) {
-      bool dup = false;
-      for (auto* t : todo) dup = dup || t == s[i];
-      if (!dup) todo.push_back(s[i]);
-    }
+    if (!s[i]->lb && seen.insert(s[i]).second) todo.push_back(s[i]);
   if (todo.empty()) return NNVHIP_OK;
   NNV_TRY(ensure_dense_batch(ctx, (int64_t)todo.size(), todo.data()));  // the scan reads every column
   const int64_t nset = (int64_t)todo.size();

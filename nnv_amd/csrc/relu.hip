@@ -638,10 +638,11 @@ static int write_tail_columns(nnvhip_ctx* ctx, nnvhip_star* s) {
 int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail) {
   // sets with a pending row reset: one arena and one apply launch per leading dimension
   std::vector<nnvhip_star*> pend;
+  std::unordered_set<nnvhip_star*> seen;
   for (int64_t i = 0; i < count; ++i) {
     nnvhip_star* s = sets[i];
     if (s->rows_pending) {
-      if (std::find(pend.begin(), pend.end(), s) == pend.end()) pend.push_back(s);
+      if (seen.insert(s).second) pend.push_back(s);
     } else if (need_tail && s->stored_cols() != s->n + 1) {
       NNV_TRY(write_tail_columns(ctx, s));
     }
@@ -747,10 +748,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
     NNV_TRY(ctx->alloc(sizeof(double) * 2 * ldr_max * count, &lbub_buf));
   }
-  std::vector<BufRef> idx_bufs(count);
+  // crossing lists of all sets in one buffer (they become the constraint nodes' index lists)
+  BufRef idx_buf;
+  NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &idx_buf));
   std::vector<ReluDesc> descs(count);
   for (int64_t i = 0; i < count; ++i) {
-    NNV_TRY(ctx->alloc(sizeof(int32_t) * ld, &idx_bufs[i]));
     ReluDesc& d = descs[i];
     d = ReluDesc{};
     if (fold_bounds) {
@@ -767,7 +769,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.plb_in = in[i]->plb;
     d.pub_in = in[i]->pub;
     d.cls = cls_buf->as<int32_t>() + ld * i;
-    d.cross_idx = idx_bufs[i]->as<int32_t>();
+    d.cross_idx = idx_buf->as<int32_t>() + ld * i;
     d.asc_idx = sorted ? asc_buf->as<int32_t>() + ld * i : nullptr;
     d.key = sorted ? key_buf->as<double>() + ld * i : nullptr;
     d.rank = sorted ? rank_buf->as<int32_t>() + ld * i : nullptr;
@@ -944,8 +946,8 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     o->n_crossing = d.m;
     if (d.m > 0) {  // the appended columns are the unit vectors of the crossing neurons
       o->oh_from = in[i]->n + 1;
-      o->oh_idx_buf = idx_bufs[i];
-      o->oh_idx = idx_bufs[i]->as<int32_t>();
+      o->oh_idx_buf = idx_buf;
+      o->oh_idx = idx_buf->as<int32_t>() + ld * i;
       if (!eager_tail) o->vcols = in[i]->n + 1;  // ... and exist only as that list
     }
     // rows of the leading columns that were not reset
@@ -964,7 +966,8 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       node->src_ld = in[i]->ld;
       node->ld_lbub = d.ld_lbub;
       node->lbub = lbub_buf;
-      node->index = idx_bufs[i];
+      node->index = idx_buf;
+      node->index_off = ld * i;
       // views into shared buffers: keep element offsets
       node->lbub_off = lbub_off[i];
       o->cons = node;
@@ -1046,7 +1049,7 @@ int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host
       const double* lbp = nd->lbub->as<double>() + nd->lbub_off;
       dim3 grid((unsigned)ceil_div(nd->m, 128), (unsigned)std::min<int64_t>(nd->n_before + 1, 1024));
       hipLaunchKernelGGL(cons_relu_kernel, grid, dim3(128), 0, ctx->stream, Cuse, ldC, dd->as<double>(), r0, (int)nd->m,
-                         (int)nd->n_before, rows, nd->src_ld, nd->index->as<int32_t>(), lbp, lbp + nd->ld_lbub);
+                         (int)nd->n_before, rows, nd->src_ld, nd->index->as<int32_t>() + nd->index_off, lbp, lbp + nd->ld_lbub);
       r0 += 3 * nd->m;
     }
   }
