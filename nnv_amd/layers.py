@@ -62,6 +62,11 @@ def _shapes(sets):
 def _wrap_like(inputs, ctx, raw, out_shape=None):
     """The output array for the handles `raw`: a Star for a Star input, an ImageStar of `out_shape`
     (default: the input's own shape) for an ImageStar input."""
+    if len(raw) == 1 and not isinstance(inputs, SetArray):   # one set: the object is wanted right away
+        s, hd = inputs[0], _Handle(raw[0], ctx)
+        if isinstance(s, ImageStar):
+            return [ImageStar(_handle=hd, shape=out_shape or (s.height, s.width, s.numChannel))]
+        return [Star._from_handle(hd)]
     shp = _shapes(inputs)
     if shp is not None and out_shape is not None:
         shp = [None if s is None else out_shape for s in shp]
@@ -323,7 +328,7 @@ class PosLin:
                 out = (C.c_void_p * len(sets))()
                 check(ctx.lib.nnvhip_relu_relax(ctx.handle, RELAX_ORDER[method], float(relaxFactor), len(sets),
                                                 _handles_array(sets), out))
-                res = SetArray(ctx, out)
+                res = SetArray(ctx, out) if len(sets) > 1 or lazy else [Star._from_handle(_Handle(out[0], ctx))]
             else:
                 # some bounds are tightened by LPs first: host LP solver fed from the resident set
                 res = [PosLin.reach_relaxed_star_lp(s, method, relaxFactor, option, dis_opt, lp_solver) for s in sets]
