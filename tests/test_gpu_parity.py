@@ -484,3 +484,45 @@ def test_ranges_of_an_array_in_one_call(nnv, oracle):
     assert_close(lb[:, 0], lbs[:, 0], "image lb")          # centre -/+ half-width: equal up to rounding
     assert_close(ub[:, 0], ubs[:, 0], "image ub")
     assert nnv.Star.estimateRanges_array([])[0].size == 0
+
+
+def test_more_sets_than_mailbox_words_and_the_array_limit(nnv, oracle):
+    """Arrays beyond 8192 sets read their counts back through a copy instead of the per-set mailbox
+    words; the result must not depend on which way the counts travel.  Beyond 65535 sets a call is
+    refused with a shape error."""
+    rs = np.random.RandomState(77)
+    n_in, hidden, count = 4, 24, 8300
+    W1, b1 = rs.randn(hidden, n_in), 0.3 * rs.randn(hidden)
+    W2, b2 = rs.randn(3, hidden), 0.1 * rs.randn(3)
+    centre = rs.rand(n_in, count)
+    half = 0.05 + 0.2 * rs.rand(n_in, count)
+    lbs, ubs = centre - half, centre + half
+    net = nnv.NN([nnv.FullyConnectedLayer(W1, b1), nnv.ReluLayer(), nnv.FullyConnectedLayer(W2, b2)])
+    opt = {"reachMethod": "relax-star-area", "relaxFactor": 1}
+    outs = net.reach(nnv.Star.from_boxes(lbs, ubs), opt)
+    assert len(outs) == count
+    lb_all, ub_all = nnv.Star.estimateRanges_array(outs)
+    layers = [{"type": "fc", "W": W1, "b": b1}, {"type": "relu"}, {"type": "fc", "W": W2, "b": b2}]
+    for i in list(range(0, count, 517)) + [8191, 8192, count - 1]:
+        E = oracle.nn_reach(layers, oracle.star_from_box(lbs[:, i], ubs[:, i]), "relax-star-area", 1.0)
+        R = outs[i]
+        assert R.nVar == E.nVar
+        assert_close(np.asarray(R.V), E.V, "V of set %d" % i, RTOL)
+        elb, eub = oracle.estimate_ranges(E)
+        assert_close(lb_all[:, i], elb, "lb of set %d" % i, RTOL)
+        assert_close(ub_all[:, i], eub, "ub of set %d" % i, RTOL)
+        assert np.array_equal(np.asarray(R.C), E.C) or np.allclose(np.asarray(R.C), E.C, rtol=RTOL, atol=0)
+    # the same sets in two smaller arrays (mailbox route): every set's bounds agree (the launch shapes,
+    # hence the summation order of the products, differ with the array length)
+    lo = net.reach(nnv.Star.from_boxes(lbs[:, :4150], ubs[:, :4150]), opt)
+    hi = net.reach(nnv.Star.from_boxes(lbs[:, 4150:], ubs[:, 4150:]), opt)
+    lb_lo, ub_lo = nnv.Star.estimateRanges_array(lo)
+    lb_hi, ub_hi = nnv.Star.estimateRanges_array(hi)
+    assert_close(np.hstack([lb_lo, lb_hi]), lb_all, "lb, split arrays", RTOL)
+    assert_close(np.hstack([ub_lo, ub_hi]), ub_all, "ub, split arrays", RTOL)
+    assert [s.nVar for s in lo] + [s.nVar for s in hi] == [s.nVar for s in outs]
+    # too many sets for one call
+    big = 65536
+    tiny_lb = np.tile(np.array([[0.0], [0.1]]), (1, big))
+    with pytest.raises(ValueError):
+        nnv.ReluLayer().reach(nnv.Star.from_boxes(tiny_lb - 0.5, tiny_lb + 0.5), "relax-star-area", None, 1)
