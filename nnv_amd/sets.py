@@ -190,20 +190,22 @@ class Box:
                 raise ValueError("The %d^th index in part_indexes array is invalid" % (i + 1))
             if num < 1:
                 raise ValueError("The %d^th number in part_numbers array is invalid" % (i + 1))
-        lbs = self.lb.reshape(-1, 1).copy()
-        ubs = self.ub.reshape(-1, 1).copy()
+        # one box per row while they are made; the transposed views returned are column-major dim x count,
+        # the layout the device constructor takes (a box is a contiguous column)
+        lbs = self.lb.reshape(1, -1).copy()
+        ubs = self.ub.reshape(1, -1).copy()
         for ix, num in zip(part_indexes, part_numbers):
             if num == 1:
                 continue
-            delta = (ubs[ix, :] - lbs[ix, :]) / num                        # one delta per current box
+            delta = (ubs[:, ix] - lbs[:, ix]) / num                        # one delta per current box
             i = np.arange(1, num + 1, dtype=np.float64)
-            new_lb = lbs[ix, :, None] + (i[None, :] - 1) * delta[:, None]  # box-major, part-minor
+            new_lb = lbs[:, ix, None] + (i[None, :] - 1) * delta[:, None]  # box-major, part-minor
             new_ub = new_lb + delta[:, None]
-            lbs = np.repeat(lbs, num, axis=1)
-            ubs = np.repeat(ubs, num, axis=1)
-            lbs[ix, :] = new_lb.reshape(-1)
-            ubs[ix, :] = new_ub.reshape(-1)
-        return lbs, ubs
+            lbs = np.repeat(lbs, num, axis=0)
+            ubs = np.repeat(ubs, num, axis=0)
+            lbs[:, ix] = new_lb.reshape(-1)
+            ubs[:, ix] = new_ub.reshape(-1)
+        return lbs.T, ubs.T
 
     def toStar(self, ctx=None):
         return Star(self.lb, self.ub, ctx=ctx)
@@ -298,13 +300,8 @@ class Star:
         N, count = lbs.shape
         out = (C.c_void_p * count)()
         check(ctx.lib.nnvhip_star_from_box(ctx.handle, N, count, ptr(lbs), ptr(ubs), out))
-        stars = []
-        for i, h in enumerate(_make_handles(ctx, out)):
-            s = Star(_handle=h)
-            s.state_lb = lbs[:, i].copy()
-            s.state_ub = ubs[:, i].copy()
-            stars.append(s)
-        return stars
+        # state_lb / state_ub of the elements (set/Star.m:232-233) are columns of private copies
+        return SetArray(ctx, out, state=(lbs.copy(order="F"), ubs.copy(order="F")))
 
     # ---- NNV properties ------------------------------------------------------------------
     @property
@@ -601,13 +598,14 @@ class SetArray(collections.abc.Sequence):
     set; indexing, iteration, ``len`` and slicing (a plain list of the elements) behave as for a list.
     """
 
-    __slots__ = ("ctx", "_raw", "_shapes", "_items")
+    __slots__ = ("ctx", "_raw", "_shapes", "_items", "_state")
 
-    def __init__(self, ctx, raw, shapes=None):
+    def __init__(self, ctx, raw, shapes=None, state=None):
         self.ctx = ctx
         self._raw = raw          # ctypes array of handles; this object owns one reference of each
         self._shapes = shapes    # None: Stars only; else per element None (Star) or (height, width, numChannel)
         self._items = None       # the elements read so far (each then owns its handle's reference)
+        self._state = state      # None, or (lb, ub) matrices whose column i is element i's state_lb / state_ub
 
     def __len__(self):
         return len(self._raw)
@@ -627,6 +625,9 @@ class SetArray(collections.abc.Sequence):
             hd = _Handle(self._raw[i], self.ctx)
             shape = None if self._shapes is None else self._shapes[i]
             it = Star._from_handle(hd) if shape is None else ImageStar(_handle=hd, shape=shape)
+            if self._state is not None:
+                it.state_lb = self._state[0][:, i]
+                it.state_ub = self._state[1][:, i]
             self._items[i] = it
         return it
 

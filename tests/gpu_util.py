@@ -80,7 +80,7 @@ def run_both(k, method="relax-star-area", shrink=1, check_constraints=True, marg
     net = NN.from_config(cfg["layers"], cfg["name"])
     dev_out = net.reach(dev_in, {"reachMethod": method, "relaxFactor": 1})
     ora_out, ora_sets = o.nn_reach(cfg["layers"], ora_in, method, 1.0, keep=True)
-    batched = isinstance(dev_in, list)
+    batched = not isinstance(dev_in, (Star, ImageStar))
     for li, (L, dset, oset) in enumerate(zip(cfg["layers"], net.reachSet, ora_sets)):
         dl = dset if batched else [dset]
         ol = oset if batched else [oset]
