@@ -937,7 +937,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         if (compact && pack) {
           st = c->alloc(sizeof(double) * kp * dense[0], &packed);
           if (st == NNVHIP_OK) {
-            PackSet ps{in[0]->V, in[0]->kept_idx, packed->as<double>(), in[0]->ld, (int32_t)kp, (int32_t)dense[0]};
+            PackSet ps = pack_of(in[0], in[0]->kept_idx, packed->as<double>(), kp, dense[0]);
             st = launch_pack_rows(c, 1, &ps);
             rows.Bk = packed->as<double>();
             rows.ldbk = kp;
@@ -1024,8 +1024,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
             if (pk[i]) {
               bk[i] = packed->as<double>() + pos;
-              packs.push_back(PackSet{in[i]->V, rws[i].kmap, packed->as<double>() + pos, in[i]->ld, (int32_t)kps[i],
-                                      (int32_t)dense[i]});
+              packs.push_back(pack_of(in[i], rws[i].kmap, packed->as<double>() + pos, kps[i], dense[i]));
               pos += kps[i] * dense[i];
             }
           if (st == NNVHIP_OK && !packs.empty()) st = launch_pack_rows(c, (int64_t)packs.size(), packs.data());
@@ -1109,7 +1108,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         if (compact && pack) {
           st = c->alloc(sizeof(double) * kp * dense[i], &packed);
           if (st != NNVHIP_OK) break;
-          PackSet ps{in[i]->V, in[i]->kept_idx, packed->as<double>(), in[i]->ld, (int32_t)kp, (int32_t)dense[i]};
+          PackSet ps = pack_of(in[i], in[i]->kept_idx, packed->as<double>(), kp, dense[i]);
           st = launch_pack_rows(c, 1, &ps);
           if (st != NNVHIP_OK) break;
           rows.Bk = packed->as<double>();
@@ -1120,6 +1119,20 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         if (st == NNVHIP_OK && gs[i].m > 0) st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[i]->ld, 1, &gs[i], 0);
       }
     }
+    // the gathered columns remember where they came from
+    for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+      if (gs[i].m > 0) {
+        nnvhip_star* o = outs[i];
+        o->wsrc_buf = fc->W;
+        o->wsrc = Wd;
+        o->wsrc_ld = fc->Mp;
+        o->wsrc_idx_buf = in[i]->oh_idx_buf;
+        o->wsrc_idx = gs[i].idx;
+        o->wsrc_scale_buf = in[i]->oh_scale_buf;
+        o->wsrc_scale = gs[i].scale;
+        o->wsrc_from = dense[i];
+        o->wsrc_cols = gs[i].m;
+      }
   }
   if (st == NNVHIP_OK) st = c->end_op();
   if (st != NNVHIP_OK) {

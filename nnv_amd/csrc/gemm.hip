@@ -445,16 +445,38 @@ __global__ __launch_bounds__(512) void pack_rows_kernel(const PackSet* __restric
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       v[u] = make_double2(0.0, 0.0);
-      if (jb + u < j1) {
-        const double* col = d.V + (int64_t)(jb + u) * d.ld;
-        if (ra >= 0) v[u].x = col[ra];
-        if (rb >= 0) v[u].y = col[rb];
+      const int j = jb + u;
+      if (j < j1) {
+        if (d.W != nullptr && j >= d.wfrom && j < d.wend) {  // the value the gather pass wrote, recomputed
+          const int src = d.widx[j - d.wfrom];
+          const double sc = d.wscale ? d.wscale[src] : 1.0;
+          const double* col = d.W + (int64_t)src * d.ldw;
+          if (ra >= 0) v[u].x = __dadd_rn(0.0, __dmul_rn(col[ra], sc));
+          if (rb >= 0) v[u].y = __dadd_rn(0.0, __dmul_rn(col[rb], sc));
+        } else {
+          const double* col = d.V + (int64_t)j * d.ld;
+          if (ra >= 0) v[u].x = col[ra];
+          if (rb >= 0) v[u].y = col[rb];
+        }
       }
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u)
       if (jb + u < j1) *reinterpret_cast<double2*>(d.Vk + t0 + (int64_t)(jb + u) * d.kp) = v[u];
   }
+}
+
+PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t kp, int64_t ncols) {
+  PackSet p{s->V, kept, dst, s->ld, (int32_t)kp, (int32_t)ncols};
+  if (s->wsrc != nullptr && s->wsrc_from < ncols) {
+    p.W = s->wsrc;
+    p.ldw = s->wsrc_ld;
+    p.widx = s->wsrc_idx;
+    p.wscale = s->wsrc_scale;
+    p.wfrom = (int32_t)s->wsrc_from;
+    p.wend = (int32_t)std::min<int64_t>(ncols, s->wsrc_from + s->wsrc_cols);
+  }
+  return p;
 }
 
 int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {

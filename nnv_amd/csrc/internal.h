@@ -210,6 +210,17 @@ struct nnvhip_star {
   const double* rng_part = nullptr;
   int64_t rng_chunks = 0;
   int64_t rng_first_col = 0;
+  // Where an FC map gathered the stored columns [wsrc_from, wsrc_from + wsrc_cols) from: column
+  // wsrc_from + t holds 0 + wsrc[:, r] * wsrc_scale[r] with r = wsrc_idx[t] (wsrc_scale == null: scale 1),
+  // wsrc being that layer's weight matrix.  A later packing of kept rows reads the (cache-resident) weight
+  // matrix instead of this set's own matrix in HBM.  wsrc == null: no such knowledge.
+  nnvhip::BufRef wsrc_buf, wsrc_idx_buf, wsrc_scale_buf;
+  const double* wsrc = nullptr;
+  int64_t wsrc_ld = 0;
+  const int32_t* wsrc_idx = nullptr;
+  const double* wsrc_scale = nullptr;
+  int64_t wsrc_from = 0;
+  int64_t wsrc_cols = 0;
 };
 
 struct nnvhip_fc {
@@ -292,7 +303,16 @@ struct PackSet {
   int64_t ld;
   int32_t kp;
   int32_t ncols;
+  // columns [wfrom, wend) are read as 0 + W(:, widx[j - wfrom]) * wscale[...] instead (W == null: none)
+  const double* W = nullptr;
+  int64_t ldw = 0;
+  const int32_t* widx = nullptr;
+  const double* wscale = nullptr;
+  int32_t wfrom = 0;
+  int32_t wend = 0;
 };
+// the packing of the first `ncols` columns of a set, with what is known about where they came from
+PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t kp, int64_t ncols);
 int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
 // A split-K product leaves `ksplit` partial matrices (Mp x ncols each, ld = Mp) in a workspace; a caller
 // that has a pass over the output coming anyway can take the workspace instead of having the reduction

@@ -689,6 +689,10 @@ int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets,
       s->rows_pending = false;
       s->cls_buf.reset();
       s->cls = nullptr;
+      s->wsrc = nullptr;  // the reset rows no longer match the weight columns
+      s->wsrc_buf.reset();
+      s->wsrc_idx_buf.reset();
+      s->wsrc_scale_buf.reset();
       if (need_tail) s->vcols = -1;
     }
     pend.swap(rest);
@@ -935,6 +939,16 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->rows_pending = true;
       o->cls_buf = cls_buf;
       o->cls = cls_buf->as<int32_t>() + ld * i;
+      // ... and what is known about where its columns came from holds for the rows that are kept
+      o->wsrc_buf = in[i]->wsrc_buf;
+      o->wsrc = in[i]->wsrc;
+      o->wsrc_ld = in[i]->wsrc_ld;
+      o->wsrc_idx_buf = in[i]->wsrc_idx_buf;
+      o->wsrc_idx = in[i]->wsrc_idx;
+      o->wsrc_scale_buf = in[i]->wsrc_scale_buf;
+      o->wsrc_scale = in[i]->wsrc_scale;
+      o->wsrc_from = in[i]->wsrc_from;
+      o->wsrc_cols = in[i]->wsrc_cols;
     } else {
       o->Vbuf = arena;
       o->V = d.Vout;
