@@ -80,6 +80,14 @@ NNVHIP_API int nnvhip_last_op_time_ms(nnvhip_ctx* ctx, double* ms);
  * reference's Star.affineMap (set/Star.m:313-343) executes it.  Initial value: 1 if the environment
  * variable NNVHIP_DENSE_AFFINE is set, else 0. */
 NNVHIP_API int nnvhip_set_dense_affine(nnvhip_ctx* ctx, int enabled);
+/* Output switch of nnvhip_affine_fc (no counterpart in the reference, where every affineMap writes its
+ * whole result, set/Star.m:313-343).  By default the columns an FC map gathers from its weight matrix
+ * are described on the output handle and written only when somebody reads them (a property read, a
+ * layer that needs the whole matrix): the ReLU step that follows works from the range sums the map
+ * leaves behind, and the FC map after that packs its rows from the weights.  enabled = 1 writes them
+ * in the call itself; a caller does that for the layer whose output it hands on (NN.reach's return
+ * value, nn/NN.m:1529-1551).  Initial value: 1 if the environment variable NNVHIP_EAGER_COLS is set. */
+NNVHIP_API int nnvhip_set_eager_columns(nnvhip_ctx* ctx, int enabled);
 /* Measurement hook (no counterpart in the reference): while timing level 2 is set, every launch of a
  * kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
  * dense GEMM kernel of the FC layers (tiles of at least 64 rows); 1: implicit-GEMM convolution

@@ -184,6 +184,8 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->dense_affine = getenv("NNVHIP_DENSE_AFFINE") != nullptr;
   c->eager_tail = getenv("NNVHIP_EAGER_TAIL") != nullptr;
   c->eager_rows = getenv("NNVHIP_EAGER_ROWS") != nullptr;
+  c->eager_cols = getenv("NNVHIP_EAGER_COLS") != nullptr;
+  c->poison_pending = getenv("NNVHIP_POISON_PENDING") != nullptr;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
@@ -229,6 +231,12 @@ int nnvhip_set_timing(nnvhip_ctx* c, int enabled) {
 int nnvhip_set_dense_affine(nnvhip_ctx* c, int enabled) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
   c->dense_affine = enabled != 0;
+  return NNVHIP_OK;
+}
+
+int nnvhip_set_eager_columns(nnvhip_ctx* c, int enabled) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  c->eager_cols = enabled != 0;
   return NNVHIP_OK;
 }
 
@@ -860,14 +868,14 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.bias = nullptr;
       g.red = nullptr;
       g.red_k = 0;
-      g.pad_ = 0;
+      g.lazy = 0;
       g.centre = nullptr;
     }
     // sets whose implicit unit-vector columns take part in the contraction after all get them written out
     // (which also runs a pending row reset)
     std::vector<nnvhip_star*> full;
     for (int64_t i = 0; i < count; ++i)
-      if (dense[i] > in[i]->stored_cols() || (dense_only && in[i]->rows_pending)) full.push_back(in[i]);
+      if (dense[i] > in[i]->stored_cols() || (dense_only && (in[i]->rows_pending || in[i]->cs.any_pending()))) full.push_back(in[i]);
     if (!full.empty()) {
       st = ensure_dense_batch(c, (int64_t)full.size(), full.data());
       contig = true;  // the sets moved: look again
@@ -910,6 +918,26 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       gs[i].fill = outs[i]->V;
       gs[i].bias = bias;
     };
+    // Inputs with columns that are described but not in memory yet: the contraction reads them from
+    // memory unless it goes over no row at all or through the packing pass (which takes such columns
+    // from the weights they were gathered from).  Everybody else has them written now.
+    if (st == NNVHIP_OK) {
+      std::vector<nnvhip_star*> cols;
+      for (int64_t i = 0; i < count; ++i) {
+        if (!in[i]->cs.any_pending()) continue;
+        GemmRows r;
+        int64_t kp = 0;
+        bool pack = false;
+        const bool compact = rows_of(i, &r, &kp, &pack);
+        if (!(compact && (nothing_kept(i, r) || (pack && r.kmap != nullptr)))) cols.push_back(in[i]);
+      }
+      if (!cols.empty()) st = write_pending_columns(c, (int64_t)cols.size(), cols.data());
+    }
+    // Gathered columns whose range sums this call leaves behind are not written: the ReLU step that
+    // follows works from the sums, and the next FC map either contracts over no row or packs its rows
+    // from the weights.  lazy[i] is set where the sums are produced.
+    std::vector<char> lazy((size_t)count, 0);
+    const bool lazy_ok = !c->eager_cols && !dense_only;
     if (count == 1) {
       // one set: the GEMM epilogue also leaves the partial sums of Star.estimateRanges, so the
       // output set carries its ranges without another pass over V
@@ -929,6 +957,8 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         if (gs[0].m > 0) {
           st = c->alloc(sizeof(double) * 4 * outs[0]->ld * ch, &part);
           if (st == NNVHIP_OK) gs[0].part = part->as<double>();
+          lazy[0] = lazy_ok;
+          gs[0].lazy = lazy[0];
         }
         if (st == NNVHIP_OK) st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), gs[0].m > 0 ? ch : 0);
         if (st == NNVHIP_OK && gs[0].m > 0) st = finalize_fused_ranges(c, outs[0], part, ch);
@@ -962,6 +992,8 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         const bool fused = st == NNVHIP_OK && (fuse.chunks > 0 || centre_only);
         if (st == NNVHIP_OK && gs[0].m > 0) {
           gs[0].part = fused ? fuse.part->as<double>() + fuse.chunks * 4 * outs[0]->ld : nullptr;
+          lazy[0] = lazy_ok && fused;
+          gs[0].lazy = lazy[0];
           st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? gch : 0);
         }
         if (st == NNVHIP_OK && fused) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0));
@@ -1079,8 +1111,11 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         BufRef sums;
         if (gch > 0) st = c->alloc(sizeof(double) * 4 * outs[0]->ld * gch * count, &sums);
         if (st == NNVHIP_OK) {
-          for (int64_t i = 0; i < count; ++i)
+          for (int64_t i = 0; i < count; ++i) {
             gs[i].part = (gch > 0 && gs[i].m > 0) ? sums->as<double>() + 4 * outs[0]->ld * gch * i : nullptr;
+            lazy[i] = lazy_ok && gs[i].part != nullptr;
+            gs[i].lazy = lazy[i];
+          }
           st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, count, gs.data(), gch);
         }
         for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
@@ -1123,15 +1158,27 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
     for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
       if (gs[i].m > 0) {
         nnvhip_star* o = outs[i];
-        o->wsrc_buf = fc->W;
-        o->wsrc = Wd;
-        o->wsrc_ld = fc->Mp;
-        o->wsrc_idx_buf = in[i]->oh_idx_buf;
-        o->wsrc_idx = gs[i].idx;
-        o->wsrc_scale_buf = in[i]->oh_scale_buf;
-        o->wsrc_scale = gs[i].scale;
-        o->wsrc_from = dense[i];
-        o->wsrc_cols = gs[i].m;
+        ColSource& cs = o->cs;
+        cs.W_buf = fc->W;
+        cs.W = Wd;
+        cs.ldw = fc->Mp;
+        cs.rows = fc->Mp;
+        cs.idx_buf = in[i]->oh_idx_buf;
+        cs.idx = gs[i].idx;
+        cs.scale_buf = in[i]->oh_scale_buf;
+        cs.scale = gs[i].scale;
+        cs.from = dense[i];
+        cs.cols = gs[i].m;
+        cs.pending = lazy[i] != 0;
+        cs.zero_to = (lazy[i] && gs[i].nfill > 0) ? gs[i].nfill : 0;  // a filled set's leading columns
+        // debugging aid: NaNs where nothing was written, so that a reader that forgets to ask for the
+        // columns cannot pass a test on what an earlier call happened to leave in the memory
+        auto poison = [&](double* p, int64_t ncols) -> int {
+          NNV_HIP_TRY(hipMemsetAsync(p, 0xff, sizeof(double) * o->ld * ncols, c->stream));
+          return NNVHIP_OK;
+        };
+        if (c->poison_pending && cs.pending) st = poison(o->V + cs.from * o->ld, cs.cols);
+        if (c->poison_pending && cs.zero_to > 1 && st == NNVHIP_OK) st = poison(o->V + o->ld, cs.zero_to - 1);
       }
   }
   if (st == NNVHIP_OK) st = c->end_op();
@@ -1179,7 +1226,7 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
       const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
       if (dense > in[i]->stored_cols())
         full.push_back(in[i]);
-      else if (in[i]->rows_pending)
+      else if (in[i]->rows_pending || in[i]->cs.any_pending())
         prefix.push_back(in[i]);
     }
     if (st == NNVHIP_OK && !full.empty()) st = ensure_dense_batch(c, (int64_t)full.size(), full.data());

@@ -446,7 +446,7 @@ __global__ __launch_bounds__(512) void pack_rows_kernel(const PackSet* __restric
     for (int u = 0; u < 4; ++u) {
       v[u] = make_double2(0.0, 0.0);
       const int j = jb + u;
-      if (j < j1) {
+      if (j < j1 && !(j >= 1 && j < d.zero_to)) {
         if (d.W != nullptr && j >= d.wfrom && j < d.wend) {  // the value the gather pass wrote, recomputed
           const int src = d.widx[j - d.wfrom];
           const double sc = d.wscale ? d.wscale[src] : 1.0;
@@ -468,14 +468,16 @@ __global__ __launch_bounds__(512) void pack_rows_kernel(const PackSet* __restric
 
 PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t kp, int64_t ncols) {
   PackSet p{s->V, kept, dst, s->ld, (int32_t)kp, (int32_t)ncols};
-  if (s->wsrc != nullptr && s->wsrc_from < ncols) {
-    p.W = s->wsrc;
-    p.ldw = s->wsrc_ld;
-    p.widx = s->wsrc_idx;
-    p.wscale = s->wsrc_scale;
-    p.wfrom = (int32_t)s->wsrc_from;
-    p.wend = (int32_t)std::min<int64_t>(ncols, s->wsrc_from + s->wsrc_cols);
+  const ColSource& cs = s->cs;
+  if (cs.W != nullptr && cs.from < ncols) {
+    p.W = cs.W;
+    p.ldw = cs.ldw;
+    p.widx = cs.idx;
+    p.wscale = cs.scale;
+    p.wfrom = (int32_t)cs.from;
+    p.wend = (int32_t)std::min<int64_t>(ncols, cs.from + cs.cols);
   }
+  p.zero_to = (int32_t)std::min<int64_t>(ncols, cs.zero_to);
   return p;
 }
 

@@ -60,6 +60,27 @@ struct Buffer {
 };
 using BufRef = std::shared_ptr<Buffer>;
 
+// Where an FC map gathered stored columns of a set from, and whether they are in memory yet.  Column
+// from + t holds 0 + W(:, r) * scale[r] with r = idx[t] (scale == null: 1).  A later packing of kept rows
+// reads the cache-resident weight matrix instead of the set's own matrix in HBM; and the FC map may leave
+// the columns unwritten (`pending`) when it has left their range sums behind: nothing on the way to the
+// next layers reads them then, and whoever does (a host read, a layer that needs the whole matrix) has
+// them written first.  Writing them is idempotent, so every handle that shares the matrix keeps a copy
+// of this description with its own flags.  W == null: no such knowledge.
+struct ColSource {
+  BufRef W_buf, idx_buf, scale_buf;
+  const double* W = nullptr;  // the layer's weight matrix: `rows` rows (a multiple of 16), leading dimension ldw
+  int64_t ldw = 0;
+  int64_t rows = 0;
+  const int32_t* idx = nullptr;
+  const double* scale = nullptr;
+  int64_t from = 0;
+  int64_t cols = 0;
+  bool pending = false;  // the columns [from, from + cols) are not in memory yet
+  int64_t zero_to = 0;   // > 1: the columns [1, zero_to) are +0 and not in memory yet
+  bool any_pending() const { return pending || zero_to > 1; }
+};
+
 // One node per ReLU layer of the structured constraint store.  The dense NNV matrix
 // [C0; C1; C2; C3] (nn/funcs/PosLin.m:711-735) is only materialised when the host reads it.
 struct ConsNode {
@@ -78,6 +99,7 @@ struct ConsNode {
   BufRef src;                    // owner of the pre-ReLU generator matrix
   const double* src_V = nullptr; // its N x (n_before+1) matrix
   int64_t src_ld = 0;
+  ColSource src_cs;              // columns of it that may not be in memory yet
   BufRef lbub;                   // lb[0..m), then ub[0..m) at offset ld_lbub; data starts at lbub_off
   int64_t lbub_off = 0;
   int64_t ld_lbub = 0;
@@ -114,6 +136,10 @@ struct nnvhip_ctx {
   // ReLU outputs reset their rows at once instead of leaving that to the first reader that needs the
   // whole matrix (environment NNVHIP_EAGER_ROWS; implied by the two switches above)
   bool eager_rows = false;
+  // FC maps always write the columns they gather (environment NNVHIP_EAGER_COLS)
+  bool eager_cols = false;
+  // debugging aid (environment NNVHIP_POISON_PENDING): columns left unwritten are filled with NaNs
+  bool poison_pending = false;
   // per-layer timing
   bool timing = false;         // per-layer events (nnvhip_last_op_time_ms)
   bool kernel_timing = false;  // additionally one event pair per launch of the timed kernel groups
@@ -210,17 +236,8 @@ struct nnvhip_star {
   const double* rng_part = nullptr;
   int64_t rng_chunks = 0;
   int64_t rng_first_col = 0;
-  // Where an FC map gathered the stored columns [wsrc_from, wsrc_from + wsrc_cols) from: column
-  // wsrc_from + t holds 0 + wsrc[:, r] * wsrc_scale[r] with r = wsrc_idx[t] (wsrc_scale == null: scale 1),
-  // wsrc being that layer's weight matrix.  A later packing of kept rows reads the (cache-resident) weight
-  // matrix instead of this set's own matrix in HBM.  wsrc == null: no such knowledge.
-  nnvhip::BufRef wsrc_buf, wsrc_idx_buf, wsrc_scale_buf;
-  const double* wsrc = nullptr;
-  int64_t wsrc_ld = 0;
-  const int32_t* wsrc_idx = nullptr;
-  const double* wsrc_scale = nullptr;
-  int64_t wsrc_from = 0;
-  int64_t wsrc_cols = 0;
+  // where gathered columns came from, and whether they (and leading zero columns) are in memory yet
+  nnvhip::ColSource cs;
 };
 
 struct nnvhip_fc {
@@ -310,6 +327,7 @@ struct PackSet {
   const double* wscale = nullptr;
   int32_t wfrom = 0;
   int32_t wend = 0;
+  int32_t zero_to = 0;  // > 1: columns [1, zero_to) are +0 whatever the memory holds
 };
 // the packing of the first `ncols` columns of a set, with what is known about where they came from
 PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t kp, int64_t ncols);
@@ -367,9 +385,12 @@ struct GatherSet {
   const double* bias;   // or null
   const double* red;    // split-K partials of the centre column (red_k vectors of Mp entries) to be summed into
   int32_t red_k;        // `centre`, plus the bias; null / 0 = the centre is final
-  int32_t pad_;
+  int32_t lazy;         // 1: only the range sums (and column 0 of the fill) are produced, the columns stay unwritten
   double* centre;
 };
+// Writes the columns of the sets that are described but not in memory yet (see ColSource).
+int write_pending_columns(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets);
+int write_pending_columns(nnvhip_ctx* ctx, double* V, int64_t ld, ColSource* cs);
 int64_t gather_chunks(int64_t Mp, int64_t m);
 int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m);
 // chunks > 0: every set's `part` receives that many chunks (sets with part == null none); chunks = 0:
@@ -380,10 +401,12 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks);
 
 // relu.hip
-// Makes V a plain stored matrix: runs a pending row reset and, with need_tail, writes the implicit
+// Makes V a plain stored matrix: writes columns that are still pending (need_cols; always when one of
+// the other two steps reads them), runs a pending row reset and, with need_tail, writes the implicit
 // unit-vector columns, into a fresh buffer.  The batch form keeps the sets of an array back to back.
 int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s, bool need_tail = true);
-int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail = true);
+int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail = true,
+                       bool need_cols = true);
 // order: NNVHIP_ORDER_* (classification from the sets' estimated ranges), or kOrderGiven with one
 // ReluGiven per set: per-row bounds to classify by (ub <= 0: reset, lb < 0 < ub: crossing, else left
 // alone) and per-row keys whose descending order is the order of the new predicates.

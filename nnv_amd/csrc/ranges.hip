@@ -211,7 +211,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
         o.x = __dadd_rn(0.0, d.bias[r0]);
         o.y = __dadd_rn(0.0, d.bias[r0 + 1]);
       }
-      *reinterpret_cast<double2*>(d.fill + r0 + (int64_t)j * a.ldout) = o;
+      if (j == 0 || !d.lazy) *reinterpret_cast<double2*>(d.fill + r0 + (int64_t)j * a.ldout) = o;
     }
   }
   double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
         double2 o;
         o.x = __dadd_rn(0.0, __dmul_rn(v[u].x, sc[u]));
         o.y = __dadd_rn(0.0, __dmul_rn(v[u].y, sc[u]));
-        *reinterpret_cast<double2*>(d.out + r0 + (int64_t)j * a.ldout) = o;
+        if (!d.lazy) *reinterpret_cast<double2*>(d.out + r0 + (int64_t)j * a.ldout) = o;
         if (part != nullptr) {
           const double pl = d.plb[j], pu = d.pub[j];
           const double px = fmax(o.x, 0.0), nx = fmin(o.x, 0.0);
@@ -321,10 +321,12 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
     NNV_TRY(ctx->upload_table(sets, sizeof(GatherSet) * count, &tab));
     table = tab->as<GatherSet>();
   }
-  // algorithmic HBM bytes: every output column written once, W read once (its columns are re-read
-  // from cache)
+  // algorithmic HBM bytes: every output column that is written, once; W read once (its columns are
+  // re-read from cache); the range sums of a set whose columns stay unwritten
   double bytes = 8.0 * (double)Mp * (double)ldw;
-  for (int64_t i = 0; i < count; ++i) bytes += 8.0 * (double)Mp * (double)(sets[i].m + sets[i].nfill);
+  for (int64_t i = 0; i < count; ++i)
+    bytes += sets[i].lazy ? 8.0 * (double)Mp * (sets[i].nfill > 0 ? 1.0 : 0.0) + (with_sums && sets[i].part ? 32.0 * (double)ldout * (double)chunks : 0.0)
+                          : 8.0 * (double)Mp * (double)(sets[i].m + sets[i].nfill);
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
              dim3(64 * kRangeWaves), 0, table, sets[0], a);
@@ -340,7 +342,17 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   for (int64_t i = 0; i < count; ++i)
     if (!s[i]->lb && seen.insert(s[i]).second) todo.push_back(s[i]);
   if (todo.empty()) return NNVHIP_OK;
-  NNV_TRY(ensure_dense_batch(ctx, (int64_t)todo.size(), todo.data()));  // the scan reads every column
+  // The scan reads the columns the producer left no sums for.  Columns that are described but not in
+  // memory yet are written first only if they are among those (they normally come with their sums).
+  {
+    std::vector<nnvhip_star*> cols;
+    for (auto* t : todo) {
+      const int64_t scan_end = (t->rng_part != nullptr && t->rng_chunks > 0 && t->rng_first_col >= 1) ? t->rng_first_col : t->n + 1;
+      if ((t->cs.pending && scan_end > t->cs.from) || (t->cs.zero_to > 1 && scan_end > 1)) cols.push_back(t);
+    }
+    if (!cols.empty()) NNV_TRY(write_pending_columns(ctx, (int64_t)cols.size(), cols.data()));
+  }
+  NNV_TRY(ensure_dense_batch(ctx, (int64_t)todo.size(), todo.data(), true, false));
   const int64_t nset = (int64_t)todo.size();
   if (nset > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
   int64_t ld = todo[0]->ld;
@@ -455,6 +467,61 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
   s->lb = d.lb;
   s->ub = d.ub;
   return NNVHIP_OK;
+}
+
+// ---- columns an FC map described but did not write ------------------------------------------------
+namespace {
+struct PendingCols {
+  double* V;
+  int64_t ld;
+  ColSource* cs;
+};
+
+// One gather launch per run of sets that share the weight matrix and the leading dimension.
+int write_cols(nnvhip_ctx* ctx, std::vector<PendingCols>& todo) {
+  size_t a = 0;
+  while (a < todo.size()) {
+    size_t b = a + 1;
+    while (b < todo.size() && b - a < 65535 && todo[b].cs->W == todo[a].cs->W && todo[b].ld == todo[a].ld &&
+           todo[b].cs->ldw == todo[a].cs->ldw && todo[b].cs->rows == todo[a].cs->rows)
+      ++b;
+    std::vector<GatherSet> gs(b - a);
+    for (size_t i = a; i < b; ++i) {
+      const ColSource& cs = *todo[i].cs;
+      GatherSet& g = gs[i - a];
+      g = GatherSet{};
+      g.idx = cs.idx;
+      g.scale = cs.scale;
+      g.out = todo[i].V + cs.from * todo[i].ld;
+      g.m = cs.pending ? (int32_t)cs.cols : 0;
+      if (cs.zero_to > 1) {  // column 0 (the centre) is in memory already
+        g.nfill = (int32_t)(cs.zero_to - 1);
+        g.fill = todo[i].V + todo[i].ld;
+      }
+    }
+    const ColSource& c0 = *todo[a].cs;
+    NNV_TRY(launch_gather_columns(ctx, c0.W, c0.ldw, c0.rows, todo[a].ld, (int64_t)(b - a), gs.data(), 0));
+    for (size_t i = a; i < b; ++i) {
+      todo[i].cs->pending = false;
+      todo[i].cs->zero_to = 0;
+    }
+    a = b;
+  }
+  return NNVHIP_OK;
+}
+}  // namespace
+
+int write_pending_columns(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets) {
+  std::vector<PendingCols> todo;
+  for (int64_t i = 0; i < count; ++i)
+    if (sets[i]->cs.any_pending()) todo.push_back(PendingCols{sets[i]->V, sets[i]->ld, &sets[i]->cs});
+  return todo.empty() ? NNVHIP_OK : write_cols(ctx, todo);
+}
+
+int write_pending_columns(nnvhip_ctx* ctx, double* V, int64_t ld, ColSource* cs) {
+  if (!cs->any_pending()) return NNVHIP_OK;
+  std::vector<PendingCols> todo{PendingCols{V, ld, cs}};
+  return write_cols(ctx, todo);
 }
 
 }  // namespace nnvhip

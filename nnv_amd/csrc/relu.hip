@@ -635,7 +635,16 @@ static int write_tail_columns(nnvhip_ctx* ctx, nnvhip_star* s) {
   return NNVHIP_OK;
 }
 
-int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail) {
+int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets, bool need_tail, bool need_cols) {
+  // columns that were described but not written: wanted by the caller, or read by the steps below
+  {
+    std::vector<nnvhip_star*> cols;
+    for (int64_t i = 0; i < count; ++i) {
+      nnvhip_star* s = sets[i];
+      if (s->cs.any_pending() && (need_cols || s->rows_pending || (need_tail && s->stored_cols() != s->n + 1))) cols.push_back(s);
+    }
+    if (!cols.empty()) NNV_TRY(write_pending_columns(ctx, (int64_t)cols.size(), cols.data()));
+  }
   // sets with a pending row reset: one arena and one apply launch per leading dimension
   std::vector<nnvhip_star*> pend;
   std::unordered_set<nnvhip_star*> seen;
@@ -689,10 +698,7 @@ int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets,
       s->rows_pending = false;
       s->cls_buf.reset();
       s->cls = nullptr;
-      s->wsrc = nullptr;  // the reset rows no longer match the weight columns
-      s->wsrc_buf.reset();
-      s->wsrc_idx_buf.reset();
-      s->wsrc_scale_buf.reset();
+      s->cs = ColSource();  // the reset rows no longer match the weight columns
       if (need_tail) s->vcols = -1;
     }
     pend.swap(rest);
@@ -701,14 +707,19 @@ int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets,
 }
 
 int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s, bool need_tail) {
-  if (!s->rows_pending && (!need_tail || s->stored_cols() == s->n + 1)) return NNVHIP_OK;
+  if (!s->rows_pending && !s->cs.any_pending() && (!need_tail || s->stored_cols() == s->n + 1)) return NNVHIP_OK;
   return ensure_dense_batch(ctx, 1, &s, need_tail);
 }
 
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out, const ReluGiven* given) {
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
   if ((order == kOrderGiven) != (given != nullptr)) NNV_FAIL(NNVHIP_ERR_ARG, "internal: explicit lists and their order go together");
-  NNV_TRY(ensure_dense_batch(ctx, count, in));
+  // the appended unit-vector columns are stored only on request or when the FC / conv maps are told to
+  // contract over every column anyway; the row reset itself is left to whoever needs the whole matrix
+  const bool eager_tail = ctx->eager_tail || ctx->dense_affine;
+  const bool lazy_rows = !eager_tail && !ctx->eager_rows;
+  // (with the reset left pending nothing here reads the inputs' columns: those not written yet stay so)
+  NNV_TRY(ensure_dense_batch(ctx, count, in, true, !lazy_rows));
   if (given == nullptr) NNV_TRY(compute_ranges(ctx, count, in));
   const int64_t N = in[0]->N;
   const int64_t ld = in[0]->ld;
@@ -731,10 +742,6 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->alloc(sizeof(double) * ld * count, &key_buf));
     NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &rank_buf));
   }
-  // the appended unit-vector columns are stored only on request or when the FC / conv maps are told to
-  // contract over every column anyway; the row reset itself is left to whoever needs the whole matrix
-  const bool eager_tail = ctx->eager_tail || ctx->dense_affine;
-  const bool lazy_rows = !eager_tail && !ctx->eager_rows;
   // With the reset pending, all that is left to write are the predicate bounds and the crossing
   // neurons' (lb, ub).  The one-block classification does that itself, into buffers sized for the worst
   // case (every neuron crossing), and the step is a single launch.
@@ -939,16 +946,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->rows_pending = true;
       o->cls_buf = cls_buf;
       o->cls = cls_buf->as<int32_t>() + ld * i;
-      // ... and what is known about where its columns came from holds for the rows that are kept
-      o->wsrc_buf = in[i]->wsrc_buf;
-      o->wsrc = in[i]->wsrc;
-      o->wsrc_ld = in[i]->wsrc_ld;
-      o->wsrc_idx_buf = in[i]->wsrc_idx_buf;
-      o->wsrc_idx = in[i]->wsrc_idx;
-      o->wsrc_scale_buf = in[i]->wsrc_scale_buf;
-      o->wsrc_scale = in[i]->wsrc_scale;
-      o->wsrc_from = in[i]->wsrc_from;
-      o->wsrc_cols = in[i]->wsrc_cols;
+      // ... and what is known about where its columns came from (and whether they are in memory yet)
+      // holds for the rows that are kept
+      o->cs = in[i]->cs;
     } else {
       o->Vbuf = arena;
       o->V = d.Vout;
@@ -978,6 +978,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       node->src = in[i]->Vbuf;  // zero-copy: C2/C3 rows are rows of the input's immutable [c V]
       node->src_V = in[i]->V;
       node->src_ld = in[i]->ld;
+      node->src_cs = in[i]->cs;
       node->ld_lbub = d.ld_lbub;
       node->lbub = lbub_buf;
       node->index = idx_buf;
@@ -1059,6 +1060,9 @@ int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host
     } else {
       double* Cuse = Cp;
       const int64_t ldC = p;
+      // the crossing rows are read from the pre-ReLU matrix: columns of it that were never needed until
+      // now are written first (into the matrix itself; the node's copy of the description is updated)
+      NNV_TRY(write_pending_columns(ctx, const_cast<double*>(nd->src_V), nd->src_ld, const_cast<ColSource*>(&nd->src_cs)));
       const double* rows = nd->src_V;
       const double* lbp = nd->lbub->as<double>() + nd->lbub_off;
       dim3 grid((unsigned)ceil_div(nd->m, 128), (unsigned)std::min<int64_t>(nd->n_before + 1, 1024));

@@ -97,12 +97,22 @@ class NN:
         rs = inSet
         ctx = rs.ctx if isinstance(rs, SetArray) else (rs[0] if isinstance(rs, (list, tuple)) else rs).ctx
         timed = self.dis_opt == "display"
+        last = len(self.Layers) - 1
         for i, layer in enumerate(self.Layers):
             if timed:
                 print("Reachability for layer %d :" % (i + 1))
                 ctx.synchronize()
             t0 = time.perf_counter()
-            rs = layer.reach(rs, self.reachMethod, self.reachOption, self.relaxFactor, self.dis_opt, self.lp_solver)
+            # the set that is handed back is written in full by the layer that produces it (the sets in
+            # between write columns nobody reads only when somebody does)
+            eager = i == last and not ctx.eager_columns
+            if eager:
+                ctx.set_eager_columns(True)
+            try:
+                rs = layer.reach(rs, self.reachMethod, self.reachOption, self.relaxFactor, self.dis_opt, self.lp_solver)
+            finally:
+                if eager:
+                    ctx.set_eager_columns(False)
             if timed:
                 ctx.synchronize()
             self.reachTime[i] = time.perf_counter() - t0
