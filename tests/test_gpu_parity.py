@@ -526,3 +526,58 @@ def test_more_sets_than_mailbox_words_and_the_array_limit(nnv, oracle):
     tiny_lb = np.tile(np.array([[0.0], [0.1]]), (1, big))
     with pytest.raises(ValueError):
         nnv.ReluLayer().reach(nnv.Star.from_boxes(tiny_lb - 0.5, tiny_lb + 0.5), "relax-star-area", None, 1)
+
+
+@pytest.mark.parametrize("count", [1, 3])
+def test_columns_left_unwritten_are_written_on_any_first_read(nnv, oracle, count):
+    """An FC map describes the columns it gathers from its weights and writes them only when somebody
+    reads them.  Whatever is read first -- the FC output, the ReLU output that shares its matrix, the
+    constraint rows that are rows of it, or nothing before the next layers ran -- every read must give
+    the oracle's dense arrays, and exactly what the write-at-once mode gives."""
+    rs = np.random.RandomState(91)
+    n_in, h1, h2 = 100, 512, 256   # large enough for every FC map to gather (tiny products stay dense)
+    L = [{"type": "fc", "W": rs.randn(h1, n_in) * 0.4, "b": 0.2 * rs.randn(h1)}, {"type": "relu"},
+         {"type": "fc", "W": rs.randn(h2, h1) * 0.1, "b": 0.1 * rs.randn(h2)}, {"type": "relu"},
+         {"type": "fc", "W": rs.randn(6, h2) * 0.2, "b": 0.1 * rs.randn(6)}]
+    centre = rs.rand(n_in, count)
+    half = 0.02 + 0.05 * rs.rand(n_in, count)
+    lbs, ubs = centre - half, centre + half
+    ctx = nnv.default_context()
+    _, exp_sets = zip(*[oracle.nn_reach(L, oracle.star_from_box(lbs[:, i], ubs[:, i]), "relax-star-area", 1.0, keep=True)
+                        for i in range(count)])
+
+    def reach():
+        net = nnv.NN.from_config(L)
+        dev_in = nnv.Star.from_boxes(lbs, ubs) if count > 1 else nnv.Star(lbs[:, 0], ubs[:, 0])
+        net.reach(dev_in, {"reachMethod": "relax-star-area", "relaxFactor": 1})
+        return [[s] if count == 1 else list(s) for s in net.reachSet]
+
+    def check(sets, layer, what):
+        for i, S in enumerate(sets[layer]):
+            E = exp_sets[i][layer]
+            if what == "V":
+                assert_close(np.asarray(S.V), E.V, "V of layer %d, set %d" % (layer, i), RTOL)
+            else:
+                assert_close(np.asarray(S.C), E.C, "C of layer %d, set %d" % (layer, i), RTOL)
+                assert_close(np.asarray(S.d), E.d, "d of layer %d, set %d" % (layer, i), RTOL)
+
+    orders = [[(0, "V"), (1, "V"), (2, "V"), (3, "V"), (4, "C"), (4, "V")],      # producers first
+              [(4, "C"), (3, "V"), (1, "V"), (0, "V"), (2, "V")],                  # constraint rows first
+              [(1, "V"), (3, "C"), (2, "V"), (0, "V")],                            # a ReLU output first
+              [(2, "V"), (1, "C"), (0, "V")]]
+    for order in orders:
+        sets = reach()
+        for layer, what in order:
+            check(sets, layer, what)
+    # the same reach with the columns written by the producing call: bit-identical reads
+    lazy = reach()
+    ctx.set_eager_columns(True)
+    try:
+        eager = reach()
+    finally:
+        ctx.set_eager_columns(False)
+    for layer in range(len(L)):
+        for A, B in zip(lazy[layer], eager[layer]):
+            assert np.array_equal(np.asarray(A.V), np.asarray(B.V))
+            assert np.array_equal(np.asarray(A.predicate_ub), np.asarray(B.predicate_ub))
+    assert np.array_equal(np.asarray(lazy[-1][0].C), np.asarray(eager[-1][0].C))
