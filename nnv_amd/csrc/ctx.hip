@@ -1007,6 +1007,17 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       std::vector<char> pk((size_t)count, 0);
       std::vector<char> filled((size_t)count, 0);
       bool any_fill = false;
+      // Range sums: chunk_off[i] .. chunk_off[i+1] are set i's chunks of [4][ld] partial sums in `sums`,
+      // first one per column tile of the segmented GEMM (tiles_of[i], filled by its epilogue), then the
+      // gather pass's gch chunks if the set has gathered columns.
+      BufRef sums;
+      std::vector<int64_t> tiles_of((size_t)count, 0), chunk_off((size_t)count + 1, 0);
+      int64_t gch = 0;
+      {
+        int64_t max_m = 0;
+        for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, gs[i].m);
+        gch = gather_chunks_batch(outs[0]->ld, count, max_m);  // 0: nothing to gather
+      }
       for (int64_t i = 0; i < count; ++i) {
         bool pack = false;
         any_rows = rows_of(i, &rws[i], &kps[i], &pack) || any_rows;
@@ -1061,10 +1072,19 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             }
           if (st == NNVHIP_OK && !packs.empty()) st = launch_pack_rows(c, (int64_t)packs.size(), packs.data());
         }
-        int64_t off = 0, off_in = 0, kp_max = kLdAlign;
+        const int64_t ldo = outs[0]->ld;
         for (int64_t i = 0; i < count; ++i) {
+          tiles_of[i] = filled[i] ? 0 : ceil_div(dense[i], tn);
+          chunk_off[i + 1] = chunk_off[i] + tiles_of[i] + (gs[i].m > 0 ? gch : 0);
+        }
+        if (st == NNVHIP_OK && chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
+        int64_t off = 0, off_in = 0, kp_max = kLdAlign;
+        for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
           for (int64_t j = 0; j < dense[i] && !filled[i]; j += tn) {
             GemmSeg sg;
+            sg.plb = outs[i]->plb;
+            sg.pub = outs[i]->pub;
+            sg.rpart = sums->as<double>() + 4 * ldo * (chunk_off[i] + j / tn);
             sg.kmap = rws[i].kmap;
             sg.Bk = bk[i];
             sg.ldbk = kps[i];
@@ -1105,28 +1125,29 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       if (st == NNVHIP_OK && (any_onehot || any_fill)) {
         // the gather also leaves the range sums of its columns on the output handles, so the ReLU
         // that follows scans only the contracted columns
-        int64_t max_m = 0;
-        for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, gs[i].m);
-        const int64_t gch = gather_chunks_batch(outs[0]->ld, count, max_m);  // 0: nothing to gather, fills only
-        BufRef sums;
-        if (gch > 0) st = c->alloc(sizeof(double) * 4 * outs[0]->ld * gch * count, &sums);
+        const int64_t ldo = outs[0]->ld;
+        if (!sums) {  // no segmented GEMM ran: the gather's chunks are all there is
+          for (int64_t i = 0; i < count; ++i) chunk_off[i + 1] = chunk_off[i] + (gs[i].m > 0 ? gch : 0);
+          if (chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
+        }
         if (st == NNVHIP_OK) {
           for (int64_t i = 0; i < count; ++i) {
-            gs[i].part = (gch > 0 && gs[i].m > 0) ? sums->as<double>() + 4 * outs[0]->ld * gch * i : nullptr;
+            gs[i].part = (gch > 0 && gs[i].m > 0) ? sums->as<double>() + 4 * ldo * (chunk_off[i] + tiles_of[i]) : nullptr;
             lazy[i] = lazy_ok && gs[i].part != nullptr;
             gs[i].lazy = lazy[i];
           }
-          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, count, gs.data(), gch);
+          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, ldo, count, gs.data(), gch);
         }
-        for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
-          if (gs[i].m > 0) {
-            outs[i]->rng_buf = sums;
-            outs[i]->rng_part = gs[i].part;
-            outs[i]->rng_chunks = gch;
-            // the columns before the gathered ones still need a scan -- unless they were filled with zeros,
-            // which add nothing to the sums
-            outs[i]->rng_first_col = filled[i] ? 1 : dense[i];
-          }
+      }
+      // what the two passes left: the GEMM tiles' chunks cover the contracted columns, the gather's its own;
+      // columns covered by neither (a GEMM without the fused sums) still need a scan, filled zeros add nothing
+      for (int64_t i = 0; i < count && st == NNVHIP_OK && sums; ++i) {
+        const int64_t nchunks = chunk_off[i + 1] - chunk_off[i];
+        if (nchunks == 0) continue;
+        outs[i]->rng_buf = sums;
+        outs[i]->rng_part = sums->as<double>() + 4 * outs[0]->ld * chunk_off[i];
+        outs[i]->rng_chunks = nchunks;
+        outs[i]->rng_first_col = (filled[i] || tiles_of[i] > 0) ? 1 : dense[i];
       }
     } else {
       for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {

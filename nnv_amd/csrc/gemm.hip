@@ -64,8 +64,17 @@ __global__ __launch_bounds__(64 * WR * WC, WPE) void gemm_f64_kernel(const doubl
   int64_t col_end = ncols;     // first column past the valid ones, in the same numbering as col_base
   int64_t bk_col0 = n0;        // column of Bk behind the tile's first column
   int64_t b_col_base = n0;     // column of B behind the tile's first column
+  // fused range sums: the tile's first column and the end of the valid ones in the numbering of plb / pub
+  // (the set's own columns), and the chunk of partial sums the tile fills
+  int64_t rcol0 = n0, rcol_end = ncols, rchunk = nt;
   if (MAPPED && segs != nullptr) {
     const GemmSeg sg = segs[nt];
+    rpart = sg.rpart;
+    plb = sg.plb;
+    pub = sg.pub;
+    rcol0 = sg.col_local0;
+    rcol_end = sg.col_local0 + sg.valid;
+    rchunk = 0;
     kmap = sg.kmap;
     Kp = sg.kp;
     col_base = sg.col_base;
@@ -202,8 +211,8 @@ __global__ __launch_bounds__(64 * WR * WC, WPE) void gemm_f64_kernel(const doubl
       for (int j = 0; j < FN; ++j) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int64_t col = n0 + wc * (TN / WC) + j * 16 + lcol + 4 * r;
-          if (col >= 1 && col < ncols) {
+          const int64_t col = rcol0 + wc * (TN / WC) + j * 16 + lcol + 4 * r;
+          if (col >= 1 && col < rcol_end) {
             const double v = acc[i][j][r];
             const double pl = plb[col - 1], pu = pub[col - 1];
             const double p = fmax(v, 0.0), q = fmin(v, 0.0);
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(64 * WR * WC, WPE) void gemm_f64_kernel(const doubl
       double s = 0.0;
 #pragma unroll
       for (int w = 0; w < WC; ++w) s += red[(w * TM + row) * 4 + q];
-      if (m0 + row < Mp) rpart[((int64_t)nt * 4 + q) * ldc + m0 + row] = s;
+      if (m0 + row < Mp) rpart[(rchunk * 4 + q) * ldc + m0 + row] = s;
     }
   }
 

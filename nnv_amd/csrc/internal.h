@@ -296,6 +296,11 @@ struct GemmSeg {
   int64_t col_base;    // column of C behind the tile's first column (output arena)
   int32_t kp;
   int32_t valid;
+  // fused range sums of this tile's columns (null: none): the set's predicate bounds (indexed by the
+  // set's own generator column) and the [4][ldc] chunk the tile fills
+  const double* plb;
+  const double* pub;
+  double* rpart;
 };
 struct GemmRows {
   const int32_t* kmap = nullptr;

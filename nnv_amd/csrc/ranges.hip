@@ -410,6 +410,11 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
       any_pending = true;
     }
   }
+  // every column of every set already has its sums from the producing kernels: no scan at all
+  bool scan = false;
+  for (int64_t i = 0; i < nset; ++i) scan = scan || !(descs[i].n == 0 && descs[i].chunks2 > 0);
+  if (!scan)
+    for (int64_t i = 0; i < nset; ++i) descs[i].chunks = 0;
   const RangeDesc* table = nullptr;
   BufRef tab;
   if (nset > 1) {
@@ -420,9 +425,11 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   double bytes = 0.0;  // algorithmic: V once, the predicate bounds, lb/ub out
   for (int64_t i = 0; i < nset; ++i)
     bytes += 8.0 * (double)todo[i]->N * (double)(descs[i].n + 1) + 16.0 * (double)descs[i].n + 16.0 * (double)todo[i]->N;
-  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  NNV_LAUNCH(ctx, ctx->kernel_timing, (ranges_partial_kernel<8, 4>), grid, dim3(64 * kRangeWaves), 0, table, descs[0]);
-  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
+  if (scan) {
+    NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
+    NNV_LAUNCH(ctx, ctx->kernel_timing, (ranges_partial_kernel<8, 4>), grid, dim3(64 * kRangeWaves), 0, table, descs[0]);
+    NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
+  }
   if (chunks > 1 || any_pending) {
     double fbytes = 0.0;  // every chunk's four sums read, lb and ub written
     for (int64_t i = 0; i < nset; ++i) fbytes += 8.0 * (double)ld * (4.0 * (double)(descs[i].chunks + descs[i].chunks2) + 3.0);
