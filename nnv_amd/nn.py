@@ -92,6 +92,9 @@ class NN:
 
     def reach_noConns(self, inSet):
         """nn/NN.m:1529-1551: layer loop; keeps every layer's output set and its wall time."""
+        # the sets of an earlier reach are let go once the first layers of this one are queued on the
+        # device: releasing thousands of handles then costs no device time
+        earlier = self.reachSet
         self.reachSet = [None] * self.numLayers
         self.reachTime = [0.0] * self.numLayers
         rs = inSet
@@ -117,6 +120,7 @@ class NN:
                 ctx.synchronize()
             self.reachTime[i] = time.perf_counter() - t0
             self.reachSet[i] = rs
+            earlier = None
         return rs
 
     # ---- robustness check (the consumer of the reach set) ---------------------------------
