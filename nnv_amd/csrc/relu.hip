@@ -833,6 +833,49 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   }
   NNV_HIP_TRY(hipGetLastError());
 
+  // Output handles: whatever does not depend on the counts is set up while the kernel runs (with the
+  // row reset pending and the bounds written by the kernel, that is nearly everything).
+  auto init_static = [&](nnvhip_star* o, ConsNode* node, int64_t i) {
+    o->N = N;
+    o->ld = ld;
+    if (lazy_rows) {  // shares the input's matrix until somebody needs the rows reset in memory
+      o->Vbuf = in[i]->Vbuf;
+      o->V = in[i]->V;
+      o->vcols = in[i]->n + 1;
+      o->rows_pending = true;
+      o->cls_buf = cls_buf;
+      o->cls = cls_buf->as<int32_t>() + ld * i;
+      // ... and what is known about where its columns came from (and whether they are in memory yet)
+      // holds for the rows that are kept
+      o->cs = in[i]->cs;
+    }
+    o->kept_buf = keep_buf;
+    o->kept_idx = keep_buf->as<int32_t>() + keep_ld * i;
+    node->prev = in[i]->cons;
+    node->n_before = in[i]->n;
+    node->src = in[i]->Vbuf;  // zero-copy: C2/C3 rows are rows of the input's immutable [c V]
+    node->src_V = in[i]->V;
+    node->src_ld = in[i]->ld;
+    node->src_cs = in[i]->cs;
+    node->index = idx_buf;
+    node->index_off = ld * i;
+  };
+  struct PreCreated {
+    std::vector<nnvhip_star*> v;
+    ~PreCreated() { release_all(v); }  // only what was not handed over
+  } pre;
+  std::vector<std::shared_ptr<ConsNode>> nodes;
+  const bool precreate = lazy_rows && fold_bounds && count > 1;
+  if (precreate) {
+    pre.v.reserve(count);
+    nodes.resize(count);
+    for (int64_t i = 0; i < count; ++i) {
+      pre.v.push_back(new_star(ctx));
+      nodes[i] = std::make_shared<ConsNode>();
+      init_static(pre.v[i], nodes[i].get(), i);
+    }
+  }
+
   // the column count of the output depends on m: fetch the counts
   std::vector<int32_t> counts(2 * count);
   if (use_mailbox) {
@@ -935,21 +978,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
 
   for (int64_t i = 0; i < count; ++i) {
     const ReluDesc& d = descs[i];
-    nnvhip_star* o = new_star(ctx);
-    o->N = N;
+    nnvhip_star* o = precreate ? pre.v[i] : new_star(ctx);
+    std::shared_ptr<ConsNode> node = precreate ? std::move(nodes[i]) : std::make_shared<ConsNode>();
+    if (!precreate) init_static(o, node.get(), i);
     o->n = in[i]->n + d.m;
-    o->ld = ld;
-    if (lazy_rows) {  // shares the input's matrix until somebody needs the rows reset in memory
-      o->Vbuf = in[i]->Vbuf;
-      o->V = in[i]->V;
-      o->vcols = in[i]->n + 1;
-      o->rows_pending = true;
-      o->cls_buf = cls_buf;
-      o->cls = cls_buf->as<int32_t>() + ld * i;
-      // ... and what is known about where its columns came from (and whether they are in memory yet)
-      // holds for the rows that are kept
-      o->cs = in[i]->cs;
-    } else {
+    if (!lazy_rows) {
       o->Vbuf = arena;
       o->V = d.Vout;
     }
@@ -966,31 +999,20 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     }
     // rows of the leading columns that were not reset
     o->n_kept = N - counts[2 * i] - counts[2 * i + 1];
-    o->kept_buf = keep_buf;
-    o->kept_idx = keep_buf->as<int32_t>() + keep_ld * i;
     if (d.m > 0) {
-      auto node = std::make_shared<ConsNode>();
-      node->prev = in[i]->cons;
       node->m = d.m;
-      node->n_before = in[i]->n;
       node->p_total = in[i]->cons->p_total + 3 * (int64_t)d.m;
       node->n_total = o->n;
-      node->src = in[i]->Vbuf;  // zero-copy: C2/C3 rows are rows of the input's immutable [c V]
-      node->src_V = in[i]->V;
-      node->src_ld = in[i]->ld;
-      node->src_cs = in[i]->cs;
       node->ld_lbub = d.ld_lbub;
       node->lbub = lbub_buf;
-      node->index = idx_buf;
-      node->index_off = ld * i;
-      // views into shared buffers: keep element offsets
-      node->lbub_off = lbub_off[i];
-      o->cons = node;
+      node->lbub_off = lbub_off[i];  // a view into a shared buffer: the element offset
+      o->cons = std::move(node);
     } else {
       o->cons = in[i]->cons;  // no crossing neuron: C, d unchanged
     }
     out[i] = o;
   }
+  pre.v.clear();  // handed over
   return NNVHIP_OK;
 }
 
