@@ -31,6 +31,25 @@ static size_t size_class(size_t bytes) {
   return (bytes + step - 1) / step * step;
 }
 
+const TuneKnobs& tune_knobs() {
+  static const TuneKnobs knobs = [] {
+    TuneKnobs k;
+    auto num = [](const char* name) {
+      const char* e = getenv(name);
+      return e ? atoi(e) : 0;
+    };
+    k.gemm_xr = num("NNVHIP_GEMM_XR");
+    k.gemm_ksplit = num("NNVHIP_GEMM_KSPLIT");
+    if (const char* e = getenv("NNVHIP_GEMM_TILE")) k.gemm_tile = e;
+    k.ranges_row_waves = num("NNVHIP_RANGES_ROW_WAVES");
+    k.ranges_blocks = num("NNVHIP_RANGES_BLOCKS");
+    k.apply_row_waves = num("NNVHIP_APPLY_ROW_WAVES");
+    k.apply_blocks = num("NNVHIP_APPLY_BLOCKS");
+    return k;
+  }();
+  return knobs;
+}
+
 nnvhip_star* new_star(nnvhip_ctx* ctx) {
   nnvhip_star* s = new nnvhip_star();
   s->ctx = ctx;

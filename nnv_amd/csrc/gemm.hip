@@ -312,8 +312,8 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
       best_slots = slots;
     }
   }
-  if (const char* e = getenv("NNVHIP_GEMM_XR")) {
-    best_xr = std::max(1, std::min(8, atoi(e)));
+  if (const int v = tune_knobs().gemm_xr) {
+    best_xr = std::max(1, std::min(8, v));
     best_slots = ceil_div(tiles_m, best_xr) * ceil_div(tiles_n, 8 / best_xr);
   }
   const int64_t local_m = ceil_div(tiles_m, best_xr);
@@ -323,7 +323,7 @@ static int launch_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, const doubl
   const int64_t nk = Kp / KT;
   int64_t ksplit = 1;
   if (blocks < 128 && nk >= 8) ksplit = std::min<int64_t>(std::min<int64_t>(16, nk / 4), ceil_div(512, blocks));
-  if (const char* e = getenv("NNVHIP_GEMM_KSPLIT")) ksplit = std::max<int64_t>(1, std::min<int64_t>(atoi(e), nk));
+  if (const int v = tune_knobs().gemm_ksplit) ksplit = std::max<int64_t>(1, std::min<int64_t>(v, nk));
   // the split-K workspace is laid out for one plain column range: no segment tables (a column map is
   // applied by the reduction)
   if (rows != nullptr && rows->segs != nullptr) ksplit = 1;
@@ -418,9 +418,9 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
   }
   if (rows != nullptr && rows->segs != nullptr)  // the table was cut for this width: see gemm_seg_cols
     return rows->seg_cols == 64 ? NNV_GEMM(64, 64, 2, 4, 16) : NNV_GEMM(128, 128, 2, 4, 16);
-  if (const char* e = getenv("NNVHIP_GEMM_TILE")) {  // tuning knob: "TMxTN" of one of the shapes above
+  if (!tune_knobs().gemm_tile.empty()) {  // tuning knob: "TMxTN" of one of the shapes above
     for (int i = 0; i < (int)(sizeof(shapes) / sizeof(shapes[0])); ++i)
-      if (std::to_string(shapes[i].tm) + "x" + std::to_string(shapes[i].tn) == e) best = i;
+      if (std::to_string(shapes[i].tm) + "x" + std::to_string(shapes[i].tn) == tune_knobs().gemm_tile) best = i;
   }
   switch (shapes[best].tm * 1000 + shapes[best].tn) {
     case 64064: return NNV_GEMM(64, 64, 2, 4, 16);

@@ -60,6 +60,16 @@ struct Buffer {
 };
 using BufRef = std::shared_ptr<Buffer>;
 
+// Tuning knobs for experiments, read from the environment once per process (0 / empty: not set):
+// NNVHIP_GEMM_XR, NNVHIP_GEMM_KSPLIT, NNVHIP_GEMM_TILE ("TMxTN"), NNVHIP_RANGES_ROW_WAVES,
+// NNVHIP_RANGES_BLOCKS, NNVHIP_APPLY_ROW_WAVES, NNVHIP_APPLY_BLOCKS.
+struct TuneKnobs {
+  int gemm_xr = 0, gemm_ksplit = 0;
+  std::string gemm_tile;
+  int ranges_row_waves = 0, ranges_blocks = 0, apply_row_waves = 0, apply_blocks = 0;
+};
+const TuneKnobs& tune_knobs();
+
 // Where an FC map gathered stored columns of a set from, and whether they are in memory yet.  Column
 // from + t holds 0 + W(:, r) * scale[r] with r = idx[t] (scale == null: 1).  A later packing of kept rows
 // reads the cache-resident weight matrix instead of the set's own matrix in HBM; and the FC map may leave

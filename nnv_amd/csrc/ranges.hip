@@ -364,13 +364,10 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   // Column chunking: enough blocks to cover the chip a few times over, at least 64 columns per
   // chunk so the partial-sum traffic stays below ~6 % of V.
   int row_waves = 1;  // measured best: all eight waves on the same 128 rows, interleaving columns
-  if (const char* e = getenv("NNVHIP_RANGES_ROW_WAVES")) {
-    const int v = atoi(e);
-    row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
-  }
+  if (const int v = tune_knobs().ranges_row_waves) row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
   const int64_t row_blocks = ceil_div(ld, kRowsPerWave * row_waves);
   int64_t want_blocks = 2048;
-  if (const char* e = getenv("NNVHIP_RANGES_BLOCKS")) want_blocks = std::max(1, atoi(e));
+  if (const int v = tune_knobs().ranges_blocks) want_blocks = std::max(1, v);
   int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * nset), ceil_div(nmax, 64)));
   chunks = std::min<int64_t>(chunks, 1024);
   // one buffer for all lb/ub, one for all partials

@@ -588,14 +588,11 @@ static int launch_apply(nnvhip_ctx* ctx, int64_t count, std::vector<ReluDesc>& d
     max_cols = std::max<int64_t>(max_cols, descs[i].ncols_in + (descs[i].write_tail ? descs[i].m : 0));
   // a couple of thousand blocks, at least two steps per wave
   int row_waves = ld >= 8 * kApplyRows ? 8 : ld >= 4 * kApplyRows ? 4 : ld >= 2 * kApplyRows ? 2 : 1;
-  if (const char* e = getenv("NNVHIP_APPLY_ROW_WAVES")) {
-    const int v = atoi(e);
-    row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
-  }
+  if (const int v = tune_knobs().apply_row_waves) row_waves = v == 8 ? 8 : v == 4 ? 4 : v == 2 ? 2 : 1;
   const int64_t row_blocks = ceil_div(ld, kApplyRows * row_waves);
   const int64_t min_cpc = (const int64_t)8 * (kApplyWaves / row_waves);  // two 4-column steps per wave
   int64_t want_blocks = 8192;
-  if (const char* e = getenv("NNVHIP_APPLY_BLOCKS")) want_blocks = std::max(1, atoi(e));
+  if (const int v = tune_knobs().apply_blocks) want_blocks = std::max(1, v);
   int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(want_blocks, row_blocks * count), ceil_div(max_cols, min_cpc)));
   const int64_t cpc = ceil_div(max_cols, chunks);
   chunks = ceil_div(max_cols, cpc);
