@@ -888,6 +888,8 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.red = nullptr;
       g.red_k = 0;
       g.lazy = 0;
+      g.cin = nullptr;
+      g.cpart = nullptr;
       g.centre = nullptr;
     }
     // sets whose implicit unit-vector columns take part in the contraction after all get them written out
@@ -994,10 +996,21 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         }
         // only the centre is contracted (a box star): the range sums are the gather's alone
         const bool centre_only = dense[0] == 1 && gs[0].m > 0;
-        SplitKDefer defer;  // ... and the gather pass also sums the centre's split-K partials
-        if (st == NNVHIP_OK)
+        // ... and when the gathered columns are all the columns of W (no degenerate dimension), the gather
+        // pass forms the centre's product as well, one partial vector per chunk: no GEMM launch at all
+        const bool centre_in_gather = centre_only && !compact && gs[0].m == fc->K && in[0]->oh_from == 1 && gch > 0;
+        SplitKDefer defer;  // (otherwise the gather pass sums the centre's split-K partials)
+        BufRef cpart;
+        if (st == NNVHIP_OK && centre_in_gather) {
+          st = c->alloc(sizeof(double) * outs[0]->ld * gch, &cpart);
+          if (st == NNVHIP_OK) {
+            gs[0].cin = in[0]->V;
+            gs[0].cpart = cpart->as<double>();
+          }
+        } else if (st == NNVHIP_OK) {
           st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias,
                            centre_only ? nullptr : &fuse, compact ? &rows : nullptr, centre_only ? &defer : nullptr);
+        }
         if (st == NNVHIP_OK && centre_only) {
           st = c->alloc(sizeof(double) * 4 * outs[0]->ld * gch, &fuse.part);
           fuse.chunks = 0;
@@ -1015,7 +1028,9 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           gs[0].lazy = lazy[0];
           st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), fused ? gch : 0);
         }
-        if (st == NNVHIP_OK && fused) st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0));
+        if (st == NNVHIP_OK && fused)
+          st = finalize_fused_ranges(c, outs[0], fuse.part, fuse.chunks + (gs[0].m > 0 ? gch : 0),
+                                     centre_in_gather ? cpart->as<double>() : nullptr, centre_in_gather ? gch : 0, bias);
       }
     } else if (contig) {
       // one launch for the whole array.  With structure to exploit, every set's dense columns are cut

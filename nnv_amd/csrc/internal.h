@@ -402,6 +402,11 @@ struct GatherSet {
   int32_t red_k;        // `centre`, plus the bias; null / 0 = the centre is final
   int32_t lazy;         // 1: only the range sums (and column 0 of the fill) are produced, the columns stay unwritten
   double* centre;
+  // The gathered columns are all the columns of W (a box star without degenerate dimensions): the pass
+  // also forms the centre's product W * cin, as one partial vector per chunk (cpart[chunk][ldout]) that
+  // the range reduction sums in chunk order.  cin == null: not asked for.
+  const double* cin;    // the input's centre, indexed by row
+  double* cpart;
 };
 // Writes the columns of the sets that are described but not in memory yet (see ColSource).
 int write_pending_columns(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets);
@@ -413,7 +418,10 @@ int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m);
 int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t Mp, int64_t ldout, int64_t count,
                           const GatherSet* sets, int64_t chunks);
 // Turns the per-column-tile partial sums a fused GEMM left behind into the set's cached lb/ub.
-int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks);
+// cpart / cchunks / cbias: the centre column of s is still to be formed as the sum of cchunks partial
+// vectors (ld entries each) plus the bias (or null); the kernel writes it into column 0 of s first.
+int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks,
+                          const double* cpart = nullptr, int64_t cchunks = 0, const double* cbias = nullptr);
 
 // relu.hip
 // Makes V a plain stored matrix: writes columns that are still pending (need_cols; always when one of

@@ -18,7 +18,10 @@ struct RangeDesc {
   double* part;       // [chunks][4][ld] partial sums (unused when chunks == 1 and chunks2 == 0)
   const double* part2;  // further chunks2 chunks left by the producer of the trailing columns, or null
   int32_t chunks2;
-  int32_t pad_;
+  int32_t cchunks;      // > 0: the centre is the sum of cchunks vectors at cpart (ld apart) plus cbias (or
+  const double* cpart;  // null), written to cout before it enters lb / ub
+  const double* cbias;
+  double* cout;
   double* lb;         // ld
   double* ub;         // ld
   int64_t ld;
@@ -116,13 +119,32 @@ __global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(c
 
 // Combines the chunk partials in chunk order.  64 rows per block; the four sums of a row are handled
 // by four different waves so that the dependent add chains are short.
-__global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
+__global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
   if (d.chunks == 1 && d.chunks2 == 0 && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
   const int lane = threadIdx.x & 63;
   const int q = threadIdx.x >> 6;
   const int64_t r = (int64_t)blockIdx.x * 64 + lane;
   __shared__ double sums[4][64];
+  __shared__ double cen[64];
+  if (q == 4) {  // a wave of its own (the launch that has a centre to form brings five)
+    if (d.cchunks > 0 && r < d.ld) {
+      double c0 = 0.0;
+      for (int c = 0; c < d.cchunks; c += 32) {
+        double v[32];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) v[u] = c + u < d.cchunks ? d.cpart[(int64_t)(c + u) * d.ld + r] : 0.0;
+#pragma unroll
+        for (int u = 0; u < 32; ++u)
+          if (c + u < d.cchunks) c0 += v[u];
+      }
+      if (d.cbias != nullptr) c0 = c0 + d.cbias[r];
+      d.cout[r] = c0;
+      cen[lane] = c0;
+    }
+    __syncthreads();
+    return;
+  }
   double s = 0.0;
   if (r < d.ld) {
     // the partial sums were written by other CUs moments ago: every load is a trip to memory, so as many
@@ -153,7 +175,7 @@ __global__ __launch_bounds__(256) void ranges_final_kernel(const RangeDesc* __re
   sums[q][lane] = s;
   __syncthreads();
   if (q == 0 && r < d.ld) {
-    const double c0 = d.V[r];
+    const double c0 = d.cchunks > 0 ? cen[lane] : d.V[r];
     d.lb[r] = (c0 + sums[0][lane]) + sums[1][lane];
     d.ub[r] = (c0 + sums[2][lane]) + sums[3][lane];
   }
@@ -173,6 +195,9 @@ struct GatherArgs {
   int64_t Mp;         // rows of W (a multiple of 16): the bias has that many entries
 };
 
+// CENTRE: the variant that also forms the centre's product (GatherSet::cin); kept apart because its extra
+// registers would cost the plain pass a resident block per CU.
+template <bool CENTRE>
 __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const GatherSet* __restrict__ table, GatherSet one,
                                                                          GatherArgs a) {
   const GatherSet d = table ? table[blockIdx.z] : one;
@@ -214,18 +239,20 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
       if (j == 0 || !d.lazy) *reinterpret_cast<double2*>(d.fill + r0 + (int64_t)j * a.ldout) = o;
     }
   }
-  double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
+  double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0}, cacc = {0, 0};
   if (active) {
     for (int jb = j0 + 4 * wave; jb < j1; jb += 4 * kRangeWaves) {
       double2 v[4];
-      double sc[4];
+      double sc[4], cj[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         v[u] = make_double2(0.0, 0.0);
         sc[u] = 1.0;
+        cj[u] = 0.0;
         if (jb + u < j1) {
           const int src = d.idx[jb + u];
           if (d.scale != nullptr) sc[u] = d.scale[src];
+          if (CENTRE && d.cin != nullptr) cj[u] = d.cin[src];
           v[u] = *reinterpret_cast<const double2*>(a.W + r0 + (int64_t)src * a.ldw);
         }
       }
@@ -233,6 +260,10 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
       for (int u = 0; u < 4; ++u) {
         const int j = jb + u;
         if (j >= j1) break;
+        if (CENTRE && d.cin != nullptr) {  // the centre's product rides along
+          cacc.x = fma(v[u].x, cj[u], cacc.x);
+          cacc.y = fma(v[u].y, cj[u], cacc.y);
+        }
         double2 o;
         o.x = __dadd_rn(0.0, __dmul_rn(v[u].x, sc[u]));
         o.y = __dadd_rn(0.0, __dmul_rn(v[u].y, sc[u]));
@@ -254,16 +285,21 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
     }
   }
   if (part == nullptr) return;
-  __shared__ double2 red[kRangeWaves][4][64];
+  __shared__ double2 red[kRangeWaves - 1][CENTRE ? 5 : 4][64];  // (wave 0 keeps its own in registers)
   if (wave > 0) {
-    red[wave][0][lane] = xmin1;
-    red[wave][1][lane] = xmin2;
-    red[wave][2][lane] = xmax1;
-    red[wave][3][lane] = xmax2;
+    red[wave - 1][0][lane] = xmin1;
+    red[wave - 1][1][lane] = xmin2;
+    red[wave - 1][2][lane] = xmax1;
+    red[wave - 1][3][lane] = xmax2;
+    if (CENTRE) red[wave - 1][4][lane] = cacc;
   }
   __syncthreads();
   if (wave == 0 && active) {
-    for (int w = 1; w < kRangeWaves; ++w) {
+    for (int w = 0; w < kRangeWaves - 1; ++w) {
+      if (CENTRE) {
+        cacc.x += red[w][4][lane].x;
+        cacc.y += red[w][4][lane].y;
+      }
       xmin1.x += red[w][0][lane].x;
       xmin1.y += red[w][0][lane].y;
       xmin2.x += red[w][1][lane].x;
@@ -278,6 +314,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
     *reinterpret_cast<double2*>(p + a.ldout) = xmin2;
     *reinterpret_cast<double2*>(p + 2 * a.ldout) = xmax1;
     *reinterpret_cast<double2*>(p + 3 * a.ldout) = xmax2;
+    if (CENTRE && d.cin != nullptr) *reinterpret_cast<double2*>(d.cpart + (int64_t)chunk * a.ldout + r0) = cacc;
   }
 }
 
@@ -328,8 +365,14 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
     bytes += sets[i].lazy ? 8.0 * (double)Mp * (sets[i].nfill > 0 ? 1.0 : 0.0) + (with_sums && sets[i].part ? 32.0 * (double)ldout * (double)chunks : 0.0)
                           : 8.0 * (double)Mp * (double)(sets[i].m + sets[i].nfill);
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
-             dim3(64 * kRangeWaves), 0, table, sets[0], a);
+  bool centre = false;
+  for (int64_t i = 0; i < count; ++i) centre = centre || sets[i].cin != nullptr;
+  if (centre)
+    NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel<true>, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
+               dim3(64 * kRangeWaves), 0, table, sets[0], a);
+  else
+    NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel<false>, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
+               dim3(64 * kRangeWaves), 0, table, sets[0], a);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
@@ -395,7 +438,10 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     d.row_waves = row_waves;
     d.part2 = nullptr;
     d.chunks2 = 0;
-    d.pad_ = 0;
+    d.cchunks = 0;
+    d.cpart = nullptr;
+    d.cbias = nullptr;
+    d.cout = nullptr;
     if (t->rng_part != nullptr && t->rng_chunks > 0 && t->rng_first_col >= 1) {
       // the producer of the trailing columns left their sums: scan only the columns before them
       d.part2 = t->rng_part;
@@ -446,7 +492,8 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   return NNVHIP_OK;
 }
 
-int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks) {
+int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, int64_t chunks, const double* cpart,
+                          int64_t cchunks, const double* cbias) {
   if (s->lb || chunks < 1) return NNVHIP_OK;
   BufRef rb;
   NNV_TRY(ctx->alloc(sizeof(double) * 2 * s->ld, &rb));
@@ -464,7 +511,12 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
   d.row_waves = 1;
   d.part2 = nullptr;
   d.chunks2 = 0;
-  NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel, dim3((unsigned)ceil_div(s->ld, 64), 1, 1), dim3(256), 0, nullptr, d);
+  d.cchunks = (int32_t)cchunks;
+  d.cpart = cpart;
+  d.cbias = cbias;
+  d.cout = s->V;
+  NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel, dim3((unsigned)ceil_div(s->ld, 64), 1, 1),
+             dim3(cchunks > 0 ? 320 : 256), 0, nullptr, d);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 7, 8.0 * (double)s->ld * (4.0 * (double)chunks + 3.0)));
   NNV_HIP_TRY(hipGetLastError());
   s->rbuf = rb;
