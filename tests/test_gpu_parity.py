@@ -581,3 +581,28 @@ def test_columns_left_unwritten_are_written_on_any_first_read(nnv, oracle, count
             assert np.array_equal(np.asarray(A.V), np.asarray(B.V))
             assert np.array_equal(np.asarray(A.predicate_ub), np.asarray(B.predicate_ub))
     assert np.array_equal(np.asarray(lazy[-1][0].C), np.asarray(eager[-1][0].C))
+
+
+@pytest.mark.parametrize("degenerate", [0, 3])
+def test_first_layer_centre_with_and_without_degenerate_dimensions(nnv, oracle, degenerate):
+    """FC map of a box star: with a generator for every dimension the gather pass also forms W*c + b;
+    with degenerate dimensions (no generator) the centre goes through the GEMM.  Both against the oracle,
+    together with the bounds that are built on the centre."""
+    rs = np.random.RandomState(123 + degenerate)
+    K, M = 300, 520
+    lb = rs.randn(K)
+    ub = lb + 0.05 + 0.1 * rs.rand(K)
+    ub[:degenerate] = lb[:degenerate]
+    W, b = rs.randn(M, K) / np.sqrt(K), rs.randn(M)
+    for bias in (b, None):
+        L = nnv.FullyConnectedLayer(W, bias if bias is not None else np.zeros(M))
+        R = L.reach(nnv.Star(lb, ub), "approx-star")
+        E = oracle.affine_map(oracle.star_from_box(lb, ub), W, bias if bias is not None else np.zeros(M))
+        assert R.nVar == K - degenerate
+        lo, hi = R.estimateRanges()          # before V: the bounds come from the sums, the centre from its partials
+        elo, ehi = oracle.estimate_ranges(E)
+        assert_close(lo, elo, "lb", RTOL)
+        assert_close(hi, ehi, "ub", RTOL)
+        assert_close(np.asarray(R.V), E.V, "V", RTOL)
+        # generator columns are plain copies of scaled weight columns: exact
+        assert np.array_equal(np.asarray(R.V)[:, 1:], E.V[:, 1:])
