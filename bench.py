@@ -148,6 +148,11 @@ def main():
     # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
     gemm_flop = conv_flop = 0.0
     relu_bytes, relu_ms = 0.0, 0.0
+    # bytes of the output columns the gather passes stand for (8 * rows per one-hot input column), whether
+    # a pass writes them or leaves them pending
+    gat_dense_bytes = 0.0
+    onehot_cols = [s._h.dims()[1] for s in (dev_in if isinstance(dev_in, (list, nnv_amd.SetArray)) else [dev_in])] \
+        if cfg["layers"][0]["type"] == "fc" else None
     layer_report = []
     prev_sets = dev_in if isinstance(dev_in, (list, nnv_amd.SetArray)) else [dev_in]
     for i, (Ld, L) in enumerate(zip(cfg["layers"], net.Layers)):
@@ -160,6 +165,9 @@ def main():
             entry["dense_equivalent_tflops"] = round(flop / (per_layer[i] * 1e-3) / 1e12, 3)
             if M > 32:  # the 64-row-tile kernel; skinnier layers use another instantiation
                 gemm_flop += flop
+            if onehot_cols is not None:
+                gat_dense_bytes += 8.0 * M * sum(onehot_cols)
+            onehot_cols = None
         elif Ld["type"] == "conv":
             fh, fw, cin, cout = Ld["W"].shape
             flop = 0.0
@@ -188,8 +196,11 @@ def main():
             entry["algo_GBps"] = round(b / (per_layer[i] * 1e-3) / 1e9, 1)
             relu_bytes += b
             relu_ms += per_layer[i]
+            onehot_cols = [so._h.dims()[1] - sp._h.dims()[1] for sp, so in zip(prev_sets, outs)]   # the appended columns
         layer_report.append(entry)
         prev_sets = outs
+        if Ld["type"] != "relu":
+            onehot_cols = None
 
     # MFMA kernels: flop the kernel executed (the library's own count for its launches: products with
     # structural zeros that the FC map skips are not counted) over the kernels' HIP-event durations;
@@ -228,6 +239,8 @@ def main():
             # all FC layers but the last leave the gathered columns unwritten (range sums only): those
             # launches run out of the cache-resident weights and are bound by L2 / ALU rate, not by HBM
             g["columns_left_unwritten"] = True
+            if all(Ld["type"] in ("fc", "relu") for Ld in cfg["layers"]):   # (CNNs: the group also holds the stamp passes)
+                g["dense_equivalent_GBps"] = round(gat_dense_bytes * reps / (gat_ms * 1e-3) / 1e9, 1)
         groups.append((gat_ms, g))
     if fin_launches:
         groups.append((fin_ms, hbm_roofline("ranges_final_kernel", fin_ms, fin_launches, fin_bytes)))
