@@ -81,7 +81,7 @@ def main():
     def step():
         out = net.reach(dev_in, opts)
         outs = out if isinstance(out, (list, nnv_amd.SetArray)) else [out]
-        arr = (ctypes.c_void_p * len(outs))(*[o_._h.h for o_ in outs])
+        arr = outs.handles() if isinstance(outs, nnv_amd.SetArray) else (ctypes.c_void_p * len(outs))(*[o_._h.h for o_ in outs])
         # output bounds of all sets in one batched call, left on the device
         nnv_amd._lib.check(lib.nnvhip_estimate_ranges_batch(h, len(outs), arr, None, None))
         return out
