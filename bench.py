@@ -303,6 +303,29 @@ def main():
     host_to_host_ms = 1e3 * (time.perf_counter() - t1) / n_h2h
     del fresh, res
 
+    # ---- the same step with every intermediate set written out in full (not `value`) -------------
+    # By default the sets between the layers keep what nobody reads before the next layer as a description
+    # (a ReLU's row reset and appended columns, columns gathered from the weights) and write it on first
+    # read; the returned set and its bounds are always written.  Here every layer writes its whole output.
+    all_written_ms = None
+    if not args.dense:
+        ctx.set_eager_columns(True)
+        ctx.set_eager_relu(True)
+        try:
+            for _ in range(3):
+                step()
+            ctx.synchronize()
+            n_aw = max(5, min(args.steps, 100))
+            t1 = time.perf_counter()
+            for _ in range(n_aw):
+                step()
+            ctx.synchronize()
+            all_written_ms = 1e3 * (time.perf_counter() - t1) / n_aw
+        finally:
+            ctx.set_eager_columns(False)
+            ctx.set_eager_relu(False)
+        net.reach(dev_in, opts)   # reachSet back to the default path for what follows
+
     # ---- specification check on the resident output sets (not part of `value`) -----------------
     spec = None
     last = net.Layers[-1]
@@ -358,10 +381,16 @@ def main():
                    "fc_affine_map": "dense" if args.dense else "structural zeros skipped (one-hot generator columns, reset rows); exact",
                    "sets": len(dev_in) if isinstance(dev_in, (list, nnv_amd.SetArray)) else 1,
                    "updates_per_step": updates,
+                   "intermediate_sets": "dense" if args.dense else
+                   "the sets between layers record a ReLU's row reset / appended columns and the columns an FC layer "
+                   "gathers from its weights and write them on first read; the returned set and its bounds are written",
                    "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, (list, nnv_amd.SetArray)) else None},
         "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec,
         "host_to_host": {"ms_per_step": round(host_to_host_ms, 4), "steps": n_h2h,
                          "what": "input bounds uploaded and the set(s) built, reach, output bounds fetched to the host"},
+        "all_sets_written": None if all_written_ms is None else
+        {"ms_per_step": round(all_written_ms, 5), "value": updates / (all_written_ms * 1e-3),
+         "what": "the same step with every layer writing its whole output matrix in the call (nothing left for a first read)"},
         "layers": layer_report,
     }))
 

@@ -88,6 +88,13 @@ NNVHIP_API int nnvhip_set_dense_affine(nnvhip_ctx* ctx, int enabled);
  * in the call itself; a caller does that for the layer whose output it hands on (NN.reach's return
  * value, nn/NN.m:1529-1551).  Initial value: 1 if the environment variable NNVHIP_EAGER_COLS is set. */
 NNVHIP_API int nnvhip_set_eager_columns(nnvhip_ctx* ctx, int enabled);
+/* Output switch of nnvhip_relu_relax (no counterpart in the reference, where
+ * multipleStepReachStarApprox_at_one builds the whole new_V = [V1 V2], nn/funcs/PosLin.m:700-709).  By
+ * default the step's output shares the input's matrix: the row reset and the appended unit-vector
+ * columns are recorded on the handle and written when somebody needs them in memory.  enabled = 1
+ * writes the whole output matrix in the call.  Initial value: 1 if the environment variables
+ * NNVHIP_EAGER_ROWS and NNVHIP_EAGER_TAIL are both set (each of them alone switches its half). */
+NNVHIP_API int nnvhip_set_eager_relu(nnvhip_ctx* ctx, int enabled);
 /* Measurement hook (no counterpart in the reference): while timing level 2 is set, every launch of a
  * kernel group is bracketed by its own pair of HIP events on the context's stream.  which = 0:
  * dense GEMM kernel of the FC layers (tiles of at least 64 rows); 1: implicit-GEMM convolution

@@ -259,6 +259,13 @@ int nnvhip_set_eager_columns(nnvhip_ctx* c, int enabled) {
   return NNVHIP_OK;
 }
 
+int nnvhip_set_eager_relu(nnvhip_ctx* c, int enabled) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  c->eager_rows = enabled != 0;
+  c->eager_tail = enabled != 0;
+  return NNVHIP_OK;
+}
+
 int nnvhip_last_op_time_ms(nnvhip_ctx* c, double* ms) {
   if (!c || !ms) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   *ms = c->last_ms;

@@ -326,6 +326,9 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
   } else if (cmd == "set_eager_columns") {  // 1: FC layers write gathered columns in the call itself
     need(nrhs, 1, "set_eager_columns");
     check(nnvhip_set_eager_columns(ctx(), mxGetScalar(prhs[1]) != 0));
+  } else if (cmd == "set_eager_relu") {  // 1: the ReLU step writes its whole output matrix in the call itself
+    need(nrhs, 1, "set_eager_relu");
+    check(nnvhip_set_eager_relu(ctx(), mxGetScalar(prhs[1]) != 0));
   } else if (cmd == "set_dense_affine") {  // 1: FC / conv layers as the full dense contraction (measurement switch)
     need(nrhs, 1, "set_dense_affine");
     check(nnvhip_set_dense_affine(ctx(), mxGetScalar(prhs[1]) != 0));
