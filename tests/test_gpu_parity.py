@@ -581,6 +581,19 @@ def test_columns_left_unwritten_are_written_on_any_first_read(nnv, oracle, count
             assert np.array_equal(np.asarray(A.V), np.asarray(B.V))
             assert np.array_equal(np.asarray(A.predicate_ub), np.asarray(B.predicate_ub))
     assert np.array_equal(np.asarray(lazy[-1][0].C), np.asarray(eager[-1][0].C))
+    # ... and with the ReLU steps writing their whole output as well (nothing left for a first read)
+    ctx.set_eager_columns(True)
+    ctx.set_eager_relu(True)
+    try:
+        full = reach()
+    finally:
+        ctx.set_eager_columns(False)
+        ctx.set_eager_relu(False)
+    for layer in range(len(L)):
+        for A, B in zip(lazy[layer], full[layer]):
+            assert np.array_equal(np.asarray(A.V), np.asarray(B.V))
+    assert np.array_equal(np.asarray(lazy[-1][0].C), np.asarray(full[-1][0].C))
+    assert np.array_equal(np.asarray(lazy[-1][0].d), np.asarray(full[-1][0].d))
 
 
 @pytest.mark.parametrize("degenerate", [0, 3])
