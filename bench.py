@@ -63,6 +63,10 @@ def main():
     ap.add_argument("--dense", action="store_true",
                     help="run every FC layer as the full dense contraction (no skipping of structural zeros)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--lean", action="store_true",
+                    help="only the timed steps and the per-kernel timing pass (no dense-contraction, host-to-host, "
+                         "all-sets-written and specification passes): what the rocprofv3 summaries in profiles/ run, so "
+                         "that their kernel tables hold the kernels of the measured path only")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (sets shard across GPUs without communication; "
@@ -261,7 +265,7 @@ def main():
             roofline["longest_kernel_by_time"] = "relu_classify_kernel (latency bound, %d block(s) per launch)" % n_sets
     # the MFMA GEMM on the full dense problem of the same reach (what Star.affineMap executes in the
     # reference): a short extra pass with the skipping of structural zeros switched off
-    if gemm_launches and not args.dense:
+    if gemm_launches and not args.dense and not args.lean:
         ctx.set_dense_affine(True)
         step()
         ctx.synchronize()
@@ -293,14 +297,15 @@ def main():
 
     # ---- the same step with the host buffers the boundary takes and returns (not `value`) -----------
     # lb / ub uploaded and the input set built on the device, the reach, the output bounds back on the host
-    n_h2h = max(5, min(args.steps, 50))
+    n_h2h = 0 if args.lean else max(5, min(args.steps, 50))
     ctx.synchronize()
     t1 = time.perf_counter()
+    fresh = res = None
     for _ in range(n_h2h):
         fresh = device_input_sets(cfg, ctx)
         res = net.reach(fresh, opts)
         nnv_amd.Star.estimateRanges_array(res if isinstance(res, (list, nnv_amd.SetArray)) else [res])
-    host_to_host_ms = 1e3 * (time.perf_counter() - t1) / n_h2h
+    host_to_host_ms = 1e3 * (time.perf_counter() - t1) / max(n_h2h, 1)
     del fresh, res
 
     # ---- the same step with every intermediate set written out in full (not `value`) -------------
@@ -308,7 +313,7 @@ def main():
     # (a ReLU's row reset and appended columns, columns gathered from the weights) and write it on first
     # read; the returned set and its bounds are always written.  Here every layer writes its whole output.
     all_written_ms = None
-    if not args.dense:
+    if not args.dense and not args.lean:
         ctx.set_eager_columns(True)
         ctx.set_eager_relu(True)
         try:
@@ -329,7 +334,7 @@ def main():
     # ---- specification check on the resident output sets (not part of `value`) -----------------
     spec = None
     last = net.Layers[-1]
-    if hasattr(last, "Bias") and len(last.Bias) > 1:
+    if hasattr(last, "Bias") and len(last.Bias) > 1 and not args.lean:
         from nnv_amd import verify
         out_sets = net.reachSet[-1]
         hs = net.robustness_set(0, "max")
@@ -386,8 +391,9 @@ def main():
                    "gathers from its weights and write them on first read; the returned set and its bounds are written",
                    "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, (list, nnv_amd.SetArray)) else None},
         "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec,
-        "host_to_host": {"ms_per_step": round(host_to_host_ms, 4), "steps": n_h2h,
-                         "what": "input bounds uploaded and the set(s) built, reach, output bounds fetched to the host"},
+        "host_to_host": None if n_h2h == 0 else
+        {"ms_per_step": round(host_to_host_ms, 4), "steps": n_h2h,
+         "what": "input bounds uploaded and the set(s) built, reach, output bounds fetched to the host"},
         "all_sets_written": None if all_written_ms is None else
         {"ms_per_step": round(all_written_ms, 5), "value": updates / (all_written_ms * 1e-3),
          "what": "the same step with every layer writing its whole output matrix in the call (nothing left for a first read)"},
