@@ -197,3 +197,10 @@ def test_set_array_makes_objects_on_demand_and_releases_every_handle_once():
     del arr3
     gc.collect()
     assert ctx2.bulk == [[4, 5, 6]]
+    # an array of boxes hands each element its own column of the bound matrices (Star(lb, ub) keeps them as
+    # state_lb / state_ub, set/Star.m:232-233)
+    lbs = np.asfortranarray(np.arange(6.0).reshape(3, 2))
+    ubs = lbs + 1.0
+    boxes = SetArray(ctx2, (C.c_void_p * 2)(7, 8), state=(lbs, ubs))
+    assert np.array_equal(boxes[1].state_lb, [1.0, 3.0, 5.0]) and np.array_equal(boxes[1].state_ub, [2.0, 4.0, 6.0])
+    assert boxes[0].state_lb.base is not None and np.array_equal(boxes[0].state_lb, lbs[:, 0])
