@@ -121,6 +121,16 @@ NNVHIP_API int nnvhip_probe_copy_bandwidth(nnvhip_ctx* ctx, int64_t bytes, int r
  * every CU (no memory traffic); returns the rate of the timed reps in TFLOP/s - the practical ceiling
  * of the matrix pipes on this box. */
 NNVHIP_API int nnvhip_probe_mfma_peak(nnvhip_ctx* ctx, int reps, double* tflops);
+/* Test hooks (no counterpart in the reference).  A ReLU step on up to 8192 sets learns its crossing /
+ * inactive counts through one 64-bit word per set that the classification kernel posts to pinned host
+ * memory: call number (16 bits) | n_crossing (24 bits) | n_inactive (24 bits).  Before the launch the host
+ * overwrites the words with the all-ones pattern, which no posted word can equal; `posted` is 0 for it.
+ * nnvhip_debug_set_relu_call_number sets the context's count of ReLU calls so that a test can place
+ * itself next to the wrap of the 16-bit field. */
+NNVHIP_API int nnvhip_debug_mailbox_pack(int32_t n_crossing, int32_t n_inactive, int32_t call_number, uint64_t* word);
+NNVHIP_API int nnvhip_debug_mailbox_unpack(uint64_t word, int32_t* posted, int32_t* n_crossing, int32_t* n_inactive,
+                                int32_t* call_number);
+NNVHIP_API int nnvhip_debug_set_relu_call_number(nnvhip_ctx* ctx, int64_t call_number);
 /* Returns every cached device block of the pool to the driver (hipFree). */
 NNVHIP_API int nnvhip_trim_pool(nnvhip_ctx* ctx);
 /* Bytes currently handed out by / cached in the pool. */

@@ -209,7 +209,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
   NNV_HIP_TRY(hipHostMalloc((void**)&c->mailbox, sizeof(int64_t) * nnvhip_ctx::kMailboxSets, hipHostMallocDefault));
-  memset((void*)c->mailbox, 0, sizeof(int64_t) * nnvhip_ctx::kMailboxSets);
+  memset((void*)c->mailbox, 0xff, sizeof(int64_t) * nnvhip_ctx::kMailboxSets);  // kMailboxEmpty everywhere
   NNV_HIP_TRY(hipEventCreate(&c->kev0));
   NNV_HIP_TRY(hipEventCreate(&c->kev1));
   *out = c;
@@ -349,6 +349,29 @@ int nnvhip_probe_mfma_peak(nnvhip_ctx* c, int reps, double* tflops) {
   NNV_HIP_TRY(hipEventElapsedTime(&ms, c->kev0, c->kev1));
   // one 16x16x4 MFMA = 2*16*16*4 flop; 8 per iteration and wave, 8 waves per block
   *tflops = 2048.0 * 8.0 * iters * 8.0 * blocks * reps / (ms * 1e-3) / 1e12;
+  return NNVHIP_OK;
+}
+
+int nnvhip_debug_mailbox_pack(int32_t n_crossing, int32_t n_inactive, int32_t call_number, uint64_t* word) {
+  if (!word) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  *word = mailbox_word(n_crossing, n_inactive, call_number);
+  return NNVHIP_OK;
+}
+
+int nnvhip_debug_mailbox_unpack(uint64_t word, int32_t* posted, int32_t* n_crossing, int32_t* n_inactive,
+                                int32_t* call_number) {
+  int m = 0, inact = 0, seq = 0;
+  mailbox_unpack(word, &m, &inact, &seq);
+  if (posted) *posted = word != kMailboxEmpty;
+  if (n_crossing) *n_crossing = m;
+  if (n_inactive) *n_inactive = inact;
+  if (call_number) *call_number = seq;
+  return NNVHIP_OK;
+}
+
+int nnvhip_debug_set_relu_call_number(nnvhip_ctx* c, int64_t call_number) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  c->mailbox_seq = (uint32_t)call_number;
   return NNVHIP_OK;
 }
 

@@ -60,6 +60,22 @@ struct Buffer {
 };
 using BufRef = std::shared_ptr<Buffer>;
 
+// Word a ReLU classification kernel posts to the host mailbox: call number in the top 16 bits, the
+// crossing and the inactive count in 24 bits each.  kMailboxEmpty is what the host stores into a word
+// before the launch that will post to it; no posted word equals it (see post_counts in relu.hip).
+constexpr int kMailboxCountBits = 24;
+constexpr unsigned long long kMailboxEmpty = ~0ull;
+__host__ __device__ inline unsigned long long mailbox_word(int m, int inactive, int seq) {
+  return ((unsigned long long)((unsigned)seq & 0xffffu) << (2 * kMailboxCountBits)) |
+         ((unsigned long long)((unsigned)m & ((1u << kMailboxCountBits) - 1)) << kMailboxCountBits) |
+         (unsigned long long)((unsigned)inactive & ((1u << kMailboxCountBits) - 1));
+}
+inline void mailbox_unpack(unsigned long long w, int* m, int* inactive, int* seq) {
+  *m = (int)((w >> kMailboxCountBits) & ((1u << kMailboxCountBits) - 1));
+  *inactive = (int)(w & ((1u << kMailboxCountBits) - 1));
+  *seq = (int)(w >> (2 * kMailboxCountBits));
+}
+
 // Tuning knobs for experiments, read from the environment once per process (0 / empty: not set):
 // NNVHIP_GEMM_XR, NNVHIP_GEMM_KSPLIT, NNVHIP_GEMM_TILE ("TMxTN"), NNVHIP_RANGES_ROW_WAVES,
 // NNVHIP_RANGES_BLOCKS, NNVHIP_APPLY_ROW_WAVES, NNVHIP_APPLY_BLOCKS.
@@ -133,11 +149,12 @@ struct nnvhip_ctx {
   std::vector<char*> retired_rings;
   size_t pinned_bytes = 0;
   size_t pinned_off = 0;
-  // mailbox in pinned host memory: a kernel posts {m, inactive, sequence number} there and the host
-  // spins on it, which is quicker than a device-to-host copy plus stream synchronisation
+  // mailbox in pinned host memory: a kernel posts {m, inactive, call number} there and the host spins
+  // on it (after having stored kMailboxEmpty there), which is quicker than a device-to-host copy plus
+  // stream synchronisation
   volatile int32_t* mailbox = nullptr;  // kMailboxSets words of 64 bits, one per set of an array
   static constexpr int64_t kMailboxSets = 8192;
-  int32_t mailbox_seq = 0;
+  uint32_t mailbox_seq = 0;  // number of the ReLU call (wraps; only its low 16 bits travel, as a cross-check)
   // FC layers as the full dense contraction (no skipping of structural zeros); default from the
   // environment variable NNVHIP_DENSE_AFFINE
   bool dense_affine = false;

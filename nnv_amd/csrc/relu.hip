@@ -9,6 +9,7 @@
 // The dense constraint matrix is never built on this path; materialize_constraints() lays it out
 // exactly as the reference does when the host asks for it.
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
@@ -54,14 +55,14 @@ struct ReluDesc {
   int32_t write_bounds; // apply pass: 1 = also write the predicate bounds and the crossing neurons' (lb, ub)
 };
 
-// Posts the counts to the host mailbox.  Payload and sequence number travel in one naturally aligned
-// 64-bit store (sequence number in the top 16 bits, the two counts in 24 bits each), so there is nothing
-// to order and nothing for the posting wave to wait for.
-constexpr int kMailboxCountBits = 24;
-__host__ __device__ __forceinline__ unsigned long long mailbox_word(int m, int inactive, int seq) {
-  return ((unsigned long long)((unsigned)seq & 0xffffu) << (2 * kMailboxCountBits)) |
-         ((unsigned long long)(unsigned)m << kMailboxCountBits) | (unsigned long long)(unsigned)inactive;
-}
+// Posts the counts to the host mailbox.  Payload and call number travel in one naturally aligned
+// 64-bit store (call number in the top 16 bits, the two counts in 24 bits each), so there is nothing
+// to order and nothing for the posting wave to wait for.  The host does not recognise a fresh word by
+// its call number: before the launch it overwrites every word the call will use with kMailboxEmpty
+// and waits until the word differs from that.  A posted word can never equal kMailboxEmpty (both
+// counts would have to be 2^24 - 1, and their sum is at most the set's dimension, which is below
+// 2^24), so a word some earlier call left behind cannot be taken for this call's, whatever the call
+// numbers are.  The 16-bit call number is only cross-checked after the word has arrived.
 __device__ __forceinline__ void post_counts(int32_t* mailbox, int m, int inactive, int seq) {
   if (mailbox == nullptr) return;
   __hip_atomic_store(reinterpret_cast<unsigned long long*>(mailbox), mailbox_word(m, inactive, seq), __ATOMIC_RELAXED,
@@ -793,10 +794,13 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const bool use_mailbox = count <= nnvhip_ctx::kMailboxSets && ctx->mailbox != nullptr && N < (int64_t(1) << kMailboxCountBits);
   if (use_mailbox) {  // every set's block posts into a word of its own
     ++ctx->mailbox_seq;
+    volatile unsigned long long* box = reinterpret_cast<volatile unsigned long long*>(ctx->mailbox);
     for (int64_t i = 0; i < count; ++i) {
+      box[i] = kMailboxEmpty;  // whatever an earlier call posted here is gone before the kernel is queued
       descs[i].mailbox = const_cast<int32_t*>(ctx->mailbox) + 2 * i;
-      descs[i].mailbox_seq = ctx->mailbox_seq;
+      descs[i].mailbox_seq = (int32_t)(ctx->mailbox_seq & 0xffffu);
     }
+    std::atomic_thread_fence(std::memory_order_seq_cst);
   }
   const ReluDesc* table = nullptr;
   BufRef tab;
@@ -876,23 +880,25 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // the column count of the output depends on m: fetch the counts
   std::vector<int32_t> counts(2 * count);
   if (use_mailbox) {
-    // one set: the kernel posts the counts to pinned host memory; spin on the sequence number
+    // the kernels post the counts to pinned host memory; spin until every word has been overwritten
     const auto t0 = std::chrono::steady_clock::now();
     long spins = 0;
     const volatile unsigned long long* box = reinterpret_cast<const volatile unsigned long long*>(ctx->mailbox);
-    const unsigned long long want = (unsigned long long)((unsigned)ctx->mailbox_seq & 0xffffu);
     for (int64_t i = 0; i < count; ++i) {
       unsigned long long w = box[i];
-      while ((w >> (2 * kMailboxCountBits)) != want) {
+      while (w == kMailboxEmpty) {
         if ((++spins & 0xfff) == 0 &&
             std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 10.0) {
           NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));  // surfaces a launch failure, if any
-          if ((box[i] >> (2 * kMailboxCountBits)) != want) NNV_FAIL(NNVHIP_ERR_HIP, "classification kernel did not report its counts");
+          if (box[i] == kMailboxEmpty) NNV_FAIL(NNVHIP_ERR_HIP, "classification kernel did not report its counts");
         }
         w = box[i];
       }
-      counts[2 * i] = (int32_t)((w >> kMailboxCountBits) & ((1u << kMailboxCountBits) - 1));
-      counts[2 * i + 1] = (int32_t)(w & ((1u << kMailboxCountBits) - 1));
+      int m_ = 0, inact_ = 0, seq_ = 0;
+      mailbox_unpack(w, &m_, &inact_, &seq_);
+      if (seq_ != (int)(ctx->mailbox_seq & 0xffffu)) NNV_FAIL(NNVHIP_ERR_HIP, "internal: mailbox word of another call");
+      counts[2 * i] = m_;
+      counts[2 * i + 1] = inact_;
     }
   } else {
     void* hc = nullptr;
