@@ -184,6 +184,20 @@ NNVHIP_API int nnvhip_estimate_ranges(nnvhip_ctx* ctx, nnvhip_star* s, double* l
 NNVHIP_API int nnvhip_estimate_ranges_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, double* lb,
                                  double* ub);
 
+/* Star.estimateRanges for callers that cannot allocate (no counterpart in the reference): code under
+ * HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same kernels and the
+ * same results as nnvhip_estimate_ranges, but the partial sums of the column pass go to a fixed
+ * workspace in device memory (32 MiB per GPU, held until the process ends) instead of the context's
+ * pool, nothing is cached on the handle, and the call issues no hipMalloc / hipFree / pool request.
+ * lb_dev / ub_dev: DEVICE pointers to N doubles each (either may be NULL); they are written on the
+ * context's stream (nnvhip_synchronize, or work queued on the same stream, orders later readers).
+ * Limits: the set must be a plain stored matrix (sets made by nnvhip_star_create / _from_box always
+ * are; a set whose rows or columns a layer left unwritten until first read is refused with
+ * NNVHIP_ERR_ARG) and 6 * roundup(N, 16) doubles must fit the workspace (N <= 699040), else
+ * NNVHIP_ERR_SHAPE.  All calls on one GPU share the workspace: calls that overlap on one GPU (two
+ * contexts, two threads) race; calls on one context are ordered by its stream. */
+NNVHIP_API int nnvhip_estimate_ranges_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, double* ub_dev);
+
 /* ---- layers ---------------------------------------------------------------------------- */
 /* FullyConnectedLayer(W, b), nn/layers/FullyConnectedLayer.m:39-99: W is M x K, b has M entries
  * (NULL = no bias, the affineMap(W, []) form). */

@@ -27,7 +27,7 @@ SYMBOLS = [
     "nnvhip_rowmap_destroy", "nnvhip_affine_rowmap", "nnvhip_avgpool2d_create", "nnvhip_avgpool2d_destroy",
     "nnvhip_avgpool2d_output_size", "nnvhip_affine_avgpool2d", "nnvhip_permute_rows",
     "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists", "nnvhip_probe_mfma_peak",
-    "nnvhip_debug_mailbox_pack", "nnvhip_debug_mailbox_unpack",
+    "nnvhip_estimate_ranges_static", "nnvhip_debug_mailbox_pack", "nnvhip_debug_mailbox_unpack",
     "nnvhip_debug_set_relu_call_number",
 ]
 
@@ -102,6 +102,7 @@ def load():
         "nnvhip_avgpool2d_output_size": [p, i64, i64, pi64, pi64],
         "nnvhip_affine_avgpool2d": [p, p, i64, i64, i64, pp, pp],
         "nnvhip_permute_rows": [p, i64, p, i64, pp, pp],
+        "nnvhip_estimate_ranges_static": [p, p, p, p],
         "nnvhip_debug_mailbox_pack": [C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_uint64)],
         "nnvhip_debug_mailbox_unpack": [C.c_uint64, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
                                         C.POINTER(C.c_int32)],

@@ -212,6 +212,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   memset((void*)c->mailbox, 0xff, sizeof(int64_t) * nnvhip_ctx::kMailboxSets);  // kMailboxEmpty everywhere
   NNV_HIP_TRY(hipEventCreate(&c->kev0));
   NNV_HIP_TRY(hipEventCreate(&c->kev1));
+  NNV_TRY(init_static_scratch(c));
   *out = c;
   return NNVHIP_OK;
 }
@@ -689,6 +690,13 @@ int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb,
 
 int nnvhip_estimate_ranges(nnvhip_ctx* c, nnvhip_star* s, double* lb, double* ub) {
   return nnvhip_estimate_ranges_batch(c, 1, &s, lb, ub);
+}
+
+int nnvhip_estimate_ranges_static(nnvhip_ctx* c, const nnvhip_star* s, double* lb_dev, double* ub_dev) {
+  CHECK_CTX(c);
+  if (!s || s->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid set handle");
+  if (!lb_dev && !ub_dev) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  return ranges_into_static(c, s, lb_dev, ub_dev);
 }
 
 int nnvhip_estimate_ranges_batch(nnvhip_ctx* c, int64_t count, nnvhip_star* const* s, double* lb, double* ub) {

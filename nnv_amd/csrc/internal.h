@@ -154,6 +154,10 @@ struct nnvhip_ctx {
   // stream synchronisation
   volatile int32_t* mailbox = nullptr;  // kMailboxSets words of 64 bits, one per set of an array
   static constexpr int64_t kMailboxSets = 8192;
+  // fixed workspace in device memory of the entry point that must not allocate (ranges.hip): this
+  // device's address of the array and its length
+  double* static_scratch = nullptr;
+  int64_t static_scratch_doubles = 0;
   uint32_t mailbox_seq = 0;  // number of the ReLU call (wraps; only its low 16 bits travel, as a cross-check)
   // FC layers as the full dense contraction (no skipping of structural zeros); default from the
   // environment variable NNVHIP_DENSE_AFFINE
@@ -401,6 +405,9 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, in
 
 // ranges.hip
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s);
+// the fixed device workspace: address look-up (once per context) and Star.estimateRanges into it
+int init_static_scratch(nnvhip_ctx* ctx);
+int ranges_into_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, double* ub_dev);
 // W * (scaled unit vectors): out(:, j) = W(:, idx[j]) * scale[idx[j]] for the one-hot column block of
 // every set (ranges.hip).  With part != null (one set) the four range sums of these columns are left
 // as `chunks` further chunks at part + part_chunk0, in the layout finalize_fused_ranges reads.

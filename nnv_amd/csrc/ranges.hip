@@ -525,6 +525,71 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
   return NNVHIP_OK;
 }
 
+// ---- estimateRanges without any allocation ----------------------------------------------------------
+// The column pass leaves one [4][ld] block of partial sums per column chunk, which the reduction kernel
+// then combines; nnvhip_estimate_ranges takes that workspace (and the lb / ub vectors) from the context's
+// pool.  The variant below takes both from a fixed array in device memory instead, so that it never
+// allocates.  Every GPU holds its own copy of the array at its own address: the address is looked up
+// once per context (with the context's device current) and the kernels get it as an argument.
+constexpr int64_t kStaticScratchDoubles = int64_t(4) << 20;  // 32 MiB per GPU, held until the process ends
+static __device__ __align__(256) double scratch[kStaticScratchDoubles];
+
+int init_static_scratch(nnvhip_ctx* ctx) {
+  void* p = nullptr;
+  NNV_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  ctx->static_scratch = static_cast<double*>(p);
+  ctx->static_scratch_doubles = kStaticScratchDoubles;
+  return NNVHIP_OK;
+}
+
+__global__ __launch_bounds__(256) void copy_ranges_kernel(const double* __restrict__ lb, const double* __restrict__ ub,
+                                                           double* __restrict__ lb_out, double* __restrict__ ub_out,
+                                                           int64_t N) {
+  const int64_t r = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (r < N) {
+    if (lb_out != nullptr) lb_out[r] = lb[r];
+    if (ub_out != nullptr) ub_out[r] = ub[r];
+  }
+}
+
+int ranges_into_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, double* ub_dev) {
+  if (ctx->static_scratch == nullptr) NNV_FAIL(NNVHIP_ERR_HIP, "internal: the static workspace has no address on this device");
+  // the set must be a plain stored matrix: writing pending columns or rows would need a buffer
+  if (s->rows_pending || s->cs.any_pending() || s->stored_cols() != s->n + 1)
+    NNV_FAIL(NNVHIP_ERR_ARG, "nnvhip_estimate_ranges_static: parts of this set are not in memory yet (read it once, or use "
+                             "nnvhip_estimate_ranges)");
+  const int64_t ld = s->ld, n = s->n;
+  if (n >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "too many predicate variables");
+  // workspace: lb (ld), ub (ld), then chunks x [4][ld] partial sums
+  if (6 * ld > ctx->static_scratch_doubles)
+    NNV_FAIL(NNVHIP_ERR_SHAPE, "nnvhip_estimate_ranges_static: a set of dimension %lld does not fit the static workspace "
+                               "(at most %lld rows)", (long long)s->N, (long long)(ctx->static_scratch_doubles / 6 / kLdAlign * kLdAlign));
+  const int64_t row_blocks = ceil_div(ld, kRowsPerWave);
+  int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(2048, row_blocks), ceil_div(n, 64)));
+  chunks = std::min<int64_t>(chunks, 1024);
+  chunks = std::min<int64_t>(chunks, (ctx->static_scratch_doubles - 2 * ld) / (4 * ld));  // >= 1, checked above
+  RangeDesc d{};
+  d.V = s->V;
+  d.plb = s->plb;
+  d.pub = s->pub;
+  d.lb = ctx->static_scratch;
+  d.ub = d.lb + ld;
+  d.part = d.ub + ld;
+  d.ld = ld;
+  d.n = (int32_t)n;
+  d.chunks = (int32_t)chunks;
+  d.cols_per_chunk = (int32_t)std::max<int64_t>(1, ceil_div(std::max<int64_t>(n, 1), chunks));
+  d.row_waves = 1;
+  hipLaunchKernelGGL((ranges_partial_kernel<8, 4>), dim3((unsigned)row_blocks, (unsigned)chunks, 1), dim3(64 * kRangeWaves), 0,
+                     ctx->stream, nullptr, d);
+  if (chunks > 1)
+    hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, 1), dim3(256), 0, ctx->stream, nullptr, d);
+  hipLaunchKernelGGL(copy_ranges_kernel, dim3((unsigned)ceil_div(s->N, 256)), dim3(256), 0, ctx->stream, d.lb, d.ub, lb_dev, ub_dev,
+                     s->N);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
 // ---- columns an FC map described but did not write ------------------------------------------------
 namespace {
 struct PendingCols {

@@ -9,6 +9,35 @@ from oracle import nnv_oracle as o
 RTOL = 1e-9  # north-star tolerance for fp64 values (relative to the array's scale)
 
 
+class DeviceDoubles:
+    """`count` doubles of device memory owned by the test (hipMalloc through the HIP runtime the library
+    itself is linked against), for entry points that take device pointers."""
+
+    def __init__(self, count, fill=np.nan):
+        import ctypes as C
+        from nnv_amd import _lib
+        _lib.load()                                   # brings the runtime into the process
+        self._hip = C.CDLL("libamdhip64.so.7")
+        self.count = int(count)
+        p = C.c_void_p()
+        assert self._hip.hipMalloc(C.byref(p), C.c_size_t(8 * self.count)) == 0
+        self.ptr = p
+        host = np.full(self.count, fill, dtype=np.float64)
+        assert self._hip.hipMemcpy(self.ptr, host.ctypes.data_as(C.c_void_p), C.c_size_t(8 * self.count), 1) == 0   # host to device
+
+    def get(self):
+        import ctypes as C
+        host = np.empty(self.count, dtype=np.float64)
+        assert self._hip.hipMemcpy(host.ctypes.data_as(C.c_void_p), self.ptr, C.c_size_t(8 * self.count), 2) == 0   # device to host
+        return host
+
+    def __del__(self):
+        try:
+            self._hip.hipFree(self.ptr)
+        except Exception:
+            pass
+
+
 def assert_close(got, exp, what, rtol=RTOL):
     got = np.asarray(got)
     exp = np.asarray(exp)
