@@ -1,24 +1,35 @@
 #!/usr/bin/env python3
 """Benchmark of the relax-star reach path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--method relax-star-area]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config k] [--method relax-star-area]
 
-A step is one full ``NN.reach`` of the benchmark configuration (default: config 2, the fully
-connected 784-1024-1024-1024-10 net with a 784-generator input box) with the input set and the
-weights already resident in HBM; it ends with the output set and its estimated output bounds
-resident in HBM.  Prints ONE JSON line:
+A step is one full ``NN.reach`` of a benchmark configuration with the input set(s) and the weights
+already resident in HBM; it ends with the output set(s) and their estimated output bounds resident in
+HBM.  Without ``--config`` all five configurations are measured in one run and ONE JSON line is printed:
 
+  headline       configuration 5 (the 1024 sub-boxes of config 2's input box, reached as one array on
+                 config 2's network) - the largest single-GPU workload: ``value``, ``ms_per_step``,
+                 ``roofline`` and ``cpu_baseline`` are its figures, over exactly K timed steps
+  per_config     the same fields for configurations 1-4 (their own step counts are stated)
   metric/value   generator-neuron updates per second = sum over layer steps of N_out*(n_out+1),
                  divided by reach wall-time (ms_per_step is the reach wall-time itself)
-  roofline       the dominant kernel (the fp64 MFMA GEMM of the hidden FC layers): dense flop
-                 2*M*K*(n+1) per launch over its HIP-event duration, against 78.6 TFLOP/s
-  cpu_baseline   the CPU oracle (numpy/OpenBLAS restatement of NNV's path, "port") timed on this
-                 host on a bounded sample of the same workload
+  roofline       the kernel group with the largest summed kernel time of a reach, whether it is bound by
+                 throughput or by latency: work of its launches over their summed durations (events that
+                 ride on the kernels' own dispatches), against 78.6 TFLOP/s (fp64 MFMA) or 8 TB/s (HBM);
+                 ``traffic`` = HBM bytes per launch from the counter tables in profiles/
+  cpu_baseline   the CPU oracle (numpy/OpenBLAS restatement of NNV's path, "port") timed on this host on
+                 a bounded sample of the same workload
+
+With ``--config k`` only that configuration is measured (k = 6: a CNN with normalisation / pooling /
+flatten layers); ``--lean`` then leaves out every extra pass, which is what the rocprofv3 summaries in
+profiles/ run.  Before anything is timed the device is kept busy with untimed steps for at least 0.3 s,
+whatever ``--warmup`` says, so that short step counts are measured on settled clocks.
 """
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -31,95 +42,140 @@ import nnv_amd  # noqa: E402
 
 FP64_MFMA_PEAK_TFLOPS = 78.6
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
-# scaled by the 1 GiB copy kernel of the same run (profiles/<workload>_hbm_traffic.md): (read, write) MiB
-# averaged over the launches of a step (dense GEMM: the 64x64, 64x96 and 128x80 tile instantiations; default
-# path: the mapped 64x64 GEMM over the kept rows; gather: the four FC layers, three of which leave their
-# columns unwritten)
-MEASURED_TRAFFIC_MIB = {("cfg2_fc_784_1024x3_10", "gemm_f64_kernel", "dense"): (51.30, 12.36),
-                        ("cfg2_fc_784_1024x3_10", "gemm_f64_kernel", "structured"): (8.89, 6.54),
-                        ("cfg2_fc_784_1024x3_10", "gather_columns_kernel", "structured"): (4.88, 0.79)}
+MIN_WARM_SECONDS = 0.3
+
+
+def profile_traffic(workload, kernel, variant=""):
+    """HBM bytes per launch of a kernel group from profiles/<workload>[_<variant>]_hbm_traffic.md (scaled
+    FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc runs; the table's last two columns are MiB read / written per
+    dispatch).  Instantiations of the group are averaged by their dispatch counts.  None if there is no table."""
+    path = os.path.join(ROOT, "profiles", "%s%s_hbm_traffic.md" % (workload, "_" + variant if variant else ""))
+    if not os.path.exists(path):
+        return None
+    disp, mib = 0, 0.0
+    for line in open(path):
+        m = re.match(r"\|\s*`([^`]+)`\s*\|\s*(\d+)\s*\|[^|]*\|[^|]*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|", line)
+        if m and kernel in m.group(1):
+            n = int(m.group(2))
+            disp += n
+            mib += n * (float(m.group(3)) + float(m.group(4)))
+    return round(mib / disp * 1048576.0) if disp else None
+
+
+def as_sets(s):
+    return s if isinstance(s, (list, nnv_amd.SetArray)) else [s]
 
 
 def layer_shapes(reach_set):
     out = []
     for s in reach_set:
-        sets = s if isinstance(s, (list, nnv_amd.SetArray)) else [s]
-        for t in sets:
+        for t in as_sets(s):
             N, n, _ = t._h.dims()
             out.append((N, n))
     return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None,
-                    help="timed steps (default: as many as fill about 0.3 s, between 10 and 1000)")
-    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: steps / 10, at least 5)")
-    ap.add_argument("--config", type=int, default=2)
-    ap.add_argument("--method", default="relax-star-area")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--dense", action="store_true",
-                    help="run every FC layer as the full dense contraction (no skipping of structural zeros)")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
-    ap.add_argument("--lean", action="store_true",
-                    help="only the timed steps and the per-kernel timing pass (no dense-contraction, host-to-host, "
-                         "all-sets-written and specification passes): what the rocprofv3 summaries in profiles/ run, so "
-                         "that their kernel tables hold the kernels of the measured path only")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only (sets shard across GPUs without communication; "
-                 "that path is not built) - use --gpus 1")
+def cpu_sample(cfg, method, updates, seconds):
+    """The oracle on this host, on a bounded sample of the workload: whole reaches where one fits the
+    budget; for the array of boxes as many of its sets as fit; for a network whose single reach takes
+    longer, its leading layers."""
+    from oracle import nnv_oracle as o
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    base = {"unit": "updates/s", "cores": threads, "kind": "port"}
+    if "partition" in cfg:
+        boxes = o.box_partition(cfg["lb"], cfg["ub"], cfg["partition"]["indexes"], cfg["partition"]["numbers"])
+        done, t_cpu, upd = 0, 0.0, 0
+        stride = max(1, len(boxes) // 64)          # spread over the array
+        for i in range(0, len(boxes), stride):
+            t1 = time.perf_counter()
+            _, sets = o.nn_reach(cfg["layers"], o.star_from_box(*boxes[i]), method, 1.0, keep=True)
+            t_cpu += time.perf_counter() - t1
+            upd += sum(s.V.shape[0] * s.V.shape[1] for s in sets)
+            done += 1
+            if t_cpu >= seconds:
+                break
+        base.update(value=upd / t_cpu, ms_per_set=round(1e3 * t_cpu / done, 2),
+                    ms_per_reach_extrapolated=round(1e3 * t_cpu / done * len(boxes), 1),
+                    sample="%d of the %d sets of %s, each reached on its own by the numpy/OpenBLAS oracle as the reference "
+                           "loops over an array (dense C built at every ReLU, as NNV does)" % (done, len(boxes), cfg["name"]))
+        return base
+    if cfg["kind"] == "image":
+        sh = cfg["image_shape"]
+        first = o.image_star_from_bounds(cfg["lb"].reshape(sh, order="F"), cfg["ub"].reshape(sh, order="F"))
+    else:
+        first = o.star_from_box(cfg["lb"], cfg["ub"])
+    # one layer at a time, so that a reach that does not fit the budget is cut after a whole layer
+    t_cpu, upd, n_reach, n_layers, partial = 0.0, 0, 0, len(cfg["layers"]), None
+    while t_cpu < seconds and n_reach < 200 and partial is None:
+        S = first
+        for li, L in enumerate(cfg["layers"]):
+            t1 = time.perf_counter()
+            S = o.nn_reach([L], S, method, 1.0)
+            t_cpu += time.perf_counter() - t1
+            V = S.V
+            upd += int(np.prod(V.shape))
+            if n_reach == 0 and t_cpu >= seconds and li + 1 < n_layers:
+                partial = li + 1
+                break
+        else:
+            n_reach += 1
+    base["value"] = upd / t_cpu
+    if partial is None:
+        base["ms_per_reach"] = round(1e3 * t_cpu / n_reach, 2)
+        base["sample"] = "%d full %s reach(es) by the numpy/OpenBLAS oracle (dense C built at every ReLU, as NNV does)" % (n_reach, cfg["name"])
+    else:
+        base["sample"] = ("the first %d of the %d layers of one %s reach by the numpy/OpenBLAS oracle (%.1f s; a whole reach "
+                          "does not fit the sample budget)" % (partial, n_layers, cfg["name"], t_cpu))
+    return base
 
+
+def measure(k, args, ctx, exact_steps, extras):
+    """One configuration: timed steps, per-kernel timing pass, and the passes named in `extras`
+    (a subset of {"dense", "h2h", "written", "spec", "cpu"})."""
     from nnv_amd.configs import count_updates, device_input_sets, make_config, make_extended_cnn
 
-    cfg = make_extended_cnn(32, 3) if args.config == 6 else make_config(args.config)
-    ctx = nnv_amd.default_context()
+    cfg = make_extended_cnn(32, 3) if k == 6 else make_config(k)
     ctx.set_dense_affine(args.dense)
     net = nnv_amd.NN.from_config(cfg["layers"], cfg["name"])
     opts = {"reachMethod": args.method, "relaxFactor": 1}
     dev_in = device_input_sets(cfg, ctx)
     lib, h = ctx.lib, ctx.handle
+    n_sets = len(dev_in) if isinstance(dev_in, (list, nnv_amd.SetArray)) else 1
 
     def step():
         out = net.reach(dev_in, opts)
-        outs = out if isinstance(out, (list, nnv_amd.SetArray)) else [out]
+        outs = as_sets(out)
         arr = outs.handles() if isinstance(outs, nnv_amd.SetArray) else (ctypes.c_void_p * len(outs))(*[o_._h.h for o_ in outs])
         # output bounds of all sets in one batched call, left on the device
         nnv_amd._lib.check(lib.nnvhip_estimate_ranges_batch(h, len(outs), arr, None, None))
         return out
 
-    if args.steps is None:
-        # a reach takes between 0.1 ms and 0.2 s depending on the workload: size the timed region so that
-        # clocks have settled and the timer's granularity does not matter
-        for _ in range(3):
-            step()
-        ctx.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(3):
-            step()
-        ctx.synchronize()
-        args.steps = int(min(1000, max(10, 0.3 / max((time.perf_counter() - t0) / 3, 1e-6))))
-    if args.warmup is None:
-        args.warmup = max(5, args.steps // 10)
+    # untimed steps until the device has been busy for MIN_WARM_SECONDS (clocks settled, pool blocks in
+    # place), then the W warm-up steps the caller asked for
+    n_warm, t0 = 0, time.perf_counter()
+    while n_warm < 3 or time.perf_counter() - t0 < MIN_WARM_SECONDS:
+        step()
+        n_warm += 1
+        if n_warm % 8 == 0:
+            ctx.synchronize()
+    ctx.synchronize()
+    t_step = (time.perf_counter() - t0) / n_warm
+    steps = args.steps if exact_steps else int(max(args.steps, min(1000, 0.2 / max(t_step, 1e-6))))
     for _ in range(args.warmup):
         step()
     ctx.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = step()
+    for _ in range(steps):
+        step()
     ctx.synchronize()
     wall = time.perf_counter() - t0
-    ms_per_step = 1e3 * wall / args.steps
+    ms_per_step = 1e3 * wall / steps
     shapes = layer_shapes(net.reachSet)
     updates = count_updates(shapes)
-    value = updates / (wall / args.steps)
+    value = updates / (wall / steps)
 
     # ---- per-layer and per-kernel timing with HIP events on the library's stream -----------------
-    # set_timing brackets every layer call (NN.reachTime) and, separately, every launch of the two
-    # MFMA kernels with their own event pair, so the kernel's duration excludes host gaps.
-    reps = max(5, min(args.steps, 20))
+    reps = max(5, min(steps, 20))
 
     def timed_pass(level):
         rs = dev_in
@@ -139,7 +195,7 @@ def main():
     per_layer = timed_pass(1)          # NN.reachTime-style device time per layer
     for grp in range(8):
         ctx.kernel_time(grp)
-    timed_pass(2)                      # per-kernel event pairs
+    timed_pass(2)                      # start / stop events on every dispatch of the timed kernel groups
     gemm_ms, gemm_launches, gemm_work = ctx.kernel_time(0)
     conv_ms, conv_launches, conv_work = ctx.kernel_time(1)
     rng_ms, rng_launches, rng_bytes = ctx.kernel_time(2)
@@ -152,15 +208,12 @@ def main():
     # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
     gemm_flop = conv_flop = 0.0
     relu_bytes, relu_ms = 0.0, 0.0
-    # bytes of the output columns the gather passes stand for (8 * rows per one-hot input column), whether
-    # a pass writes them or leaves them pending
     gat_dense_bytes = 0.0
-    onehot_cols = [s._h.dims()[1] for s in (dev_in if isinstance(dev_in, (list, nnv_amd.SetArray)) else [dev_in])] \
-        if cfg["layers"][0]["type"] == "fc" else None
+    onehot_cols = [s._h.dims()[1] for s in as_sets(dev_in)] if cfg["layers"][0]["type"] == "fc" else None
     layer_report = []
-    prev_sets = dev_in if isinstance(dev_in, (list, nnv_amd.SetArray)) else [dev_in]
+    prev_sets = as_sets(dev_in)
     for i, (Ld, L) in enumerate(zip(cfg["layers"], net.Layers)):
-        outs = net.reachSet[i] if isinstance(net.reachSet[i], (list, nnv_amd.SetArray)) else [net.reachSet[i]]
+        outs = as_sets(net.reachSet[i])
         entry = {"layer": i + 1, "type": Ld["type"], "ms": round(float(per_layer[i]), 4)}
         if Ld["type"] == "fc":
             M, K = Ld["W"].shape
@@ -188,14 +241,10 @@ def main():
             b = 0.0
             for sp, so in zip(prev_sets, outs):
                 N, n, _ = sp._h.dims()
-                m = so._h.dims()[1] - n
-                # read of the rows the step keeps + write of the N x (n+1+m) output, plus the
-                # estimateRanges read of V unless the producing FC layer already left the range sums
                 fused = i > 0 and cfg["layers"][i - 1]["type"] == "fc" and len(outs) == 1
                 ni, nc = ctypes.c_int64(), ctypes.c_int64()
                 nnv_amd._lib.check(ctx.lib.nnvhip_star_relu_counts(so._h.h, ctypes.byref(ni), ctypes.byref(nc)))
                 kept = N - ni.value - nc.value
-                # (the m appended unit-vector columns stay implicit unless a later read asks for them)
                 b += 8.0 * N * (n + 1) * (0 if fused else 1) + 8.0 * kept * (n + 1) + 8.0 * N * (n + 1)
             entry["algo_GBps"] = round(b / (per_layer[i] * 1e-3) / 1e9, 1)
             relu_bytes += b
@@ -225,7 +274,6 @@ def main():
                 "frac": round(g / HBM_PEAK_GBS, 4), "traffic": None, "launches_per_step": n_ // reps,
                 "avg_launch_ms": round(ms_ / n_, 5), "bytes_per_launch": b_ / n_, "ms_per_step": round(ms_ / reps, 5)}
 
-    # the dominant kernel group of a reach, by summed kernel time
     groups = []
     if gemm_launches:
         groups.append((gemm_ms, mfma_roofline("gemm_f64_kernel", gemm_work, gemm_flop, gemm_ms, gemm_launches)))
@@ -240,7 +288,7 @@ def main():
     if gat_launches:
         g = hbm_roofline("gather_columns_kernel", gat_ms, gat_launches, gat_bytes)
         if not ctx.eager_columns and not args.dense:
-            # all FC layers but the last leave the gathered columns unwritten (range sums only): those
+            # FC layers whose gathered columns nobody reads leave them unwritten (range sums only): those
             # launches run out of the cache-resident weights and are bound by L2 / ALU rate, not by HBM
             g["columns_left_unwritten"] = True
             if all(Ld["type"] in ("fc", "relu") for Ld in cfg["layers"]):   # (CNNs: the group also holds the stamp passes)
@@ -248,24 +296,27 @@ def main():
         groups.append((gat_ms, g))
     if fin_launches:
         groups.append((fin_ms, hbm_roofline("ranges_final_kernel", fin_ms, fin_launches, fin_bytes)))
+    if cls_launches:
+        # classification, sort of the crossing list and the new predicate bounds: one block per set of up
+        # to 8192 neurons - with a single input set a dependent chain on one CU, bound by latency, which
+        # the fraction of the HBM peak then shows
+        c = hbm_roofline("relu_classify_kernel", cls_ms, cls_launches, cls_bytes)
+        c["blocks_per_launch"] = n_sets
+        if n_sets < 256:
+            c["latency_bound"] = True
+        groups.append((cls_ms, c))
     groups.sort(key=lambda g: -g[0])
     roofline = dict(groups[0][1])
     roofline["other_kernels"] = [g[1] for g in groups[1:]]
-    n_sets = len(dev_in) if isinstance(dev_in, (list, nnv_amd.SetArray)) else 1
-    if cls_launches:
-        # One block per set (classification, in-block sort of the crossing list, new predicate bounds): a
-        # dependent chain on a single CU, bound by latency and not by a roofline.  It is listed with the
-        # bytes it touches; with a single input set it can be the longest kernel of a reach, and the
-        # roofline object above then describes the longest throughput-bound kernel.
-        c = hbm_roofline("relu_classify_kernel", cls_ms, cls_launches, cls_bytes)
-        c["latency_bound"] = True
-        c["blocks_per_launch"] = n_sets
-        roofline["other_kernels"].append(c)
-        if cls_ms > groups[0][0]:
-            roofline["longest_kernel_by_time"] = "relu_classify_kernel (latency bound, %d block(s) per launch)" % n_sets
+    variant = "dense_contraction" if args.dense else ""
+    if args.method == "relax-star-area":
+        roofline["traffic"] = profile_traffic(cfg["name"], roofline["kernel"], variant)
+        for g in roofline["other_kernels"]:
+            g["traffic"] = profile_traffic(cfg["name"], g["kernel"], variant)
+
     # the MFMA GEMM on the full dense problem of the same reach (what Star.affineMap executes in the
     # reference): a short extra pass with the skipping of structural zeros switched off
-    if gemm_launches and not args.dense and not args.lean:
+    if gemm_launches and not args.dense and "dense" in extras:
         ctx.set_dense_affine(True)
         step()
         ctx.synchronize()
@@ -282,13 +333,9 @@ def main():
         if d_launches:
             dr = mfma_roofline("gemm_f64_kernel", d_work, gemm_flop, d_ms, d_launches)
             dr["reach_ms_per_step"] = round(dense_ms_per_step, 5)
-            tr = MEASURED_TRAFFIC_MIB.get((cfg["name"], "gemm_f64_kernel", "dense"))
-            if tr is not None and args.method == "relax-star-area":
-                dr["traffic"] = round((tr[0] + tr[1]) * 1048576.0)
+            if args.method == "relax-star-area":
+                dr["traffic"] = profile_traffic(cfg["name"], "gemm_f64_kernel", "dense_contraction")
             roofline["dense_contraction"] = dr
-    t = MEASURED_TRAFFIC_MIB.get((cfg["name"], roofline["kernel"], "dense" if args.dense else "structured"))
-    if t is not None and args.method == "relax-star-area":
-        roofline["traffic"] = round((t[0] + t[1]) * 1048576.0)
     if relu_ms > 0:
         # bytes the dense materialisation of the ReLU steps would move (read V for the ranges, read the kept
         # rows, write the output) over the time the steps took; the steps leave most of that undone (pending
@@ -296,36 +343,42 @@ def main():
         roofline["relu_step_dense_equivalent_GBps"] = round(relu_bytes / (relu_ms * 1e-3) / 1e9, 1)
 
     # ---- the same step with the host buffers the boundary takes and returns (not `value`) -----------
-    # lb / ub uploaded and the input set built on the device, the reach, the output bounds back on the host
-    n_h2h = 0 if args.lean else max(5, min(args.steps, 50))
-    ctx.synchronize()
-    t1 = time.perf_counter()
-    fresh = res = None
-    for _ in range(n_h2h):
-        fresh = device_input_sets(cfg, ctx)
-        res = net.reach(fresh, opts)
-        nnv_amd.Star.estimateRanges_array(res if isinstance(res, (list, nnv_amd.SetArray)) else [res])
-    host_to_host_ms = 1e3 * (time.perf_counter() - t1) / max(n_h2h, 1)
-    del fresh, res
+    host_to_host = None
+    if "h2h" in extras:
+        n_h2h = max(5, min(steps, 50))
+        ctx.synchronize()
+        t1 = time.perf_counter()
+        fresh = res = None
+        for _ in range(n_h2h):
+            fresh = device_input_sets(cfg, ctx)
+            res = net.reach(fresh, opts)
+            nnv_amd.Star.estimateRanges_array(as_sets(res))
+        host_to_host = {"ms_per_step": round(1e3 * (time.perf_counter() - t1) / n_h2h, 4), "steps": n_h2h,
+                        "what": "input bounds uploaded and the set(s) built, reach, output bounds fetched to the host"}
+        del fresh, res
 
     # ---- the same step with every intermediate set written out in full (not `value`) -------------
     # By default the sets between the layers keep what nobody reads before the next layer as a description
     # (a ReLU's row reset and appended columns, columns gathered from the weights) and write it on first
-    # read; the returned set and its bounds are always written.  Here every layer writes its whole output.
-    all_written_ms = None
-    if not args.dense and not args.lean:
+    # read; the returned set and its bounds are always written.  Here every layer writes its whole output,
+    # which is what the reference's NN.reachSet{i} holds.
+    all_written = None
+    if not args.dense and "written" in extras:
         ctx.set_eager_columns(True)
         ctx.set_eager_relu(True)
         try:
             for _ in range(3):
                 step()
             ctx.synchronize()
-            n_aw = max(5, min(args.steps, 100))
+            n_aw = max(5, min(steps, 100))
             t1 = time.perf_counter()
             for _ in range(n_aw):
                 step()
             ctx.synchronize()
-            all_written_ms = 1e3 * (time.perf_counter() - t1) / n_aw
+            aw_ms = 1e3 * (time.perf_counter() - t1) / n_aw
+            all_written = {"ms_per_step": round(aw_ms, 5), "value": updates / (aw_ms * 1e-3), "steps": n_aw,
+                           "what": "the same step with every layer writing its whole output matrix in the call "
+                                   "(nothing left for a first read), as the reference's reachSet{i} holds it"}
         finally:
             ctx.set_eager_columns(False)
             ctx.set_eager_relu(False)
@@ -334,7 +387,7 @@ def main():
     # ---- specification check on the resident output sets (not part of `value`) -----------------
     spec = None
     last = net.Layers[-1]
-    if hasattr(last, "Bias") and len(last.Bias) > 1 and not args.lean:
+    if hasattr(last, "Bias") and len(last.Bias) > 1 and "spec" in extras:
         from nnv_amd import verify
         out_sets = net.reachSet[-1]
         hs = net.robustness_set(0, "max")
@@ -349,55 +402,81 @@ def main():
                 "decided_without_lp": int(np.sum(verdict != verify.HS_UNDECIDED)), "pairs": int(verdict.size),
                 "what": "LP-free pass of verify_specification for robustness_set(target=0): G*[c V], row bounds, verdicts"}
 
-    # practical HBM ceiling on this box: a plain copy kernel over 1 GiB (read + write bytes)
-    roofline["measured_mfma_TFLOPs"] = round(ctx.probe_mfma_peak(3), 2)     # register-resident MFMA loop
-    roofline["measured_copy_GBps"] = round(ctx.probe_copy_bandwidth(1 << 30, 5), 1)
+    single = not isinstance(dev_in, (list, nnv_amd.SetArray))
+    del dev_in, prev_sets
+    net.reachSet = []
+    del net
     ctx.trim_pool()
 
-    # ---- CPU baseline: the oracle on this host -------------------------------------------------
-    cpu = None
-    if not args.no_cpu:
-        from oracle import nnv_oracle as o
-        if "partition" in cfg:
-            ora_in = [o.star_from_box(l, u) for (l, u) in o.box_partition(
-                cfg["lb"], cfg["ub"], cfg["partition"]["indexes"], cfg["partition"]["numbers"])]
-        elif cfg["kind"] == "image":
-            sh = cfg["image_shape"]
-            ora_in = o.image_star_from_bounds(cfg["lb"].reshape(sh, order="F"), cfg["ub"].reshape(sh, order="F"))
-        else:
-            ora_in = o.star_from_box(cfg["lb"], cfg["ub"])
-        n_cpu, t_cpu = 0, 0.0
-        while t_cpu < args.cpu_seconds and n_cpu < 200:
-            t1 = time.perf_counter()
-            o.nn_reach(cfg["layers"], ora_in, args.method, 1.0)
-            t_cpu += time.perf_counter() - t1
-            n_cpu += 1
-        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-        cpu = {"value": updates / (t_cpu / n_cpu), "unit": "updates/s", "cores": threads, "kind": "port",
-               "ms_per_reach": round(1e3 * t_cpu / n_cpu, 2),
-               "sample": "%d full %s reach(es) by the numpy/OpenBLAS oracle (dense C built at every ReLU, as NNV does)"
-                         % (n_cpu, cfg["name"])}
+    cpu = cpu_sample(cfg, args.method, updates, args.cpu_seconds if exact_steps else args.cpu_seconds / 3.0) if "cpu" in extras else None
 
-    print(json.dumps({
-        "metric": "generator_neuron_updates_per_s", "value": value, "unit": "updates/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+    return {
+        "value": value, "steps": steps, "warmup": args.warmup, "warm_steps_by_time": n_warm, "ms_per_step": ms_per_step,
         "config": {"workload": cfg["name"], "reach_method": args.method, "relax_factor": 1,
                    "fc_affine_map": "dense" if args.dense else "structural zeros skipped (one-hot generator columns, reset rows); exact",
-                   "sets": len(dev_in) if isinstance(dev_in, (list, nnv_amd.SetArray)) else 1,
-                   "updates_per_step": updates,
+                   "sets": n_sets, "updates_per_step": updates,
                    "intermediate_sets": "dense" if args.dense else
                    "the sets between layers record a ReLU's row reset / appended columns and the columns an FC layer "
                    "gathers from its weights and write them on first read; the returned set and its bounds are written",
-                   "predicates_per_layer": [n for (_, n) in shapes][:len(net.Layers)] if not isinstance(dev_in, (list, nnv_amd.SetArray)) else None},
-        "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec,
-        "host_to_host": None if n_h2h == 0 else
-        {"ms_per_step": round(host_to_host_ms, 4), "steps": n_h2h,
-         "what": "input bounds uploaded and the set(s) built, reach, output bounds fetched to the host"},
-        "all_sets_written": None if all_written_ms is None else
-        {"ms_per_step": round(all_written_ms, 5), "value": updates / (all_written_ms * 1e-3),
-         "what": "the same step with every layer writing its whole output matrix in the call (nothing left for a first read)"},
-        "layers": layer_report,
+                   "predicates_per_layer": [n for (_, n) in shapes][:len(cfg["layers"])] if single else None},
+        "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec, "host_to_host": host_to_host,
+        "all_sets_written": all_written, "layers": layer_report,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20, help="timed steps of the headline configuration")
+    ap.add_argument("--warmup", type=int, default=5,
+                    help="untimed steps right before the timed ones (on top of the 0.3 s of untimed steps every run starts with)")
+    ap.add_argument("--config", type=int, default=None,
+                    help="measure this configuration only (1-5; 6: CNN with normalisation / pooling / flatten layers); "
+                         "default: all five, headline = config 5")
+    ap.add_argument("--method", default="relax-star-area")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--dense", action="store_true",
+                    help="run every FC layer as the full dense contraction (no skipping of structural zeros)")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0,
+                    help="budget of the headline's CPU baseline sample (the other configurations get a third each)")
+    ap.add_argument("--lean", action="store_true",
+                    help="only the timed steps and the per-kernel timing pass (no dense-contraction, host-to-host, "
+                         "all-sets-written and specification passes): what the rocprofv3 summaries in profiles/ run, so "
+                         "that their kernel tables hold the kernels of the measured path only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (sets shard across GPUs without communication; "
+                 "that path is not built) - use --gpus 1")
+
+    ctx = nnv_amd.default_context()
+    cpu = set() if args.no_cpu else {"cpu"}
+    if args.config is not None:
+        extras = cpu if args.lean else cpu | {"dense", "h2h", "written", "spec"}
+        head = measure(args.config, args, ctx, True, extras)
+        per_config = None
+    else:
+        # the four smaller configurations first (the headline's 6.6 GB arena then meets an empty pool)
+        per_config = []
+        for k in (1, 2, 3, 4):
+            extras = cpu if args.lean else cpu | {"written"} | ({"dense"} if k == 2 else set())
+            r = measure(k, args, ctx, False, extras)
+            r = {"metric": "generator_neuron_updates_per_s", "unit": "updates/s", **{kk: r[kk] for kk in
+                 ("value", "ms_per_step", "steps", "config", "roofline", "all_sets_written", "cpu_baseline")}}
+            per_config.append(r)
+        head = measure(5, args, ctx, True, cpu if args.lean else cpu | {"written", "spec", "h2h"})
+    # practical ceilings on this box: a register-resident MFMA loop and a plain copy kernel over 1 GiB
+    head["roofline"]["measured_mfma_TFLOPs"] = round(ctx.probe_mfma_peak(3), 2)
+    head["roofline"]["measured_copy_GBps"] = round(ctx.probe_copy_bandwidth(1 << 30, 5), 1)
+    ctx.trim_pool()
+
+    print(json.dumps({
+        "metric": "generator_neuron_updates_per_s", "value": head["value"], "unit": "updates/s", "n_gpus": 1,
+        "steps": head["steps"], "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": head["config"], "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"],
+        "warm_steps_by_time": head["warm_steps_by_time"],
+        "spec_check": head["spec_check"], "host_to_host": head["host_to_host"],
+        "all_sets_written": head["all_sets_written"], "layers": head["layers"], "per_config": per_config,
     }))
 
 
