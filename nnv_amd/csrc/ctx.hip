@@ -493,6 +493,7 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
   std::vector<double> center(N * count), vec(N * count);
   std::vector<int32_t> gen_dim;
   std::vector<int64_t> col_off(count + 1, 0), gen_off(count + 1, 0);
+  std::vector<char> neg_scale((size_t)count, 0);
   for (int64_t s = 0; s < count; ++s) {
     int64_t n = 0;
     for (int64_t i = 0; i < N; ++i) {
@@ -500,6 +501,7 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
       center[s * N + i] = 0.5 * (l + u);
       double v = 0.5 * (u - l);
       vec[s * N + i] = v;
+      if (v < 0.0) neg_scale[s] = 1;
       // zero columns are deleted only when the generator matrix has more than one element
       if (v != 0.0 || N == 1) {
         gen_dim.push_back((int32_t)i);
@@ -558,6 +560,7 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
       st->oh_idx = dgen->as<int32_t>() + gen_off[s];
       st->oh_scale_buf = dvec;
       st->oh_scale = dvec->as<double>() + s * N;
+      st->oh_scale_neg = neg_scale[s] != 0;
     }
     out[s] = st;
   }
@@ -1090,6 +1093,12 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         for (int64_t i = 0; i < count; ++i) max_m = std::max<int64_t>(max_m, gs[i].m);
         gch = gather_chunks_batch(outs[0]->ld, count, max_m);  // 0: nothing to gather
       }
+      // large arrays: the sums of the gathered columns come from one matrix product instead (gch_part = 0:
+      // the gather pass leaves no chunks)
+      bool use_mm = lazy_ok && gch > 0 && count >= 64;
+      for (int64_t i = 0; i < count; ++i) use_mm = use_mm && !(gs[i].m > 0 && in[i]->oh_scale_neg);
+      const int64_t gch_part = use_mm ? 0 : gch;
+      BufRef mm_sums;
       for (int64_t i = 0; i < count; ++i) {
         bool pack = false;
         any_rows = rows_of(i, &rws[i], &kps[i], &pack) || any_rows;
@@ -1147,7 +1156,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         const int64_t ldo = outs[0]->ld;
         for (int64_t i = 0; i < count; ++i) {
           tiles_of[i] = filled[i] ? 0 : ceil_div(dense[i], tn);
-          chunk_off[i + 1] = chunk_off[i] + tiles_of[i] + (gs[i].m > 0 ? gch : 0);
+          chunk_off[i + 1] = chunk_off[i] + tiles_of[i] + (gs[i].m > 0 ? gch_part : 0);
         }
         if (st == NNVHIP_OK && chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
         int64_t off = 0, off_in = 0, kp_max = kLdAlign;
@@ -1199,26 +1208,34 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         // that follows scans only the contracted columns
         const int64_t ldo = outs[0]->ld;
         if (!sums) {  // no segmented GEMM ran: the gather's chunks are all there is
-          for (int64_t i = 0; i < count; ++i) chunk_off[i + 1] = chunk_off[i] + (gs[i].m > 0 ? gch : 0);
+          for (int64_t i = 0; i < count; ++i) chunk_off[i + 1] = chunk_off[i] + (gs[i].m > 0 ? gch_part : 0);
           if (chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
         }
+        if (st == NNVHIP_OK && use_mm) st = launch_range_sums_mm(c, fc, count, gs.data(), &mm_sums);
         if (st == NNVHIP_OK) {
           for (int64_t i = 0; i < count; ++i) {
-            gs[i].part = (gch > 0 && gs[i].m > 0) ? sums->as<double>() + 4 * ldo * (chunk_off[i] + tiles_of[i]) : nullptr;
-            lazy[i] = lazy_ok && gs[i].part != nullptr;
+            gs[i].part = (gch_part > 0 && gs[i].m > 0) ? sums->as<double>() + 4 * ldo * (chunk_off[i] + tiles_of[i]) : nullptr;
+            lazy[i] = lazy_ok && (gs[i].part != nullptr || (use_mm && gs[i].m > 0));
             gs[i].lazy = lazy[i];
           }
-          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, ldo, count, gs.data(), gch);
+          st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, ldo, count, gs.data(), gch_part);
         }
       }
       // what the two passes left: the GEMM tiles' chunks cover the contracted columns, the gather's its own;
       // columns covered by neither (a GEMM without the fused sums) still need a scan, filled zeros add nothing
-      for (int64_t i = 0; i < count && st == NNVHIP_OK && sums; ++i) {
+      for (int64_t i = 0; i < count && st == NNVHIP_OK && (sums || mm_sums); ++i) {
         const int64_t nchunks = chunk_off[i + 1] - chunk_off[i];
-        if (nchunks == 0) continue;
-        outs[i]->rng_buf = sums;
-        outs[i]->rng_part = sums->as<double>() + 4 * outs[0]->ld * chunk_off[i];
-        outs[i]->rng_chunks = nchunks;
+        const bool mm = mm_sums && gs[i].m > 0;
+        if (nchunks == 0 && !mm) continue;
+        if (nchunks > 0) {
+          outs[i]->rng_buf = sums;
+          outs[i]->rng_part = sums->as<double>() + 4 * outs[0]->ld * chunk_off[i];
+          outs[i]->rng_chunks = nchunks;
+        }
+        if (mm) {
+          outs[i]->rng_mm_buf = mm_sums;
+          outs[i]->rng_mm = mm_sums->as<double>() + 4 * outs[0]->ld * i;  // two columns of 2 * ld entries per set
+        }
         outs[i]->rng_first_col = (filled[i] || tiles_of[i] > 0) ? 1 : dense[i];
       }
     } else {

@@ -267,6 +267,14 @@ struct nnvhip_star {
   const double* rng_part = nullptr;
   int64_t rng_chunks = 0;
   int64_t rng_first_col = 0;
+  // The same four sums for the gathered columns of a set in an array, as one matrix product left them
+  // (launch_range_sums_mm): two vectors of 2 * ld entries, [xmin1; xmax2] and then [xmax1; xmin2].  They
+  // cover columns from rng_first_col on, like the chunks above, and are added after them.
+  nnvhip::BufRef rng_mm_buf;
+  const double* rng_mm = nullptr;
+  bool has_producer_sums() const { return (rng_part != nullptr && rng_chunks > 0) || rng_mm != nullptr; }
+  // some scale of the unit-vector block is negative (a box with ub < lb): sign-split products do not apply
+  bool oh_scale_neg = false;
   // where gathered columns came from, and whether they (and leading zero columns) are in memory yet
   nnvhip::ColSource cs;
 };
@@ -276,6 +284,8 @@ struct nnvhip_fc {
   int64_t M = 0, K = 0, Mp = 0, Kp = 0;
   nnvhip::BufRef W;     // Mp x Kp, zero padded, ld = Mp
   nnvhip::BufRef bias;  // Mp entries (zero padded) or null
+  // [max(W, 0); min(W, 0)], 2*Mp x Kp with ld = 2*Mp: made on first use by launch_range_sums_mm
+  mutable nnvhip::BufRef Wpn;
 };
 
 struct nnvhip_conv2d {
@@ -441,6 +451,13 @@ int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m);
 // no range sums, the launcher picks the chunking.
 int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t Mp, int64_t ldout, int64_t count,
                           const GatherSet* sets, int64_t chunks);
+// Range sums of the gathered columns of every set of an array as one matrix product.  For a column
+// sc * e_r with sc >= 0 the product column is W(:, r) * sc, so
+//   sum_j max(v_ij, 0) * pl_j = sum_r max(W_ir, 0) * (sc_r * pl_r)   (and likewise for min and for pu):
+// with a = scatter(sc * plb), b = scatter(sc * pub) per set, [max(W,0); min(W,0)] * [a b] holds
+// [xmin1; xmax2] and [xmax1; xmin2].  One fp64 MFMA product over all sets instead of a pass over the
+// cache-resident weights per set.  out: 2*Mp x 2*count, ld = 2*Mp, columns 2i and 2i+1 belong to set i.
+int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out);
 // Turns the per-column-tile partial sums a fused GEMM left behind into the set's cached lb/ub.
 // cpart / cchunks / cbias: the centre column of s is still to be formed as the sum of cchunks partial
 // vectors (ld entries each) plus the bias (or null); the kernel writes it into column 0 of s first.

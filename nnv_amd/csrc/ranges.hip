@@ -17,6 +17,7 @@ struct RangeDesc {
   const double* pub;  // n
   double* part;       // [chunks][4][ld] partial sums (unused when chunks == 1 and chunks2 == 0)
   const double* part2;  // further chunks2 chunks left by the producer of the trailing columns, or null
+  const double* part3;  // sums of gathered columns from the matrix product: [xmin1; xmax2], [xmax1; xmin2] (2*ld each), or null
   int32_t chunks2;
   int32_t cchunks;      // > 0: the centre is the sum of cchunks vectors at cpart (ld apart) plus cbias (or
   const double* cpart;  // null), written to cout before it enters lb / ub
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(c
       xmax2.x += red[src][3][lane].x;
       xmax2.y += red[src][3][lane].y;
     }
-    if (d.chunks == 1 && d.chunks2 == 0) {
+    if (d.chunks == 1 && d.chunks2 == 0 && d.part3 == nullptr) {
       // lb = (c + xmin1) + xmin2, the reference's left-to-right order
       const double2 c = *reinterpret_cast<const double2*>(d.V + r0);
       *reinterpret_cast<double2*>(d.lb + r0) = make_double2((c.x + xmin1.x) + xmin2.x, (c.y + xmin1.y) + xmin2.y);
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(c
 // by four different waves so that the dependent add chains are short.
 __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
-  if (d.chunks == 1 && d.chunks2 == 0 && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
+  if (d.chunks == 1 && d.chunks2 == 0 && d.part3 == nullptr && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
   const int lane = threadIdx.x & 63;
   const int q = threadIdx.x >> 6;
   const int64_t r = (int64_t)blockIdx.x * 64 + lane;
@@ -171,6 +172,8 @@ __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __re
 #pragma unroll 8
       for (int c2 = 0; c2 < d.chunks2; ++c2) s += p2[(int64_t)c2 * 4 * d.ld];
     }
+    // xmin1, xmin2, xmax1, xmax2 sit in blocks 0, 3, 2, 1 of the product's two columns
+    if (d.part3 != nullptr) s += d.part3[(int64_t)((4 - q) & 3) * d.ld + r];
   }
   sums[q][lane] = s;
   __syncthreads();
@@ -205,7 +208,9 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   const int j0 = chunk * a.cols_per_chunk;
   double* part = a.with_sums ? d.part : nullptr;
   if (j0 >= d.m && part == nullptr && d.nfill == 0 && d.red == nullptr) return;
-  const int j1 = min(d.m, j0 + a.cols_per_chunk);
+  // a set whose columns stay unwritten and whose sums come from elsewhere has no column work here
+  const bool no_cols = d.lazy && part == nullptr && !(CENTRE && d.cin != nullptr);
+  const int j1 = no_cols ? j0 : min(d.m, j0 + a.cols_per_chunk);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t r0 = (int64_t)blockIdx.x * kRowsPerWave + 2 * lane;
@@ -228,8 +233,9 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   // A contraction over no rows at all leaves +0 everywhere and the bias on the centre: this chunk's share
   // of those columns is written here instead of by a GEMM launch (they add nothing to the range sums).
   if (d.nfill > 0 && active) {
-    const int fpc = (d.nfill + (int)gridDim.y - 1) / (int)gridDim.y;
-    const int f1 = min(d.nfill, (chunk + 1) * fpc);
+    const int nf = d.lazy ? 1 : d.nfill;  // unwritten columns: only the centre is stored
+    const int fpc = (nf + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int f1 = min(nf, (chunk + 1) * fpc);
     for (int j = chunk * fpc + wave; j < f1; j += kRangeWaves) {
       double2 o = make_double2(0.0, 0.0);
       if (j == 0 && d.bias != nullptr && r0 < a.Mp) {
@@ -336,14 +342,18 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
                           const GatherSet* sets, int64_t chunks) {
   if (count <= 0) return NNVHIP_OK;
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  const bool with_sums = chunks > 0;
+  // columns the launch has work for (a set that neither writes its columns nor wants their sums has none)
   int64_t max_m = 0, max_fill = 0;
   for (int64_t i = 0; i < count; ++i) {
-    max_m = std::max<int64_t>(max_m, sets[i].m);
-    max_fill = std::max<int64_t>(max_fill, sets[i].nfill);
+    const bool idle = sets[i].lazy && !(with_sums && sets[i].part != nullptr) && sets[i].cin == nullptr;
+    max_m = std::max<int64_t>(max_m, idle ? 0 : sets[i].m);
+    max_fill = std::max<int64_t>(max_fill, sets[i].lazy ? std::min<int32_t>(sets[i].nfill, 1) : sets[i].nfill);
   }
-  if (max_m == 0 && max_fill == 0) return NNVHIP_OK;
+  bool any_red = false;
+  for (int64_t i = 0; i < count; ++i) any_red = any_red || sets[i].red != nullptr;
+  if (max_m == 0 && max_fill == 0 && !any_red) return NNVHIP_OK;
   const int64_t row_blocks = ceil_div(ldout, kRowsPerWave);
-  const bool with_sums = chunks > 0;
   if (!with_sums) chunks = std::max<int64_t>(1, gather_chunks_batch(ldout, count, std::max(max_m, max_fill)));
   GatherArgs a{};
   a.W = W;
@@ -378,6 +388,56 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
   return NNVHIP_OK;
 }
 
+// ---- range sums of gathered columns as one matrix product --------------------------------------------
+__global__ __launch_bounds__(256) void split_sign_kernel(const double* __restrict__ W, double* __restrict__ Wpn, int64_t Mp,
+                                                          int64_t Kp) {
+  const int64_t total = Mp * Kp;
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = t % Mp, c = t / Mp;
+    const double w = W[t];
+    Wpn[r + c * 2 * Mp] = fmax(w, 0.0);
+    Wpn[Mp + r + c * 2 * Mp] = fmin(w, 0.0);
+  }
+}
+
+// Columns 2i and 2i+1 of X (Kp rows): a = scatter(sc * plb), b = scatter(sc * pub) of set i.
+__global__ __launch_bounds__(256) void sum_vectors_kernel(const GatherSet* __restrict__ table, double* __restrict__ X, int Kp) {
+  const GatherSet d = table[blockIdx.x];
+  double* xa = X + (int64_t)2 * blockIdx.x * Kp;
+  double* xb = xa + Kp;
+  for (int k = threadIdx.x; k < Kp; k += 256) {
+    xa[k] = 0.0;
+    xb[k] = 0.0;
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < d.m; j += 256) {
+    const int r = d.idx[j];
+    const double sc = d.scale != nullptr ? d.scale[r] : 1.0;
+    xa[r] = __dmul_rn(sc, d.plb[j]);
+    xb[r] = __dmul_rn(sc, d.pub[j]);
+  }
+}
+
+int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out) {
+  const int64_t Mp = fc->Mp, Kp = fc->Kp;
+  if (!fc->Wpn) {
+    BufRef w;
+    NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * Kp, &w));
+    hipLaunchKernelGGL(split_sign_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(Mp * Kp, 256), 4096)), dim3(256), 0, ctx->stream,
+                       fc->W->as<double>(), w->as<double>(), Mp, Kp);
+    NNV_HIP_TRY(hipGetLastError());
+    fc->Wpn = w;
+  }
+  BufRef X, tab;
+  NNV_TRY(ctx->alloc(sizeof(double) * Kp * 2 * count, &X));
+  NNV_TRY(ctx->upload(sets, sizeof(GatherSet) * count, &tab));
+  hipLaunchKernelGGL(sum_vectors_kernel, dim3((unsigned)count), dim3(256), 0, ctx->stream, tab->as<GatherSet>(), X->as<double>(), (int)Kp);
+  NNV_HIP_TRY(hipGetLastError());
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * count, out));
+  return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, 2 * count, Kp,
+                     nullptr);
+}
+
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   // sets that already carry ranges are skipped
   std::vector<nnvhip_star*> todo;
@@ -390,7 +450,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   {
     std::vector<nnvhip_star*> cols;
     for (auto* t : todo) {
-      const int64_t scan_end = (t->rng_part != nullptr && t->rng_chunks > 0 && t->rng_first_col >= 1) ? t->rng_first_col : t->n + 1;
+      const int64_t scan_end = (t->has_producer_sums() && t->rng_first_col >= 1) ? t->rng_first_col : t->n + 1;
       if ((t->cs.pending && scan_end > t->cs.from) || (t->cs.zero_to > 1 && scan_end > 1)) cols.push_back(t);
     }
     if (!cols.empty()) NNV_TRY(write_pending_columns(ctx, (int64_t)cols.size(), cols.data()));
@@ -417,7 +477,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   BufRef rb, pb;
   NNV_TRY(ctx->alloc(sizeof(double) * 2 * ld * nset, &rb));
   bool pending = false;
-  for (auto* t : todo) pending = pending || (t->rng_part != nullptr && t->rng_chunks > 0);
+  for (auto* t : todo) pending = pending || t->has_producer_sums();
   if (chunks > 1 || pending) NNV_TRY(ctx->alloc(sizeof(double) * 4 * ld * chunks * nset, &pb));
   std::vector<RangeDesc> descs(nset);
   bool any_pending = false;
@@ -437,15 +497,17 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     d.ub = d.lb + ld;
     d.row_waves = row_waves;
     d.part2 = nullptr;
+    d.part3 = nullptr;
     d.chunks2 = 0;
     d.cchunks = 0;
     d.cpart = nullptr;
     d.cbias = nullptr;
     d.cout = nullptr;
-    if (t->rng_part != nullptr && t->rng_chunks > 0 && t->rng_first_col >= 1) {
+    if (t->has_producer_sums() && t->rng_first_col >= 1) {
       // the producer of the trailing columns left their sums: scan only the columns before them
-      d.part2 = t->rng_part;
-      d.chunks2 = (int32_t)t->rng_chunks;
+      d.part2 = t->rng_chunks > 0 ? t->rng_part : nullptr;
+      d.chunks2 = d.part2 ? (int32_t)t->rng_chunks : 0;
+      d.part3 = t->rng_mm;
       d.n = (int32_t)(t->rng_first_col - 1);
       ch = std::max<int64_t>(1, std::min<int64_t>(chunks, ceil_div(std::max<int64_t>(d.n, 1), 64)));
       d.chunks = (int32_t)ch;
@@ -455,7 +517,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   }
   // every column of every set already has its sums from the producing kernels: no scan at all
   bool scan = false;
-  for (int64_t i = 0; i < nset; ++i) scan = scan || !(descs[i].n == 0 && descs[i].chunks2 > 0);
+  for (int64_t i = 0; i < nset; ++i) scan = scan || !(descs[i].n == 0 && (descs[i].chunks2 > 0 || descs[i].part3 != nullptr));
   if (!scan)
     for (int64_t i = 0; i < nset; ++i) descs[i].chunks = 0;
   const RangeDesc* table = nullptr;
@@ -488,6 +550,8 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     todo[i]->rng_buf.reset();  // the sums are folded in
     todo[i]->rng_part = nullptr;
     todo[i]->rng_chunks = 0;
+    todo[i]->rng_mm_buf.reset();
+    todo[i]->rng_mm = nullptr;
   }
   return NNVHIP_OK;
 }
@@ -510,6 +574,7 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
   d.cols_per_chunk = 0;
   d.row_waves = 1;
   d.part2 = nullptr;
+  d.part3 = nullptr;
   d.chunks2 = 0;
   d.cchunks = (int32_t)cchunks;
   d.cpart = cpart;
