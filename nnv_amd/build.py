@@ -14,7 +14,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libnnvhip.so")
-SOURCES = ["ctx.hip", "gemm.hip", "conv.hip", "ranges.hip", "relu.hip", "spec.hip", "elementwise.hip"]
+SOURCES = ["ctx.hip", "gemm.hip", "gemm_seg.hip", "conv.hip", "ranges.hip", "relu.hip", "spec.hip", "elementwise.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden",
@@ -31,7 +31,7 @@ def _run(cmd):
     return p.stdout
 
 
-def build(verbose: bool = False, jobs: int = 5) -> str:
+def build(verbose: bool = False, jobs: int = 8) -> str:
     """Compile every HIP source for gfx950 and link nnv_amd/libnnvhip.so.  Always recompiles."""
     os.makedirs(OBJ, exist_ok=True)
     objs = [os.path.join(OBJ, s.replace(".hip", ".o")) for s in SOURCES]

@@ -756,7 +756,8 @@ int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M,
   fc->K = K;
   fc->Mp = round_up(M, kLdAlign);
   fc->Kp = round_up(K, kLdAlign);
-  NNV_TRY(c->alloc(sizeof(double) * fc->Mp * fc->Kp, &fc->W));
+  // (128 doubles of slack: the tile kernel of gemm_seg.hip reads whole 128-row pieces of a column)
+  NNV_TRY(c->alloc(sizeof(double) * (fc->Mp * fc->Kp + 128), &fc->W));
   NNV_HIP_TRY(hipMemsetAsync(fc->W->ptr, 0, sizeof(double) * fc->Mp * fc->Kp, c->stream));
   NNV_HIP_TRY(hipMemcpy2DAsync(fc->W->ptr, sizeof(double) * fc->Mp, W, sizeof(double) * M, sizeof(double) * M, K,
                                hipMemcpyHostToDevice, c->stream));
@@ -1076,7 +1077,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
     } else if (contig) {
       // one launch for the whole array.  With structure to exploit, every set's dense columns are cut
       // into tiles of 128 that carry their own description (row list, position in the arena).
-      bool any_rows = false;
+      bool any_rows = false, bias_in_kernel = false;
       std::vector<GemmRows> rws((size_t)count);
       std::vector<int64_t> kps((size_t)count);
       std::vector<char> pk((size_t)count, 0);
@@ -1135,6 +1136,74 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         GemmRows rows;
         const int64_t tn = gemm_seg_cols(fc->Mp, count, dense.data());
         rows.seg_cols = (int32_t)tn;
+        // Large arrays whose sets all come with packed rows take the tile kernel of gemm_seg.hip: rows packed
+        // transposed, operands staged straight into LDS, a narrow last tile per set, bias added in the kernel.
+        bool seg_tiles = tn == 128 && !dense_only;
+        for (int64_t i = 0; i < count; ++i)
+          if (!filled[i] && (!pk[i] || kps[i] > 2048 || dense[i] >= (int64_t(1) << 24))) seg_tiles = false;
+        if (seg_tiles) {
+          const int64_t ldo = outs[0]->ld;
+          BufRef packed;
+          std::vector<PackSet> packs;
+          std::vector<const double*> bt((size_t)count, nullptr);
+          std::vector<int64_t> ldt((size_t)count, 0);
+          int64_t total = 0;
+          for (int64_t i = 0; i < count; ++i)
+            if (!filled[i]) {
+              ldt[i] = round_up(dense[i], 128);
+              total += kps[i] * ldt[i];
+            }
+          if (total > 0) st = c->alloc(sizeof(double) * total, &packed);
+          int64_t pos = 0;
+          for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
+            if (!filled[i]) {
+              bt[i] = packed->as<double>() + pos;
+              PackSet ps = pack_of(in[i], rws[i].kmap, packed->as<double>() + pos, kps[i], dense[i]);
+              ps.ldt = ldt[i];
+              packs.push_back(ps);
+              pos += kps[i] * ldt[i];
+            }
+          if (st == NNVHIP_OK && !packs.empty()) st = launch_pack_rows_t(c, (int64_t)packs.size(), packs.data());
+          for (int64_t i = 0; i < count; ++i) {
+            tiles_of[i] = filled[i] ? 0 : ceil_div(dense[i], 128);
+            chunk_off[i + 1] = chunk_off[i] + tiles_of[i] + (gs[i].m > 0 ? gch_part : 0);
+          }
+          if (st == NNVHIP_OK && chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
+          // tiles by width: [0] 128 columns, [1] 64, [2] 32 (the last tile of a set whose remainder fits)
+          std::vector<SegTile> tiles[3];
+          double flop[3] = {0.0, 0.0, 0.0};
+          int64_t off = 0;
+          for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
+            for (int64_t j = 0; j < dense[i] && !filled[i]; j += 128) {
+              const int64_t valid = std::min<int64_t>(128, dense[i] - j);
+              const int w = valid > 64 ? 0 : valid > 32 ? 1 : 2;
+              SegTile sg;
+              sg.kmap = rws[i].kmap;
+              sg.Bt = bt[i];
+              sg.ldbt = ldt[i];
+              sg.col_local0 = j;
+              sg.col_base = off + j;
+              sg.kp = (int32_t)kps[i];
+              sg.valid = (int32_t)valid;
+              sg.plb = outs[i]->plb;
+              sg.pub = outs[i]->pub;
+              sg.rpart = sums->as<double>() + 4 * ldo * (chunk_off[i] + j / 128);
+              tiles[w].push_back(sg);
+              flop[w] += 2.0 * (double)fc->Mp * (double)kps[i] * (double)valid;
+            }
+            off += in[i]->n + 1;
+          }
+          static const int widths[3] = {128, 64, 32};
+          for (int w = 0; w < 3 && st == NNVHIP_OK; ++w) {
+            if (tiles[w].empty()) continue;
+            BufRef dt;
+            st = c->upload_table(tiles[w].data(), sizeof(SegTile) * tiles[w].size(), &dt);
+            if (st == NNVHIP_OK)
+              st = launch_gemm_seg(c, Wd, fc->Mp, outs[0]->V, ldo, fc->Mp, bias, widths[w], dt->as<SegTile>(), (int64_t)tiles[w].size(),
+                                   flop[w]);
+          }
+          bias_in_kernel = true;
+        } else {
         // several row tiles would each gather the kept rows of B: pack them once per set instead
         BufRef packed;
         std::vector<PackSet> packs;
@@ -1190,10 +1259,11 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, tn * (int64_t)segs.size(),
                            kp_max, bias, nullptr, &rows);
         }
+        }
       } else {
         st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, cols, fc->Kp, bias);
       }
-      if (st == NNVHIP_OK && bias && count > 1) {
+      if (st == NNVHIP_OK && bias && count > 1 && !bias_in_kernel) {
         // the GEMM adds the bias to column 0 of the arena (the first set's centre); the other sets'
         // centres get it here (a set whose dense columns the gather pass fills has it from there)
         std::vector<double*> centres;

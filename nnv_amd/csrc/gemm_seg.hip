@@ -1,0 +1,333 @@
+// affineMap of a fully connected layer over an array of sets whose rows were mostly reset by the ReLU
+// step before it: C_s = W(:, kept_s) * [c V]_s(kept_s, :) for every set s, in one launch.
+//
+// Every set contracts over its own short list of kept rows (config 5: 240 of 1024), so the product is
+// cut into 128-row x TN-column tiles that each belong to one set (SegTile).  The B operand comes from the
+// set's packed rows, stored transposed (row k of the packed matrix = the set's columns, contiguous), and
+// the A operand is gathered column by column from the weight matrix; both reach LDS through the direct
+// global-to-LDS path (global_load_lds_dwordx4: no staging registers, four stages in flight), one 1 KiB
+// wave transfer per stage row.  The MFMA operand roles follow gemm.hip, but every lane owns FM consecutive
+// rows and FN consecutive columns of its wave's sub-tile: operands are read from LDS with 128-bit loads
+// and the result is stored in 128-bit pieces.  The epilogue leaves the tile's four Star.estimateRanges
+// partial sums (set/Star.m:1098-1104) as gemm.hip's fused epilogue does, and adds the bias to a set's
+// centre column.  Sets whose column count is not a multiple of 128 end in a narrower tile (32 or 64
+// columns) from a second launch, so a 785-column set costs 6.3 tiles instead of 7.
+#include <algorithm>
+#include <cstdlib>
+
+#include "internal.h"
+#include "mfma_tile.h"
+
+namespace nnvhip {
+
+typedef double double2_t __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int kSegTM = 128;  // rows of a tile
+constexpr int kSegKS = 8;    // rows of W / of the packed matrix per pipeline stage
+constexpr int kSegS = 4;     // stages in LDS
+constexpr int kSegNT = 512;  // threads per block
+
+#pragma clang diagnostic ignored "-Winline-asm"
+// 64 lanes x 16 bytes from global memory straight into LDS: lane l's 16 bytes at gbase + voff land at
+// lds_addr + 16 * l.  The compiler does not see the LDS write; the caller orders readers behind it with
+// wait_vm + block_barrier.  (m0 carries the LDS address of the transfer.)
+__device__ __forceinline__ void lds_dma16(const double* gbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase)
+               : "memory", "m0");
+}
+__device__ __forceinline__ unsigned lds_addr_of(const void* p) {
+  return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+__device__ __forceinline__ void block_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  // vmcnt <= N and nothing else (gfx9 encoding: vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8])
+  __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8));
+}
+
+// TN columns per tile; WR x WC waves, each owning (16*FM) rows x (16*FN) columns.
+template <int TN, int WR, int WC, int FM, int FN>
+__global__ __launch_bounds__(kSegNT, 4) void gemm_seg_kernel(const double* __restrict__ A, int64_t lda,
+                                                            double* __restrict__ C, int64_t ldc, int Mp,
+                                                            const double* __restrict__ bias, int tiles_m, int64_t tiles_n,
+                                                            int xr, int local_m, const SegTile* __restrict__ segs) {
+  static_assert(WR * WC == 8 && 16 * FM * WR == kSegTM && 16 * FN * WC == TN, "eight waves cover the tile");
+  constexpr int kStageA = kSegKS * kSegTM;        // doubles per stage of A
+  constexpr int kStageB = kSegKS * TN;            // ... of B
+  constexpr int kBLoads = kStageB / 128;          // 1 KiB wave transfers per stage of B
+  constexpr int kRed = WC * 4 * 4 * kSegTM;       // epilogue: [WC * 4 partials][4 sums][128 rows]
+  constexpr int kLds = kSegS * (kStageA + kStageB) > kRed ? kSegS * (kStageA + kStageB) : kRed;
+  __shared__ __attribute__((aligned(1024))) double smem[kLds];
+  __shared__ double pbs[2][TN];
+  double* const As = smem;
+  double* const Bs = smem + kSegS * kStageA;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr = wave % WR, wc = wave / WR;
+  const int l16 = lane & 15, q = lane >> 4;
+  // XCD-aware tile mapping, as in gemm.hip
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int xc = 8 / xr;
+  const int mt = (slot % local_m) * xr + (xcd % xr);
+  const int64_t nt = (int64_t)(slot / local_m) * xc + (xcd / xr);
+  if (mt >= tiles_m || nt >= tiles_n) return;
+  const int m0 = mt * kSegTM;
+  const SegTile sg = segs[nt];
+  const int nst = sg.kp / kSegKS;
+
+  // predicate bounds of the tile's columns (zero for the centre and for columns past the set's end, which
+  // then add nothing to the sums): loaded now, parked in a register, stored to LDS after the K loop
+  double pb_reg = 0.0;
+  if (tid < 2 * TN) {
+    const int t = tid % TN;
+    const int64_t sc = sg.col_local0 + t;
+    const bool ok = t < sg.valid && sc >= 1 && sg.rpart != nullptr;
+    const double* src = tid < TN ? sg.plb : sg.pub;
+    if (ok) pb_reg = src[sc - 1];
+  }
+  // row list: wave w stages row 8 * st + w of stage st; lane j keeps the entries of stages j, j + 64, ...
+  int kq[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int st = u * 64 + lane;
+    const int c = st < nst ? sg.kmap[st * kSegKS + wave] : 0;
+    kq[u] = c < 0 ? 0 : c;  // a padding entry: its packed row is zero, any column of W will do
+  }
+  const unsigned a_lds = lds_addr_of(As + wave * kSegTM);
+  const unsigned a_voff = lane * 16;
+  const double* a_base = A + m0;
+  // B: the stage's kSegKS x TN block is kBLoads transfers; transfer w (waves 0 .. kBLoads-1) brings 128 / TN rows
+  constexpr int kRowsPerLoad = 128 / TN;
+  const unsigned b_lds = lds_addr_of(Bs + wave * 128);
+  const unsigned b_voff = (unsigned)(((lane / (TN / 2)) * sg.ldbt + 2 * (lane % (TN / 2))) * 8);
+  const double* b_base = sg.Bt + sg.col_local0 + (int64_t)wave * kRowsPerLoad * sg.ldbt;
+  auto issue = [&](int st) {
+    const int u = st >> 6;
+    const int c = __builtin_amdgcn_readlane(u == 0 ? kq[0] : u == 1 ? kq[1] : u == 2 ? kq[2] : kq[3], st & 63);
+    const int b = st % kSegS;
+    lds_dma16(a_base + (int64_t)c * lda, a_voff, a_lds + (unsigned)(b * kStageA * 8));
+    if (wave < kBLoads) lds_dma16(b_base + (int64_t)st * kSegKS * sg.ldbt, b_voff, b_lds + (unsigned)(b * kStageB * 8));
+  };
+  // transfers a wave has in flight per stage (vmcnt is per wave)
+  const bool two = wave < kBLoads;
+
+  double4_t acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j) acc[i][j] = double4_t{0.0, 0.0, 0.0, 0.0};
+
+#pragma unroll
+  for (int st = 0; st < kSegS - 1; ++st)
+    if (st < nst) issue(st);
+
+  for (int t = 0; t < nst; ++t) {
+    // this wave's transfers of stage t have landed (those of up to two later stages may be in flight) ...
+    const int ahead = nst - 1 - t;
+    if (two) {
+      if (ahead >= kSegS - 2) wait_vm<2 * (kSegS - 2)>();
+      else if (ahead == 1) wait_vm<2>();
+      else wait_vm<0>();
+    } else {
+      if (ahead >= kSegS - 2) wait_vm<kSegS - 2>();
+      else if (ahead == 1) wait_vm<1>();
+      else wait_vm<0>();
+    }
+    block_barrier();  // ... and everybody's; everybody is done with stage t - 1, whose buffer the next transfer takes
+    if (t + kSegS - 1 < nst) issue(t + kSegS - 1);
+    const double* as = As + (t % kSegS) * kStageA + wr * (16 * FM) + l16 * FM;
+    const double* bs = Bs + (t % kSegS) * kStageB + wc * (16 * FN) + l16 * FN;
+#pragma unroll
+    for (int s = 0; s < kSegKS / 4; ++s) {
+      const int k = s * 4 + q;
+      double wv[FM], vv[FN];
+      if constexpr (FM == 4) {
+        const double2_t w01 = *reinterpret_cast<const double2_t*>(as + k * kSegTM);
+        const double2_t w23 = *reinterpret_cast<const double2_t*>(as + k * kSegTM + 2);
+        wv[0] = w01[0], wv[1] = w01[1], wv[2] = w23[0], wv[3] = w23[1];
+      } else if constexpr (FM == 2) {
+        const double2_t w01 = *reinterpret_cast<const double2_t*>(as + k * kSegTM);
+        wv[0] = w01[0], wv[1] = w01[1];
+      } else {
+        wv[0] = as[k * kSegTM];
+      }
+      if constexpr (FN == 2) {
+        const double2_t v01 = *reinterpret_cast<const double2_t*>(bs + k * TN);
+        vv[0] = v01[0], vv[1] = v01[1];
+      } else {
+        vv[0] = bs[k * TN];
+      }
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(vv[j], wv[i], acc[i][j], 0, 0, 0);
+    }
+  }
+  // lane (l16, q), accumulator (i, j), register r: row = wr*16*FM + l16*FM + i, column = wc*16*FN + (q + 4r)*FN + j
+
+  // ---- fused estimateRanges: partial sums of this column tile ------------------------------------
+  // xmin1 = sum max(v,0)*plb, xmin2 = sum min(v,0)*pub, xmax1 = sum max(v,0)*pub, xmax2 = sum min(v,0)*plb
+  if (sg.rpart != nullptr) {
+    if (tid < 2 * TN) pbs[tid / TN][tid % TN] = pb_reg;
+    __syncthreads();  // the stages are free, the bounds in place
+    double* red = smem;
+    double s[4][FM];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int i = 0; i < FM; ++i) s[a][i] = 0.0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int ct = wc * (16 * FN) + (q + 4 * r) * FN + j;
+        const double pl = pbs[0][ct], pu = pbs[1][ct];
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const double v = acc[i][j][r];
+          const double p = fmax(v, 0.0), n = fmin(v, 0.0);
+          s[0][i] = fma(p, pl, s[0][i]);
+          s[1][i] = fma(n, pu, s[1][i]);
+          s[2][i] = fma(p, pu, s[2][i]);
+          s[3][i] = fma(n, pl, s[3][i]);
+        }
+      }
+    const int part = wc * 4 + q;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      double* dst = red + (part * 4 + a) * kSegTM + wr * (16 * FM) + l16 * FM;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) dst[i] = s[a][i];
+    }
+    __syncthreads();
+    {  // the partial sums of a row are added in a fixed order
+      const int row = tid & (kSegTM - 1), a = tid >> 7;
+      double sum = 0.0;
+#pragma unroll
+      for (int pp = 0; pp < WC * 4; ++pp) sum += red[(pp * 4 + a) * kSegTM + row];
+      if (m0 + row < Mp) sg.rpart[(int64_t)a * ldc + m0 + row] = sum;
+    }
+  }
+
+  // ---- epilogue: bias on a set's centre column, FM consecutive rows per store -----------------------
+  const int row = m0 + wr * (16 * FM) + l16 * FM;
+  if (row < Mp) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int ct = wc * (16 * FN) + (q + 4 * r) * FN + j;
+        if (ct < sg.valid) {
+          double v[FM];
+#pragma unroll
+          for (int i = 0; i < FM; ++i) v[i] = acc[i][j][r];
+          if (bias != nullptr && sg.col_local0 + ct == 0) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) v[i] = v[i] + bias[row + i];
+          }
+          double* dst = C + (sg.col_base + ct) * ldc + row;
+          if constexpr (FM == 1) {
+            dst[0] = v[0];
+          } else {
+#pragma unroll
+            for (int i = 0; i < FM; i += 2) *reinterpret_cast<double2_t*>(dst + i) = double2_t{v[i], v[i + 1]};
+          }
+        }
+      }
+  }
+}
+
+// Packs the listed rows of a set's leading columns transposed: Vt(t, j) = V(kept[t], j) for t < kp
+// (zero where kept[t] < 0) and j < ncols, zero for ncols <= j < ldt; Vt is kp x ldt, row-major.  A block
+// transposes a 64 x 64 piece through LDS: it reads like pack_rows_kernel (lanes along the kept rows of one
+// column) and writes 512 contiguous bytes per row.
+__global__ __launch_bounds__(256) void pack_rows_t_kernel(const PackSet* __restrict__ table, PackSet one) {
+  const PackSet d = table ? table[blockIdx.z] : one;
+  const int t0 = blockIdx.x * 64, j0 = blockIdx.y * 64;
+  if (t0 >= d.kp || j0 >= d.ldt) return;
+  __shared__ double tile[64][65];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int t = t0 + lane;
+  const int ra = t < d.kp ? d.kept[t] : -1;
+  for (int cc = wave; cc < 64; cc += 4) {
+    const int j = j0 + cc;
+    double v = 0.0;
+    if (ra >= 0 && j < d.ncols && !(j >= 1 && j < d.zero_to)) {
+      if (d.W != nullptr && j >= d.wfrom && j < d.wend) {  // the value the gather pass wrote, recomputed
+        const int src = d.widx[j - d.wfrom];
+        const double sc = d.wscale ? d.wscale[src] : 1.0;
+        v = __dadd_rn(0.0, __dmul_rn(d.W[(int64_t)src * d.ldw + ra], sc));
+      } else {
+        v = d.V[(int64_t)j * d.ld + ra];
+      }
+    }
+    tile[cc][lane] = v;
+  }
+  __syncthreads();
+  const int j = j0 + lane;
+  if (j < d.ldt)
+    for (int kk = wave; kk < 64 && t0 + kk < d.kp; kk += 4) d.Vk[(int64_t)(t0 + kk) * d.ldt + j] = tile[lane][kk];
+}
+
+template <int TN, int WR, int WC, int FM, int FN>
+int launch_seg_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
+                   const SegTile* segs, int64_t ntiles, double flop) {
+  const int64_t tiles_m = ceil_div(Mp, kSegTM);
+  if (tiles_m * ntiles >= (int64_t(1) << 28)) NNV_FAIL(NNVHIP_ERR_SHAPE, "matrix too large for one launch");
+  // all row tiles of a column tile on one XCD, next to one another: the tile's packed rows are fetched once
+  // and the gathered columns of W (short row lists) stay in that XCD's L2
+  const int64_t xr = 1, local_m = tiles_m;
+  const int64_t slots = local_m * ceil_div(ntiles, 8 / xr);
+  const bool timed = ctx->kernel_timing;
+  NNV_LAUNCH(ctx, timed, (gemm_seg_kernel<TN, WR, WC, FM, FN>), dim3((unsigned)(8 * slots)), dim3(kSegNT), 0, A, lda, C, ldc, (int)Mp,
+             bias, (int)tiles_m, ntiles, (int)xr, (int)local_m, segs);
+  NNV_TRY(ctx->kernel_timer_end(timed, 0, flop));
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+}  // namespace
+
+int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {
+  if (count <= 0) return NNVHIP_OK;
+  if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
+  int64_t max_kp = 0, max_ld = 0;
+  for (int64_t i = 0; i < count; ++i) {
+    max_kp = std::max<int64_t>(max_kp, sets[i].kp);
+    max_ld = std::max<int64_t>(max_ld, sets[i].ldt);
+  }
+  if (max_kp == 0 || max_ld == 0) return NNVHIP_OK;
+  const PackSet* table = nullptr;
+  BufRef tab;
+  if (count > 1) {
+    NNV_TRY(ctx->upload_table(sets, sizeof(PackSet) * count, &tab));
+    table = tab->as<PackSet>();
+  }
+  hipLaunchKernelGGL(pack_rows_t_kernel, dim3((unsigned)ceil_div(max_kp, 64), (unsigned)ceil_div(max_ld, 64), (unsigned)count), dim3(256),
+                     0, ctx->stream, table, sets[0]);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+int launch_gemm_seg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
+                    int tn, const SegTile* segs, int64_t ntiles, double flop) {
+  if (ntiles == 0) return NNVHIP_OK;
+  if (Mp % 16 || lda % 2 || Mp > ldc) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: GEMM operands violate the padding contract");
+  switch (tn) {
+    case 128: return launch_seg_cfg<128, 2, 4, 4, 2>(ctx, A, lda, C, ldc, Mp, bias, segs, ntiles, flop);
+    case 64: return launch_seg_cfg<64, 4, 2, 2, 2>(ctx, A, lda, C, ldc, Mp, bias, segs, ntiles, flop);
+    case 32: return launch_seg_cfg<32, 4, 2, 2, 1>(ctx, A, lda, C, ldc, Mp, bias, segs, ntiles, flop);
+  }
+  NNV_FAIL(NNVHIP_ERR_ARG, "internal: no tile of %d columns", tn);
+}
+
+}  // namespace nnvhip

@@ -374,10 +374,30 @@ struct PackSet {
   int32_t wfrom = 0;
   int32_t wend = 0;
   int32_t zero_to = 0;  // > 1: columns [1, zero_to) are +0 whatever the memory holds
+  int64_t ldt = 0;      // launch_pack_rows_t: Vk is kp x ldt, row-major (columns [ncols, ldt) are written as zeros)
 };
 // the packing of the first `ncols` columns of a set, with what is known about where they came from
 PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t kp, int64_t ncols);
 int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
+
+// gemm_seg.hip: tiles of 128 rows x tn columns (tn = 128, 64 or 32), each belonging to one set:
+// C(:, col_base + [0, valid)) = A(:, kmap) * Bt(:, col_local0 + [0, valid)), with the bias on the column whose
+// number in the set (col_local0 + offset) is 0 and, with rpart, the tile's four range sums ([4][ldc]).
+struct SegTile {
+  const int32_t* kmap;  // kp entries (a multiple of 16), -1 where the list is padded
+  const double* Bt;     // the set's packed rows, transposed: kp x ldbt, row-major (launch_pack_rows_t)
+  int64_t ldbt;
+  int64_t col_local0;   // the tile's first column in the set's own numbering
+  int64_t col_base;     // ... and in C
+  int32_t kp;
+  int32_t valid;        // columns of the tile that exist
+  const double* plb;    // the set's predicate bounds (indexed by generator column), for the range sums
+  const double* pub;
+  double* rpart;        // or null
+};
+int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
+int launch_gemm_seg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
+                    int tn, const SegTile* segs, int64_t ntiles, double flop);
 // A split-K product leaves `ksplit` partial matrices (Mp x ncols each, ld = Mp) in a workspace; a caller
 // that has a pass over the output coming anyway can take the workspace instead of having the reduction
 // kernel launched (sum in split order, then the bias on column 0).  ksplit = 1: C is final.
