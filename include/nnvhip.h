@@ -231,6 +231,19 @@ NNVHIP_API int nnvhip_affine_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, 
  * three triangle constraints and predicate bounds [0, ub].  relax_factor must be 1 (no LP). */
 NNVHIP_API int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor, int64_t count,
                       nnvhip_star* const* in, nnvhip_star** out);
+/* The layer loop of NN.reach for a network made of the three layer kinds above, in one call
+ * (NN.reach_noConns, nn/NN.m:1529-1551: rs = Layers{i}.reach(rs, method, ...); reachSet{i} = rs).  Layer i is
+ * kind[i] = NNVHIP_LAYER_FC / _CONV2D / _RELU with handle layer[i] (nnvhip_fc*, nnvhip_conv2d*, NULL) and,
+ * for a convolution, the input image size hw[2*i], hw[2*i+1].  The result is what calling nnvhip_affine_fc /
+ * nnvhip_affine_conv2d / nnvhip_relu_relax one after the other gives -- the same kernels in the same order;
+ * only the host's work between the layers shrinks, which is what a reach of a small network consists of.
+ * out receives the n_layers * count handles of reachSet, layer-major (out[i*count + k] = set k after layer
+ * i); the sets of the last layer are written in full (nnvhip_set_eager_columns), as for a caller that hands
+ * them on.  On failure nothing is returned and every handle made on the way is released. */
+enum { NNVHIP_LAYER_FC = 0, NNVHIP_LAYER_CONV2D = 1, NNVHIP_LAYER_RELU = 2 };
+NNVHIP_API int nnvhip_reach_layers(nnvhip_ctx* ctx, int64_t n_layers, const int32_t* kind, const void* const* layer,
+                        const int64_t* hw, int order, double relax_factor, int64_t count, nnvhip_star* const* in,
+                        nnvhip_star** out);
 /* PosLin.multipleStepReachStarApprox_at_one(I.resetRow(reset_rows), index, lb, ub),
  * nn/funcs/PosLin.m:685-742 and set/Star.m:1442-1461: the step with the lists handed in instead of
  * derived from estimateRanges -- what the relaxFactor < 1 branches call once the host LPs

@@ -50,6 +50,11 @@ const TuneKnobs& tune_knobs() {
   return knobs;
 }
 
+int enter_ctx(nnvhip_ctx* ctx) {
+  NNV_HIP_TRY(hipSetDevice(ctx->device));
+  return NNVHIP_OK;
+}
+
 nnvhip_star* new_star(nnvhip_ctx* ctx) {
   nnvhip_star* s = new nnvhip_star();
   s->ctx = ctx;
@@ -181,7 +186,7 @@ int nnvhip_ctx::end_op() {
 #define CHECK_CTX(c)                                                  \
   do {                                                                \
     if (!(c)) NNV_FAIL(NNVHIP_ERR_ARG, "null context");               \
-    NNV_HIP_TRY(hipSetDevice((c)->device));                           \
+    NNV_TRY(nnvhip::enter_ctx(c));                                    \
   } while (0)
 
 extern "C" {
@@ -221,7 +226,7 @@ int nnvhip_destroy(nnvhip_ctx* c) {
   if (!c) return NNVHIP_OK;
   if (c->live_handles != 0)
     NNV_FAIL(NNVHIP_ERR_ARG, "context still has %lld live handles", (long long)c->live_handles);
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   c->trim();
   if (c->pinned) (void)hipHostFree(c->pinned);
   if (c->mailbox) (void)hipHostFree((void*)c->mailbox);
@@ -615,7 +620,7 @@ int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p) {
 int nnvhip_star_fetch_V(const nnvhip_star* s, double* V) {
   if (!s || !V) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   nnvhip_ctx* c = s->ctx;
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   NNV_TRY(ensure_dense(c, const_cast<nnvhip_star*>(s)));  // implicit columns are written out on first read
   NNV_HIP_TRY(hipMemcpy2DAsync(V, sizeof(double) * s->N, s->V, sizeof(double) * s->ld, sizeof(double) * s->N,
                                s->n + 1, hipMemcpyDeviceToHost, c->stream));
@@ -629,7 +634,7 @@ int nnvhip_star_fetch_rows(const nnvhip_star* s, int64_t R, const int32_t* rows,
   nnvhip_ctx* c = s->ctx;
   for (int64_t t = 0; t < R; ++t)
     if (rows[t] < 0 || rows[t] >= s->N) NNV_FAIL(NNVHIP_ERR_ARG, "Invalid index");
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   NNV_TRY(ensure_dense(c, const_cast<nnvhip_star*>(s)));
   // gather on the device into an Rp x (n+1) matrix (Rp = R rounded up to whole K-tiles, the packing
   // kernel's granularity), one contiguous copy, then drop the padding rows on the host
@@ -651,7 +656,7 @@ int nnvhip_star_fetch_rows(const nnvhip_star* s, int64_t R, const int32_t* rows,
 int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* lb, double* ub) {
   if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
   nnvhip_ctx* c = s->ctx;
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   if (s->n > 0) {
     if (lb) NNV_HIP_TRY(hipMemcpyAsync(lb, s->plb, sizeof(double) * s->n, hipMemcpyDeviceToHost, c->stream));
     if (ub) NNV_HIP_TRY(hipMemcpyAsync(ub, s->pub, sizeof(double) * s->n, hipMemcpyDeviceToHost, c->stream));
@@ -662,7 +667,7 @@ int nnvhip_star_fetch_pred_bounds(const nnvhip_star* s, double* lb, double* ub) 
 
 int nnvhip_star_fetch_constraints(const nnvhip_star* s, double* C, double* d) {
   if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
-  NNV_HIP_TRY(hipSetDevice(s->ctx->device));
+  NNV_TRY(nnvhip::enter_ctx(s->ctx));
   return materialize_constraints(s, C, d);
 }
 
@@ -678,7 +683,7 @@ int nnvhip_star_fetch_crossing(const nnvhip_star* s, int32_t* index, double* lb,
   if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
   if (s->n_crossing < 0) NNV_FAIL(NNVHIP_ERR_ARG, "set was not produced by the ReLU step");
   nnvhip_ctx* c = s->ctx;
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   const ConsNode* node = s->cons.get();
   int64_t m = s->n_crossing;
   if (m > 0) {
@@ -934,6 +939,16 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.cpart = nullptr;
       g.centre = nullptr;
     }
+    // One set whose gathered columns can stay unwritten and are either all the generators of a box star or the
+    // columns a ReLU step appended (with that step's per-row classes still on the handle): the output's lb / ub
+    // come from launch_fc_rowsum: one kernel over the weights instead of a gather pass plus a reduction.
+    const bool lazy_ok = !c->eager_cols && !dense_only;
+    const bool box_in = count == 1 && in[0]->oh_from == 1 && in[0]->oh_scale != nullptr && !in[0]->oh_scale_neg && dense[0] == 1 &&
+                        gs[0].m > 0;
+    const bool relu_in = count == 1 && in[0]->oh_from > 1 && in[0]->oh_scale == nullptr && gs[0].m > 0 && dense[0] == in[0]->oh_from &&
+                         in[0]->rows_pending && in[0]->cls != nullptr && in[0]->pre_ub != nullptr;
+    // (skinny layers keep the gather pass: a handful of 16-row blocks would not cover the chip)
+    bool rowsum = (box_in || relu_in) && fc->Mp >= 128 && fc->K < (int64_t(1) << 31);
     // sets whose implicit unit-vector columns take part in the contraction after all get them written out
     // (which also runs a pending row reset)
     std::vector<nnvhip_star*> full;
@@ -1000,8 +1015,50 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
     // follows works from the sums, and the next FC map either contracts over no row or packs its rows
     // from the weights.  lazy[i] is set where the sums are produced.
     std::vector<char> lazy((size_t)count, 0);
-    const bool lazy_ok = !c->eager_cols && !dense_only;
-    if (count == 1) {
+    if (count == 1 && rowsum && st == NNVHIP_OK) {
+      GemmRows rows;
+      int64_t kp = fc->Kp;
+      bool pack = false;
+      const bool compact = rows_of(0, &rows, &kp, &pack);
+      const int mode = box_in ? 0 : 1;
+      if (box_in) {
+        // the centre's product W * c + b is formed along the way: no GEMM launch at all
+        st = launch_fc_rowsum(c, fc, outs[0], mode, in[0]->oh_scale, nullptr, nullptr, 1, in[0]->V, nullptr, 0);
+        lazy[0] = lazy_ok;
+      } else if (compact && nothing_kept(0, rows)) {
+        // no row kept: the contracted columns are the bias and zeros, of which only the centre is stored
+        fill_by_gather(0);
+        st = launch_fc_rowsum(c, fc, outs[0], mode, nullptr, in[0]->cls, in[0]->pre_ub, 2, nullptr, nullptr, 0);
+        lazy[0] = lazy_ok;
+      } else {
+        RangeFuse fuse;
+        fuse.plb = outs[0]->plb;
+        fuse.pub = outs[0]->pub;
+        BufRef packed;
+        if (compact && pack) {
+          st = c->alloc(sizeof(double) * kp * dense[0], &packed);
+          if (st == NNVHIP_OK) {
+            PackSet ps = pack_of(in[0], in[0]->kept_idx, packed->as<double>(), kp, dense[0]);
+            st = launch_pack_rows(c, 1, &ps);
+            rows.Bk = packed->as<double>();
+            rows.ldbk = kp;
+          }
+        }
+        if (st == NNVHIP_OK)
+          st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
+                           compact ? &rows : nullptr);
+        if (st == NNVHIP_OK && fuse.chunks > 0) {
+          st = launch_fc_rowsum(c, fc, outs[0], mode, nullptr, in[0]->cls, in[0]->pre_ub, 0, nullptr, fuse.part->as<double>(), fuse.chunks);
+          lazy[0] = lazy_ok;
+        } else if (st == NNVHIP_OK) {
+          // the product was split along K and left no sums: the columns are written
+          if (st == NNVHIP_OK) st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), 0);
+        }
+      }
+      // a caller that wants the gathered columns in memory gets them written now (same values as a later
+      // first read would write)
+      if (st == NNVHIP_OK && outs[0]->lb != nullptr && !lazy_ok) st = launch_gather_columns(c, Wd, fc->Mp, fc->Mp, outs[0]->ld, 1, gs.data(), 0);
+    } else if (count == 1) {
       // one set: the GEMM epilogue also leaves the partial sums of Star.estimateRanges, so the
       // output set carries its ranges without another pass over V
       RangeFuse fuse;
@@ -1467,6 +1524,52 @@ int nnvhip_relu_relax(nnvhip_ctx* c, int order, double relax_factor, int64_t cou
   NNV_TRY(c->begin_op());
   NNV_TRY(relu_relax(c, order, count, in, out));
   return c->end_op();
+}
+
+int nnvhip_reach_layers(nnvhip_ctx* c, int64_t n_layers, const int32_t* kind, const void* const* layer, const int64_t* hw,
+                        int order, double relax_factor, int64_t count, nnvhip_star* const* in, nnvhip_star** out) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  if (n_layers < 0 || count <= 0 || !in || (n_layers > 0 && (!kind || !layer || !out))) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  nnvhip_star* const* cur = in;
+  int st = NNVHIP_OK;
+  int64_t done = 0;
+  for (int64_t l = 0; l < n_layers && st == NNVHIP_OK; ++l) {
+    nnvhip_star** dst = out + l * count;
+    // the set that is handed back is written in full by the layer that produces it
+    const bool eager = l == n_layers - 1 && !c->eager_cols;
+    if (eager) c->eager_cols = true;
+    switch (kind[l]) {
+      case NNVHIP_LAYER_FC:
+        st = nnvhip_affine_fc(c, static_cast<const nnvhip_fc*>(layer[l]), count, cur, dst);
+        break;
+      case NNVHIP_LAYER_CONV2D:
+        if (!hw) {
+          set_error("null argument");
+          st = NNVHIP_ERR_ARG;
+        } else {
+          st = nnvhip_affine_conv2d(c, static_cast<const nnvhip_conv2d*>(layer[l]), hw[2 * l], hw[2 * l + 1], count, cur, dst);
+        }
+        break;
+      case NNVHIP_LAYER_RELU:
+        st = nnvhip_relu_relax(c, order, relax_factor, count, cur, dst);
+        break;
+      default:
+        set_error("unknown layer kind %d", (int)kind[l]);
+        st = NNVHIP_ERR_ARG;
+    }
+    if (eager) c->eager_cols = false;
+    if (st == NNVHIP_OK) {
+      cur = dst;
+      done = l + 1;
+    }
+  }
+  if (st != NNVHIP_OK) {
+    for (int64_t t = 0; t < done * count; ++t) {
+      nnvhip_star_release(out[t]);
+      out[t] = nullptr;
+    }
+  }
+  return st;
 }
 
 int nnvhip_relu_apply_lists(nnvhip_ctx* c, nnvhip_star* in, int64_t n_reset, const int32_t* reset_rows, int64_t m,

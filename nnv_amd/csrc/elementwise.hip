@@ -293,7 +293,7 @@ extern "C" {
 int nnvhip_rowmap_create(nnvhip_ctx* c, int64_t N, int32_t n_steps, const int32_t* op, const int32_t* scope,
                          const double* params, nnvhip_rowmap** out) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   if (!op || !scope || !params || !out) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   if (N <= 0 || n_steps <= 0 || n_steps > kMaxSteps) NNV_FAIL(NNVHIP_ERR_SHAPE, "a row map has 1 to 8 steps");
   std::unique_ptr<nnvhip_rowmap> m(new nnvhip_rowmap());
@@ -328,7 +328,7 @@ int nnvhip_rowmap_destroy(nnvhip_rowmap* m) {
 int nnvhip_affine_rowmap(nnvhip_ctx* c, const nnvhip_rowmap* m, int64_t count, nnvhip_star* const* in,
                          nnvhip_star** out) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   if (!m || m->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid layer handle");
   NNV_TRY(check_set_array(c, count, in, out));
   for (int64_t i = 0; i < count; ++i)
@@ -390,7 +390,7 @@ int nnvhip_avgpool2d_output_size(const nnvhip_avgpool2d* p, int64_t H, int64_t W
 int nnvhip_affine_avgpool2d(nnvhip_ctx* c, const nnvhip_avgpool2d* p, int64_t H, int64_t W, int64_t count,
                             nnvhip_star* const* in, nnvhip_star** out) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   if (!p || p->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "invalid layer handle");
   NNV_TRY(check_set_array(c, count, in, out));
   if (H <= 0 || W <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "The input is not an ImageStar object");
@@ -425,7 +425,7 @@ int nnvhip_affine_avgpool2d(nnvhip_ctx* c, const nnvhip_avgpool2d* p, int64_t H,
 int nnvhip_permute_rows(nnvhip_ctx* c, int64_t N, const int32_t* src_row, int64_t count, nnvhip_star* const* in,
                         nnvhip_star** out) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   if (!src_row) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   NNV_TRY(check_set_array(c, count, in, out));
   for (int64_t i = 0; i < count; ++i)

@@ -134,6 +134,9 @@ struct ConsNode {
 };
 using ConsRef = std::shared_ptr<ConsNode>;
 
+// start of every entry point that touches device data: selects the context's device
+int enter_ctx(nnvhip_ctx* ctx);
+
 }  // namespace nnvhip
 
 struct nnvhip_ctx {
@@ -243,6 +246,9 @@ struct nnvhip_star {
   nnvhip::BufRef rbuf;
   double* lb = nullptr;
   double* ub = nullptr;
+  // set by the ReLU step: the estimated upper bounds of its input, by neuron (the range buffer is kept alive)
+  nnvhip::BufRef pre_ub_buf;
+  const double* pre_ub = nullptr;
   // filled for sets produced by the ReLU step
   int64_t n_inactive = -1;
   int64_t n_crossing = -1;
@@ -478,6 +484,10 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 // [xmin1; xmax2] and [xmax1; xmin2].  One fp64 MFMA product over all sets instead of a pass over the
 // cache-resident weights per set.  out: 2*Mp x 2*count, ld = 2*Mp, columns 2i and 2i+1 belong to set i.
 int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out);
+// lb / ub (and, by centre_mode, the centre column) of a fully connected layer's output for one set whose
+// gathered columns need no pass of their own, finished in one kernel (ranges.hip).
+int launch_fc_rowsum(nnvhip_ctx* ctx, const nnvhip_fc* fc, nnvhip_star* out, int mode, const double* scale, const int32_t* cls,
+                     const double* pre_ub, int centre_mode, const double* cin, const double* part, int64_t chunks);
 // Turns the per-column-tile partial sums a fused GEMM left behind into the set's cached lb/ub.
 // cpart / cchunks / cbias: the centre column of s is still to be formed as the sum of cchunks partial
 // vectors (ld entries each) plus the bias (or null); the kernel writes it into column 0 of s first.

@@ -388,6 +388,168 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
   return NNVHIP_OK;
 }
 
+// ---- lb / ub of a fully connected layer's output straight from the weights (one set) -----------------
+// The generator columns the layer gathers are W(:, r) * sc_r, one per input row r that carries a unit
+// vector, so their four range sums are signed dot products of a row of W with one vector:
+//   box star (bounds -1 / +1, sc >= 0):   S+ = sum_r max(W_ir, 0) * sc_r,  S- = sum_r min(W_ir, 0) * sc_r,
+//                                          xmin1 = -S+, xmin2 = S-, xmax1 = S+, xmax2 = -S-
+//   ReLU output (bounds 0 / ub_r, sc = 1): the same with sc_r = ub_r for crossing neurons (0 otherwise),
+//                                          xmin1 = xmax2 = 0, xmin2 = S-, xmax1 = S+.
+// One block owns 8 output rows and walks over all input rows: 8 lanes read 64 contiguous bytes of a column
+// of W, the eight lane groups and the sixteen waves take different columns, and the block ends with the
+// finished lb / ub of its rows (plus the partial sums the GEMM over the other columns left, plus the centre:
+// taken from memory, formed along the way as W * c + b, or just b).  No partial sums leave the kernel and no
+// reduction kernel follows.
+struct RowSumArgs {
+  const double* W;
+  int64_t ldw;
+  int32_t Mp, K;
+  int32_t mode;         // 0: box star (scale), 1: ReLU output (cls, pre_ub)
+  int32_t centre_mode;  // 0: the centre is in memory; 1: W * cin + bias, written; 2: 0 + bias, written
+  const double* scale;
+  const int32_t* cls;
+  const double* pre_ub;
+  const double* cin;
+  const double* bias;
+  double* centre;
+  const double* part;  // [chunks][4][ld] from the GEMM epilogue, or null
+  int32_t chunks;
+  int32_t pad_;
+  int64_t ld;
+  double* lb;
+  double* ub;
+};
+
+constexpr int kRowSumRows = 8;  // output rows per block
+
+__global__ __launch_bounds__(1024) void fc_rowsum_kernel(RowSumArgs a) {
+  __shared__ double red[16][3][kRowSumRows];
+  __shared__ double skey[4 * kRowSumRows];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rl = lane & 7, cs = lane >> 3;
+  const int row = blockIdx.x * kRowSumRows + rl;
+  const double* wrow = a.W + row;
+  const bool with_centre = a.centre_mode == 1;
+  double sp = 0.0, sn = 0.0, cacc = 0.0;
+  // 128 input rows per step (16 waves x 8 lane groups, 8 lanes = 64 contiguous bytes of a column of W);
+  // eight steps' loads -- none depends on another -- are issued before any is used
+  for (int r0 = wave * 8 + cs; r0 < a.K; r0 += 8 * 128) {
+    double w[8], b[8], cj[8];
+    int cl[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int r = r0 + u * 128;
+      w[u] = 0.0;
+      b[u] = 0.0;
+      cj[u] = 0.0;
+      cl[u] = -1;
+      if (r < a.K) {
+        w[u] = wrow[(int64_t)r * a.ldw];
+        if (a.mode == 0) {
+          b[u] = a.scale[r];
+          cl[u] = 0;
+        } else {
+          b[u] = a.pre_ub[r];
+          cl[u] = a.cls[r];
+        }
+        if (with_centre) cj[u] = a.cin[r];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const double bu = cl[u] >= 0 ? b[u] : 0.0;  // ReLU output: only crossing neurons carry a column
+      sp = fma(fmax(w[u], 0.0), bu, sp);
+      sn = fma(fmin(w[u], 0.0), bu, sn);
+      cacc = fma(w[u], cj[u], cacc);
+    }
+  }
+  // the eight lane groups, then the sixteen waves, in a fixed order
+#pragma unroll
+  for (int off = 8; off < 64; off <<= 1) {
+    sp += __shfl_xor(sp, off);
+    sn += __shfl_xor(sn, off);
+    cacc += __shfl_xor(cacc, off);
+  }
+  if (cs == 0) {
+    red[wave][0][rl] = sp;
+    red[wave][1][rl] = sn;
+    red[wave][2][rl] = cacc;
+  }
+  __syncthreads();
+  if (tid < 3 * kRowSumRows) {
+    const int which = tid / kRowSumRows, r8 = tid % kRowSumRows;
+    double t = 0.0;
+#pragma unroll
+    for (int w2 = 0; w2 < 16; ++w2) t += red[w2][which][r8];
+    red[0][which][r8] = t;  // (the thread's own slot: read before it is written)
+  }
+  __syncthreads();
+  if (tid < 4 * kRowSumRows) {  // sum q of a row: the GEMM tiles' chunks in order, then the gathered columns' term
+    const int q = tid / kRowSumRows, r8 = tid % kRowSumRows;
+    const int orow = blockIdx.x * kRowSumRows + r8;
+    double x = 0.0;
+    if (a.part != nullptr)
+      for (int c = 0; c < a.chunks; ++c) x += a.part[((int64_t)c * 4 + q) * a.ld + orow];
+    const double Sp = red[0][0][r8], Sn = red[0][1][r8];
+    double term;
+    if (a.mode == 0) term = q == 0 ? -Sp : q == 1 ? Sn : q == 2 ? Sp : -Sn;
+    else term = q == 1 ? Sn : q == 2 ? Sp : 0.0;
+    x += term;
+    skey[tid] = x;
+  }
+  __syncthreads();
+  if (tid < kRowSumRows) {
+    const int orow = blockIdx.x * kRowSumRows + tid;
+    double c0;
+    if (a.centre_mode == 0) {
+      c0 = a.centre[orow];
+    } else {
+      c0 = a.centre_mode == 1 ? red[0][2][tid] : 0.0;
+      if (a.bias != nullptr) c0 = c0 + a.bias[orow];
+      a.centre[orow] = c0;
+    }
+    // lb = (c + xmin1) + xmin2, the reference's left-to-right order (set/Star.m:1098-1104)
+    a.lb[orow] = (c0 + skey[tid]) + skey[kRowSumRows + tid];
+    a.ub[orow] = (c0 + skey[2 * kRowSumRows + tid]) + skey[3 * kRowSumRows + tid];
+  }
+}
+
+int launch_fc_rowsum(nnvhip_ctx* ctx, const nnvhip_fc* fc, nnvhip_star* out, int mode, const double* scale, const int32_t* cls,
+                     const double* pre_ub, int centre_mode, const double* cin, const double* part, int64_t chunks) {
+  BufRef rb;
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * out->ld, &rb));
+  RowSumArgs a{};
+  a.W = fc->W->as<double>();
+  a.ldw = fc->Mp;
+  a.Mp = (int32_t)fc->Mp;
+  a.K = (int32_t)fc->K;
+  a.mode = mode;
+  a.centre_mode = centre_mode;
+  a.scale = scale;
+  a.cls = cls;
+  a.pre_ub = pre_ub;
+  a.cin = cin;
+  a.bias = fc->bias ? fc->bias->as<double>() : nullptr;
+  a.centre = out->V;
+  a.part = part;
+  a.chunks = (int32_t)chunks;
+  a.ld = out->ld;
+  a.lb = rb->as<double>();
+  a.ub = a.lb + out->ld;
+  const int64_t row_blocks = fc->Mp / kRowSumRows;
+  // algorithmic bytes: W once, the finished ranges (timed with the gather passes it stands in for)
+  const double bytes = 8.0 * (double)fc->Mp * (double)fc->K + 16.0 * (double)fc->Mp;
+  NNV_LAUNCH(ctx, ctx->kernel_timing, fc_rowsum_kernel, dim3((unsigned)row_blocks), dim3(1024), 0, a);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
+  NNV_HIP_TRY(hipGetLastError());
+  out->rbuf = rb;
+  out->lb = a.lb;
+  out->ub = a.ub;
+  return NNVHIP_OK;
+}
+
 // ---- range sums of gathered columns as one matrix product --------------------------------------------
 __global__ __launch_bounds__(256) void split_sign_kernel(const double* __restrict__ W, double* __restrict__ Wpn, int64_t Mp,
                                                           int64_t Kp) {

@@ -44,7 +44,7 @@ extern "C" {
 int nnvhip_halfspace_check(nnvhip_ctx* c, int64_t count, nnvhip_star* const* sets, int64_t n_hs, const int64_t* row_ptr,
                            const double* G, const double* g, int64_t N, int32_t* verdict, double* lo, double* hi) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   if (!row_ptr || !G || !g || n_hs <= 0) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   if (row_ptr[0] != 0) NNV_FAIL(NNVHIP_ERR_ARG, "row_ptr must start at 0");
   for (int64_t h = 0; h < n_hs; ++h)
@@ -81,7 +81,7 @@ int nnvhip_halfspace_check(nnvhip_ctx* c, int64_t count, nnvhip_star* const* set
 int nnvhip_halfspace_rows(nnvhip_ctx* c, nnvhip_star* s, int64_t R, const double* G, const double* g, int64_t N,
                           double* C1, double* d1) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
-  NNV_HIP_TRY(hipSetDevice(c->device));
+  NNV_TRY(nnvhip::enter_ctx(c));
   if (!G || !g || R <= 0) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   NNV_TRY(check_sets(c, 1, &s, N));
   FcGuard map;

@@ -8,7 +8,7 @@ import numpy as np
 from .layers import Conv2DLayer, FullyConnectedLayer, ReluLayer
 from .layers_affine import (AveragePooling2DLayer, BatchNormalizationLayer, FlattenLayer, ImageInputLayer,
                             LayerS)
-from .sets import ImageStar, SetArray, Star
+from .sets import ImageStar, SetArray, Star, _Handle
 from .verify import HalfSpace, verify_specification
 
 
@@ -100,6 +100,8 @@ class NN:
         rs = inSet
         ctx = rs.ctx if isinstance(rs, SetArray) else (rs[0] if isinstance(rs, (list, tuple)) else rs).ctx
         timed = self.dis_opt == "display"
+        if not timed and self._reach_in_one_call(inSet, ctx):
+            return self.reachSet[-1]
         last = len(self.Layers) - 1
         for i, layer in enumerate(self.Layers):
             if timed:
@@ -122,6 +124,67 @@ class NN:
             self.reachSet[i] = rs
             earlier = None
         return rs
+
+    def _reach_in_one_call(self, inSet, ctx):
+        """The layer loop above as one library call (nnvhip_reach_layers) when the network consists of fully
+        connected, convolutional and ReLU layers and the method is a relax-star one at relaxFactor = 1: the same
+        layer operations in the same order, without a round trip through Python between them.  Fills reachSet
+        (reachTime stays zero: per-layer times need the loop, dis_opt = 'display').  False: not applicable."""
+        import ctypes as C
+        from . import _lib
+        from .layers import RELAX_ORDER, _as_list, _handles_array, _shapes
+        if self.reachMethod not in RELAX_ORDER or self.relaxFactor != 1 or not self.Layers:
+            return False
+        if not all(type(L) in (FullyConnectedLayer, Conv2DLayer, ReluLayer) for L in self.Layers):
+            return False
+        if self.reachOption not in (None, "", "single", "parallel") and not (isinstance(self.reachOption, (list, tuple)) and not self.reachOption):
+            return False
+        sets, single = _as_list(inSet)
+        if not len(sets):
+            return False
+        try:
+            shapes = _shapes(sets)
+        except TypeError:
+            return False
+        if shapes is not None and any(s is None or s != shapes[0] for s in shapes):
+            return False       # mixed arrays take the general loop
+        shape = None if shapes is None else shapes[0]
+        n, count = len(self.Layers), len(sets)
+        kind = (C.c_int32 * n)()
+        layer = (C.c_void_p * n)()
+        hw = (C.c_int64 * (2 * n))()
+        out_shapes = []
+        for i, L in enumerate(self.Layers):
+            if type(L) is FullyConnectedLayer:
+                size = sets[0].dim if shape is None else shape[0] * shape[1] * shape[2]
+                if size != L.InputSize:
+                    return False   # the loop raises the reference's error
+                kind[i], layer[i] = 0, L._weights(ctx).h
+                shape = None if shape is None else (1, 1, L.OutputSize)
+            elif type(L) is Conv2DLayer:
+                if shape is None or shape[2] != L.NumChannels:
+                    return False
+                kind[i], layer[i] = 1, L._weights(ctx).h
+                hw[2 * i], hw[2 * i + 1] = shape[0], shape[1]
+                ho, wo = L.output_size(shape[0], shape[1])
+                if ho < 1 or wo < 1:
+                    return False
+                shape = (ho, wo, L.NumFilters)
+            else:
+                kind[i], layer[i] = 2, None
+            out_shapes.append(shape)
+        out = (C.c_void_p * (n * count))()
+        _lib.check(ctx.lib.nnvhip_reach_layers(ctx.handle, n, kind, layer, hw, RELAX_ORDER[self.reachMethod], 1.0, count,
+                                               _handles_array(sets), out))
+        for i in range(n):
+            raw = (C.c_void_p * count)(*out[i * count:(i + 1) * count])
+            shp = out_shapes[i]
+            if single:
+                hd = _Handle(raw[0], ctx)
+                self.reachSet[i] = Star._from_handle(hd) if shp is None else ImageStar(_handle=hd, shape=shp)
+            else:
+                self.reachSet[i] = SetArray(ctx, raw, None if shp is None else [shp] * count)
+        return True
 
     # ---- robustness check (the consumer of the reach set) ---------------------------------
     def robustness_set(self, target, class_type="max"):
