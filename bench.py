@@ -192,9 +192,18 @@ def measure(k, args, ctx, exact_steps, extras):
         ctx.set_timing(0)
         return acc / reps
 
-    per_layer = timed_pass(1)          # NN.reachTime-style device time per layer
-    for grp in range(8):
+    # a small FC / ReLU network is reached by ONE launch (nnvhip_reach_layers): time that kernel on the step's own path
+    for grp in range(10):
         ctx.kernel_time(grp)
+    ctx.set_timing(2)
+    for _ in range(reps):
+        step()
+    ctx.set_timing(0)
+    chain_ms, chain_launches, chain_bytes = ctx.kernel_time(8)
+    for grp in range(10):
+        ctx.kernel_time(grp)
+
+    per_layer = timed_pass(1)          # NN.reachTime-style device time per layer (layer-by-layer calls)
     timed_pass(2)                      # start / stop events on every dispatch of the timed kernel groups
     gemm_ms, gemm_launches, gemm_work = ctx.kernel_time(0)
     conv_ms, conv_launches, conv_work = ctx.kernel_time(1)
@@ -306,8 +315,21 @@ def measure(k, args, ctx, exact_steps, extras):
             c["latency_bound"] = True
         groups.append((cls_ms, c))
     groups.sort(key=lambda g: -g[0])
-    roofline = dict(groups[0][1])
-    roofline["other_kernels"] = [g[1] for g in groups[1:]]
+    if chain_launches:
+        # the measured step is one launch of the whole-reach kernel, one block per set: a chain of dependent phases
+        # on one CU per set, bound by latency; the groups above belong to the layer-by-layer calls of the same
+        # network (what the per-layer times below were taken on) and are listed for comparison only
+        c = hbm_roofline("reach_chain_kernel", chain_ms, chain_launches, chain_bytes)
+        c["blocks_per_launch"] = n_sets
+        c["latency_bound"] = n_sets < 256
+        c["what"] = ("the whole reach in one launch (every layer's set written in full); bytes = weights read once per set "
+                     "+ every layer's output matrix written once")
+        roofline = c
+        roofline["other_kernels"] = []
+        roofline["layer_by_layer_kernels"] = [g[1] for g in groups]
+    else:
+        roofline = dict(groups[0][1])
+        roofline["other_kernels"] = [g[1] for g in groups[1:]]
     variant = "dense_contraction" if args.dense else ""
     if args.method == "relax-star-area":
         roofline["traffic"] = profile_traffic(cfg["name"], roofline["kernel"], variant)
@@ -416,6 +438,7 @@ def measure(k, args, ctx, exact_steps, extras):
                    "fc_affine_map": "dense" if args.dense else "structural zeros skipped (one-hot generator columns, reset rows); exact",
                    "sets": n_sets, "updates_per_step": updates,
                    "intermediate_sets": "dense" if args.dense else
+                   "every layer's set is written in full by the one launch that reaches the whole network" if chain_launches else
                    "the sets between layers record a ReLU's row reset / appended columns and the columns an FC layer "
                    "gathers from its weights and write them on first read; the returned set and its bounds are written",
                    "predicates_per_layer": [n for (_, n) in shapes][:len(cfg["layers"])] if single else None},

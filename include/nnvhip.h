@@ -101,7 +101,8 @@ NNVHIP_API int nnvhip_set_eager_relu(nnvhip_ctx* ctx, int enabled);
  * kernel; 2: estimateRanges column pass; 3: ReLU apply pass; 4: row-wise affine layers (row map,
  * average pooling, row permutation); 5: column gather of an FC layer (its one-hot generator columns);
  * 6: classification of the ReLU step (incl. the sort of the crossing list and, for sets of up to 8192
- * neurons, the new predicate bounds); 7: the reduction of range partial sums into lb / ub.
+ * neurons, the new predicate bounds); 7: the reduction of range partial sums into lb / ub; 8: the
+ * whole-reach kernel of small fully connected networks (nnvhip_reach_layers).
  * Returns accumulated kernel time,
  * launch count and work since the last reset.  Work is the flop executed for 0 and 1 (GEMM:
  * 2*Mp*Kp*ncols over the columns and rows the launch contracts, M and K padded to 16; conv:
@@ -109,7 +110,7 @@ NNVHIP_API int nnvhip_set_eager_relu(nnvhip_ctx* ctx, int enabled);
  * 2 (8*N*(n+1) + 16*n + 16*N per set), 3 (8*kept*(n+1) read + 8*N*(n+1+m) written per set, kept =
  * rows that are neither inactive nor crossing), 4 (8*(Nin + Nout)*(n+1) per set), 5 (8*M per
  * gathered column written + W read once), 6 (24*N per set, + 32*n when the bounds are written too)
- * and 7 (8*N*(4*chunks + 3) per set). */
+ * 7 (8*N*(4*chunks + 3) per set) and 8 (per set: 8*M*K per FC layer + 8*N_out*(n_out+1) per layer). */
 NNVHIP_API int nnvhip_kernel_time(nnvhip_ctx* ctx, int which, double* total_ms, int64_t* launches, double* total_work,
                        int reset);
 /* Measurement hook (no counterpart in the reference): runs a plain device-to-device copy kernel over
@@ -239,7 +240,16 @@ NNVHIP_API int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor
  * only the host's work between the layers shrinks, which is what a reach of a small network consists of.
  * out receives the n_layers * count handles of reachSet, layer-major (out[i*count + k] = set k after layer
  * i); the sets of the last layer are written in full (nnvhip_set_eager_columns), as for a caller that hands
- * them on.  On failure nothing is returned and every handle made on the way is released. */
+ * them on.  On failure nothing is returned and every handle made on the way is released.
+ * Small networks of FC and ReLU layers only (at most 32 layers, at most 512 neurons per layer, and a worst
+ * case -- every neuron of every ReLU layer crossing -- of at most 2^18 matrix entries per set over all
+ * layers) take ONE launch for the whole loop, one thread block per input set: such a reach is otherwise a
+ * chain of launches and host waits, each longer than its work.  Every set of reachSet is then written in
+ * full, in buffers sized for that worst case; values agree with the layer-by-layer calls to rounding (sums
+ * are cut differently), structure and index lists exactly unless a bound or a sort key ties to the last bit.
+ * nnvhip_set_small_chain(ctx, 0) (or the environment variable NNVHIP_NO_SMALL_CHAIN) keeps such networks
+ * on the layer-by-layer path. */
+NNVHIP_API int nnvhip_set_small_chain(nnvhip_ctx* ctx, int enabled);
 enum { NNVHIP_LAYER_FC = 0, NNVHIP_LAYER_CONV2D = 1, NNVHIP_LAYER_RELU = 2 };
 NNVHIP_API int nnvhip_reach_layers(nnvhip_ctx* ctx, int64_t n_layers, const int32_t* kind, const void* const* layer,
                         const int64_t* hw, int order, double relax_factor, int64_t count, nnvhip_star* const* in,

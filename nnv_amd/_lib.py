@@ -16,7 +16,7 @@ HS_DISJOINT, HS_UNDECIDED, HS_INSIDE = 1, 2, 3
 # every entry point declared in include/nnvhip.h
 SYMBOLS = [
     "nnvhip_create", "nnvhip_destroy", "nnvhip_last_error", "nnvhip_synchronize", "nnvhip_set_timing",
-    "nnvhip_last_op_time_ms", "nnvhip_set_dense_affine", "nnvhip_set_eager_columns", "nnvhip_set_eager_relu", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
+    "nnvhip_last_op_time_ms", "nnvhip_set_dense_affine", "nnvhip_set_eager_columns", "nnvhip_set_eager_relu", "nnvhip_set_small_chain", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
     "nnvhip_trim_pool", "nnvhip_pool_stats", "nnvhip_star_create",
     "nnvhip_star_from_box", "nnvhip_star_retain", "nnvhip_star_release", "nnvhip_star_release_array", "nnvhip_star_dims",
     "nnvhip_star_fetch_V", "nnvhip_star_fetch_pred_bounds", "nnvhip_star_fetch_constraints",
@@ -63,6 +63,7 @@ def load():
         "nnvhip_set_dense_affine": [p, C.c_int],
         "nnvhip_set_eager_columns": [p, C.c_int],
         "nnvhip_set_eager_relu": [p, C.c_int],
+        "nnvhip_set_small_chain": [p, C.c_int],
         "nnvhip_last_op_time_ms": [p, C.POINTER(dbl)],
         "nnvhip_kernel_time": [p, C.c_int, C.POINTER(dbl), pi64, C.POINTER(dbl), C.c_int],
         "nnvhip_probe_copy_bandwidth": [p, i64, C.c_int, C.POINTER(dbl)],
@@ -174,6 +175,11 @@ class Context:
         """True: the ReLU step writes its whole output matrix in the call (reset rows zeroed, appended
         columns stored); False (default): both are recorded on the handle and written on first read."""
         check(self.lib.nnvhip_set_eager_relu(self.handle, 1 if enabled else 0))
+
+    def set_small_chain(self, enabled):
+        """True (default): NN.reach of a small FC / ReLU network is one launch (nnvhip_reach_layers); False: such
+        networks go layer by layer like every other."""
+        check(self.lib.nnvhip_set_small_chain(self.handle, 1 if enabled else 0))
 
     def set_dense_affine(self, enabled):
         """True: FC layers run as the full dense contraction; False (default): products with the

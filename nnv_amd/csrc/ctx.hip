@@ -210,6 +210,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->eager_rows = getenv("NNVHIP_EAGER_ROWS") != nullptr;
   c->eager_cols = getenv("NNVHIP_EAGER_COLS") != nullptr;
   c->poison_pending = getenv("NNVHIP_POISON_PENDING") != nullptr;
+  c->small_chain = getenv("NNVHIP_NO_SMALL_CHAIN") == nullptr;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
@@ -269,6 +270,12 @@ int nnvhip_set_eager_relu(nnvhip_ctx* c, int enabled) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
   c->eager_rows = enabled != 0;
   c->eager_tail = enabled != 0;
+  return NNVHIP_OK;
+}
+
+int nnvhip_set_small_chain(nnvhip_ctx* c, int enabled) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  c->small_chain = enabled != 0;
   return NNVHIP_OK;
 }
 
@@ -1533,6 +1540,21 @@ int nnvhip_reach_layers(nnvhip_ctx* c, int64_t n_layers, const int32_t* kind, co
   nnvhip_star* const* cur = in;
   int st = NNVHIP_OK;
   int64_t done = 0;
+  if (n_layers > 0 && relax_factor == 1.0) {
+    // small fully connected networks: the whole loop below as one launch
+    NNV_TRY(nnvhip::enter_ctx(c));
+    bool taken = false;
+    for (int64_t t = 0; t < n_layers * count; ++t) out[t] = nullptr;
+    st = reach_small_chain(c, n_layers, kind, layer, order, count, in, out, &taken);
+    if (taken) {
+      if (st != NNVHIP_OK)
+        for (int64_t t = 0; t < n_layers * count; ++t) {
+          nnvhip_star_release(out[t]);
+          out[t] = nullptr;
+        }
+      return st;
+    }
+  }
   for (int64_t l = 0; l < n_layers && st == NNVHIP_OK; ++l) {
     nnvhip_star** dst = out + l * count;
     // the set that is handed back is written in full by the layer that produces it

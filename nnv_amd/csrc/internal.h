@@ -172,6 +172,9 @@ struct nnvhip_ctx {
   bool eager_rows = false;
   // FC maps always write the columns they gather (environment NNVHIP_EAGER_COLS)
   bool eager_cols = false;
+  // small fully connected networks are reached in one launch (chain.hip); environment NNVHIP_NO_SMALL_CHAIN
+  // or nnvhip_set_small_chain(ctx, 0) keeps them on the layer-by-layer path
+  bool small_chain = true;
   // debugging aid (environment NNVHIP_POISON_PENDING): columns left unwritten are filled with NaNs
   bool poison_pending = false;
   // per-layer timing
@@ -185,7 +188,8 @@ struct nnvhip_ctx {
   // [2] estimateRanges column pass, [3] ReLU apply pass, [4] row-wise affine layers (batch
   // normalisation, input normalisation, average pooling, flatten), [5] gather of W's columns for the
   // one-hot generator columns of an FC layer (work = algorithmic bytes)
-  static constexpr int kKernelGroups = 8;
+  // [6] ReLU classification, [7] range reduction, [8] whole-reach kernel of small networks (chain.hip)
+  static constexpr int kKernelGroups = 10;
   double kern_ms[kKernelGroups] = {};
   int64_t kern_launches[kKernelGroups] = {};
   double kern_flop[kKernelGroups] = {};
@@ -513,5 +517,10 @@ struct ReluGiven {
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out,
                const ReluGiven* given = nullptr);
 int materialize_constraints(const nnvhip_star* s, double* C_host, double* d_host);
+
+// chain.hip: the layer loop of a small FC / ReLU network as one launch (one block per set).  *taken = false:
+// not applicable (nothing was done; the caller runs the layer loop).  out: n_layers x count handles.
+int reach_small_chain(nnvhip_ctx* c, int64_t n_layers, const int32_t* kind, const void* const* layer, int order, int64_t count,
+                      nnvhip_star* const* in, nnvhip_star** out, bool* taken);
 
 }  // namespace nnvhip

@@ -149,6 +149,7 @@ class NN:
         if shapes is not None and any(s is None or s != shapes[0] for s in shapes):
             return False       # mixed arrays take the general loop
         shape = None if shapes is None else shapes[0]
+        dim = sets[0].dim if shape is None else shape[0] * shape[1] * shape[2]   # dimension of the current layer's input
         n, count = len(self.Layers), len(sets)
         kind = (C.c_int32 * n)()
         layer = (C.c_void_p * n)()
@@ -156,11 +157,11 @@ class NN:
         out_shapes = []
         for i, L in enumerate(self.Layers):
             if type(L) is FullyConnectedLayer:
-                size = sets[0].dim if shape is None else shape[0] * shape[1] * shape[2]
-                if size != L.InputSize:
+                if dim != L.InputSize:
                     return False   # the loop raises the reference's error
                 kind[i], layer[i] = 0, L._weights(ctx).h
                 shape = None if shape is None else (1, 1, L.OutputSize)
+                dim = L.OutputSize
             elif type(L) is Conv2DLayer:
                 if shape is None or shape[2] != L.NumChannels:
                     return False
@@ -170,6 +171,7 @@ class NN:
                 if ho < 1 or wo < 1:
                     return False
                 shape = (ho, wo, L.NumFilters)
+                dim = ho * wo * L.NumFilters
             else:
                 kind[i], layer[i] = 2, None
             out_shapes.append(shape)
