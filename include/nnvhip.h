@@ -136,6 +136,13 @@ NNVHIP_API int nnvhip_debug_set_relu_call_number(nnvhip_ctx* ctx, int64_t call_n
 NNVHIP_API int nnvhip_trim_pool(nnvhip_ctx* ctx);
 /* Bytes currently handed out by / cached in the pool. */
 NNVHIP_API int nnvhip_pool_stats(nnvhip_ctx* ctx, int64_t* bytes_in_use, int64_t* bytes_cached);
+/* Host-to-device traffic of the context since it was created (no counterpart in the reference, whose arrays
+ * never leave the host): the number of layers whose weights were uploaded (nnvhip_fc_create /
+ * nnvhip_conv2d_create calls that did not find their arrays resident), the bytes of those uploads, and all
+ * bytes the library copied from host to device (sets, bounds, weights, descriptor tables that do not fit the
+ * pinned ring the kernels read directly).  A repeated NN.reach or Star.affineMap(W, b) adds nothing to the
+ * first two. */
+NNVHIP_API int nnvhip_upload_stats(nnvhip_ctx* ctx, int64_t* weight_uploads, int64_t* weight_bytes, int64_t* h2d_bytes);
 
 /* ---- sets ----------------------------------------------------------------------------- */
 /* Star(V, C, d, pred_lb, pred_ub), set/Star.m:153-189: uploads host arrays.  V is N x (n+1),
@@ -201,7 +208,15 @@ NNVHIP_API int nnvhip_estimate_ranges_static(nnvhip_ctx* ctx, const nnvhip_star*
 
 /* ---- layers ---------------------------------------------------------------------------- */
 /* FullyConnectedLayer(W, b), nn/layers/FullyConnectedLayer.m:39-99: W is M x K, b has M entries
- * (NULL = no bias, the affineMap(W, []) form). */
+ * (NULL = no bias, the affineMap(W, []) form).
+ * Weight cache: the reference passes weights by value (FullyConnectedLayer(W, b), Star.affineMap(W, b),
+ * set/Star.m:313-343), so a caller that builds the layer again -- every call of affineMap, every NN object a
+ * sweep over properties or a branch-and-bound loop constructs -- would upload the same arrays again.  Each
+ * context therefore keeps the layers it has created, keyed by a 128-bit hash of W and b plus the geometry;
+ * creating a layer whose arrays are resident returns that handle with one more reference and copies nothing
+ * (nnvhip_upload_stats).  Every create is paired with a destroy as before; entries nobody else holds are
+ * dropped least recently used first beyond NNVHIP_WEIGHT_CACHE_MB (environment, default 8192; 0 = no cache).
+ * The same holds for nnvhip_conv2d_create. */
 NNVHIP_API int nnvhip_fc_create(nnvhip_ctx* ctx, const double* W, const double* b, int64_t M, int64_t K,
                      nnvhip_fc** out);
 NNVHIP_API int nnvhip_fc_destroy(nnvhip_fc* fc);

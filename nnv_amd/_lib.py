@@ -16,7 +16,7 @@ HS_DISJOINT, HS_UNDECIDED, HS_INSIDE = 1, 2, 3
 # every entry point declared in include/nnvhip.h
 SYMBOLS = [
     "nnvhip_create", "nnvhip_destroy", "nnvhip_last_error", "nnvhip_synchronize", "nnvhip_set_timing",
-    "nnvhip_last_op_time_ms", "nnvhip_set_dense_affine", "nnvhip_set_eager_columns", "nnvhip_set_eager_relu", "nnvhip_set_small_chain", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
+    "nnvhip_last_op_time_ms", "nnvhip_set_dense_affine", "nnvhip_set_eager_columns", "nnvhip_set_eager_relu", "nnvhip_set_small_chain", "nnvhip_upload_stats", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
     "nnvhip_trim_pool", "nnvhip_pool_stats", "nnvhip_star_create",
     "nnvhip_star_from_box", "nnvhip_star_retain", "nnvhip_star_release", "nnvhip_star_release_array", "nnvhip_star_dims",
     "nnvhip_star_fetch_V", "nnvhip_star_fetch_pred_bounds", "nnvhip_star_fetch_constraints",
@@ -64,6 +64,7 @@ def load():
         "nnvhip_set_eager_columns": [p, C.c_int],
         "nnvhip_set_eager_relu": [p, C.c_int],
         "nnvhip_set_small_chain": [p, C.c_int],
+        "nnvhip_upload_stats": [p, p, p, p],
         "nnvhip_last_op_time_ms": [p, C.POINTER(dbl)],
         "nnvhip_kernel_time": [p, C.c_int, C.POINTER(dbl), pi64, C.POINTER(dbl), C.c_int],
         "nnvhip_probe_copy_bandwidth": [p, i64, C.c_int, C.POINTER(dbl)],
@@ -215,6 +216,13 @@ class Context:
         a, b = C.c_int64(), C.c_int64()
         check(self.lib.nnvhip_pool_stats(self.handle, C.byref(a), C.byref(b)))
         return a.value, b.value
+
+    def upload_stats(self):
+        """(layers whose weights were uploaded, bytes of those uploads, all host-to-device bytes) since the
+        context was created."""
+        a, b, c = C.c_int64(), C.c_int64(), C.c_int64()
+        check(self.lib.nnvhip_upload_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
 
     def trim_pool(self):
         check(self.lib.nnvhip_trim_pool(self.handle))

@@ -50,6 +50,33 @@ const TuneKnobs& tune_knobs() {
   return knobs;
 }
 
+void hash_bytes(const void* data, size_t bytes, uint64_t* h0, uint64_t* h1) {
+  auto fold = [](uint64_t a, uint64_t b) {
+    const __uint128_t r = (__uint128_t)a * b;
+    return (uint64_t)r ^ (uint64_t)(r >> 64);
+  };
+  const uint64_t k0 = 0xa0761d6478bd642full, k1 = 0xe7037ed1a0b428dbull, k2 = 0x8ebc6af09c88c6e3ull, k3 = 0x589965cc75374cc3ull;
+  uint64_t a = k0 ^ bytes, b = k1 ^ bytes, c = k2 ^ bytes, d = k3 ^ bytes;
+  const unsigned char* p = static_cast<const unsigned char*>(data);
+  size_t i = 0;
+  for (; i + 32 <= bytes; i += 32) {  // four words a round, two independent pairs of streams
+    uint64_t w[4];
+    memcpy(w, p + i, 32);
+    a = fold(a ^ w[0], k1 ^ w[1]);
+    b = fold(b ^ w[2], k2 ^ w[3]);
+    c = fold(c ^ w[1], k3 ^ w[2]);
+    d = fold(d ^ w[3], k0 ^ w[0]);
+  }
+  uint64_t tail[4] = {0, 0, 0, 0};
+  if (i < bytes) memcpy(tail, p + i, bytes - i);
+  a = fold(a ^ tail[0], k1 ^ tail[1]);
+  b = fold(b ^ tail[2], k2 ^ tail[3]);
+  c = fold(c ^ tail[1], k3 ^ tail[2]);
+  d = fold(d ^ tail[3], k0 ^ tail[0]);
+  *h0 = fold(a ^ k2, b ^ k3) ^ a;
+  *h1 = fold(c ^ k0, d ^ k1) ^ d;
+}
+
 int enter_ctx(nnvhip_ctx* ctx) {
   NNV_HIP_TRY(hipSetDevice(ctx->device));
   return NNVHIP_OK;
@@ -150,7 +177,32 @@ int nnvhip_ctx::upload(const void* host, size_t bytes, BufRef* out) {
   memcpy(st, host, bytes);
   NNV_TRY(alloc(bytes, out));
   NNV_HIP_TRY(hipMemcpyAsync((*out)->ptr, st, bytes, hipMemcpyHostToDevice, stream));
+  h2d_bytes += (int64_t)bytes;
   return NNVHIP_OK;
+}
+
+// Frees the cache's references: every entry (all), or least recently used entries that nobody else holds
+// until the cache is back under its budget.
+void nnvhip_ctx::drop_weight_cache(bool all) {
+  while (!weight_cache.empty() && (all || weight_cache_bytes > weight_cache_budget)) {
+    auto victim = weight_cache.end();
+    for (auto it = weight_cache.begin(); it != weight_cache.end(); ++it) {
+      const int refs = it->first.kind == 0 ? static_cast<nnvhip_fc*>(it->second.handle)->refs.load()
+                                           : static_cast<nnvhip_conv2d*>(it->second.handle)->refs.load();
+      if (!all && refs > 1) continue;  // in use by a layer object
+      if (victim == weight_cache.end() || it->second.last_use < victim->second.last_use) victim = it;
+    }
+    if (victim == weight_cache.end()) break;
+    weight_cache_bytes -= victim->second.bytes;
+    if (victim->first.kind == 0) {
+      nnvhip_fc* f = static_cast<nnvhip_fc*>(victim->second.handle);
+      if (f->refs.fetch_sub(1) == 1) delete f;
+    } else {
+      nnvhip_conv2d* v = static_cast<nnvhip_conv2d*>(victim->second.handle);
+      if (v->refs.fetch_sub(1) == 1) delete v;
+    }
+    weight_cache.erase(victim);
+  }
 }
 
 int nnvhip_ctx::kernel_timer_begin(bool) { return NNVHIP_OK; }  // the events travel with the launch (NNV_LAUNCH)
@@ -211,6 +263,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->eager_cols = getenv("NNVHIP_EAGER_COLS") != nullptr;
   c->poison_pending = getenv("NNVHIP_POISON_PENDING") != nullptr;
   c->small_chain = getenv("NNVHIP_NO_SMALL_CHAIN") == nullptr;
+  if (const char* e = getenv("NNVHIP_WEIGHT_CACHE_MB")) c->weight_cache_budget = (int64_t)atoll(e) << 20;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
   NNV_HIP_TRY(hipEventCreate(&c->ev1));
@@ -225,6 +278,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
 
 int nnvhip_destroy(nnvhip_ctx* c) {
   if (!c) return NNVHIP_OK;
+  c->drop_weight_cache(true);
   if (c->live_handles != 0)
     NNV_FAIL(NNVHIP_ERR_ARG, "context still has %lld live handles", (long long)c->live_handles);
   NNV_TRY(nnvhip::enter_ctx(c));
@@ -393,6 +447,14 @@ int nnvhip_trim_pool(nnvhip_ctx* c) {
   return c->trim();
 }
 
+int nnvhip_upload_stats(nnvhip_ctx* c, int64_t* weight_uploads, int64_t* weight_bytes, int64_t* h2d_bytes) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  if (weight_uploads) *weight_uploads = c->weight_uploads;
+  if (weight_bytes) *weight_bytes = c->weight_upload_bytes;
+  if (h2d_bytes) *h2d_bytes = c->h2d_bytes;
+  return NNVHIP_OK;
+}
+
 int nnvhip_pool_stats(nnvhip_ctx* c, int64_t* in_use, int64_t* cached) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
   if (in_use) *in_use = c->bytes_in_use;
@@ -412,6 +474,7 @@ static int upload_matrix(nnvhip_ctx* c, const double* host, int64_t rows, int64_
   if (ld != rows) NNV_HIP_TRY(hipMemsetAsync(dev, 0, sizeof(double) * ld * cols, c->stream));
   NNV_HIP_TRY(hipMemcpy2DAsync(dev, sizeof(double) * ld, host, sizeof(double) * rows, sizeof(double) * rows,
                                cols, hipMemcpyHostToDevice, c->stream));
+  c->h2d_bytes += (int64_t)sizeof(double) * rows * cols;
   // the source is pageable caller memory: finish before returning
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   return NNVHIP_OK;
@@ -445,6 +508,7 @@ int nnvhip_star_create(nnvhip_ctx* c, int64_t N, int64_t n, const double* V, con
       tmp[npad + i] = pred_ub ? pred_ub[i] : 1.0;
     }
     NNV_HIP_TRY(hipMemcpyAsync(s->plb, tmp.data(), sizeof(double) * 2 * npad, hipMemcpyHostToDevice, c->stream));
+    c->h2d_bytes += (int64_t)sizeof(double) * 2 * npad;
     NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   }
   auto base = std::make_shared<ConsNode>();
@@ -458,6 +522,7 @@ int nnvhip_star_create(nnvhip_ctx* c, int64_t N, int64_t n, const double* V, con
   if (p > 0) {
     NNV_TRY(c->alloc(sizeof(double) * p, &base->d0));
     NNV_HIP_TRY(hipMemcpyAsync(base->d0->ptr, d, sizeof(double) * p, hipMemcpyHostToDevice, c->stream));
+    c->h2d_bytes += (int64_t)sizeof(double) * p;
     NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   }
   s->cons = base;
@@ -762,6 +827,30 @@ int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M,
   CHECK_CTX(c);
   if (!W || !out) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   if (M <= 0 || K <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistent dimension between the weight matrix and bias vector");
+  // the same arrays again (a layer object rebuilt around them, Star.affineMap called once more): the resident copy
+  WeightKey key;
+  key.kind = 0;
+  key.geo[0] = M;
+  key.geo[1] = K;
+  key.geo[2] = b ? 1 : 0;
+  hash_bytes(W, sizeof(double) * M * K, &key.h0, &key.h1);
+  if (b) {
+    uint64_t b0 = 0, b1 = 0;
+    hash_bytes(b, sizeof(double) * M, &b0, &b1);
+    key.geo[3] = (int64_t)b0;
+    key.geo[4] = (int64_t)b1;
+  }
+  if (c->weight_cache_budget > 0) {
+    auto hit = c->weight_cache.find(key);
+    if (hit != c->weight_cache.end()) {
+      nnvhip_fc* f = static_cast<nnvhip_fc*>(hit->second.handle);
+      f->refs.fetch_add(1);
+      hit->second.last_use = ++c->weight_clock;
+      c->live_handles++;
+      *out = f;
+      return NNVHIP_OK;
+    }
+  }
   std::unique_ptr<nnvhip_fc> fc(new nnvhip_fc());
   fc->ctx = c;
   fc->M = M;
@@ -779,15 +868,29 @@ int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M,
     NNV_HIP_TRY(hipMemcpyAsync(fc->bias->ptr, b, sizeof(double) * M, hipMemcpyHostToDevice, c->stream));
   }
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  const int64_t wbytes = (int64_t)sizeof(double) * (M * K + (b ? M : 0));
+  c->weight_uploads++;
+  c->weight_upload_bytes += wbytes;
+  c->h2d_bytes += wbytes;
   c->live_handles++;
   *out = fc.release();
+  if (c->weight_cache_budget > 0) {
+    (*out)->refs.fetch_add(1);  // the cache's reference
+    WeightEntry e;
+    e.handle = *out;
+    e.bytes = (int64_t)sizeof(double) * (*out)->Mp * ((*out)->Kp + 1);
+    e.last_use = ++c->weight_clock;
+    c->weight_cache[key] = e;
+    c->weight_cache_bytes += e.bytes;
+    c->drop_weight_cache(false);
+  }
   return NNVHIP_OK;
 }
 
 int nnvhip_fc_destroy(nnvhip_fc* fc) {
   if (!fc) return NNVHIP_OK;
   nnvhip_ctx* c = fc->ctx;
-  delete fc;
+  if (fc->refs.fetch_sub(1) == 1) delete fc;
   c->live_handles--;
   return NNVHIP_OK;
 }
@@ -802,6 +905,33 @@ int nnvhip_conv2d_create(nnvhip_ctx* c, const double* W, const double* bias, int
     if (padding[i] < 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Invalid padding matrix");
   if (stride[0] <= 0 || stride[1] <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Invalid stride matrix");
   if (dilation[0] <= 0 || dilation[1] <= 0) NNV_FAIL(NNVHIP_ERR_SHAPE, "Invalid dilation matrix");
+  WeightKey key;
+  key.kind = 1;
+  key.geo[0] = FH;
+  key.geo[1] = FW;
+  key.geo[2] = Cin;
+  key.geo[3] = Cout;
+  for (int i = 0; i < 4; ++i) key.geo[4 + i] = padding[i];
+  key.geo[8] = stride[0] | (stride[1] << 20) | (dilation[0] << 40) | ((int64_t)(bias ? 1 : 0) << 62);
+  key.geo[9] = dilation[1];
+  hash_bytes(W, sizeof(double) * FH * FW * Cin * Cout, &key.h0, &key.h1);
+  if (bias) {
+    uint64_t b0 = 0, b1 = 0;
+    hash_bytes(bias, sizeof(double) * Cout, &b0, &b1);
+    key.geo[10] = (int64_t)b0;
+    key.geo[11] = (int64_t)b1;
+  }
+  if (c->weight_cache_budget > 0) {
+    auto hit = c->weight_cache.find(key);
+    if (hit != c->weight_cache.end()) {
+      nnvhip_conv2d* v = static_cast<nnvhip_conv2d*>(hit->second.handle);
+      v->refs.fetch_add(1);
+      hit->second.last_use = ++c->weight_clock;
+      c->live_handles++;
+      *out = v;
+      return NNVHIP_OK;
+    }
+  }
   std::unique_ptr<nnvhip_conv2d> cv(new nnvhip_conv2d());
   cv->ctx = c;
   cv->FH = FH;
@@ -825,15 +955,29 @@ int nnvhip_conv2d_create(nnvhip_ctx* c, const double* W, const double* bias, int
     NNV_HIP_TRY(hipMemcpyAsync(cv->bias->ptr, bias, sizeof(double) * Cout, hipMemcpyHostToDevice, c->stream));
   }
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  const int64_t wbytes = (int64_t)sizeof(double) * (cv->K * Cout + (bias ? Cout : 0));
+  c->weight_uploads++;
+  c->weight_upload_bytes += wbytes;
+  c->h2d_bytes += wbytes;
   c->live_handles++;
   *out = cv.release();
+  if (c->weight_cache_budget > 0) {
+    (*out)->refs.fetch_add(1);  // the cache's reference
+    WeightEntry e;
+    e.handle = *out;
+    e.bytes = (int64_t)sizeof(double) * ((*out)->Kp + 1) * Cout;
+    e.last_use = ++c->weight_clock;
+    c->weight_cache[key] = e;
+    c->weight_cache_bytes += e.bytes;
+    c->drop_weight_cache(false);
+  }
   return NNVHIP_OK;
 }
 
 int nnvhip_conv2d_destroy(nnvhip_conv2d* cv) {
   if (!cv) return NNVHIP_OK;
   nnvhip_ctx* c = cv->ctx;
-  delete cv;
+  if (cv->refs.fetch_sub(1) == 1) delete cv;
   c->live_handles--;
   return NNVHIP_OK;
 }

@@ -315,6 +315,7 @@ int nnvhip_rowmap_create(nnvhip_ctx* c, int64_t N, int32_t n_steps, const int32_
   }
   NNV_TRY(c->alloc(sizeof(double) * host.size(), &m->params));
   NNV_HIP_TRY(hipMemcpyAsync(m->params->ptr, host.data(), sizeof(double) * host.size(), hipMemcpyHostToDevice, c->stream));
+  c->h2d_bytes += (int64_t)(sizeof(double) * host.size());
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   *out = m.release();
   return NNVHIP_OK;

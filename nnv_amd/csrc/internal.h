@@ -137,6 +137,30 @@ using ConsRef = std::shared_ptr<ConsNode>;
 // start of every entry point that touches device data: selects the context's device
 int enter_ctx(nnvhip_ctx* ctx);
 
+// Key of the per-context weight cache: a 128-bit hash of the layer's host arrays plus its geometry.  Layers are
+// created from host arrays by value (FullyConnectedLayer(W, b), Star.affineMap(W, b) have no handle to pass
+// around), so "the same layer again" can only be recognised by content.
+struct WeightKey {
+  uint64_t h0 = 0, h1 = 0;
+  int64_t geo[12] = {};
+  int kind = 0;  // 0 fc, 1 conv2d
+  bool operator<(const WeightKey& o) const {
+    if (kind != o.kind) return kind < o.kind;
+    if (h0 != o.h0) return h0 < o.h0;
+    if (h1 != o.h1) return h1 < o.h1;
+    for (int i = 0; i < 12; ++i)
+      if (geo[i] != o.geo[i]) return geo[i] < o.geo[i];
+    return false;
+  }
+};
+struct WeightEntry {
+  void* handle = nullptr;  // nnvhip_fc* / nnvhip_conv2d*; the cache owns one reference
+  int64_t bytes = 0;
+  uint64_t last_use = 0;
+};
+// 128-bit content hash (two multiply-fold streams with different constants) of a host array
+void hash_bytes(const void* data, size_t bytes, uint64_t* h0, uint64_t* h1);
+
 }  // namespace nnvhip
 
 struct nnvhip_ctx {
@@ -161,6 +185,17 @@ struct nnvhip_ctx {
   // device's address of the array and its length
   double* static_scratch = nullptr;
   int64_t static_scratch_doubles = 0;
+  // Layer weights by content: creating a layer whose arrays are already on the device returns the resident
+  // handle (one more reference) instead of uploading them again.  Entries nobody else holds are dropped,
+  // least recently used first, once the cache passes its budget (environment NNVHIP_WEIGHT_CACHE_MB, default 8192).
+  std::map<nnvhip::WeightKey, nnvhip::WeightEntry> weight_cache;
+  int64_t weight_cache_bytes = 0;
+  int64_t weight_cache_budget = int64_t(8192) << 20;
+  uint64_t weight_clock = 0;
+  // uploads since the context was created: layers whose weights went to the device, their bytes, and all
+  // bytes the library copied from host to device (sets, bounds, descriptor tables, weights)
+  int64_t weight_uploads = 0, weight_upload_bytes = 0, h2d_bytes = 0;
+  void drop_weight_cache(bool all);
   uint32_t mailbox_seq = 0;  // number of the ReLU call (wraps; only its low 16 bits travel, as a cross-check)
   // FC layers as the full dense contraction (no skipping of structural zeros); default from the
   // environment variable NNVHIP_DENSE_AFFINE
@@ -290,6 +325,7 @@ struct nnvhip_star {
 };
 
 struct nnvhip_fc {
+  std::atomic<int> refs{1};
   nnvhip_ctx* ctx = nullptr;
   int64_t M = 0, K = 0, Mp = 0, Kp = 0;
   nnvhip::BufRef W;     // Mp x Kp, zero padded, ld = Mp
@@ -299,6 +335,7 @@ struct nnvhip_fc {
 };
 
 struct nnvhip_conv2d {
+  std::atomic<int> refs{1};
   nnvhip_ctx* ctx = nullptr;
   int64_t FH = 0, FW = 0, Cin = 0, Cout = 0;
   int64_t pad[4] = {0, 0, 0, 0}, stride[2] = {1, 1}, dil[2] = {1, 1};
