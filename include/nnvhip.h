@@ -247,6 +247,16 @@ NNVHIP_API int nnvhip_affine_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, 
  * three triangle constraints and predicate bounds [0, ub].  relax_factor must be 1 (no LP). */
 NNVHIP_API int nnvhip_relu_relax(nnvhip_ctx* ctx, int order, double relax_factor, int64_t count,
                       nnvhip_star* const* in, nnvhip_star** out);
+/* The 'reduceMem' suffix of a relax-star method on a ReLU layer, nn/layers/ReluLayer.m:107-112, 119-146: the
+ * ImageStar the ReLU step returned (in, of height H, width W, C channels) is replaced by the box-like ImageStar
+ * the reference builds from its estimated ranges [l, u]: centre 0.5*(u+l), numel(find(l-u)) predicates with
+ * bounds -1 / +1, C = zeros(1, n), d = 0, and one generator per pixel (rows outer, columns inner) whose
+ * first-channel half-width 0.5*(u-l) is non-zero, holding that value on every channel of the pixel; generators
+ * the loop never reaches stay zero -- the reference's statements as they stand, also for C > 1.  im_lb / im_ub
+ * (host, H*W*C doubles each, or NULL) receive l and u, which the reference stores as the set's im_lb / im_ub.
+ * The ranges come from the device; the N x (n+1) matrix is filled by one kernel and never crosses the bus. */
+NNVHIP_API int nnvhip_relu_reduce_mem(nnvhip_ctx* ctx, nnvhip_star* in, int64_t H, int64_t W, int64_t C, nnvhip_star** out,
+                           double* im_lb, double* im_ub);
 /* The layer loop of NN.reach for a network made of the three layer kinds above, in one call
  * (NN.reach_noConns, nn/NN.m:1529-1551: rs = Layers{i}.reach(rs, method, ...); reachSet{i} = rs).  Layer i is
  * kind[i] = NNVHIP_LAYER_FC / _CONV2D / _RELU with handle layer[i] (nnvhip_fc*, nnvhip_conv2d*, NULL) and,

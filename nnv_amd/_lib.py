@@ -28,7 +28,7 @@ SYMBOLS = [
     "nnvhip_avgpool2d_output_size", "nnvhip_affine_avgpool2d", "nnvhip_permute_rows",
     "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists", "nnvhip_probe_mfma_peak",
     "nnvhip_estimate_ranges_static", "nnvhip_debug_mailbox_pack", "nnvhip_debug_mailbox_unpack",
-    "nnvhip_debug_set_relu_call_number", "nnvhip_reach_layers",
+    "nnvhip_debug_set_relu_call_number", "nnvhip_reach_layers", "nnvhip_relu_reduce_mem",
 ]
 
 
@@ -110,6 +110,7 @@ def load():
                                         C.POINTER(C.c_int32)],
         "nnvhip_debug_set_relu_call_number": [p, i64],
         "nnvhip_reach_layers": [p, i64, p, p, p, C.c_int, dbl, i64, pp, pp],
+        "nnvhip_relu_reduce_mem": [p, p, i64, i64, i64, pp, p, p],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)

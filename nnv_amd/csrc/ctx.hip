@@ -659,6 +659,115 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
   return NNVHIP_OK;
 }
 
+// Columns of the set the reduceMem suffix of the ReLU layer builds: column 0 the centre, column 1 + g the value
+// val[g] on every channel of pixel pix[g] (rows pix[g] + k * HW), every other entry zero.
+__global__ void rebox_fill_kernel(double* __restrict__ V, int64_t ld, int N, int HW, int64_t ncols, int ngen,
+                                  const double* __restrict__ center, const int32_t* __restrict__ pix,
+                                  const double* __restrict__ val) {
+  for (int64_t j = blockIdx.y; j < ncols; j += gridDim.y) {
+    double* col = V + j * ld;
+    const int p = (j >= 1 && j - 1 < ngen) ? pix[j - 1] : -1;
+    const double pv = p >= 0 ? val[j - 1] : 0.0;
+    for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < ld; r += gridDim.x * blockDim.x) {
+      double v = 0.0;
+      if (r < N) {
+        if (j == 0) v = center[r];
+        else if (p >= 0 && r % HW == p) v = pv;
+      }
+      col[r] = v;
+    }
+  }
+}
+
+int nnvhip_relu_reduce_mem(nnvhip_ctx* c, nnvhip_star* in, int64_t H, int64_t W, int64_t C, nnvhip_star** out, double* im_lb,
+                           double* im_ub) {
+  CHECK_CTX(c);
+  if (!in || in->ctx != c || !out) NNV_FAIL(NNVHIP_ERR_ARG, "invalid set handle");
+  if (H <= 0 || W <= 0 || C <= 0 || H * W * C != in->N)
+    NNV_FAIL(NNVHIP_ERR_SHAPE, "Inconsistent dimension in the ImageStar and the original Star set");
+  const int64_t N = in->N, HW = H * W;
+  // [l, u] = images(i).estimateRanges
+  NNV_TRY(compute_ranges(c, 1, &in));
+  std::vector<double> l((size_t)N), u((size_t)N);
+  NNV_HIP_TRY(hipMemcpyAsync(l.data(), in->lb, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
+  NNV_HIP_TRY(hipMemcpyAsync(u.data(), in->ub, sizeof(double) * N, hipMemcpyDeviceToHost, c->stream));
+  NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  // center = 0.5*(u+l); v = 0.5*(u-l); n = numel(find(l-u)); one generator per pixel (i1 outer, i2 inner) whose
+  // first-channel half-width is non-zero
+  std::vector<double> center((size_t)N), val;
+  std::vector<int32_t> pix;
+  int64_t n = 0;
+  for (int64_t i = 0; i < N; ++i) {
+    center[i] = 0.5 * (u[i] + l[i]);
+    if (l[i] - u[i] != 0.0) ++n;
+  }
+  for (int64_t i1 = 0; i1 < H; ++i1)
+    for (int64_t i2 = 0; i2 < W; ++i2) {
+      const double bv = 0.5 * (u[i1 + i2 * H] - l[i1 + i2 * H]);
+      if (bv != 0.0) {
+        pix.push_back((int32_t)(i1 + i2 * H));
+        val.push_back(bv);
+      }
+    }
+  if ((int64_t)pix.size() > n) NNV_FAIL(NNVHIP_ERR_SHAPE, "Index exceeds the number of array elements");  // (cannot happen: C >= 1)
+  nnvhip_star* s = new_star(c);
+  std::unique_ptr<nnvhip_star, int (*)(nnvhip_star*)> guard(s, nnvhip_star_release);
+  s->N = N;
+  s->n = n;
+  s->ld = round_up(N, kLdAlign);
+  NNV_TRY(c->alloc(sizeof(double) * s->ld * (n + 1), &s->Vbuf));
+  s->V = s->Vbuf->as<double>();
+  BufRef dcen, dpix, dval;
+  NNV_TRY(c->upload(center.data(), sizeof(double) * N, &dcen));
+  const int ngen = (int)pix.size();
+  if (pix.empty()) {  // (something to upload)
+    pix.push_back(0);
+    val.push_back(0.0);
+  }
+  NNV_TRY(c->upload(pix.data(), sizeof(int32_t) * pix.size(), &dpix));
+  NNV_TRY(c->upload(val.data(), sizeof(double) * val.size(), &dval));
+  dim3 grid((unsigned)std::min<int64_t>(ceil_div(s->ld, 256), 64), (unsigned)std::min<int64_t>(n + 1, 4096));
+  hipLaunchKernelGGL(rebox_fill_kernel, grid, dim3(256), 0, c->stream, s->V, s->ld, (int)N, (int)HW, n + 1, ngen,
+                     dcen->as<double>(), dpix->as<int32_t>(), dval->as<double>());
+  NNV_HIP_TRY(hipGetLastError());
+  // predicate bounds -1 / +1; C = zeros(1, n), d = 0
+  const int64_t npad = round_up(std::max<int64_t>(n, 1), kLdAlign);
+  NNV_TRY(c->alloc(sizeof(double) * 2 * npad, &s->pbuf));
+  s->plb = s->pbuf->as<double>();
+  s->pub = s->plb + npad;
+  {
+    const int64_t pinfo[2] = {0, npad};
+    BufRef dinfo;
+    NNV_TRY(c->upload(pinfo, sizeof(pinfo), &dinfo));
+    hipLaunchKernelGGL(fill_pm_one_kernel, dim3((unsigned)ceil_div(npad, 256), 1), dim3(256), 0, c->stream, s->plb, dinfo->as<int64_t>());
+    NNV_HIP_TRY(hipGetLastError());
+  }
+  auto base = std::make_shared<ConsNode>();
+  base->p_total = 1;
+  base->n_total = n;
+  s->cons = base;
+  if (C == 1 && ngen == n && n > 0) {  // a plain box star: every generator is val * e_pix
+    std::vector<double> scale((size_t)N, 0.0);
+    bool neg = false;
+    for (size_t g = 0; g < (size_t)ngen; ++g) {
+      scale[pix[g]] = val[g];
+      neg = neg || val[g] < 0.0;
+    }
+    BufRef dscale;
+    NNV_TRY(c->upload(scale.data(), sizeof(double) * N, &dscale));
+    s->oh_from = 1;
+    s->oh_idx_buf = dpix;
+    s->oh_idx = dpix->as<int32_t>();
+    s->oh_scale_buf = dscale;
+    s->oh_scale = dscale->as<double>();
+    s->oh_scale_neg = neg;
+  }
+  if (im_lb) memcpy(im_lb, l.data(), sizeof(double) * N);
+  if (im_ub) memcpy(im_ub, u.data(), sizeof(double) * N);
+  *out = guard.release();
+  return NNVHIP_OK;
+}
+
 int nnvhip_star_retain(nnvhip_star* s) {
   if (!s) NNV_FAIL(NNVHIP_ERR_ARG, "null set handle");
   s->refs.fetch_add(1);

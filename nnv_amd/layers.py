@@ -425,6 +425,20 @@ def _relaxed_star_lp(I, method, relaxFactor, option=None, dis_opt=None, lp_solve
     return PosLin.multipleStepReachStarApprox_at_one(I, index, lbs, ubs, reset=map11)
 
 
+def _reduce_mem(image):
+    """nn/layers/ReluLayer.m:119-146: the box-like ImageStar of the set's estimated ranges, built on the device."""
+    ctx = image.ctx
+    h, w, c = image.height, image.width, image.numChannel
+    out = (C.c_void_p * 1)()
+    lb = np.empty(h * w * c)
+    ub = np.empty(h * w * c)
+    check(ctx.lib.nnvhip_relu_reduce_mem(ctx.handle, image._h.h, h, w, c, out, ptr(lb), ptr(ub)))
+    res = ImageStar(_handle=_Handle(C.c_void_p(out[0]), ctx), shape=(h, w, c))
+    res.im_lb = lb.reshape((h, w, c), order="F")
+    res.im_ub = ub.reshape((h, w, c), order="F")
+    return res
+
+
 class ReluLayer:
     """nn/layers/ReluLayer.m (+ ActivationFunctionLayer.m:108-172)."""
 
@@ -442,8 +456,14 @@ class ReluLayer:
         toStar -> PosLin.reach -> toImageStar, which on the device is the same memory."""
         if option not in (None, "", "single", "parallel") and not (isinstance(option, (list, tuple)) and len(option) == 0):
             raise ValueError("Unknown computation option")
-        if "reduceMem" in method:
-            raise NotImplementedError("the reduceMem variants are outside this library")
+        reduce_mem = "reduceMem" in method
+        if reduce_mem:
+            # nn/layers/ReluLayer.m:107-112: the suffix is split off for ImageStars only; a Star hands the whole
+            # string to PosLin.reach, which does not know it
+            in_images = list(in_images)
+            if any(isinstance(s, Star) and not isinstance(s, ImageStar) for s in in_images):
+                raise ValueError("This reachability method does not exist")
+            method = "-".join(method.split("-")[:-1])
         if isinstance(in_images, SetArray) and method in RELAX_ORDER and relaxFactor == 1 and dis_opt != "display":
             # an array straight from the previous layer: no object per set is needed
             ctx, shapes = in_images.ctx, in_images.shapes
@@ -458,7 +478,8 @@ class ReluLayer:
         res = PosLin.reach(stars, method, None, relaxFactor, dis_opt, lp_solver) if stars else []
         out = []
         for s, r in zip(in_images, res):
-            out.append(r.toImageStar(s.height, s.width, s.numChannel) if isinstance(s, ImageStar) else r)
+            o = r.toImageStar(s.height, s.width, s.numChannel) if isinstance(s, ImageStar) else r
+            out.append(_reduce_mem(o) if reduce_mem else o)
         return out
 
     def reach(self, in_images, method, option="single", relaxFactor=0, dis_opt=None, lp_solver="linprog"):

@@ -1,6 +1,9 @@
 classdef ImageStar < ImageStar
     % NNV ImageStar resident in HBM: the H x W x C x (numPred+1) tensor is the same device memory as
     % the (H*W*C) x (numPred+1) Star matrix (ImageStar.m:569-592, Star.m:1398-1418).
+    % ImageStar is a handle class: the first read of V, C, d, pred_lb or pred_ub from outside the class fetches the
+    % dense NNV array from the device and keeps it in the inherited field (subsref below); NNV methods that read
+    % them from inside the class are overridden to fill the fields first (materialize()).
     properties
         dev = [];   % nnvhip.DeviceSet
     end
@@ -53,6 +56,29 @@ classdef ImageStar < ImageStar
             end
             S = obj;
         end
+        function materialize(obj)
+            % fills the inherited dense fields from the device, once
+            if isempty(obj.dev) || ~isempty(builtin('subsref', obj, substruct('.', 'V'))), return; end
+            V = nnvhip_mex('fetch_V', obj.dev.h);
+            obj.V = reshape(V, obj.height, obj.width, obj.numChannel, []);
+            [obj.C, obj.d] = nnvhip_mex('fetch_constraints', obj.dev.h);
+            [obj.pred_lb, obj.pred_ub] = nnvhip_mex('fetch_pred', obj.dev.h);
+        end
+        function varargout = subsref(obj, s)
+            if isscalar(obj) && strcmp(s(1).type, '.') && any(strcmp(s(1).subs, {'V', 'C', 'd', 'pred_lb', 'pred_ub'}))
+                obj.materialize();
+            end
+            [varargout{1:nargout}] = builtin('subsref', obj, s);
+        end
+        % ---- NNV methods that read the dense fields from inside the class ------------------------------------
+        function varargout = getRanges(obj, varargin),  obj.materialize(); [varargout{1:nargout}] = getRanges@ImageStar(obj, varargin{:}); end
+        function varargout = getRange(obj, varargin),   obj.materialize(); [varargout{1:nargout}] = getRange@ImageStar(obj, varargin{:}); end
+        function varargout = estimateRange(obj, varargin), obj.materialize(); [varargout{1:nargout}] = estimateRange@ImageStar(obj, varargin{:}); end
+        function bool = isEmptySet(obj),                 obj.materialize(); bool = isEmptySet@ImageStar(obj); end
+        function bool = contains(obj, image),            obj.materialize(); bool = contains@ImageStar(obj, image); end
+        function images = sample(obj, N),                obj.materialize(); images = sample@ImageStar(obj, N); end
+        function image = evaluate(obj, pred_val),        obj.materialize(); image = evaluate@ImageStar(obj, pred_val); end
+        function IS = affineMap(obj, scale, offset),     obj.materialize(); IS = affineMap@ImageStar(obj, scale, offset); end
         function IS = gather(obj)
             V = nnvhip_mex('fetch_V', obj.dev.h);
             [C, d] = nnvhip_mex('fetch_constraints', obj.dev.h);

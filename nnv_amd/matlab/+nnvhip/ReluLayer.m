@@ -7,6 +7,19 @@ classdef ReluLayer < ReluLayer
             obj = obj@ReluLayer(varargin{:});
         end
         function images = reach_star_multipleInputs(obj, in_images, method, option, relaxFactor, dis_opt, lp_solver) %#ok<INUSL>
+            % 'reduceMem' suffix (ReluLayer.m:107-112): split off for ImageStars only; for a Star the whole string
+            % reaches PosLin.reach, which does not know it (PosLin.m:2165-2166)
+            reduceMem = false;
+            if contains(method, "reduceMem")
+                for i = 1:length(in_images)
+                    if ~isa(in_images(i), 'ImageStar')
+                        error("This reachability method does not exist");
+                    end
+                end
+                parts = split(string(method), '-');
+                method = strjoin(parts(1:end-1), '-');
+                reduceMem = true;
+            end
             switch char(method)
                 case 'relax-star-range', order = 2;                       % PosLin.m:934-936
                 case 'relax-star-area',  order = 1;                       % PosLin.m:1049-1052
@@ -28,7 +41,15 @@ classdef ReluLayer < ReluLayer
                 for i = 1:n, out(i) = nnvhip.relaxed_star_lp(hs(i), method, relaxFactor, lp_solver, dis_opt); end
             end
             for i = n:-1:1
-                if isa(in_images(i), 'ImageStar')
+                if isa(in_images(i), 'ImageStar') && reduceMem
+                    % ReluLayer.m:119-146: the box-like ImageStar of the estimated ranges, filled on the device
+                    hh = in_images(i).height; ww = in_images(i).width; cc = in_images(i).numChannel;
+                    [boxed, l, u] = nnvhip_mex('relu_reduce_mem', out(i), hh, ww, cc);
+                    nnvhip_mex('star_release', out(i));
+                    images(i) = nnvhip.ImageStar(nnvhip.DeviceSet(boxed), hh, ww, cc);
+                    images(i).im_lb = reshape(l, hh, ww, cc);
+                    images(i).im_ub = reshape(u, hh, ww, cc);
+                elseif isa(in_images(i), 'ImageStar')
                     images(i) = nnvhip.ImageStar(nnvhip.DeviceSet(out(i)), in_images(i).height, in_images(i).width, in_images(i).numChannel);
                 else
                     images(i) = nnvhip.Star(nnvhip.DeviceSet(out(i)));

@@ -1,7 +1,11 @@
 classdef Star < Star
     % NNV Star whose [c V], predicate bounds and constraints live in HBM.
     % isa(S,'Star') stays true, so PosLin/NN guards (PosLin.m:902, NN.m:204-207) pass.
-    % V, C, d stay empty on the host until gather() is called; dim/nVar are kept current.
+    % dim/nVar are kept current.  The inherited fields V, C, d, predicate_lb, predicate_ub stay empty in the object;
+    % a read of one of them from outside the class (S.V, S.C(1,:), ...) goes through subsref below, which fetches the
+    % dense NNV array from the device (C, d in NNV's [C0;C1;C2;C3] layout, PosLin.m:711-735).  NNV methods that read
+    % those fields from inside the class (a value class cannot intercept that) are overridden at the end of this
+    % file: they gather() once and run NNV's own code on the plain Star.
     properties
         dev = [];   % nnvhip.DeviceSet
     end
@@ -62,6 +66,47 @@ classdef Star < Star
             [C, d] = nnvhip_mex('fetch_constraints', obj.dev.h);
             [plb, pub] = nnvhip_mex('fetch_pred', obj.dev.h);
             S = Star(V, C, d, plb, pub);
+            S.state_lb = obj.state_lb; S.state_ub = obj.state_ub;
         end
+        function varargout = subsref(obj, s)
+            % lazy property reads: S.V, S.C, S.d, S.predicate_lb, S.predicate_ub fetch from the device
+            if isscalar(obj) && strcmp(s(1).type, '.') && ~isempty(obj.dev) && ...
+                    any(strcmp(s(1).subs, {'V', 'C', 'd', 'predicate_lb', 'predicate_ub'}))
+                switch s(1).subs
+                    case 'V', val = nnvhip_mex('fetch_V', obj.dev.h);
+                    case 'C', [val, ~] = nnvhip_mex('fetch_constraints', obj.dev.h);
+                    case 'd', [~, val] = nnvhip_mex('fetch_constraints', obj.dev.h);
+                    case 'predicate_lb', [val, ~] = nnvhip_mex('fetch_pred', obj.dev.h);
+                    case 'predicate_ub', [~, val] = nnvhip_mex('fetch_pred', obj.dev.h);
+                end
+                if numel(s) > 1
+                    [varargout{1:nargout}] = subsref(val, s(2:end));
+                else
+                    varargout{1} = val;
+                end
+            else
+                [varargout{1:nargout}] = builtin('subsref', obj, s);
+            end
+        end
+        % ---- NNV methods that read V / C / d from inside the class: run on the gathered set ----------------
+        function S = intersectHalfSpace(obj, H, g),   S = obj.gather().intersectHalfSpace(H, g); end      % Star.m:555-589
+        function bool = isEmptySet(obj),              bool = obj.gather().isEmptySet(); end                % Star.m:1216-1232
+        function [lb, ub] = getRanges(obj, varargin), [lb, ub] = obj.gather().getRanges(varargin{:}); end  % Star.m:973-990
+        function B = getBox(obj),                     B = obj.gather().getBox(); end                       % Star.m:620-664
+        function B = getBoxFast(obj),                 B = obj.gather().getBoxFast(); end
+        function x = getMin(obj, varargin),           x = obj.gather().getMin(varargin{:}); end            % Star.m:710-745
+        function x = getMax(obj, varargin),           x = obj.gather().getMax(varargin{:}); end
+        function x = getMins(obj, varargin),          x = obj.gather().getMins(varargin{:}); end           % Star.m:784-870
+        function x = getMaxs(obj, varargin),          x = obj.gather().getMaxs(varargin{:}); end
+        function [lb, ub] = getRange(obj, varargin),  [lb, ub] = obj.gather().getRange(varargin{:}); end
+        function bool = contains(obj, x),             bool = obj.gather().contains(x); end
+        function bool = isSubSet(obj, S),             bool = obj.gather().isSubSet(S); end
+        function V = sample(obj, N),                  V = obj.gather().sample(N); end
+        function P = toPolyhedron(obj),               P = obj.gather().toPolyhedron(); end
+        function Z = getZono(obj),                    Z = obj.gather().getZono(); end
+        function S = MinkowskiSum(obj, X),            S = obj.gather().MinkowskiSum(X); end
+        function S = resetRow(obj, map),              S = obj.gather().resetRow(map); end                  % Star.m:1442-1461
+        function S = scalarMap(obj, a),               S = obj.gather().scalarMap(a); end
+        function varargout = plot(obj, varargin),     [varargout{1:nargout}] = plot(obj.gather(), varargin{:}); end
     end
 end

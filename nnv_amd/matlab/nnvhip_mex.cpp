@@ -199,6 +199,17 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
     std::vector<nnvhip_star*> in = handles_of(prhs[3]), out(in.size());
     check(nnvhip_relu_relax(ctx(), (int)mxGetScalar(prhs[1]), mxGetScalar(prhs[2]), (int64_t)in.size(), in.data(), out.data()));
     plhs[0] = to_mx(out);
+  } else if (cmd == "relu_reduce_mem") {  // (handle, H, W, C) -> [handle, l, u]      ReluLayer.m:119-146
+    need(nrhs, 4, "relu_reduce_mem");
+    nnvhip_star* s = handle_of<nnvhip_star>(prhs[1]);
+    const int64_t H = (int64_t)mxGetScalar(prhs[2]), W = (int64_t)mxGetScalar(prhs[3]), C = (int64_t)mxGetScalar(prhs[4]);
+    mxArray* l = mxCreateDoubleMatrix((mwSize)(H * W * C), 1, mxREAL);
+    mxArray* u = mxCreateDoubleMatrix((mwSize)(H * W * C), 1, mxREAL);
+    nnvhip_star* out = nullptr;
+    check(nnvhip_relu_reduce_mem(ctx(), s, H, W, C, &out, mxGetDoubles(l), mxGetDoubles(u)));
+    plhs[0] = to_mx(out);
+    if (nlhs > 1) plhs[1] = l;
+    if (nlhs > 2) plhs[2] = u;
   } else if (cmd == "fetch_rows") {  // (handle, rows 1-based) -> V(rows, :)      objective rows of Star.getMin/getMax
     need(nrhs, 2, "fetch_rows");
     nnvhip_star* s = handle_of<nnvhip_star>(prhs[1]);

@@ -689,6 +689,47 @@ def relu_reach(I, method, relax_factor=1.0):
 # --------------------------------------------------------------------------------------
 # network loop
 # --------------------------------------------------------------------------------------
+def relu_reduce_mem(I: OImageStar) -> OImageStar:
+    """The reduceMem suffix of ReluLayer.reach_star_single_input, nn/layers/ReluLayer.m:119-146, statement
+    for statement: the ReLU's output ImageStar is replaced by a box-like ImageStar built from its estimated
+    ranges.  n counts every element with l ~= u; a generator is made per PIXEL (i1 outer, i2 inner) whose
+    first-channel half-width v(i1,i2) is non-zero, and that value is written to every channel of the pixel
+    (V(i1,i2,:,bCount) = v(i1,i2)); generators that are never filled stay zero."""
+    l, u = image_star_estimate_ranges(I)
+    l = np.asarray(l, dtype=np.float64)
+    u = np.asarray(u, dtype=np.float64)
+    h, w, c = I.height, I.width, I.numChannel
+    center = 0.5 * (u + l)
+    v = 0.5 * (u - l)
+    n = int(np.count_nonzero(l - u))            # idxRegion = find((l-u)); n = length(idxRegion)
+    V = np.zeros((h, w, c, n))
+    b_count = 0
+    for i1 in range(h):
+        for i2 in range(w):
+            basis = v[i1, i2, 0]                # v(i1,i2) of a 3-D array is v(i1,i2,1)
+            if basis:
+                V[i1, i2, :, b_count] = basis
+                b_count += 1
+    Cm = np.zeros((1, n))
+    d = np.zeros(1)
+    return OImageStar(np.concatenate([center[:, :, :, None], V], axis=3), Cm, d, -np.ones(n), np.ones(n), l, u)
+
+
+def relu_layer_reach(I, method, relax_factor=1.0):
+    """ReluLayer.reach_star_single_input, nn/layers/ReluLayer.m:72-150, for a Star or an ImageStar: the
+    'reduceMem' suffix is split off the method for ImageStars only (:107-112); a Star hands the whole string
+    to PosLin.reach, which does not know it (nn/funcs/PosLin.m:2165-2166)."""
+    if isinstance(I, OImageStar):
+        reduce_mem = "reduceMem" in method
+        if reduce_mem:
+            method = "-".join(method.split("-")[:-1])
+        R = relu_reach(I, method, relax_factor)
+        return relu_reduce_mem(R) if reduce_mem else R
+    if "reduceMem" in method:
+        raise ValueError("This reachability method does not exist")
+    return relu_reach(I, method, relax_factor)
+
+
 def nn_reach(layers, input_set, reach_method="relax-star-area", relax_factor=1.0, keep=False):
     """NN.reach -> reach_noConns, nn/NN.m:189-278, 1529-1551, for a list of layer dicts:
 
@@ -715,7 +756,7 @@ def nn_reach(layers, input_set, reach_method="relax-star-area", relax_factor=1.0
                 out.append(conv2d_reach(S, L["W"], L.get("b"), L.get("padding", (0, 0, 0, 0)),
                                         L.get("stride", (1, 1)), L.get("dilation", (1, 1))))
             elif L["type"] == "relu":
-                out.append(relu_reach(S, reach_method, relax_factor))
+                out.append(relu_layer_reach(S, reach_method, relax_factor))
             elif L["type"] == "batchnorm":
                 out.append(batchnorm_reach(S, L["mean"], L["var"], L["eps"], L["scale"], L["offset"]))
             elif L["type"] == "avgpool":

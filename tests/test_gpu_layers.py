@@ -176,3 +176,43 @@ def test_cnn_with_all_layers_end_to_end(nnv, method):
         x = (cfg["lb"] + (cfg["ub"] - cfg["lb"]) * rs.rand(cfg["lb"].size)).reshape(cfg["image_shape"], order="F")
         y = o.evaluate(cfg["layers"], x).reshape(-1)
         assert np.all(y >= lb.reshape(-1) - 1e-9) and np.all(y <= ub.reshape(-1) + 1e-9)
+
+
+# ---- the reduceMem suffix of the ReLU layer (nn/layers/ReluLayer.m:107-146) -------------------------------
+@pytest.mark.parametrize("H,W,C,n", [(6, 5, 1, 9), (4, 4, 3, 6), (28, 28, 1, 50)])
+def test_relu_reduce_mem(nnv, H, W, C, n):
+    rs = np.random.RandomState(H + 10 * C)
+    D, O = _pair(nnv, rs, H, W, C, n)
+    R = nnv.ReluLayer().reach(D, "relax-star-area-reduceMem", "single", 1)
+    E = o.relu_layer_reach(O, "relax-star-area-reduceMem", 1.0)
+    assert (R.height, R.width, R.numChannel) == (H, W, C)
+    assert R.numPred == E.numPred
+    # the box is built from the estimated ranges of the ReLU's output, which the device and the oracle sum in
+    # different orders: values to rounding, structure (which entries are zero, generator order) exactly
+    assert_close(R.V, E.V, "reduceMem V", 1e-12)
+    assert np.array_equal(np.asarray(R.V) == 0, E.V == 0)
+    assert np.array_equal(R.C, E.C) and np.array_equal(R.d, E.d)
+    assert np.array_equal(R.pred_lb, E.pred_lb) and np.array_equal(R.pred_ub, E.pred_ub)
+    assert_close(R.im_lb, E.im_lb, "im_lb", 1e-12)
+    assert_close(R.im_ub, E.im_ub, "im_ub", 1e-12)
+    # the set goes on through the network like any other
+    Wt = rs.randn(3, 3, C, 2)
+    conv = nnv.Conv2DLayer(Wt, rs.randn(2), [1, 1, 1, 1], [1, 1], [1, 1])
+    R2 = conv.reach(R, "relax-star-area")
+    E2 = o.conv2d_reach(E, Wt, conv.Bias, (1, 1, 1, 1), (1, 1), (1, 1))
+    assert_close(R2.V, E2.V, "conv after reduceMem")
+
+
+def test_relu_reduce_mem_degenerate_and_star_inputs(nnv):
+    # every neuron inactive: the output is the zero set, l = u = 0, no predicate at all
+    V = np.zeros((3, 3, 1, 3))
+    V[..., 0] = -1.0
+    V[..., 1] = 0.1
+    D = nnv.ImageStar(V, np.zeros((1, 2)), np.zeros(1), -np.ones(2), np.ones(2))
+    O = o.OImageStar(V, np.zeros((1, 2)), np.zeros(1), -np.ones(2), np.ones(2))
+    R = nnv.ReluLayer().reach(D, "relax-star-range-reduceMem", "single", 1)
+    E = o.relu_layer_reach(O, "relax-star-range-reduceMem", 1.0)
+    assert R.numPred == E.numPred == 0
+    assert np.array_equal(np.asarray(R.V), E.V)
+    with pytest.raises(ValueError, match="This reachability method does not exist"):
+        nnv.ReluLayer().reach(D.toStar(), "relax-star-area-reduceMem", "single", 1)

@@ -149,3 +149,59 @@ def test_layers_wrapper():
     assert np.array_equal(rel.V, ref.V) and np.array_equal(rel.C, ref.C)
     with pytest.raises(ValueError):
         o.layers_reach(S, W, b, "tansig", "relax-star-area")
+
+
+# ---- the reduceMem suffix of the ReLU layer (nn/layers/ReluLayer.m:107-146) ---------------------------------
+def test_reduce_mem_single_channel_is_the_box_of_the_ranges_in_pixel_row_order():
+    """One channel: the statements build exactly ImageStar(l, u) of the estimated ranges, except that the
+    generators come in row-major pixel order (i1 outer, i2 inner) instead of MATLAB's column-major one."""
+    rs = np.random.RandomState(0)
+    l = rs.rand(3, 4, 1) - 0.5
+    u = l + rs.rand(3, 4, 1)
+    u[1, 2, 0] = l[1, 2, 0]                     # a degenerate pixel: no generator, not counted
+    I = o.image_star_from_bounds(l, u)
+    I.im_lb = I.im_ub = None                    # (ranges are then recomputed from V: l, u up to rounding)
+    R = o.relu_reduce_mem(I)
+    rl, ru = o.image_star_estimate_ranges(I)
+    assert R.numPred == 11 and R.V.shape == (3, 4, 1, 12)
+    assert np.array_equal(R.V[..., 0], 0.5 * (ru + rl))
+    order = [(i1, i2) for i1 in range(3) for i2 in range(4) if (i1, i2) != (1, 2)]
+    for g, (i1, i2) in enumerate(order):
+        col = R.V[..., 1 + g]
+        assert col[i1, i2, 0] == 0.5 * (ru[i1, i2, 0] - rl[i1, i2, 0])
+        assert np.count_nonzero(col) == 1
+    assert np.array_equal(R.C, np.zeros((1, 11))) and np.array_equal(R.d, np.zeros(1))
+    assert np.array_equal(R.pred_lb, -np.ones(11)) and np.array_equal(R.pred_ub, np.ones(11))
+    assert R.im_lb is not None and np.array_equal(R.im_lb, rl) and np.array_equal(R.im_ub, ru)
+    # closed form: the new set's own ranges are centre -/+ half-width
+    R.im_lb = R.im_ub = None
+    bl, bu = o.image_star_estimate_ranges(R)
+    assert np.allclose(bl, rl, rtol=0, atol=1e-15) and np.allclose(bu, ru, rtol=0, atol=1e-15)
+
+
+def test_reduce_mem_with_channels_follows_the_reference_statements():
+    """Hand-written 2 x 1 x 2 case.  v(i1,i2) reads channel 1 only; its value goes to every channel of the pixel;
+    n counts elements, so one generator per pixel is filled and the others stay zero."""
+    l = np.array([[[0.0, -1.0]], [[2.0, 3.0]]])       # l(:,:,1) = [0; 2], l(:,:,2) = [-1; 3]
+    u = np.array([[[4.0, 1.0]], [[2.0, 5.0]]])        # u(:,:,1) = [4; 2], u(:,:,2) = [ 1; 5]
+    I = o.image_star_from_bounds(l, u)
+    R = o.relu_reduce_mem(I)
+    # l - u is non-zero for three elements -> n = 3; pixel (1,1): v = 2 -> generator 1 = 2 on both channels;
+    # pixel (2,1): v(2,1) = 0 on channel 1 -> no generator although channel 2 has width 2
+    assert R.numPred == 3
+    exp = np.zeros((2, 1, 2, 4))
+    exp[:, 0, 0, 0] = [2.0, 2.0]
+    exp[:, 0, 1, 0] = [0.0, 4.0]
+    exp[0, 0, :, 1] = 2.0
+    assert np.array_equal(R.V, exp)
+
+
+def test_reduce_mem_routing_by_set_type():
+    rs = np.random.RandomState(1)
+    lb = rs.rand(4, 4, 1) - 0.6
+    I = o.image_star_from_bounds(lb, lb + 0.5)
+    A = o.relu_layer_reach(I, "relax-star-area-reduceMem")
+    B = o.relu_reduce_mem(o.relu_reach(I, "relax-star-area"))
+    assert np.array_equal(A.V, B.V)
+    with pytest.raises(ValueError, match="This reachability method does not exist"):
+        o.relu_layer_reach(I.to_star(), "relax-star-area-reduceMem")
