@@ -204,3 +204,28 @@ def test_relu_layer_on_an_image_star_with_relax_factor(nnv, oracle):
         assert_close(R.V.reshape(-1, R.numPred + 1, order="F"), E.V.reshape(-1, E.numPred + 1, order="F"), "V", 1e-7)
         assert_close(R.C, E.C, "C", 1e-7)
         assert_close(R.pred_ub, E.pred_ub, "pred_ub", 1e-7)
+
+
+# ---- the six heuristics' bookkeeping on the hand-built star (expectations derived on paper from the reference's
+# statements: tests/relax_lp_hand_case.py), device path against those lists, not against the oracle's twin of the
+# same bookkeeping
+@pytest.mark.parametrize("method,rf", [("relax-star-range", 0.5), ("relax-star-area", 0.5), ("relax-star-static", 0.5),
+                                       ("relax-star-random", 0.5), ("relax-star-bound", 0.5), ("relax-star-bound", 0.25),
+                                       ("relax-star-ub", 0.5), ("relax-star-ub", 0.25)])
+def test_hand_case_bookkeeping(nnv, oracle, method, rf):
+    from tests import relax_lp_hand_case as h
+    S = nnv.Star(h.V, h.C, h.d, h.PRED_LB, h.PRED_UB)
+    reset, index, lbs, ubs = h.EXPECTED[(method, rf)]
+    R = nnv.PosLin.reach_relaxed_star_lp(S, method, rf, rng=h.FixedPermutation(h.RANDPERM[3]))
+    ni, idx, clb, cub = R.relu_info()
+    assert ni == len(reset)
+    assert np.array_equal(idx, np.array(index) - 1), "new-predicate order"
+    np.testing.assert_allclose(clb, lbs, rtol=0, atol=1e-8)
+    np.testing.assert_allclose(cub, ubs, rtol=0, atol=1e-8)
+    # the set itself: what the reference's one-shot step gives for exactly these lists
+    O = oracle.OStar(h.V, h.C, h.d, h.PRED_LB, h.PRED_UB)
+    E = oracle.multiple_step_reach_star_approx_at_one(oracle.reset_row(O, np.array(reset) - 1), np.array(index) - 1,
+                                                      np.array(lbs), np.array(ubs))
+    _same_set(R, E, 1e-8, "%s rf=%g" % (method, rf))
+    zero_rows = np.flatnonzero(~np.asarray(R.V)[:, :3].any(axis=1))
+    assert sorted(zero_rows + 1) == sorted(reset + index)

@@ -189,3 +189,32 @@ def test_lp_box_and_interval_box_known_answers(golden):
     lb, ub = o.estimate_ranges(o.OStar(I1.V, I1.C, I1.d, plb, pub))
     np.testing.assert_allclose(lb, g["B2_lb"].reshape(-1), rtol=0, atol=1e-8)
     np.testing.assert_allclose(ub, g["B2_ub"].reshape(-1), rtol=0, atol=1e-8)
+
+
+# ---- the six heuristics' bookkeeping on a star whose LPs can be done by hand -------------------------------
+def test_hand_case_lp_values():
+    from tests import relax_lp_hand_case as h
+    S = o.OStar(h.V, h.C, h.d, h.PRED_LB, h.PRED_UB)
+    lb, ub = o.estimate_ranges(S)
+    assert np.array_equal(lb, [-1, -4.5, -1.5, -2.5, 1.5, -1.75, -1.125, -0.75])
+    assert np.array_equal(ub, [3, 3.5, 6.5, -1.5, 2.5, 2.25, 0.875, 1.25])
+    np.testing.assert_allclose(o.get_maxs(S, np.arange(8)), [1, -0.5, 6.5, -1.5, 2.5, 2.25, 0.875, 0.25], rtol=0, atol=1e-9)
+    np.testing.assert_allclose(o.get_mins(S, np.arange(8)), [-1, -4.5, 2.5, -2.5, 1.5, -1.75, -1.125, -0.75], rtol=0, atol=1e-9)
+
+
+@pytest.mark.parametrize("method,rf", [("relax-star-range", 0.5), ("relax-star-area", 0.5), ("relax-star-static", 0.5),
+                                       ("relax-star-random", 0.5), ("relax-star-bound", 0.5), ("relax-star-bound", 0.25),
+                                       ("relax-star-ub", 0.5), ("relax-star-ub", 0.25)])
+def test_hand_case_bookkeeping(method, rf):
+    from tests import relax_lp_hand_case as h
+    S = o.OStar(h.V, h.C, h.d, h.PRED_LB, h.PRED_UB)
+    reset, index, lbs, ubs = h.EXPECTED[(method, rf)]
+    R = o.reach_relaxed_star_lp(S, method, rf, rng=h.FixedPermutation(h.RANDPERM[3]))
+    E = o.multiple_step_reach_star_approx_at_one(o.reset_row(S, np.array(reset) - 1), np.array(index) - 1,
+                                                 np.array(lbs), np.array(ubs))
+    assert R.V.shape == E.V.shape and R.C.shape == E.C.shape
+    assert np.array_equal(R.V, E.V)                      # rows reset, unit vectors in the expected order
+    np.testing.assert_allclose(R.C, E.C, rtol=0, atol=1e-8)
+    np.testing.assert_allclose(R.d, E.d, rtol=0, atol=1e-8)
+    np.testing.assert_allclose(R.predicate_ub, E.predicate_ub, rtol=0, atol=1e-8)
+    assert np.array_equal(R.predicate_lb, E.predicate_lb)
