@@ -166,6 +166,12 @@ NNVHIP_API int nnvhip_star_release(nnvhip_star* s);
 NNVHIP_API int nnvhip_star_release_array(int64_t count, nnvhip_star* const* sets);
 /* dim, nVar and the number of constraint rows size(C,1). */
 NNVHIP_API int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p);
+/* flag = 1 when the set, or the set it was derived from by the layers of this library, was created with
+ * constraint rows of the caller's (the five-argument Star(V, C, d, lb, ub), set/Star.m:153-189, with a non-empty
+ * C).  Such a set may be empty; Star(lb, ub) and everything the affine and ReLU layers make of a non-empty set
+ * is not.  verify_specification uses it to decide whether Star.isEmptySet (set/Star.m:1216-1232) may be
+ * skipped for a set that lies inside a half-space. */
+NNVHIP_API int nnvhip_star_has_user_constraints(const nnvhip_star* s, int32_t* flag);
 /* Property reads: dense MATLAB arrays.  V: N x (n+1).  Bounds: n each.  C: p x n, d: p, laid out
  * exactly as PosLin.multipleStepReachStarApprox_at_one builds them, [C0;C1;C2;C3]
  * (nn/funcs/PosLin.m:711-735), materialised from the device's structured store. */

@@ -798,6 +798,14 @@ int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p) {
   return NNVHIP_OK;
 }
 
+int nnvhip_star_has_user_constraints(const nnvhip_star* s, int32_t* flag) {
+  if (!s || !flag) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  const ConsNode* nd = s->cons.get();
+  while (nd && nd->prev) nd = nd->prev.get();
+  *flag = (nd && nd->C0) ? 1 : 0;  // the base node holds dense rows only when a caller handed some in
+  return NNVHIP_OK;
+}
+
 int nnvhip_star_fetch_V(const nnvhip_star* s, double* V) {
   if (!s || !V) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   nnvhip_ctx* c = s->ctx;

@@ -3,6 +3,8 @@
 // are bounded over the predicate box by the estimateRanges kernels, and the three-way verdict per
 // (set, half-space) is formed on the host from R x count doubles.  The dense constraint matrix is
 // never touched here.
+#include <algorithm>
+#include <cmath>
 #include <memory>
 #include <vector>
 
@@ -11,6 +13,8 @@
 using namespace nnvhip;
 
 namespace {
+
+constexpr double kSpecMargin = 1e-9;  // relative to max(|lo|, |hi|, |g|) of the row
 
 struct FcGuard {
   nnvhip_fc* fc = nullptr;
@@ -67,7 +71,11 @@ int nnvhip_halfspace_check(nnvhip_ctx* c, int64_t count, nnvhip_star* const* set
     for (int64_t h = 0; h < n_hs; ++h) {
       bool disjoint = false, inside = true;
       for (int64_t r = row_ptr[h]; r < row_ptr[h + 1]; ++r) {
-        disjoint = disjoint || l[r] > g[r];
+        // "disjoint" is the verdict a caller reports as robust, and the bounds carry rounding of the order of
+        // the row's scale: a pair is only called disjoint with a margin beyond that; a pair inside the margin
+        // stays undecided and goes to the LP, as the reference decides every pair
+        const double scale = std::max(std::max(std::fabs(l[r]), std::fabs(u[r])), std::fabs(g[r]));
+        disjoint = disjoint || l[r] - g[r] > kSpecMargin * scale;
         inside = inside && u[r] <= g[r];
       }
       if (verdict) verdict[s + count * h] = disjoint ? NNVHIP_HS_DISJOINT : inside ? NNVHIP_HS_INSIDE : NNVHIP_HS_UNDECIDED;

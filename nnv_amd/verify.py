@@ -125,13 +125,23 @@ def intersection_is_empty(S: Star, H: HalfSpace, cache=None) -> bool:
     return _lp_is_empty(np.vstack([Cm, C1]), np.concatenate([d, d1]), plb, pub)
 
 
-def verify_specification(reachSet, property, assume_nonempty=True) -> int:
+def _may_be_empty(S) -> bool:
+    """True for a set that carries constraint rows of the caller's (it may be empty); False for Star(lb, ub) and
+    whatever the layers of this library made of it."""
+    flag = C.c_int32(0)
+    check(S.ctx.lib.nnvhip_star_has_user_constraints(S._h.h, C.byref(flag)))
+    return bool(flag.value)
+
+
+def verify_specification(reachSet, property, assume_nonempty=None) -> int:
     """utils/verify_specification.m:36-80.  property: a HalfSpace or a list of them (an OR of unsafe
     regions).  Returns 1 when no output set meets any half-space, else 2.
 
     assume_nonempty: sets produced by reach from a non-empty input set are non-empty (they contain
     the image of every input point), so a pair the device reports INSIDE is a non-empty
-    intersection without an LP.  Pass False for hand-built sets whose (C, d) may be infeasible.
+    intersection without an LP.  Default (None): decided per set -- a set that goes back to a
+    Star(V, C, d, ...) with constraint rows of the caller's may be empty and gets its LP; True / False
+    force the choice for every set.
     """
     global last_stats
     last_stats = SpecStats()
@@ -149,7 +159,7 @@ def verify_specification(reachSet, property, assume_nonempty=True) -> int:
             v = verdict[k, h]
             if v == HS_DISJOINT:
                 continue
-            if v == HS_INSIDE and assume_nonempty:
+            if v == HS_INSIDE and (assume_nonempty if assume_nonempty is not None else not _may_be_empty(S)):
                 return 2
             if not intersection_is_empty(S, H, caches[k]):
                 return 2

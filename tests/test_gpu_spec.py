@@ -160,9 +160,29 @@ def test_hand_built_empty_set_and_errors(nnv):
     S = nnv.Star(np.array([[0.0, 1.0], [0.0, 0.5]]), np.array([[1.0]]), np.array([-2.0]), [-1.0], [1.0])
     H = nnv.HalfSpace([[1.0, 0.0]], [10.0])
     assert nnv.verify_specification(S, H, assume_nonempty=False) == 1
+    assert nnv.verify_specification(S, H) == 1            # default: a set with the caller's own constraints gets its LP
+    assert nnv.verify_specification(S, H, assume_nonempty=True) == 2
+    # ... also after it went through layers: the emptiness travels with the constraints
+    mapped = nnv.PosLin.reach(S.affineMap(np.array([[1.0, -1.0], [0.5, 2.0]]), np.array([0.1, -0.2])), "relax-star-area", [], 1)
+    assert nnv.verify_specification(mapped, nnv.HalfSpace([[1.0, 0.0]], [100.0])) == 1
     So = o.OStar(np.array([[0.0, 1.0], [0.0, 0.5]]), np.array([[1.0]]), np.array([-2.0]), [-1.0], [1.0])
     assert o.verify_specification(So, o.OHalfSpace([[1.0, 0.0]], [10.0])) == 1
     with pytest.raises(ValueError, match="Inconsistent dimension between halfspace and star set"):
         nnv.verify_specification(S, nnv.HalfSpace([[1.0, 0.0, 0.0]], [0.0]))
     with pytest.raises(ValueError, match="Inconsistent dimension between half-space matrix and half-space vector"):
         nnv.HalfSpace([[1.0, 0.0]], [0.0, 1.0])
+
+
+def test_disjoint_needs_a_margin(nnv):
+    """A set that touches the half-space to within rounding is not called disjoint by the device pass: the pair
+    goes to the LP like every pair does in the reference."""
+    from nnv_amd import verify
+    S = nnv.Star(np.array([1.0, 0.0]), np.array([2.0, 1.0]))        # x1 in [1, 2]
+    near = nnv.HalfSpace([[1.0, 0.0]], [1.0 - 1e-13])                # x1 <= 1 - 1e-13: lo - g = 1e-13, inside the margin
+    far = nnv.HalfSpace([[1.0, 0.0]], [1.0 - 1e-6])
+    v, lo, hi = verify.halfspace_check(S, [near, far])
+    assert v[0, 0] == verify.HS_UNDECIDED and v[0, 1] == verify.HS_DISJOINT
+    # the LP settles it as the reference's does: feasible within the solver's tolerance -> "unknown", not "robust"
+    So = o.star_from_box(np.array([1.0, 0.0]), np.array([2.0, 1.0]))
+    assert nnv.verify_specification(S, near) == o.verify_specification(So, o.OHalfSpace([[1.0, 0.0]], [1.0 - 1e-13])) == 2
+    assert nnv.verify_specification(S, far) == o.verify_specification(So, o.OHalfSpace([[1.0, 0.0]], [1.0 - 1e-6])) == 1
