@@ -38,8 +38,18 @@ function result = verify_specification(reachSet, property)
                 case 1
                     continue;    % lower bound of some row exceeds g: the LP is infeasible
                 case 3
-                    result = 2;  % the whole (non-empty) reach set satisfies the half-space
-                    return;
+                    % the whole reach set satisfies the half-space.  A set made by reach from Star(lb,ub) is not
+                    % empty; one that goes back to constraint rows of the caller's gets Star.isEmptySet
+                    dims = nnvhip_mex('star_dims', h(k));
+                    if dims(4) == 0
+                        result = 2;
+                        return;
+                    end
+                    if isempty(host{k}), host{k} = sets(k).gather(); end
+                    if ~host{k}.isEmptySet
+                        result = 2;
+                        return;
+                    end
                 otherwise
                     if isempty(host{k}), host{k} = sets(k).gather(); end   % Star(V, C, d, pred_lb, pred_ub)
                     S = host{k}.intersectHalfSpace(double(property(c).G), double(property(c).g));
