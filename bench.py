@@ -45,17 +45,26 @@ HBM_PEAK_GBS = 8000.0
 MIN_WARM_SECONDS = 0.3
 
 
+# kernels whose launches a timed group of the library covers (nnvhip_kernel_time), by the group's label below
+GROUP_KERNELS = {
+    "gemm_f64_kernel": ("gemm_f64_kernel", "gemm_seg_kernel"),
+    "gather_columns_kernel": ("gather_columns_kernel", "fc_rowsum_kernel", "conv_stamp_kernel"),
+    "relu_classify_kernel": ("relu_classify_kernel", "relu_count_kernel", "relu_compact_kernel"),
+}
+
+
 def profile_traffic(workload, kernel, variant=""):
     """HBM bytes per launch of a kernel group from profiles/<workload>[_<variant>]_hbm_traffic.md (scaled
     FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc runs; the table's last two columns are MiB read / written per
-    dispatch).  Instantiations of the group are averaged by their dispatch counts.  None if there is no table."""
+    dispatch).  The kernels of the group are averaged by their dispatch counts.  None if there is no table."""
     path = os.path.join(ROOT, "profiles", "%s%s_hbm_traffic.md" % (workload, "_" + variant if variant else ""))
     if not os.path.exists(path):
         return None
+    names = GROUP_KERNELS.get(kernel, (kernel,))
     disp, mib = 0, 0.0
     for line in open(path):
         m = re.match(r"\|\s*`([^`]+)`\s*\|\s*(\d+)\s*\|[^|]*\|[^|]*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|", line)
-        if m and kernel in m.group(1):
+        if m and any(nm in m.group(1) for nm in names):
             n = int(m.group(2))
             disp += n
             mib += n * (float(m.group(3)) + float(m.group(4)))
@@ -314,6 +323,9 @@ def measure(k, args, ctx, exact_steps, extras):
         if n_sets < 256:
             c["latency_bound"] = True
         groups.append((cls_ms, c))
+    for _, g in groups:
+        if g["kernel"] in GROUP_KERNELS:
+            g["kernels_in_group"] = list(GROUP_KERNELS[g["kernel"]])
     groups.sort(key=lambda g: -g[0])
     if chain_launches:
         # the measured step is one launch of the whole-reach kernel, one block per set: a chain of dependent phases
@@ -327,6 +339,8 @@ def measure(k, args, ctx, exact_steps, extras):
         roofline = c
         roofline["other_kernels"] = []
         roofline["layer_by_layer_kernels"] = [g[1] for g in groups]
+        if args.method == "relax-star-area":
+            roofline["traffic"] = profile_traffic(cfg["name"], "reach_chain_kernel", variant)
     else:
         roofline = dict(groups[0][1])
         roofline["other_kernels"] = [g[1] for g in groups[1:]]

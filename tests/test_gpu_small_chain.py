@@ -1,6 +1,8 @@
 """NN.reach of small fully connected networks as ONE launch (nnvhip_reach_layers, chain.hip) against the
 oracle and against the layer-by-layer path of the same library: every layer's set, the crossing lists in
 new-predicate order, the constraint rows, for single sets and arrays, in all three crossing orders."""
+import os
+
 import numpy as np
 import pytest
 
@@ -52,7 +54,10 @@ def _check_against_oracle(nnv, oracle, layers, dev_in, ora_in, method, expect_ch
     ctx = nnv.default_context()
     net = nnv.NN.from_config(layers)
     out, launches = _chain_launches(ctx, lambda: net.reach(dev_in, {"reachMethod": method, "relaxFactor": 1}))
-    assert launches == (1 if expect_chain else 0)
+    if os.environ.get("NNVHIP_NO_SMALL_CHAIN") or os.environ.get("NNVHIP_DENSE_AFFINE"):
+        assert launches in (0, 1)     # a run under the switches that keep networks on the layer-by-layer path
+    else:
+        assert launches == (1 if expect_chain else 0)
     exp, exp_sets = oracle.nn_reach(layers, ora_in, method, 1.0, keep=True)
     many = isinstance(ora_in, list)
     prev = ora_in
