@@ -323,6 +323,7 @@ def measure(k, args, ctx, exact_steps, extras):
         if n_sets < 256:
             c["latency_bound"] = True
         groups.append((cls_ms, c))
+    variant = "dense_contraction" if args.dense else ""
     for _, g in groups:
         if g["kernel"] in GROUP_KERNELS:
             g["kernels_in_group"] = list(GROUP_KERNELS[g["kernel"]])
@@ -344,7 +345,6 @@ def measure(k, args, ctx, exact_steps, extras):
     else:
         roofline = dict(groups[0][1])
         roofline["other_kernels"] = [g[1] for g in groups[1:]]
-    variant = "dense_contraction" if args.dense else ""
     if args.method == "relax-star-area":
         roofline["traffic"] = profile_traffic(cfg["name"], roofline["kernel"], variant)
         for g in roofline["other_kernels"]:

@@ -142,6 +142,11 @@ class NN:
         sets, single = _as_list(inSet)
         if not len(sets):
             return False
+        if len(sets) >= 64:
+            # a large array: its layers take milliseconds, the loop's Python costs nothing next to them, and the loop
+            # lets go of the previous reach's thousands of handles while the first layer runs (here they would go
+            # after the call, with the device idle)
+            return False
         try:
             shapes = _shapes(sets)
         except TypeError:
