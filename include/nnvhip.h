@@ -172,6 +172,13 @@ NNVHIP_API int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, in
  * is not.  verify_specification uses it to decide whether Star.isEmptySet (set/Star.m:1216-1232) may be
  * skipped for a set that lies inside a half-space. */
 NNVHIP_API int nnvhip_star_has_user_constraints(const nnvhip_star* s, int32_t* flag);
+/* flag = 1 when the reference's Star would carry an outer zonotope Z here: Star(lb, ub) sets
+ * Z = Zono(center, gens) (set/Star.m:230-236), Star.affineMap maps it along (set/Star.m:332-340,
+ * set/Zono.m:47-74), the five-argument constructor and the ReLU step leave it empty
+ * (nn/funcs/PosLin.m:740).  Z is not stored: wherever it exists it is Zono(V(:,1), V(:,2:end)) of the same set
+ * (both start from the same centre and generators and are mapped by the same W, b), so a caller that wants it
+ * reads V. */
+NNVHIP_API int nnvhip_star_has_zono(const nnvhip_star* s, int32_t* flag);
 /* Property reads: dense MATLAB arrays.  V: N x (n+1).  Bounds: n each.  C: p x n, d: p, laid out
  * exactly as PosLin.multipleStepReachStarApprox_at_one builds them, [C0;C1;C2;C3]
  * (nn/funcs/PosLin.m:711-735), materialised from the device's structured store. */

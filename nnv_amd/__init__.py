@@ -8,5 +8,5 @@ from .layers import Conv2DLayer, FullyConnectedLayer, PosLin, ReluLayer  # noqa:
 from .layers_affine import (AveragePooling2DLayer, BatchNormalizationLayer, FlattenLayer,  # noqa: F401
                             ImageInputLayer, LayerS)
 from .nn import NN  # noqa: F401
-from .sets import Box, ImageStar, SetArray, Star  # noqa: F401
+from .sets import Box, ImageStar, SetArray, Star, Zono  # noqa: F401
 from .verify import HalfSpace, verify_specification  # noqa: F401

@@ -18,7 +18,7 @@ SYMBOLS = [
     "nnvhip_create", "nnvhip_destroy", "nnvhip_last_error", "nnvhip_synchronize", "nnvhip_set_timing",
     "nnvhip_last_op_time_ms", "nnvhip_set_dense_affine", "nnvhip_set_eager_columns", "nnvhip_set_eager_relu", "nnvhip_set_small_chain", "nnvhip_upload_stats", "nnvhip_kernel_time", "nnvhip_probe_copy_bandwidth",
     "nnvhip_trim_pool", "nnvhip_pool_stats", "nnvhip_star_create",
-    "nnvhip_star_from_box", "nnvhip_star_retain", "nnvhip_star_release", "nnvhip_star_release_array", "nnvhip_star_dims", "nnvhip_star_has_user_constraints",
+    "nnvhip_star_from_box", "nnvhip_star_retain", "nnvhip_star_release", "nnvhip_star_release_array", "nnvhip_star_dims", "nnvhip_star_has_user_constraints", "nnvhip_star_has_zono",
     "nnvhip_star_fetch_V", "nnvhip_star_fetch_pred_bounds", "nnvhip_star_fetch_constraints",
     "nnvhip_star_relu_counts", "nnvhip_star_fetch_crossing", "nnvhip_estimate_ranges",
     "nnvhip_estimate_ranges_batch", "nnvhip_fc_create", "nnvhip_fc_destroy", "nnvhip_conv2d_create",
@@ -77,6 +77,7 @@ def load():
         "nnvhip_star_release_array": [i64, pp],
         "nnvhip_star_dims": [p, pi64, pi64, pi64],
         "nnvhip_star_has_user_constraints": [p, p],
+        "nnvhip_star_has_zono": [p, p],
         "nnvhip_star_fetch_V": [p, p],
         "nnvhip_star_fetch_rows": [p, i64, p, p],
         "nnvhip_star_fetch_pred_bounds": [p, p, p],

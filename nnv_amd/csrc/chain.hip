@@ -661,6 +661,7 @@ int reach_small_chain(nnvhip_ctx* c, int64_t n_layers, const int32_t* kind, cons
         o->plb = prev->plb;
         o->pub = prev->pub;
         o->cons = prev->cons;
+        o->has_zono = prev->has_zono;
         o->rbuf = arena;
         o->lb = A + L.rng_off;
         o->ub = o->lb + L.ld;

@@ -631,6 +631,7 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
     base->p_total = 1;
     base->n_total = st->n;
     st->cons = base;  // C0/d0 left null = all zeros
+    st->has_zono = true;  // Z = Zono(center, gens), set/Star.m:230-236
     if (st->n > 0) {  // every generator column is vec(dim) * e_dim
       st->oh_from = 1;
       st->oh_idx_buf = dgen;
@@ -795,6 +796,12 @@ int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p) {
   if (N) *N = s->N;
   if (n) *n = s->n;
   if (p) *p = s->cons ? s->cons->p_total : 0;
+  return NNVHIP_OK;
+}
+
+int nnvhip_star_has_zono(const nnvhip_star* s, int32_t* flag) {
+  if (!s || !flag) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  *flag = s->has_zono ? 1 : 0;
   return NNVHIP_OK;
 }
 
@@ -1173,6 +1180,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
   NNV_TRY(c->begin_op());
   int st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
   if (st == NNVHIP_OK) {
+    for (int64_t i = 0; i < count; ++i) outs[i]->has_zono = in[i]->has_zono;  // Z.affineMap(W, b), set/Star.m:332-340
     const double* bias = fc->bias ? fc->bias->as<double>() : nullptr;
     const double* Wd = fc->W->as<double>();
     // Columns of V that are scaled unit vectors (all generators of a box star, the columns a ReLU

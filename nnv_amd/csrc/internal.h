@@ -320,6 +320,12 @@ struct nnvhip_star {
   bool has_producer_sums() const { return (rng_part != nullptr && rng_chunks > 0) || rng_mm != nullptr; }
   // some scale of the unit-vector block is negative (a box with ub < lb): sign-split products do not apply
   bool oh_scale_neg = false;
+  // The reference's Star carries an outer zonotope Z from Star(lb, ub) on (set/Star.m:220-237) and maps it along in
+  // affineMap (:332-340, set/Zono.m:47-74) until the ReLU step returns a Star without one (nn/funcs/PosLin.m:740).
+  // Z = Zono(V(:,1), V(:,2:end)) of the same set all the way -- Star(lb, ub) builds both from the same centre and
+  // generators, and both are mapped by the same W, b -- so it is not stored: the handle only remembers whether
+  // the reference's set would have one.
+  bool has_zono = false;
   // where gathered columns came from, and whether they (and leading zero columns) are in memory yet
   nnvhip::ColSource cs;
 };

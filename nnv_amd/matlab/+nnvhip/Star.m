@@ -65,19 +65,32 @@ classdef Star < Star
             V = nnvhip_mex('fetch_V', obj.dev.h);
             [C, d] = nnvhip_mex('fetch_constraints', obj.dev.h);
             [plb, pub] = nnvhip_mex('fetch_pred', obj.dev.h);
-            S = Star(V, C, d, plb, pub);
+            dims = nnvhip_mex('star_dims', obj.dev.h);
+            if dims(5) ~= 0      % the outer zonotope of Star(lb,ub) and its affine images (Star.m:230-236, 332-340)
+                S = Star(V, C, d, plb, pub, Zono(V(:, 1), V(:, 2:end)));
+            else
+                S = Star(V, C, d, plb, pub);
+            end
             S.state_lb = obj.state_lb; S.state_ub = obj.state_ub;
         end
         function varargout = subsref(obj, s)
             % lazy property reads: S.V, S.C, S.d, S.predicate_lb, S.predicate_ub fetch from the device
             if isscalar(obj) && strcmp(s(1).type, '.') && ~isempty(obj.dev) && ...
-                    any(strcmp(s(1).subs, {'V', 'C', 'd', 'predicate_lb', 'predicate_ub'}))
+                    any(strcmp(s(1).subs, {'V', 'C', 'd', 'predicate_lb', 'predicate_ub', 'Z'}))
                 switch s(1).subs
                     case 'V', val = nnvhip_mex('fetch_V', obj.dev.h);
                     case 'C', [val, ~] = nnvhip_mex('fetch_constraints', obj.dev.h);
                     case 'd', [~, val] = nnvhip_mex('fetch_constraints', obj.dev.h);
                     case 'predicate_lb', [val, ~] = nnvhip_mex('fetch_pred', obj.dev.h);
                     case 'predicate_ub', [~, val] = nnvhip_mex('fetch_pred', obj.dev.h);
+                    case 'Z'     % Star(lb,ub) and its affine images: Zono(c, gens) of the same set (Star.m:230-236, 332-340)
+                        dims = nnvhip_mex('star_dims', obj.dev.h);
+                        if dims(5) ~= 0
+                            Vz = nnvhip_mex('fetch_V', obj.dev.h);
+                            val = Zono(Vz(:, 1), Vz(:, 2:end));
+                        else
+                            val = [];
+                        end
                 end
                 if numel(s) > 1
                     [varargout{1:nargout}] = subsref(val, s(2:end));

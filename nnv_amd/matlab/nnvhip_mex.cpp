@@ -100,18 +100,21 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
     need(nrhs, 1, "star_release");
     const std::vector<nnvhip_star*> hs = handles_of(prhs[1]);
     check(nnvhip_star_release_array((int64_t)hs.size(), hs.data()));
-  } else if (cmd == "star_dims") {  // handle -> [dim nVar nConstraintRows mayBeEmpty]
+  } else if (cmd == "star_dims") {  // handle -> [dim nVar nConstraintRows mayBeEmpty hasZono]
     need(nrhs, 1, "star_dims");
     int64_t N, n, p;
     int32_t user = 0;
     check(nnvhip_star_dims(handle_of<nnvhip_star>(prhs[1]), &N, &n, &p));
     check(nnvhip_star_has_user_constraints(handle_of<nnvhip_star>(prhs[1]), &user));
-    plhs[0] = mxCreateDoubleMatrix(1, 4, mxREAL);
+    int32_t zono = 0;
+    check(nnvhip_star_has_zono(handle_of<nnvhip_star>(prhs[1]), &zono));
+    plhs[0] = mxCreateDoubleMatrix(1, 5, mxREAL);
     double* o = mxGetDoubles(plhs[0]);
     o[0] = (double)N;
     o[1] = (double)n;
     o[2] = (double)p;
     o[3] = (double)user;  // 1: the set goes back to constraint rows the caller handed in (it may be empty)
+    o[4] = (double)zono;  // 1: the reference's Star carries an outer zonotope here (= Zono(V(:,1), V(:,2:end)))
   } else if (cmd == "fetch_V") {  // handle -> V (dim x (nVar+1))
     need(nrhs, 1, "fetch_V");
     nnvhip_star* s = handle_of<nnvhip_star>(prhs[1]);

@@ -211,17 +211,36 @@ class Box:
         return Star(self.lb, self.ub, ctx=ctx)
 
 
+class Zono:
+    """Zono(c, V), set/Zono.m:13-45: x = c + V*a, -1 <= a <= 1 (a plain host object)."""
+
+    def __init__(self, c, V):
+        self.c = np.asarray(c, dtype=np.float64).reshape(-1)
+        self.V = np.asarray(V, dtype=np.float64).reshape(self.c.size, -1)
+        self.dim = self.c.size
+
+    def affineMap(self, W, b=None):
+        """Zono.affineMap, set/Zono.m:47-74."""
+        W = np.asarray(W, dtype=np.float64)
+        c = W @ self.c
+        if b is not None and np.size(b):
+            c = c + np.asarray(b, dtype=np.float64).reshape(-1)
+        return Zono(c, W @ self.V)
+
+
 class Star:
     """Device-resident Star: x = c + V*a, C*a <= d, predicate_lb <= a <= predicate_ub.
 
     Constructors (set/Star.m:29-275): ``Star(V, C, d, pred_lb, pred_ub)``, ``Star(V, C, d)``,
-    ``Star(lb, ub)``.  The outer zonotope ``Z`` of the reference is not carried (only the
-    approx-zono method reads it).
+    ``Star(lb, ub)``.  The outer zonotope ``Z`` of the reference (set by Star(lb, ub), mapped along by
+    affineMap, dropped by the ReLU step) is not stored: where it exists it is Zono(V(:,1), V(:,2:end)) of the
+    same set, and the ``Z`` property builds it from there.
     """
 
     # defaults of the fields a constructor may leave alone (instances made by _from_handle set only _h)
     state_lb = None
     state_ub = None
+    _no_Z = False      # a Star made by ImageStar.toStar (7-argument constructor: no Z, set/ImageStar.m:584-590)
     Z = None
     _lp = None
     _unbounded_predicates = False
@@ -335,6 +354,18 @@ class Star:
     @property
     def predicate_ub(self):
         return self._h.fetch_pred()[1]
+
+    @property
+    def Z(self):
+        """The outer zonotope the reference's Star holds here (set/Star.m:230-236, 332-340), or None."""
+        if self._no_Z:
+            return None
+        flag = C.c_int32(0)
+        check(self.ctx.lib.nnvhip_star_has_zono(self._h.h, C.byref(flag)))
+        if not flag.value:
+            return None
+        V = self._h.fetch_V()
+        return Zono(V[:, 0].copy(), V[:, 1:].copy())
 
     # ---- methods on the path -------------------------------------------------------------
     def affineMap(self, W, b=None):
@@ -565,6 +596,7 @@ class ImageStar:
     def toStar(self):
         """ImageStar.toStar, set/ImageStar.m:569-592: flatten in column-major order (shared data)."""
         S = Star(_handle=self._h)
+        S._no_Z = True
         if self.im_lb is not None and self.im_ub is not None:
             S.state_lb = np.asarray(self.im_lb).reshape(-1, order="F")
             S.state_ub = np.asarray(self.im_ub).reshape(-1, order="F")

@@ -619,3 +619,32 @@ def test_first_layer_centre_with_and_without_degenerate_dimensions(nnv, oracle, 
         assert_close(np.asarray(R.V), E.V, "V", RTOL)
         # generator columns are plain copies of scaled weight columns: exact
         assert np.array_equal(np.asarray(R.V)[:, 1:], E.V[:, 1:])
+
+
+def test_outer_zonotope_follows_the_reference(nnv, oracle):
+    """Star.Z: Zono(center, gens) from Star(lb, ub) (set/Star.m:230-236), mapped by affineMap (:332-340), gone after
+    the ReLU step (nn/funcs/PosLin.m:740) and for sets built from matrices or taken from an ImageStar."""
+    o = oracle
+    rs = np.random.RandomState(4)
+    lb = rs.rand(6) - 0.5
+    ub = lb + rs.rand(6)
+    ub[3] = lb[3]                                   # a degenerate dimension: no generator for it
+    S, O = nnv.Star(lb, ub), o.star_from_box(lb, ub)
+    assert np.array_equal(S.Z.c, O.Z[0]) and np.array_equal(S.Z.V, O.Z[1])
+    W1, b1, W2 = rs.randn(9, 6), rs.randn(9), rs.randn(4, 9)
+    S1, O1 = S.affineMap(W1, b1), o.affine_map(O, W1, b1)
+    S2, O2 = S1.affineMap(W2), o.affine_map(O1, W2)
+    for A, B in ((S1, O1), (S2, O2)):
+        assert_close(A.Z.c, B.Z[0], "Z.c", 1e-13)
+        assert_close(A.Z.V, B.Z[1], "Z.V", 1e-13)
+    R = nnv.PosLin.reach(S1, "relax-star-area", [], 1)
+    assert R.Z is None and o.reach_relaxed_star(O1, "relax-star-area", 1.0).Z is None
+    assert R.affineMap(W2).Z is None
+    # an FC layer on the Star keeps it, the whole-network call too (every set in front of the first ReLU)
+    net = nnv.NN.from_config([{"type": "fc", "W": W1, "b": b1}, {"type": "relu"}, {"type": "fc", "W": W2, "b": np.zeros(4)}])
+    net.reach(S, {"reachMethod": "relax-star-area", "relaxFactor": 1})
+    assert_close(net.reachSet[0].Z.V, O1.Z[1], "Z.V after the FC layer", 1e-13)
+    assert net.reachSet[1].Z is None and net.reachSet[2].Z is None
+    # sets built from matrices and Stars taken from an ImageStar have none
+    assert nnv.Star(rs.randn(3, 3), np.zeros((1, 2)), np.zeros(1), [-1, -1], [1, 1]).Z is None
+    assert nnv.ImageStar(np.zeros((2, 2, 1)), np.ones((2, 2, 1))).toStar().Z is None
