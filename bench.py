@@ -48,6 +48,7 @@ MIN_WARM_SECONDS = 0.3
 # kernels whose launches a timed group of the library covers (nnvhip_kernel_time), by the group's label below
 GROUP_KERNELS = {
     "gemm_f64_kernel": ("gemm_f64_kernel", "gemm_seg_kernel"),
+    "conv2d_fast_kernel": ("conv2d_fast_kernel", "conv2d_f64_kernel"),
     "gather_columns_kernel": ("gather_columns_kernel", "fc_rowsum_kernel", "conv_stamp_kernel"),
     "relu_classify_kernel": ("relu_classify_kernel", "relu_count_kernel", "relu_compact_kernel"),
 }
@@ -296,7 +297,7 @@ def measure(k, args, ctx, exact_steps, extras):
     if gemm_launches:
         groups.append((gemm_ms, mfma_roofline("gemm_f64_kernel", gemm_work, gemm_flop, gemm_ms, gemm_launches)))
     if conv_launches:
-        groups.append((conv_ms, mfma_roofline("conv2d_f64_kernel", conv_work, conv_flop, conv_ms, conv_launches)))
+        groups.append((conv_ms, mfma_roofline("conv2d_fast_kernel", conv_work, conv_flop, conv_ms, conv_launches)))
     if rng_launches:
         groups.append((rng_ms, hbm_roofline("ranges_partial_kernel", rng_ms, rng_launches, rng_bytes)))
     if app_launches:

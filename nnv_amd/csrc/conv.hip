@@ -11,9 +11,12 @@
 // carries output channels.
 #include <algorithm>
 #include <cstring>
+#include <type_traits>
 
 #include "internal.h"
+#include "lds_dma.h"
 #include "mfma_tile.h"
+#include "relu_sort.h"
 
 namespace nnvhip {
 
@@ -26,6 +29,7 @@ struct ConvGeom {
 };
 
 constexpr int kMaxTaps = 4096;  // tap table held in LDS: 8 bytes per (padded) tap
+constexpr size_t kConvLdsLimit = 64 * 1024;  // LDS of one block: operand tiles + tap table + row mask
 
 // Tap k = fh + FH*(fw + FW*ci) -> packed (input offset ci*H*W : 32 | fh*dh : 16 | fw*dw : 16).
 __device__ __forceinline__ unsigned long long pack_tap(const ConvGeom& g, int k) {
@@ -38,12 +42,46 @@ __device__ __forceinline__ unsigned long long pack_tap(const ConvGeom& g, int k)
          (unsigned long long)(fw * g.dw);
 }
 
-template <int TP, int TC, int WR, int WC>
+// Stores a block's accumulators: lane l, register r of acc[i][j] holds out[position R0 + ... + l%16][channel c0 +
+// ... + l/16 + 4r]; the bias goes onto the centre image only.
+template <int TP, int TC, int WR, int WC, int FM, int FN>
+__device__ __forceinline__ void conv_store_tile(const double4_t (&acc)[FM][FN], double* __restrict__ out, int64_t ldout,
+                                                const double* __restrict__ bias, const ConvGeom& g, int64_t total_rows,
+                                                int64_t R0, int c0, int wr, int wc, int lane) {
+  const int lrow = lane & 15;
+  const int lcol = lane >> 4;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int64_t Rr = R0 + wr * (TP / WR) + i * 16 + lrow;
+    if (Rr >= total_rows) continue;
+    const int64_t gi = Rr / g.P;
+    const int p = (int)(Rr - gi * g.P);
+    double* o = out + gi * ldout + p;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int co = c0 + wc * (TC / WC) + j * 16 + lcol + 4 * r;
+        if (co < g.Cout) {
+          double v = acc[i][j][r];
+          if (bias != nullptr && gi == 0) v = v + bias[co];  // centre image only
+          o[(int64_t)co * g.P] = v;
+        }
+      }
+    }
+  }
+}
+
+// MASK: the input is the matrix in front of a ReLU step whose row reset has not been run; `keep` holds one
+// bit per input row (1 = the row is kept, 0 = it reads as zero: PosLin.m:700-709, Star.m:1442-1461), copied
+// into LDS behind the tap table.  A reset row is never loaded.
+template <int TP, int TC, int WR, int WC, bool MASK>
 __global__ __launch_bounds__(64 * WR * WC) void conv2d_f64_kernel(const double* __restrict__ in, int64_t ldin,
                                                           double* __restrict__ out, int64_t ldout,
                                                           const double* __restrict__ Wt,
                                                           const double* __restrict__ bias, ConvGeom g,
-                                                          int64_t total_rows, int tiles_c) {
+                                                          int64_t total_rows, int tiles_c,
+                                                          const uint32_t* __restrict__ keep, int keep_words) {
   constexpr int NT = 64 * WR * WC;  // threads per block
   static_assert(NT % TP == 0 && (TP * kKt) % NT == 0, "gather mapping needs NT = TP * (taps per pass)");
   constexpr int FM = TP / WR / 16;
@@ -64,6 +102,9 @@ __global__ __launch_bounds__(64 * WR * WC) void conv2d_f64_kernel(const double* 
   const int64_t R0 = (bid / tiles_c) * TP;
 
   for (int k = tid; k < g.Kp; k += NT) taps[k] = pack_tap(g, k);
+  uint32_t* keep_s = reinterpret_cast<uint32_t*>(taps + g.Kp);
+  if (MASK)
+    for (int k = tid; k < keep_words; k += NT) keep_s[k] = keep[k];
 
   // this thread's gather position (fixed for the whole K loop)
   constexpr int P_PASS = TP * kKt / NT;  // gathered elements per thread per K-tile
@@ -95,8 +136,10 @@ __global__ __launch_bounds__(64 * WR * WC) void conv2d_f64_kernel(const double* 
       const unsigned long long t = taps[k0 + k_first + q * K_STEP];
       const int h = h0 + (int)((t >> 16) & 0xffffu);
       const int w = w0 + (int)(t & 0xffffu);
-      const bool ok = rvalid && t != ~0ull && (unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W;
-      rp[q] = ok ? img[(int64_t)(unsigned)(t >> 32) + h + (int64_t)w * g.H] : 0.0;
+      bool ok = rvalid && t != ~0ull && (unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W;
+      const int row = ok ? (int)(unsigned)(t >> 32) + h + w * g.H : 0;  // row of the input set (< 2^31)
+      if (MASK) ok = ok && ((keep_s[row >> 5] >> (row & 31)) & 1u) != 0;
+      rp[q] = ok ? img[row] : 0.0;
     }
 #pragma unroll
     for (int q = 0; q < W_PASS; ++q) {
@@ -142,29 +185,188 @@ __global__ __launch_bounds__(64 * WR * WC) void conv2d_f64_kernel(const double* 
     __syncthreads();
   }
 
-  // epilogue: lane l, register r holds out[position R0 + ... + l%16][channel c0 + ... + l/16 + 4r]
-  const int lrow = lane & 15;
-  const int lcol = lane >> 4;
-#pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int64_t Rr = R0 + wr * (TP / WR) + i * 16 + lrow;
-    if (Rr >= total_rows) continue;
-    const int64_t gi = Rr / g.P;
-    const int p = (int)(Rr - gi * g.P);
-    double* o = out + gi * ldout + p;
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int co = c0 + wc * (TC / WC) + j * 16 + lcol + 4 * r;
-        if (co < g.Cout) {
-          double v = acc[i][j][r];
-          if (bias != nullptr && gi == 0) v = v + bias[co];  // centre image only
-          o[(int64_t)co * g.P] = v;
-        }
-      }
-    }
+  conv_store_tile<TP, TC, WR, WC, FM, FN>(acc, out, ldout, bias, g, total_rows, R0, c0, wr, wc, lane);
+}
+
+// ---- the same convolution with little vector-ALU work per MFMA ------------------------------------
+// On this chip the vector ALU does not issue in the shadow of an fp64 MFMA (measured: every extra VALU
+// instruction of a wave costs about as many matrix-pipe cycles as it takes to issue), so the gather of the
+// kernel above - tap decode, bounds checks, a 32-bit multiply and 64-bit address arithmetic per element -
+// costs a third of the MFMA time.  Here a tap is a wave-uniform (row offset, spatial bit) pair read through
+// the scalar unit from a table in global memory, a thread's padding pattern is one 32-bit mask computed once
+// (bit fh + FH*fw: that tap falls inside the image), the element's row is one addition, and its address a
+// 32-bit offset from a block-uniform base.  The weight tile comes k-major from a second copy of the weights
+// straight into LDS (global_load_lds_dwordx4), with no registers or address arithmetic in between.
+// Needs FH*FW <= 32 and a tile's images within 2 GiB of its first one; the host checks both.
+struct FastTap {
+  int32_t off;   // ci*H*W + fh*dh + fw*dw*H: row of the tap relative to the row of tap (0, 0, 0)
+  uint32_t bit;  // 1 << (fh + FH*fw); 0 for a padding entry
+};
+
+__global__ void conv_fast_taps_kernel(FastTap* __restrict__ tab, ConvGeom g) {
+  const int k = blockIdx.x * 256 + threadIdx.x;
+  if (k >= g.Kp) return;
+  FastTap t{0, 0u};
+  if (k < g.K) {
+    const int fh = k % g.FH;
+    const int r = k / g.FH;
+    const int fw = r % g.FW;
+    const int ci = r / g.FW;
+    t.off = ci * g.HW + fh * g.dh + fw * g.dw * g.H;
+    t.bit = 1u << (fh + g.FH * fw);
   }
+  tab[k] = t;
+}
+
+// Wk(k, co) = W(k, co) for co < Cout, zero up to coutp: the weights k-major (row k contiguous over channels)
+__global__ void conv_weights_kmajor_kernel(const double* __restrict__ W, double* __restrict__ Wk, int Kp, int Cout, int coutp) {
+  const int64_t idx = blockIdx.x * (int64_t)256 + threadIdx.x;
+  if (idx >= (int64_t)Kp * coutp) return;
+  const int k = (int)(idx / coutp), co = (int)(idx % coutp);
+  Wk[idx] = co < Cout ? W[k + (int64_t)co * Kp] : 0.0;
+}
+
+template <int TC, int WR, int WC, bool MASK>
+__global__ __launch_bounds__(512) void conv2d_fast_kernel(const double* __restrict__ in, int64_t ldin, double* __restrict__ out,
+                                                          int64_t ldout, const double* __restrict__ Wk, int coutp,
+                                                          const double* __restrict__ bias, ConvGeom g, int64_t total_rows,
+                                                          int tiles_c, const FastTap* __restrict__ taps,
+                                                          const uint32_t* __restrict__ keep, int keep_words) {
+  constexpr int TP = 128, NT = 512;
+  static_assert(WR * WC == 8, "eight waves");
+  constexpr int FM = TP / WR / 16;
+  constexpr int FN = TC / WC / 16;
+  constexpr int kWLoads = kKt * TC / 128;  // 1 KiB wave transfers per K-tile of weights
+  constexpr int kRowsPerLoad = 128 / TC;   // rows of Wk per transfer
+  __shared__ double Ps[2][kKt * TP];                                      // [k][position]
+  __shared__ __attribute__((aligned(1024))) double Wts[2][kKt * TC];     // [k][channel]
+  extern __shared__ uint32_t keep_s[];                                    // row mask (MASK only)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wr = wave % WR;
+  const int wc = wave / WR;
+  const int64_t bid = blockIdx.x;
+  const int c0 = (int)(bid % tiles_c) * TC;
+  const int64_t R0 = (bid / tiles_c) * TP;
+
+  if (MASK)
+    for (int k = tid; k < keep_words; k += NT) keep_s[k] = keep[k];
+
+  // this thread's position (fixed for the whole K loop) and the four consecutive taps of a K-tile it gathers
+  const int p_local = tid & (TP - 1);
+  const int kq = __builtin_amdgcn_readfirstlane(tid >> 7);
+  const int64_t R = R0 + p_local;
+  const bool rvalid = R < total_rows;
+  const int64_t gi0 = R0 / g.P;
+  const char* const base = reinterpret_cast<const char*>(in + gi0 * ldin);  // block-uniform
+  uint32_t toff = 0;
+  int base_row = 0;
+  uint32_t vmask = 0;
+  if (rvalid) {
+    const int64_t gi = R / g.P;
+    const int p = (int)(R - gi * g.P);
+    const int wo = p / g.Ho;
+    const int ho = p - wo * g.Ho;
+    const int h0 = ho * g.sh - g.pt;
+    const int w0 = wo * g.sw - g.pl;
+    toff = (uint32_t)((gi - gi0) * ldin * 8);
+    base_row = h0 + w0 * g.H;
+    for (int fw = 0; fw < g.FW; ++fw)
+      for (int fh = 0; fh < g.FH; ++fh) {
+        const int h = h0 + fh * g.dh, w = w0 + fw * g.dw;
+        if ((unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W) vmask |= 1u << (fh + g.FH * fw);
+      }
+  }
+
+  double rp[4];
+  struct alignas(32) Tap4 {
+    FastTap t[4];
+  };
+  auto gather = [&](int k0) {
+    const Tap4 t4 = *reinterpret_cast<const Tap4*>(taps + k0 + kq * 4);  // wave-uniform: one scalar load
+    int row[4];
+    bool ok[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      row[q] = base_row + t4.t[q].off;
+      ok[q] = (vmask & t4.t[q].bit) != 0;
+    }
+    if (MASK) {
+      // (the row of a tap outside the image may lie outside the mask, even outside the block's LDS, where a
+      // read returns zero: the word read for it is not used)
+      uint32_t b[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) b[q] = keep_s[row[q] >> 5];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) ok[q] = ok[q] && __builtin_amdgcn_ubfe(b[q], (uint32_t)row[q] & 31u, 1u) != 0;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      double v = 0.0;
+      if (ok[q]) v = *reinterpret_cast<const double*>(base + (toff + ((uint32_t)row[q] << 3)));
+      rp[q] = v;
+    }
+  };
+  auto store = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) Ps[buf][(kq * 4 + q) * TP + p_local] = rp[q];
+  };
+  // weights: transfer w of a K-tile brings rows w*kRowsPerLoad ... of the tile; lane l its 16 bytes
+  const unsigned w_lds = lds_addr_of(&Wts[0][0]) + (unsigned)wave * 1024u;
+  const unsigned w_voff = (unsigned)(((lane / (TC / 2)) * coutp + 2 * (lane % (TC / 2))) * 8);
+  const double* const w_base = Wk + (int64_t)(wave * kRowsPerLoad) * coutp + c0;
+  auto dma = [&](int k0, int buf) {
+    if (wave < kWLoads) lds_dma16(w_base + (int64_t)k0 * coutp, w_voff, w_lds + (unsigned)(buf * kKt * TC * 8));
+  };
+
+  double4_t acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j) acc[i][j] = double4_t{0.0, 0.0, 0.0, 0.0};
+
+  __syncthreads();  // row mask in place
+  const int nk = g.Kp / kKt;
+  gather(0);
+  dma(0, 0);
+  store(0);
+  wait_vm<0>();
+  block_barrier();
+  const int l16 = lane & 15, lq = lane >> 4;
+  const double* const ps0 = &Ps[0][wr * (TP / WR) + l16 + lq * TP];
+  const double* const ws0 = &Wts[0][wc * (TC / WC) + l16 + lq * TC];
+  // one K-tile out of buffer `cur` (a constant, so that every LDS address is a base register plus an immediate)
+  auto step = [&](int kt, auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+    if (kt + 1 < nk) {
+      gather((kt + 1) * kKt);
+      dma((kt + 1) * kKt, cur ^ 1);
+    }
+    const double* ps = ps0 + cur * (kKt * TP);
+    const double* ws = ws0 + cur * (kKt * TC);
+#pragma unroll
+    for (int kk = 0; kk < kKt / 4; ++kk) {
+      double b[FM], a[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) b[i] = ps[kk * 4 * TP + i * 16];
+#pragma unroll
+      for (int j = 0; j < FN; ++j) a[j] = ws[kk * 4 * TC + j * 16];
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[j], b[i], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) store(cur ^ 1);
+    wait_vm<0>();     // this wave's weight transfer has landed ...
+    block_barrier();  // ... and everybody's; everybody is done with the tiles of this step
+  };
+  for (int kt = 0; kt < nk; kt += 2) {
+    step(kt, std::integral_constant<int, 0>());
+    if (kt + 1 < nk) step(kt + 1, std::integral_constant<int, 1>());
+  }
+  conv_store_tile<TP, TC, WR, WC, FM, FN>(acc, out, ldout, bias, g, total_rows, R0, c0, wr, wc, lane);
 }
 
 __global__ void zero_pad_rows_kernel(double* __restrict__ V, int64_t ld, int64_t N, int64_t ncols) {
@@ -302,18 +504,42 @@ __global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restr
   }
 }
 
+// One bit per row of a set with a pending row reset: 1 where the row is kept.  Word w covers rows 32w..32w+31.
+__global__ __launch_bounds__(256) void keep_bits_kernel(const int32_t* __restrict__ cls, int64_t N, uint32_t* __restrict__ bits,
+                                                        int words) {
+  const int64_t r = blockIdx.x * (int64_t)256 + threadIdx.x;
+  const unsigned long long b = __ballot(r < N && cls[r] == kKeep);
+  const int lane = threadIdx.x & 63;
+  const int64_t w = r >> 5;
+  if ((lane & 31) == 0 && w < words) bits[w] = (uint32_t)(b >> lane);
+}
+
+// LDS of the convolution kernel beside its tap table and row mask: the two double-buffered operand tiles
+template <int TP, int TC>
+constexpr size_t conv_static_lds() {
+  return sizeof(double) * 2 * (kKt * (TP + kPadRow) + TC * (kKt + kPadK));
+}
+
 template <int TP, int TC, int WR, int WC>
 static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGeom& g, const double* in, int64_t ldin,
-                           double* out, int64_t ldout, int64_t ncols) {
+                           double* out, int64_t ldout, int64_t ncols, const uint32_t* keep, int keep_words) {
   const int64_t total_rows = (int64_t)g.P * ncols;
   const int64_t tiles_c = ceil_div(g.Cout, TC);
   const int64_t blocks = ceil_div(total_rows, TP) * tiles_c;
   if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
-  const size_t dyn = sizeof(unsigned long long) * g.Kp;
+  const size_t dyn = sizeof(unsigned long long) * g.Kp + (keep ? sizeof(uint32_t) * (size_t)keep_words : 0);
+  if (conv_static_lds<TP, TC>() + dyn > kConvLdsLimit)
+    NNV_FAIL(NNVHIP_ERR_SHAPE, "filters with %d taps (FH*FW*Cin) and %d output channels are not supported: at most %d taps", g.K, g.Cout,
+             (int)((kConvLdsLimit - conv_static_lds<TP, TC>()) / sizeof(unsigned long long) / kKt * kKt));
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_f64_kernel<TP, TC, WR, WC>), dim3((unsigned)blocks), dim3(64 * WR * WC), dyn, in, ldin,
-             out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows,
-                     (int)tiles_c);
+  if (keep)
+    NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_f64_kernel<TP, TC, WR, WC, true>), dim3((unsigned)blocks), dim3(64 * WR * WC), dyn, in,
+               ldin, out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows, (int)tiles_c, keep,
+               keep_words);
+  else
+    NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_f64_kernel<TP, TC, WR, WC, false>), dim3((unsigned)blocks), dim3(64 * WR * WC), dyn, in,
+               ldin, out, ldout, cv->W->as<double>(), cv->bias ? cv->bias->as<double>() : nullptr, g, total_rows, (int)tiles_c, keep,
+               keep_words);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 1, 2.0 * (double)total_rows * g.Cout * g.K));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
@@ -321,24 +547,124 @@ static int launch_conv_cfg(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvG
 
 static void fill_geom(ConvGeom& g, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo);
 
+// ---- which kernel, and whether it can mask rows on load --------------------------------------------
+constexpr size_t conv_fast_static_lds(int tc) { return sizeof(double) * 2 * kKt * (128 + (size_t)tc); }
+static int conv_tile_channels(const nnvhip_conv2d* cv) { return cv->Cout <= 16 ? 16 : cv->Cout <= 32 ? 32 : 64; }
+
+// The kernel with scalar tap decoding: at most 32 spatial taps (one mask bit each), every byte offset it forms
+// (a row of the image plus the images a 128-position tile can span) below 2^31.
+static bool conv_fast_ok(const nnvhip_conv2d* cv, const ConvGeom& g, int64_t ldin) {
+  if (tune_knobs().conv_general != 0 || cv->Wk == nullptr) return false;
+  if (cv->FH * cv->FW > 32) return false;
+  const int64_t n_in = (int64_t)g.HW * g.Cin;
+  const int64_t images_per_tile = 127 / g.P + 2;
+  return (n_in + images_per_tile * ldin) * 8 < (int64_t(1) << 31);
+}
+
+bool conv2d_can_mask(const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin) {
+  ConvGeom g;
+  fill_geom(g, cv, H, W, Ho, Wo);
+  const int64_t n_in = H * W * cv->Cin;
+  if (n_in >= (int64_t(1) << 31) || cv->Kp > kMaxTaps) return false;
+  const size_t mask = sizeof(uint32_t) * (size_t)ceil_div(n_in, 32);
+  if (conv_fast_ok(cv, g, ldin)) return conv_fast_static_lds(conv_tile_channels(cv)) + mask <= kConvLdsLimit;
+  // the general kernel, sized for its widest tile (128 x 64): the mask shares the dynamic LDS with the tap table
+  return conv_static_lds<128, 64>() + sizeof(unsigned long long) * (size_t)cv->Kp + mask <= kConvLdsLimit;
+}
+
+int conv2d_prepare_weights(nnvhip_ctx* ctx, nnvhip_conv2d* cv) {
+  cv->coutp = round_up(cv->Cout, 64);
+  if (cv->Kp * cv->coutp >= (int64_t(1) << 28)) return NNVHIP_OK;  // stays on the general kernel
+  NNV_TRY(ctx->alloc(sizeof(double) * cv->Kp * cv->coutp, &cv->Wk));
+  hipLaunchKernelGGL(conv_weights_kmajor_kernel, dim3((unsigned)ceil_div(cv->Kp * cv->coutp, 256)), dim3(256), 0, ctx->stream,
+                     cv->W->as<double>(), cv->Wk->as<double>(), (int)cv->Kp, (int)cv->Cout, (int)cv->coutp);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+static int conv_fast_taps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGeom& g, const FastTap** tab) {
+  for (const auto& t : cv->tap_tables)
+    if (t.H == g.H && t.W == g.W) {
+      *tab = t.tab->as<FastTap>();
+      return NNVHIP_OK;
+    }
+  nnvhip_conv2d::TapTable t;
+  t.H = g.H;
+  t.W = g.W;
+  NNV_TRY(ctx->alloc(sizeof(FastTap) * (size_t)g.Kp, &t.tab));
+  hipLaunchKernelGGL(conv_fast_taps_kernel, dim3((unsigned)ceil_div(g.Kp, 256)), dim3(256), 0, ctx->stream, t.tab->as<FastTap>(), g);
+  NNV_HIP_TRY(hipGetLastError());
+  if (cv->tap_tables.size() >= 8) cv->tap_tables.erase(cv->tap_tables.begin());
+  cv->tap_tables.push_back(t);
+  *tab = t.tab->as<FastTap>();
+  return NNVHIP_OK;
+}
+
+template <int TC, int WR, int WC>
+static int launch_conv_fast(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGeom& g, const double* in, int64_t ldin, double* out,
+                            int64_t ldout, int64_t ncols, const uint32_t* keep, int keep_words) {
+  const int64_t total_rows = (int64_t)g.P * ncols;
+  const int64_t tiles_c = ceil_div(g.Cout, TC);
+  const int64_t blocks = ceil_div(total_rows, 128) * tiles_c;
+  if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
+  const size_t dyn = keep ? sizeof(uint32_t) * (size_t)keep_words : 0;
+  if (conv_fast_static_lds(TC) + dyn > kConvLdsLimit) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: row mask too large for the convolution kernel");
+  const FastTap* taps = nullptr;
+  NNV_TRY(conv_fast_taps(ctx, cv, g, &taps));
+  const double* bias = cv->bias ? cv->bias->as<double>() : nullptr;
+  NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
+  if (keep)
+    NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, true>), dim3((unsigned)blocks), dim3(512), dyn, in, ldin, out,
+               ldout, cv->Wk->as<double>(), (int)cv->coutp, bias, g, total_rows, (int)tiles_c, taps, keep, keep_words);
+  else
+    NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, false>), dim3((unsigned)blocks), dim3(512), dyn, in, ldin, out,
+               ldout, cv->Wk->as<double>(), (int)cv->coutp, bias, g, total_rows, (int)tiles_c, taps, keep, keep_words);
+  NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 1, 2.0 * (double)total_rows * g.Cout * g.K));
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
-                  const int32_t* /*centre_flags*/) {
+                  const int32_t* pending_cls) {
   if (cv->Kp > kMaxTaps) NNV_FAIL(NNVHIP_ERR_SHAPE, "filters with more than %d taps (FH*FW*Cin) are not supported", kMaxTaps);
   if ((cv->FH - 1) * cv->dil[0] > 0xffff || (cv->FW - 1) * cv->dil[1] > 0xffff)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "dilated filter extent too large");
   ConvGeom g;
   fill_geom(g, cv, H, W, Ho, Wo);
   const int64_t Nout = Ho * Wo * cv->Cout;
+  // a pending row reset of the input is applied on load, from one bit per input row
+  const int64_t n_in = H * W * cv->Cin;
+  const uint32_t* keep = nullptr;
+  int keep_words = 0;
+  BufRef bits;
+  if (pending_cls != nullptr) {
+    if (!conv2d_can_mask(cv, H, W, Ho, Wo, ldin)) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: row mask too large for the convolution kernel");
+    keep_words = (int)ceil_div(n_in, 32);
+    NNV_TRY(ctx->alloc(sizeof(uint32_t) * (size_t)keep_words, &bits));
+    // whole waves only, so that every word is written by a lane that exists
+    hipLaunchKernelGGL(keep_bits_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, ctx->stream, pending_cls, n_in,
+                       bits->as<uint32_t>(), keep_words);
+    NNV_HIP_TRY(hipGetLastError());
+    keep = bits->as<uint32_t>();
+  }
   // 128 positions x Cout tile, eight waves per block (two per SIMD keep the MFMA pipe fed while
   // the other wave gathers)
   int st;
-  if (cv->Cout <= 16)
-    st = launch_conv_cfg<128, 16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols);
-  else if (cv->Cout <= 32)
-    st = launch_conv_cfg<128, 32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
-  else
-    st = launch_conv_cfg<128, 64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols);
+  if (conv_fast_ok(cv, g, ldin)) {
+    if (cv->Cout <= 16)
+      st = launch_conv_fast<16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+    else if (cv->Cout <= 32)
+      st = launch_conv_fast<32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+    else
+      st = launch_conv_fast<64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+  } else if (cv->Cout <= 16) {
+    st = launch_conv_cfg<128, 16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+  } else if (cv->Cout <= 32) {
+    st = launch_conv_cfg<128, 32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+  } else {
+    st = launch_conv_cfg<128, 64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+  }
   NNV_TRY(st);
   if (ldout != Nout) {  // keep the padding rows of the output at zero
     hipLaunchKernelGGL(zero_pad_rows_kernel, dim3(256), dim3(256), 0, ctx->stream, out, ldout, Nout, ncols);

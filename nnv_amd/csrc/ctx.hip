@@ -45,6 +45,7 @@ const TuneKnobs& tune_knobs() {
     k.ranges_blocks = num("NNVHIP_RANGES_BLOCKS");
     k.apply_row_waves = num("NNVHIP_APPLY_ROW_WAVES");
     k.apply_blocks = num("NNVHIP_APPLY_BLOCKS");
+    k.conv_general = num("NNVHIP_CONV_GENERAL");
     return k;
   }();
   return knobs;
@@ -263,6 +264,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->eager_cols = getenv("NNVHIP_EAGER_COLS") != nullptr;
   c->poison_pending = getenv("NNVHIP_POISON_PENDING") != nullptr;
   c->small_chain = getenv("NNVHIP_NO_SMALL_CHAIN") == nullptr;
+  c->no_conv_mask = getenv("NNVHIP_NO_CONV_MASK") != nullptr;
   if (const char* e = getenv("NNVHIP_WEIGHT_CACHE_MB")) c->weight_cache_budget = (int64_t)atoll(e) << 20;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
@@ -1078,6 +1080,7 @@ int nnvhip_conv2d_create(nnvhip_ctx* c, const double* W, const double* bias, int
     NNV_TRY(c->alloc(sizeof(double) * Cout, &cv->bias));
     NNV_HIP_TRY(hipMemcpyAsync(cv->bias->ptr, bias, sizeof(double) * Cout, hipMemcpyHostToDevice, c->stream));
   }
+  NNV_TRY(conv2d_prepare_weights(c, cv.get()));
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   const int64_t wbytes = (int64_t)sizeof(double) * (cv->K * Cout + (bias ? Cout : 0));
   c->weight_uploads++;
@@ -1089,7 +1092,7 @@ int nnvhip_conv2d_create(nnvhip_ctx* c, const double* W, const double* bias, int
     (*out)->refs.fetch_add(1);  // the cache's reference
     WeightEntry e;
     e.handle = *out;
-    e.bytes = (int64_t)sizeof(double) * ((*out)->Kp + 1) * Cout;
+    e.bytes = (int64_t)sizeof(double) * (((*out)->Kp + 1) * Cout + ((*out)->Wk ? (*out)->Kp * (*out)->coutp : 0));
     e.last_use = ++c->weight_clock;
     c->weight_cache[key] = e;
     c->weight_cache_bytes += e.bytes;
@@ -1728,18 +1731,22 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
   // generator images that are scaled unit vectors (box ImageStars, columns appended by a ReLU) turn
   // into stamps of the filter; the implicit GEMM runs over the leading dense images only
   std::vector<ConvStampSet> stamps((size_t)count);
+  auto mask_on_load = [&](const nnvhip_star* s) {
+    return !c->no_conv_mask && s->cls != nullptr && conv2d_can_mask(cv, H, W, Ho, Wo, s->ld);
+  };
   bool any_stamps = false;
   int64_t max_m = 0;
   {
     // the implicit GEMM reads whole images: pending row resets are run first, and sets whose unit-vector
     // columns take part in the contraction get those written out
+    // (a pending reset alone is applied by the kernel as it loads, from one bit per row, where that fits)
     std::vector<nnvhip_star*> full, prefix;
     for (int64_t i = 0; i < count; ++i) {
       const int64_t nc = in[i]->n + 1;
       const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
       if (dense > in[i]->stored_cols())
         full.push_back(in[i]);
-      else if (in[i]->rows_pending || in[i]->cs.any_pending())
+      else if (in[i]->cs.any_pending() || (in[i]->rows_pending && !mask_on_load(in[i])))
         prefix.push_back(in[i]);
     }
     if (st == NNVHIP_OK && !full.empty()) st = ensure_dense_batch(c, (int64_t)full.size(), full.data());
@@ -1758,7 +1765,8 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
     stamps[i].pad_ = 0;
     any_stamps = any_stamps || dense < nc;
     max_m = std::max<int64_t>(max_m, nc - dense);
-    st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, dense, nullptr);
+    st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, dense,
+                       in[i]->rows_pending ? in[i]->cls : nullptr);
   }
   if (st == NNVHIP_OK && any_stamps) {
     // the stamp pass also leaves the range sums of its columns on the output handles

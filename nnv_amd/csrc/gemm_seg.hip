@@ -16,6 +16,7 @@
 #include <cstdlib>
 
 #include "internal.h"
+#include "lds_dma.h"
 #include "mfma_tile.h"
 
 namespace nnvhip {
@@ -28,28 +29,6 @@ constexpr int kSegTM = 128;  // rows of a tile
 constexpr int kSegKS = 8;    // rows of W / of the packed matrix per pipeline stage
 constexpr int kSegS = 4;     // stages in LDS
 constexpr int kSegNT = 512;  // threads per block
-
-#pragma clang diagnostic ignored "-Winline-asm"
-// 64 lanes x 16 bytes from global memory straight into LDS: lane l's 16 bytes at gbase + voff land at
-// lds_addr + 16 * l.  The compiler does not see the LDS write; the caller orders readers behind it with
-// wait_vm + block_barrier.  (m0 carries the LDS address of the transfer.)
-__device__ __forceinline__ void lds_dma16(const double* gbase, unsigned voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(gbase)
-               : "memory", "m0");
-}
-__device__ __forceinline__ unsigned lds_addr_of(const void* p) {
-  return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
-}
-__device__ __forceinline__ void block_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-template <int N>
-__device__ __forceinline__ void wait_vm() {
-  // vmcnt <= N and nothing else (gfx9 encoding: vmcnt in bits [3:0] and [15:14], expcnt [6:4], lgkmcnt [11:8])
-  __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8));
-}
 
 // TN columns per tile; WR x WC waves, each owning (16*FM) rows x (16*FN) columns.
 template <int TN, int WR, int WC, int FM, int FN>

@@ -78,11 +78,13 @@ inline void mailbox_unpack(unsigned long long w, int* m, int* inactive, int* seq
 
 // Tuning knobs for experiments, read from the environment once per process (0 / empty: not set):
 // NNVHIP_GEMM_XR, NNVHIP_GEMM_KSPLIT, NNVHIP_GEMM_TILE ("TMxTN"), NNVHIP_RANGES_ROW_WAVES,
-// NNVHIP_RANGES_BLOCKS, NNVHIP_APPLY_ROW_WAVES, NNVHIP_APPLY_BLOCKS.
+// NNVHIP_RANGES_BLOCKS, NNVHIP_APPLY_ROW_WAVES, NNVHIP_APPLY_BLOCKS, NNVHIP_CONV_GENERAL (1: every convolution
+// on the general kernel).
 struct TuneKnobs {
   int gemm_xr = 0, gemm_ksplit = 0;
   std::string gemm_tile;
   int ranges_row_waves = 0, ranges_blocks = 0, apply_row_waves = 0, apply_blocks = 0;
+  int conv_general = 0;
 };
 const TuneKnobs& tune_knobs();
 
@@ -210,6 +212,9 @@ struct nnvhip_ctx {
   // small fully connected networks are reached in one launch (chain.hip); environment NNVHIP_NO_SMALL_CHAIN
   // or nnvhip_set_small_chain(ctx, 0) keeps them on the layer-by-layer path
   bool small_chain = true;
+  // a convolution whose input has a pending row reset runs that reset first instead of masking the rows as
+  // it loads them (environment NNVHIP_NO_CONV_MASK)
+  bool no_conv_mask = false;
   // debugging aid (environment NNVHIP_POISON_PENDING): columns left unwritten are filled with NaNs
   bool poison_pending = false;
   // per-layer timing
@@ -348,6 +353,16 @@ struct nnvhip_conv2d {
   int64_t K = 0, Kp = 0;  // K = FH*FW*Cin taps, Kp = padded
   nnvhip::BufRef W;       // Kp x Cout, zero padded rows, ld = Kp (MATLAB layout is already K x Cout)
   nnvhip::BufRef bias;    // Cout entries or null
+  // the same weights k-major for the kernel that brings its weight tiles straight into LDS: Kp rows of
+  // coutp channels (Cout padded with zeros to a multiple of 64); null if the layer is too large for it
+  nnvhip::BufRef Wk;
+  int64_t coutp = 0;
+  // tap tables of that kernel, one per input size the layer has seen (they depend on H and W)
+  struct TapTable {
+    int64_t H = 0, W = 0;
+    nnvhip::BufRef tab;
+  };
+  mutable std::vector<TapTable> tap_tables;
 };
 
 namespace nnvhip {
@@ -468,7 +483,10 @@ int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t
 // conv.hip
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
-                  const int32_t* centre_flags /* per column: 1 = add bias */);
+                  const int32_t* pending_cls /* per input row, or null: rows whose class is not kKeep read as zero */);
+// whether launch_conv2d takes pending_cls for such an input (H x W x Cin images, leading dimension ldin)
+bool conv2d_can_mask(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin);
+int conv2d_prepare_weights(nnvhip_ctx* ctx, nnvhip_conv2d* conv);  // builds conv->Wk from conv->W (at creation)
 
 // Convolution of the one-hot generator columns of every set ("stamps" of the filter), conv.hip.
 struct ConvStampSet {

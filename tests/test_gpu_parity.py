@@ -102,7 +102,8 @@ def test_affine_fc(nnv, oracle, M, K, n):
 @pytest.mark.parametrize("H,W,Cin,Cout,FH,FW,s,p,dil,n", [
     (5, 5, 1, 1, 3, 3, 1, 0, 1, 1), (7, 6, 3, 4, 3, 3, 1, 1, 1, 9), (9, 9, 2, 5, 3, 3, 2, 0, 1, 30),
     (8, 10, 1, 2, 3, 2, 2, 1, 1, 17), (11, 9, 2, 3, 3, 3, 1, 2, 2, 5), (28, 28, 1, 16, 3, 3, 1, 1, 1, 40),
-    (14, 14, 16, 32, 3, 3, 2, 1, 1, 33), (15, 15, 32, 64, 3, 3, 1, 1, 1, 20), (12, 12, 40, 70, 5, 5, 2, 2, 1, 7)])
+    (14, 14, 16, 32, 3, 3, 2, 1, 1, 33), (15, 15, 32, 64, 3, 3, 1, 1, 1, 20), (12, 12, 40, 70, 5, 5, 2, 2, 1, 7),
+    (13, 12, 2, 5, 6, 6, 1, 2, 1, 4), (20, 20, 3, 40, 7, 5, 2, 3, 2, 6)])   # more than 32 spatial taps: the general kernel
 def test_affine_conv2d(nnv, oracle, H, W, Cin, Cout, FH, FW, s, p, dil, n):
     rs = np.random.RandomState(H * 31 + Cout)
     V = rs.randn(H, W, Cin, n + 1)
@@ -648,3 +649,71 @@ def test_outer_zonotope_follows_the_reference(nnv, oracle):
     # sets built from matrices and Stars taken from an ImageStar have none
     assert nnv.Star(rs.randn(3, 3), np.zeros((1, 2)), np.zeros(1), [-1, -1], [1, 1]).Z is None
     assert nnv.ImageStar(np.zeros((2, 2, 1)), np.ones((2, 2, 1))).toStar().Z is None
+
+
+def _relu_then_conv(nnv, oracle, rs, H, W, Cin, Cout, FH, FW, s, p, dil, n, count=1, spread=2.0):
+    """ReLU step on ImageStars with rows of all three kinds, then a convolution; returns (device sets, oracle
+    sets, launches of the apply pass while the convolution ran)."""
+    ctx = nnv.default_context()
+    Wt = rs.randn(FH, FW, Cin, Cout)
+    b = rs.randn(Cout)
+    dev_in, ora_in = [], []
+    for _ in range(count):
+        V = rs.randn(H, W, Cin, n + 1) * 0.3
+        V[..., 0] = rs.randn(H, W, Cin) * spread          # centres spread so that many rows are clearly on or off
+        lb, ub = -np.ones(n), np.ones(n)
+        dev_in.append(nnv.ImageStar(V, np.zeros((1, n)), np.zeros(1), lb, ub))
+        ora_in.append(oracle.OImageStar(V, np.zeros((1, n)), np.zeros(1), lb, ub))
+    relu = nnv.ReluLayer()
+    conv = nnv.Conv2DLayer(Wt, b, [p, p, p, p], [s, s], [dil, dil])
+    mid = relu.reach(dev_in if count > 1 else dev_in[0], "relax-star-area", "single", 1)
+    ctx.kernel_time(3)
+    ctx.set_timing(2)
+    try:
+        out = conv.reach(mid, "relax-star-area", "single")
+    finally:
+        ctx.set_timing(0)
+    applies = ctx.kernel_time(3)[1]
+    exp_mid = [oracle.relu_layer_reach(o, "relax-star-area", 1.0) for o in ora_in]
+    exp = [oracle.conv2d_reach(o, Wt, b, [p, p, p, p], [s, s], [dil, dil]) for o in exp_mid]
+    return (list(out) if count > 1 else [out]), exp, applies, list(zip(list(mid) if count > 1 else [mid], exp_mid))
+
+
+@pytest.mark.parametrize("H,W,Cin,Cout,FH,FW,s,p,dil,n,count", [
+    (5, 5, 1, 1, 3, 3, 1, 0, 1, 2, 1), (7, 9, 3, 4, 3, 3, 1, 1, 1, 6, 1), (9, 7, 5, 20, 3, 3, 2, 0, 1, 11, 3),
+    (11, 9, 2, 3, 3, 3, 1, 2, 2, 5, 1), (15, 15, 32, 64, 3, 3, 1, 1, 1, 20, 1), (13, 13, 7, 40, 5, 5, 2, 2, 1, 9, 2),
+    (13, 12, 2, 5, 6, 6, 1, 2, 1, 4, 2)])   # the last one has more than 32 spatial taps: the general kernel
+def test_conv_reads_through_a_pending_row_reset(nnv, oracle, H, W, Cin, Cout, FH, FW, s, p, dil, n, count):
+    """The convolution after a ReLU step zeroes the reset rows as it loads them (Star.m:1442-1461 applied at
+    the reader): same sets as the oracle's, no apply pass, and the ReLU's own output still reads correctly."""
+    import os
+    rs = np.random.RandomState(H * 100 + Cout)
+    out, exp, applies, mid = _relu_then_conv(nnv, oracle, rs, H, W, Cin, Cout, FH, FW, s, p, dil, n, count)
+    switched = any(os.environ.get(k) for k in ("NNVHIP_NO_CONV_MASK", "NNVHIP_EAGER_ROWS", "NNVHIP_EAGER_TAIL",
+                                               "NNVHIP_DENSE_AFFINE"))
+    if not switched:
+        assert applies == 0
+    for R, E in zip(out, exp):
+        assert R.V.shape == E.V.shape
+        compare_sets(R, E, "conv after ReLU")
+    # the ReLU output, read afterwards, has its rows reset (first read runs the pass)
+    for M, EM in mid:
+        compare_sets(M, EM, "the ReLU output itself", True)
+
+
+def test_conv_after_relu_on_an_image_too_large_for_the_row_mask(nnv, oracle):
+    """135168 input rows and a 64-channel tile: the bit mask does not fit beside the operand tiles, the reset is
+    run first."""
+    import os
+    rs = np.random.RandomState(8)
+    out, exp, applies, _ = _relu_then_conv(nnv, oracle, rs, 64, 64, 33, 40, 3, 3, 2, 1, 1, 2, spread=100.0)
+    if not os.environ.get("NNVHIP_EAGER_ROWS") and not os.environ.get("NNVHIP_EAGER_TAIL") and not os.environ.get("NNVHIP_DENSE_AFFINE"):
+        assert applies == 1
+    compare_sets(out[0], exp[0], "conv after ReLU, large image")
+
+
+def test_filters_with_too_many_taps_are_refused(nnv):
+    rs = np.random.RandomState(1)
+    I = nnv.ImageStar(np.zeros((9, 9, 32, 2)), np.zeros((1, 1)), np.zeros(1), [-1.0], [1.0])
+    with pytest.raises(ValueError, match="taps"):
+        nnv.Conv2DLayer(rs.randn(8, 8, 32, 64), np.zeros(64)).reach(I, "relax-star-area")
