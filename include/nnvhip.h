@@ -162,7 +162,9 @@ NNVHIP_API int nnvhip_star_retain(nnvhip_star* s);
 NNVHIP_API int nnvhip_star_release(nnvhip_star* s);
 /* Releases one reference of each of `count` handles (null entries are skipped): what clearing an
  * object array of sets does in the reference, e.g. when NN.reach overwrites the per-layer outputs
- * it keeps in reachSet (nn/NN.m:1531, 1547). */
+ * it keeps in reachSet (nn/NN.m:1531, 1547).  The handles are invalid once the call returns; for arrays of
+ * 256 handles and more the library may give their device memory back to its pool later (during its next
+ * wait for the device, or as soon as the pool needs a block). */
 NNVHIP_API int nnvhip_star_release_array(int64_t count, nnvhip_star* const* sets);
 /* dim, nVar and the number of constraint rows size(C,1). */
 NNVHIP_API int nnvhip_star_dims(const nnvhip_star* s, int64_t* N, int64_t* n, int64_t* p);

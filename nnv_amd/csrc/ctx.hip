@@ -94,10 +94,26 @@ nnvhip_star* new_star(nnvhip_ctx* ctx) {
 
 using namespace nnvhip;
 
+void nnvhip_ctx::drain_deferred(size_t at_most) {
+  while (!deferred.empty() && at_most-- > 0) {
+    nnvhip_star* s = deferred.back();
+    deferred.pop_back();
+    nnvhip_star_release(s);
+  }
+}
+
 int nnvhip_ctx::alloc(size_t bytes, BufRef* out) {
   size_t cls = size_class(bytes ? bytes : 1);
   void* p = nullptr;
   auto it = free_blocks.find(cls);
+  // A released array that has not been let go yet may hold such a block.  While the pool is small next to the
+  // device's memory it grows instead (a loop of reaches then alternates between two generations of blocks and
+  // never waits for the handles of the previous one); past that share the array is let go now.
+  if (it == free_blocks.end() && !deferred.empty() &&
+      (double)(bytes_in_use + bytes_cached) + (double)cls > 0.4 * (double)device_bytes) {
+    drain_deferred();
+    it = free_blocks.find(cls);
+  }
   if (it != free_blocks.end()) {
     p = it->second;
     free_blocks.erase(it);
@@ -106,7 +122,7 @@ int nnvhip_ctx::alloc(size_t bytes, BufRef* out) {
     hipError_t e = hipMalloc(&p, cls);
     if (e != hipSuccess) {
       (void)hipGetLastError();
-      trim();  // give cached blocks back and retry once
+      trim();  // let released arrays go, give cached blocks back and retry once
       e = hipMalloc(&p, cls);
       if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -133,6 +149,7 @@ void nnvhip_ctx::release_block(void* p, size_t bytes) {
 
 int nnvhip_ctx::trim() {
   if (stream) (void)hipStreamSynchronize(stream);
+  drain_deferred();
   for (auto& kv : free_blocks) (void)hipFree(kv.second);
   free_blocks.clear();
   bytes_cached = 0;
@@ -258,6 +275,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
     NNV_FAIL(NNVHIP_ERR_ARG, "libnnvhip is built for gfx950 (MI355X); device %d is %s", device, prop.gcnArchName);
   nnvhip_ctx* c = new nnvhip_ctx();
   c->device = device;
+  c->device_bytes = (int64_t)prop.totalGlobalMem;
   c->dense_affine = getenv("NNVHIP_DENSE_AFFINE") != nullptr;
   c->eager_tail = getenv("NNVHIP_EAGER_TAIL") != nullptr;
   c->eager_rows = getenv("NNVHIP_EAGER_ROWS") != nullptr;
@@ -281,6 +299,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
 int nnvhip_destroy(nnvhip_ctx* c) {
   if (!c) return NNVHIP_OK;
   c->drop_weight_cache(true);
+  c->drain_deferred();
   if (c->live_handles != 0)
     NNV_FAIL(NNVHIP_ERR_ARG, "context still has %lld live handles", (long long)c->live_handles);
   NNV_TRY(nnvhip::enter_ctx(c));
@@ -299,7 +318,11 @@ int nnvhip_destroy(nnvhip_ctx* c) {
 
 int nnvhip_synchronize(nnvhip_ctx* c) {
   CHECK_CTX(c);
+  // released arrays are let go while the device works; whatever is left, once it is done
+  while (!c->deferred.empty() && hipStreamQuery(c->stream) == hipErrorNotReady) c->drain_deferred(64);
+  (void)hipGetLastError();
   NNV_HIP_TRY(hipStreamSynchronize(c->stream));
+  c->drain_deferred();
   return NNVHIP_OK;
 }
 
@@ -459,6 +482,7 @@ int nnvhip_upload_stats(nnvhip_ctx* c, int64_t* weight_uploads, int64_t* weight_
 
 int nnvhip_pool_stats(nnvhip_ctx* c, int64_t* in_use, int64_t* cached) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  c->drain_deferred();
   if (in_use) *in_use = c->bytes_in_use;
   if (cached) *cached = c->bytes_cached;
   return NNVHIP_OK;
@@ -789,7 +813,14 @@ int nnvhip_star_release(nnvhip_star* s) {
 
 int nnvhip_star_release_array(int64_t count, nnvhip_star* const* sets) {
   if (count < 0 || (count > 0 && !sets)) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
-  for (int64_t i = 0; i < count; ++i) nnvhip_star_release(sets[i]);
+  // a large array is let go later, where the host waits for the device anyway (nnvhip_ctx::deferred)
+  const bool later = count >= 256;
+  for (int64_t i = 0; i < count; ++i) {
+    if (later && sets[i] != nullptr)
+      sets[i]->ctx->deferred.push_back(sets[i]);
+    else
+      nnvhip_star_release(sets[i]);
+  }
   return NNVHIP_OK;
 }
 

@@ -173,6 +173,13 @@ struct nnvhip_ctx {
   int64_t bytes_in_use = 0;
   int64_t bytes_cached = 0;
   int64_t live_handles = 0;
+  // Handles of large arrays that the caller has released but that have not been let go yet: destroying
+  // thousands of handles costs hundreds of microseconds of host time, which is spent where the host waits
+  // for the device anyway (the ReLU step's wait for its counts, a synchronisation) or when the pool runs
+  // short of a block; pool_stats, trim and destroy let them go first.
+  std::vector<nnvhip_star*> deferred;
+  void drain_deferred(size_t at_most = ~size_t(0));
+  int64_t device_bytes = 0;  // memory of the device (the pool grows past a released array only below a share of it)
   // pinned staging ring for descriptor tables and small read-backs
   char* pinned = nullptr;
   std::vector<char*> retired_rings;

@@ -722,6 +722,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     for (int64_t i = 0; i < count; ++i) {
       unsigned long long w = box[i];
       while (w == kMailboxEmpty) {
+        if (!ctx->deferred.empty()) ctx->drain_deferred(16);  // something useful to do while the device works
         if ((++spins & 0xfff) == 0 &&
             std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() > 10.0) {
           NNV_HIP_TRY(hipStreamSynchronize(ctx->stream));  // surfaces a launch failure, if any
