@@ -152,6 +152,15 @@ __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __re
     // as possible are in flight at once; the additions stay in chunk order
     const double* p = d.part + (int64_t)q * d.ld + r;
     int c = 0;
+    if (d.chunks <= 8) {  // the common case after a fused GEMM epilogue: one short batch
+      double v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = u < d.chunks ? p[(int64_t)u * 4 * d.ld] : 0.0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (u < d.chunks) s += v[u];
+      c = d.chunks;
+    }
     for (; c + 32 <= d.chunks; c += 32) {
       double v[32];
 #pragma unroll
@@ -159,7 +168,7 @@ __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __re
 #pragma unroll
       for (int u = 0; u < 32; ++u) s += v[u];
     }
-    {
+    if (c < d.chunks) {
       double v[32];
 #pragma unroll
       for (int u = 0; u < 32; ++u) v[u] = c + u < d.chunks ? p[(int64_t)(c + u) * 4 * d.ld] : 0.0;

@@ -717,3 +717,39 @@ def test_filters_with_too_many_taps_are_refused(nnv):
     I = nnv.ImageStar(np.zeros((9, 9, 32, 2)), np.zeros((1, 1)), np.zeros(1), [-1.0], [1.0])
     with pytest.raises(ValueError, match="taps"):
         nnv.Conv2DLayer(rs.randn(8, 8, 32, 64), np.zeros(64)).reach(I, "relax-star-area")
+
+
+def test_released_arrays_give_their_memory_back(nnv):
+    """Arrays of 256 sets and more are let go lazily (while the library waits for the device); the pool's figures,
+    a later reach and an element that was read out of the array before behave as if they had gone at once."""
+    ctx = nnv.default_context()
+    rs = np.random.RandomState(5)
+    n_in, hidden, count = 6, 40, 700
+    net = nnv.NN([nnv.FullyConnectedLayer(rs.randn(hidden, n_in), rs.randn(hidden)), nnv.ReluLayer(),
+                  nnv.FullyConnectedLayer(rs.randn(5, hidden), rs.randn(5))])
+    opt = {"reachMethod": "relax-star-area", "relaxFactor": 1}
+    lbs = rs.rand(n_in, count) - 0.5
+    ubs = lbs + 0.2
+    net.reach(nnv.Star.from_boxes(lbs[:, :2], ubs[:, :2]), opt)   # the layers' weights are on the device now
+    net.reachSet = []
+    ctx.synchronize()
+    used0, _ = ctx.pool_stats()
+    ins = nnv.Star.from_boxes(lbs, ubs)
+    outs = net.reach(ins, opt)
+    kept = outs[3]                       # an element read out of the array owns its handle
+    lb_kept, ub_kept = kept.estimateRanges()
+    used1, _ = ctx.pool_stats()
+    assert used1 > used0
+    del outs, ins
+    net.reachSet = []
+    used2, _ = ctx.pool_stats()
+    assert used0 < used2 < used1         # everything but what `kept` holds on to is back in the pool
+    # a second reach runs while the first one's arrays may still be queued for release, with the same result
+    outs2 = net.reach(nnv.Star.from_boxes(lbs, ubs), opt)
+    lb2, ub2 = outs2[3].estimateRanges()
+    assert np.array_equal(lb2, lb_kept) and np.array_equal(ub2, ub_kept)
+    assert np.array_equal(np.asarray(kept.V), np.asarray(outs2[3].V))
+    del outs2, kept
+    net.reachSet = []
+    ctx.synchronize()
+    assert ctx.pool_stats()[0] == used0
