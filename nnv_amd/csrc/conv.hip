@@ -42,20 +42,60 @@ __device__ __forceinline__ unsigned long long pack_tap(const ConvGeom& g, int k)
          (unsigned long long)(fw * g.dw);
 }
 
-// Stores a block's accumulators: lane l, register r of acc[i][j] holds out[position R0 + ... + l%16][channel c0 +
+// How the rows of the implicit GEMM map to (image, output position).  box == null: row R is position R % P of
+// image R / P.  Otherwise rows [0, P) are the centre image and every further image owns `area` = eh x ew rows,
+// the positions of its window's corner onwards (row t of the slot: ho = h0 + t % eh, wo = w0 + t / eh; slots of
+// positions outside the window are idle): a generator image is computed inside its window only.
+struct ConvRows {
+  const ColBox* box;
+  int eh, area;
+};
+
+template <bool COMPACT>
+__device__ __forceinline__ bool conv_row(const ConvGeom& g, const ConvRows& cr, int64_t R, int64_t total_rows, int64_t* gi,
+                                         int* ho, int* wo) {
+  if (R >= total_rows) return false;
+  if (!COMPACT || R < g.P) {
+    const int64_t im = COMPACT ? 0 : R / g.P;
+    const int p = (int)(R - im * g.P);
+    *gi = im;
+    *wo = p / g.Ho;
+    *ho = p - *wo * g.Ho;
+    return true;
+  }
+  const int64_t q = R - g.P;
+  const int64_t im = q / cr.area;
+  const int t = (int)(q - im * cr.area);
+  const ColBox bb = cr.box[1 + im];
+  *gi = 1 + im;
+  const int tw = t / cr.eh;
+  *ho = bb.h0 + (t - tw * cr.eh);
+  *wo = bb.w0 + tw;
+  return *ho <= bb.h1 && *wo <= bb.w1;
+}
+
+template <bool COMPACT>
+__device__ __forceinline__ int64_t conv_first_image(const ConvGeom& g, const ConvRows& cr, int64_t R0) {
+  if (!COMPACT) return R0 / g.P;
+  return R0 < g.P ? 0 : 1 + (R0 - g.P) / cr.area;
+}
+
+// Stores a block's accumulators: lane l, register r of acc[i][j] holds out[row R0 + ... + l%16][channel c0 +
 // ... + l/16 + 4r]; the bias goes onto the centre image only.
-template <int TP, int TC, int WR, int WC, int FM, int FN>
+template <int TP, int TC, int WR, int WC, int FM, int FN, bool COMPACT = false>
 __device__ __forceinline__ void conv_store_tile(const double4_t (&acc)[FM][FN], double* __restrict__ out, int64_t ldout,
                                                 const double* __restrict__ bias, const ConvGeom& g, int64_t total_rows,
-                                                int64_t R0, int c0, int wr, int wc, int lane) {
+                                                int64_t R0, int c0, int wr, int wc, int lane,
+                                                const ConvRows cr = ConvRows{nullptr, 0, 0}) {
   const int lrow = lane & 15;
   const int lcol = lane >> 4;
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
     const int64_t Rr = R0 + wr * (TP / WR) + i * 16 + lrow;
-    if (Rr >= total_rows) continue;
-    const int64_t gi = Rr / g.P;
-    const int p = (int)(Rr - gi * g.P);
+    int64_t gi;
+    int ho, wo;
+    if (!conv_row<COMPACT>(g, cr, Rr, total_rows, &gi, &ho, &wo)) continue;
+    const int p = ho + wo * g.Ho;
     double* o = out + gi * ldout + p;
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
@@ -226,12 +266,12 @@ __global__ void conv_weights_kmajor_kernel(const double* __restrict__ W, double*
   Wk[idx] = co < Cout ? W[k + (int64_t)co * Kp] : 0.0;
 }
 
-template <int TC, int WR, int WC, bool MASK>
+template <int TC, int WR, int WC, bool MASK, bool COMPACT>
 __global__ __launch_bounds__(512) void conv2d_fast_kernel(const double* __restrict__ in, int64_t ldin, double* __restrict__ out,
                                                           int64_t ldout, const double* __restrict__ Wk, int coutp,
                                                           const double* __restrict__ bias, ConvGeom g, int64_t total_rows,
                                                           int tiles_c, const FastTap* __restrict__ taps,
-                                                          const uint32_t* __restrict__ keep, int keep_words) {
+                                                          const uint32_t* __restrict__ keep, int keep_words, ConvRows cr) {
   constexpr int TP = 128, NT = 512;
   static_assert(WR * WC == 8, "eight waves");
   constexpr int FM = TP / WR / 16;
@@ -258,17 +298,14 @@ __global__ __launch_bounds__(512) void conv2d_fast_kernel(const double* __restri
   const int p_local = tid & (TP - 1);
   const int kq = __builtin_amdgcn_readfirstlane(tid >> 7);
   const int64_t R = R0 + p_local;
-  const bool rvalid = R < total_rows;
-  const int64_t gi0 = R0 / g.P;
+  const int64_t gi0 = conv_first_image<COMPACT>(g, cr, R0);
   const char* const base = reinterpret_cast<const char*>(in + gi0 * ldin);  // block-uniform
   uint32_t toff = 0;
   int base_row = 0;
   uint32_t vmask = 0;
-  if (rvalid) {
-    const int64_t gi = R / g.P;
-    const int p = (int)(R - gi * g.P);
-    const int wo = p / g.Ho;
-    const int ho = p - wo * g.Ho;
+  int64_t gi = 0;
+  int ho = 0, wo = 0;
+  if (conv_row<COMPACT>(g, cr, R, total_rows, &gi, &ho, &wo)) {
     const int h0 = ho * g.sh - g.pt;
     const int w0 = wo * g.sw - g.pl;
     toff = (uint32_t)((gi - gi0) * ldin * 8);
@@ -366,7 +403,36 @@ __global__ __launch_bounds__(512) void conv2d_fast_kernel(const double* __restri
     step(kt, std::integral_constant<int, 0>());
     if (kt + 1 < nk) step(kt + 1, std::integral_constant<int, 1>());
   }
-  conv_store_tile<TP, TC, WR, WC, FM, FN>(acc, out, ldout, bias, g, total_rows, R0, c0, wr, wc, lane);
+  conv_store_tile<TP, TC, WR, WC, FM, FN, COMPACT>(acc, out, ldout, bias, g, total_rows, R0, c0, wr, wc, lane, cr);
+}
+
+// Windows of the output columns of a convolution (see launch_conv_boxes in internal.h).
+__global__ void conv_boxes_kernel(const ColBox* __restrict__ in_box, int64_t dense, const int32_t* __restrict__ onehot_idx,
+                                  int64_t m, ColBox* __restrict__ out_box, ConvGeom g) {
+  const int64_t j = blockIdx.x * (int64_t)256 + threadIdx.x;
+  if (j >= dense + m) return;
+  int h0 = 0, h1 = g.H - 1, w0 = 0, w1 = g.W - 1;  // window of the input column
+  if (j >= dense) {
+    const int src = onehot_idx[j - dense] % g.HW;
+    w0 = w1 = src / g.H;
+    h0 = h1 = src - w0 * g.H;
+  } else if (j > 0 && in_box != nullptr) {
+    const ColBox b = in_box[j];
+    h0 = b.h0, h1 = b.h1, w0 = b.w0, w1 = b.w1;
+  }
+  ColBox o;
+  if (h0 > h1 || w0 > w1) {
+    o = ColBox{1, 0, 1, 0};
+  } else {
+    // output rows whose taps ho*sh - pt + fh*dh (0 <= fh < FH) reach [h0, h1]
+    auto floordiv = [](int a, int s) { return a >= 0 ? a / s : -((-a + s - 1) / s); };
+    const int a0 = h0 + g.pt - (g.FH - 1) * g.dh, a1 = h1 + g.pt;
+    const int b0 = w0 + g.pl - (g.FW - 1) * g.dw, b1 = w1 + g.pl;
+    const int ho0 = max(0, -floordiv(-a0, g.sh)), ho1 = min(g.Ho - 1, floordiv(a1, g.sh));
+    const int wo0 = max(0, -floordiv(-b0, g.sw)), wo1 = min(g.Wo - 1, floordiv(b1, g.sw));
+    o = (ho0 > ho1 || wo0 > wo1) ? ColBox{1, 0, 1, 0} : ColBox{(int16_t)ho0, (int16_t)ho1, (int16_t)wo0, (int16_t)wo1};
+  }
+  out_box[j] = o;
 }
 
 __global__ void zero_pad_rows_kernel(double* __restrict__ V, int64_t ld, int64_t N, int64_t ncols) {
@@ -553,11 +619,11 @@ static int conv_tile_channels(const nnvhip_conv2d* cv) { return cv->Cout <= 16 ?
 
 // The kernel with scalar tap decoding: at most 32 spatial taps (one mask bit each), every byte offset it forms
 // (a row of the image plus the images a 128-position tile can span) below 2^31.
-static bool conv_fast_ok(const nnvhip_conv2d* cv, const ConvGeom& g, int64_t ldin) {
+static bool conv_fast_ok(const nnvhip_conv2d* cv, const ConvGeom& g, int64_t ldin, int64_t rows_per_image = 0) {
   if (tune_knobs().conv_general != 0 || cv->Wk == nullptr) return false;
   if (cv->FH * cv->FW > 32) return false;
   const int64_t n_in = (int64_t)g.HW * g.Cin;
-  const int64_t images_per_tile = 127 / g.P + 2;
+  const int64_t images_per_tile = 127 / (rows_per_image > 0 ? rows_per_image : g.P) + 2;
   return (n_in + images_per_tile * ldin) * 8 < (int64_t(1) << 31);
 }
 
@@ -602,8 +668,9 @@ static int conv_fast_taps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGe
 
 template <int TC, int WR, int WC>
 static int launch_conv_fast(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGeom& g, const double* in, int64_t ldin, double* out,
-                            int64_t ldout, int64_t ncols, const uint32_t* keep, int keep_words) {
-  const int64_t total_rows = (int64_t)g.P * ncols;
+                            int64_t ldout, int64_t ncols, const uint32_t* keep, int keep_words, const ConvRows& cr) {
+  const bool compact = cr.box != nullptr;
+  const int64_t total_rows = compact ? (int64_t)g.P + (ncols - 1) * cr.area : (int64_t)g.P * ncols;
   const int64_t tiles_c = ceil_div(g.Cout, TC);
   const int64_t blocks = ceil_div(total_rows, 128) * tiles_c;
   if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
@@ -613,20 +680,42 @@ static int launch_conv_fast(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const Conv
   NNV_TRY(conv_fast_taps(ctx, cv, g, &taps));
   const double* bias = cv->bias ? cv->bias->as<double>() : nullptr;
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-  if (keep)
-    NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, true>), dim3((unsigned)blocks), dim3(512), dyn, in, ldin, out,
-               ldout, cv->Wk->as<double>(), (int)cv->coutp, bias, g, total_rows, (int)tiles_c, taps, keep, keep_words);
+#define NNV_CONV_FAST(MASK, COMPACT)                                                                                              \
+  NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, MASK, COMPACT>), dim3((unsigned)blocks), dim3(512), dyn, in, \
+             ldin, out, ldout, cv->Wk->as<double>(), (int)cv->coutp, bias, g, total_rows, (int)tiles_c, taps, keep, keep_words, cr)
+  if (keep && compact)
+    NNV_CONV_FAST(true, true);
+  else if (keep)
+    NNV_CONV_FAST(true, false);
+  else if (compact)
+    NNV_CONV_FAST(false, true);
   else
-    NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, false>), dim3((unsigned)blocks), dim3(512), dyn, in, ldin, out,
-               ldout, cv->Wk->as<double>(), (int)cv->coutp, bias, g, total_rows, (int)tiles_c, taps, keep, keep_words);
+    NNV_CONV_FAST(false, false);
+#undef NNV_CONV_FAST
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 1, 2.0 * (double)total_rows * g.Cout * g.K));
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+int64_t conv_box_extent(const nnvhip_conv2d* cv, int dim, int64_t e, int64_t out_size) {
+  // output positions whose taps reach a run of e input positions: floor((e - 1 + (F - 1) * dil) / stride) + 1
+  const int64_t F = dim == 0 ? cv->FH : cv->FW;
+  return std::min<int64_t>(out_size, (e - 1 + (F - 1) * cv->dil[dim]) / cv->stride[dim] + 1);
+}
+
+int launch_conv_boxes(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                      const ColBox* in_box, int64_t dense, const int32_t* onehot_idx, int64_t m, ColBox* out_box) {
+  ConvGeom g;
+  fill_geom(g, cv, H, W, Ho, Wo);
+  hipLaunchKernelGGL(conv_boxes_kernel, dim3((unsigned)ceil_div(dense + m, 256)), dim3(256), 0, ctx->stream, in_box, dense, onehot_idx, m,
+                     out_box, g);
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }
 
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
-                  const int32_t* pending_cls) {
+                  const int32_t* pending_cls, const ColBox* out_box, int eh, int ew) {
   if (cv->Kp > kMaxTaps) NNV_FAIL(NNVHIP_ERR_SHAPE, "filters with more than %d taps (FH*FW*Cin) are not supported", kMaxTaps);
   if ((cv->FH - 1) * cv->dil[0] > 0xffff || (cv->FW - 1) * cv->dil[1] > 0xffff)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "dilated filter extent too large");
@@ -651,13 +740,20 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W
   // 128 positions x Cout tile, eight waves per block (two per SIMD keep the MFMA pipe fed while
   // the other wave gathers)
   int st;
-  if (conv_fast_ok(cv, g, ldin)) {
+  // Generator images with known windows are computed inside them only (the caller has zeroed the rest) when that
+  // at least halves the rows; it takes the kernel with scalar tap decoding.
+  ConvRows cr{nullptr, 0, 0};
+  if (out_box != nullptr && ncols > 1 && eh > 0 && ew > 0 && 2 * (int64_t)eh * ew <= g.P && conv_fast_ok(cv, g, ldin, (int64_t)eh * ew))
+    cr = ConvRows{out_box, eh, eh * ew};
+  if (cr.box != nullptr)  // everything outside the windows
+    NNV_HIP_TRY(hipMemsetAsync(out + ldout, 0, sizeof(double) * (size_t)ldout * (size_t)(ncols - 1), ctx->stream));
+  if (cr.box != nullptr || conv_fast_ok(cv, g, ldin)) {
     if (cv->Cout <= 16)
-      st = launch_conv_fast<16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+      st = launch_conv_fast<16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr);
     else if (cv->Cout <= 32)
-      st = launch_conv_fast<32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+      st = launch_conv_fast<32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr);
     else
-      st = launch_conv_fast<64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
+      st = launch_conv_fast<64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr);
   } else if (cv->Cout <= 16) {
     st = launch_conv_cfg<128, 16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
   } else if (cv->Cout <= 32) {

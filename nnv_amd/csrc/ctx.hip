@@ -283,6 +283,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->poison_pending = getenv("NNVHIP_POISON_PENDING") != nullptr;
   c->small_chain = getenv("NNVHIP_NO_SMALL_CHAIN") == nullptr;
   c->no_conv_mask = getenv("NNVHIP_NO_CONV_MASK") != nullptr;
+  c->no_conv_boxes = getenv("NNVHIP_NO_CONV_BOXES") != nullptr;
   if (const char* e = getenv("NNVHIP_WEIGHT_CACHE_MB")) c->weight_cache_budget = (int64_t)atoll(e) << 20;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
@@ -1783,9 +1784,43 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
     if (st == NNVHIP_OK && !full.empty()) st = ensure_dense_batch(c, (int64_t)full.size(), full.data());
     if (st == NNVHIP_OK && !prefix.empty()) st = ensure_dense_batch(c, (int64_t)prefix.size(), prefix.data(), false);
   }
+  // windows of the output's generator images (internal.h, nnvhip_star::box): from the input's windows and from
+  // the pixels of its unit-vector columns; without either the images count as full
+  const bool track_boxes = !c->no_conv_boxes && H < 32768 && W < 32768 && Ho < 32768 && Wo < 32768;
   for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
     const int64_t nc = in[i]->n + 1;
     const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
+    const ColBox* dense_box = nullptr;
+    int dense_eh = 0, dense_ew = 0;
+    if (track_boxes) {
+      const bool in_ok = in[i]->box != nullptr && in[i]->box_H == H && in[i]->box_W == W && in[i]->box_cols >= dense;
+      const int64_t m = nc - dense;
+      if (in_ok || (m > 0 && dense == 1)) {
+        st = c->alloc(sizeof(ColBox) * (size_t)nc, &outs[i]->box_buf);
+        if (st != NNVHIP_OK) break;
+        ColBox* ob = outs[i]->box_buf->as<ColBox>();
+        st = launch_conv_boxes(c, cv, H, W, Ho, Wo, in_ok ? in[i]->box : nullptr, dense, in[i]->oh_idx, m, ob);
+        if (st != NNVHIP_OK) break;
+        int64_t eh = 0, ew = 0;
+        if (dense > 1) {  // (only reached with in_ok)
+          dense_eh = (int)conv_box_extent(cv, 0, in[i]->box_eh, Ho);
+          dense_ew = (int)conv_box_extent(cv, 1, in[i]->box_ew, Wo);
+          dense_box = ob;
+          eh = dense_eh;
+          ew = dense_ew;
+        }
+        if (m > 0) {
+          eh = std::max(eh, conv_box_extent(cv, 0, 1, Ho));
+          ew = std::max(ew, conv_box_extent(cv, 1, 1, Wo));
+        }
+        outs[i]->box = ob;
+        outs[i]->box_cols = nc;
+        outs[i]->box_H = (int32_t)Ho;
+        outs[i]->box_W = (int32_t)Wo;
+        outs[i]->box_eh = (int32_t)eh;
+        outs[i]->box_ew = (int32_t)ew;
+      }
+    }
     stamps[i].idx = in[i]->oh_idx;
     stamps[i].scale = in[i]->oh_scale;
     stamps[i].out = outs[i]->V + dense * outs[i]->ld;
@@ -1797,7 +1832,7 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
     any_stamps = any_stamps || dense < nc;
     max_m = std::max<int64_t>(max_m, nc - dense);
     st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, dense,
-                       in[i]->rows_pending ? in[i]->cls : nullptr);
+                       in[i]->rows_pending ? in[i]->cls : nullptr, dense_box, dense_eh, dense_ew);
   }
   if (st == NNVHIP_OK && any_stamps) {
     // the stamp pass also leaves the range sums of its columns on the output handles

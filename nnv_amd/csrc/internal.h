@@ -88,6 +88,11 @@ struct TuneKnobs {
 };
 const TuneKnobs& tune_knobs();
 
+// Window of an image (rows h0..h1, columns w0..w1, inclusive) outside which a generator image is zero.
+struct ColBox {
+  int16_t h0, h1, w0, w1;
+};
+
 // Where an FC map gathered stored columns of a set from, and whether they are in memory yet.  Column
 // from + t holds 0 + W(:, r) * scale[r] with r = idx[t] (scale == null: 1).  A later packing of kept rows
 // reads the cache-resident weight matrix instead of the set's own matrix in HBM; and the FC map may leave
@@ -222,6 +227,9 @@ struct nnvhip_ctx {
   // a convolution whose input has a pending row reset runs that reset first instead of masking the rows as
   // it loads them (environment NNVHIP_NO_CONV_MASK)
   bool no_conv_mask = false;
+  // convolutions compute every generator image in full instead of inside its window (nnvhip_star::box;
+  // environment NNVHIP_NO_CONV_BOXES)
+  bool no_conv_boxes = false;
   // debugging aid (environment NNVHIP_POISON_PENDING): columns left unwritten are filled with NaNs
   bool poison_pending = false;
   // per-layer timing
@@ -340,6 +348,16 @@ struct nnvhip_star {
   bool has_zono = false;
   // where gathered columns came from, and whether they (and leading zero columns) are in memory yet
   nnvhip::ColSource cs;
+  // Spatial support of the generator images of an ImageStar that a convolution produced: stored column j
+  // (j < box_cols) is zero in every row (h, w, channel) of the box_H x box_W x C image outside the window
+  // box[j] (h0..h1, w0..w1, inclusive; h0 > h1: the whole column is zero).  Generators of a box ImageStar
+  // start as single pixels and grow by a filter's reach per convolution; a ReLU step only resets rows, so
+  // its output keeps the windows.  box_eh x box_ew bounds the window of every column but the centre's.  The
+  // next convolution computes a generator's image inside its (grown) window only.  null: no such knowledge.
+  nnvhip::BufRef box_buf;
+  const nnvhip::ColBox* box = nullptr;
+  int64_t box_cols = 0;
+  int32_t box_H = 0, box_W = 0, box_eh = 0, box_ew = 0;
 };
 
 struct nnvhip_fc {
@@ -490,7 +508,17 @@ int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t
 // conv.hip
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
-                  const int32_t* pending_cls /* per input row, or null: rows whose class is not kKeep read as zero */);
+                  const int32_t* pending_cls /* per input row, or null: rows whose class is not kKeep read as zero */,
+                  const ColBox* out_box = nullptr /* per output column, or null: with it, columns 1.. are computed inside
+                                                    their windows only (at most eh x ew positions) and must be zero
+                                                    elsewhere already */,
+                  int eh = 0, int ew = 0);
+// Windows of a convolution's output columns: column 0 the whole image; columns below `dense` from the input's
+// windows (in_box null: whole image); the `m` columns from `dense` on from the pixels onehot_idx names.
+int launch_conv_boxes(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                      const ColBox* in_box, int64_t dense, const int32_t* onehot_idx, int64_t m, ColBox* out_box);
+// Bound on the extent of an output window whose input window spans at most `e` rows (dim 0) or columns (dim 1).
+int64_t conv_box_extent(const nnvhip_conv2d* conv, int dim, int64_t e, int64_t out_size);
 // whether launch_conv2d takes pending_cls for such an input (H x W x Cin images, leading dimension ldin)
 bool conv2d_can_mask(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin);
 int conv2d_prepare_weights(nnvhip_ctx* ctx, nnvhip_conv2d* conv);  // builds conv->Wk from conv->W (at creation)

@@ -685,6 +685,17 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       // holds for the rows that are kept
       o->cs = in[i]->cs;
     }
+    {
+      // resetting rows leaves every generator image inside its window (the columns the step appends come
+      // after the ones the windows describe)
+      o->box_buf = in[i]->box_buf;
+      o->box = in[i]->box;
+      o->box_cols = in[i]->box_cols;
+      o->box_H = in[i]->box_H;
+      o->box_W = in[i]->box_W;
+      o->box_eh = in[i]->box_eh;
+      o->box_ew = in[i]->box_ew;
+    }
     o->kept_buf = keep_buf;
     o->kept_idx = keep_buf->as<int32_t>() + keep_ld * i;
     node->prev = in[i]->cons;

@@ -104,7 +104,11 @@ def run_both(k, method="relax-star-area", shrink=1, check_constraints=True, marg
 
     Classification parity (bit-exact): inactive counts, crossing index lists in new-predicate order.
     Returns (device output, oracle output, NN object)."""
-    cfg = make_config(k, shrink)
+    return run_cfg(make_config(k, shrink), method, check_constraints, margins, tie_tolerant)
+
+
+def run_cfg(cfg, method="relax-star-area", check_constraints=True, margins=None, tie_tolerant=False):
+    """run_both for a configuration dictionary (name, kind, layers, lb, ub[, image_shape, partition])."""
     dev_in, ora_in = input_sets(cfg)
     net = NN.from_config(cfg["layers"], cfg["name"])
     dev_out = net.reach(dev_in, {"reachMethod": method, "relaxFactor": 1})

@@ -2,7 +2,7 @@
 import numpy as np
 import pytest
 
-from tests.gpu_util import RTOL, assert_close, compare_sets, flat_V, input_sets, run_both
+from tests.gpu_util import RTOL, assert_close, compare_sets, flat_V, input_sets, run_both, run_cfg
 
 pytestmark = pytest.mark.gpu
 
@@ -753,3 +753,32 @@ def test_released_arrays_give_their_memory_back(nnv):
     net.reachSet = []
     ctx.synchronize()
     assert ctx.pool_stats()[0] == used0
+
+
+@pytest.mark.parametrize("method", ["relax-star-area", "relax-star-random"])
+@pytest.mark.parametrize("shape,specs", [
+    # (FH, FW, Cout, stride, padding [t b l r], dilation) per convolution, a ReLU after each but the last
+    ((9, 8, 2), [(3, 3, 5, 1, [1, 1, 1, 1], 1), (3, 3, 6, 2, [0, 0, 0, 0], 1), (2, 3, 4, 1, [1, 0, 2, 1], 2), (1, 1, 3, 1, [0, 0, 0, 0], 1)]),
+    ((16, 16, 3), [(3, 3, 20, 1, [1, 1, 1, 1], 1), (5, 5, 33, 2, [2, 2, 2, 2], 1), (3, 3, 40, 1, [0, 0, 0, 0], 1), (3, 3, 8, 2, [1, 1, 1, 1], 1)]),
+    ((12, 20, 1), [(3, 1, 4, 1, [0, 0, 0, 0], 1), (1, 3, 4, 1, [0, 0, 1, 1], 1), (3, 3, 4, 3, [1, 1, 1, 1], 1)])])
+def test_chains_of_convolutions_keep_generator_images_inside_their_windows(nnv, oracle, method, shape, specs):
+    """Generators of a box ImageStar are single pixels; every convolution widens their images by its filter's
+    reach, and the device computes them inside those windows only.  Every layer's set against the oracle (zero
+    pattern included), over strides, asymmetric padding, dilation, windows cut by the image border, and a final
+    fully connected layer that reads the whole images."""
+    rs = np.random.RandomState(shape[0] * 7 + len(specs))
+    H, W, C = shape
+    layers = []
+    h, w, c = H, W, C
+    for i, (fh, fw, co, st, pad, dil) in enumerate(specs):
+        Wt = rs.randn(fh, fw, c, co) * np.sqrt(2.0 / (fh * fw * c))
+        L = {"type": "conv", "W": Wt, "b": 0.1 * rs.randn(co), "padding": pad, "stride": [st, st], "dilation": [dil, dil]}
+        layers.append(L)
+        h, w = oracle.conv2d_output_size(h, w, fh, fw, pad, [st, st], [dil, dil])
+        c = co
+        layers.append({"type": "relu"})
+    layers.append({"type": "fc", "W": rs.randn(7, h * w * c) / np.sqrt(h * w * c), "b": rs.randn(7)})
+    x = rs.rand(H * W * C)
+    cfg = {"name": "conv chain %dx%dx%d" % shape, "kind": "image", "image_shape": shape, "layers": layers,
+           "lb": x - 0.05, "ub": x + 0.05}
+    run_cfg(cfg, method)
