@@ -126,6 +126,57 @@ def test_random_cnn_sequences(nnv, oracle, seed):
     _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area")
 
 
+ALL_RELAX = ["relax-star-area", "relax-star-range", "relax-star-static", "relax-star-random", "relax-star-bound",
+             "relax-star-ub"]
+
+
+@pytest.mark.parametrize("seed", range(300, 324))
+def test_random_chains_of_convolutions(nnv, oracle, seed):
+    """One to four convolutions of random geometry (filter 1..5, stride 1..3, dilation 1..2, asymmetric padding, 2 to
+    40 output channels) on a box ImageStar with a different width per pixel (so that no two sort keys tie), with
+    ReLUs, doubled ReLUs, batch normalisation, convolutions straight on convolutions and average pooling in between,
+    most of them ending in two fully connected layers: every layer's set against the oracle, zero pattern included."""
+    rs = np.random.RandomState(seed)
+    H, W, c = int(rs.choice([6, 9, 12, 17])), int(rs.choice([6, 8, 13, 16])), int(rs.choice([1, 2, 3]))
+    cin = c
+    h, w = H, W
+    layers = []
+    for _ in range(int(rs.choice([1, 2, 3, 4]))):
+        fh, fw = int(rs.choice([1, 2, 3, 5])), int(rs.choice([1, 2, 3, 5]))
+        st = [int(rs.choice([1, 1, 2, 3])), int(rs.choice([1, 1, 2]))]
+        dil = [int(rs.choice([1, 1, 2])), int(rs.choice([1, 1, 2]))]
+        pad = [int(v) for v in rs.randint(0, 3, size=4)]
+        ho = (h + pad[0] + pad[1] - (fh - 1) * dil[0] - 1) // st[0] + 1
+        wo = (w + pad[2] + pad[3] - (fw - 1) * dil[1] - 1) // st[1] + 1
+        if h + pad[0] + pad[1] - (fh - 1) * dil[0] - 1 < 0 or w + pad[2] + pad[3] - (fw - 1) * dil[1] - 1 < 0:
+            fh = fw = 1
+            st, dil, pad = [1, 1], [1, 1], [0, 0, 0, 0]
+            ho, wo = h, w
+        co = int(rs.choice([2, 5, 17, 33, 40]))
+        layers.append({"type": "conv", "W": rs.randn(fh, fw, c, co) * np.sqrt(2.0 / (fh * fw * c)), "b": rs.randn(co) * 0.1,
+                       "padding": pad, "stride": st, "dilation": dil})
+        h, w, c = ho, wo, co
+        r = rs.rand()
+        if r < 0.7:
+            layers.append({"type": "relu"})
+            if rs.rand() < 0.15:
+                layers.append({"type": "relu"})
+        elif r < 0.85:
+            layers += [_bn(rs, c), {"type": "relu"}]
+        if rs.rand() < 0.15 and h >= 2 and w >= 2:
+            layers.append({"type": "avgpool", "pool": [2, 2], "stride": [2, 2], "padding": [0, 0, 0, 0]})
+            h, w = (h - 2) // 2 + 1, (w - 2) // 2 + 1
+    if rs.rand() < 0.7:
+        layers += [_fc(rs, 12, h * w * c, 2.0), {"type": "relu"}, _fc(rs, 4, 12)]
+    x = rs.rand(H, W, cin)
+    e = float(rs.choice([0.005, 0.05, 0.3])) * (0.5 + rs.rand(H, W, cin))
+    lo, hi = x - e, x + e
+    if rs.rand() < 0.3:
+        k = rs.randint(lo.size)
+        hi.reshape(-1)[k] = lo.reshape(-1)[k]
+    _compare(nnv, oracle, layers, nnv.ImageStar(lo, hi), oracle.image_star_from_bounds(lo, hi), ALL_RELAX[seed % 6])
+
+
 @pytest.mark.parametrize("wide,count,method", [(9000, 1, "relax-star-range"), (8200, 2, "relax-star-static")])
 def test_wide_layers_in_a_sequence(nnv, oracle, wide, count, method):
     # more than 8192 neurons: classification, sort and bounds run as separate multi-block kernels, and
