@@ -49,6 +49,7 @@ __device__ __forceinline__ unsigned long long pack_tap(const ConvGeom& g, int k)
 struct ConvRows {
   const ColBox* box;
   int eh, area;
+  const ColBox* in_box;  // windows of the input images, or null: a tap outside its image's window is not read
 };
 
 template <bool COMPACT>
@@ -86,7 +87,7 @@ template <int TP, int TC, int WR, int WC, int FM, int FN, bool COMPACT = false>
 __device__ __forceinline__ void conv_store_tile(const double4_t (&acc)[FM][FN], double* __restrict__ out, int64_t ldout,
                                                 const double* __restrict__ bias, const ConvGeom& g, int64_t total_rows,
                                                 int64_t R0, int c0, int wr, int wc, int lane,
-                                                const ConvRows cr = ConvRows{nullptr, 0, 0}) {
+                                                const ConvRows cr = ConvRows{nullptr, 0, 0, nullptr}) {
   const int lrow = lane & 15;
   const int lcol = lane >> 4;
 #pragma unroll
@@ -310,10 +311,17 @@ __global__ __launch_bounds__(512) void conv2d_fast_kernel(const double* __restri
     const int w0 = wo * g.sw - g.pl;
     toff = (uint32_t)((gi - gi0) * ldin * 8);
     base_row = h0 + w0 * g.H;
+    // taps inside the image - and, where the input images come with windows, inside this image's window (the
+    // rows outside it are zero and may not be in memory)
+    int ha = 0, hb = g.H - 1, wa = 0, wb = g.W - 1;
+    if (COMPACT && cr.in_box != nullptr) {
+      const ColBox b = cr.in_box[gi];
+      ha = max(ha, (int)b.h0), hb = min(hb, (int)b.h1), wa = max(wa, (int)b.w0), wb = min(wb, (int)b.w1);
+    }
     for (int fw = 0; fw < g.FW; ++fw)
       for (int fh = 0; fh < g.FH; ++fh) {
         const int h = h0 + fh * g.dh, w = w0 + fw * g.dw;
-        if ((unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W) vmask |= 1u << (fh + g.FH * fw);
+        if (h >= ha && h <= hb && w >= wa && w <= wb) vmask |= 1u << (fh + g.FH * fw);
       }
   }
 
@@ -421,7 +429,10 @@ __global__ void conv_boxes_kernel(const ColBox* __restrict__ in_box, int64_t den
     h0 = b.h0, h1 = b.h1, w0 = b.w0, w1 = b.w1;
   }
   ColBox o;
-  if (h0 > h1 || w0 > w1) {
+  if (j == 0) {
+    // the centre image is not sparse: where every tap falls into the padding it still holds the bias
+    o = ColBox{0, (int16_t)(g.Ho - 1), 0, (int16_t)(g.Wo - 1)};
+  } else if (h0 > h1 || w0 > w1) {
     o = ColBox{1, 0, 1, 0};
   } else {
     // output rows whose taps ho*sh - pt + fh*dh (0 <= fh < FH) reach [h0, h1]
@@ -457,7 +468,7 @@ struct StampSet {
   const double* pub;
   double* part;         // [chunks][4][ldout] range sums of these columns (as the estimateRanges pass leaves them)
   int32_t m;
-  int32_t pad_;
+  int32_t win_only;     // 1: only the rows inside a column's window (the positions whose taps span its pixel) are written
 };
 
 __global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restrict__ table, StampSet one, ConvGeom g,
@@ -509,10 +520,12 @@ __global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restr
       const int h = s_h[t], w = s_w[t], kc = s_k[t];
       const double s = s_s[t];
       double v[2];
+      bool inwin[2];
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         v[e] = 0.0;
         const int th = h - hb[e], tw = w - wb[e];
+        inwin[e] = real[e] && th >= 0 && tw >= 0 && th <= (g.FH - 1) * g.dh && tw <= (g.FW - 1) * g.dw;
         if (real[e] && th >= 0 && tw >= 0) {
           int fh = th, fw = tw;
           bool hit = true;
@@ -527,7 +540,13 @@ __global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restr
           }
         }
       }
-      if (r0 < ldout) *reinterpret_cast<double2*>(d.out + r0 + (int64_t)(jb + t) * ldout) = make_double2(v[0], v[1]);
+      if (d.win_only) {
+        double* o = d.out + r0 + (int64_t)(jb + t) * ldout;
+        if (inwin[0]) o[0] = v[0];
+        if (inwin[1]) o[1] = v[1];
+      } else if (r0 < ldout) {
+        *reinterpret_cast<double2*>(d.out + r0 + (int64_t)(jb + t) * ldout) = make_double2(v[0], v[1]);
+      }
       const double pl = d.plb[jb + t], pu = d.pub[jb + t];
       const double px = fmax(v[0], 0.0), nx = fmin(v[0], 0.0);
       const double py = fmax(v[1], 0.0), ny = fmin(v[1], 0.0);
@@ -697,6 +716,13 @@ static int launch_conv_fast(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const Conv
   return NNVHIP_OK;
 }
 
+int launch_zero_pad_rows(nnvhip_ctx* ctx, double* V, int64_t ld, int64_t N, int64_t ncols) {
+  if (ld == N || ncols <= 0) return NNVHIP_OK;
+  hipLaunchKernelGGL(zero_pad_rows_kernel, dim3(256), dim3(256), 0, ctx->stream, V, ld, N, ncols);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
 int64_t conv_box_extent(const nnvhip_conv2d* cv, int dim, int64_t e, int64_t out_size) {
   // output positions whose taps reach a run of e input positions: floor((e - 1 + (F - 1) * dil) / stride) + 1
   const int64_t F = dim == 0 ? cv->FH : cv->FW;
@@ -713,9 +739,17 @@ int launch_conv_boxes(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64
   return NNVHIP_OK;
 }
 
+bool conv2d_in_windows(const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin, int64_t ncols,
+                       const ColBox* out_box, int eh, int ew) {
+  ConvGeom g;
+  fill_geom(g, cv, H, W, Ho, Wo);
+  return out_box != nullptr && ncols > 1 && eh > 0 && ew > 0 && 2 * (int64_t)eh * ew <= g.P &&
+         conv_fast_ok(cv, g, ldin, (int64_t)eh * ew);
+}
+
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
-                  const int32_t* pending_cls, const ColBox* out_box, int eh, int ew) {
+                  const int32_t* pending_cls, const ColBox* out_box, int eh, int ew, const ColBox* in_box, bool leave_outside) {
   if (cv->Kp > kMaxTaps) NNV_FAIL(NNVHIP_ERR_SHAPE, "filters with more than %d taps (FH*FW*Cin) are not supported", kMaxTaps);
   if ((cv->FH - 1) * cv->dil[0] > 0xffff || (cv->FW - 1) * cv->dil[1] > 0xffff)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "dilated filter extent too large");
@@ -742,10 +776,11 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W
   int st;
   // Generator images with known windows are computed inside them only (the caller has zeroed the rest) when that
   // at least halves the rows; it takes the kernel with scalar tap decoding.
-  ConvRows cr{nullptr, 0, 0};
-  if (out_box != nullptr && ncols > 1 && eh > 0 && ew > 0 && 2 * (int64_t)eh * ew <= g.P && conv_fast_ok(cv, g, ldin, (int64_t)eh * ew))
-    cr = ConvRows{out_box, eh, eh * ew};
-  if (cr.box != nullptr)  // everything outside the windows
+  ConvRows cr{nullptr, 0, 0, nullptr};
+  if (conv2d_in_windows(cv, H, W, Ho, Wo, ldin, ncols, out_box, eh, ew)) cr = ConvRows{out_box, eh, eh * ew, in_box};
+  if (cr.box == nullptr && (in_box != nullptr || leave_outside))
+    NNV_FAIL(NNVHIP_ERR_ARG, "internal: the convolution was to stay inside the images' windows");
+  if (cr.box != nullptr && !leave_outside)  // everything outside the windows
     NNV_HIP_TRY(hipMemsetAsync(out + ldout, 0, sizeof(double) * (size_t)ldout * (size_t)(ncols - 1), ctx->stream));
   if (cr.box != nullptr || conv_fast_ok(cv, g, ldin)) {
     if (cv->Cout <= 16)
@@ -790,7 +825,74 @@ static void fill_geom(ConvGeom& g, const nnvhip_conv2d* cv, int64_t H, int64_t W
   g.HW = (int)(H * W);
 }
 
-int64_t conv_stamp_chunks(int64_t ldout, int64_t count, int64_t max_m) {
+// ---- the stamps by output row (undilated filters) ---------------------------------------------------
+// Row r = (ho, wo, co) of the output meets the stamps of the pixels under its filter window, one per tap: for
+// tap k = (fh, fw, ci) the pixel (ho*sh - pt + fh, wo*sw - pl + fw, ci), whose unit-vector column t (pixel_col,
+// -1: none) gets out(r, t) = 0 + W(k, co) * scale.  One thread per row writes those elements - exactly the
+// non-zero candidates, i.e. the rows inside every column's window - and adds up the row's four range sums tap
+// by tap.  Everything else in the columns is zero and is written by the caller (or left for later).
+__global__ void stamp_pixel_columns_kernel(const int32_t* __restrict__ idx, int m, int32_t* __restrict__ pixel_col) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t < m) pixel_col[idx[t]] = t;
+}
+
+// S lanes share a row, lane s taking the taps k = s, s + S, ...; their sums are combined by a butterfly (a fixed
+// order).  S = 1 for filters with few taps, 16 otherwise (a row's taps are then walked by 16 lanes at once).
+template <int S>
+__global__ __launch_bounds__(256) void conv_stamp_rows_kernel(StampSet d, ConvGeom g, const double* __restrict__ Wt,
+                                                              const int32_t* __restrict__ pixel_col, int64_t ldout) {
+  const int64_t gt = blockIdx.x * (int64_t)256 + threadIdx.x;
+  const int64_t r = gt / S;
+  const int s = (int)(gt % S);
+  const bool row = r < ldout;
+  const int64_t Nout = (int64_t)g.P * g.Cout;
+  double x1 = 0.0, x2 = 0.0, y1 = 0.0, y2 = 0.0;
+  if (row && r < Nout) {
+    const int co = (int)(r / g.P);
+    const int p = (int)(r - (int64_t)co * g.P);
+    const int wo = p / g.Ho, ho = p - wo * g.Ho;
+    const int hb = ho * g.sh - g.pt, wb = wo * g.sw - g.pl;
+    const double* wcol = Wt + (int64_t)co * g.Kp;
+    for (int k = s; k < g.K; k += S) {
+      const int fh = k % g.FH;
+      const int q = k / g.FH;
+      const int fw = q % g.FW;
+      const int ci = q / g.FW;
+      const int h = hb + fh, w = wb + fw;
+      if ((unsigned)h >= (unsigned)g.H || (unsigned)w >= (unsigned)g.W) continue;
+      const int pixel = h + g.H * (w + g.W * ci);
+      const int t = pixel_col[pixel];
+      if (t < 0) continue;
+      const double sc = d.scale != nullptr ? d.scale[pixel] : 1.0;
+      const double v = __dadd_rn(0.0, __dmul_rn(wcol[k], sc));
+      d.out[r + (int64_t)t * ldout] = v;
+      const double pl = d.plb[t], pu = d.pub[t];
+      const double vp = fmax(v, 0.0), vn = fmin(v, 0.0);
+      x1 = fma(vp, pl, x1);  // xmin1
+      x2 = fma(vn, pu, x2);  // xmin2
+      y1 = fma(vp, pu, y1);  // xmax1
+      y2 = fma(vn, pl, y2);  // xmax2
+    }
+  }
+#pragma unroll
+  for (int off = 1; off < S; off <<= 1) {
+    x1 += __shfl_xor(x1, off);
+    x2 += __shfl_xor(x2, off);
+    y1 += __shfl_xor(y1, off);
+    y2 += __shfl_xor(y2, off);
+  }
+  if (row && s == 0) {
+    d.part[r] = x1;
+    d.part[ldout + r] = x2;
+    d.part[2 * ldout + r] = y1;
+    d.part[3 * ldout + r] = y2;
+  }
+}
+
+static bool conv_stamps_by_row(const nnvhip_conv2d* cv) { return cv->dil[0] == 1 && cv->dil[1] == 1; }
+
+int64_t conv_stamp_chunks(const nnvhip_conv2d* cv, int64_t ldout, int64_t count, int64_t max_m) {
+  if (conv_stamps_by_row(cv)) return 1;
   const int64_t row_blocks = ceil_div(ldout, 128);
   int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks * count), ceil_div(std::max<int64_t>(max_m, 1), 32)));
   const int64_t cpc = ceil_div(std::max<int64_t>(max_m, 1), chunks);
@@ -811,6 +913,32 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int6
   if (max_m == 0) return NNVHIP_OK;
   ConvGeom g;
   fill_geom(g, cv, H, W, Ho, Wo);
+  if (conv_stamps_by_row(cv)) {
+    if (chunks != 1) NNV_FAIL(NNVHIP_ERR_ARG, "internal: one chunk of range sums per set");
+    const int64_t n_in = H * W * cv->Cin;
+    BufRef inv;
+    NNV_TRY(ctx->alloc(sizeof(int32_t) * (size_t)n_in * (size_t)count, &inv));
+    NNV_HIP_TRY(hipMemsetAsync(inv->ptr, 0xff, sizeof(int32_t) * (size_t)n_in * (size_t)count, ctx->stream));
+    NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
+    for (int64_t i = 0; i < count; ++i) {
+      if (sets[i].m == 0) continue;
+      StampSet one;
+      memcpy(&one, &sets[i], sizeof one);
+      int32_t* pc = inv->as<int32_t>() + n_in * i;
+      if (!one.win_only)  // whole columns: the zeros first
+        NNV_HIP_TRY(hipMemsetAsync(one.out, 0, sizeof(double) * (size_t)ldout * (size_t)one.m, ctx->stream));
+      hipLaunchKernelGGL(stamp_pixel_columns_kernel, dim3((unsigned)ceil_div(one.m, 256)), dim3(256), 0, ctx->stream, one.idx, one.m, pc);
+      if (g.K <= 32)
+        NNV_LAUNCH(ctx, ctx->kernel_timing && i == 0, conv_stamp_rows_kernel<1>, dim3((unsigned)ceil_div(ldout, 256)), dim3(256), 0, one, g,
+                   cv->W->as<double>(), pc, ldout);
+      else
+        NNV_LAUNCH(ctx, ctx->kernel_timing && i == 0, conv_stamp_rows_kernel<16>, dim3((unsigned)ceil_div(ldout * 16, 256)), dim3(256), 0,
+                   one, g, cv->W->as<double>(), pc, ldout);
+    }
+    NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
+    NNV_HIP_TRY(hipGetLastError());
+    return NNVHIP_OK;
+  }
   const int64_t row_blocks = ceil_div(ldout, 128);
   const int64_t cpc = ceil_div(max_m, chunks);
   const StampSet* table = nullptr;

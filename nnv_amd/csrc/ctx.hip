@@ -1768,75 +1768,109 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
   };
   bool any_stamps = false;
   int64_t max_m = 0;
+  // Windows of the generator images (internal.h, nnvhip_star::box).  The output's come from the input's windows and
+  // from the pixels of its unit-vector columns (without either an image counts as full); where the input's dense
+  // images have small windows the implicit GEMM computes inside the output windows only.
+  const bool track_boxes = !c->no_conv_boxes && H < 32768 && W < 32768 && Ho < 32768 && Wo < 32768;
+  struct Plan {
+    int64_t nc = 0, dense = 0, m = 0;
+    bool in_ok = false;      // the input's windows describe its dense images
+    bool out_boxes = false;  // the output gets windows
+    bool compact = false;    // the dense images are computed inside their windows only
+    int dense_eh = 0, dense_ew = 0;
+  };
+  std::vector<Plan> plan((size_t)count);
+  for (int64_t i = 0; i < count; ++i) {
+    Plan& pl = plan[i];
+    pl.nc = in[i]->n + 1;
+    pl.dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < pl.nc) ? in[i]->oh_from : pl.nc;
+    pl.m = pl.nc - pl.dense;
+    if (!track_boxes) continue;
+    pl.in_ok = in[i]->box != nullptr && in[i]->box_H == H && in[i]->box_W == W && in[i]->box_cols >= pl.dense;
+    pl.out_boxes = pl.in_ok || (pl.m > 0 && pl.dense == 1);
+    if (pl.in_ok && pl.dense > 1) {
+      pl.dense_eh = (int)conv_box_extent(cv, 0, in[i]->box_eh, Ho);
+      pl.dense_ew = (int)conv_box_extent(cv, 1, in[i]->box_ew, Wo);
+      // (any table will do for the question; the real one is made below)
+      pl.compact = conv2d_in_windows(cv, H, W, Ho, Wo, in[i]->ld, pl.dense, in[i]->box, pl.dense_eh, pl.dense_ew);
+    }
+  }
   {
-    // the implicit GEMM reads whole images: pending row resets are run first, and sets whose unit-vector
-    // columns take part in the contraction get those written out
-    // (a pending reset alone is applied by the kernel as it loads, from one bit per row, where that fits)
+    // The implicit GEMM reads whole images: pending row resets are run first, and sets whose unit-vector
+    // columns take part in the contraction get those written out.  (A pending reset alone is applied by the
+    // kernel as it loads, from one bit per row, where that fits; images that are in memory inside their windows
+    // only are fine for the kernel that stays inside the windows.)
     std::vector<nnvhip_star*> full, prefix;
     for (int64_t i = 0; i < count; ++i) {
-      const int64_t nc = in[i]->n + 1;
-      const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
-      if (dense > in[i]->stored_cols())
+      const ColSource& cs = in[i]->cs;
+      if (plan[i].dense > in[i]->stored_cols())
         full.push_back(in[i]);
-      else if (in[i]->cs.any_pending() || (in[i]->rows_pending && !mask_on_load(in[i])))
+      else if (cs.pending || cs.zero_to > 1 || (cs.win_pending() && !plan[i].compact) ||
+               (in[i]->rows_pending && !mask_on_load(in[i])))
         prefix.push_back(in[i]);
     }
     if (st == NNVHIP_OK && !full.empty()) st = ensure_dense_batch(c, (int64_t)full.size(), full.data());
     if (st == NNVHIP_OK && !prefix.empty()) st = ensure_dense_batch(c, (int64_t)prefix.size(), prefix.data(), false);
   }
-  // windows of the output's generator images (internal.h, nnvhip_star::box): from the input's windows and from
-  // the pixels of its unit-vector columns; without either the images count as full
-  const bool track_boxes = !c->no_conv_boxes && H < 32768 && W < 32768 && Ho < 32768 && Wo < 32768;
   for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
-    const int64_t nc = in[i]->n + 1;
-    const int64_t dense = (!c->dense_affine && in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
-    const ColBox* dense_box = nullptr;
-    int dense_eh = 0, dense_ew = 0;
-    if (track_boxes) {
-      const bool in_ok = in[i]->box != nullptr && in[i]->box_H == H && in[i]->box_W == W && in[i]->box_cols >= dense;
-      const int64_t m = nc - dense;
-      if (in_ok || (m > 0 && dense == 1)) {
-        st = c->alloc(sizeof(ColBox) * (size_t)nc, &outs[i]->box_buf);
-        if (st != NNVHIP_OK) break;
-        ColBox* ob = outs[i]->box_buf->as<ColBox>();
-        st = launch_conv_boxes(c, cv, H, W, Ho, Wo, in_ok ? in[i]->box : nullptr, dense, in[i]->oh_idx, m, ob);
-        if (st != NNVHIP_OK) break;
-        int64_t eh = 0, ew = 0;
-        if (dense > 1) {  // (only reached with in_ok)
-          dense_eh = (int)conv_box_extent(cv, 0, in[i]->box_eh, Ho);
-          dense_ew = (int)conv_box_extent(cv, 1, in[i]->box_ew, Wo);
-          dense_box = ob;
-          eh = dense_eh;
-          ew = dense_ew;
-        }
-        if (m > 0) {
-          eh = std::max(eh, conv_box_extent(cv, 0, 1, Ho));
-          ew = std::max(ew, conv_box_extent(cv, 1, 1, Wo));
-        }
-        outs[i]->box = ob;
-        outs[i]->box_cols = nc;
-        outs[i]->box_H = (int32_t)Ho;
-        outs[i]->box_W = (int32_t)Wo;
-        outs[i]->box_eh = (int32_t)eh;
-        outs[i]->box_ew = (int32_t)ew;
+    const Plan& pl = plan[i];
+    nnvhip_star* o = outs[i];
+    const ColBox* ob = nullptr;
+    if (pl.out_boxes) {
+      st = c->alloc(sizeof(ColBox) * (size_t)pl.nc, &o->box_buf);
+      if (st != NNVHIP_OK) break;
+      ColBox* tab = o->box_buf->as<ColBox>();
+      st = launch_conv_boxes(c, cv, H, W, Ho, Wo, pl.in_ok ? in[i]->box : nullptr, pl.dense, in[i]->oh_idx, pl.m, tab);
+      if (st != NNVHIP_OK) break;
+      int64_t eh = pl.dense > 1 ? pl.dense_eh : 0, ew = pl.dense > 1 ? pl.dense_ew : 0;
+      if (pl.m > 0) {
+        eh = std::max(eh, conv_box_extent(cv, 0, 1, Ho));
+        ew = std::max(ew, conv_box_extent(cv, 1, 1, Wo));
       }
+      ob = tab;
+      o->box = tab;
+      o->box_cols = pl.nc;
+      o->box_H = (int32_t)Ho;
+      o->box_W = (int32_t)Wo;
+      o->box_eh = (int32_t)eh;
+      o->box_ew = (int32_t)ew;
+    }
+    // Images with windows are written inside them only; the zeros around them wait for a reader of whole
+    // columns (ColSource::win_*).  Not when the caller wants every column in memory.
+    const bool lazy = ob != nullptr && !c->eager_cols;
+    const int64_t win_from = lazy ? (pl.compact ? 1 : pl.dense) : 0;
+    const int64_t win_to = lazy ? (pl.m > 0 ? pl.nc : (pl.compact ? pl.dense : 0)) : 0;
+    if (win_to > win_from) {
+      o->cs.win_box_buf = o->box_buf;
+      o->cs.win_box = ob;
+      o->cs.win_from = win_from;
+      o->cs.win_to = win_to;
+      o->cs.win_rows = Nout;
+      o->cs.win_H = (int32_t)Ho;
+      o->cs.win_W = (int32_t)Wo;
+      if (c->poison_pending)  // debugging aid: NaNs where nothing will be written
+        NNV_HIP_TRY(hipMemsetAsync(o->V + win_from * o->ld, 0xff, sizeof(double) * o->ld * (win_to - win_from), c->stream));
     }
     stamps[i].idx = in[i]->oh_idx;
     stamps[i].scale = in[i]->oh_scale;
-    stamps[i].out = outs[i]->V + dense * outs[i]->ld;
-    stamps[i].plb = outs[i]->plb + (dense - 1);
-    stamps[i].pub = outs[i]->pub + (dense - 1);
+    stamps[i].out = o->V + pl.dense * o->ld;
+    stamps[i].plb = o->plb + (pl.dense - 1);
+    stamps[i].pub = o->pub + (pl.dense - 1);
     stamps[i].part = nullptr;
-    stamps[i].m = (int32_t)(nc - dense);
-    stamps[i].pad_ = 0;
-    any_stamps = any_stamps || dense < nc;
-    max_m = std::max<int64_t>(max_m, nc - dense);
-    st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, outs[i]->V, outs[i]->ld, dense,
-                       in[i]->rows_pending ? in[i]->cls : nullptr, dense_box, dense_eh, dense_ew);
+    stamps[i].m = (int32_t)pl.m;
+    stamps[i].win_only = (lazy && pl.m > 0) ? 1 : 0;
+    any_stamps = any_stamps || pl.m > 0;
+    max_m = std::max<int64_t>(max_m, pl.m);
+    st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, o->V, o->ld, pl.dense,
+                       in[i]->rows_pending ? in[i]->cls : nullptr, pl.compact ? ob : nullptr, pl.dense_eh, pl.dense_ew,
+                       pl.compact ? in[i]->box : nullptr, pl.compact && lazy);
+    // (launch_conv2d zeroes the padding rows of the columns it writes; the stamp kernel only writes them when
+    // it writes whole columns)
+    if (st == NNVHIP_OK && stamps[i].win_only && o->ld != Nout) st = launch_zero_pad_rows(c, stamps[i].out, o->ld, Nout, pl.m);
   }
   if (st == NNVHIP_OK && any_stamps) {
     // the stamp pass also leaves the range sums of its columns on the output handles
-    const int64_t sch = conv_stamp_chunks(outs[0]->ld, count, max_m);
+    const int64_t sch = conv_stamp_chunks(cv, outs[0]->ld, count, max_m);
     BufRef sums;
     st = c->alloc(sizeof(double) * 4 * outs[0]->ld * sch * count, &sums);
     if (st == NNVHIP_OK) {

@@ -449,6 +449,14 @@ __global__ __launch_bounds__(512) void pack_rows_kernel(const PackSet* __restric
   const int t0 = blockIdx.x * 128 + 2 * lane;
   if (t0 >= d.kp) return;
   const int ra = d.kept[t0], rb = d.kept[t0 + 1];
+  // image positions of the two rows, for columns that are only defined inside their windows
+  int ha = 0, wa = 0, hb = 0, wb = 0;
+  if (d.box != nullptr) {
+    const int P = d.bH * d.bW;
+    const int pa = max(ra, 0) % P, pb = max(rb, 0) % P;
+    wa = pa / d.bH, ha = pa - wa * d.bH;
+    wb = pb / d.bH, hb = pb - wb * d.bH;
+  }
   for (int jb = j0 + 4 * wave; jb < j1; jb += 32) {
     double2 v[4];
 #pragma unroll
@@ -464,8 +472,14 @@ __global__ __launch_bounds__(512) void pack_rows_kernel(const PackSet* __restric
           if (rb >= 0) v[u].y = __dadd_rn(0.0, __dmul_rn(col[rb], sc));
         } else {
           const double* col = d.V + (int64_t)j * d.ld;
-          if (ra >= 0) v[u].x = col[ra];
-          if (rb >= 0) v[u].y = col[rb];
+          bool ina = ra >= 0, inb = rb >= 0;
+          if (d.box != nullptr && j >= d.box_from && j < d.box_to) {
+            const ColBox b = d.box[j];
+            ina = ina && ha >= b.h0 && ha <= b.h1 && wa >= b.w0 && wa <= b.w1;
+            inb = inb && hb >= b.h0 && hb <= b.h1 && wb >= b.w0 && wb <= b.w1;
+          }
+          if (ina) v[u].x = col[ra];
+          if (inb) v[u].y = col[rb];
         }
       }
     }
@@ -487,6 +501,13 @@ PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t 
     p.wend = (int32_t)std::min<int64_t>(ncols, cs.from + cs.cols);
   }
   p.zero_to = (int32_t)std::min<int64_t>(ncols, cs.zero_to);
+  if (cs.win_pending() && cs.win_from < ncols) {
+    p.box = cs.win_box;
+    p.box_from = (int32_t)cs.win_from;
+    p.box_to = (int32_t)std::min<int64_t>(ncols, cs.win_to);
+    p.bH = cs.win_H;
+    p.bW = cs.win_W;
+  }
   return p;
 }
 

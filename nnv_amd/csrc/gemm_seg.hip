@@ -237,10 +237,20 @@ __global__ __launch_bounds__(256) void pack_rows_t_kernel(const PackSet* __restr
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int t = t0 + lane;
   const int ra = t < d.kp ? d.kept[t] : -1;
+  int ha = 0, wa = 0;  // image position of the row, for columns that are only defined inside their windows
+  if (d.box != nullptr) {
+    const int pa = max(ra, 0) % (d.bH * d.bW);
+    wa = pa / d.bH, ha = pa - wa * d.bH;
+  }
   for (int cc = wave; cc < 64; cc += 4) {
     const int j = j0 + cc;
     double v = 0.0;
-    if (ra >= 0 && j < d.ncols && !(j >= 1 && j < d.zero_to)) {
+    bool in = ra >= 0 && j < d.ncols && !(j >= 1 && j < d.zero_to);
+    if (in && d.box != nullptr && j >= d.box_from && j < d.box_to) {
+      const ColBox b = d.box[j];
+      in = ha >= b.h0 && ha <= b.h1 && wa >= b.w0 && wa <= b.w1;
+    }
+    if (in) {
       if (d.W != nullptr && j >= d.wfrom && j < d.wend) {  // the value the gather pass wrote, recomputed
         const int src = d.widx[j - d.wfrom];
         const double sc = d.wscale ? d.wscale[src] : 1.0;

@@ -111,7 +111,17 @@ struct ColSource {
   int64_t cols = 0;
   bool pending = false;  // the columns [from, from + cols) are not in memory yet
   int64_t zero_to = 0;   // > 1: the columns [1, zero_to) are +0 and not in memory yet
-  bool any_pending() const { return pending || zero_to > 1; }
+  // Generator images of a convolution's output that are in memory inside their windows only (win_box[j], an
+  // image of win_H x win_W positions per channel): columns [win_from, win_to); the rows outside the windows,
+  // which are zero, have not been written.  The next convolution and the range scan read inside the windows
+  // only; whoever reads whole columns has the zeros written first (write_pending_columns).
+  BufRef win_box_buf;
+  const ColBox* win_box = nullptr;
+  int64_t win_from = 0, win_to = 0;
+  int64_t win_rows = 0;  // rows of the image (H * W * channels)
+  int32_t win_H = 0, win_W = 0;
+  bool win_pending() const { return win_to > win_from; }
+  bool any_pending() const { return pending || zero_to > 1 || win_pending(); }
 };
 
 // One node per ReLU layer of the structured constraint store.  The dense NNV matrix
@@ -468,6 +478,11 @@ struct PackSet {
   int32_t wend = 0;
   int32_t zero_to = 0;  // > 1: columns [1, zero_to) are +0 whatever the memory holds
   int64_t ldt = 0;      // launch_pack_rows_t: Vk is kp x ldt, row-major (columns [ncols, ldt) are written as zeros)
+  // columns [box_from, box_to) are +0 outside their windows box[j] (images of bH x bW positions per channel),
+  // whatever the memory holds there (box == null: none)
+  const ColBox* box = nullptr;
+  int32_t box_from = 0, box_to = 0;
+  int32_t bH = 0, bW = 0;
 };
 // the packing of the first `ncols` columns of a set, with what is known about where they came from
 PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t kp, int64_t ncols);
@@ -509,10 +524,16 @@ int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
                   const int32_t* pending_cls /* per input row, or null: rows whose class is not kKeep read as zero */,
-                  const ColBox* out_box = nullptr /* per output column, or null: with it, columns 1.. are computed inside
-                                                    their windows only (at most eh x ew positions) and must be zero
-                                                    elsewhere already */,
-                  int eh = 0, int ew = 0);
+                  const ColBox* out_box = nullptr /* per output column, or null: with it (and conv2d_in_windows), columns
+                                                    1.. are computed inside their windows only, at most eh x ew positions */,
+                  int eh = 0, int ew = 0,
+                  const ColBox* in_box = nullptr /* windows of the input columns: taps outside them are not read (the input
+                                                    may be in memory inside its windows only); needs conv2d_in_windows */,
+                  bool leave_outside = false /* do not write the zeros outside the output windows */);
+int launch_zero_pad_rows(nnvhip_ctx* ctx, double* V, int64_t ld, int64_t N, int64_t ncols);  // rows [N, ld) of ncols columns := 0
+// whether launch_conv2d computes the generator images of such a call inside their windows only
+bool conv2d_in_windows(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin, int64_t ncols,
+                       const ColBox* out_box, int eh, int ew);
 // Windows of a convolution's output columns: column 0 the whole image; columns below `dense` from the input's
 // windows (in_box null: whole image); the `m` columns from `dense` on from the pixels onehot_idx names.
 int launch_conv_boxes(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
@@ -532,10 +553,10 @@ struct ConvStampSet {
   const double* pub;
   double* part;         // this set's [chunks][4][ldout] range sums
   int32_t m;
-  int32_t pad_;
+  int32_t win_only;     // 1: write the rows inside each column's window only
 };
 // Number of column chunks (= range-sum chunks per set) the stamp launch will use.
-int64_t conv_stamp_chunks(int64_t ldout, int64_t count, int64_t max_m);
+int64_t conv_stamp_chunks(const nnvhip_conv2d* conv, int64_t ldout, int64_t count, int64_t max_m);
 int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                        int64_t ldout, int64_t count, const ConvStampSet* sets, int64_t chunks);
 

@@ -30,6 +30,10 @@ struct RangeDesc {
   int32_t chunks;
   int32_t cols_per_chunk;
   int32_t row_waves;  // waves of a block laid along rows (1, 2, 4 or 8); the others interleave columns
+  // windows of the generator images (column j is zero, and possibly not in memory, outside box[j]: images of
+  // bH x bW positions per channel), or null: a row outside a column's window is not loaded
+  const ColBox* box;
+  int32_t bH, bW;
 };
 
 constexpr int kRowsPerWave = 128;  // 64 lanes x 2 rows
@@ -114,6 +118,120 @@ __global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(c
       *reinterpret_cast<double2*>(p + d.ld) = xmin2;
       *reinterpret_cast<double2*>(p + 2 * d.ld) = xmax1;
       *reinterpret_cast<double2*>(p + 3 * d.ld) = xmax2;
+    }
+  }
+}
+
+// The same sums for a set whose generator images come with windows (RangeDesc::box), read inside the windows only:
+// the images may not even be in memory outside them.  Lane = image position, a block covers 64 positions of
+// kWinCG channels, so that one window test serves kWinCG loads.  Columns are dealt to the eight waves, added up
+// and combined exactly as in ranges_partial_kernel with row_waves = 1 (wave w takes the columns j0 + 8w + 64k ...
+// + 7 in order; wave 0 then adds the other waves' sums in wave order): skipping the exact zeros outside a window
+// leaves every sum as it is, so both kernels give the same bits.
+constexpr int kWinCG = 4;
+__global__ __launch_bounds__(512) void ranges_window_kernel(const RangeDesc* __restrict__ table, RangeDesc one, int nposb, int C) {
+  const RangeDesc d = table ? table[blockIdx.z] : one;
+  const int chunk = blockIdx.y;
+  if (chunk >= d.chunks) return;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pb = blockIdx.x % nposb, cg = blockIdx.x / nposb;
+  const int P = d.bH * d.bW;
+  const int p = pb * 64 + lane;
+  const bool pvalid = p < P;
+  const int w = p / d.bH, h = p - w * d.bH;
+  const int c0 = cg * kWinCG;
+  const int nc = min(kWinCG, C - c0);
+  const int j0 = 1 + chunk * d.cols_per_chunk;
+  const int j1 = min(d.n, (chunk + 1) * d.cols_per_chunk) + 1;
+  double s[kWinCG][4];
+#pragma unroll
+  for (int cc = 0; cc < kWinCG; ++cc)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) s[cc][a] = 0.0;
+  const double* base = d.V + p + (int64_t)P * c0;
+#pragma unroll 1
+  for (int jb = j0 + 8 * wave; jb < j1; jb += 64) {
+    // the wave's eight columns of this step: window tests first, then all their loads (four channels at a
+    // time) in flight together, then the sums column by column
+    bool in[8];
+    double pl[8], pu[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      in[u] = false;
+      pl[u] = pu[u] = 0.0;
+      if (jb + u < j1) {
+        const ColBox b = d.box[jb + u];
+        in[u] = pvalid && h >= b.h0 && h <= b.h1 && w >= b.w0 && w <= b.w1;
+        pl[u] = d.plb[jb + u - 1];
+        pu[u] = d.pub[jb + u - 1];
+      }
+    }
+#pragma unroll
+    for (int half = 0; half < kWinCG; half += 4) {
+      if (half >= nc) break;  // (uniform)
+      double v[8][4];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const double* col = base + (int64_t)(jb + u) * d.ld + (int64_t)P * half;
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) v[u][cc] = (in[u] && half + cc < nc) ? col[(int64_t)P * cc] : 0.0;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+          const double px = fmax(v[u][cc], 0.0), nx = fmin(v[u][cc], 0.0);
+          s[half + cc][0] = fma(px, pl[u], s[half + cc][0]);  // xmin1
+          s[half + cc][1] = fma(nx, pu[u], s[half + cc][1]);  // xmin2
+          s[half + cc][2] = fma(px, pu[u], s[half + cc][2]);  // xmax1
+          s[half + cc][3] = fma(nx, pl[u], s[half + cc][3]);  // xmax2
+        }
+    }
+  }
+  __shared__ double red[8][4][64];
+  const bool direct = d.chunks == 1 && d.chunks2 == 0 && d.part3 == nullptr;
+#pragma unroll
+  for (int cc = 0; cc < kWinCG; ++cc) {
+    if (cc < nc) {  // (uniform over the block)
+      if (wave > 0) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) red[wave][a][lane] = s[cc][a];
+      }
+      __syncthreads();
+      if (wave == 0 && pvalid) {
+        double t[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          t[a] = s[cc][a];
+          for (int w2 = 1; w2 < 8; ++w2) t[a] += red[w2][a][lane];
+        }
+        const int64_t r = p + (int64_t)P * (c0 + cc);
+        if (direct) {
+          const double c = d.V[r];
+          d.lb[r] = (c + t[0]) + t[1];
+          d.ub[r] = (c + t[2]) + t[3];
+        } else {
+          double* q = d.part + ((int64_t)chunk * 4) * d.ld + r;
+          q[0] = t[0];
+          q[d.ld] = t[1];
+          q[2 * d.ld] = t[2];
+          q[3 * d.ld] = t[3];
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // the padding rows behind the image: no generator reaches them
+  if (blockIdx.x == 0 && wave == 0) {
+    const int64_t r = (int64_t)P * C + lane;
+    if (r < d.ld) {
+      if (direct) {
+        d.lb[r] = d.ub[r] = d.V[r];
+      } else {
+        double* q = d.part + ((int64_t)chunk * 4) * d.ld + r;
+        q[0] = q[d.ld] = q[2 * d.ld] = q[3 * d.ld] = 0.0;
+      }
     }
   }
 }
@@ -609,6 +727,15 @@ int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, co
                      nullptr);
 }
 
+// Whether the range scan of a set reads its generator images inside their windows only: the windows must cover
+// every column the scan reads (all stored ones), describe this set's image, and be small next to it.
+static bool scan_in_windows(const nnvhip_star* t) {
+  if (t->box == nullptr || t->rows_pending || t->box_H <= 0 || t->box_W <= 0) return false;
+  const int64_t P = (int64_t)t->box_H * t->box_W;
+  if (t->N % P != 0 || t->box_cols < t->stored_cols()) return false;
+  return 2 * (int64_t)t->box_eh * t->box_ew <= P;
+}
+
 int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   // sets that already carry ranges are skipped
   std::vector<nnvhip_star*> todo;
@@ -616,13 +743,26 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   for (int64_t i = 0; i < count; ++i)
     if (!s[i]->lb && seen.insert(s[i]).second) todo.push_back(s[i]);
   if (todo.empty()) return NNVHIP_OK;
+  // Sets whose generator images are in memory inside their windows only are scanned inside the windows (all
+  // sets of the call, or none: one launch serves them all; the same sums to the bit either way).
+  bool in_windows = tune_knobs().ranges_row_waves == 0;
+  {
+    bool any_win = false;
+    for (auto* t : todo) {
+      in_windows = in_windows && scan_in_windows(t) && t->box_H == todo[0]->box_H && t->box_W == todo[0]->box_W && t->N == todo[0]->N;
+      any_win = any_win || t->cs.win_pending();
+    }
+    in_windows = in_windows && any_win;
+  }
   // The scan reads the columns the producer left no sums for.  Columns that are described but not in
   // memory yet are written first only if they are among those (they normally come with their sums).
   {
     std::vector<nnvhip_star*> cols;
     for (auto* t : todo) {
       const int64_t scan_end = (t->has_producer_sums() && t->rng_first_col >= 1) ? t->rng_first_col : t->n + 1;
-      if ((t->cs.pending && scan_end > t->cs.from) || (t->cs.zero_to > 1 && scan_end > 1)) cols.push_back(t);
+      // (columns that are in memory inside their windows only are fine for a scan that stays inside the windows)
+      const bool win = t->cs.win_pending() && scan_end > t->cs.win_from && !in_windows;
+      if ((t->cs.pending && scan_end > t->cs.from) || (t->cs.zero_to > 1 && scan_end > 1) || win) cols.push_back(t);
     }
     if (!cols.empty()) NNV_TRY(write_pending_columns(ctx, (int64_t)cols.size(), cols.data()));
   }
@@ -674,6 +814,13 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     d.cpart = nullptr;
     d.cbias = nullptr;
     d.cout = nullptr;
+    d.box = nullptr;
+    d.bH = d.bW = 0;
+    if (in_windows) {
+      d.box = t->box;
+      d.bH = t->box_H;
+      d.bW = t->box_W;
+    }
     if (t->has_producer_sums() && t->rng_first_col >= 1) {
       // the producer of the trailing columns left their sums: scan only the columns before them
       d.part2 = t->rng_chunks > 0 ? t->rng_part : nullptr;
@@ -701,7 +848,15 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   double bytes = 0.0;  // algorithmic: V once, the predicate bounds, lb/ub out
   for (int64_t i = 0; i < nset; ++i)
     bytes += 8.0 * (double)todo[i]->N * (double)(descs[i].n + 1) + 16.0 * (double)descs[i].n + 16.0 * (double)todo[i]->N;
-  if (scan) {
+  if (scan && in_windows) {
+    const int P = descs[0].bH * descs[0].bW;
+    const int C = (int)(todo[0]->N / P);
+    const int nposb = (int)ceil_div(P, 64);
+    NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
+    NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_window_kernel, dim3((unsigned)(nposb * ceil_div(C, kWinCG)), (unsigned)chunks, (unsigned)nset),
+               dim3(512), 0, table, descs[0], nposb, C);
+    NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
+  } else if (scan) {
     NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
     NNV_LAUNCH(ctx, ctx->kernel_timing, (ranges_partial_kernel<8, 4>), grid, dim3(64 * kRangeWaves), 0, table, descs[0]);
     NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
@@ -834,8 +989,51 @@ struct PendingCols {
   ColSource* cs;
 };
 
+// Writes the zeros outside the windows of the columns [j0, j1) of a matrix of N = H * W * C rows (the rows inside
+// a window hold values and are left alone).  Lane = one row, the waves of a block interleave columns.
+__global__ __launch_bounds__(512) void zero_outside_windows_kernel(double* __restrict__ V, int64_t ld, int64_t N,
+                                                                   const ColBox* __restrict__ box, int64_t j0, int64_t j1, int H,
+                                                                   int W, int cols_per_chunk) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t r = (int64_t)blockIdx.x * 64 + lane;
+  if (r >= N) return;
+  const int p = (int)(r % ((int64_t)H * W));
+  const int w = p / H, h = p - w * H;
+  const int64_t ja = j0 + (int64_t)blockIdx.y * cols_per_chunk;
+  const int64_t jb = min(j1, ja + cols_per_chunk);
+  for (int64_t j = ja + wave; j < jb; j += 8) {
+    const ColBox b = box[j];
+    if (!(h >= b.h0 && h <= b.h1 && w >= b.w0 && w <= b.w1)) V[r + j * ld] = 0.0;
+  }
+}
+
+static int write_window_zeros(nnvhip_ctx* ctx, double* V, int64_t ld, ColSource* cs) {
+  const int64_t ncols = cs->win_to - cs->win_from;
+  if (ncols > 0) {
+    const int64_t rows = cs->win_rows;  // (the padding rows up to ld are zero already)
+    const int64_t row_blocks = ceil_div(rows, 64);
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(8192, row_blocks), ceil_div(ncols, 32)));
+    const int64_t cpc = ceil_div(ncols, chunks);
+    chunks = ceil_div(ncols, cpc);
+    hipLaunchKernelGGL(zero_outside_windows_kernel, dim3((unsigned)row_blocks, (unsigned)chunks), dim3(512), 0, ctx->stream, V, ld, rows,
+                       cs->win_box, cs->win_from, cs->win_to, (int)cs->win_H, (int)cs->win_W, (int)cpc);
+    NNV_HIP_TRY(hipGetLastError());
+  }
+  cs->win_from = cs->win_to = 0;
+  return NNVHIP_OK;
+}
+
 // One gather launch per run of sets that share the weight matrix and the leading dimension.
 int write_cols(nnvhip_ctx* ctx, std::vector<PendingCols>& todo) {
+  {  // columns written inside their windows only: the zeros around them
+    std::vector<PendingCols> rest;
+    for (auto& t : todo) {
+      if (t.cs->win_pending()) NNV_TRY(write_window_zeros(ctx, t.V, t.ld, t.cs));
+      if (t.cs->any_pending()) rest.push_back(t);
+    }
+    todo.swap(rest);
+  }
   size_t a = 0;
   while (a < todo.size()) {
     size_t b = a + 1;
