@@ -31,6 +31,21 @@ static size_t size_class(size_t bytes) {
   return (bytes + step - 1) / step * step;
 }
 
+// Wt(r, k) = W(r, k): the Mp x Kp column-major weights row-major (ld = Kp), 32 x 32 tiles through LDS
+__global__ __launch_bounds__(256) void transpose_weights_kernel(const double* __restrict__ W, double* __restrict__ Wt, int Mp, int Kp) {
+  __shared__ double tile[32][33];
+  const int k0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  for (int i = threadIdx.y; i < 32; i += 8) {
+    const int k = k0 + i, r = r0 + threadIdx.x;
+    tile[i][threadIdx.x] = (k < Kp && r < Mp) ? W[r + (int64_t)k * Mp] : 0.0;
+  }
+  __syncthreads();
+  for (int i = threadIdx.y; i < 32; i += 8) {
+    const int r = r0 + i, k = k0 + threadIdx.x;
+    if (r < Mp && k < Kp) Wt[(int64_t)r * Kp + k] = tile[threadIdx.x][i];
+  }
+}
+
 const TuneKnobs& tune_knobs() {
   static const TuneKnobs knobs = [] {
     TuneKnobs k;
@@ -1703,6 +1718,21 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       }
     }
     // the gathered columns remember where they came from
+    // (arrays: the next layer packs kept rows of these columns, i.e. reads rows of W - from a row-major copy)
+    if (st == NNVHIP_OK && count >= 64 && !fc->Wt && fc->Mp * fc->Kp < (int64_t(1) << 31)) {
+      bool any = false;
+      for (int64_t i = 0; i < count; ++i) any = any || gs[i].m > 0;
+      if (any) {
+        BufRef wt;
+        st = c->alloc(sizeof(double) * fc->Mp * fc->Kp, &wt);
+        if (st == NNVHIP_OK) {
+          hipLaunchKernelGGL(transpose_weights_kernel, dim3((unsigned)ceil_div(fc->Kp, 32), (unsigned)ceil_div(fc->Mp, 32)), dim3(32, 8), 0,
+                             c->stream, Wd, wt->as<double>(), (int)fc->Mp, (int)fc->Kp);
+          if (hipGetLastError() != hipSuccess) st = NNVHIP_ERR_HIP;
+          fc->Wt = wt;
+        }
+      }
+    }
     for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
       if (gs[i].m > 0) {
         nnvhip_star* o = outs[i];
@@ -1711,6 +1741,11 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         cs.W = Wd;
         cs.ldw = fc->Mp;
         cs.rows = fc->Mp;
+        if (fc->Wt) {
+          cs.Wt_buf = fc->Wt;
+          cs.Wt = fc->Wt->as<double>();
+          cs.ldwt = fc->Kp;
+        }
         cs.idx_buf = in[i]->oh_idx_buf;
         cs.idx = gs[i].idx;
         cs.scale_buf = in[i]->oh_scale_buf;

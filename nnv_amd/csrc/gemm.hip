@@ -495,6 +495,9 @@ PackSet pack_of(const nnvhip_star* s, const int32_t* kept, double* dst, int64_t 
   if (cs.W != nullptr && cs.from < ncols) {
     p.W = cs.W;
     p.ldw = cs.ldw;
+    p.Wt = cs.Wt;
+    p.ldwt = cs.ldwt;
+    p.wrows = cs.rows;
     p.widx = cs.idx;
     p.wscale = cs.scale;
     p.wfrom = (int32_t)cs.from;

@@ -267,6 +267,78 @@ __global__ __launch_bounds__(256) void pack_rows_t_kernel(const PackSet* __restr
     for (int kk = wave; kk < 64 && t0 + kk < d.kp; kk += 4) d.Vk[(int64_t)(t0 + kk) * d.ldt + j] = tile[lane][kk];
 }
 
+// The same packing when every column but the centre is a scaled weight column and the weights are at hand
+// row-major: row t of Vt is a row of the weights, read and written contiguously.  The weights are larger than
+// an XCD's L2, so the grid walks them in slices of kPackSlice rows with the sets innermost (blockIdx.x = set):
+// while a slice is being read by every set it stays in the cache.  Block (set, slice) packs the kept rows of the
+// set that fall into the slice (the list is ascending; its -1 padding belongs to the last slice).
+constexpr int kPackSlice = 64;
+__global__ __launch_bounds__(256) void pack_rows_t_direct_kernel(const PackSet* __restrict__ table, PackSet one, int slices) {
+  const PackSet d = table ? table[blockIdx.x] : one;
+  const int lo_row = blockIdx.y * kPackSlice, hi_row = lo_row + kPackSlice;
+  // first entry >= lo_row and first entry >= hi_row among the real (non-negative, ascending) entries
+  int nreal = 0;
+  {
+    int a = 0, b = d.kp;  // first padding entry
+    while (a < b) {
+      const int m = (a + b) >> 1;
+      if (d.kept[m] >= 0) a = m + 1; else b = m;
+    }
+    nreal = a;
+  }
+  auto lower = [&](int row) {
+    int a = 0, b = nreal;
+    while (a < b) {
+      const int m = (a + b) >> 1;
+      if (d.kept[m] < row) a = m + 1; else b = m;
+    }
+    return a;
+  };
+  const int t0 = lower(lo_row);
+  const int t1 = (int)blockIdx.y == slices - 1 ? d.kp : lower(hi_row);
+  // a thread's columns (4 * tid .. 4 * tid + 3, then 1024 further on) and what they read do not depend on the
+  // row: weight column and scale are looked up once, the rows then stream out in 16-byte pieces
+  constexpr int kQ = 4;
+  for (int jb = 0; jb < d.ldt; jb += 256 * kQ) {
+    const int j0 = jb + kQ * (int)threadIdx.x;
+    int src[kQ];
+    double sc[kQ];
+    int kind[kQ];  // 0: zero, 1: the centre, 2: a weight column
+#pragma unroll
+    for (int e = 0; e < kQ; ++e) {
+      const int j = j0 + e;
+      src[e] = 0;
+      sc[e] = 0.0;
+      kind[e] = 0;
+      if (j < d.ncols) {
+        if (j == 0) {
+          kind[e] = 1;
+        } else if (j >= d.zero_to) {
+          kind[e] = 2;
+          src[e] = d.widx[j - d.wfrom];
+          sc[e] = d.wscale ? d.wscale[src[e]] : 1.0;
+        }
+      }
+    }
+    if (j0 >= d.ldt) continue;  // (ldt is a multiple of four)
+#pragma unroll 2
+    for (int t = t0; t < t1; ++t) {
+      const int ra = d.kept[t];
+      const double* wrow = d.Wt + (int64_t)max(ra, 0) * d.ldwt;
+      double* dst = d.Vk + (int64_t)t * d.ldt + j0;
+      double v[kQ];
+#pragma unroll
+      for (int e = 0; e < kQ; ++e) {
+        v[e] = 0.0;
+        if (ra >= 0 && kind[e] == 2) v[e] = __dadd_rn(0.0, __dmul_rn(wrow[src[e]], sc[e]));
+        if (ra >= 0 && kind[e] == 1) v[e] = d.V[ra];
+      }
+      *reinterpret_cast<double2_t*>(dst) = double2_t{v[0], v[1]};
+      *reinterpret_cast<double2_t*>(dst + 2) = double2_t{v[2], v[3]};
+    }
+  }
+}
+
 template <int TN, int WR, int WC, int FM, int FN>
 int launch_seg_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
                    const SegTile* segs, int64_t ntiles, double flop) {
@@ -300,6 +372,22 @@ int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {
   if (count > 1) {
     NNV_TRY(ctx->upload_table(sets, sizeof(PackSet) * count, &tab));
     table = tab->as<PackSet>();
+  }
+  // every column but the centre a scaled weight column, the weights at hand row-major, no windows: rows of the weights
+  bool direct = true;
+  int64_t wrows = 0;
+  for (int64_t i = 0; i < count; ++i) {
+    direct = direct && sets[i].Wt != nullptr && sets[i].wfrom == 1 && sets[i].wend >= sets[i].ncols && sets[i].box == nullptr &&
+             sets[i].ldt % 4 == 0;
+    wrows = std::max<int64_t>(wrows, sets[i].wrows);
+  }
+  direct = direct && wrows > 0 && ceil_div(wrows, kPackSlice) <= 65535;
+  if (direct) {
+    const int slices = (int)ceil_div(wrows, kPackSlice);
+    hipLaunchKernelGGL(pack_rows_t_direct_kernel, dim3((unsigned)count, (unsigned)slices), dim3(256), 0, ctx->stream, table, sets[0],
+                       slices);
+    NNV_HIP_TRY(hipGetLastError());
+    return NNVHIP_OK;
   }
   hipLaunchKernelGGL(pack_rows_t_kernel, dim3((unsigned)ceil_div(max_kp, 64), (unsigned)ceil_div(max_ld, 64), (unsigned)count), dim3(256),
                      0, ctx->stream, table, sets[0]);

@@ -101,7 +101,9 @@ struct ColBox {
 // them written first.  Writing them is idempotent, so every handle that shares the matrix keeps a copy
 // of this description with its own flags.  W == null: no such knowledge.
 struct ColSource {
-  BufRef W_buf, idx_buf, scale_buf;
+  BufRef W_buf, idx_buf, scale_buf, Wt_buf;
+  const double* Wt = nullptr;  // the same matrix row-major (row r at Wt + r * ldwt), or null
+  int64_t ldwt = 0;
   const double* W = nullptr;  // the layer's weight matrix: `rows` rows (a multiple of 16), leading dimension ldw
   int64_t ldw = 0;
   int64_t rows = 0;
@@ -378,6 +380,9 @@ struct nnvhip_fc {
   nnvhip::BufRef bias;  // Mp entries (zero padded) or null
   // [max(W, 0); min(W, 0)], 2*Mp x Kp with ld = 2*Mp: made on first use by launch_range_sums_mm
   mutable nnvhip::BufRef Wpn;
+  // the weights row-major (Mp rows of Kp entries), made on first use for arrays of sets: the next layer packs
+  // kept rows of columns that are scaled weight columns, i.e. reads rows of W
+  mutable nnvhip::BufRef Wt;
 };
 
 struct nnvhip_conv2d {
@@ -472,6 +477,9 @@ struct PackSet {
   // columns [wfrom, wend) are read as 0 + W(:, widx[j - wfrom]) * wscale[...] instead (W == null: none)
   const double* W = nullptr;
   int64_t ldw = 0;
+  const double* Wt = nullptr;  // W row-major (row r at Wt + r * ldwt), or null
+  int64_t ldwt = 0;
+  int64_t wrows = 0;           // rows of W
   const int32_t* widx = nullptr;
   const double* wscale = nullptr;
   int32_t wfrom = 0;

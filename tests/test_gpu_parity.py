@@ -730,7 +730,7 @@ def test_released_arrays_give_their_memory_back(nnv):
     opt = {"reachMethod": "relax-star-area", "relaxFactor": 1}
     lbs = rs.rand(n_in, count) - 0.5
     ubs = lbs + 0.2
-    net.reach(nnv.Star.from_boxes(lbs[:, :2], ubs[:, :2]), opt)   # the layers' weights are on the device now
+    net.reach(nnv.Star.from_boxes(lbs[:, :300], ubs[:, :300]), opt)   # the layers' weights (and what arrays derive from them) are on the device now
     net.reachSet = []
     ctx.synchronize()
     used0, _ = ctx.pool_stats()
