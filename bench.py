@@ -49,7 +49,7 @@ MIN_WARM_SECONDS = 0.3
 GROUP_KERNELS = {
     "gemm_f64_kernel": ("gemm_f64_kernel", "gemm_seg_kernel"),
     "conv2d_fast_kernel": ("conv2d_fast_kernel", "conv2d_f64_kernel"),
-    "gather_columns_kernel": ("gather_columns_kernel", "fc_rowsum_kernel", "conv_stamp_kernel", "conv_stamp_rows_kernel"),
+    "gather_columns_kernel": ("gather_columns_kernel", "gather_skinny_kernel", "fc_rowsum_kernel", "conv_stamp_kernel", "conv_stamp_rows_kernel"),
     "ranges_partial_kernel": ("ranges_partial_kernel", "ranges_window_kernel"),
     "relu_classify_kernel": ("relu_classify_kernel", "relu_count_kernel", "relu_compact_kernel"),
 }

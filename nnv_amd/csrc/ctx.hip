@@ -1228,7 +1228,31 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
   bool contig = false;
   int64_t cols = 0;
   NNV_TRY(c->begin_op());
-  int st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
+  // A large array whose gathered columns will stay unwritten gets their range sums from one matrix product
+  // (see below).  Nothing of it depends on the outputs, so it is queued before anything else: the device
+  // works on it while the host sets up the outputs and the tiles of the contraction.
+  BufRef mm_early;
+  int st = NNVHIP_OK;
+  if (count >= 64 && !c->eager_cols && !c->dense_affine) {
+    std::vector<GatherSet> es((size_t)count);
+    bool ok = true, any = false;
+    for (int64_t i = 0; i < count; ++i) {
+      const int64_t nc = in[i]->n + 1;
+      int64_t d = (in[i]->oh_from > 0 && in[i]->oh_from < nc) ? in[i]->oh_from : nc;
+      if ((double)fc->Mp * (double)fc->Kp * (double)(nc - d) * (double)count < 4.0e6) d = nc;
+      GatherSet& g = es[i];
+      g = GatherSet{};
+      g.idx = in[i]->oh_idx;
+      g.scale = in[i]->oh_scale;
+      g.plb = in[i]->plb + (d - 1);  // the output shares the input's predicate bounds
+      g.pub = in[i]->pub + (d - 1);
+      g.m = (int32_t)(nc - d);
+      ok = ok && !(g.m > 0 && in[i]->oh_scale_neg);
+      any = any || g.m > 0;
+    }
+    if (ok && any) st = launch_range_sums_mm(c, fc, count, es.data(), &mm_early);
+  }
+  if (st == NNVHIP_OK) st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
   if (st == NNVHIP_OK) {
     for (int64_t i = 0; i < count; ++i) outs[i]->has_zono = in[i]->has_zono;  // Z.affineMap(W, b), set/Star.m:332-340
     const double* bias = fc->bias ? fc->bias->as<double>() : nullptr;
@@ -1664,7 +1688,10 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           for (int64_t i = 0; i < count; ++i) chunk_off[i + 1] = chunk_off[i] + (gs[i].m > 0 ? gch_part : 0);
           if (chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
         }
-        if (st == NNVHIP_OK && use_mm) st = launch_range_sums_mm(c, fc, count, gs.data(), &mm_sums);
+        if (st == NNVHIP_OK && use_mm) {
+          if (mm_early) mm_sums = mm_early;  // queued at the start of the call, from the same lists
+          else st = launch_range_sums_mm(c, fc, count, gs.data(), &mm_sums);
+        }
         if (st == NNVHIP_OK) {
           for (int64_t i = 0; i < count; ++i) {
             gs[i].part = (gch_part > 0 && gs[i].m > 0) ? sums->as<double>() + 4 * ldo * (chunk_off[i] + tiles_of[i]) : nullptr;

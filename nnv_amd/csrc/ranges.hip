@@ -236,78 +236,128 @@ __global__ __launch_bounds__(512) void ranges_window_kernel(const RangeDesc* __r
   }
 }
 
-// Combines the chunk partials in chunk order.  64 rows per block; the four sums of a row are handled
-// by four different waves so that the dependent add chains are short.
+// R consecutive rows (R = 1 or 2) from 8 * R-byte aligned memory
+template <int R>
+__device__ __forceinline__ void load_rows(const double* __restrict__ p, double (&v)[R]) {
+  if constexpr (R == 2) {
+    const double2 t = *reinterpret_cast<const double2*>(p);
+    v[0] = t.x;
+    v[1] = t.y;
+  } else {
+    v[0] = p[0];
+  }
+}
+
+// Combines the chunk partials in chunk order.  64 * R rows per block (every lane owns R consecutive rows: with
+// R = 2 the partials are read 16 bytes at a time, which is what an array of many sets wants; a single set gets
+// more blocks out of R = 1); the four sums of a row are handled by four different waves so that the dependent
+// add chains are short.
+template <int R>
 __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
   if (d.chunks == 1 && d.chunks2 == 0 && d.part3 == nullptr && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
   const int lane = threadIdx.x & 63;
   const int q = threadIdx.x >> 6;
-  const int64_t r = (int64_t)blockIdx.x * 64 + lane;
-  __shared__ double sums[4][64];
-  __shared__ double cen[64];
+  const int64_t r = ((int64_t)blockIdx.x * 64 + lane) * R;
+  __shared__ double sums[4][64 * R];
+  __shared__ double cen[64 * R];
   if (q == 4) {  // a wave of its own (the launch that has a centre to form brings five)
     if (d.cchunks > 0 && r < d.ld) {
-      double c0 = 0.0;
-      for (int c = 0; c < d.cchunks; c += 32) {
-        double v[32];
 #pragma unroll
-        for (int u = 0; u < 32; ++u) v[u] = c + u < d.cchunks ? d.cpart[(int64_t)(c + u) * d.ld + r] : 0.0;
+      for (int e = 0; e < R; ++e) {
+        double c0 = 0.0;
+        for (int c = 0; c < d.cchunks; c += 32) {
+          double v[32];
 #pragma unroll
-        for (int u = 0; u < 32; ++u)
-          if (c + u < d.cchunks) c0 += v[u];
+          for (int u = 0; u < 32; ++u) v[u] = c + u < d.cchunks ? d.cpart[(int64_t)(c + u) * d.ld + r + e] : 0.0;
+#pragma unroll
+          for (int u = 0; u < 32; ++u)
+            if (c + u < d.cchunks) c0 += v[u];
+        }
+        if (d.cbias != nullptr) c0 = c0 + d.cbias[r + e];
+        d.cout[r + e] = c0;
+        cen[lane * R + e] = c0;
       }
-      if (d.cbias != nullptr) c0 = c0 + d.cbias[r];
-      d.cout[r] = c0;
-      cen[lane] = c0;
     }
     __syncthreads();
     return;
   }
-  double s = 0.0;
+  double s[R];
+#pragma unroll
+  for (int e = 0; e < R; ++e) s[e] = 0.0;
   if (r < d.ld) {
     // the partial sums were written by other CUs moments ago: every load is a trip to memory, so as many
     // as possible are in flight at once; the additions stay in chunk order
     const double* p = d.part + (int64_t)q * d.ld + r;
     int c = 0;
     if (d.chunks <= 8) {  // the common case after a fused GEMM epilogue: one short batch
-      double v[8];
+      double v[8][R];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = u < d.chunks ? p[(int64_t)u * 4 * d.ld] : 0.0;
+      for (int u = 0; u < 8; ++u) {
+#pragma unroll
+        for (int e = 0; e < R; ++e) v[u][e] = 0.0;
+        if (u < d.chunks) load_rows<R>(p + (int64_t)u * 4 * d.ld, v[u]);
+      }
 #pragma unroll
       for (int u = 0; u < 8; ++u)
-        if (u < d.chunks) s += v[u];
+        if (u < d.chunks) {
+#pragma unroll
+          for (int e = 0; e < R; ++e) s[e] += v[u][e];
+        }
       c = d.chunks;
     }
-    for (; c + 32 <= d.chunks; c += 32) {
-      double v[32];
+    constexpr int kBatch = 32 / R;
+    for (; c < d.chunks; c += kBatch) {
+      double v[kBatch][R];
 #pragma unroll
-      for (int u = 0; u < 32; ++u) v[u] = p[(int64_t)(c + u) * 4 * d.ld];
+      for (int u = 0; u < kBatch; ++u) {
 #pragma unroll
-      for (int u = 0; u < 32; ++u) s += v[u];
-    }
-    if (c < d.chunks) {
-      double v[32];
+        for (int e = 0; e < R; ++e) v[u][e] = 0.0;
+        if (c + u < d.chunks) load_rows<R>(p + (int64_t)(c + u) * 4 * d.ld, v[u]);
+      }
 #pragma unroll
-      for (int u = 0; u < 32; ++u) v[u] = c + u < d.chunks ? p[(int64_t)(c + u) * 4 * d.ld] : 0.0;
+      for (int u = 0; u < kBatch; ++u)
+        if (c + u < d.chunks) {
 #pragma unroll
-      for (int u = 0; u < 32; ++u)
-        if (c + u < d.chunks) s += v[u];
+          for (int e = 0; e < R; ++e) s[e] += v[u][e];
+        }
     }
     if (d.chunks2 > 0) {
       const double* p2 = d.part2 + (int64_t)q * d.ld + r;
-#pragma unroll 8
-      for (int c2 = 0; c2 < d.chunks2; ++c2) s += p2[(int64_t)c2 * 4 * d.ld];
+      for (int c2 = 0; c2 < d.chunks2; c2 += 8) {
+        double v[8][R];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+#pragma unroll
+          for (int e = 0; e < R; ++e) v[u][e] = 0.0;
+          if (c2 + u < d.chunks2) load_rows<R>(p2 + (int64_t)(c2 + u) * 4 * d.ld, v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (c2 + u < d.chunks2) {
+#pragma unroll
+            for (int e = 0; e < R; ++e) s[e] += v[u][e];
+          }
+      }
     }
     // xmin1, xmin2, xmax1, xmax2 sit in blocks 0, 3, 2, 1 of the product's two columns
-    if (d.part3 != nullptr) s += d.part3[(int64_t)((4 - q) & 3) * d.ld + r];
+    if (d.part3 != nullptr) {
+      double v[R];
+      load_rows<R>(d.part3 + (int64_t)((4 - q) & 3) * d.ld + r, v);
+#pragma unroll
+      for (int e = 0; e < R; ++e) s[e] += v[e];
+    }
   }
-  sums[q][lane] = s;
+#pragma unroll
+  for (int e = 0; e < R; ++e) sums[q][lane * R + e] = s[e];
   __syncthreads();
   if (q == 0 && r < d.ld) {
-    const double c0 = d.cchunks > 0 ? cen[lane] : d.V[r];
-    d.lb[r] = (c0 + sums[0][lane]) + sums[1][lane];
-    d.ub[r] = (c0 + sums[2][lane]) + sums[3][lane];
+#pragma unroll
+    for (int e = 0; e < R; ++e) {
+      const double c0 = d.cchunks > 0 ? cen[lane * R + e] : d.V[r + e];
+      d.lb[r + e] = (c0 + sums[0][lane * R + e]) + sums[1][lane * R + e];
+      d.ub[r + e] = (c0 + sums[2][lane * R + e]) + sums[3][lane * R + e];
+    }
   }
 }
 
@@ -451,6 +501,102 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   }
 }
 
+// The same pass for outputs of at most 32 rows (the last layer of a classifier): with one lane per two rows only
+// 8 or 16 lanes of a wave would have rows, so a wave takes 64 / HL columns at once instead (HL = ldout / 2 lanes
+// per column; a wave writes 1 KiB of consecutive columns per step).  Columns and, with part != null, their four
+// range sums, and filled leading columns; nothing else (no split-K centre, no centre product, no unwritten columns).
+template <int HL>
+__global__ __launch_bounds__(256) void gather_skinny_kernel(const GatherSet* __restrict__ table, GatherSet one, GatherArgs a) {
+  constexpr int CPW = 64 / HL;  // columns per wave and step
+  const GatherSet d = table ? table[blockIdx.z] : one;
+  const int chunk = blockIdx.y;
+  const int j0 = chunk * a.cols_per_chunk;
+  double* part = a.with_sums ? d.part : nullptr;
+  if (j0 >= d.m && part == nullptr && d.nfill == 0) return;
+  const int j1 = min(d.m, j0 + a.cols_per_chunk);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r0 = 2 * (lane % HL), cs = lane / HL;
+  // leading columns a contraction over no rows would have left: the bias on the centre, +0 elsewhere
+  if (d.nfill > 0) {
+    const int fpc = (d.nfill + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int f1 = min(d.nfill, (chunk + 1) * fpc);
+    for (int j = chunk * fpc + wave * CPW + cs; j < f1; j += 4 * CPW) {
+      double2 o = make_double2(0.0, 0.0);
+      if (j == 0 && d.bias != nullptr && r0 < a.Mp) {
+        o.x = __dadd_rn(0.0, d.bias[r0]);
+        o.y = __dadd_rn(0.0, d.bias[r0 + 1]);
+      }
+      *reinterpret_cast<double2*>(d.fill + r0 + (int64_t)j * a.ldout) = o;
+    }
+  }
+  double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
+  for (int jb = j0 + wave * CPW + cs; jb < j1; jb += 4 * 4 * CPW) {
+    double2 v[4];
+    double sc[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = jb + u * 4 * CPW;
+      v[u] = make_double2(0.0, 0.0);
+      sc[u] = 1.0;
+      if (j < j1) {
+        const int src = d.idx[j];
+        if (d.scale != nullptr) sc[u] = d.scale[src];
+        v[u] = *reinterpret_cast<const double2*>(a.W + r0 + (int64_t)src * a.ldw);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = jb + u * 4 * CPW;
+      if (j >= j1) break;
+      double2 o;
+      o.x = __dadd_rn(0.0, __dmul_rn(v[u].x, sc[u]));
+      o.y = __dadd_rn(0.0, __dmul_rn(v[u].y, sc[u]));
+      *reinterpret_cast<double2*>(d.out + r0 + (int64_t)j * a.ldout) = o;
+      if (part != nullptr) {
+        const double pl = d.plb[j], pu = d.pub[j];
+        const double px = fmax(o.x, 0.0), nx = fmin(o.x, 0.0);
+        const double py = fmax(o.y, 0.0), ny = fmin(o.y, 0.0);
+        xmin1.x = fma(px, pl, xmin1.x);
+        xmin1.y = fma(py, pl, xmin1.y);
+        xmax1.x = fma(px, pu, xmax1.x);
+        xmax1.y = fma(py, pu, xmax1.y);
+        xmin2.x = fma(nx, pu, xmin2.x);
+        xmin2.y = fma(ny, pu, xmin2.y);
+        xmax2.x = fma(nx, pl, xmax2.x);
+        xmax2.y = fma(ny, pl, xmax2.y);
+      }
+    }
+  }
+  if (part == nullptr) return;
+  // the column slots of a wave are added pairwise (always the same tree), the waves then in wave order
+  double2* acc[4] = {&xmin1, &xmin2, &xmax1, &xmax2};
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int mask = HL; mask < 64; mask *= 2) {
+      acc[k]->x += __shfl_xor(acc[k]->x, mask);
+      acc[k]->y += __shfl_xor(acc[k]->y, mask);
+    }
+  __shared__ double2 red[3][4][HL];
+  if (wave > 0 && cs == 0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) red[wave - 1][k][lane] = *acc[k];
+  }
+  __syncthreads();
+  if (wave == 0 && cs == 0) {
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        acc[k]->x += red[w][k][lane].x;
+        acc[k]->y += red[w][k][lane].y;
+      }
+    double* q = part + ((int64_t)chunk * 4) * a.ldout + r0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) *reinterpret_cast<double2*>(q + k * a.ldout) = *acc[k];
+  }
+}
+
 // Column chunks of a gather over `count` sets with at most max_m one-hot columns each.
 int64_t gather_chunks_batch(int64_t ldout, int64_t count, int64_t max_m) {
   if (max_m <= 0) return 0;
@@ -504,7 +650,16 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
   bool centre = false;
   for (int64_t i = 0; i < count; ++i) centre = centre || sets[i].cin != nullptr;
-  if (centre)
+  // a skinny output whose columns are all written and that asks for nothing but columns and their sums
+  bool skinny = (ldout == 16 || ldout == 32) && !centre && !any_red;
+  for (int64_t i = 0; i < count && skinny; ++i) skinny = !sets[i].lazy;
+  if (skinny) {
+    const dim3 grid(1, (unsigned)chunks, (unsigned)count);
+    if (ldout == 16)
+      NNV_LAUNCH(ctx, ctx->kernel_timing, gather_skinny_kernel<8>, grid, dim3(256), 0, table, sets[0], a);
+    else
+      NNV_LAUNCH(ctx, ctx->kernel_timing, gather_skinny_kernel<16>, grid, dim3(256), 0, table, sets[0], a);
+  } else if (centre)
     NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel<true>, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
                dim3(64 * kRangeWaves), 0, table, sets[0], a);
   else
@@ -864,8 +1019,18 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   if (chunks > 1 || any_pending) {
     double fbytes = 0.0;  // every chunk's four sums read, lb and ub written
     for (int64_t i = 0; i < nset; ++i) fbytes += 8.0 * (double)ld * (4.0 * (double)(descs[i].chunks + descs[i].chunks2) + 3.0);
-    NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,
-               table, descs[0]);
+    // an array of sets has blocks to spare: two rows per lane, read 16 bytes at a time
+    bool wide = ceil_div(ld, 64) * nset >= 4096;
+    auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    for (int64_t i = 0; i < nset && wide; ++i)
+      wide = aligned16(descs[i].part) && aligned16(descs[i].part2) && aligned16(descs[i].part3) && aligned16(descs[i].V) &&
+             aligned16(descs[i].lb);
+    if (wide)
+      NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel<2>, dim3((unsigned)ceil_div(ld, 128), 1, (unsigned)nset), dim3(256), 0,
+                 table, descs[0]);
+    else
+      NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel<1>, dim3((unsigned)ceil_div(ld, 64), 1, (unsigned)nset), dim3(256), 0,
+                 table, descs[0]);
     NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 7, fbytes));
   }
   NNV_HIP_TRY(hipGetLastError());
@@ -906,7 +1071,7 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
   d.cpart = cpart;
   d.cbias = cbias;
   d.cout = s->V;
-  NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel, dim3((unsigned)ceil_div(s->ld, 64), 1, 1),
+  NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel<1>, dim3((unsigned)ceil_div(s->ld, 64), 1, 1),
              dim3(cchunks > 0 ? 320 : 256), 0, nullptr, d);
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 7, 8.0 * (double)s->ld * (4.0 * (double)chunks + 3.0)));
   NNV_HIP_TRY(hipGetLastError());
@@ -974,7 +1139,7 @@ int ranges_into_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, do
   hipLaunchKernelGGL((ranges_partial_kernel<8, 4>), dim3((unsigned)row_blocks, (unsigned)chunks, 1), dim3(64 * kRangeWaves), 0,
                      ctx->stream, nullptr, d);
   if (chunks > 1)
-    hipLaunchKernelGGL(ranges_final_kernel, dim3((unsigned)ceil_div(ld, 64), 1, 1), dim3(256), 0, ctx->stream, nullptr, d);
+    hipLaunchKernelGGL(ranges_final_kernel<1>, dim3((unsigned)ceil_div(ld, 64), 1, 1), dim3(256), 0, ctx->stream, nullptr, d);
   hipLaunchKernelGGL(copy_ranges_kernel, dim3((unsigned)ceil_div(s->N, 256)), dim3(256), 0, ctx->stream, d.lb, d.ub, lb_dev, ub_dev,
                      s->N);
   NNV_HIP_TRY(hipGetLastError());

@@ -35,11 +35,36 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   static_assert(sizeof(double) == sizeof(long long), "keys are sorted through their bit patterns");
   int base = 0, inact_total = 0, keep_base = 0;
   int32_t* idx_out = d.order == NNVHIP_ORDER_INDEX ? d.cross_idx : d.asc_idx;
+  // the first 1024 ranges are asked for before anything else ...
+  const double l_first = tid < d.N ? d.lb[tid] : 0.0;
+  const double u_first = tid < d.N ? d.ub[tid] : 1.0;
+  // ... and while they travel, the bounds of the predicates the set already has are copied (new_pred_lb =
+  // [plb; ...], new_pred_ub = [pub; ...]): nothing of that depends on the classification
+  if (d.write_bounds) {
+    const int n_in = d.ncols_in - 1;
+    for (int jb = tid; jb < n_in; jb += 4096) {
+      double a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = jb + u * 1024;
+        a[u] = j < n_in ? d.plb_in[j] : 0.0;
+        b[u] = j < n_in ? d.pub_in[j] : 0.0;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int j = jb + u * 1024;
+        if (j < n_in) {
+          d.plb_out[j] = a[u];
+          d.pub_out[j] = b[u];
+        }
+      }
+    }
+  }
   for (int r0 = 0; r0 < d.N; r0 += 1024) {
     const int r = r0 + tid;
     const bool valid = r < d.N;
-    const double l = valid ? d.lb[r] : 0.0;
-    const double u = valid ? d.ub[r] : 1.0;
+    const double l = r0 == 0 ? l_first : valid ? d.lb[r] : 0.0;
+    const double u = r0 == 0 ? u_first : valid ? d.ub[r] : 1.0;
     const bool inactive = valid && (u <= 0.0);              // map1 = find(ub <= 0)
     const bool crossing = valid && (l < 0.0) && (u > 0.0);  // map2 = find(lb < 0 & ub > 0)
     const bool kept = valid && !inactive && !crossing;
@@ -108,39 +133,45 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
     d.counts[1] = inact_total;
     post_counts(d.mailbox, m, inact_total, d.mailbox_seq);  // the host can size the output while we sort
   }
+  int mine = 0;  // entry tid of the sorted list
   if (sort_here)  // the staged doubles are read back as their bit patterns
-    sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
-  if (d.write_bounds && order_known) {  // the output buffers were sized for the worst case: finish the set here
+    mine = sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
+  if (d.write_bounds && sort_here) {
+    // the output buffers were sized for the worst case: finish the set here.  New predicate tid belongs to the
+    // neuron this thread holds: new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]
+    if (tid < m) {
+      const int n_in = d.ncols_in - 1;
+      const double b = d.ub[mine], c = d.lb[mine];
+      d.plb_out[n_in + tid] = 0.0;
+      d.pub_out[n_in + tid] = b;
+      d.lbub[tid] = c;
+      d.lbub[d.ld_lbub + tid] = b;
+    }
+  } else if (d.write_bounds && order_known) {
     __syncthreads();     // cross_idx is complete
     const int n_in = d.ncols_in - 1;
-    const int n_out = n_in + m;
-    // four entries per thread and step, all loads issued before the first store (the dependent
-    // index -> bound look-ups of the new predicates would otherwise queue up behind one another)
-    for (int jb = tid; jb < n_out; jb += 4096) {
-      double a[4], b[4], c[4];
+    // the new predicates, four per thread and step, all loads issued before the first store (the dependent
+    // index -> bound look-ups would otherwise queue up behind one another)
+    for (int ib = tid; ib < m; ib += 4096) {
+      double b[4], c[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int j = jb + u * 1024;
-        a[u] = b[u] = c[u] = 0.0;
-        if (j < n_in) {
-          a[u] = d.plb_in[j];
-          b[u] = d.pub_in[j];
-        } else if (j < n_out) {
-          const int neuron = d.cross_idx[j - n_in];
+        const int i = ib + u * 1024;
+        b[u] = c[u] = 0.0;
+        if (i < m) {
+          const int neuron = d.cross_idx[i];
           b[u] = d.ub[neuron];
           c[u] = d.lb[neuron];
         }
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int j = jb + u * 1024;
-        if (j >= n_out) break;
-        d.plb_out[j] = a[u];  // new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]
-        d.pub_out[j] = b[u];
-        if (j >= n_in) {
-          d.lbub[j - n_in] = c[u];
-          d.lbub[d.ld_lbub + (j - n_in)] = b[u];
-        }
+        const int i = ib + u * 1024;
+        if (i >= m) break;
+        d.plb_out[n_in + i] = 0.0;  // new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]
+        d.pub_out[n_in + i] = b[u];
+        d.lbub[i] = c[u];
+        d.lbub[d.ld_lbub + i] = b[u];
       }
     }
   }

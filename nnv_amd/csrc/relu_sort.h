@@ -142,8 +142,9 @@ __device__ __forceinline__ void sort_merges(long long& key, int& idx, long long*
 }
 
 // Sorts m <= 1024 (key bits, neuron) pairs staged in skey/sidx[0..m) and writes the neuron indices
-// in sorted order to out[0..m).  All 1024 threads of the block must call it.
-__device__ __forceinline__ void sort_small_desc(long long* skey, int* sidx, int m, int tid, int32_t* __restrict__ out) {
+// in sorted order to out[0..m).  All 1024 threads of the block must call it; thread t < m gets back entry t of
+// the sorted list.
+__device__ __forceinline__ int sort_small_desc(long long* skey, int* sidx, int m, int tid, int32_t* __restrict__ out) {
   long long key = tid < m ? skey[tid] : (long long)0x8000000000000000ull;
   int idx = tid < m ? sidx[tid] : 0x7fffffff;
   if (m <= 64) sort_merges<64, 2>(key, idx, skey, sidx, tid);
@@ -152,6 +153,7 @@ __device__ __forceinline__ void sort_small_desc(long long* skey, int* sidx, int 
   else if (m <= 512) sort_merges<512, 2>(key, idx, skey, sidx, tid);
   else sort_merges<1024, 2>(key, idx, skey, sidx, tid);
   if (tid < m) out[tid] = idx;
+  return idx;
 }
 
 // Entry j of the output's predicate bounds, new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]
