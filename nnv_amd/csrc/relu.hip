@@ -104,7 +104,6 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
         if (SORT_CAP > kSortInBlock) {
           idx_out[pos] = r;
           d.key[pos] = key;
-          d.rank[pos] = 0;
         }
         if (SORT_CAP > 0 && pos < kSortInBlock) {
           skey[pos] = key;
@@ -282,7 +281,6 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
     d.cls[r] = pos;
     if (d.order != NNVHIP_ORDER_INDEX) {
       d.key[pos] = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : d.order == NNVHIP_ORDER_RANGE ? u - l : d.given_key[r];
-      d.rank[pos] = 0;
     }
   } else if (valid) {
     d.cls[r] = inactive ? kZero : kKeep;
@@ -304,41 +302,61 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
 
 // Stable descending sort by counting: rank(i) = #{j : key_j > key_i or (key_j == key_i and j < i)}.
 // j < i in the ascending list is "smaller neuron index", which is what MATLAB's stable sort keeps.
-// The m x m comparison grid is cut into 256 x 256 tiles, one block each; partial counts are added
-// with integer atomics (exact, order-independent).
-__global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+// A block owns kRankI entries of the list and compares them with the whole list, staged through LDS in pieces of
+// kRankStage keys: thread (entry, slice) counts over every 16th key, the 16 slices of an entry are then added.
+// No block needs anything from another one (the XCDs of this chip share no cache, so counters and atomics
+// between blocks are the expensive part of a tiled count), and a block knows the final places of its entries:
+// it puts their neurons there and, with kRankNewBounds, writes what the new predicates need (new_pred_lb =
+// [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)], and the crossing neurons' (lb, ub)).  kRankOldBounds: the
+// blocks also share out the copy of the bounds of the predicates the set already has.
+constexpr int kRankI = 16;
+constexpr int kRankStage = 2048;
+constexpr int kRankNewBounds = 1, kRankOldBounds = 2;
+__global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restrict__ table, ReluDesc one, int flags) {
   const ReluDesc d = table ? table[blockIdx.z] : one;
   const int m = d.m;
-  const int i0 = blockIdx.x * 256, j0 = blockIdx.y * 256;
-  if (i0 >= m || j0 >= m) return;
-  const int i = i0 + threadIdx.x;
-  const double ki = i < m ? d.key[i] : 0.0;
-  __shared__ double tile[256];
-  const int j = j0 + threadIdx.x;
-  tile[threadIdx.x] = j < m ? d.key[j] : 0.0;
-  __syncthreads();
-  const int lim = min(256, m - j0);
-  int cnt = 0;
-  if (lim == 256) {
-#pragma unroll 8
-    for (int t = 0; t < 256; ++t) {
-      const double kj = tile[t];
-      cnt += (kj > ki || (kj == ki && (j0 + t) < i)) ? 1 : 0;
-    }
-  } else {
-    for (int t = 0; t < lim; ++t) {
-      const double kj = tile[t];
-      cnt += (kj > ki || (kj == ki && (j0 + t) < i)) ? 1 : 0;
+  const int tid = threadIdx.x;
+  const int n_in = d.ncols_in - 1;
+  if (flags & kRankOldBounds) {
+    for (int j = blockIdx.x * 256 + tid; j < n_in; j += gridDim.x * 256) {
+      d.plb_out[j] = d.plb_in[j];
+      d.pub_out[j] = d.pub_in[j];
     }
   }
-  if (i < m && cnt) atomicAdd(&d.rank[i], cnt);
-}
-
-__global__ __launch_bounds__(256) void relu_scatter_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
-  const ReluDesc d = table ? table[blockIdx.z] : one;
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= d.m) return;
-  d.cross_idx[d.rank[i]] = d.asc_idx[i];
+  const int i0 = blockIdx.x * kRankI;
+  if (i0 >= m) return;
+  const int il = tid & (kRankI - 1), slice = tid / kRankI;  // 256 / kRankI = 16 slices
+  const int i = i0 + il;
+  const double ki = i < m ? d.key[i] : 0.0;
+  __shared__ double keys[kRankStage];
+  __shared__ int part[16][kRankI];
+  int cnt = 0;
+  for (int base = 0; base < m; base += kRankStage) {
+    const int n = min(kRankStage, m - base);
+    if (base > 0) __syncthreads();  // everybody is done with the previous piece
+    for (int t = tid; t < n; t += 256) keys[t] = d.key[base + t];
+    __syncthreads();
+#pragma unroll 8
+    for (int t = slice; t < n; t += 16) {
+      const double kj = keys[t];
+      cnt += (kj > ki || (kj == ki && (base + t) < i)) ? 1 : 0;
+    }
+  }
+  part[slice][il] = cnt;
+  __syncthreads();
+  if (slice != 0 || i >= m) return;
+  int r = 0;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) r += part[q][il];
+  const int neuron = d.asc_idx[i];
+  d.cross_idx[r] = neuron;
+  if (flags & kRankNewBounds) {
+    const double ub = d.ub[neuron];
+    d.plb_out[n_in + r] = 0.0;
+    d.pub_out[n_in + r] = ub;
+    d.lbub[r] = d.lb[neuron];
+    d.lbub[d.ld_lbub + r] = ub;
+  }
 }
 
 constexpr int kApplyRows = 128;  // 64 lanes x 2 rows, the four waves interleave columns
@@ -591,7 +609,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const bool sorted = order != NNVHIP_ORDER_INDEX;
 
   // scratch shared by all sets: cls | counts ; cross_idx is kept (it becomes the node's index list)
-  BufRef cls_buf, cnt_buf, asc_buf, key_buf, rank_buf, blk_buf;
+  BufRef cls_buf, cnt_buf, asc_buf, key_buf, blk_buf;
   const int64_t nblk = ceil_div(N, 1024);
   NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &cls_buf));
   NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * count, &cnt_buf));
@@ -604,7 +622,6 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   if (sorted) {
     NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &asc_buf));
     NNV_TRY(ctx->alloc(sizeof(double) * ld * count, &key_buf));
-    NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &rank_buf));
   }
   // With the reset pending, all that is left to write are the predicate bounds and the crossing
   // neurons' (lb, ub).  The one-block classification does that itself, into buffers sized for the worst
@@ -647,7 +664,6 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.cross_idx = idx_buf->as<int32_t>() + ld * i;
     d.asc_idx = sorted ? asc_buf->as<int32_t>() + ld * i : nullptr;
     d.key = sorted ? key_buf->as<double>() + ld * i : nullptr;
-    d.rank = sorted ? rank_buf->as<int32_t>() + ld * i : nullptr;
     d.counts = cnt_buf->as<int32_t>() + 2 * i;
     d.blk_counts = blk_buf ? blk_buf->as<int32_t>() + 3 * nblk * i : nullptr;
     d.keep_idx = keep_buf->as<int32_t>() + keep_ld * i;
@@ -827,19 +843,25 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   }
   // lists the classification block left unsorted (and, with them, bounds it left unwritten)
   const bool need_rank = sorted && sort_cap > 0 && max_m > sort_cap;
+  // lists too long for any in-LDS sort go to the rank kernel
+  const bool rank_lists = sorted && max_m > sort_cap && !(sort_cap == 0 && max_m <= 1024);
+  bool ranked_with_bounds = false;
   if (count > 1 && (!fold_bounds || need_rank)) {
     NNV_TRY(ctx->upload_table(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
   if (sorted && sort_cap == 0 && max_m > 0 && max_m <= 1024) {
     hipLaunchKernelGGL(relu_sort_small_kernel, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
-  } else if (sorted && max_m > sort_cap) {  // lists too long for the in-LDS sort: rank every list
-    const unsigned t = (unsigned)ceil_div(max_m, 256);
-    if (t > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "too many crossing neurons for the sort kernel");
-    hipLaunchKernelGGL(relu_rank_kernel, dim3(t, t, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
-    hipLaunchKernelGGL(relu_scatter_kernel, dim3(t, 1, (unsigned)count), dim3(256), 0, ctx->stream, table, descs[0]);
+  } else if (rank_lists) {
+
+    // with the reset pending the kernel also writes the predicate bounds (the old ones were copied by the
+    // one-block classification where that ran with the output buffers in place)
+    ranked_with_bounds = lazy_rows;
+    const int flags = lazy_rows ? (kRankNewBounds | (fold_bounds ? 0 : kRankOldBounds)) : 0;
+    hipLaunchKernelGGL(relu_rank_kernel, dim3((unsigned)ceil_div(max_m, kRankI), 1, (unsigned)count), dim3(256), 0, ctx->stream, table,
+                       descs[0], flags);
   }
-  if (fold_bounds && !need_rank) {
+  if ((fold_bounds && !need_rank) || ranked_with_bounds) {
     // nothing left to launch
   } else if (lazy_rows) {
     if (max_pred > 0) {

@@ -21,7 +21,6 @@ struct ReluDesc {
   int32_t* asc_idx;    // crossing neuron indices in ascending order (sort orders only)
   double* key;         // sort keys, ascending-index order
   const double* given_key;  // order kOrderGiven: the key of every row is handed in (callers with an explicit list)
-  int32_t* rank;       // rank of every ascending-list entry under the stable descending key sort
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
   int32_t* keep_idx;   // rows left untouched (active neurons), ascending, then -1 up to a multiple of 16
   int32_t* blk_counts; // multi-block classification: per 1024-row block {crossing, inactive, kept}
