@@ -123,13 +123,16 @@ __global__ __launch_bounds__(64 * kRangeWaves, OCC) void ranges_partial_kernel(c
 }
 
 // The same sums for a set whose generator images come with windows (RangeDesc::box), read inside the windows only:
-// the images may not even be in memory outside them.  Lane = image position, a block covers 64 positions of
-// kWinCG channels, so that one window test serves kWinCG loads.  Columns are dealt to the eight waves, added up
-// and combined exactly as in ranges_partial_kernel with row_waves = 1 (wave w takes the columns j0 + 8w + 64k ...
-// + 7 in order; wave 0 then adds the other waves' sums in wave order): skipping the exact zeros outside a window
-// leaves every sum as it is, so both kernels give the same bits.
-constexpr int kWinCG = 4;
-__global__ __launch_bounds__(512) void ranges_window_kernel(const RangeDesc* __restrict__ table, RangeDesc one, int nposb, int C) {
+// the images may not even be in memory outside them.  A lane owns PW consecutive image positions (PW = 2 where the
+// image has an even number of positions: 16-byte loads) of 4 / PW channels, a block 64 * PW positions, so that one
+// window test serves several loads.  Columns are dealt to the eight waves, added up and combined exactly as in
+// ranges_partial_kernel with row_waves = 1 (wave w takes the columns j0 + 8w + 64k ... + 7 in order; wave 0 then
+// adds the other waves' sums in wave order): skipping the exact zeros outside a window (whole columns whose
+// window misses the block included) leaves every sum as it is, so both kernels give the same bits.
+constexpr int kTake = 4;  // columns whose loads a wave has in flight together
+template <int PW>
+__global__ __launch_bounds__(512, 4) void ranges_window_kernel(const RangeDesc* __restrict__ table, RangeDesc one, int nposb, int C) {
+  constexpr int CG = 4 / PW;  // channels of a block
   const RangeDesc d = table ? table[blockIdx.z] : one;
   const int chunk = blockIdx.y;
   if (chunk >= d.chunks) return;
@@ -137,86 +140,154 @@ __global__ __launch_bounds__(512) void ranges_window_kernel(const RangeDesc* __r
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int pb = blockIdx.x % nposb, cg = blockIdx.x / nposb;
   const int P = d.bH * d.bW;
-  const int p = pb * 64 + lane;
-  const bool pvalid = p < P;
-  const int w = p / d.bH, h = p - w * d.bH;
-  const int c0 = cg * kWinCG;
-  const int nc = min(kWinCG, C - c0);
+  const int p = (pb * 64 + lane) * PW;  // first of the lane's positions
+  bool pvalid[PW];
+  int w[PW], h[PW];
+#pragma unroll
+  for (int e = 0; e < PW; ++e) {
+    pvalid[e] = p + e < P;
+    w[e] = (p + e) / d.bH;
+    h[e] = (p + e) - w[e] * d.bH;
+  }
+  const int c0 = cg * CG;
+  const int nc = min(CG, C - c0);
   const int j0 = 1 + chunk * d.cols_per_chunk;
   const int j1 = min(d.n, (chunk + 1) * d.cols_per_chunk) + 1;
-  double s[kWinCG][4];
+  double s[CG][4][PW];
 #pragma unroll
-  for (int cc = 0; cc < kWinCG; ++cc)
+  for (int cc = 0; cc < CG; ++cc)
 #pragma unroll
-    for (int a = 0; a < 4; ++a) s[cc][a] = 0.0;
-  const double* base = d.V + p + (int64_t)P * c0;
-#pragma unroll 1
-  for (int jb = j0 + 8 * wave; jb < j1; jb += 64) {
-    // the wave's eight columns of this step: window tests first, then all their loads (four channels at a
-    // time) in flight together, then the sums column by column
-    bool in[8];
-    double pl[8], pu[8];
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      in[u] = false;
+      for (int e = 0; e < PW; ++e) s[cc][a][e] = 0.0;
+  // the image positions of the block: a window that misses all of them is skipped by the whole block (what it
+  // would add are exact zeros)
+  const int pfirst = pb * 64 * PW, plast = min(P - 1, pfirst + 64 * PW - 1);
+  const int wlo = pfirst / d.bH, whi = plast / d.bH;
+  const int hlo = wlo == whi ? pfirst - wlo * d.bH : 0, hhi = wlo == whi ? plast - wlo * d.bH : d.bH - 1;
+  // Most windows miss the positions of a block altogether.  A wave therefore first looks at the windows of 64
+  // of its columns at a time (one per lane) and queues the ones that reach the block, in ascending order; the
+  // queue is worked off kTake columns at a time, so that the loads of a step are all wanted.
+  __shared__ int queue[8][64 + kTake];
+  int* const qw = queue[wave];
+  int qn = 0;
+  auto take = [&](int first, int cnt) {
+    // up to kTake queued columns: window tests first, then all their loads in flight together, then the sums
+    // column by column
+    bool in[kTake][PW];
+    double pl[kTake], pu[kTake];
+    int col_j[kTake];
+#pragma unroll
+    for (int u = 0; u < kTake; ++u) {
+#pragma unroll
+      for (int e = 0; e < PW; ++e) in[u][e] = false;
       pl[u] = pu[u] = 0.0;
-      if (jb + u < j1) {
-        const ColBox b = d.box[jb + u];
-        in[u] = pvalid && h >= b.h0 && h <= b.h1 && w >= b.w0 && w <= b.w1;
-        pl[u] = d.plb[jb + u - 1];
-        pu[u] = d.pub[jb + u - 1];
+      col_j[u] = 0;
+      if (u < cnt) {
+        const int j = __builtin_amdgcn_readfirstlane(qw[first + u]);
+        col_j[u] = j;
+        const ColBox b = d.box[j];
+#pragma unroll
+        for (int e = 0; e < PW; ++e) in[u][e] = pvalid[e] && h[e] >= b.h0 && h[e] <= b.h1 && w[e] >= b.w0 && w[e] <= b.w1;
+        pl[u] = d.plb[j - 1];
+        pu[u] = d.pub[j - 1];
+      }
+    }
+    double v[kTake][CG][PW];
+#pragma unroll
+    for (int u = 0; u < kTake; ++u) {
+      // (a block-uniform address plus the lane's position: one offset register serves every load)
+      const double* col = d.V + (int64_t)col_j[u] * d.ld + (int64_t)P * c0;
+#pragma unroll
+      for (int cc = 0; cc < CG; ++cc) {
+        const double* src = col + (int64_t)P * cc;
+        if constexpr (PW == 2) {
+          // both positions in one load; what lies outside the window may never have been written
+          double2 t = make_double2(0.0, 0.0);
+          if ((in[u][0] || in[u][1]) && cc < nc) t = *reinterpret_cast<const double2*>(src + (unsigned)p);
+          v[u][cc][0] = in[u][0] ? t.x : 0.0;
+          v[u][cc][1] = in[u][1] ? t.y : 0.0;
+        } else {
+          v[u][cc][0] = (in[u][0] && cc < nc) ? src[(unsigned)p] : 0.0;
+        }
       }
     }
 #pragma unroll
-    for (int half = 0; half < kWinCG; half += 4) {
-      if (half >= nc) break;  // (uniform)
-      double v[8][4];
+    for (int u = 0; u < kTake; ++u) {
+      if (u >= cnt) break;  // (uniform)
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const double* col = base + (int64_t)(jb + u) * d.ld + (int64_t)P * half;
+      for (int cc = 0; cc < CG; ++cc)
 #pragma unroll
-        for (int cc = 0; cc < 4; ++cc) v[u][cc] = (in[u] && half + cc < nc) ? col[(int64_t)P * cc] : 0.0;
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-#pragma unroll
-        for (int cc = 0; cc < 4; ++cc) {
-          const double px = fmax(v[u][cc], 0.0), nx = fmin(v[u][cc], 0.0);
-          s[half + cc][0] = fma(px, pl[u], s[half + cc][0]);  // xmin1
-          s[half + cc][1] = fma(nx, pu[u], s[half + cc][1]);  // xmin2
-          s[half + cc][2] = fma(px, pu[u], s[half + cc][2]);  // xmax1
-          s[half + cc][3] = fma(nx, pl[u], s[half + cc][3]);  // xmax2
+        for (int e = 0; e < PW; ++e) {
+          const double px = fmax(v[u][cc][e], 0.0), nx = fmin(v[u][cc][e], 0.0);
+          s[cc][0][e] = fma(px, pl[u], s[cc][0][e]);  // xmin1
+          s[cc][1][e] = fma(nx, pu[u], s[cc][1][e]);  // xmin2
+          s[cc][2][e] = fma(px, pu[u], s[cc][2][e]);  // xmax1
+          s[cc][3][e] = fma(nx, pl[u], s[cc][3][e]);  // xmax2
         }
     }
+  };
+  // the wave's columns in its order: entry e is column j0 + 8 * wave + 64 * (e / 8) + e % 8
+#pragma unroll 1
+  for (int e0 = 0; j0 + 8 * wave + 8 * e0 < j1; e0 += 64) {
+    const int e = e0 + lane;
+    const int j = j0 + 8 * wave + 64 * (e >> 3) + (e & 7);
+    bool hit = false;
+    if (j < j1) {
+      const ColBox b = d.box[j];
+      hit = b.w1 >= wlo && b.w0 <= whi && b.h1 >= hlo && b.h0 <= hhi;
+    }
+    const unsigned long long mask = __ballot(hit);
+    if (hit) qw[qn + __popcll(mask & ((1ull << lane) - 1ull))] = j;
+    qn += __popcll(mask);
+    __builtin_amdgcn_wave_barrier();
+    int qh = 0;
+    for (; qn - qh >= kTake; qh += kTake) take(qh, kTake);
+    if (qh > 0) {  // the (fewer than kTake) columns left over move to the front
+      const int rem = qn - qh;
+      int keep = 0;
+      if (lane < rem) keep = qw[qh + lane];
+      __builtin_amdgcn_wave_barrier();
+      if (lane < rem) qw[lane] = keep;
+      __builtin_amdgcn_wave_barrier();
+      qn = rem;
+    }
   }
-  __shared__ double red[8][4][64];
+  if (qn > 0) take(0, qn);
+  __shared__ double red[8][4][64 * PW];
   const bool direct = d.chunks == 1 && d.chunks2 == 0 && d.part3 == nullptr;
 #pragma unroll
-  for (int cc = 0; cc < kWinCG; ++cc) {
+  for (int cc = 0; cc < CG; ++cc) {
     if (cc < nc) {  // (uniform over the block)
       if (wave > 0) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a) red[wave][a][lane] = s[cc][a];
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int e = 0; e < PW; ++e) red[wave][a][lane * PW + e] = s[cc][a][e];
       }
       __syncthreads();
-      if (wave == 0 && pvalid) {
-        double t[4];
+      if (wave == 0) {
 #pragma unroll
-        for (int a = 0; a < 4; ++a) {
-          t[a] = s[cc][a];
-          for (int w2 = 1; w2 < 8; ++w2) t[a] += red[w2][a][lane];
-        }
-        const int64_t r = p + (int64_t)P * (c0 + cc);
-        if (direct) {
-          const double c = d.V[r];
-          d.lb[r] = (c + t[0]) + t[1];
-          d.ub[r] = (c + t[2]) + t[3];
-        } else {
-          double* q = d.part + ((int64_t)chunk * 4) * d.ld + r;
-          q[0] = t[0];
-          q[d.ld] = t[1];
-          q[2 * d.ld] = t[2];
-          q[3 * d.ld] = t[3];
+        for (int e = 0; e < PW; ++e) {
+          if (!pvalid[e]) continue;
+          double t[4];
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            t[a] = s[cc][a][e];
+            for (int w2 = 1; w2 < 8; ++w2) t[a] += red[w2][a][lane * PW + e];
+          }
+          const int64_t r = p + e + (int64_t)P * (c0 + cc);
+          if (direct) {
+            const double c = d.V[r];
+            d.lb[r] = (c + t[0]) + t[1];
+            d.ub[r] = (c + t[2]) + t[3];
+          } else {
+            double* q = d.part + ((int64_t)chunk * 4) * d.ld + r;
+            q[0] = t[0];
+            q[d.ld] = t[1];
+            q[2 * d.ld] = t[2];
+            q[3 * d.ld] = t[3];
+          }
         }
       }
       __syncthreads();
@@ -1006,10 +1077,19 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   if (scan && in_windows) {
     const int P = descs[0].bH * descs[0].bW;
     const int C = (int)(todo[0]->N / P);
-    const int nposb = (int)ceil_div(P, 64);
+    // two positions per lane (16-byte loads) where every image row then starts on a 16-byte boundary
+    bool wide = P % 2 == 0;
+    for (int64_t i = 0; i < nset && wide; ++i) wide = (reinterpret_cast<uintptr_t>(descs[i].V) & 15) == 0;
     NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-    NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_window_kernel, dim3((unsigned)(nposb * ceil_div(C, kWinCG)), (unsigned)chunks, (unsigned)nset),
-               dim3(512), 0, table, descs[0], nposb, C);
+    if (wide) {
+      const int nposb = (int)ceil_div(P, 128);
+      NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_window_kernel<2>, dim3((unsigned)(nposb * ceil_div(C, 2)), (unsigned)chunks, (unsigned)nset),
+                 dim3(512), 0, table, descs[0], nposb, C);
+    } else {
+      const int nposb = (int)ceil_div(P, 64);
+      NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_window_kernel<1>, dim3((unsigned)(nposb * ceil_div(C, 4)), (unsigned)chunks, (unsigned)nset),
+                 dim3(512), 0, table, descs[0], nposb, C);
+    }
     NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 2, bytes));
   } else if (scan) {
     NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
