@@ -1385,7 +1385,51 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         fuse.plb = outs[0]->plb;
         fuse.pub = outs[0]->pub;
         BufRef packed;
-        if (compact && pack) {
+        // enough 128 x 128 tiles to go round: the tile kernel of gemm_seg.hip (rows packed transposed, operands
+        // staged straight into LDS), as for an array of sets
+        const int64_t tiles128 = ceil_div(dense[0], 128) * ceil_div(fc->Mp, 128);
+        const bool tile_kernel = compact && pack && rows.kmap != nullptr && !dense_only && tiles128 >= 128 && kp <= 2048 &&
+                                 dense[0] < (int64_t(1) << 24);
+        if (tile_kernel) {
+          const int64_t ldo = outs[0]->ld, ldt = round_up(dense[0], 128), ntiles = ceil_div(dense[0], 128);
+          st = c->alloc(sizeof(double) * kp * ldt, &packed);
+          if (st == NNVHIP_OK) {
+            PackSet ps = pack_of(in[0], in[0]->kept_idx, packed->as<double>(), kp, dense[0]);
+            ps.ldt = ldt;
+            st = launch_pack_rows_t(c, 1, &ps);
+          }
+          if (st == NNVHIP_OK) st = c->alloc(sizeof(double) * 4 * ldo * ntiles, &fuse.part);
+          fuse.chunks = ntiles;
+          // tiles by width: [0] 128 columns, [1] 64, [2] 32 (the last tile, if the remainder fits)
+          std::vector<SegTile> tiles[3];
+          double flop[3] = {0.0, 0.0, 0.0};
+          for (int64_t j = 0; j < dense[0] && st == NNVHIP_OK; j += 128) {
+            const int64_t valid = std::min<int64_t>(128, dense[0] - j);
+            const int w = valid > 64 ? 0 : valid > 32 ? 1 : 2;
+            SegTile sg;
+            sg.kmap = rows.kmap;
+            sg.Bt = packed->as<double>();
+            sg.ldbt = ldt;
+            sg.col_local0 = j;
+            sg.col_base = j;
+            sg.kp = (int32_t)kp;
+            sg.valid = (int32_t)valid;
+            sg.plb = outs[0]->plb;
+            sg.pub = outs[0]->pub;
+            sg.rpart = fuse.part->as<double>() + 4 * ldo * (j / 128);
+            tiles[w].push_back(sg);
+            flop[w] += 2.0 * (double)fc->Mp * (double)kp * (double)valid;
+          }
+          static const int widths[3] = {128, 64, 32};
+          for (int w = 0; w < 3 && st == NNVHIP_OK; ++w) {
+            if (tiles[w].empty()) continue;
+            BufRef dt;
+            st = c->upload_table(tiles[w].data(), sizeof(SegTile) * tiles[w].size(), &dt);
+            if (st == NNVHIP_OK)
+              st = launch_gemm_seg(c, Wd, fc->Mp, outs[0]->V, ldo, fc->Mp, bias, widths[w], dt->as<SegTile>(), (int64_t)tiles[w].size(),
+                                   flop[w]);
+          }
+        } else if (compact && pack) {
           st = c->alloc(sizeof(double) * kp * dense[0], &packed);
           if (st == NNVHIP_OK) {
             PackSet ps = pack_of(in[0], in[0]->kept_idx, packed->as<double>(), kp, dense[0]);
@@ -1394,7 +1438,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             rows.ldbk = kp;
           }
         }
-        if (st == NNVHIP_OK)
+        if (st == NNVHIP_OK && !tile_kernel)
           st = launch_gemm(c, Wd, fc->Mp, in[0]->V, in[0]->ld, outs[0]->V, outs[0]->ld, fc->Mp, dense[0], kp, bias, &fuse,
                            compact ? &rows : nullptr);
         if (st == NNVHIP_OK && fuse.chunks > 0) {

@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kSegNT, 4) void gemm_seg_kernel(const double* __res
 // Packs the listed rows of a set's leading columns transposed: Vt(t, j) = V(kept[t], j) for t < kp
 // (zero where kept[t] < 0) and j < ncols, zero for ncols <= j < ldt; Vt is kp x ldt, row-major.  A block
 // transposes a 64 x 64 piece through LDS: it reads like pack_rows_kernel (lanes along the kept rows of one
-// column) and writes 512 contiguous bytes per row.
+// column) and writes 512 contiguous bytes per row, 16 per lane.
 __global__ __launch_bounds__(256) void pack_rows_t_kernel(const PackSet* __restrict__ table, PackSet one) {
   const PackSet d = table ? table[blockIdx.z] : one;
   const int t0 = blockIdx.x * 64, j0 = blockIdx.y * 64;
@@ -262,9 +262,11 @@ __global__ __launch_bounds__(256) void pack_rows_t_kernel(const PackSet* __restr
     tile[cc][lane] = v;
   }
   __syncthreads();
-  const int j = j0 + lane;
-  if (j < d.ldt)
-    for (int kk = wave; kk < 64 && t0 + kk < d.kp; kk += 4) d.Vk[(int64_t)(t0 + kk) * d.ldt + j] = tile[lane][kk];
+  // two columns per lane (16-byte stores), two rows per wave and pass; ldt is even
+  const int jl = 2 * (lane & 31), kh = lane >> 5;
+  if (j0 + jl < d.ldt)
+    for (int kk = 2 * wave + kh; kk < 64 && t0 + kk < d.kp; kk += 8)
+      *reinterpret_cast<double2_t*>(d.Vk + (int64_t)(t0 + kk) * d.ldt + j0 + jl) = double2_t{tile[jl][kk], tile[jl + 1][kk]};
 }
 
 // The same packing when every column but the centre is a scaled weight column and the weights are at hand
@@ -363,6 +365,7 @@ int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
   int64_t max_kp = 0, max_ld = 0;
   for (int64_t i = 0; i < count; ++i) {
+    if (sets[i].ldt % 2) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: packed rows must have an even length");
     max_kp = std::max<int64_t>(max_kp, sets[i].kp);
     max_ld = std::max<int64_t>(max_ld, sets[i].ldt);
   }
