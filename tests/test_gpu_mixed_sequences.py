@@ -194,3 +194,17 @@ def test_wide_layers_in_a_sequence(nnv, oracle, wide, count, method):
         dev_in = nnv.Star.from_boxes(lbs, ubs)
         ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
     _compare(nnv, oracle, layers, dev_in, ora_in, method)
+
+
+@pytest.mark.parametrize("method", ["relax-star-area", "relax-star-static"])
+def test_one_wide_set_through_the_tile_kernel(nnv, oracle, method):
+    # one set with thousands of predicates whose row reset is pending: the FC layer after the ReLU contracts the
+    # kept rows of 4201 columns into 520 outputs, enough 128 x 128 tiles for the kernel that arrays of sets use
+    # (rows packed transposed, narrow last tile); a skinny layer with 20 outputs (two rows of 16) ends the net
+    rs = np.random.RandomState(77)
+    N, n = 300, 4200
+    V = np.c_[rs.randn(N) * 2.0, rs.randn(N, n) * 5e-4]
+    V[rs.choice(N, size=20, replace=False), 1:] = 0.0          # some neurons with a point range
+    args = (V, np.zeros((1, n)), np.zeros(1), -np.ones(n), np.ones(n))
+    layers = [{"type": "relu"}, _fc(rs, 520, N, 2.0), {"type": "relu"}, _fc(rs, 20, 520)]
+    _compare(nnv, oracle, layers, nnv.Star(*args), oracle.OStar(*args), method)
