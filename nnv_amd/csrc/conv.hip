@@ -838,9 +838,21 @@ __global__ void stamp_pixel_columns_kernel(const int32_t* __restrict__ idx, int 
 
 // S lanes share a row, lane s taking the taps k = s, s + S, ...; their sums are combined by a butterfly (a fixed
 // order).  S = 1 for filters with few taps, 16 otherwise (a row's taps are then walked by 16 lanes at once).
+// A block first decodes the taps once into LDS (filter position and the tap's offset from the pixel under the
+// filter's corner), so that the walk has no division in it, and looks up four taps' pixels before it handles them.
+constexpr int kStampTapTable = kMaxTaps;  // taps per output (FH * FW * Cin): no layer has more
 template <int S>
 __global__ __launch_bounds__(256) void conv_stamp_rows_kernel(StampSet d, ConvGeom g, const double* __restrict__ Wt,
                                                               const int32_t* __restrict__ pixel_col, int64_t ldout) {
+  __shared__ int2 taps[kStampTapTable];  // x: fh | fw << 16, y: fh + H * (fw + W * ci)
+  for (int k = threadIdx.x; k < g.K; k += 256) {
+    const int fh = k % g.FH;
+    const int q = k / g.FH;
+    const int fw = q % g.FW;
+    const int ci = q / g.FW;
+    taps[k] = make_int2(fh | (fw << 16), fh + g.H * (fw + g.W * ci));
+  }
+  __syncthreads();
   const int64_t gt = blockIdx.x * (int64_t)256 + threadIdx.x;
   const int64_t r = gt / S;
   const int s = (int)(gt % S);
@@ -852,26 +864,38 @@ __global__ __launch_bounds__(256) void conv_stamp_rows_kernel(StampSet d, ConvGe
     const int p = (int)(r - (int64_t)co * g.P);
     const int wo = p / g.Ho, ho = p - wo * g.Ho;
     const int hb = ho * g.sh - g.pt, wb = wo * g.sw - g.pl;
+    const int pbase = hb + g.H * wb;  // the pixel under the filter's corner (may lie outside the image)
     const double* wcol = Wt + (int64_t)co * g.Kp;
-    for (int k = s; k < g.K; k += S) {
-      const int fh = k % g.FH;
-      const int q = k / g.FH;
-      const int fw = q % g.FW;
-      const int ci = q / g.FW;
-      const int h = hb + fh, w = wb + fw;
-      if ((unsigned)h >= (unsigned)g.H || (unsigned)w >= (unsigned)g.W) continue;
-      const int pixel = h + g.H * (w + g.W * ci);
-      const int t = pixel_col[pixel];
-      if (t < 0) continue;
-      const double sc = d.scale != nullptr ? d.scale[pixel] : 1.0;
-      const double v = __dadd_rn(0.0, __dmul_rn(wcol[k], sc));
-      d.out[r + (int64_t)t * ldout] = v;
-      const double pl = d.plb[t], pu = d.pub[t];
-      const double vp = fmax(v, 0.0), vn = fmin(v, 0.0);
-      x1 = fma(vp, pl, x1);  // xmin1
-      x2 = fma(vn, pu, x2);  // xmin2
-      y1 = fma(vp, pu, y1);  // xmax1
-      y2 = fma(vn, pl, y2);  // xmax2
+    for (int k0 = s; k0 < g.K; k0 += 4 * S) {
+      int t[4], pix[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + u * S;
+        t[u] = -1;
+        pix[u] = 0;
+        if (k < g.K) {
+          const int2 tp = taps[k];
+          const int h = hb + (tp.x & 0xffff), w = wb + (tp.x >> 16);
+          if ((unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W) {
+            pix[u] = pbase + tp.y;
+            t[u] = pixel_col[pix[u]];
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (t[u] < 0) continue;
+        const int k = k0 + u * S;
+        const double sc = d.scale != nullptr ? d.scale[pix[u]] : 1.0;
+        const double v = __dadd_rn(0.0, __dmul_rn(wcol[k], sc));
+        d.out[r + (int64_t)t[u] * ldout] = v;
+        const double pl = d.plb[t[u]], pu = d.pub[t[u]];
+        const double vp = fmax(v, 0.0), vn = fmin(v, 0.0);
+        x1 = fma(vp, pl, x1);  // xmin1
+        x2 = fma(vn, pu, x2);  // xmin2
+        y1 = fma(vp, pu, y1);  // xmax1
+        y2 = fma(vn, pl, y2);  // xmax2
+      }
     }
   }
 #pragma unroll
@@ -915,6 +939,7 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int6
   fill_geom(g, cv, H, W, Ho, Wo);
   if (conv_stamps_by_row(cv)) {
     if (chunks != 1) NNV_FAIL(NNVHIP_ERR_ARG, "internal: one chunk of range sums per set");
+    if (g.K > kStampTapTable) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: more taps than the stamp kernel's table holds");
     const int64_t n_in = H * W * cv->Cin;
     BufRef inv;
     NNV_TRY(ctx->alloc(sizeof(int32_t) * (size_t)n_in * (size_t)count, &inv));
