@@ -61,6 +61,7 @@ const TuneKnobs& tune_knobs() {
     k.apply_row_waves = num("NNVHIP_APPLY_ROW_WAVES");
     k.apply_blocks = num("NNVHIP_APPLY_BLOCKS");
     k.conv_general = num("NNVHIP_CONV_GENERAL");
+    k.one_block_n = num("NNVHIP_ONE_BLOCK_N");
     return k;
   }();
   return knobs;

@@ -79,12 +79,13 @@ inline void mailbox_unpack(unsigned long long w, int* m, int* inactive, int* seq
 // Tuning knobs for experiments, read from the environment once per process (0 / empty: not set):
 // NNVHIP_GEMM_XR, NNVHIP_GEMM_KSPLIT, NNVHIP_GEMM_TILE ("TMxTN"), NNVHIP_RANGES_ROW_WAVES,
 // NNVHIP_RANGES_BLOCKS, NNVHIP_APPLY_ROW_WAVES, NNVHIP_APPLY_BLOCKS, NNVHIP_CONV_GENERAL (1: every convolution
-// on the general kernel).
+// on the general kernel), NNVHIP_ONE_BLOCK_N (1024 .. 8192: largest set the one-block classification takes).
 struct TuneKnobs {
   int gemm_xr = 0, gemm_ksplit = 0;
   std::string gemm_tile;
   int ranges_row_waves = 0, ranges_blocks = 0, apply_row_waves = 0, apply_blocks = 0;
   int conv_general = 0;
+  int one_block_n = 0;
 };
 const TuneKnobs& tune_knobs();
 

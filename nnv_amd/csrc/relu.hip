@@ -593,6 +593,14 @@ int ensure_dense(nnvhip_ctx* ctx, nnvhip_star* s, bool need_tail) {
   return ensure_dense_batch(ctx, 1, &s, need_tail);
 }
 
+// Sets of up to this many neurons are classified by one block each (one launch for the whole step when the
+// crossing list fits the in-block sort); larger ones by the multi-block kernels.  The one-block kernel walks a set
+// 1024 neurons at a time, two barriers a round: 19 us at 7200 neurons, where count + compact take 4 us each.
+static int64_t one_block_limit() {
+  const int n = tune_knobs().one_block_n;
+  return n >= 1024 && n <= 8192 ? n : 2048;
+}
+
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out, const ReluGiven* given) {
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
   if ((order == kOrderGiven) != (given != nullptr)) NNV_FAIL(NNVHIP_ERR_ARG, "internal: explicit lists and their order go together");
@@ -605,6 +613,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   if (given == nullptr) NNV_TRY(compute_ranges(ctx, count, in));
   const int64_t N = in[0]->N;
   const int64_t ld = in[0]->ld;
+  const int64_t kOneBlockN = one_block_limit();
   if (N >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "set dimension too large");
   const bool sorted = order != NNVHIP_ORDER_INDEX;
 
@@ -613,7 +622,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const int64_t nblk = ceil_div(N, 1024);
   NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &cls_buf));
   NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * count, &cnt_buf));
-  if (N > 8192) NNV_TRY(ctx->alloc(sizeof(int32_t) * 3 * nblk * count, &blk_buf));
+  if (N > kOneBlockN) NNV_TRY(ctx->alloc(sizeof(int32_t) * 3 * nblk * count, &blk_buf));
   // kept-row lists of all sets in one buffer; the classification pads each list with -1 up to a whole
   // K-tile (at least one), which is what the GEMM's row map expects
   const int64_t keep_ld = round_up(N, kLdAlign) + kLdAlign;
@@ -626,7 +635,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // With the reset pending, all that is left to write are the predicate bounds and the crossing
   // neurons' (lb, ub).  The one-block classification does that itself, into buffers sized for the worst
   // case (every neuron crossing), and the step is a single launch.
-  const bool fold_bounds = lazy_rows && N <= 8192;
+  const bool fold_bounds = lazy_rows && N <= kOneBlockN;
   BufRef pred_buf, lbub_buf;
   std::vector<int64_t> pred_off(count), lbub_off(count);
   const int64_t ldr_max = round_up(N, kLdAlign);
@@ -693,13 +702,13 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // Up to 8192 neurons: one block per set classifies, compacts and sorts crossing lists of up to 1024
   // entries (sorting network).  Larger sets: two multi-block passes.  Whatever is still unsorted after
   // the read-back of the counts goes to the multi-block rank kernels.
-  const int sort_cap = !sorted ? 0 : N <= 8192 ? kSortInBlock : 0;
+  const int sort_cap = !sorted ? 0 : N <= kOneBlockN ? kSortInBlock : 0;
   // algorithmic bytes of the classification: lb and ub read, the per-row class and the two index lists
   // written (plus, when it also writes the predicate bounds, the copy of the input's)
   double cls_bytes = 0.0;
   for (int64_t i = 0; i < count; ++i) cls_bytes += 24.0 * (double)N + (fold_bounds ? 32.0 * (double)in[i]->n : 0.0);
   const bool tk = ctx->kernel_timing;
-  if (N <= 8192) {
+  if (N <= kOneBlockN) {
     if (!sorted)
       NNV_LAUNCH(ctx, tk, relu_classify_kernel<0>, dim3((unsigned)count), dim3(1024), 0, table, descs[0]);
     else if (N <= 1024)
