@@ -177,9 +177,10 @@ def test_random_chains_of_convolutions(nnv, oracle, seed):
     _compare(nnv, oracle, layers, nnv.ImageStar(lo, hi), oracle.image_star_from_bounds(lo, hi), ALL_RELAX[seed % 6])
 
 
-@pytest.mark.parametrize("wide,count,method", [(9000, 1, "relax-star-range"), (8200, 2, "relax-star-static")])
+@pytest.mark.parametrize("wide,count,method", [(9000, 1, "relax-star-range"), (8200, 2, "relax-star-static"),
+                                               (2049, 1, "relax-star-area"), (3000, 3, "relax-star-bound")])
 def test_wide_layers_in_a_sequence(nnv, oracle, wide, count, method):
-    # more than 8192 neurons: classification, sort and bounds run as separate multi-block kernels, and
+    # more than 2048 neurons: classification, sort and bounds run as separate multi-block kernels, and
     # the sets that come out of them feed batch normalisation, another ReLU and an FC layer
     rs = np.random.RandomState(wide)
     n_in = 10
