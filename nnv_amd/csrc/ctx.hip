@@ -614,6 +614,11 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
   std::vector<int32_t> gen_dim;
   std::vector<int64_t> col_off(count + 1, 0), gen_off(count + 1, 0);
   std::vector<char> neg_scale((size_t)count, 0);
+  // Sets with the same half-widths, bit for bit (the boxes of a regular partition), share one scale vector and one
+  // index list on the device: layers downstream recognise by the pointers that such sets gather the same scaled
+  // weight columns.  shape_of[s] = the first set with set s's half-widths (among the first few distinct shapes).
+  std::vector<int64_t> shape_of((size_t)count);
+  std::vector<int64_t> shapes;
   for (int64_t s = 0; s < count; ++s) {
     int64_t n = 0;
     for (int64_t i = 0; i < N; ++i) {
@@ -630,6 +635,13 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
     }
     gen_off[s + 1] = gen_off[s] + n;
     col_off[s + 1] = col_off[s] + n + 1;
+    shape_of[s] = s;
+    for (int64_t r : shapes)
+      if (memcmp(&vec[r * N], &vec[s * N], sizeof(double) * N) == 0) {
+        shape_of[s] = r;
+        break;
+      }
+    if (shape_of[s] == s && shapes.size() < 16) shapes.push_back(s);
   }
   int64_t ld = round_up(N, kLdAlign);
   int64_t total_cols = col_off[count];
@@ -678,9 +690,9 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
     if (st->n > 0) {  // every generator column is vec(dim) * e_dim
       st->oh_from = 1;
       st->oh_idx_buf = dgen;
-      st->oh_idx = dgen->as<int32_t>() + gen_off[s];
+      st->oh_idx = dgen->as<int32_t>() + gen_off[shape_of[s]];
       st->oh_scale_buf = dvec;
-      st->oh_scale = dvec->as<double>() + s * N;
+      st->oh_scale = dvec->as<double>() + shape_of[s] * N;
       st->oh_scale_neg = neg_scale[s] != 0;
     }
     out[s] = st;
@@ -1407,10 +1419,11 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           for (int64_t j = 0; j < dense[0] && st == NNVHIP_OK; j += 128) {
             const int64_t valid = std::min<int64_t>(128, dense[0] - j);
             const int w = valid > 64 ? 0 : valid > 32 ? 1 : 2;
-            SegTile sg;
+            SegTile sg{};
             sg.kmap = rows.kmap;
             sg.Bt = packed->as<double>();
             sg.ldbt = ldt;
+            sg.b_col0 = j;
             sg.col_local0 = j;
             sg.col_base = j;
             sg.kp = (int32_t)kp;
@@ -1595,23 +1608,85 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           if (!filled[i] && (!pk[i] || kps[i] > 2048 || dense[i] >= (int64_t(1) << 24))) seg_tiles = false;
         if (seg_tiles) {
           const int64_t ldo = outs[0]->ld;
-          BufRef packed;
+          BufRef packed, shared_rows;
           std::vector<PackSet> packs;
           std::vector<const double*> bt((size_t)count, nullptr);
           std::vector<int64_t> ldt((size_t)count, 0);
+          // Sets whose generator columns are all the same scaled weight columns (boxes of one shape through an FC
+          // layer and a ReLU: same index list, same scales) have the same packed rows wherever they keep the same
+          // row.  One matrix then serves them all - row r = what any of them would pack for input row r - and the
+          // 128-column tiles gather its rows through their own kept-row lists; only a set's centre column (patched
+          // in by its first tile) and the columns past the last whole tile (packed as before) are its own.
+          struct RowShape {  // what decides a set's packed rows besides its kept-row list
+            const double* Wt;
+            int64_t ldwt, rows;
+            const int32_t* idx;
+            const double* scale;
+            int64_t dense, ldws, nfull, off;
+          };
+          std::vector<RowShape> shapes;
+          std::vector<int> shape_of((size_t)count, -1);
+          bool shared = !c->eager_cols;
+          for (int64_t i = 0; i < count && shared; ++i) {
+            if (filled[i]) continue;
+            const ColSource& cs = in[i]->cs;
+            shared = cs.W != nullptr && cs.Wt != nullptr && cs.from == 1 && cs.from + cs.cols >= dense[i] && cs.zero_to <= 1 &&
+                     !cs.win_pending() && dense[i] >= 128 && cs.rows < (int64_t(1) << 30);
+            if (!shared) break;
+            for (size_t k = 0; k < shapes.size() && shape_of[i] < 0; ++k) {
+              const RowShape& r = shapes[k];
+              if (r.Wt == cs.Wt && r.ldwt == cs.ldwt && r.rows == cs.rows && r.idx == cs.idx && r.scale == cs.scale && r.dense == dense[i])
+                shape_of[i] = (int)k;
+            }
+            if (shape_of[i] < 0) {
+              if (shapes.size() == 16) {  // too many different shapes for the matrices to pay
+                shared = false;
+                break;
+              }
+              shape_of[i] = (int)shapes.size();
+              shapes.push_back(RowShape{cs.Wt, cs.ldwt, cs.rows, cs.idx, cs.scale, dense[i], round_up(dense[i], 128), dense[i] / 128, 0});
+            }
+          }
+          shared = shared && !shapes.empty();
+          if (shared) {
+            int64_t doubles = 0;
+            for (RowShape& r : shapes) {
+              r.off = doubles;
+              doubles += (r.rows + 1) * r.ldws;
+            }
+            st = c->alloc(sizeof(double) * doubles, &shared_rows);
+            ScaledRows sr{};
+            for (size_t k = 0; k < shapes.size(); ++k) {
+              const RowShape& r = shapes[k];
+              sr.s[k] = ScaledRows::One{r.Wt, r.ldwt, r.idx, r.scale, shared_rows ? shared_rows->as<double>() + r.off : nullptr, r.ldws,
+                                        (int32_t)r.rows, (int32_t)r.dense};
+            }
+            sr.count = (int32_t)shapes.size();
+            if (st == NNVHIP_OK) st = launch_scaled_rows(c, sr);
+          }
+          auto nfull_of = [&](int64_t i) { return shared ? shapes[(size_t)shape_of[i]].nfull : 0; };
           int64_t total = 0;
           for (int64_t i = 0; i < count; ++i)
             if (!filled[i]) {
-              ldt[i] = round_up(dense[i], 128);
+              if (shared) {  // the columns past the last whole tile only, in a tile of their own width
+                const int64_t rem = dense[i] - 128 * nfull_of(i);
+                ldt[i] = rem > 64 ? 128 : rem > 32 ? 64 : rem > 0 ? 32 : 0;
+              } else {
+                ldt[i] = round_up(dense[i], 128);
+              }
               total += kps[i] * ldt[i];
             }
-          if (total > 0) st = c->alloc(sizeof(double) * total, &packed);
+          if (total > 0 && st == NNVHIP_OK) st = c->alloc(sizeof(double) * total, &packed);
           int64_t pos = 0;
           for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
-            if (!filled[i]) {
+            if (!filled[i] && ldt[i] > 0) {
               bt[i] = packed->as<double>() + pos;
               PackSet ps = pack_of(in[i], rws[i].kmap, packed->as<double>() + pos, kps[i], dense[i]);
               ps.ldt = ldt[i];
+              if (shared) {
+                ps.col0 = (int32_t)(128 * nfull_of(i));
+                ps.ncols = (int32_t)(dense[i] - 128 * nfull_of(i));
+              }
               packs.push_back(ps);
               pos += kps[i] * ldt[i];
             }
@@ -1621,18 +1696,31 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             chunk_off[i + 1] = chunk_off[i] + tiles_of[i] + (gs[i].m > 0 ? gch_part : 0);
           }
           if (st == NNVHIP_OK && chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
-          // tiles by width: [0] 128 columns, [1] 64, [2] 32 (the last tile of a set whose remainder fits)
-          std::vector<SegTile> tiles[3];
-          double flop[3] = {0.0, 0.0, 0.0};
+          // tiles by width: [0] 128 columns, [1] 64, [2] 32 (the last tile of a set whose remainder fits); [3]: the
+          // 128-column tiles that gather their rows of B from the shared matrix
+          std::vector<SegTile> tiles[4];
+          double flop[4] = {0.0, 0.0, 0.0, 0.0};
           int64_t off = 0;
           for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
             for (int64_t j = 0; j < dense[i] && !filled[i]; j += 128) {
               const int64_t valid = std::min<int64_t>(128, dense[i] - j);
-              const int w = valid > 64 ? 0 : valid > 32 ? 1 : 2;
-              SegTile sg;
+              const bool gather = shared && j < 128 * nfull_of(i);
+              const int w = gather ? 3 : valid > 64 ? 0 : valid > 32 ? 1 : 2;
+              SegTile sg{};
               sg.kmap = rws[i].kmap;
-              sg.Bt = bt[i];
-              sg.ldbt = ldt[i];
+              if (gather) {
+                const RowShape& r = shapes[(size_t)shape_of[i]];
+                sg.Bt = shared_rows->as<double>() + r.off;
+                sg.ldbt = r.ldws;
+                sg.b_col0 = j;
+                sg.centre = in[i]->V;
+                sg.gather_b = 1;
+                sg.zero_row = (int32_t)r.rows;
+              } else {
+                sg.Bt = bt[i];
+                sg.ldbt = ldt[i];
+                sg.b_col0 = shared ? 0 : j;
+              }
               sg.col_local0 = j;
               sg.col_base = off + j;
               sg.kp = (int32_t)kps[i];
@@ -1645,14 +1733,14 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             }
             off += in[i]->n + 1;
           }
-          static const int widths[3] = {128, 64, 32};
-          for (int w = 0; w < 3 && st == NNVHIP_OK; ++w) {
+          static const int widths[4] = {128, 64, 32, 128};
+          for (int w = 3; w >= 0 && st == NNVHIP_OK; --w) {
             if (tiles[w].empty()) continue;
             BufRef dt;
             st = c->upload_table(tiles[w].data(), sizeof(SegTile) * tiles[w].size(), &dt);
             if (st == NNVHIP_OK)
               st = launch_gemm_seg(c, Wd, fc->Mp, outs[0]->V, ldo, fc->Mp, bias, widths[w], dt->as<SegTile>(), (int64_t)tiles[w].size(),
-                                   flop[w]);
+                                   flop[w], w == 3);
           }
           bias_in_kernel = true;
         } else {

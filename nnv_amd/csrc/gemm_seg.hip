@@ -31,7 +31,7 @@ constexpr int kSegS = 4;     // stages in LDS
 constexpr int kSegNT = 512;  // threads per block
 
 // TN columns per tile; WR x WC waves, each owning (16*FM) rows x (16*FN) columns.
-template <int TN, int WR, int WC, int FM, int FN>
+template <int TN, int WR, int WC, int FM, int FN, bool GATHER = false>
 __global__ __launch_bounds__(kSegNT, 4) void gemm_seg_kernel(const double* __restrict__ A, int64_t lda,
                                                             double* __restrict__ C, int64_t ldc, int Mp,
                                                             const double* __restrict__ bias, int tiles_m, int64_t tiles_n,
@@ -73,12 +73,19 @@ __global__ __launch_bounds__(kSegNT, 4) void gemm_seg_kernel(const double* __res
     if (ok) pb_reg = src[sc - 1];
   }
   // row list: wave w stages row 8 * st + w of stage st; lane j keeps the entries of stages j, j + 64, ...
+  static_assert(!GATHER || TN == 128, "rows of B are gathered one per wave");
+  const bool centre_tile = GATHER && sg.col_local0 == 0 && sg.centre != nullptr;
   int kq[4];
+  double cq[4];  // GATHER, a set's first tile: the centre's entries of the same rows
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int st = u * 64 + lane;
     const int c = st < nst ? sg.kmap[st * kSegKS + wave] : 0;
-    kq[u] = c < 0 ? 0 : c;  // a padding entry: its packed row is zero, any column of W will do
+    // a padding entry: its packed row is zero, any column of W will do (GATHER: the entry stays negative and the
+    // row of B is taken from the row of zeros)
+    kq[u] = (c < 0 && !GATHER) ? 0 : c;
+    cq[u] = 0.0;
+    if (GATHER && centre_tile && st < nst && c >= 0) cq[u] = sg.centre[c];
   }
   const unsigned a_lds = lds_addr_of(As + wave * kSegTM);
   const unsigned a_voff = lane * 16;
@@ -87,13 +94,18 @@ __global__ __launch_bounds__(kSegNT, 4) void gemm_seg_kernel(const double* __res
   constexpr int kRowsPerLoad = 128 / TN;
   const unsigned b_lds = lds_addr_of(Bs + wave * 128);
   const unsigned b_voff = (unsigned)(((lane / (TN / 2)) * sg.ldbt + 2 * (lane % (TN / 2))) * 8);
-  const double* b_base = sg.Bt + sg.col_local0 + (int64_t)wave * kRowsPerLoad * sg.ldbt;
+  const double* b_base = sg.Bt + sg.b_col0 + (GATHER ? 0 : (int64_t)wave * kRowsPerLoad * sg.ldbt);
   auto issue = [&](int st) {
     const int u = st >> 6;
     const int c = __builtin_amdgcn_readlane(u == 0 ? kq[0] : u == 1 ? kq[1] : u == 2 ? kq[2] : kq[3], st & 63);
     const int b = st % kSegS;
-    lds_dma16(a_base + (int64_t)c * lda, a_voff, a_lds + (unsigned)(b * kStageA * 8));
-    if (wave < kBLoads) lds_dma16(b_base + (int64_t)st * kSegKS * sg.ldbt, b_voff, b_lds + (unsigned)(b * kStageB * 8));
+    if constexpr (GATHER) {
+      lds_dma16(a_base + (int64_t)(c < 0 ? 0 : c) * lda, a_voff, a_lds + (unsigned)(b * kStageA * 8));
+      lds_dma16(b_base + (int64_t)(c < 0 ? sg.zero_row : c) * sg.ldbt, b_voff, b_lds + (unsigned)(b * kStageB * 8));
+    } else {
+      lds_dma16(a_base + (int64_t)c * lda, a_voff, a_lds + (unsigned)(b * kStageA * 8));
+      if (wave < kBLoads) lds_dma16(b_base + (int64_t)st * kSegKS * sg.ldbt, b_voff, b_lds + (unsigned)(b * kStageB * 8));
+    }
   };
   // transfers a wave has in flight per stage (vmcnt is per wave)
   const bool two = wave < kBLoads;
@@ -119,6 +131,17 @@ __global__ __launch_bounds__(kSegNT, 4) void gemm_seg_kernel(const double* __res
       if (ahead >= kSegS - 2) wait_vm<kSegS - 2>();
       else if (ahead == 1) wait_vm<1>();
       else wait_vm<0>();
+    }
+    if constexpr (GATHER) {
+      // a set's first tile: column 0 of the row this wave brought is the centre's entry, not the shared matrix's
+      if (centre_tile) {
+        const int u = t >> 6;
+        const double cu = u == 0 ? cq[0] : u == 1 ? cq[1] : u == 2 ? cq[2] : cq[3];
+        const int lo = __builtin_amdgcn_readlane((int)(unsigned)(__double_as_longlong(cu) & 0xffffffffll), t & 63);
+        const int hi = __builtin_amdgcn_readlane((int)(__double_as_longlong(cu) >> 32), t & 63);
+        if (lane == 0) Bs[(t % kSegS) * kStageB + wave * TN] = __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+        __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0x0 << 8));  // lgkmcnt(0): the patch is in LDS
+      }
     }
     block_barrier();  // ... and everybody's; everybody is done with stage t - 1, whose buffer the next transfer takes
     if (t + kSegS - 1 < nst) issue(t + kSegS - 1);
@@ -298,11 +321,16 @@ __global__ __launch_bounds__(256) void pack_rows_t_direct_kernel(const PackSet* 
   };
   const int t0 = lower(lo_row);
   const int t1 = (int)blockIdx.y == slices - 1 ? d.kp : lower(hi_row);
-  // a thread's columns (4 * tid .. 4 * tid + 3, then 1024 further on) and what they read do not depend on the
-  // row: weight column and scale are looked up once, the rows then stream out in 16-byte pieces
+  // a thread's four columns (and, if a row is longer than 1024 columns, the ones 1024 further on) and what they
+  // read do not depend on the row: weight column and scale are looked up once, the rows then stream out in
+  // 16-byte pieces.  Short rows (the narrow last tile of a set packed on its own) share the block's threads:
+  // 256 / (ldt / 4) rows per pass.
   constexpr int kQ = 4;
-  for (int jb = 0; jb < d.ldt; jb += 256 * kQ) {
-    const int j0 = jb + kQ * (int)threadIdx.x;
+  const int qpr = min(d.ldt / kQ, 256);  // column quads of a row that one pass covers
+  const int rp = 256 / qpr;              // rows per pass
+  const int q = (int)threadIdx.x % qpr, ro = (int)threadIdx.x / qpr;
+  for (int jb = 0; jb < d.ldt; jb += qpr * kQ) {
+    const int j0 = jb + kQ * q;
     int src[kQ];
     double sc[kQ];
     int kind[kQ];  // 0: zero, 1: the centre, 2: a weight column
@@ -313,18 +341,19 @@ __global__ __launch_bounds__(256) void pack_rows_t_direct_kernel(const PackSet* 
       sc[e] = 0.0;
       kind[e] = 0;
       if (j < d.ncols) {
-        if (j == 0) {
+        const int js = d.col0 + j;  // the set's column
+        if (js == 0) {
           kind[e] = 1;
-        } else if (j >= d.zero_to) {
+        } else if (js >= d.zero_to) {
           kind[e] = 2;
-          src[e] = d.widx[j - d.wfrom];
+          src[e] = d.widx[js - d.wfrom];
           sc[e] = d.wscale ? d.wscale[src[e]] : 1.0;
         }
       }
     }
-    if (j0 >= d.ldt) continue;  // (ldt is a multiple of four)
+    if (j0 >= d.ldt || ro >= rp) continue;  // (ldt is a multiple of four)
 #pragma unroll 2
-    for (int t = t0; t < t1; ++t) {
+    for (int t = t0 + ro; t < t1; t += rp) {
       const int ra = d.kept[t];
       const double* wrow = d.Wt + (int64_t)max(ra, 0) * d.ldwt;
       double* dst = d.Vk + (int64_t)t * d.ldt + j0;
@@ -341,7 +370,7 @@ __global__ __launch_bounds__(256) void pack_rows_t_direct_kernel(const PackSet* 
   }
 }
 
-template <int TN, int WR, int WC, int FM, int FN>
+template <int TN, int WR, int WC, int FM, int FN, bool GATHER = false>
 int launch_seg_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
                    const SegTile* segs, int64_t ntiles, double flop) {
   const int64_t tiles_m = ceil_div(Mp, kSegTM);
@@ -351,7 +380,7 @@ int launch_seg_cfg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int
   const int64_t xr = 1, local_m = tiles_m;
   const int64_t slots = local_m * ceil_div(ntiles, 8 / xr);
   const bool timed = ctx->kernel_timing;
-  NNV_LAUNCH(ctx, timed, (gemm_seg_kernel<TN, WR, WC, FM, FN>), dim3((unsigned)(8 * slots)), dim3(kSegNT), 0, A, lda, C, ldc, (int)Mp,
+  NNV_LAUNCH(ctx, timed, (gemm_seg_kernel<TN, WR, WC, FM, FN, GATHER>), dim3((unsigned)(8 * slots)), dim3(kSegNT), 0, A, lda, C, ldc, (int)Mp,
              bias, (int)tiles_m, ntiles, (int)xr, (int)local_m, segs);
   NNV_TRY(ctx->kernel_timer_end(timed, 0, flop));
   NNV_HIP_TRY(hipGetLastError());
@@ -380,11 +409,13 @@ int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {
   bool direct = true;
   int64_t wrows = 0;
   for (int64_t i = 0; i < count; ++i) {
-    direct = direct && sets[i].Wt != nullptr && sets[i].wfrom == 1 && sets[i].wend >= sets[i].ncols && sets[i].box == nullptr &&
-             sets[i].ldt % 4 == 0;
+    direct = direct && sets[i].Wt != nullptr && sets[i].wfrom == 1 && sets[i].wend >= sets[i].col0 + sets[i].ncols &&
+             sets[i].box == nullptr && sets[i].ldt % 4 == 0;
     wrows = std::max<int64_t>(wrows, sets[i].wrows);
   }
   direct = direct && wrows > 0 && ceil_div(wrows, kPackSlice) <= 65535;
+  for (int64_t i = 0; i < count; ++i)
+    if (sets[i].col0 != 0 && !direct) NNV_FAIL(NNVHIP_ERR_ARG, "internal: a column offset needs the rows of the weights");
   if (direct) {
     const int slices = (int)ceil_div(wrows, kPackSlice);
     hipLaunchKernelGGL(pack_rows_t_direct_kernel, dim3((unsigned)count, (unsigned)slices), dim3(256), 0, ctx->stream, table, sets[0],
@@ -398,10 +429,42 @@ int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets) {
   return NNVHIP_OK;
 }
 
+namespace {
+__global__ __launch_bounds__(256) void scaled_rows_kernel(ScaledRows a) {
+  const ScaledRows::One d = a.s[blockIdx.y];
+  const int r = blockIdx.x;  // row `rows` is the row of zeros
+  if (r > d.rows) return;
+  double* o = d.out + (int64_t)r * d.ld;
+  const double* w = d.Wt + (int64_t)min(r, d.rows - 1) * d.ldwt;
+  for (int j = threadIdx.x; j < d.ld; j += 256) {
+    double v = 0.0;
+    if (r < d.rows && j >= 1 && j < d.ncols) {  // the value the gather pass would write, as the packing kernels form it
+      const int src = d.idx[j - 1];
+      v = __dadd_rn(0.0, __dmul_rn(w[src], d.scale ? d.scale[src] : 1.0));
+    }
+    o[j] = v;
+  }
+}
+}  // namespace
+
+int launch_scaled_rows(nnvhip_ctx* ctx, const ScaledRows& a) {
+  if (a.count < 1 || a.count > 16) NNV_FAIL(NNVHIP_ERR_ARG, "internal: one to sixteen matrices per launch");
+  int32_t max_rows = 0;
+  for (int k = 0; k < a.count; ++k) {
+    if (a.s[k].rows <= 0 || a.s[k].ncols > a.s[k].ld) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: scaled rows out of range");
+    max_rows = std::max(max_rows, a.s[k].rows);
+  }
+  hipLaunchKernelGGL(scaled_rows_kernel, dim3((unsigned)(max_rows + 1), (unsigned)a.count), dim3(256), 0, ctx->stream, a);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
 int launch_gemm_seg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
-                    int tn, const SegTile* segs, int64_t ntiles, double flop) {
+                    int tn, const SegTile* segs, int64_t ntiles, double flop, bool gather_b) {
   if (ntiles == 0) return NNVHIP_OK;
   if (Mp % 16 || lda % 2 || Mp > ldc) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: GEMM operands violate the padding contract");
+  if (gather_b && tn != 128) NNV_FAIL(NNVHIP_ERR_ARG, "internal: rows of B are gathered by the 128-column tile only");
+  if (gather_b) return launch_seg_cfg<128, 2, 4, 4, 2, true>(ctx, A, lda, C, ldc, Mp, bias, segs, ntiles, flop);
   switch (tn) {
     case 128: return launch_seg_cfg<128, 2, 4, 4, 2>(ctx, A, lda, C, ldc, Mp, bias, segs, ntiles, flop);
     case 64: return launch_seg_cfg<64, 4, 2, 2, 2>(ctx, A, lda, C, ldc, Mp, bias, segs, ntiles, flop);

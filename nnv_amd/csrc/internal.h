@@ -487,6 +487,8 @@ struct PackSet {
   int32_t wend = 0;
   int32_t zero_to = 0;  // > 1: columns [1, zero_to) are +0 whatever the memory holds
   int64_t ldt = 0;      // launch_pack_rows_t: Vk is kp x ldt, row-major (columns [ncols, ldt) are written as zeros)
+  int32_t col0 = 0;     // launch_pack_rows_t, rows of the weights only: packed column j is the set's column col0 + j
+                        // (ncols counts from there)
   // columns [box_from, box_to) are +0 outside their windows box[j] (images of bH x bW positions per channel),
   // whatever the memory holds there (box == null: none)
   const ColBox* box = nullptr;
@@ -502,10 +504,17 @@ int launch_pack_rows(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
 // number in the set (col_local0 + offset) is 0 and, with rpart, the tile's four range sums ([4][ldc]).
 struct SegTile {
   const int32_t* kmap;  // kp entries (a multiple of 16), -1 where the list is padded
-  const double* Bt;     // the set's packed rows, transposed: kp x ldbt, row-major (launch_pack_rows_t)
+  const double* Bt;     // the set's packed rows, transposed: kp x ldbt, row-major (launch_pack_rows_t); or, with
+                        // gather_b, a matrix shared by all sets whose row kmap[t] is the set's packed row t
   int64_t ldbt;
+  int64_t b_col0;       // the tile's first column in Bt
   int64_t col_local0;   // the tile's first column in the set's own numbering
   int64_t col_base;     // ... and in C
+  // gather_b (128-column tiles only): Bt holds one row per input row plus a row of zeros at index zero_row (for
+  // the padded entries of kmap); a tile with col_local0 == 0 takes its column 0 from centre[kmap[t]] instead
+  const double* centre;
+  int32_t gather_b;
+  int32_t zero_row;
   int32_t kp;
   int32_t valid;        // columns of the tile that exist
   const double* plb;    // the set's predicate bounds (indexed by generator column), for the range sums
@@ -514,7 +523,22 @@ struct SegTile {
 };
 int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
 int launch_gemm_seg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
-                    int tn, const SegTile* segs, int64_t ntiles, double flop);
+                    int tn, const SegTile* segs, int64_t ntiles, double flop, bool gather_b = false);
+// The matrices the gathering tiles read, up to 16 per launch: row r < rows of one is [0, Wt(r, idx[j - 1]) *
+// scale[idx[j - 1]] for 1 <= j < ncols, zeros up to ld], row `rows` is all zeros.  out: (rows + 1) x ld, row-major.
+struct ScaledRows {
+  struct One {
+    const double* Wt;
+    int64_t ldwt;
+    const int32_t* idx;
+    const double* scale;
+    double* out;
+    int64_t ld;
+    int32_t rows, ncols;
+  } s[16];
+  int32_t count;
+};
+int launch_scaled_rows(nnvhip_ctx* ctx, const ScaledRows& a);
 // A split-K product leaves `ksplit` partial matrices (Mp x ncols each, ld = Mp) in a workspace; a caller
 // that has a pass over the output coming anyway can take the workspace instead of having the reduction
 // kernel launched (sum in split order, then the bias on column 0).  ksplit = 1: C is final.

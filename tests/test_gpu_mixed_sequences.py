@@ -209,3 +209,24 @@ def test_one_wide_set_through_the_tile_kernel(nnv, oracle, method):
     args = (V, np.zeros((1, n)), np.zeros(1), -np.ones(n), np.ones(n))
     layers = [{"type": "relu"}, _fc(rs, 520, N, 2.0), {"type": "relu"}, _fc(rs, 20, 520)]
     _compare(nnv, oracle, layers, nnv.Star(*args), oracle.OStar(*args), method)
+
+
+@pytest.mark.parametrize("shapes", [1, 3, 40])
+def test_arrays_of_boxes_that_share_their_half_widths(nnv, oracle, shapes):
+    # 64 boxes with `shapes` different half-width vectors among them: sets of one shape gather the same scaled weight
+    # columns, so the second FC layer reads their packed rows from one matrix per shape (up to 16 shapes; with more
+    # every set packs its own rows).  201 columns per set: one whole 128-column tile and a 73-column remainder.
+    rs = np.random.RandomState(500 + shapes)
+    n_in, count = 200, 64
+    # (centres and half-widths on a binary grid: lb, ub and 0.5 * (ub - lb) are then exact, and sets of one shape
+    # have the same half-widths to the bit, which is what the library looks for)
+    widths = rs.randint(1, 128, size=(n_in, shapes)) / 4096.0
+    widths[rs.randint(n_in), :] = 0.0 if shapes == 3 else widths[0, :]    # a degenerate dimension in one of the cases
+    half = widths[:, np.arange(count) % shapes]
+    centre = rs.randint(0, 1024, size=(n_in, count)) / 1024.0
+    lbs, ubs = centre - half, centre + half
+    assert np.array_equal(0.5 * (ubs - lbs), half)
+    layers = [_fc(rs, 300, n_in, 2.0), {"type": "relu"}, _fc(rs, 300, 300, 2.0), {"type": "relu"}, _fc(rs, 6, 300)]
+    dev_in = nnv.Star.from_boxes(lbs, ubs)
+    ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
+    _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area")
