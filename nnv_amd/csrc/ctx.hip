@@ -619,13 +619,19 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
   // weight columns.  shape_of[s] = the first set with set s's half-widths (among the first few distinct shapes).
   std::vector<int64_t> shape_of((size_t)count);
   std::vector<int64_t> shapes;
+  std::vector<uint64_t> shape_hash;
   for (int64_t s = 0; s < count; ++s) {
     int64_t n = 0;
+    uint64_t hash = 0x9E3779B97F4A7C15ull;  // of the half-widths' bit patterns: vectors are compared only when it matches
     for (int64_t i = 0; i < N; ++i) {
       double l = lb[s * N + i], u = ub[s * N + i];
       center[s * N + i] = 0.5 * (l + u);
       double v = 0.5 * (u - l);
       vec[s * N + i] = v;
+      uint64_t bits;
+      memcpy(&bits, &v, sizeof bits);
+      hash = (hash ^ bits) * 0x100000001B3ull;
+      hash ^= hash >> 29;
       if (v < 0.0) neg_scale[s] = 1;
       // zero columns are deleted only when the generator matrix has more than one element
       if (v != 0.0 || N == 1) {
@@ -636,12 +642,15 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
     gen_off[s + 1] = gen_off[s] + n;
     col_off[s + 1] = col_off[s] + n + 1;
     shape_of[s] = s;
-    for (int64_t r : shapes)
-      if (memcmp(&vec[r * N], &vec[s * N], sizeof(double) * N) == 0) {
-        shape_of[s] = r;
+    for (size_t k = 0; k < shapes.size(); ++k)
+      if (shape_hash[k] == hash && memcmp(&vec[shapes[k] * N], &vec[s * N], sizeof(double) * N) == 0) {
+        shape_of[s] = shapes[k];
         break;
       }
-    if (shape_of[s] == s && shapes.size() < 16) shapes.push_back(s);
+    if (shape_of[s] == s && shapes.size() < 16) {
+      shapes.push_back(s);
+      shape_hash.push_back(hash);
+    }
   }
   int64_t ld = round_up(N, kLdAlign);
   int64_t total_cols = col_off[count];
