@@ -688,7 +688,7 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
     st->V = arena->as<double>() + col_off[s] * ld;
     st->pbuf = pb;
     int64_t npad = round_up(std::max<int64_t>(st->n, 1), kLdAlign);
-    st->plb = pb->as<double>() + poff[s];
+    st->plb = pb->as<double>() + poff[shape_of[s]];  // (the same -1 / +1 for every set of the shape)
     st->pub = st->plb + npad;
     // C = zeros(1, n), d = 0 (set/Star.m:226-227): a base node with one all-zero row
     auto base = std::make_shared<ConsNode>();
@@ -1254,6 +1254,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
   // (see below).  Nothing of it depends on the outputs, so it is queued before anything else: the device
   // works on it while the host sets up the outputs and the tiles of the contraction.
   BufRef mm_early;
+  std::vector<int64_t> mm_slot;  // which pair of the product's columns holds a set's sums
   int st = NNVHIP_OK;
   if (count >= 64 && !c->eager_cols && !c->dense_affine) {
     std::vector<GatherSet> es((size_t)count);
@@ -1272,7 +1273,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       ok = ok && !(g.m > 0 && in[i]->oh_scale_neg);
       any = any || g.m > 0;
     }
-    if (ok && any) st = launch_range_sums_mm(c, fc, count, es.data(), &mm_early);
+    if (ok && any) st = launch_range_sums_mm(c, fc, count, es.data(), &mm_early, &mm_slot);
   }
   if (st == NNVHIP_OK) st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
   if (st == NNVHIP_OK) {
@@ -1832,7 +1833,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         }
         if (st == NNVHIP_OK && use_mm) {
           if (mm_early) mm_sums = mm_early;  // queued at the start of the call, from the same lists
-          else st = launch_range_sums_mm(c, fc, count, gs.data(), &mm_sums);
+          else st = launch_range_sums_mm(c, fc, count, gs.data(), &mm_sums, &mm_slot);
         }
         if (st == NNVHIP_OK) {
           for (int64_t i = 0; i < count; ++i) {
@@ -1856,7 +1857,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         }
         if (mm) {
           outs[i]->rng_mm_buf = mm_sums;
-          outs[i]->rng_mm = mm_sums->as<double>() + 4 * outs[0]->ld * i;  // two columns of 2 * ld entries per set
+          outs[i]->rng_mm = mm_sums->as<double>() + 4 * outs[0]->ld * mm_slot[(size_t)i];  // two columns of 2 * ld entries
         }
         outs[i]->rng_first_col = (filled[i] || tiles_of[i] > 0) ? 1 : dense[i];
       }

@@ -637,7 +637,8 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 // with a = scatter(sc * plb), b = scatter(sc * pub) per set, [max(W,0); min(W,0)] * [a b] holds
 // [xmin1; xmax2] and [xmax1; xmin2].  One fp64 MFMA product over all sets instead of a pass over the
 // cache-resident weights per set.  out: 2*Mp x 2*count, ld = 2*Mp, columns 2i and 2i+1 belong to set i.
-int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out);
+int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out,
+                         std::vector<int64_t>* slot);  // slot[i]: which pair of columns of `out` holds set i's sums
 // lb / ub (and, by centre_mode, the centre column) of a fully connected layer's output for one set whose
 // gathered columns need no pass of their own, finished in one kernel (ranges.hip).
 int launch_fc_rowsum(nnvhip_ctx* ctx, const nnvhip_fc* fc, nnvhip_star* out, int mode, const double* scale, const int32_t* cls,

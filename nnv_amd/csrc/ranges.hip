@@ -933,7 +933,8 @@ __global__ __launch_bounds__(256) void sum_vectors_kernel(const GatherSet* __res
   }
 }
 
-int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out) {
+int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out,
+                         std::vector<int64_t>* slot) {
   const int64_t Mp = fc->Mp, Kp = fc->Kp;
   if (!fc->Wpn) {
     BufRef w;
@@ -943,13 +944,31 @@ int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, co
     NNV_HIP_TRY(hipGetLastError());
     fc->Wpn = w;
   }
+  // Sets that gather the same columns with the same scales under the same bounds (the boxes of one shape,
+  // nnvhip_star_from_box) have the same sums: one pair of columns serves them all.  Only runs of a few distinct
+  // descriptions are looked for (a set is compared with the last 16 new ones).
+  std::vector<GatherSet> uniq;
+  slot->assign((size_t)count, 0);
+  for (int64_t i = 0; i < count; ++i) {
+    int64_t found = -1;
+    for (int64_t k = (int64_t)uniq.size() - 1; k >= 0 && k >= (int64_t)uniq.size() - 16 && found < 0; --k) {
+      const GatherSet& u = uniq[(size_t)k];
+      if (u.idx == sets[i].idx && u.scale == sets[i].scale && u.plb == sets[i].plb && u.pub == sets[i].pub && u.m == sets[i].m) found = k;
+    }
+    if (found < 0) {
+      found = (int64_t)uniq.size();
+      uniq.push_back(sets[i]);
+    }
+    (*slot)[(size_t)i] = found;
+  }
+  const int64_t nu = (int64_t)uniq.size();
   BufRef X, tab;
-  NNV_TRY(ctx->alloc(sizeof(double) * Kp * 2 * count, &X));
-  NNV_TRY(ctx->upload(sets, sizeof(GatherSet) * count, &tab));
-  hipLaunchKernelGGL(sum_vectors_kernel, dim3((unsigned)count), dim3(256), 0, ctx->stream, tab->as<GatherSet>(), X->as<double>(), (int)Kp);
+  NNV_TRY(ctx->alloc(sizeof(double) * Kp * 2 * nu, &X));
+  NNV_TRY(ctx->upload(uniq.data(), sizeof(GatherSet) * nu, &tab));
+  hipLaunchKernelGGL(sum_vectors_kernel, dim3((unsigned)nu), dim3(256), 0, ctx->stream, tab->as<GatherSet>(), X->as<double>(), (int)Kp);
   NNV_HIP_TRY(hipGetLastError());
-  NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * count, out));
-  return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, 2 * count, Kp,
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * nu, out));
+  return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, 2 * nu, Kp,
                      nullptr);
 }
 
