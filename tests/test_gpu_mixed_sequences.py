@@ -211,11 +211,12 @@ def test_one_wide_set_through_the_tile_kernel(nnv, oracle, method):
     _compare(nnv, oracle, layers, nnv.Star(*args), oracle.OStar(*args), method)
 
 
-@pytest.mark.parametrize("shapes", [1, 3, 40])
-def test_arrays_of_boxes_that_share_their_half_widths(nnv, oracle, shapes):
+@pytest.mark.parametrize("shapes,hidden", [(1, 300), (3, 300), (40, 300), (2, 1400)])
+def test_arrays_of_boxes_that_share_their_half_widths(nnv, oracle, shapes, hidden):
     # 64 boxes with `shapes` different half-width vectors among them: sets of one shape gather the same scaled weight
     # columns, so the second FC layer reads their packed rows from one matrix per shape (up to 16 shapes; with more
     # every set packs its own rows).  201 columns per set: one whole 128-column tile and a 73-column remainder.
+    # With 1400 hidden neurons a set keeps more than 512 rows: kept-row lists of more than 64 stages of eight.
     rs = np.random.RandomState(500 + shapes)
     n_in, count = 200, 64
     # (centres and half-widths on a binary grid: lb, ub and 0.5 * (ub - lb) are then exact, and sets of one shape
@@ -226,7 +227,7 @@ def test_arrays_of_boxes_that_share_their_half_widths(nnv, oracle, shapes):
     centre = rs.randint(0, 1024, size=(n_in, count)) / 1024.0
     lbs, ubs = centre - half, centre + half
     assert np.array_equal(0.5 * (ubs - lbs), half)
-    layers = [_fc(rs, 300, n_in, 2.0), {"type": "relu"}, _fc(rs, 300, 300, 2.0), {"type": "relu"}, _fc(rs, 6, 300)]
+    layers = [_fc(rs, hidden, n_in, 2.0), {"type": "relu"}, _fc(rs, 300, hidden, 2.0), {"type": "relu"}, _fc(rs, 6, 300)]
     dev_in = nnv.Star.from_boxes(lbs, ubs)
     ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
     _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area")
