@@ -176,21 +176,41 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   }
 }
 
+// What the kernels that settle the order of a crossing list write besides the list: kRankNewBounds: the bounds
+// of the new predicates (new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]) and the crossing
+// neurons' (lb, ub); kRankOldBounds: also the copy of the bounds of the predicates the set already has.
+constexpr int kRankNewBounds = 1, kRankOldBounds = 2;
+
 // Sorts a crossing list of at most 1024 entries that the multi-block classification left in
-// ascending order (keys in d.key, neurons in d.asc_idx).  One block per set.
-__global__ __launch_bounds__(1024) void relu_sort_small_kernel(const ReluDesc* __restrict__ table, ReluDesc one) {
+// ascending order (keys in d.key, neurons in d.asc_idx).  One block per set; every thread ends up with entry
+// tid of the sorted list and writes that predicate's bounds itself (see the flags above).
+__global__ __launch_bounds__(1024) void relu_sort_small_kernel(const ReluDesc* __restrict__ table, ReluDesc one, int flags) {
   const ReluDesc d = table ? table[blockIdx.x] : one;
   const int m = d.m;
+  const int tid = threadIdx.x;
+  const int n_in = d.ncols_in - 1;
+  if (flags & kRankOldBounds) {
+    for (int j = tid; j < n_in; j += 1024) {
+      d.plb_out[j] = d.plb_in[j];
+      d.pub_out[j] = d.pub_in[j];
+    }
+  }
   if (m <= 0 || m > 1024) return;
   __shared__ double skey[1024];
   __shared__ int sidx[1024];
-  const int tid = threadIdx.x;
   if (tid < m) {
     skey[tid] = d.key[tid];
     sidx[tid] = d.asc_idx[tid];
   }
   __syncthreads();
-  sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
+  const int mine = sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
+  if ((flags & kRankNewBounds) && tid < m) {
+    const double ub = d.ub[mine];
+    d.plb_out[n_in + tid] = 0.0;
+    d.pub_out[n_in + tid] = ub;
+    d.lbub[tid] = d.lb[mine];
+    d.lbub[d.ld_lbub + tid] = ub;
+  }
 }
 
 // Multi-block classification for sets with more than 1024 neurons: pass 1 counts the crossing and
@@ -311,7 +331,6 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
 // blocks also share out the copy of the bounds of the predicates the set already has.
 constexpr int kRankI = 16;
 constexpr int kRankStage = 2048;
-constexpr int kRankNewBounds = 1, kRankOldBounds = 2;
 __global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restrict__ table, ReluDesc one, int flags) {
   const ReluDesc d = table ? table[blockIdx.z] : one;
   const int m = d.m;
@@ -860,7 +879,10 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     table = tab->as<ReluDesc>();
   }
   if (sorted && sort_cap == 0 && max_m > 0 && max_m <= 1024) {
-    hipLaunchKernelGGL(relu_sort_small_kernel, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0]);
+    // (with the reset pending the kernel also writes the predicate bounds, as the rank kernel below does)
+    ranked_with_bounds = lazy_rows;
+    const int flags = lazy_rows ? (kRankNewBounds | (fold_bounds ? 0 : kRankOldBounds)) : 0;
+    hipLaunchKernelGGL(relu_sort_small_kernel, dim3((unsigned)count), dim3(1024), 0, ctx->stream, table, descs[0], flags);
   } else if (rank_lists) {
 
     // with the reset pending the kernel also writes the predicate bounds (the old ones were copied by the
