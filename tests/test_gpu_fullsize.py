@@ -153,3 +153,30 @@ def test_reach_is_deterministic(nnv):
     Va, la = a.V, a.estimateRanges()[0]
     b = net.reach(nnv.Star(cfg["lb"], cfg["ub"]), opts)
     assert np.array_equal(Va, b.V) and np.array_equal(la, b.estimateRanges()[0])   # no atomics on fp data
+
+
+def test_config4_full_against_the_recorded_oracle(nnv):
+    # The CPU oracle's answers for configuration 4 at full size (100 s and several GB on the host, recorded once by
+    # tests/golden/make_fullsize_fixtures.py): inactive counts and crossing lists in new-predicate order must match
+    # exactly, sampled entries of every layer's generator matrix and the output ranges within the tolerance.
+    import os
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "cfg4_fullsize_relax_star_area.npz"))
+    cfg = make_config(4)
+    assert int(gold["n_layers"][0]) == len(cfg["layers"])
+    dev_in, _ = input_sets(cfg)
+    net = nnv.NN.from_config(cfg["layers"], cfg["name"])
+    out = net.reach(dev_in, {"reachMethod": "relax-star-area", "relaxFactor": 1})
+    for li, (L, s) in enumerate(zip(cfg["layers"], net.reachSet)):
+        what = "cfg4 layer %d (%s)" % (li + 1, L["type"])
+        if L["type"] == "relu":
+            ni, idx, _, _ = s.relu_info()
+            assert ni == int(gold["inactive_%d" % li][0]), what + ": inactive count"
+            assert np.array_equal(idx, gold["crossing_%d" % li]), what + ": crossing list / order"
+        V = flat_V(s)
+        assert tuple(V.shape) == tuple(int(v) for v in gold["shape_%d" % li]), what + ": shape"
+        got = V[gold["rows_%d" % li], gold["cols_%d" % li]]
+        assert_close(got, gold["vals_%d" % li], what + ": sampled entries of V", 1e-9)
+        del V
+    olb, oub = (x.reshape(-1, order="F") for x in out.estimateRanges())
+    assert_close(olb, gold["out_lb"], "cfg4 output lb", 1e-9)
+    assert_close(oub, gold["out_ub"], "cfg4 output ub", 1e-9)

@@ -89,3 +89,30 @@ def test_relu_evaluate_known_answer(golden):
     # tests/nn/layers/ReluLayer/test_layers_relu.m:19-33
     g = golden["relu_evaluate"]
     assert np.array_equal(o.evaluate([{"type": "relu"}], g["IM"]), g["IM_out"])
+
+
+def test_recorded_fullsize_reach_is_consistent_with_its_configuration():
+    # tests/golden/cfg4_fullsize_relax_star_area.npz (written by make_fullsize_fixtures.py from the oracle at full
+    # size): layer count, matrix shapes and index ranges must fit configuration 4 as make_config builds it today,
+    # so a change of the synthetic inputs cannot silently leave a stale recording behind
+    import os
+    import numpy as np
+    from nnv_amd.configs import make_config
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "cfg4_fullsize_relax_star_area.npz"))
+    cfg = make_config(4)
+    assert int(gold["n_layers"][0]) == len(cfg["layers"])
+    n = cfg["lb"].size            # one predicate per pixel of the input box (no degenerate dimension)
+    assert np.all(cfg["ub"] > cfg["lb"])
+    for li, L in enumerate(cfg["layers"]):
+        N, cols = (int(v) for v in gold["shape_%d" % li])
+        if L["type"] == "relu":   # one new predicate per crossing neuron
+            idx = gold["crossing_%d" % li]
+            assert idx.min() >= 0 and idx.max() < N and np.unique(idx).size == idx.size
+            assert 0 <= int(gold["inactive_%d" % li][0]) <= N - idx.size
+            n += idx.size
+        assert cols == n + 1
+        assert gold["rows_%d" % li].max() < N and gold["cols_%d" % li].max() < cols
+        assert np.all(np.isfinite(gold["vals_%d" % li]))
+        if L["type"] == "fc":
+            assert N == len(L["b"])
+    assert gold["out_lb"].shape == gold["out_ub"].shape and np.all(gold["out_lb"] <= gold["out_ub"])
