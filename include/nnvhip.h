@@ -100,9 +100,10 @@ NNVHIP_API int nnvhip_set_eager_relu(nnvhip_ctx* ctx, int enabled);
  * dense GEMM kernel of the FC layers (tiles of at least 64 rows); 1: implicit-GEMM convolution
  * kernel; 2: estimateRanges column pass; 3: ReLU apply pass; 4: row-wise affine layers (row map,
  * average pooling, row permutation); 5: column gather of an FC layer (its one-hot generator columns);
- * 6: classification of the ReLU step (incl. the sort of the crossing list and, for sets of up to 8192
- * neurons, the new predicate bounds); 7: the reduction of range partial sums into lb / ub; 8: the
- * whole-reach kernel of small fully connected networks (nnvhip_reach_layers).
+ * 6: classification of the ReLU step (incl. the sort of the crossing list and, for small sets,
+ * the new predicate bounds); 7: the reduction of range partial sums into lb / ub; 8: the
+ * whole-reach kernel of small fully connected networks (nnvhip_reach_layers); 9: the tile kernel that
+ * contracts kept rows only, for arrays of sets and wide single sets (work: 2*Mp*kept*columns per set).
  * Returns accumulated kernel time,
  * launch count and work since the last reset.  Work is the flop executed for 0 and 1 (GEMM:
  * 2*Mp*Kp*ncols over the columns and rows the launch contracts, M and K padded to 16; conv:
