@@ -281,7 +281,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const double* __rest
   const int64_t total = (int64_t)Mp * ncols;
   if (t >= total) return;
   double s = 0.0;
-  for (int k = 0; k < ksplit; ++k) s += part[(int64_t)k * total + t];
+  for (int k0 = 0; k0 < ksplit; k0 += 16) {  // sixteen loads in flight, added in split order
+    double v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = k0 + u < ksplit ? part[(int64_t)(k0 + u) * total + t] : 0.0;
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      if (k0 + u < ksplit) s += v[u];
+  }
   const int64_t col = t / Mp;
   const int row = (int)(t - col * Mp);
   if (bias != nullptr && col == 0) s = s + bias[row];

@@ -843,8 +843,17 @@ __global__ __launch_bounds__(1024) void fc_rowsum_kernel(RowSumArgs a) {
     const int q = tid / kRowSumRows, r8 = tid % kRowSumRows;
     const int orow = blockIdx.x * kRowSumRows + r8;
     double x = 0.0;
-    if (a.part != nullptr)
-      for (int c = 0; c < a.chunks; ++c) x += a.part[((int64_t)c * 4 + q) * a.ld + orow];
+    if (a.part != nullptr) {
+      // (sixteen loads in flight at a time, added in chunk order: one at a time they cost a trip to memory each)
+      for (int c = 0; c < a.chunks; c += 16) {
+        double v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = c + u < a.chunks ? a.part[((int64_t)(c + u) * 4 + q) * a.ld + orow] : 0.0;
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+          if (c + u < a.chunks) x += v[u];
+      }
+    }
     const double Sp = red[0][0][r8], Sn = red[0][1][r8];
     double term;
     if (a.mode == 0) term = q == 0 ? -Sp : q == 1 ? Sn : q == 2 ? Sp : -Sn;
