@@ -583,13 +583,16 @@ __global__ void box_fill_kernel(double* __restrict__ V, int64_t ld, int N, const
   for (int64_t j = blockIdx.y; j < ncols; j += gridDim.y) {
     double* col = V + (col_off[set] + j) * ld;
     int dim = j == 0 ? -1 : gen_dim[gen_off[set] + j - 1];
-    for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < ld; r += gridDim.x * blockDim.x) {
-      double v = 0.0;
-      if (r < N) {
-        if (j == 0) v = center[(int64_t)set * N + r];
-        else if (r == dim) v = vec[(int64_t)set * N + r];
-      }
-      col[r] = v;
+    // two rows per thread, one 16-byte store (ld is even and every column starts on a 16-byte boundary)
+    for (int r = 2 * (blockIdx.x * blockDim.x + threadIdx.x); r < ld; r += 2 * gridDim.x * blockDim.x) {
+      double v[2] = {0.0, 0.0};
+#pragma unroll
+      for (int e = 0; e < 2; ++e)
+        if (r + e < N) {
+          if (j == 0) v[e] = center[(int64_t)set * N + r + e];
+          else if (r + e == dim) v[e] = vec[(int64_t)set * N + r + e];
+        }
+      *reinterpret_cast<double2*>(col + r) = make_double2(v[0], v[1]);
     }
   }
 }
@@ -664,7 +667,7 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
   NNV_TRY(c->upload(gen_off.data(), sizeof(int64_t) * gen_off.size(), &dgoff));
   int64_t max_cols = 0;
   for (int64_t s = 0; s < count; ++s) max_cols = std::max(max_cols, col_off[s + 1] - col_off[s]);
-  dim3 grid((unsigned)std::min<int64_t>(ceil_div(ld, 256), 64), (unsigned)std::min<int64_t>(max_cols, 4096),
+  dim3 grid((unsigned)std::min<int64_t>(ceil_div(ld, 512), 64), (unsigned)std::min<int64_t>(max_cols, 4096),
             (unsigned)count);
   hipLaunchKernelGGL(box_fill_kernel, grid, dim3(256), 0, c->stream, arena->as<double>(), ld, (int)N,
                      dcenter->as<double>(), dvec->as<double>(), dgen->as<int32_t>(), dcol->as<int64_t>(),
