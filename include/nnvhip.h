@@ -145,6 +145,17 @@ NNVHIP_API int nnvhip_pool_stats(nnvhip_ctx* ctx, int64_t* bytes_in_use, int64_t
  * first two. */
 NNVHIP_API int nnvhip_upload_stats(nnvhip_ctx* ctx, int64_t* weight_uploads, int64_t* weight_bytes, int64_t* h2d_bytes);
 
+/* The weight cache (see nnvhip_fc_create), no counterpart in the reference: the number of cached layers, the
+ * device bytes they hold, and how many of those bytes belong to layers that only the cache still references
+ * (every layer object made from them has been destroyed). */
+NNVHIP_API int nnvhip_weight_cache_stats(nnvhip_ctx* ctx, int64_t* entries, int64_t* device_bytes, int64_t* unreferenced_bytes);
+/* Frees every cached layer that only the cache still references (the library does so itself before it reports
+ * NNVHIP_ERR_OOM); *dropped (may be NULL) receives their number. */
+NNVHIP_API int nnvhip_weight_cache_release(nnvhip_ctx* ctx, int64_t* dropped);
+/* Test hook (no counterpart in the reference): with on != 0 every array hashes to the same value, so that a test
+ * can show that the cache tells layers apart by comparing their arrays, not by their hash.  Process-wide. */
+NNVHIP_API int nnvhip_debug_weak_weight_hash(int on);
+
 /* ---- sets ----------------------------------------------------------------------------- */
 /* Star(V, C, d, pred_lb, pred_ub), set/Star.m:153-189: uploads host arrays.  V is N x (n+1),
  * C is p x n, d has p entries; pred_lb/pred_ub may be NULL (both) for the -1/+1 default of
@@ -208,18 +219,23 @@ NNVHIP_API int nnvhip_estimate_ranges(nnvhip_ctx* ctx, nnvhip_star* s, double* l
 NNVHIP_API int nnvhip_estimate_ranges_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, double* lb,
                                  double* ub);
 
-/* Star.estimateRanges for callers that cannot allocate (no counterpart in the reference): code under
- * HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same kernels and the
+/* Star.estimateRanges for callers that cannot allocate (no counterpart in the reference): tight serving
+ * loops and harnesses that forbid hipMalloc (it allocates nothing, which is also what a caller under HIP
+ * graph capture needs, but the library has not been exercised under capture).  Same kernels and the
  * same results as nnvhip_estimate_ranges, but the partial sums of the column pass go to a fixed
  * workspace in device memory (32 MiB per GPU, held until the process ends) instead of the context's
  * pool, nothing is cached on the handle, and the call issues no hipMalloc / hipFree / pool request.
+ * A set whose handle already caches its ranges is served from that cache and uses no workspace.
  * lb_dev / ub_dev: DEVICE pointers to N doubles each (either may be NULL); they are written on the
  * context's stream (nnvhip_synchronize, or work queued on the same stream, orders later readers).
  * Limits: the set must be a plain stored matrix (sets made by nnvhip_star_create / _from_box always
  * are; a set whose rows or columns a layer left unwritten until first read is refused with
  * NNVHIP_ERR_ARG) and 6 * roundup(N, 16) doubles must fit the workspace (N <= 699040), else
- * NNVHIP_ERR_SHAPE.  All calls on one GPU share the workspace: calls that overlap on one GPU (two
- * contexts, two threads) race; calls on one context are ordered by its stream. */
+ * NNVHIP_ERR_SHAPE.  All calls on one GPU share the workspace.  Calls on one context are ordered by its
+ * stream; a call from another context of the same process first makes its stream wait for the previous
+ * user's kernels (an event per device), so contexts driven one after the other are safe; calls issued
+ * from several processes, or kernels of a caller's own that read lb_dev / ub_dev on another stream without
+ * synchronising, still race. */
 NNVHIP_API int nnvhip_estimate_ranges_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, double* ub_dev);
 
 /* ---- layers ---------------------------------------------------------------------------- */
@@ -228,9 +244,10 @@ NNVHIP_API int nnvhip_estimate_ranges_static(nnvhip_ctx* ctx, const nnvhip_star*
  * Weight cache: the reference passes weights by value (FullyConnectedLayer(W, b), Star.affineMap(W, b),
  * set/Star.m:313-343), so a caller that builds the layer again -- every call of affineMap, every NN object a
  * sweep over properties or a branch-and-bound loop constructs -- would upload the same arrays again.  Each
- * context therefore keeps the layers it has created, keyed by a 128-bit hash of W and b plus the geometry;
- * creating a layer whose arrays are resident returns that handle with one more reference and copies nothing
- * (nnvhip_upload_stats).  Every create is paired with a destroy as before; entries nobody else holds are
+ * context therefore keeps the layers it has created, found by a 128-bit hash of W and b plus the geometry and
+ * confirmed by comparing the caller's arrays byte for byte with the host copy the cache keeps (equal hashes
+ * alone never make a hit); creating a layer whose arrays are resident returns that handle with one more
+ * reference and copies nothing (nnvhip_upload_stats).  Every create is paired with a destroy as before; entries nobody else holds are
  * dropped least recently used first beyond NNVHIP_WEIGHT_CACHE_MB (environment, default 8192; 0 = no cache).
  * The same holds for nnvhip_conv2d_create. */
 NNVHIP_API int nnvhip_fc_create(nnvhip_ctx* ctx, const double* W, const double* b, int64_t M, int64_t K,

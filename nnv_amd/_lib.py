@@ -29,6 +29,7 @@ SYMBOLS = [
     "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists", "nnvhip_probe_mfma_peak",
     "nnvhip_estimate_ranges_static", "nnvhip_debug_mailbox_pack", "nnvhip_debug_mailbox_unpack",
     "nnvhip_debug_set_relu_call_number", "nnvhip_reach_layers", "nnvhip_relu_reduce_mem",
+    "nnvhip_weight_cache_stats", "nnvhip_weight_cache_release", "nnvhip_debug_weak_weight_hash",
 ]
 
 
@@ -113,6 +114,9 @@ def load():
         "nnvhip_debug_set_relu_call_number": [p, i64],
         "nnvhip_reach_layers": [p, i64, p, p, p, C.c_int, dbl, i64, pp, pp],
         "nnvhip_relu_reduce_mem": [p, p, i64, i64, i64, pp, p, p],
+        "nnvhip_weight_cache_stats": [p, pi64, pi64, pi64],
+        "nnvhip_weight_cache_release": [p, pi64],
+        "nnvhip_debug_weak_weight_hash": [C.c_int],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -229,6 +233,18 @@ class Context:
 
     def trim_pool(self):
         check(self.lib.nnvhip_trim_pool(self.handle))
+
+    def weight_cache_stats(self):
+        """(cached layers, their device bytes, device bytes of layers only the cache still references)."""
+        a, b, c = C.c_int64(), C.c_int64(), C.c_int64()
+        check(self.lib.nnvhip_weight_cache_stats(self.handle, C.byref(a), C.byref(b), C.byref(c)))
+        return a.value, b.value, c.value
+
+    def weight_cache_release(self) -> int:
+        """Frees the cached layers that no layer object references any more; returns how many went."""
+        n = C.c_int64()
+        check(self.lib.nnvhip_weight_cache_release(self.handle, C.byref(n)))
+        return n.value
 
 
 def default_context() -> Context:

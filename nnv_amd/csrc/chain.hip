@@ -325,7 +325,12 @@ __global__ __launch_bounds__(kChainThreads) void reach_chain_kernel(const ChainS
         s_counts[2 * l] = 0;
         s_counts[2 * l + 1] = 0;
       }
-      lds_barrier();
+      // A ReLU layer next reads the ranges from LDS and meets a full barrier before anybody loads the matrix; an FC
+      // layer next loads the matrix other waves have just stored, so their stores must have completed.
+      if (l + 1 < a.n_layers && a.layers[l + 1].kind == NNVHIP_LAYER_FC)
+        __syncthreads();
+      else
+        lds_barrier();
       V = O;
       Vsrc = O;
       plb_s = plb;

@@ -67,31 +67,42 @@ const TuneKnobs& tune_knobs() {
   return knobs;
 }
 
+static bool g_weak_weight_hash = false;  // test hook: every array hashes alike, so only the byte comparison tells layers apart
+
 void hash_bytes(const void* data, size_t bytes, uint64_t* h0, uint64_t* h1) {
   auto fold = [](uint64_t a, uint64_t b) {
     const __uint128_t r = (__uint128_t)a * b;
     return (uint64_t)r ^ (uint64_t)(r >> 64);
   };
+  auto rotl = [](uint64_t x, int r) { return (x << r) | (x >> (64 - r)); };
   const uint64_t k0 = 0xa0761d6478bd642full, k1 = 0xe7037ed1a0b428dbull, k2 = 0x8ebc6af09c88c6e3ull, k3 = 0x589965cc75374cc3ull;
+  if (g_weak_weight_hash) {
+    *h0 = k0;
+    *h1 = k1;
+    return;
+  }
   uint64_t a = k0 ^ bytes, b = k1 ^ bytes, c = k2 ^ bytes, d = k3 ^ bytes;
   const unsigned char* p = static_cast<const unsigned char*>(data);
   size_t i = 0;
-  for (; i + 32 <= bytes; i += 32) {  // four words a round, two independent pairs of streams
+  // Four words a round, four streams.  A product alone would forget its stream's past whenever one factor is zero
+  // (a block that equals the constants it is mixed with), so every stream also carries its previous state and
+  // the words along additively.
+  for (; i + 32 <= bytes; i += 32) {
     uint64_t w[4];
     memcpy(w, p + i, 32);
-    a = fold(a ^ w[0], k1 ^ w[1]);
-    b = fold(b ^ w[2], k2 ^ w[3]);
-    c = fold(c ^ w[1], k3 ^ w[2]);
-    d = fold(d ^ w[3], k0 ^ w[0]);
+    a = fold(a ^ w[0], k1 ^ w[1]) + rotl(a, 29) + w[1];
+    b = fold(b ^ w[2], k2 ^ w[3]) + rotl(b, 31) + w[3];
+    c = fold(c ^ w[1], k3 ^ w[2]) + rotl(c, 37) + w[2];
+    d = fold(d ^ w[3], k0 ^ w[0]) + rotl(d, 41) + w[0];
   }
   uint64_t tail[4] = {0, 0, 0, 0};
   if (i < bytes) memcpy(tail, p + i, bytes - i);
-  a = fold(a ^ tail[0], k1 ^ tail[1]);
-  b = fold(b ^ tail[2], k2 ^ tail[3]);
-  c = fold(c ^ tail[1], k3 ^ tail[2]);
-  d = fold(d ^ tail[3], k0 ^ tail[0]);
-  *h0 = fold(a ^ k2, b ^ k3) ^ a;
-  *h1 = fold(c ^ k0, d ^ k1) ^ d;
+  a = fold(a ^ tail[0], k1 ^ tail[1]) + rotl(a, 29) + tail[1];
+  b = fold(b ^ tail[2], k2 ^ tail[3]) + rotl(b, 31) + tail[3];
+  c = fold(c ^ tail[1], k3 ^ tail[2]) + rotl(c, 37) + tail[2];
+  d = fold(d ^ tail[3], k0 ^ tail[0]) + rotl(d, 41) + tail[0];
+  *h0 = fold(a ^ k2, b ^ k3) ^ a ^ rotl(b, 17);
+  *h1 = fold(c ^ k0, d ^ k1) ^ d ^ rotl(c, 19);
 }
 
 int enter_ctx(nnvhip_ctx* ctx) {
@@ -138,7 +149,8 @@ int nnvhip_ctx::alloc(size_t bytes, BufRef* out) {
     hipError_t e = hipMalloc(&p, cls);
     if (e != hipSuccess) {
       (void)hipGetLastError();
-      trim();  // let released arrays go, give cached blocks back and retry once
+      drop_unreferenced_weights();  // layers that only the weight cache still holds
+      trim();                       // let released arrays go, give cached blocks back and retry once
       e = hipMalloc(&p, cls);
       if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -236,6 +248,42 @@ void nnvhip_ctx::drop_weight_cache(bool all) {
       if (v->refs.fetch_sub(1) == 1) delete v;
     }
     weight_cache.erase(victim);
+  }
+}
+
+int64_t nnvhip_ctx::drop_unreferenced_weights() {
+  int64_t dropped = 0;
+  for (auto it = weight_cache.begin(); it != weight_cache.end();) {
+    const bool fc = it->first.kind == 0;
+    const int refs = fc ? static_cast<nnvhip_fc*>(it->second.handle)->refs.load()
+                        : static_cast<nnvhip_conv2d*>(it->second.handle)->refs.load();
+    if (refs > 1) {
+      ++it;
+      continue;
+    }
+    weight_cache_bytes -= it->second.bytes;
+    if (fc)
+      delete static_cast<nnvhip_fc*>(it->second.handle);
+    else
+      delete static_cast<nnvhip_conv2d*>(it->second.handle);
+    it = weight_cache.erase(it);
+    ++dropped;
+  }
+  return dropped;
+}
+
+// The cached layer that was made from exactly these host arrays, or null.  Entries whose hash and geometry agree
+// but whose arrays differ are stepped over by raising key.salt, which is then also the key a new entry goes under.
+static void* weight_cache_find(nnvhip_ctx* c, WeightKey* key, const double* W, size_t nw, const double* b, size_t nb) {
+  for (key->salt = 0;; ++key->salt) {
+    auto hit = c->weight_cache.find(*key);
+    if (hit == c->weight_cache.end()) return nullptr;
+    const WeightEntry& e = hit->second;
+    if (e.host_w.size() == nw && e.host_b.size() == nb && memcmp(e.host_w.data(), W, sizeof(double) * nw) == 0 &&
+        (nb == 0 || memcmp(e.host_b.data(), b, sizeof(double) * nb) == 0)) {
+      hit->second.last_use = ++c->weight_clock;
+      return e.handle;
+    }
   }
 }
 
@@ -494,6 +542,32 @@ int nnvhip_upload_stats(nnvhip_ctx* c, int64_t* weight_uploads, int64_t* weight_
   if (weight_uploads) *weight_uploads = c->weight_uploads;
   if (weight_bytes) *weight_bytes = c->weight_upload_bytes;
   if (h2d_bytes) *h2d_bytes = c->h2d_bytes;
+  return NNVHIP_OK;
+}
+
+int nnvhip_weight_cache_stats(nnvhip_ctx* c, int64_t* entries, int64_t* device_bytes, int64_t* unreferenced_bytes) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  int64_t unref = 0;
+  for (const auto& kv : c->weight_cache) {
+    const int refs = kv.first.kind == 0 ? static_cast<nnvhip_fc*>(kv.second.handle)->refs.load()
+                                        : static_cast<nnvhip_conv2d*>(kv.second.handle)->refs.load();
+    if (refs <= 1) unref += kv.second.bytes;
+  }
+  if (entries) *entries = (int64_t)c->weight_cache.size();
+  if (device_bytes) *device_bytes = c->weight_cache_bytes;
+  if (unreferenced_bytes) *unreferenced_bytes = unref;
+  return NNVHIP_OK;
+}
+
+int nnvhip_weight_cache_release(nnvhip_ctx* c, int64_t* dropped) {
+  CHECK_CTX(c);
+  const int64_t n = c->drop_unreferenced_weights();
+  if (dropped) *dropped = n;
+  return NNVHIP_OK;
+}
+
+int nnvhip_debug_weak_weight_hash(int on) {
+  g_weak_weight_hash = on != 0;
   return NNVHIP_OK;
 }
 
@@ -1039,11 +1113,9 @@ int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M,
     key.geo[4] = (int64_t)b1;
   }
   if (c->weight_cache_budget > 0) {
-    auto hit = c->weight_cache.find(key);
-    if (hit != c->weight_cache.end()) {
-      nnvhip_fc* f = static_cast<nnvhip_fc*>(hit->second.handle);
+    if (void* hit = weight_cache_find(c, &key, W, (size_t)(M * K), b, b ? (size_t)M : 0)) {
+      nnvhip_fc* f = static_cast<nnvhip_fc*>(hit);
       f->refs.fetch_add(1);
-      hit->second.last_use = ++c->weight_clock;
       c->live_handles++;
       *out = f;
       return NNVHIP_OK;
@@ -1078,7 +1150,9 @@ int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M,
     e.handle = *out;
     e.bytes = (int64_t)sizeof(double) * (*out)->Mp * ((*out)->Kp + 1);
     e.last_use = ++c->weight_clock;
-    c->weight_cache[key] = e;
+    e.host_w.assign(W, W + M * K);
+    if (b) e.host_b.assign(b, b + M);
+    c->weight_cache[key] = std::move(e);
     c->weight_cache_bytes += e.bytes;
     c->drop_weight_cache(false);
   }
@@ -1120,11 +1194,9 @@ int nnvhip_conv2d_create(nnvhip_ctx* c, const double* W, const double* bias, int
     key.geo[11] = (int64_t)b1;
   }
   if (c->weight_cache_budget > 0) {
-    auto hit = c->weight_cache.find(key);
-    if (hit != c->weight_cache.end()) {
-      nnvhip_conv2d* v = static_cast<nnvhip_conv2d*>(hit->second.handle);
+    if (void* hit = weight_cache_find(c, &key, W, (size_t)(FH * FW * Cin * Cout), bias, bias ? (size_t)Cout : 0)) {
+      nnvhip_conv2d* v = static_cast<nnvhip_conv2d*>(hit);
       v->refs.fetch_add(1);
-      hit->second.last_use = ++c->weight_clock;
       c->live_handles++;
       *out = v;
       return NNVHIP_OK;
@@ -1166,7 +1238,9 @@ int nnvhip_conv2d_create(nnvhip_ctx* c, const double* W, const double* bias, int
     e.handle = *out;
     e.bytes = (int64_t)sizeof(double) * (((*out)->Kp + 1) * Cout + ((*out)->Wk ? (*out)->Kp * (*out)->coutp : 0));
     e.last_use = ++c->weight_clock;
-    c->weight_cache[key] = e;
+    e.host_w.assign(W, W + FH * FW * Cin * Cout);
+    if (bias) e.host_b.assign(bias, bias + Cout);
+    c->weight_cache[key] = std::move(e);
     c->weight_cache_bytes += e.bytes;
     c->drop_weight_cache(false);
   }

@@ -164,8 +164,10 @@ struct WeightKey {
   uint64_t h0 = 0, h1 = 0;
   int64_t geo[12] = {};
   int kind = 0;  // 0 fc, 1 conv2d
+  int salt = 0;  // > 0: another layer whose hash and geometry equal those of the entries with lower salts
   bool operator<(const WeightKey& o) const {
     if (kind != o.kind) return kind < o.kind;
+    if (salt != o.salt) return salt < o.salt;
     if (h0 != o.h0) return h0 < o.h0;
     if (h1 != o.h1) return h1 < o.h1;
     for (int i = 0; i < 12; ++i)
@@ -175,10 +177,14 @@ struct WeightKey {
 };
 struct WeightEntry {
   void* handle = nullptr;  // nnvhip_fc* / nnvhip_conv2d*; the cache owns one reference
+  // The host arrays the layer was made from, by value.  A hit on the hash is only taken after they compare equal
+  // to the caller's arrays: equal hashes prove nothing, and a wrong hit would run another network's weights.
+  std::vector<double> host_w, host_b;
   int64_t bytes = 0;
   uint64_t last_use = 0;
 };
-// 128-bit content hash (two multiply-fold streams with different constants) of a host array
+// 128-bit content hash (multiply-fold streams that carry their previous state along) of a host array; only a
+// filter in front of the byte-wise comparison
 void hash_bytes(const void* data, size_t bytes, uint64_t* h0, uint64_t* h1);
 
 }  // namespace nnvhip
@@ -223,6 +229,8 @@ struct nnvhip_ctx {
   // bytes the library copied from host to device (sets, bounds, descriptor tables, weights)
   int64_t weight_uploads = 0, weight_upload_bytes = 0, h2d_bytes = 0;
   void drop_weight_cache(bool all);
+  // frees the device memory of every cached layer that nobody but the cache holds; returns how many went
+  int64_t drop_unreferenced_weights();
   uint32_t mailbox_seq = 0;  // number of the ReLU call (wraps; only its low 16 bits travel, as a cross-check)
   // FC layers as the full dense contraction (no skipping of structural zeros); default from the
   // environment variable NNVHIP_DENSE_AFFINE

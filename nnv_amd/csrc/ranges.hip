@@ -9,6 +9,8 @@
 
 #include "internal.h"
 
+#include <mutex>
+
 namespace nnvhip {
 
 struct RangeDesc {
@@ -1198,11 +1200,30 @@ int finalize_fused_ranges(nnvhip_ctx* ctx, nnvhip_star* s, const BufRef& part, i
 constexpr int64_t kStaticScratchDoubles = int64_t(4) << 20;  // 32 MiB per GPU, held until the process ends
 static __device__ __align__(256) double scratch[kStaticScratchDoubles];
 
+// Every context has a stream of its own, and all contexts on one GPU share the array: the last use on each
+// device is marked by an event, and a call from another context makes its stream wait for that event first, so
+// that calls from several contexts of one host thread (or of threads that do not overlap in time) are ordered
+// on the device as well.  The events are made when a device sees its first context and live until the process ends.
+namespace {
+constexpr int kMaxDevices = 64;
+struct StaticUse {
+  hipEvent_t done = nullptr;
+  const nnvhip_ctx* last = nullptr;  // whose stream recorded `done` (compared, never dereferenced)
+};
+StaticUse g_static_use[kMaxDevices];
+std::mutex g_static_use_mutex;
+}  // namespace
+
 int init_static_scratch(nnvhip_ctx* ctx) {
   void* p = nullptr;
   NNV_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
   ctx->static_scratch = static_cast<double*>(p);
   ctx->static_scratch_doubles = kStaticScratchDoubles;
+  if (ctx->device >= 0 && ctx->device < kMaxDevices) {
+    std::lock_guard<std::mutex> lock(g_static_use_mutex);
+    StaticUse& u = g_static_use[ctx->device];
+    if (u.done == nullptr) NNV_HIP_TRY(hipEventCreateWithFlags(&u.done, hipEventDisableTiming));
+  }
   return NNVHIP_OK;
 }
 
@@ -1218,6 +1239,14 @@ __global__ __launch_bounds__(256) void copy_ranges_kernel(const double* __restri
 
 int ranges_into_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, double* ub_dev) {
   if (ctx->static_scratch == nullptr) NNV_FAIL(NNVHIP_ERR_HIP, "internal: the static workspace has no address on this device");
+  if (s->lb != nullptr && s->ub != nullptr) {
+    // the handle already caches its ranges (an earlier estimateRanges, a producing layer): no workspace is needed
+    hipLaunchKernelGGL(copy_ranges_kernel, dim3((unsigned)ceil_div(s->N, 256)), dim3(256), 0, ctx->stream, s->lb, s->ub, lb_dev,
+                       ub_dev, s->N);
+    NNV_HIP_TRY(hipGetLastError());
+    return NNVHIP_OK;
+  }
+  if (ctx->device < 0 || ctx->device >= kMaxDevices) NNV_FAIL(NNVHIP_ERR_ARG, "device number %d is out of range", ctx->device);
   // the set must be a plain stored matrix: writing pending columns or rows would need a buffer
   if (s->rows_pending || s->cs.any_pending() || s->stored_cols() != s->n + 1)
     NNV_FAIL(NNVHIP_ERR_ARG, "nnvhip_estimate_ranges_static: parts of this set are not in memory yet (read it once, or use "
@@ -1244,6 +1273,9 @@ int ranges_into_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, do
   d.chunks = (int32_t)chunks;
   d.cols_per_chunk = (int32_t)std::max<int64_t>(1, ceil_div(std::max<int64_t>(n, 1), chunks));
   d.row_waves = 1;
+  std::lock_guard<std::mutex> lock(g_static_use_mutex);
+  StaticUse& use = g_static_use[ctx->device];
+  if (use.last != nullptr && use.last != ctx) NNV_HIP_TRY(hipStreamWaitEvent(ctx->stream, use.done, 0));
   hipLaunchKernelGGL((ranges_partial_kernel<8, 4>), dim3((unsigned)row_blocks, (unsigned)chunks, 1), dim3(64 * kRangeWaves), 0,
                      ctx->stream, nullptr, d);
   if (chunks > 1)
@@ -1251,6 +1283,8 @@ int ranges_into_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, do
   hipLaunchKernelGGL(copy_ranges_kernel, dim3((unsigned)ceil_div(s->N, 256)), dim3(256), 0, ctx->stream, d.lb, d.ub, lb_dev, ub_dev,
                      s->N);
   NNV_HIP_TRY(hipGetLastError());
+  NNV_HIP_TRY(hipEventRecord(use.done, ctx->stream));
+  use.last = ctx;
   return NNVHIP_OK;
 }
 

@@ -110,3 +110,73 @@ def test_entries_nobody_holds_are_dropped_beyond_the_budget(nnv):
     assert ctx.upload_stats()[0] == 4
     assert np.array_equal(again, outs[0])
     del S
+
+
+def test_equal_hashes_are_not_a_hit(nnv):
+    """With every array hashing alike only the byte comparison can tell layers apart: two matrices of one shape
+    must give two layers and two different results, and each must be found again by its own values."""
+    from nnv_amd import _lib
+    lib = _lib.load()
+    ctx = _lib.Context(0)
+    rs = np.random.RandomState(11)
+    Wa, Wb = rs.randn(24, 16), rs.randn(24, 16)
+    b = rs.randn(24)
+    S = nnv.Star(-np.ones(16), np.ones(16), ctx=ctx)
+    _lib.check(lib.nnvhip_debug_weak_weight_hash(1))
+    try:
+        A = np.asarray(S.affineMap(Wa, b).V)
+        B = np.asarray(S.affineMap(Wb, b).V)
+        assert ctx.upload_stats()[0] == 2
+        assert_close(A, np.hstack([b[:, None], Wa]), "first layer", 1e-15)
+        assert_close(B, np.hstack([b[:, None], Wb]), "second layer (same hash, other values)", 1e-15)
+        A2 = np.asarray(S.affineMap(Wa.copy(), b.copy()).V)
+        B2 = np.asarray(S.affineMap(Wb.copy(), b.copy()).V)
+        assert ctx.upload_stats()[0] == 2, "layers with equal hashes were not found again by their values"
+        assert np.array_equal(A, A2) and np.array_equal(B, B2)
+        Bb = np.asarray(S.affineMap(Wb, b + 1.0).V)          # same matrix, other bias, same (weak) hash
+        assert ctx.upload_stats()[0] == 3
+        assert_close(Bb[:, 0], b + 1.0, "bias of the third layer", 1e-15)
+    finally:
+        _lib.check(lib.nnvhip_debug_weak_weight_hash(0))
+    del S
+
+
+def test_block_of_hash_constants_does_not_hide_what_came_before(nnv):
+    """Two matrices that differ only in front of a 32-byte block equal to the hash's own mixing constants (a product
+    that forgets its past would hash them alike) are different layers."""
+    ctx = nnv.default_context()
+    consts = np.array([0xa0761d6478bd642f, 0xe7037ed1a0b428db, 0x589965cc75374cc3, 0x8ebc6af09c88c6e3], dtype=np.uint64)
+    Wa = np.zeros((8, 2))
+    Wa.reshape(-1, order="F")[:4] = [1.0, 2.0, 3.0, 4.0]
+    flat = Wa.reshape(-1, order="F").copy()
+    flat[4:8] = consts.view(np.float64)
+    flat[8:] = 0.5
+    Wa = flat.reshape(8, 2, order="F")
+    Wb = Wa.copy()
+    Wb[0, 0] = -7.0
+    assert np.all(np.isfinite(Wa))
+    S = nnv.Star(-np.ones(2), np.ones(2))
+    u0 = ctx.upload_stats()[0]
+    A = np.asarray(S.affineMap(Wa).V)
+    B = np.asarray(S.affineMap(Wb).V)
+    assert ctx.upload_stats()[0] == u0 + 2
+    assert A[0, 1] == 1.0 and B[0, 1] == -7.0
+
+
+def test_unreferenced_layers_are_reported_and_released(nnv):
+    from nnv_amd import _lib
+    ctx = _lib.Context(0)
+    rs = np.random.RandomState(5)
+    S = nnv.Star(-np.ones(64), np.ones(64), ctx=ctx)
+    W = rs.randn(64, 64)
+    layer = nnv.FullyConnectedLayer(W, np.zeros(64))
+    out = layer.reach(S, "approx-star")
+    np.asarray(S.affineMap(rs.randn(64, 64)).V)              # its layer object is gone when affineMap returns
+    n, dev, unref = ctx.weight_cache_stats()
+    assert n == 2 and dev > 0 and 0 < unref < dev
+    assert ctx.weight_cache_release() == 1
+    n2, dev2, unref2 = ctx.weight_cache_stats()
+    assert n2 == 1 and unref2 == 0 and dev2 == dev - unref
+    again = layer.reach(S, "approx-star")                     # the layer somebody holds still works
+    assert np.array_equal(np.asarray(out.V), np.asarray(again.V))
+    del S, out, again, layer

@@ -63,3 +63,35 @@ def test_static_workspace_limits_are_errors():
     ctx.synchronize()
     assert np.array_equal(buf.get(), R.estimateRanges()[0])
     assert ctx.lib.nnvhip_estimate_ranges_static(ctx.handle, R._h.h, None, None) == _lib.ERR_ARG
+
+
+def test_two_contexts_share_the_workspace_in_turn_and_cached_ranges_need_none():
+    """Two contexts (two streams) on the one GPU call the entry point alternately without synchronising in
+    between: every result must be the context's own.  A handle that already caches its ranges is served from
+    the cache."""
+    import nnv_amd as nnv
+    from nnv_amd import _lib
+    from tests.gpu_util import DeviceDoubles
+    a, b = _lib.Context(0), _lib.Context(0)
+    rs = np.random.RandomState(9)
+    sets, outs = [], []
+    for i in range(6):
+        ctx = a if i % 2 == 0 else b
+        N, n = 1500 - 100 * i, 500 + 30 * i
+        V = rs.randn(N, n + 1)
+        S = nnv.Star(V, np.zeros((1, n)), np.zeros(1), -np.ones(n), np.ones(n), ctx=ctx)
+        lb_d, ub_d = DeviceDoubles(N), DeviceDoubles(N)
+        _lib.check(ctx.lib.nnvhip_estimate_ranges_static(ctx.handle, S._h.h, lb_d.ptr, ub_d.ptr))
+        sets.append((ctx, S))
+        outs.append((lb_d, ub_d))
+    a.synchronize()
+    b.synchronize()
+    for (ctx, S), (lb_d, ub_d) in zip(sets, outs):
+        elb, eub = S.estimateRanges()
+        assert np.array_equal(lb_d.get(), elb) and np.array_equal(ub_d.get(), eub)
+        # the handle now caches its ranges: the same call copies them and leaves the workspace alone
+        lb2 = DeviceDoubles(S.dim)
+        _lib.check(ctx.lib.nnvhip_estimate_ranges_static(ctx.handle, S._h.h, lb2.ptr, None))
+        ctx.synchronize()
+        assert np.array_equal(lb2.get(), elb)
+    del sets, outs, S
