@@ -308,6 +308,14 @@ NNVHIP_API int nnvhip_relu_reduce_mem(nnvhip_ctx* ctx, nnvhip_star* in, int64_t 
  * nnvhip_set_small_chain(ctx, 0) (or the environment variable NNVHIP_NO_SMALL_CHAIN) keeps such networks
  * on the layer-by-layer path. */
 NNVHIP_API int nnvhip_set_small_chain(nnvhip_ctx* ctx, int enabled);
+/* The switches a context reads from the environment when it is created, by name, for the rest of its life or
+ * until set again (no counterpart in the reference; they select between routes of this library that give the
+ * same sets, and exist so that a test suite can drive every route in one process): "dense_affine"
+ * (NNVHIP_DENSE_AFFINE), "eager_rows", "eager_tail", "eager_cols" (NNVHIP_EAGER_*), "poison_pending"
+ * (NNVHIP_POISON_PENDING: whatever a layer leaves unwritten until first read is filled with NaNs),
+ * "no_small_chain", "no_conv_mask", "no_conv_boxes" (NNVHIP_NO_*).  A switch applies to the layer calls made
+ * after it; sets produced before keep what they recorded.  Unknown name: NNVHIP_ERR_ARG. */
+NNVHIP_API int nnvhip_set_switch(nnvhip_ctx* ctx, const char* name, int enabled);
 enum { NNVHIP_LAYER_FC = 0, NNVHIP_LAYER_CONV2D = 1, NNVHIP_LAYER_RELU = 2 };
 NNVHIP_API int nnvhip_reach_layers(nnvhip_ctx* ctx, int64_t n_layers, const int32_t* kind, const void* const* layer,
                         const int64_t* hw, int order, double relax_factor, int64_t count, nnvhip_star* const* in,

@@ -29,8 +29,15 @@ SYMBOLS = [
     "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists", "nnvhip_probe_mfma_peak",
     "nnvhip_estimate_ranges_static", "nnvhip_debug_mailbox_pack", "nnvhip_debug_mailbox_unpack",
     "nnvhip_debug_set_relu_call_number", "nnvhip_reach_layers", "nnvhip_relu_reduce_mem",
-    "nnvhip_weight_cache_stats", "nnvhip_weight_cache_release", "nnvhip_debug_weak_weight_hash",
+    "nnvhip_set_switch", "nnvhip_weight_cache_stats", "nnvhip_weight_cache_release", "nnvhip_debug_weak_weight_hash",
 ]
+
+
+# route switches of a context (nnvhip_set_switch) and the environment variable each one starts from
+SWITCH_ENV = {"dense_affine": "NNVHIP_DENSE_AFFINE", "eager_rows": "NNVHIP_EAGER_ROWS", "eager_tail": "NNVHIP_EAGER_TAIL",
+              "eager_cols": "NNVHIP_EAGER_COLS", "poison_pending": "NNVHIP_POISON_PENDING",
+              "no_small_chain": "NNVHIP_NO_SMALL_CHAIN", "no_conv_mask": "NNVHIP_NO_CONV_MASK",
+              "no_conv_boxes": "NNVHIP_NO_CONV_BOXES"}
 
 
 class NNVHipError(RuntimeError):
@@ -114,6 +121,7 @@ def load():
         "nnvhip_debug_set_relu_call_number": [p, i64],
         "nnvhip_reach_layers": [p, i64, p, p, p, C.c_int, dbl, i64, pp, pp],
         "nnvhip_relu_reduce_mem": [p, p, i64, i64, i64, pp, p, p],
+        "nnvhip_set_switch": [p, C.c_char_p, C.c_int],
         "nnvhip_weight_cache_stats": [p, pi64, pi64, pi64],
         "nnvhip_weight_cache_release": [p, pi64],
         "nnvhip_debug_weak_weight_hash": [C.c_int],
@@ -165,6 +173,12 @@ class Context:
         self.release_set = lib.nnvhip_star_release   # looked up once: every set handle calls it when it dies
         self.release_sets = lib.nnvhip_star_release_array
         self.eager_columns = bool(os.environ.get("NNVHIP_EAGER_COLS"))
+        # the route switches as the library read them from the environment; set_switch keeps the mirror current
+        self.switches = {nm: os.environ.get(env) is not None for nm, env in SWITCH_ENV.items()}
+
+    def switch_is_on(self, *names) -> bool:
+        """Whether any of the named route switches is on (the Python side's record of nnvhip_set_switch)."""
+        return any(self.switches[nm] for nm in names)
 
     def synchronize(self):
         check(self.lib.nnvhip_synchronize(self.handle))
@@ -178,21 +192,25 @@ class Context:
         (default): those columns are written when somebody reads them."""
         check(self.lib.nnvhip_set_eager_columns(self.handle, 1 if enabled else 0))
         self.eager_columns = bool(enabled)
+        self.switches["eager_cols"] = bool(enabled)
 
     def set_eager_relu(self, enabled):
         """True: the ReLU step writes its whole output matrix in the call (reset rows zeroed, appended
         columns stored); False (default): both are recorded on the handle and written on first read."""
         check(self.lib.nnvhip_set_eager_relu(self.handle, 1 if enabled else 0))
+        self.switches["eager_rows"] = self.switches["eager_tail"] = bool(enabled)
 
     def set_small_chain(self, enabled):
         """True (default): NN.reach of a small FC / ReLU network is one launch (nnvhip_reach_layers); False: such
         networks go layer by layer like every other."""
         check(self.lib.nnvhip_set_small_chain(self.handle, 1 if enabled else 0))
+        self.switches["no_small_chain"] = not enabled
 
     def set_dense_affine(self, enabled):
         """True: FC layers run as the full dense contraction; False (default): products with the
         structural zeros recorded on the set handles are left out (same result)."""
         check(self.lib.nnvhip_set_dense_affine(self.handle, 1 if enabled else 0))
+        self.switches["dense_affine"] = bool(enabled)
 
     def last_op_time_ms(self) -> float:
         ms = C.c_double()
@@ -233,6 +251,13 @@ class Context:
 
     def trim_pool(self):
         check(self.lib.nnvhip_trim_pool(self.handle))
+
+    def set_switch(self, name: str, on: bool):
+        """One of the route switches a context otherwise reads from the environment (nnvhip_set_switch)."""
+        check(self.lib.nnvhip_set_switch(self.handle, name.encode(), 1 if on else 0))
+        self.switches[name] = bool(on)
+        if name == "eager_cols":
+            self.eager_columns = bool(on)
 
     def weight_cache_stats(self):
         """(cached layers, their device bytes, device bytes of layers only the cache still references)."""

@@ -423,6 +423,27 @@ int nnvhip_set_small_chain(nnvhip_ctx* c, int enabled) {
   return NNVHIP_OK;
 }
 
+int nnvhip_set_switch(nnvhip_ctx* c, const char* name, int enabled) {
+  if (!c || !name) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
+  const bool on = enabled != 0;
+  const struct {
+    const char* name;
+    bool* flag;
+    bool inverted;
+  } table[] = {
+      {"dense_affine", &c->dense_affine, false},   {"eager_rows", &c->eager_rows, false},
+      {"eager_tail", &c->eager_tail, false},       {"eager_cols", &c->eager_cols, false},
+      {"poison_pending", &c->poison_pending, false}, {"no_small_chain", &c->small_chain, true},
+      {"no_conv_mask", &c->no_conv_mask, false},   {"no_conv_boxes", &c->no_conv_boxes, false},
+  };
+  for (const auto& t : table)
+    if (strcmp(t.name, name) == 0) {
+      *t.flag = t.inverted ? !on : on;
+      return NNVHIP_OK;
+    }
+  NNV_FAIL(NNVHIP_ERR_ARG, "unknown switch '%s'", name);
+}
+
 int nnvhip_last_op_time_ms(nnvhip_ctx* c, double* ms) {
   if (!c || !ms) NNV_FAIL(NNVHIP_ERR_ARG, "null argument");
   *ms = c->last_ms;

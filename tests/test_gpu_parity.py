@@ -689,8 +689,7 @@ def test_conv_reads_through_a_pending_row_reset(nnv, oracle, H, W, Cin, Cout, FH
     import os
     rs = np.random.RandomState(H * 100 + Cout)
     out, exp, applies, mid = _relu_then_conv(nnv, oracle, rs, H, W, Cin, Cout, FH, FW, s, p, dil, n, count)
-    switched = any(os.environ.get(k) for k in ("NNVHIP_NO_CONV_MASK", "NNVHIP_EAGER_ROWS", "NNVHIP_EAGER_TAIL",
-                                               "NNVHIP_DENSE_AFFINE"))
+    switched = nnv.default_context().switch_is_on("no_conv_mask", "eager_rows", "eager_tail", "dense_affine")
     if not switched:
         assert applies == 0
     for R, E in zip(out, exp):
@@ -707,7 +706,7 @@ def test_conv_after_relu_on_an_image_too_large_for_the_row_mask(nnv, oracle):
     import os
     rs = np.random.RandomState(8)
     out, exp, applies, _ = _relu_then_conv(nnv, oracle, rs, 64, 64, 33, 40, 3, 3, 2, 1, 1, 2, spread=100.0)
-    if not os.environ.get("NNVHIP_EAGER_ROWS") and not os.environ.get("NNVHIP_EAGER_TAIL") and not os.environ.get("NNVHIP_DENSE_AFFINE"):
+    if not nnv.default_context().switch_is_on("eager_rows", "eager_tail", "dense_affine"):
         assert applies == 1
     compare_sets(out[0], exp[0], "conv after ReLU, large image")
 

@@ -54,7 +54,7 @@ def _check_against_oracle(nnv, oracle, layers, dev_in, ora_in, method, expect_ch
     ctx = nnv.default_context()
     net = nnv.NN.from_config(layers)
     out, launches = _chain_launches(ctx, lambda: net.reach(dev_in, {"reachMethod": method, "relaxFactor": 1}))
-    if os.environ.get("NNVHIP_NO_SMALL_CHAIN") or os.environ.get("NNVHIP_DENSE_AFFINE"):
+    if ctx.switch_is_on("no_small_chain", "dense_affine"):
         assert launches in (0, 1)     # a run under the switches that keep networks on the layer-by-layer path
     else:
         assert launches == (1 if expect_chain else 0)

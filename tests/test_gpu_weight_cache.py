@@ -146,9 +146,8 @@ def test_block_of_hash_constants_does_not_hide_what_came_before(nnv):
     that forgets its past would hash them alike) are different layers."""
     ctx = nnv.default_context()
     consts = np.array([0xa0761d6478bd642f, 0xe7037ed1a0b428db, 0x589965cc75374cc3, 0x8ebc6af09c88c6e3], dtype=np.uint64)
-    Wa = np.zeros((8, 2))
-    Wa.reshape(-1, order="F")[:4] = [1.0, 2.0, 3.0, 4.0]
-    flat = Wa.reshape(-1, order="F").copy()
+    flat = np.zeros(16)
+    flat[:4] = [1.0, 2.0, 3.0, 4.0]
     flat[4:8] = consts.view(np.float64)
     flat[8:] = 0.5
     Wa = flat.reshape(8, 2, order="F")
