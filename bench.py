@@ -148,6 +148,8 @@ def measure(k, args, ctx, exact_steps, extras):
 
     cfg = make_extended_cnn(32, 3) if k == 6 else make_config(k)
     ctx.set_dense_affine(args.dense)
+    ctx.set_eager_columns(args.written)
+    ctx.set_eager_relu(args.written)
     net = nnv_amd.NN.from_config(cfg["layers"], cfg["name"])
     opts = {"reachMethod": args.method, "relaxFactor": 1}
     dev_in = device_input_sets(cfg, ctx)
@@ -182,6 +184,25 @@ def measure(k, args, ctx, exact_steps, extras):
     ctx.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = 1e3 * wall / steps
+    # the same steps once more, each one bracketed by a synchronisation of its own: the spread of single steps
+    # (ms_per_step above is the mean of steps queued back to back, which is what `value` is quoted on)
+    each, slow = [], []
+    n_each = max(20, min(steps, 200))
+    for _ in range(n_each):
+        c0 = ctx.debug_counters()
+        t1 = time.perf_counter()
+        step()
+        ctx.synchronize()
+        each.append(1e3 * (time.perf_counter() - t1))
+        c1 = ctx.debug_counters()
+        if len(each) > 5 and each[-1] > 1.5 * float(np.median(each[:-1])):
+            used, cached = ctx.pool_stats()
+            slow.append({"step": len(each) - 1, "ms": round(each[-1], 4), "pool_bytes_in_use": used, "pool_bytes_cached": cached,
+                         "during_the_step": {k_: c1[k_] - c0[k_] for k_ in ("device_mallocs", "staging_waits")},
+                         "deferred_handles_before": c0["deferred_handles"], "deferred_handles_after": c1["deferred_handles"],
+                         "live_handles": c1["live_handles"]})
+    step_ms = {"n": n_each, "min": round(min(each), 5), "median": round(float(np.median(each)), 5), "max": round(max(each), 5),
+               "what": "single steps, each followed by a synchronisation", "steps_over_1p5x_median": slow[:8]}
     shapes = layer_shapes(net.reachSet)
     updates = count_updates(shapes)
     value = updates / (wall / steps)
@@ -331,7 +352,7 @@ def measure(k, args, ctx, exact_steps, extras):
         if n_sets < 256:
             c["latency_bound"] = True
         groups.append((cls_ms, c))
-    variant = "dense_contraction" if args.dense else ""
+    variant = "dense_contraction" if args.dense else "all_written" if args.written else ""
     for _, g in groups:
         if g["kernel"] in GROUP_KERNELS:
             g["kernels_in_group"] = list(GROUP_KERNELS[g["kernel"]])
@@ -407,7 +428,7 @@ def measure(k, args, ctx, exact_steps, extras):
     # read; the returned set and its bounds are always written.  Here every layer writes its whole output,
     # which is what the reference's NN.reachSet{i} holds.
     all_written = None
-    if not args.dense and "written" in extras:
+    if not args.dense and not args.written and "written" in extras:
         ctx.set_eager_columns(True)
         ctx.set_eager_relu(True)
         try:
@@ -420,9 +441,13 @@ def measure(k, args, ctx, exact_steps, extras):
                 step()
             ctx.synchronize()
             aw_ms = 1e3 * (time.perf_counter() - t1) / n_aw
+            aw_gbps = 8.0 * updates / (aw_ms * 1e-3) / 1e9
             all_written = {"ms_per_step": round(aw_ms, 5), "value": updates / (aw_ms * 1e-3), "steps": n_aw,
+                           "bytes_written_per_step": 8.0 * updates, "written_GBps": round(aw_gbps, 1),
+                           "frac_of_hbm_peak": round(aw_gbps / HBM_PEAK_GBS, 4),
                            "what": "the same step with every layer writing its whole output matrix in the call "
-                                   "(nothing left for a first read), as the reference's reachSet{i} holds it"}
+                                   "(nothing left for a first read), as the reference's reachSet{i} holds it; the rate "
+                                   "counts the bytes of those matrices only (8 bytes per update), not what the step reads"}
         finally:
             ctx.set_eager_columns(False)
             ctx.set_eager_relu(False)
@@ -456,10 +481,15 @@ def measure(k, args, ctx, exact_steps, extras):
 
     return {
         "value": value, "steps": steps, "warmup": args.warmup, "warm_steps_by_time": n_warm, "ms_per_step": ms_per_step,
+        "step_ms": step_ms,
         "config": {"workload": cfg["name"], "reach_method": args.method, "relax_factor": 1,
+                   "all_sets_written_ms": all_written["ms_per_step"] if all_written else None,
+                   "all_sets_written_updates_per_s": all_written["value"] if all_written else None,
+                   "all_sets_written_frac_of_hbm_peak": all_written["frac_of_hbm_peak"] if all_written else None,
                    "fc_affine_map": "dense" if args.dense else "structural zeros skipped (one-hot generator columns, reset rows); exact",
                    "sets": n_sets, "updates_per_step": updates,
                    "intermediate_sets": "dense" if args.dense else
+                   "every layer writes its whole output matrix in the call, as the reference's reachSet{i} holds it" if args.written else
                    "every layer's set is written in full by the one launch that reaches the whole network" if chain_launches else
                    "the sets between layers record a ReLU's row reset / appended columns and the columns an FC layer "
                    "gathers from its weights and write them on first read; the returned set and its bounds are written",
@@ -482,6 +512,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--dense", action="store_true",
                     help="run every FC layer as the full dense contraction (no skipping of structural zeros)")
+    ap.add_argument("--written", action="store_true",
+                    help="every layer writes its whole output matrix in the call (nothing is left for a first read): the "
+                         "all_sets_written figure of a default run as a run of its own, for profiles")
     ap.add_argument("--cpu-seconds", type=float, default=10.0,
                     help="budget of the headline's CPU baseline sample (the other configurations get a third each)")
     ap.add_argument("--lean", action="store_true",
@@ -506,20 +539,45 @@ def main():
             extras = cpu if args.lean else cpu | {"written"} | ({"dense"} if k == 2 else set())
             r = measure(k, args, ctx, False, extras)
             r = {"metric": "generator_neuron_updates_per_s", "unit": "updates/s", **{kk: r[kk] for kk in
-                 ("value", "ms_per_step", "steps", "config", "roofline", "all_sets_written", "cpu_baseline")}}
+                 ("value", "ms_per_step", "step_ms", "steps", "config", "roofline", "all_sets_written", "cpu_baseline")}}
             per_config.append(r)
         head = measure(5, args, ctx, True, cpu if args.lean else cpu | {"written", "spec", "h2h"})
     # practical ceilings on this box: a register-resident MFMA loop and a plain copy kernel over 1 GiB
     head["roofline"]["measured_mfma_TFLOPs"] = round(ctx.probe_mfma_peak(3), 2)
     head["roofline"]["measured_copy_GBps"] = round(ctx.probe_copy_bandwidth(1 << 30, 5), 1)
     ctx.trim_pool()
+    # HBM fractions are quoted against the datasheet's 8 TB/s; the same rates against what a plain copy kernel
+    # reaches on this box are put beside them
+    copy_gbps = head["roofline"]["measured_copy_GBps"]
+
+    def beside(r):
+        if r and r.get("bound") == "hbm" and copy_gbps > 0:
+            r["frac_of_measured_copy"] = round(r["achieved"] / copy_gbps, 4)
+        for g in (r or {}).get("other_kernels", []) + (r or {}).get("layer_by_layer_kernels", []):
+            beside(g)
+
+    for r in [head] + (per_config or []):
+        beside(r["roofline"])
+        if r.get("all_sets_written"):
+            r["all_sets_written"]["frac_of_measured_copy"] = round(r["all_sets_written"]["written_GBps"] / copy_gbps, 4)
+            r["config"]["all_sets_written_frac_of_measured_copy"] = r["all_sets_written"]["frac_of_measured_copy"]
+    cpu = head["cpu_baseline"]
+    if cpu and head["all_sets_written"]:
+        # the CPU oracle builds every set in full, so the like-for-like device figure is the all-sets-written one
+        cpu["device_over_cpu_all_sets_written"] = round(head["all_sets_written"]["value"] / cpu["value"], 1)
+        cpu["device_over_cpu_sets_described"] = round(head["value"] / cpu["value"], 1)
 
     print(json.dumps({
         "metric": "generator_neuron_updates_per_s", "value": head["value"], "unit": "updates/s", "n_gpus": 1,
         "steps": head["steps"], "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": head["config"], "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"],
-        "warm_steps_by_time": head["warm_steps_by_time"],
+        "warm_steps_by_time": head["warm_steps_by_time"], "step_ms": head["step_ms"],
+        "value_is": "reach with the sets between layers kept as descriptions (written on first read); the returned set and "
+                    "its bounds are written.  The figure with every layer's set written in full, as the reference's "
+                    "reachSet{i} holds them, is value_all_sets_written / ms_per_step_all_sets_written",
+        "value_all_sets_written": head["all_sets_written"]["value"] if head["all_sets_written"] else None,
+        "ms_per_step_all_sets_written": head["all_sets_written"]["ms_per_step"] if head["all_sets_written"] else None,
         "spec_check": head["spec_check"], "host_to_host": head["host_to_host"],
         "all_sets_written": head["all_sets_written"], "layers": head["layers"], "per_config": per_config,
     }))

@@ -137,6 +137,13 @@ NNVHIP_API int nnvhip_debug_set_relu_call_number(nnvhip_ctx* ctx, int64_t call_n
 NNVHIP_API int nnvhip_trim_pool(nnvhip_ctx* ctx);
 /* Bytes currently handed out by / cached in the pool. */
 NNVHIP_API int nnvhip_pool_stats(nnvhip_ctx* ctx, int64_t* bytes_in_use, int64_t* bytes_cached);
+/* Diagnostic counters of a context since it was created (no counterpart in the reference), none of which this call
+ * changes: hipMalloc calls of the pool (a steady loop of reaches makes none after its first pass), waits for the
+ * stream because the pinned staging ring wrapped or grew, handles of released arrays that are still queued for
+ * destruction (this call does not drain the queue, unlike nnvhip_pool_stats), and live handles.  Any pointer may
+ * be NULL.  A benchmark reads them around a step that took unusually long. */
+NNVHIP_API int nnvhip_debug_counters(nnvhip_ctx* ctx, int64_t* device_mallocs, int64_t* staging_waits, int64_t* deferred_handles,
+                          int64_t* live_handles);
 /* Host-to-device traffic of the context since it was created (no counterpart in the reference, whose arrays
  * never leave the host): the number of layers whose weights were uploaded (nnvhip_fc_create /
  * nnvhip_conv2d_create calls that did not find their arrays resident), the bytes of those uploads, and all

@@ -932,7 +932,11 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int6
   double bytes = 0.0;
   for (int64_t i = 0; i < count; ++i) {
     max_m = std::max<int64_t>(max_m, sets[i].m);
-    bytes += 8.0 * (double)(Ho * Wo * cv->Cout) * (double)sets[i].m;  // algorithmic: the output columns
+    // algorithmic: the output columns -- whole ones, or, when only the rows inside each column's window are written,
+    // the filter stamp itself (at most FH * FW positions of every output channel)
+    const double rows_written = sets[i].win_only ? (double)std::min<int64_t>(Ho * Wo, cv->FH * cv->FW) * (double)cv->Cout
+                                                 : (double)(Ho * Wo * cv->Cout);
+    bytes += 8.0 * rows_written * (double)sets[i].m;
   }
   if (max_m == 0) return NNVHIP_OK;
   ConvGeom g;

@@ -147,6 +147,7 @@ int nnvhip_ctx::alloc(size_t bytes, BufRef* out) {
     bytes_cached -= (int64_t)cls;
   } else {
     hipError_t e = hipMalloc(&p, cls);
+    n_device_mallocs++;
     if (e != hipSuccess) {
       (void)hipGetLastError();
       drop_unreferenced_weights();  // layers that only the weight cache still holds
@@ -187,6 +188,7 @@ int nnvhip_ctx::trim() {
 int nnvhip_ctx::stage(size_t bytes, void** host) {
   bytes = (bytes + 255) & ~size_t(255);
   if (bytes > pinned_bytes) {
+    n_staging_waits++;
     NNV_HIP_TRY(hipStreamSynchronize(stream));
     // a table handed out from the old ring may still be named by a launch that is about to be issued:
     // the old ring stays allocated until the context goes (rings only ever grow, by doubling)
@@ -197,6 +199,7 @@ int nnvhip_ctx::stage(size_t bytes, void** host) {
     pinned_off = 0;
   }
   if (pinned_off + bytes > pinned_bytes) {
+    n_staging_waits++;
     NNV_HIP_TRY(hipStreamSynchronize(stream));  // earlier async copies out of the ring are done
     pinned_off = 0;
   }
@@ -589,6 +592,16 @@ int nnvhip_weight_cache_release(nnvhip_ctx* c, int64_t* dropped) {
 
 int nnvhip_debug_weak_weight_hash(int on) {
   g_weak_weight_hash = on != 0;
+  return NNVHIP_OK;
+}
+
+int nnvhip_debug_counters(nnvhip_ctx* c, int64_t* device_mallocs, int64_t* staging_waits, int64_t* deferred_handles,
+                          int64_t* live_handles) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  if (device_mallocs) *device_mallocs = c->n_device_mallocs;
+  if (staging_waits) *staging_waits = c->n_staging_waits;
+  if (deferred_handles) *deferred_handles = (int64_t)c->deferred.size();
+  if (live_handles) *live_handles = c->live_handles;
   return NNVHIP_OK;
 }
 

@@ -203,6 +203,9 @@ struct nnvhip_ctx {
   // short of a block; pool_stats, trim and destroy let them go first.
   std::vector<nnvhip_star*> deferred;
   void drain_deferred(size_t at_most = ~size_t(0));
+  // counters for diagnosing a slow step: hipMalloc calls of the pool, waits for the stream because the pinned
+  // staging ring wrapped or grew, mailbox waits that went through the slow path
+  int64_t n_device_mallocs = 0, n_staging_waits = 0;
   int64_t device_bytes = 0;  // memory of the device (the pool grows past a released array only below a share of it)
   // pinned staging ring for descriptor tables and small read-backs
   char* pinned = nullptr;

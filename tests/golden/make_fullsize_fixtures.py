@@ -1,4 +1,6 @@
-"""Writes tests/golden/cfg4_fullsize_relax_star_area.npz: what the CPU oracle (oracle/nnv_oracle.py) computes for
+"""Writes the full-size fixtures of configurations 4 and 5.
+
+tests/golden/cfg4_fullsize_relax_star_area.npz: what the CPU oracle (oracle/nnv_oracle.py) computes for
 configuration 4 (the 32x32x3 CNN) at its full size under relax-star-area, in a form small enough to commit.
 
 The oracle needs about 100 s and several GB for this reach, too much for a test that runs with every GPU check, so
@@ -10,7 +12,18 @@ its answers are recorded once:
   * the estimated ranges of the output set.
 tests/test_gpu_fullsize.py compares the device path with these.
 
-Run from the repository root:  python tests/golden/make_fullsize_fixtures.py
+tests/golden/cfg5_fullsize_relax_star_area.npz: configuration 5 (the 1024 sub-boxes of configuration 2's input box on
+configuration 2's network), every set reached on its own by the oracle as the reference loops over an array (about
+two minutes on eight cores):
+  * per set and ReLU layer the number of inactive neurons, the number of crossing neurons and a 64-bit hash
+    (blake2b of the little-endian int32 indices) of the crossing list in new-predicate order;
+  * per set the estimated ranges of the output set;
+  * per set and ReLU layer the classification margin min(|lb|, |ub|) over the layer's neurons, relative to the
+    largest bound of the layer, and the neuron and bound at which it is reached; and every pre-ReLU bound whose
+    magnitude is below 1e-6 of that scale (set, layer, neuron, lower / upper, value): the entries whose sign
+    decides a classification.
+
+Run from the repository root:  python tests/golden/make_fullsize_fixtures.py [4] [5]
 """
 import os
 import sys
@@ -30,6 +43,86 @@ METHOD = "relax-star-area"
 
 def flat(V):
     return V.reshape(-1, V.shape[-1], order="F") if V.ndim == 4 else V
+
+
+def crossing_hash(idx):
+    """64-bit hash of a crossing list in new-predicate order (what the test computes from the device's list)."""
+    import hashlib
+    return np.frombuffer(hashlib.blake2b(np.ascontiguousarray(idx, dtype="<i4").tobytes(), digest_size=8).digest(), dtype="<u8")[0]
+
+
+NEAR_ZERO = 1e-6
+
+
+def _cfg5_one(args):
+    """One sub-box through the oracle: per ReLU layer (inactive, crossing, hash, margin, its neuron, its bound, scale,
+    the near-zero bounds) and the output ranges."""
+    i, lb, ub = args
+    layers = _cfg5_one.layers
+    S = o.star_from_box(lb, ub)
+    per_layer = []
+    for L in layers:
+        if L["type"] == "relu":
+            elb, eub = o.estimate_ranges(S)
+            m1, m2 = o.relax_classify(elb, eub, METHOD)
+            scale = max(np.max(np.abs(elb)), np.max(np.abs(eub)))
+            both = np.concatenate([np.abs(elb), np.abs(eub)])
+            k = int(np.argmin(both))
+            vals = np.concatenate([elb, eub])
+            near = np.flatnonzero(both < NEAR_ZERO * scale)
+            per_layer.append((m1.size, m2.size, crossing_hash(m2), both[k] / scale, k % elb.size, k // elb.size, vals[k], scale,
+                              [(int(j % elb.size), int(j // elb.size), float(vals[j])) for j in near]))
+        S = o.nn_reach([L], S, METHOD, 1.0)
+    olb, oub = o.output_ranges(S)
+    return i, per_layer, np.asarray(olb).reshape(-1), np.asarray(oub).reshape(-1)
+
+
+def _cfg5_init(layers):
+    _cfg5_one.layers = layers
+    try:
+        from threadpoolctl import threadpool_limits
+        _cfg5_one.limit = threadpool_limits(2)
+    except Exception:
+        pass
+
+
+def main_cfg5(workers=4):
+    import multiprocessing as mp
+    cfg = make_config(5)
+    boxes = o.box_partition(cfg["lb"], cfg["ub"], cfg["partition"]["indexes"], cfg["partition"]["numbers"])
+    relu_layers = [li for li, L in enumerate(cfg["layers"]) if L["type"] == "relu"]
+    n_sets, n_relu = len(boxes), len(relu_layers)
+    inactive = np.zeros((n_sets, n_relu), dtype=np.int32)
+    crossing = np.zeros((n_sets, n_relu), dtype=np.int32)
+    hashes = np.zeros((n_sets, n_relu), dtype=np.uint64)
+    margin = np.zeros((n_sets, n_relu))
+    margin_neuron = np.zeros((n_sets, n_relu), dtype=np.int32)
+    margin_upper = np.zeros((n_sets, n_relu), dtype=np.int8)
+    margin_value = np.zeros((n_sets, n_relu))
+    scale = np.zeros((n_sets, n_relu))
+    near = []
+    out_lb = np.zeros((n_sets, cfg["layers"][-1]["W"].shape[0]))
+    out_ub = np.zeros_like(out_lb)
+    t0 = time.time()
+    with mp.Pool(workers, initializer=_cfg5_init, initargs=(cfg["layers"],)) as pool:
+        for done, (i, per_layer, olb, oub) in enumerate(pool.imap_unordered(_cfg5_one, [(i, b[0], b[1]) for i, b in enumerate(boxes)],
+                                                                             chunksize=4)):
+            for r, (ni, m, h, mg, neuron, upper, val, sc, nz) in enumerate(per_layer):
+                inactive[i, r], crossing[i, r], hashes[i, r] = ni, m, h
+                margin[i, r], margin_neuron[i, r], margin_upper[i, r], margin_value[i, r], scale[i, r] = mg, neuron, upper, val, sc
+                near.extend((i, r, nn_, up, v) for (nn_, up, v) in nz)
+            out_lb[i], out_ub[i] = olb, oub
+            if (done + 1) % 64 == 0:
+                print("  %d / %d sets, %.0f s" % (done + 1, n_sets, time.time() - t0), flush=True)
+    near.sort()
+    data = {"relu_layers": np.array(relu_layers, dtype=np.int64), "inactive": inactive, "crossing": crossing, "crossing_hash": hashes,
+            "margin": margin, "margin_neuron": margin_neuron, "margin_upper": margin_upper, "margin_value": margin_value,
+            "scale": scale, "out_lb": out_lb, "out_ub": out_ub,
+            "near_zero_where": np.array([(a, b, c, d) for (a, b, c, d, _) in near], dtype=np.int32).reshape(-1, 4),
+            "near_zero_value": np.array([v for (_, _, _, _, v) in near], dtype=np.float64)}
+    path = os.path.join(ROOT, "tests", "golden", "cfg5_fullsize_relax_star_area.npz")
+    np.savez_compressed(path, **data)
+    print("wrote", path, os.path.getsize(path), "bytes; smallest margin per ReLU layer:", margin.min(axis=0), "near-zero bounds:", len(near))
 
 
 def main():
@@ -69,4 +162,8 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    which = sys.argv[1:] or ["4", "5"]
+    if "4" in which:
+        main()
+    if "5" in which:
+        main_cfg5()

@@ -49,6 +49,33 @@ def assert_close(got, exp, what, rtol=RTOL):
     assert err <= rtol * scale, "%s: max abs err %.3e (scale %.3e, rel %.3e)" % (what, err, scale, err / scale)
 
 
+def assert_close_elementwise(got, exp, what, rtol=RTOL, atol_of_scale=1e-12):
+    """Entry by entry: |got - exp| <= rtol * |exp| + atol_of_scale * max|exp|, and the same sign wherever the expected
+    entry is not zero.  The absolute term covers sums that cancel (a bound near zero is a difference of large
+    terms; its error is that of the terms), the sign is what a classification depends on."""
+    got = np.asarray(got, dtype=np.float64)
+    exp = np.asarray(exp, dtype=np.float64)
+    assert got.shape == exp.shape, "%s: shape %s vs %s" % (what, got.shape, exp.shape)
+    if exp.size == 0:
+        return
+    scale = max(np.max(np.abs(exp)), 1e-300)
+    err = np.abs(got - exp)
+    bad = err > rtol * np.abs(exp) + atol_of_scale * scale
+    assert not bad.any(), "%s: %d entries off, worst |err| %.3e at expected value %.3e (scale %.3e)" % (
+        what, int(bad.sum()), float(err[bad].max()), float(exp[bad][np.argmax(err[bad])]), scale)
+    flipped = (exp != 0) & (np.sign(got) != np.sign(exp))
+    assert not flipped.any(), "%s: %d entries changed sign, e.g. expected %.3e got %.3e" % (
+        what, int(flipped.sum()), float(exp[flipped][0]), float(got[flipped][0]))
+
+
+def classification_margin(lb, ub):
+    """min(|lb|, |ub|) over the neurons of a layer, relative to the largest bound: how far the closest bound is
+    from changing a neuron's class."""
+    lb, ub = np.asarray(lb), np.asarray(ub)
+    scale = max(np.max(np.abs(lb)), np.max(np.abs(ub)), 1e-300)
+    return float(min(np.min(np.abs(lb)), np.min(np.abs(ub))) / scale)
+
+
 def input_sets(cfg):
     """Build the device input set(s) and the oracle's, exactly as Star(lb,ub)/ImageStar(lb,ub)."""
     if "partition" in cfg:
@@ -129,6 +156,12 @@ def run_cfg(cfg, method="relax-star-area", check_constraints=True, margins=None,
                 ni, idx, clb, cub = ds.relu_info()
                 if margins is not None:
                     margins.append(float(np.min(np.minimum(np.abs(lb), np.abs(ub)) / max(np.max(np.abs(ub - lb)), 1e-300))))
+                # the device's own bounds of the ReLU's input, entry by entry: a bound near zero must keep its sign
+                dprev = (net.reachSet[li - 1] if li > 0 else dev_in)
+                dprev = dprev[si] if batched else dprev
+                dlb, dub = (np.asarray(x).reshape(-1, order="F") for x in dprev.estimateRanges())
+                assert_close_elementwise(dlb, lb, tag + ": lb of the ReLU's input")
+                assert_close_elementwise(dub, ub, tag + ": ub of the ReLU's input")
                 assert ni == m1.size, "%s: inactive count %d vs %d" % (tag, ni, m1.size)
                 if tie_tolerant and not np.array_equal(idx, m2):
                     # Sort keys that are equal in exact arithmetic (e.g. ub-lb of a conv layer under a

@@ -7,7 +7,7 @@ import pytest
 
 from nnv_amd.configs import make_config
 from oracle import nnv_oracle as o
-from tests.gpu_util import assert_close, flat_V, input_sets
+from tests.gpu_util import assert_close, assert_close_elementwise, classification_margin, flat_V, input_sets
 
 pytestmark = pytest.mark.gpu
 
@@ -180,3 +180,54 @@ def test_config4_full_against_the_recorded_oracle(nnv):
     olb, oub = (x.reshape(-1, order="F") for x in out.estimateRanges())
     assert_close(olb, gold["out_lb"], "cfg4 output lb", 1e-9)
     assert_close(oub, gold["out_ub"], "cfg4 output ub", 1e-9)
+
+
+def test_config5_full_against_the_recorded_oracle(nnv, capsys):
+    """All 1024 sets of configuration 5 against what the CPU oracle computes for each sub-box on its own (recorded by
+    tests/golden/make_fullsize_fixtures.py): per set and ReLU layer the inactive count, the number of crossing
+    neurons and the crossing list in new-predicate order (by a 64-bit hash) exactly; the output ranges entry by entry;
+    every pre-ReLU bound close to zero (the ones whose sign decides a class) with the oracle's sign; and the
+    classification margins of the device's own bounds next to the oracle's."""
+    import hashlib
+    import os
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "cfg5_fullsize_relax_star_area.npz"))
+    cfg = make_config(5)
+    stars, _ = input_sets(cfg)
+    net = nnv.NN.from_config(cfg["layers"], cfg["name"])
+    outs = net.reach(stars, {"reachMethod": "relax-star-area", "relaxFactor": 1})
+    n_sets = len(outs)
+    assert n_sets == gold["inactive"].shape[0] == 1024
+    relu_layers = [int(v) for v in gold["relu_layers"]]
+    assert relu_layers == [li for li, L in enumerate(cfg["layers"]) if L["type"] == "relu"]
+    near_where, near_value = gold["near_zero_where"], gold["near_zero_value"]
+    dev_margin = np.zeros((n_sets, len(relu_layers)))
+    for r, li in enumerate(relu_layers):
+        pre_lb, pre_ub = nnv.Star.estimateRanges_array(net.reachSet[li - 1])    # the ReLU's input: ranges cached by the step
+        post = net.reachSet[li]
+        for i in range(n_sets):
+            ni, idx, clb, cub = post[i].relu_info()
+            tag = "set %d ReLU layer %d" % (i, li + 1)
+            assert ni == int(gold["inactive"][i, r]), tag + ": inactive count"
+            assert idx.size == int(gold["crossing"][i, r]), tag + ": number of crossing neurons"
+            h = np.frombuffer(hashlib.blake2b(np.ascontiguousarray(idx, dtype="<i4").tobytes(), digest_size=8).digest(), dtype="<u8")[0]
+            assert h == gold["crossing_hash"][i, r], tag + ": crossing list / new-predicate order"
+            assert np.array_equal(clb, pre_lb[idx, i]) and np.array_equal(cub, pre_ub[idx, i]), tag
+            dev_margin[i, r] = classification_margin(pre_lb[:, i], pre_ub[:, i])
+            # the bound the oracle found closest to zero: same sign, same value
+            k, upper = int(gold["margin_neuron"][i, r]), int(gold["margin_upper"][i, r])
+            got = (pre_ub if upper else pre_lb)[k, i]
+            exp = gold["margin_value"][i, r]
+            assert abs(got - exp) <= 1e-12 * gold["scale"][i, r] and np.sign(got) == np.sign(exp), tag + ": closest bound"
+        sel = near_where[:, 1] == r
+        for (i, _, k, upper), exp in zip(near_where[sel], near_value[sel]):
+            got = (pre_ub if upper else pre_lb)[k, i]
+            assert np.sign(got) == np.sign(exp) and abs(got - exp) <= 1e-12 * gold["scale"][i, r], \
+                "set %d ReLU layer %d neuron %d: bound near zero, expected %.3e got %.3e" % (i, li + 1, k, exp, got)
+    lb, ub = nnv.Star.estimateRanges_array(outs)
+    assert_close_elementwise(lb.T, gold["out_lb"], "output lb of all 1024 sets")
+    assert_close_elementwise(ub.T, gold["out_ub"], "output ub of all 1024 sets")
+    with capsys.disabled():
+        print("\ncfg5 classification margins per ReLU layer (min over 1024 sets): device %s, oracle %s; %d bounds below 1e-6 of scale"
+              % (np.array2string(dev_margin.min(axis=0), precision=3), np.array2string(gold["margin"].min(axis=0), precision=3),
+                 near_value.size))
+    assert np.all(dev_margin.min(axis=0) > 0)

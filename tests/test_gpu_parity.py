@@ -1,8 +1,10 @@
 """GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs."""
+import contextlib
+
 import numpy as np
 import pytest
 
-from tests.gpu_util import RTOL, assert_close, compare_sets, flat_V, input_sets, run_both, run_cfg
+from tests.gpu_util import RTOL, assert_close, assert_close_elementwise, compare_sets, flat_V, input_sets, run_both, run_cfg
 
 pytestmark = pytest.mark.gpu
 
@@ -215,20 +217,28 @@ def test_config1_full(nnv, method):
     assert min(margins) > 1e-12
 
 
-def test_config2_full(nnv, oracle):
-    dev, ora, net = run_both(2, "relax-star-area")
+def test_config2_full(nnv, oracle, capsys):
+    margins = []
+    dev, ora, net = run_both(2, "relax-star-area", margins=margins)
     dl, du = dev.estimateRanges()
     ol, ou = oracle.output_ranges(ora)
-    assert_close(dl, ol, "output lb")
-    assert_close(du, ou, "output ub")
+    assert_close_elementwise(dl, ol, "output lb")
+    assert_close_elementwise(du, ou, "output ub")
+    with capsys.disabled() if capsys is not None else contextlib.nullcontext():
+        print("\ncfg2 classification margin per ReLU layer (min |bound| / max width):", ["%.2e" % m for m in margins])
+    assert min(margins) > 1e-12
 
 
-def test_config3_full(nnv, oracle):
-    dev, ora, net = run_both(3, "relax-star-area")
+def test_config3_full(nnv, oracle, capsys):
+    margins = []
+    dev, ora, net = run_both(3, "relax-star-area", margins=margins)
     dl, du = dev.estimateRanges()
     ol, ou = oracle.output_ranges(ora)
-    assert_close(dl.reshape(-1), ol, "output lb")
-    assert_close(du.reshape(-1), ou, "output ub")
+    assert_close_elementwise(dl.reshape(-1), ol, "output lb")
+    assert_close_elementwise(du.reshape(-1), ou, "output ub")
+    with capsys.disabled() if capsys is not None else contextlib.nullcontext():
+        print("\ncfg3 classification margin per ReLU layer (min |bound| / max width):", ["%.2e" % m for m in margins])
+    assert min(margins) > 1e-12
 
 
 def test_config4_shrunk(nnv):

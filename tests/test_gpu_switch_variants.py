@@ -106,11 +106,11 @@ def test_config1(route, nnv):
 
 
 def test_config2(route, nnv, oracle):
-    parity.test_config2_full(nnv, oracle)
+    parity.test_config2_full(nnv, oracle, None)
 
 
 def test_config3(route, nnv, oracle):
-    parity.test_config3_full(nnv, oracle)
+    parity.test_config3_full(nnv, oracle, None)
 
 
 def test_config4_shrunk(route, nnv):
