@@ -1747,7 +1747,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
           };
           std::vector<RowShape> shapes;
           std::vector<int> shape_of((size_t)count, -1);
-          bool shared = !c->eager_cols;
+          bool shared = true;
           for (int64_t i = 0; i < count && shared; ++i) {
             if (filled[i]) continue;
             const ColSource& cs = in[i]->cs;

@@ -446,6 +446,10 @@ struct GatherArgs {
   int32_t cols_per_chunk;
   int32_t with_sums;  // every chunk of the grid leaves range sums in the set's `part` (if it has one)
   int64_t Mp;         // rows of W (a multiple of 16): the bias has that many entries
+  // XCD-aware block order (xcd_row_blocks > 0; the grid is then one-dimensional): workgroups are dealt to the eight
+  // XCDs round-robin, and every block of a 128-row slice of W goes to the same XCD (row block mod 8), sets and
+  // column chunks in turn, so that the slice stays in that XCD's L2 while all sets gather from it.
+  int32_t xcd_row_blocks, xcd_chunks, xcd_count;
 };
 
 // CENTRE: the variant that also forms the centre's product (GatherSet::cin); kept apart because its extra
@@ -453,8 +457,18 @@ struct GatherArgs {
 template <bool CENTRE>
 __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const GatherSet* __restrict__ table, GatherSet one,
                                                                          GatherArgs a) {
-  const GatherSet d = table ? table[blockIdx.z] : one;
-  const int chunk = blockIdx.y;
+  int row_block = blockIdx.x, chunk = blockIdx.y, set = blockIdx.z, nchunks = gridDim.y;
+  if (a.xcd_row_blocks > 0) {
+    const unsigned xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const unsigned per_rb = (unsigned)a.xcd_chunks * (unsigned)a.xcd_count;
+    row_block = (int)((slot / per_rb) * 8u + xcd);
+    if (row_block >= a.xcd_row_blocks) return;
+    const unsigned rem = slot % per_rb;
+    set = (int)(rem / (unsigned)a.xcd_chunks);
+    chunk = (int)(rem % (unsigned)a.xcd_chunks);
+    nchunks = a.xcd_chunks;
+  }
+  const GatherSet d = table ? table[set] : one;
   const int j0 = chunk * a.cols_per_chunk;
   double* part = a.with_sums ? d.part : nullptr;
   if (j0 >= d.m && part == nullptr && d.nfill == 0 && d.red == nullptr) return;
@@ -463,7 +477,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   const int j1 = no_cols ? j0 : min(d.m, j0 + a.cols_per_chunk);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t r0 = (int64_t)blockIdx.x * kRowsPerWave + 2 * lane;
+  const int64_t r0 = (int64_t)row_block * kRowsPerWave + 2 * lane;
   const bool active = r0 < a.ldout;
   // The centre column came out of a split-K product: the first chunk's blocks sum its partial vectors in
   // split order and add the bias, as the reduction kernel would have.
@@ -484,7 +498,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
   // of those columns is written here instead of by a GEMM launch (they add nothing to the range sums).
   if (d.nfill > 0 && active) {
     const int nf = d.lazy ? 1 : d.nfill;  // unwritten columns: only the centre is stored
-    const int fpc = (nf + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int fpc = (nf + nchunks - 1) / nchunks;
     const int f1 = min(nf, (chunk + 1) * fpc);
     for (int j = chunk * fpc + wave; j < f1; j += kRangeWaves) {
       double2 o = make_double2(0.0, 0.0);
@@ -732,12 +746,22 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
       NNV_LAUNCH(ctx, ctx->kernel_timing, gather_skinny_kernel<8>, grid, dim3(256), 0, table, sets[0], a);
     else
       NNV_LAUNCH(ctx, ctx->kernel_timing, gather_skinny_kernel<16>, grid, dim3(256), 0, table, sets[0], a);
-  } else if (centre)
-    NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel<true>, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
-               dim3(64 * kRangeWaves), 0, table, sets[0], a);
-  else
-    NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel<false>, dim3((unsigned)row_blocks, (unsigned)chunks, (unsigned)count),
-               dim3(64 * kRangeWaves), 0, table, sets[0], a);
+  } else {
+    // large launches over arrays: blocks ordered so that a row slice of W is served from one XCD's L2
+    dim3 grid((unsigned)row_blocks, (unsigned)chunks, (unsigned)count);
+    const int64_t xcd_blocks = 8 * ceil_div(row_blocks, 8) * chunks * count;
+    if (count >= 8 && row_blocks >= 8 && row_blocks * chunks * count >= 4096 && xcd_blocks < (int64_t(1) << 31) &&
+        xcd_blocks * 4 <= row_blocks * chunks * count * 5) {
+      a.xcd_row_blocks = (int32_t)row_blocks;
+      a.xcd_chunks = (int32_t)chunks;
+      a.xcd_count = (int32_t)count;
+      grid = dim3((unsigned)xcd_blocks, 1, 1);
+    }
+    if (centre)
+      NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel<true>, grid, dim3(64 * kRangeWaves), 0, table, sets[0], a);
+    else
+      NNV_LAUNCH(ctx, ctx->kernel_timing, gather_columns_kernel<false>, grid, dim3(64 * kRangeWaves), 0, table, sets[0], a);
+  }
   NNV_TRY(ctx->kernel_timer_end(ctx->kernel_timing, 5, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;

@@ -599,7 +599,11 @@ int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets,
       s->rows_pending = false;
       s->cls_buf.reset();
       s->cls = nullptr;
-      s->cs = ColSource();  // the reset rows no longer match the weight columns
+      // The rows that were kept still hold the gathered weight columns, which is all a later packing of kept rows
+      // asks of this description; nothing of it is pending any more (the apply pass read whole columns).
+      s->cs.pending = false;
+      s->cs.zero_to = 0;
+      s->cs.win_from = s->cs.win_to = 0;
       if (need_tail) s->vcols = -1;
     }
     pend.swap(rest);
@@ -919,6 +923,12 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     if (!lazy_rows) {
       o->Vbuf = arena;
       o->V = d.Vout;
+      // where the input's columns were gathered from: still true of the rows this step keeps (a later packing of
+      // kept rows reads the cache-resident weights instead of this matrix); everything is in memory
+      o->cs = in[i]->cs;
+      o->cs.pending = false;
+      o->cs.zero_to = 0;
+      o->cs.win_from = o->cs.win_to = 0;
     }
     o->pbuf = pred_buf;
     o->plb = d.plb_out;
