@@ -226,14 +226,14 @@ def measure(k, args, ctx, exact_steps, extras):
         return acc / reps
 
     # a small FC / ReLU network is reached by ONE launch (nnvhip_reach_layers): time that kernel on the step's own path
-    for grp in range(10):
+    for grp in range(11):
         ctx.kernel_time(grp)
     ctx.set_timing(2)
     for _ in range(reps):
         step()
     ctx.set_timing(0)
     chain_ms, chain_launches, chain_bytes = ctx.kernel_time(8)
-    for grp in range(10):
+    for grp in range(11):
         ctx.kernel_time(grp)
 
     per_layer = timed_pass(1)          # NN.reachTime-style device time per layer (layer-by-layer calls)
@@ -247,6 +247,7 @@ def measure(k, args, ctx, exact_steps, extras):
     cls_ms, cls_launches, cls_bytes = ctx.kernel_time(6)
     fin_ms, fin_launches, fin_bytes = ctx.kernel_time(7)
     seg_ms, seg_launches, seg_work = ctx.kernel_time(9)
+    dlt_ms, dlt_launches, dlt_bytes = ctx.kernel_time(10)
 
     # algorithmic (unpadded, dense) flop of the launches the kernel timers cover
     gemm_flop = conv_flop = 0.0
@@ -343,6 +344,17 @@ def measure(k, args, ctx, exact_steps, extras):
         groups.append((gat_ms, g))
     if fin_launches:
         groups.append((fin_ms, hbm_roofline("ranges_final_kernel", fin_ms, fin_launches, fin_bytes)))
+    if dlt_launches:
+        # outputs that start from a product shared by the sets of a group and add only the rows in which a set differs
+        # from the group's list: a block reads its piece of the shared product (from cache), adds a few rank-one
+        # terms and writes itself out - bound by the bytes of output it writes
+        g = hbm_roofline("delta_tiles_kernel", dlt_ms, dlt_launches, dlt_bytes)
+        g["what"] = ("FC layer over an array of sets of one shape: the product over the rows most sets keep is formed once per "
+                     "shape, every set's tiles start from it and contract over the rows in which the set differs; bytes = the "
+                     "output matrices written")
+        g["dense_equivalent_flop_per_step"] = gemm_flop
+        g["dense_equivalent_achieved_TFLOPs"] = round(gemm_flop * reps / (dlt_ms * 1e-3) / 1e12, 1)
+        groups.append((dlt_ms, g))
     if cls_launches:
         # classification, sort of the crossing list and the new predicate bounds: one block per set of up
         # to 8192 neurons - with a single input set a dependent chain on one CU, bound by latency, which

@@ -320,7 +320,10 @@ NNVHIP_API int nnvhip_set_small_chain(nnvhip_ctx* ctx, int enabled);
  * same sets, and exist so that a test suite can drive every route in one process): "dense_affine"
  * (NNVHIP_DENSE_AFFINE), "eager_rows", "eager_tail", "eager_cols" (NNVHIP_EAGER_*), "poison_pending"
  * (NNVHIP_POISON_PENDING: whatever a layer leaves unwritten until first read is filled with NaNs),
- * "no_small_chain", "no_conv_mask", "no_conv_boxes" (NNVHIP_NO_*).  A switch applies to the layer calls made
+ * "no_small_chain", "no_conv_mask", "no_conv_boxes" (NNVHIP_NO_*), "no_row_deltas" (NNVHIP_NO_ROW_DELTAS: an FC
+ * layer over an array of sets of one shape contracts every set over its whole kept-row list instead of forming
+ * the product over the rows most sets keep once and contracting each set over its differences from that list).
+ * A switch applies to the layer calls made
  * after it; sets produced before keep what they recorded.  Unknown name: NNVHIP_ERR_ARG. */
 NNVHIP_API int nnvhip_set_switch(nnvhip_ctx* ctx, const char* name, int enabled);
 enum { NNVHIP_LAYER_FC = 0, NNVHIP_LAYER_CONV2D = 1, NNVHIP_LAYER_RELU = 2 };

@@ -351,6 +351,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->small_chain = getenv("NNVHIP_NO_SMALL_CHAIN") == nullptr;
   c->no_conv_mask = getenv("NNVHIP_NO_CONV_MASK") != nullptr;
   c->no_conv_boxes = getenv("NNVHIP_NO_CONV_BOXES") != nullptr;
+  c->no_row_deltas = getenv("NNVHIP_NO_ROW_DELTAS") != nullptr;
   if (const char* e = getenv("NNVHIP_WEIGHT_CACHE_MB")) c->weight_cache_budget = (int64_t)atoll(e) << 20;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
@@ -438,6 +439,7 @@ int nnvhip_set_switch(nnvhip_ctx* c, const char* name, int enabled) {
       {"eager_tail", &c->eager_tail, false},       {"eager_cols", &c->eager_cols, false},
       {"poison_pending", &c->poison_pending, false}, {"no_small_chain", &c->small_chain, true},
       {"no_conv_mask", &c->no_conv_mask, false},   {"no_conv_boxes", &c->no_conv_boxes, false},
+      {"no_row_deltas", &c->no_row_deltas, false},
   };
   for (const auto& t : table)
     if (strcmp(t.name, name) == 0) {
@@ -1769,6 +1771,14 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             }
           }
           shared = shared && !shapes.empty();
+          // Sets of one shape differ in their products only through their kept-row lists (and their centres).  Where
+          // the lists of a group are nearly the same - the sub-boxes of one box, whose first-layer bounds differ by
+          // little - the group's product over the rows most of its sets keep is formed once (by the tile kernel), and a
+          // set's output is that product plus the few rows in which the set differs, written by one streaming pass
+          // (delta_try / delta_done below).
+          bool delta_try = shared && count >= 32 && !c->no_row_deltas;
+          for (size_t k = 1; k < shapes.size() && delta_try; ++k) delta_try = shapes[k].rows == shapes[0].rows;
+          delta_try = delta_try && !shapes.empty() && shapes[0].rows == fc->Kp && shapes[0].rows < (int64_t(1) << 20);
           if (shared) {
             int64_t doubles = 0;
             for (RowShape& r : shapes) {
@@ -1785,8 +1795,158 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
             sr.count = (int32_t)shapes.size();
             if (st == NNVHIP_OK) st = launch_scaled_rows(c, sr);
           }
+          bool delta_done = false;
+          if (delta_try && st == NNVHIP_OK) {
+            constexpr int kDeltaCap = 64;
+            const int groups = (int)shapes.size();
+            const int64_t rowsK = shapes[0].rows, rows_pad = round_up(rowsK, 16);
+            std::vector<int64_t> act;  // the sets that take part (not filled)
+            std::vector<DeltaSet> dsets;
+            std::vector<CentreSet> csets;
+            std::vector<int32_t> gsize((size_t)groups, 0);
+            for (int64_t i = 0; i < count; ++i)
+              if (!filled[i]) {
+                act.push_back(i);
+                dsets.push_back(DeltaSet{rws[i].kmap, (int32_t)kps[i], (int32_t)shape_of[i]});
+                csets.push_back(CentreSet{rws[i].kmap, in[i]->V, (int32_t)kps[i]});
+                gsize[(size_t)shape_of[i]]++;
+              }
+            const int64_t nact = (int64_t)act.size();
+            BufRef dtab, ctab, gtab, votes, common, lens, delta;
+            if (nact == 0) st = NNVHIP_OK;
+            if (nact > 0) {
+              st = c->upload_table(dsets.data(), sizeof(DeltaSet) * dsets.size(), &dtab);
+              if (st == NNVHIP_OK) st = c->upload_table(gsize.data(), sizeof(int32_t) * gsize.size(), &gtab);
+              if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * groups * rowsK, &votes);
+              if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * groups * rows_pad, &common);
+              if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * (groups + nact), &lens);  // ncommon, then dlen
+              if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * nact * kDeltaCap, &delta);
+              if (st == NNVHIP_OK)
+                st = launch_delta_lists(c, nact, dtab->as<DeltaSet>(), groups, gtab->as<int32_t>(), rowsK, rows_pad, kDeltaCap,
+                                        votes->as<int32_t>(), common->as<int32_t>(), lens->as<int32_t>(), delta->as<int32_t>(),
+                                        lens->as<int32_t>() + groups);
+              std::vector<int32_t> hl((size_t)(groups + nact));
+              if (st == NNVHIP_OK) {
+                void* hp = nullptr;
+                st = c->stage(sizeof(int32_t) * hl.size(), &hp);
+                if (st == NNVHIP_OK) {
+                  if (hipMemcpyAsync(hp, lens->ptr, sizeof(int32_t) * hl.size(), hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+                      hipStreamSynchronize(c->stream) != hipSuccess) {
+                    set_error("HIP error reading the row-difference lists back");
+                    st = NNVHIP_ERR_HIP;
+                  } else {
+                    memcpy(hl.data(), hp, sizeof(int32_t) * hl.size());
+                  }
+                }
+              }
+              bool fits = st == NNVHIP_OK;
+              int64_t delta_rows = 0;
+              for (int64_t a = 0; a < nact && fits; ++a) {
+                fits = hl[(size_t)(groups + a)] >= 0;
+                delta_rows += std::max<int32_t>(hl[(size_t)(groups + a)], 0);
+              }
+              // worth it when a set's differences are a small part of its list
+              int64_t kept_rows = 0;
+              for (int64_t a = 0; a < nact; ++a) kept_rows += kps[act[(size_t)a]];
+              fits = fits && 4 * delta_rows <= kept_rows;
+              if (fits) {
+                const int64_t ldo = outs[0]->ld, Mp = fc->Mp;
+                // the groups' shared products: the same tiles, over the majority lists, into a buffer of their own
+                int64_t base_cols = 0;
+                std::vector<int64_t> base_off((size_t)groups);
+                for (int g = 0; g < groups; ++g) {
+                  base_off[(size_t)g] = base_cols;
+                  base_cols += shapes[(size_t)g].ldws;
+                }
+                BufRef basebuf, cm, cprod;
+                st = c->alloc(sizeof(double) * Mp * base_cols, &basebuf);
+                std::vector<SegTile> bt_tiles;
+                double base_flop = 0.0;
+                for (int g = 0; g < groups && st == NNVHIP_OK; ++g) {
+                  const RowShape& r = shapes[(size_t)g];
+                  if (gsize[(size_t)g] == 0) continue;
+                  for (int64_t j = 0; j < r.dense; j += 128) {
+                    SegTile sg{};
+                    sg.kmap = common->as<int32_t>() + (int64_t)g * rows_pad;
+                    sg.Bt = shared_rows->as<double>() + r.off;
+                    sg.ldbt = r.ldws;
+                    sg.b_col0 = j;
+                    sg.col_local0 = j;
+                    sg.col_base = base_off[(size_t)g] + j;
+                    sg.gather_b = 1;
+                    sg.zero_row = (int32_t)r.rows;
+                    sg.kp = hl[(size_t)g];
+                    sg.valid = (int32_t)std::min<int64_t>(128, r.dense - j);
+                    bt_tiles.push_back(sg);
+                    base_flop += 2.0 * (double)Mp * (double)sg.kp * (double)sg.valid;
+                  }
+                }
+                if (st == NNVHIP_OK && !bt_tiles.empty()) {
+                  BufRef dt;
+                  st = c->upload_table(bt_tiles.data(), sizeof(SegTile) * bt_tiles.size(), &dt);
+                  if (st == NNVHIP_OK)
+                    st = launch_gemm_seg(c, Wd, Mp, basebuf->as<double>(), Mp, Mp, nullptr, 128, dt->as<SegTile>(), (int64_t)bt_tiles.size(),
+                                         base_flop, true);
+                }
+                // the centres, which are the sets' own: W * (centre masked to the kept rows), all sets in one product
+                if (st == NNVHIP_OK) st = c->upload_table(csets.data(), sizeof(CentreSet) * csets.size(), &ctab);
+                if (st == NNVHIP_OK) st = c->alloc(sizeof(double) * fc->Kp * nact, &cm);
+                if (st == NNVHIP_OK) st = c->alloc(sizeof(double) * Mp * nact, &cprod);
+                if (st == NNVHIP_OK) st = launch_masked_centres(c, nact, ctab->as<CentreSet>(), cm->as<double>(), fc->Kp);
+                if (st == NNVHIP_OK)
+                  st = launch_gemm(c, Wd, Mp, cm->as<double>(), fc->Kp, cprod->as<double>(), Mp, Mp, nact, fc->Kp, nullptr);
+                // the sets' tiles, by column tile and group so that tiles that read the same piece of a shared product
+                // run next to one another
+                for (int64_t i = 0; i < count; ++i) {
+                  tiles_of[i] = filled[i] ? 0 : delta_tile_chunks(dense[i]);
+                  chunk_off[i + 1] = chunk_off[i] + tiles_of[i] + (gs[i].m > 0 ? gch_part : 0);
+                }
+                if (st == NNVHIP_OK && chunk_off[count] > 0) st = c->alloc(sizeof(double) * 4 * ldo * chunk_off[count], &sums);
+                std::vector<int64_t> col_off((size_t)count, 0);
+                {
+                  int64_t off = 0;
+                  for (int64_t i = 0; i < count; ++i) {
+                    col_off[(size_t)i] = off;
+                    off += in[i]->n + 1;
+                  }
+                }
+                // the sets by group, so that neighbours in the table read the same shared product
+                std::vector<DeltaOut> douts;
+                std::vector<int32_t> dgroup;
+                double dbytes = 0.0;
+                int64_t max_cols = 0;
+                for (int g = 0; g < groups && st == NNVHIP_OK; ++g)
+                  for (int64_t a = 0; a < nact; ++a) {
+                    const int64_t i = act[(size_t)a];
+                    if (shape_of[i] != g) continue;
+                    const RowShape& r = shapes[(size_t)g];
+                    DeltaOut d{};
+                    d.delta = delta->as<int32_t>() + a * kDeltaCap;
+                    d.base = basebuf->as<double>() + base_off[(size_t)g] * Mp;
+                    d.S = shared_rows->as<double>() + r.off;
+                    d.lds = r.ldws;
+                    d.cprod = cprod->as<double>() + a * Mp;
+                    d.out = outs[0]->V + col_off[(size_t)i] * ldo;
+                    d.plb = outs[i]->plb;
+                    d.pub = outs[i]->pub;
+                    d.rpart = sums->as<double>() + 4 * ldo * chunk_off[i];
+                    d.dlen = hl[(size_t)(groups + a)];
+                    d.ncols = (int32_t)dense[i];
+                    douts.push_back(d);
+                    dgroup.push_back((int32_t)g);
+                    dbytes += 8.0 * (double)Mp * (double)dense[i];
+                    max_cols = std::max<int64_t>(max_cols, dense[i]);
+                  }
+                if (st == NNVHIP_OK && !douts.empty())
+                  st = launch_delta_tiles(c, Wd, Mp, Mp, bias, ldo, (int64_t)douts.size(), douts.data(), dgroup.data(), max_cols, dbytes);
+                delta_done = true;
+                bias_in_kernel = true;
+              }
+            }
+          }
           auto nfull_of = [&](int64_t i) { return shared ? shapes[(size_t)shape_of[i]].nfull : 0; };
           int64_t total = 0;
+          if (!delta_done) {
           for (int64_t i = 0; i < count; ++i)
             if (!filled[i]) {
               if (shared) {  // the columns past the last whole tile only, in a tile of their own width
@@ -1864,6 +2024,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                                    flop[w], w == 3);
           }
           bias_in_kernel = true;
+          }  // !delta_done
         } else {
         // several row tiles would each gather the kept rows of B: pack them once per set instead
         BufRef packed;

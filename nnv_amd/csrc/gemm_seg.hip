@@ -445,6 +445,232 @@ __global__ __launch_bounds__(256) void scaled_rows_kernel(ScaledRows a) {
     o[j] = v;
   }
 }
+
+// ---- row lists of an array of sets against their group's majority list --------------------------------------
+__global__ __launch_bounds__(256) void vote_rows_kernel(const DeltaSet* __restrict__ sets, int32_t* __restrict__ votes, int rows) {
+  const DeltaSet d = sets[blockIdx.x];
+  for (int t = threadIdx.x; t < d.kp; t += 256) {
+    const int r = d.kept[t];
+    if (r >= 0 && r < rows) atomicAdd(&votes[(int64_t)d.group * rows + r], 1);
+  }
+}
+
+// one block per group: the rows more than half of the group's sets keep, ascending, -1 padded to a multiple of 16
+__global__ __launch_bounds__(1024) void common_rows_kernel(const int32_t* __restrict__ votes, const int32_t* __restrict__ group_size,
+                                                           int rows, int rows_pad, int32_t* __restrict__ common,
+                                                           int32_t* __restrict__ ncommon) {
+  const int g = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = group_size[g];
+  __shared__ int wsum[16];
+  __shared__ int base;
+  if (tid == 0) base = 0;
+  __syncthreads();
+  int32_t* out = common + (int64_t)g * rows_pad;
+  for (int r0 = 0; r0 < rows; r0 += 1024) {
+    const int r = r0 + tid;
+    const bool in = r < rows && 2 * votes[(int64_t)g * rows + r] > half;
+    const unsigned long long bal = __ballot(in);
+    if (lane == 0) wsum[wave] = __popcll(bal);
+    __syncthreads();
+    int off = base;
+    for (int w = 0; w < wave; ++w) off += wsum[w];
+    if (in) out[off + __popcll(bal & ((1ull << lane) - 1))] = r;
+    __syncthreads();
+    if (tid == 0) {
+      int t = 0;
+      for (int w = 0; w < 16; ++w) t += wsum[w];
+      base += t;
+    }
+    __syncthreads();
+  }
+  const int n = base, npad = (n + 15) / 16 * 16;
+  for (int t = n + tid; t < npad; t += 1024) out[t] = -1;
+  if (tid == 0) ncommon[g] = npad;
+}
+
+// one block per set: the rows in which the set's list differs from its group's majority list
+__global__ __launch_bounds__(1024) void delta_rows_kernel(const DeltaSet* __restrict__ sets, const int32_t* __restrict__ votes,
+                                                          const int32_t* __restrict__ group_size, int rows, int cap,
+                                                          int32_t* __restrict__ delta, int32_t* __restrict__ dlen) {
+  extern __shared__ unsigned keptbits[];  // one bit per row
+  const DeltaSet d = sets[blockIdx.x];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int words = (rows + 31) / 32;
+  for (int w = tid; w < words; w += 1024) keptbits[w] = 0u;
+  __shared__ int wsum[16];
+  __shared__ int base;
+  if (tid == 0) base = 0;
+  __syncthreads();
+  for (int t = tid; t < d.kp; t += 1024) {
+    const int r = d.kept[t];
+    if (r >= 0 && r < rows) atomicOr(&keptbits[r >> 5], 1u << (r & 31));
+  }
+  __syncthreads();
+  const int half = group_size[d.group];
+  int32_t* out = delta + (int64_t)blockIdx.x * cap;
+  for (int r0 = 0; r0 < rows; r0 += 1024) {
+    const int r = r0 + tid;
+    bool kept = false, common = false;
+    if (r < rows) {
+      kept = (keptbits[r >> 5] >> (r & 31)) & 1u;
+      common = 2 * votes[(int64_t)d.group * rows + r] > half;
+    }
+    const bool diff = kept != common;
+    const unsigned long long bal = __ballot(diff);
+    if (lane == 0) wsum[wave] = __popcll(bal);
+    __syncthreads();
+    int off = base;
+    for (int w = 0; w < wave; ++w) off += wsum[w];
+    if (diff) {
+      const int pos = off + __popcll(bal & ((1ull << lane) - 1));
+      if (pos < cap) out[pos] = kept ? r : (r | kSegSubtract);  // kept but not common: add; common but not kept: take away
+    }
+    __syncthreads();
+    if (tid == 0) {
+      int t = 0;
+      for (int w = 0; w < 16; ++w) t += wsum[w];
+      base += t;
+    }
+    __syncthreads();
+  }
+  const int n = base;
+  if (n > cap) {
+    if (tid == 0) dlen[blockIdx.x] = -1;
+    return;
+  }
+  const int npad = (n + kSegKS - 1) / kSegKS * kSegKS;
+  for (int t = n + tid; t < npad; t += 1024) out[t] = -1;
+  if (tid == 0) dlen[blockIdx.x] = n;
+}
+
+// Sets that start from their group's shared product (DeltaOut).  A block takes 128 rows x 64 columns of that product
+// into registers once (four waves of 16 columns each, a lane owns two adjacent rows) and then writes that piece of
+// one set after the other of a batch of sets of the group: per set the few rank-one terms of its row differences,
+// the four range sums of the piece, and 16-byte streaming stores.  The shared product is read once per batch, so
+// the pass moves little more than the bytes it writes.
+constexpr int kDeltaCols = 64;  // columns of a block's piece = columns per chunk of range sums
+struct DeltaBatch {
+  int32_t first, nsets;  // sets [first, first + nsets) of the table, all of one group
+};
+__global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaOut* __restrict__ sets, const DeltaBatch* __restrict__ batches,
+                                                          const double* __restrict__ A, int64_t lda, int Mp,
+                                                          const double* __restrict__ bias, int64_t ldo) {
+  const DeltaBatch bt = batches[blockIdx.z];
+  const DeltaOut d0 = sets[bt.first];
+  const int cc = blockIdx.x, rb = blockIdx.y;
+  const int j0 = cc * kDeltaCols;
+  if (j0 >= d0.ncols) return;  // (the sets of a group have the same columns)
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r0 = rb * 128 + 2 * lane;
+  const bool active = r0 < Mp;
+  const int jw = j0 + 16 * wave;                // this wave's first column
+  const int nj = max(0, min(16, d0.ncols - jw));  // ... and how many it has
+  double2_t base[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    base[u] = double2_t{0.0, 0.0};
+    if (active && u < nj) base[u] = *reinterpret_cast<const double2_t*>(d0.base + (int64_t)(jw + u) * Mp + r0);
+  }
+  __shared__ double2_t red[2][3][4][64];  // the sums of waves 1-3 of a set, two sets in flight
+  for (int s = 0; s < bt.nsets; ++s) {
+    const DeltaOut d = sets[bt.first + s];
+    double2_t x1 = {0.0, 0.0}, x2 = {0.0, 0.0}, y1 = {0.0, 0.0}, y2 = {0.0, 0.0};
+    // the set's row differences (usually a handful): the first four are looked up once per set - entry, weight column
+    // entries of the lane's rows, row of the shared operand - and any more go through the loop per column
+    int e4[4];
+    double2_t w4[4];
+    const double* s4[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      e4[t] = t < d.dlen ? d.delta[t] : -1;
+      const int r = max(e4[t], 0) & (kSegSubtract - 1);
+      w4[t] = double2_t{0.0, 0.0};
+      if (e4[t] >= 0 && active) w4[t] = *reinterpret_cast<const double2_t*>(A + (int64_t)r * lda + r0);
+      if (e4[t] >= 0 && (e4[t] & kSegSubtract)) w4[t] = -w4[t];  // the row is taken away: -(w * s) = (-w) * s
+      s4[t] = d.S + (int64_t)r * d.lds;
+    }
+    if (active && nj > 0) {
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        if (u < nj) {
+          const int j = jw + u;
+          double2_t o = base[u];
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (e4[t] >= 0) {
+              const double sv = s4[t][j];
+              o[0] = fma(w4[t][0], sv, o[0]);
+              o[1] = fma(w4[t][1], sv, o[1]);
+            }
+          for (int t = 4; t < d.dlen; ++t) {
+            const int e = d.delta[t];
+            const int r = e & (kSegSubtract - 1);
+            const double2_t w = *reinterpret_cast<const double2_t*>(A + (int64_t)r * lda + r0);
+            double sv = d.S[(int64_t)r * d.lds + j];
+            if (e & kSegSubtract) sv = -sv;
+            o[0] = fma(w[0], sv, o[0]);
+            o[1] = fma(w[1], sv, o[1]);
+          }
+          if (j == 0) {  // the centre is the set's own product, bias last
+            o = *reinterpret_cast<const double2_t*>(d.cprod + r0);
+            if (bias != nullptr) {
+              o[0] = o[0] + bias[r0];
+              o[1] = o[1] + bias[r0 + 1];
+            }
+          } else if (d.rpart != nullptr) {
+            const double pl = d.plb[j - 1], pu = d.pub[j - 1];
+            const double px = fmax(o[0], 0.0), nx = fmin(o[0], 0.0), py = fmax(o[1], 0.0), ny = fmin(o[1], 0.0);
+            x1[0] = fma(px, pl, x1[0]);
+            x1[1] = fma(py, pl, x1[1]);
+            x2[0] = fma(nx, pu, x2[0]);
+            x2[1] = fma(ny, pu, x2[1]);
+            y1[0] = fma(px, pu, y1[0]);
+            y1[1] = fma(py, pu, y1[1]);
+            y2[0] = fma(nx, pl, y2[0]);
+            y2[1] = fma(ny, pl, y2[1]);
+          }
+          // (streaming store: the output is not read again here)
+          __builtin_nontemporal_store(o, reinterpret_cast<double2_t*>(d.out + (int64_t)j * ldo + r0));
+        }
+      }
+    }
+    if (d.rpart == nullptr) continue;  // (all sets of a call agree on this)
+    const int par = s & 1;
+    if (wave > 0) {
+      red[par][wave - 1][0][lane] = x1;
+      red[par][wave - 1][1][lane] = x2;
+      red[par][wave - 1][2][lane] = y1;
+      red[par][wave - 1][3][lane] = y2;
+    }
+    // one barrier per set: wave 0 reads this buffer before it reaches the next barrier, and the buffer is written
+    // again only after that one (two sets later).  The barrier waits for the LDS writes only: __syncthreads would
+    // also sit out the round trip of every output store in flight.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (wave == 0 && active) {
+      for (int w = 0; w < 3; ++w) {  // the waves in order
+        x1 += red[par][w][0][lane];
+        x2 += red[par][w][1][lane];
+        y1 += red[par][w][2][lane];
+        y2 += red[par][w][3][lane];
+      }
+      double* dst = d.rpart + (int64_t)cc * 4 * ldo + r0;
+      *reinterpret_cast<double2_t*>(dst) = x1;            // xmin1 = sum max(v,0)*plb
+      *reinterpret_cast<double2_t*>(dst + ldo) = x2;      // xmin2 = sum min(v,0)*pub
+      *reinterpret_cast<double2_t*>(dst + 2 * ldo) = y1;  // xmax1 = sum max(v,0)*pub
+      *reinterpret_cast<double2_t*>(dst + 3 * ldo) = y2;  // xmax2 = sum min(v,0)*plb
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void masked_centres_kernel(const CentreSet* __restrict__ sets, double* __restrict__ Cm, int64_t Kp) {
+  const CentreSet d = sets[blockIdx.x];
+  double* col = Cm + (int64_t)blockIdx.x * Kp;
+  for (int t = threadIdx.x; t < d.kp; t += 256) {
+    const int r = d.kept[t];
+    if (r >= 0) col[r] = d.centre[r];
+  }
+}
 }  // namespace
 
 int launch_scaled_rows(nnvhip_ctx* ctx, const ScaledRows& a) {
@@ -455,6 +681,62 @@ int launch_scaled_rows(nnvhip_ctx* ctx, const ScaledRows& a) {
     max_rows = std::max(max_rows, a.s[k].rows);
   }
   hipLaunchKernelGGL(scaled_rows_kernel, dim3((unsigned)(max_rows + 1), (unsigned)a.count), dim3(256), 0, ctx->stream, a);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev, int groups, const int32_t* group_size_dev,
+                       int64_t rows, int64_t rows_pad, int cap, int32_t* votes, int32_t* common, int32_t* ncommon, int32_t* delta,
+                       int32_t* dlen) {
+  if (count <= 0 || groups <= 0 || rows <= 0 || rows >= (int64_t(1) << 30) || cap % kSegKS != 0 || rows_pad % 16 != 0 ||
+      rows_pad < rows)
+    NNV_FAIL(NNVHIP_ERR_ARG, "internal: row-difference lists out of range");
+  const size_t bits = sizeof(unsigned) * (size_t)ceil_div(rows, 32);
+  if (bits > (size_t)48 << 10) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: too many rows for the row-difference lists");
+  NNV_HIP_TRY(hipMemsetAsync(votes, 0, sizeof(int32_t) * (size_t)groups * (size_t)rows, ctx->stream));
+  hipLaunchKernelGGL(vote_rows_kernel, dim3((unsigned)count), dim3(256), 0, ctx->stream, sets_dev, votes, (int)rows);
+  hipLaunchKernelGGL(common_rows_kernel, dim3((unsigned)groups), dim3(1024), 0, ctx->stream, votes, group_size_dev, (int)rows,
+                     (int)rows_pad, common, ncommon);
+  hipLaunchKernelGGL(delta_rows_kernel, dim3((unsigned)count), dim3(1024), bits, ctx->stream, sets_dev, votes, group_size_dev, (int)rows,
+                     cap, delta, dlen);
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+int delta_tile_chunks(int64_t ncols) { return (int)ceil_div(ncols, kDeltaCols); }
+
+int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp, const double* bias, int64_t ldo, int64_t count,
+                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes) {
+  if (count <= 0 || max_cols <= 0) return NNVHIP_OK;
+  if (Mp % 16 || Mp > ldo || count >= (int64_t(1) << 24)) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: shared-product tiles out of range");
+  // batches of neighbouring sets of one group: long enough to make the read of the shared piece small next to the
+  // writes, short enough for a grid that covers the chip a few times over
+  const int64_t row_blocks = ceil_div(Mp, 128), col_chunks = ceil_div(max_cols, kDeltaCols);
+  int64_t per_batch = 16;
+  while (per_batch > 2 && ceil_div(count, per_batch) * row_blocks * col_chunks < 4096) per_batch /= 2;
+  std::vector<DeltaBatch> batches;
+  for (int64_t a = 0; a < count;) {
+    int64_t b = a + 1;
+    while (b < count && b - a < per_batch && group_of[b] == group_of[a]) ++b;
+    batches.push_back(DeltaBatch{(int32_t)a, (int32_t)(b - a)});
+    a = b;
+  }
+  if (batches.size() > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "array too large for one launch");
+  BufRef tab, btab;
+  NNV_TRY(ctx->upload_table(sets, sizeof(DeltaOut) * count, &tab));
+  NNV_TRY(ctx->upload_table(batches.data(), sizeof(DeltaBatch) * batches.size(), &btab));
+  const bool timed = ctx->kernel_timing;
+  NNV_LAUNCH(ctx, timed, delta_tiles_kernel, dim3((unsigned)col_chunks, (unsigned)row_blocks, (unsigned)batches.size()), dim3(256), 0,
+             tab->as<DeltaOut>(), btab->as<DeltaBatch>(), A, lda, (int)Mp, bias, ldo);
+  NNV_TRY(ctx->kernel_timer_end(timed, 10, bytes));
+  NNV_HIP_TRY(hipGetLastError());
+  return NNVHIP_OK;
+}
+
+int launch_masked_centres(nnvhip_ctx* ctx, int64_t count, const CentreSet* sets_dev, double* Cm, int64_t Kp) {
+  if (count <= 0) return NNVHIP_OK;
+  NNV_HIP_TRY(hipMemsetAsync(Cm, 0, sizeof(double) * (size_t)Kp * (size_t)count, ctx->stream));
+  hipLaunchKernelGGL(masked_centres_kernel, dim3((unsigned)count), dim3(256), 0, ctx->stream, sets_dev, Cm, Kp);
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }

@@ -254,6 +254,9 @@ struct nnvhip_ctx {
   // convolutions compute every generator image in full instead of inside its window (nnvhip_star::box;
   // environment NNVHIP_NO_CONV_BOXES)
   bool no_conv_boxes = false;
+  // arrays of sets of one shape always contract over their whole kept-row lists instead of starting from their
+  // group's shared product and contracting over the rows in which they differ (environment NNVHIP_NO_ROW_DELTAS)
+  bool no_row_deltas = false;
   // debugging aid (environment NNVHIP_POISON_PENDING): columns left unwritten are filled with NaNs
   bool poison_pending = false;
   // per-layer timing
@@ -268,7 +271,9 @@ struct nnvhip_ctx {
   // normalisation, input normalisation, average pooling, flatten), [5] gather of W's columns for the
   // one-hot generator columns of an FC layer (work = algorithmic bytes)
   // [6] ReLU classification, [7] range reduction, [8] whole-reach kernel of small networks (chain.hip)
-  static constexpr int kKernelGroups = 10;
+  // [9] tile kernel of gemm_seg.hip (work = flop), [10] outputs that start from a product shared by many sets and
+  // add only the rows in which a set differs from it (delta_tiles_kernel; work = bytes written)
+  static constexpr int kKernelGroups = 11;
   double kern_ms[kKernelGroups] = {};
   int64_t kern_launches[kKernelGroups] = {};
   double kern_flop[kKernelGroups] = {};
@@ -532,9 +537,53 @@ struct SegTile {
   const double* pub;
   double* rpart;        // or null
 };
+// flag of an entry of a row-difference list (launch_delta_lists): the row is taken away, not added
+constexpr int32_t kSegSubtract = 1 << 30;
 int launch_pack_rows_t(nnvhip_ctx* ctx, int64_t count, const PackSet* sets);
 int launch_gemm_seg(nnvhip_ctx* ctx, const double* A, int64_t lda, double* C, int64_t ldc, int64_t Mp, const double* bias,
                     int tn, const SegTile* segs, int64_t ntiles, double flop, bool gather_b = false);
+// Row lists of the sets of an array, by group (sets whose packed rows agree wherever they keep the same row): the
+// rows a majority of a group keeps (`common`, ascending, padded with -1 to a multiple of 16; its padded length in
+// ncommon[group]) and, per set, the rows in which it differs from its group's list (`delta`: at most cap entries
+// per set, ascending, r or r | kSegSubtract, padded with -1 to a multiple of 8; dlen[set] = their number, or -1
+// if the set differs in more than cap rows).
+struct DeltaSet {
+  const int32_t* kept;  // ascending, kp entries, -1 padded
+  int32_t kp;
+  int32_t group;
+};
+int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev, int groups, const int32_t* group_size_dev,
+                       int64_t rows, int64_t rows_pad, int cap, int32_t* votes /* groups x rows, scratch */, int32_t* common /* groups x rows_pad */,
+                       int32_t* ncommon, int32_t* delta /* count x cap */, int32_t* dlen);
+// The output of one set that starts from its group's shared product: out(:, j) = base(:, j) + sum over the set's
+// row differences of (+/-) A(:, r) * S(r, j) for j < ncols, the centre column (j = 0) replaced by cprod (+ bias), and
+// the four Star.estimateRanges partial sums of every piece of delta_tile_chunks' columns in rpart ([piece][4][ldo]).  A streaming
+// pass (gemm_seg.hip, delta_tiles_kernel): bound by the bytes it writes.
+struct DeltaOut {
+  const int32_t* delta;  // dlen entries: r or r | kSegSubtract
+  const double* base;    // Mp x ncols, leading dimension Mp
+  const double* S;       // the group's scaled rows, row-major: S(r, j) at S[r * lds + j]
+  int64_t lds;
+  const double* cprod;   // Mp entries
+  double* out;           // the set's column 0 (leading dimension ldo)
+  const double* plb;     // the set's predicate bounds, by generator column
+  const double* pub;
+  double* rpart;
+  int32_t dlen;
+  int32_t ncols;
+};
+// (sets: host table, neighbours of one group next to one another; group_of[i]: group of set i of the table; the
+// pass leaves delta_tile_chunks(ncols) chunks of range sums per set)
+int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp, const double* bias, int64_t ldo, int64_t count,
+                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes);
+int delta_tile_chunks(int64_t ncols);
+// Cm(r, s) = centre of set s at row r if the set keeps row r, else +0: Cm is Kp x count (ld = Kp), zeroed here.
+struct CentreSet {
+  const int32_t* kept;
+  const double* centre;
+  int32_t kp;
+};
+int launch_masked_centres(nnvhip_ctx* ctx, int64_t count, const CentreSet* sets_dev, double* Cm, int64_t Kp);
 // The matrices the gathering tiles read, up to 16 per launch: row r < rows of one is [0, Wt(r, idx[j - 1]) *
 // scale[idx[j - 1]] for 1 <= j < ncols, zeros up to ld], row `rows` is all zeros.  out: (rows + 1) x ld, row-major.
 struct ScaledRows {

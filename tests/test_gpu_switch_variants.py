@@ -24,6 +24,7 @@ VARIANTS = {
     "no_conv_boxes": ("no_conv_boxes",),
     "poison_without_conv_boxes": ("poison_pending", "no_conv_boxes"),
     "dense_affine": ("dense_affine",),
+    "no_row_deltas": ("no_row_deltas",),
 }
 
 
