@@ -231,3 +231,40 @@ def test_arrays_of_boxes_that_share_their_half_widths(nnv, oracle, shapes, hidde
     dev_in = nnv.Star.from_boxes(lbs, ubs)
     ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
     _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area")
+
+
+def _shared_product_launches(ctx, fn):
+    """Runs fn with per-kernel timing on; returns (result, launches of the pass that writes sets as their group's
+    shared product plus row differences)."""
+    ctx.kernel_time(10)
+    ctx.set_timing(2)
+    try:
+        res = fn()
+    finally:
+        ctx.set_timing(0)
+    return res, ctx.kernel_time(10)[1]
+
+
+@pytest.mark.parametrize("spread,shapes,expect", [(0.0, 1, True), (2e-3, 2, True), (2e-2, 3, True), (0.1, 2, None), (0.5, 2, False)])
+def test_neighbouring_boxes_share_the_product_over_their_common_rows(nnv, oracle, spread, shapes, expect):
+    """96 boxes around one centre, in `shapes` different half-width vectors.  The closer the centres, the more alike
+    the rows the first ReLU keeps: the second FC layer then forms one product per shape over the rows most sets keep
+    and adds, per set, the rows in which it differs (none at spread 0; 0-2; 1-9, more than the kernel looks up once
+    per set; a few dozen at spread 0.1, where either route may be taken); far-apart boxes (66-118 rows) differ in too
+    many rows and every set contracts over its own list.  Every set against the oracle either way, and the
+    route that was taken is checked."""
+    rs = np.random.RandomState(900 + shapes)
+    n_in, count, hidden = 200, 96, 400
+    widths = rs.randint(1, 64, size=(n_in, shapes)) / 8192.0
+    half = widths[:, np.arange(count) % shapes]
+    c0 = rs.randint(256, 768, size=(n_in, 1)) / 1024.0
+    centre = c0 + np.round(rs.randn(n_in, count) * spread * 1024.0) / 1024.0
+    lbs, ubs = centre - half, centre + half
+    assert np.array_equal(0.5 * (ubs - lbs), half)
+    layers = [_fc(rs, hidden, n_in, 2.0), {"type": "relu"}, _fc(rs, 260, hidden, 2.0), {"type": "relu"}, _fc(rs, 6, 260)]
+    dev_in = nnv.Star.from_boxes(lbs, ubs)
+    ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
+    ctx = nnv.default_context()
+    _, launches = _shared_product_launches(ctx, lambda: _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area"))
+    if expect is not None and not ctx.switch_is_on("no_row_deltas", "dense_affine", "eager_tail"):
+        assert (launches > 0) == expect, "spread %g: %d launches of the shared-product pass" % (spread, launches)

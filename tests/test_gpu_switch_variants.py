@@ -77,6 +77,11 @@ def test_arrays_of_boxes_that_share_their_half_widths(route, nnv, oracle, shapes
     seqs.test_arrays_of_boxes_that_share_their_half_widths(nnv, oracle, shapes, hidden)
 
 
+@pytest.mark.parametrize("spread,shapes", [(2e-3, 2), (2e-2, 3)])
+def test_neighbouring_boxes_share_the_product_over_their_common_rows(route, nnv, oracle, spread, shapes):
+    seqs.test_neighbouring_boxes_share_the_product_over_their_common_rows(nnv, oracle, spread, shapes, None)
+
+
 def test_one_wide_set_through_the_tile_kernel(route, nnv, oracle):
     seqs.test_one_wide_set_through_the_tile_kernel(nnv, oracle, "relax-star-area")
 
