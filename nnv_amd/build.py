@@ -14,7 +14,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libnnvhip.so")
-SOURCES = ["ctx.hip", "gemm.hip", "gemm_seg.hip", "conv.hip", "ranges.hip", "relu.hip", "chain.hip", "spec.hip", "elementwise.hip"]
+SOURCES = ["ctx.hip", "sets.hip", "weights.hip", "fc_layer.hip", "layers.hip", "gemm.hip", "gemm_seg.hip", "conv.hip", "ranges.hip", "relu.hip", "chain.hip", "spec.hip", "elementwise.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fvisibility=hidden",

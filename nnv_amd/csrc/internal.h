@@ -44,6 +44,13 @@ void set_error(const char* fmt, ...);
     if (s_ != NNVHIP_OK) return s_;   \
   } while (0)
 
+// start of every entry point that takes a context: rejects null and selects the context's device
+#define CHECK_CTX(c)                                                  \
+  do {                                                                \
+    if (!(c)) NNV_FAIL(NNVHIP_ERR_ARG, "null context");               \
+    NNV_TRY(nnvhip::enter_ctx(c));                                    \
+  } while (0)
+
 #define NNV_FAIL(code, ...)             \
   do {                                  \
     ::nnvhip::set_error(__VA_ARGS__);   \
