@@ -689,7 +689,7 @@ int reach_small_chain(nnvhip_ctx* c, int64_t n_layers, const int32_t* kind, cons
           o->oh_from = prev->n + 1;
           o->oh_idx_buf = iarena;
           o->oh_idx = IA + L.idx_off;
-          auto node = std::make_shared<ConsNode>();
+          auto node = make_ref<ConsNode>();
           node->prev = prev->cons;
           node->n_before = prev->n;
           node->src = prev->Vbuf;  // C2/C3 rows are rows of the pre-ReLU [c V]

@@ -107,7 +107,7 @@ int nnvhip_ctx::alloc(size_t bytes, BufRef* out) {
     }
   }
   bytes_in_use += (int64_t)cls;
-  auto b = std::make_shared<Buffer>();
+  auto b = make_ref<Buffer>();
   b->ctx = this;
   b->ptr = p;
   b->bytes = cls;
@@ -160,7 +160,7 @@ int nnvhip_ctx::upload_table(const void* host, size_t bytes, BufRef* out) {
   void* st = nullptr;
   NNV_TRY(stage(bytes, &st));
   memcpy(st, host, bytes);
-  auto b = std::make_shared<Buffer>();  // no owner: the slot belongs to the ring
+  auto b = make_ref<Buffer>();  // no owner: the slot belongs to the ring
   b->ptr = st;
   b->bytes = bytes;
   *out = std::move(b);

@@ -57,7 +57,64 @@ void set_error(const char* fmt, ...);
     return (code);                      \
   } while (0)
 
+// Reference-counted pointer with a plain count inside the object it points to.  A context and everything made from
+// it are used from one host thread at a time (the reference's layer loop is single-threaded, and the pool below
+// has no lock either), so the count needs no atomic operations: an array of a thousand sets copies tens of
+// thousands of these per layer, and the locked increments of std::shared_ptr were most of the host time of a
+// ReLU step over such an array.
+template <class T>
+class Ref {
+ public:
+  Ref() = default;
+  Ref(std::nullptr_t) {}
+  explicit Ref(T* p) : p_(p) {
+    if (p_) ++p_->ref_count;
+  }
+  Ref(const Ref& o) : p_(o.p_) {
+    if (p_) ++p_->ref_count;
+  }
+  Ref(Ref&& o) noexcept : p_(o.p_) { o.p_ = nullptr; }
+  Ref& operator=(const Ref& o) {
+    if (o.p_) ++o.p_->ref_count;
+    release();
+    p_ = o.p_;
+    return *this;
+  }
+  Ref& operator=(Ref&& o) noexcept {
+    if (this != &o) {
+      release();
+      p_ = o.p_;
+      o.p_ = nullptr;
+    }
+    return *this;
+  }
+  ~Ref() { release(); }
+  void reset() {
+    release();
+    p_ = nullptr;
+  }
+  T* get() const { return p_; }
+  T* operator->() const { return p_; }
+  T& operator*() const { return *p_; }
+  explicit operator bool() const { return p_ != nullptr; }
+  bool operator==(const Ref& o) const { return p_ == o.p_; }
+  bool operator!=(const Ref& o) const { return p_ != o.p_; }
+  bool operator==(std::nullptr_t) const { return p_ == nullptr; }
+  bool operator!=(std::nullptr_t) const { return p_ != nullptr; }
+
+ private:
+  void release() {
+    if (p_ && --p_->ref_count == 0) delete p_;
+  }
+  T* p_ = nullptr;
+};
+template <class T>
+Ref<T> make_ref() {
+  return Ref<T>(new T());
+}
+
 struct Buffer {
+  int64_t ref_count = 0;
   nnvhip_ctx* ctx = nullptr;
   void* ptr = nullptr;
   size_t bytes = 0;  // size class the block belongs to
@@ -65,7 +122,7 @@ struct Buffer {
   template <class T>
   T* as() const { return static_cast<T*>(ptr); }
 };
-using BufRef = std::shared_ptr<Buffer>;
+using BufRef = Ref<Buffer>;
 
 // Word a ReLU classification kernel posts to the host mailbox: call number in the top 16 bits, the
 // crossing and the inactive count in 24 bits each.  kMailboxEmpty is what the host stores into a word
@@ -137,7 +194,8 @@ struct ColSource {
 // One node per ReLU layer of the structured constraint store.  The dense NNV matrix
 // [C0; C1; C2; C3] (nn/funcs/PosLin.m:711-735) is only materialised when the host reads it.
 struct ConsNode {
-  std::shared_ptr<ConsNode> prev;  // null for the base node
+  int64_t ref_count = 0;
+  Ref<ConsNode> prev;  // null for the base node
   int64_t p_total = 0;             // constraint rows up to and including this node
   int64_t n_total = 0;             // predicate variables up to and including this node
   // base node: dense C0 (p_total x n_total, ld = ldc) and d0
@@ -159,7 +217,7 @@ struct ConsNode {
   BufRef index;                  // crossing neuron indices in new-predicate order: int32[m] at index_off
   int64_t index_off = 0;
 };
-using ConsRef = std::shared_ptr<ConsNode>;
+using ConsRef = Ref<ConsNode>;
 
 // start of every entry point that touches device data: selects the context's device
 int enter_ctx(nnvhip_ctx* ctx);

@@ -790,14 +790,14 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     std::vector<nnvhip_star*> v;
     ~PreCreated() { release_all(v); }  // only what was not handed over
   } pre;
-  std::vector<std::shared_ptr<ConsNode>> nodes;
+  std::vector<ConsRef> nodes;
   const bool precreate = lazy_rows && fold_bounds && count > 1;
   if (precreate) {
     pre.v.reserve(count);
     nodes.resize(count);
     for (int64_t i = 0; i < count; ++i) {
       pre.v.push_back(new_star(ctx));
-      nodes[i] = std::make_shared<ConsNode>();
+      nodes[i] = make_ref<ConsNode>();
       init_static(pre.v[i], nodes[i].get(), i);
     }
   }
@@ -917,7 +917,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   for (int64_t i = 0; i < count; ++i) {
     const ReluDesc& d = descs[i];
     nnvhip_star* o = precreate ? pre.v[i] : new_star(ctx);
-    std::shared_ptr<ConsNode> node = precreate ? std::move(nodes[i]) : std::make_shared<ConsNode>();
+    ConsRef node = precreate ? std::move(nodes[i]) : make_ref<ConsNode>();
     if (!precreate) init_static(o, node.get(), i);
     o->n = in[i]->n + d.m;
     if (!lazy_rows) {

@@ -60,7 +60,7 @@ int nnvhip_star_create(nnvhip_ctx* c, int64_t N, int64_t n, const double* V, con
     c->h2d_bytes += (int64_t)sizeof(double) * 2 * npad;
     NNV_HIP_TRY(hipStreamSynchronize(c->stream));
   }
-  auto base = std::make_shared<ConsNode>();
+  auto base = make_ref<ConsNode>();
   base->p_total = p;
   base->n_total = n;
   if (p > 0 && n > 0) {
@@ -200,7 +200,7 @@ int nnvhip_star_from_box(nnvhip_ctx* c, int64_t N, int64_t count, const double* 
     st->plb = pb->as<double>() + poff[shape_of[s]];  // (the same -1 / +1 for every set of the shape)
     st->pub = st->plb + npad;
     // C = zeros(1, n), d = 0 (set/Star.m:226-227): a base node with one all-zero row
-    auto base = std::make_shared<ConsNode>();
+    auto base = make_ref<ConsNode>();
     base->p_total = 1;
     base->n_total = st->n;
     st->cons = base;  // C0/d0 left null = all zeros
@@ -316,7 +316,7 @@ int nnvhip_relu_reduce_mem(nnvhip_ctx* c, nnvhip_star* in, int64_t H, int64_t W,
     hipLaunchKernelGGL(fill_pm_one_kernel, dim3((unsigned)ceil_div(npad, 256), 1), dim3(256), 0, c->stream, s->plb, dinfo->as<int64_t>());
     NNV_HIP_TRY(hipGetLastError());
   }
-  auto base = std::make_shared<ConsNode>();
+  auto base = make_ref<ConsNode>();
   base->p_total = 1;
   base->n_total = n;
   s->cons = base;
