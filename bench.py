@@ -150,6 +150,8 @@ def measure(k, args, ctx, exact_steps, extras):
     ctx.set_dense_affine(args.dense)
     ctx.set_eager_columns(args.written)
     ctx.set_eager_relu(args.written)
+    for nm in args.switch:
+        ctx.set_switch(nm, True)
     net = nnv_amd.NN.from_config(cfg["layers"], cfg["name"])
     opts = {"reachMethod": args.method, "relaxFactor": 1}
     dev_in = device_input_sets(cfg, ctx)
@@ -364,7 +366,7 @@ def measure(k, args, ctx, exact_steps, extras):
         if n_sets < 256:
             c["latency_bound"] = True
         groups.append((cls_ms, c))
-    variant = "dense_contraction" if args.dense else "all_written" if args.written else ""
+    variant = "dense_contraction" if args.dense else "all_written" if args.written else "_".join(args.switch)
     for _, g in groups:
         if g["kernel"] in GROUP_KERNELS:
             g["kernels_in_group"] = list(GROUP_KERNELS[g["kernel"]])
@@ -494,7 +496,7 @@ def measure(k, args, ctx, exact_steps, extras):
     return {
         "value": value, "steps": steps, "warmup": args.warmup, "warm_steps_by_time": n_warm, "ms_per_step": ms_per_step,
         "step_ms": step_ms,
-        "config": {"workload": cfg["name"], "reach_method": args.method, "relax_factor": 1,
+        "config": {"workload": cfg["name"], "reach_method": args.method, "relax_factor": 1, "switches": list(args.switch),
                    "all_sets_written_ms": all_written["ms_per_step"] if all_written else None,
                    "all_sets_written_updates_per_s": all_written["value"] if all_written else None,
                    "all_sets_written_frac_of_hbm_peak": all_written["frac_of_hbm_peak"] if all_written else None,
@@ -527,6 +529,9 @@ def main():
     ap.add_argument("--written", action="store_true",
                     help="every layer writes its whole output matrix in the call (nothing is left for a first read): the "
                          "all_sets_written figure of a default run as a run of its own, for profiles")
+    ap.add_argument("--switch", action="append", default=[],
+                    help="a route switch of the library to set for the run (nnvhip_set_switch), e.g. no_row_deltas: an FC layer "
+                         "over an array contracts every set over its whole kept-row list on the tile kernel; may be repeated")
     ap.add_argument("--cpu-seconds", type=float, default=10.0,
                     help="budget of the headline's CPU baseline sample (the other configurations get a third each)")
     ap.add_argument("--lean", action="store_true",
