@@ -687,6 +687,7 @@ int reach_small_chain(nnvhip_ctx* c, int64_t n_layers, const int32_t* kind, cons
         o->kept_idx = IA + L.idx_off + L.ld;
         if (m > 0) {
           o->oh_from = prev->n + 1;
+          o->oh_plb_zero = true;
           o->oh_idx_buf = iarena;
           o->oh_idx = IA + L.idx_off;
           auto node = make_ref<ConsNode>();

@@ -93,6 +93,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
   // works on it while the host sets up the outputs and the tiles of the contraction.
   BufRef mm_early;
   std::vector<int64_t> mm_slot;  // which pair of the product's columns holds a set's sums
+  bool mm_plb_zero = true;       // every gathered column of every set has predicate lower bound 0
   int st = NNVHIP_OK;
   if (count >= 64 && !c->eager_cols && !c->dense_affine) {
     std::vector<GatherSet> es((size_t)count);
@@ -110,8 +111,9 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       g.m = (int32_t)(nc - d);
       ok = ok && !(g.m > 0 && in[i]->oh_scale_neg);
       any = any || g.m > 0;
+      mm_plb_zero = mm_plb_zero && (g.m == 0 || in[i]->oh_plb_zero);
     }
-    if (ok && any) st = launch_range_sums_mm(c, fc, count, es.data(), &mm_early, &mm_slot);
+    if (ok && any) st = launch_range_sums_mm(c, fc, count, es.data(), &mm_early, &mm_slot, mm_plb_zero);
   }
   if (st == NNVHIP_OK) st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
   if (st == NNVHIP_OK) {
@@ -830,7 +832,11 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
         }
         if (st == NNVHIP_OK && use_mm) {
           if (mm_early) mm_sums = mm_early;  // queued at the start of the call, from the same lists
-          else st = launch_range_sums_mm(c, fc, count, gs.data(), &mm_sums, &mm_slot);
+          else {
+            bool zero = true;
+            for (int64_t i = 0; i < count; ++i) zero = zero && (gs[i].m == 0 || in[i]->oh_plb_zero);
+            st = launch_range_sums_mm(c, fc, count, gs.data(), &mm_sums, &mm_slot, zero);
+          }
         }
         if (st == NNVHIP_OK) {
           for (int64_t i = 0; i < count; ++i) {

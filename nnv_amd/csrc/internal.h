@@ -434,6 +434,9 @@ struct nnvhip_star {
   bool has_producer_sums() const { return (rng_part != nullptr && rng_chunks > 0) || rng_mm != nullptr; }
   // some scale of the unit-vector block is negative (a box with ub < lb): sign-split products do not apply
   bool oh_scale_neg = false;
+  // the predicates of the unit-vector block all have lower bound 0 (the block was appended by a ReLU step:
+  // new_pred_lb = [plb; zeros(m,1)], nn/funcs/PosLin.m:737): products with those bounds are zero
+  bool oh_plb_zero = false;
   // The reference's Star carries an outer zonotope Z from Star(lb, ub) on (set/Star.m:220-237) and maps it along in
   // affineMap (:332-340, set/Zono.m:47-74) until the ReLU step returns a Star without one (nn/funcs/PosLin.m:740).
   // Z = Zono(V(:,1), V(:,2:end)) of the same set all the way -- Star(lb, ub) builds both from the same centre and
@@ -763,7 +766,9 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 // [xmin1; xmax2] and [xmax1; xmin2].  One fp64 MFMA product over all sets instead of a pass over the
 // cache-resident weights per set.  out: 2*Mp x 2*count, ld = 2*Mp, columns 2i and 2i+1 belong to set i.
 int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out,
-                         std::vector<int64_t>* slot);  // slot[i]: which pair of columns of `out` holds set i's sums
+                         std::vector<int64_t>* slot,  // slot[i]: which pair of columns of `out` holds set i's sums
+                         bool plb_zero = false);      // every lower bound involved is 0: the first column of every pair is
+                                                      // zero and only the second is multiplied out
 // lb / ub (and, by centre_mode, the centre column) of a fully connected layer's output for one set whose
 // gathered columns need no pass of their own, finished in one kernel (ranges.hip).
 int launch_fc_rowsum(nnvhip_ctx* ctx, const nnvhip_fc* fc, nnvhip_star* out, int mode, const double* scale, const int32_t* cls,

@@ -969,7 +969,7 @@ __global__ __launch_bounds__(256) void sum_vectors_kernel(const GatherSet* __res
 }
 
 int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out,
-                         std::vector<int64_t>* slot) {
+                         std::vector<int64_t>* slot, bool plb_zero) {
   const int64_t Mp = fc->Mp, Kp = fc->Kp;
   if (!fc->Wpn) {
     BufRef w;
@@ -1003,6 +1003,19 @@ int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, co
   hipLaunchKernelGGL(sum_vectors_kernel, dim3((unsigned)nu), dim3(256), 0, ctx->stream, tab->as<GatherSet>(), X->as<double>(), (int)Kp);
   NNV_HIP_TRY(hipGetLastError());
   NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * nu, out));
+  if (plb_zero && nu < (int64_t(1) << 30)) {
+    // a = scatter(sc * plb) is zero for every set: its products [xmin1; xmax2] are +0 (a fill), and only the columns
+    // of b = scatter(sc * pub) go through the matrix cores
+    NNV_HIP_TRY(hipMemsetAsync((*out)->ptr, 0, sizeof(double) * 2 * Mp * 2 * nu, ctx->stream));
+    std::vector<int32_t> odd((size_t)nu);
+    for (int64_t k = 0; k < nu; ++k) odd[(size_t)k] = (int32_t)(2 * k + 1);
+    BufRef cmap;
+    NNV_TRY(ctx->upload_table(odd.data(), sizeof(int32_t) * odd.size(), &cmap));
+    GemmRows rows;
+    rows.colmap = cmap->as<int32_t>();
+    return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, nu, Kp, nullptr,
+                       nullptr, &rows);
+  }
   return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, 2 * nu, Kp,
                      nullptr);
 }

@@ -941,6 +941,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     }
     if (d.m > 0) {  // the appended columns are the unit vectors of the crossing neurons
       o->oh_from = in[i]->n + 1;
+      o->oh_plb_zero = true;
       o->oh_idx_buf = idx_buf;
       o->oh_idx = idx_buf->as<int32_t>() + ld * i;
       if (!eager_tail) o->vcols = in[i]->n + 1;  // ... and exist only as that list
