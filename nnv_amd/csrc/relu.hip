@@ -179,7 +179,9 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
 // What the kernels that settle the order of a crossing list write besides the list: kRankNewBounds: the bounds
 // of the new predicates (new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]) and the crossing
 // neurons' (lb, ub); kRankOldBounds: also the copy of the bounds of the predicates the set already has.
-constexpr int kRankNewBounds = 1, kRankOldBounds = 2;
+// kRankCountOnDevice: the length of the list is read from the set's counters (the kernel was queued before the host
+// knew it, with a grid for the longest possible list).
+constexpr int kRankNewBounds = 1, kRankOldBounds = 2, kRankCountOnDevice = 4;
 
 // Sorts a crossing list of at most 1024 entries that the multi-block classification left in
 // ascending order (keys in d.key, neurons in d.asc_idx).  One block per set; every thread ends up with entry
@@ -333,7 +335,7 @@ constexpr int kRankI = 16;
 constexpr int kRankStage = 2048;
 __global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restrict__ table, ReluDesc one, int flags) {
   const ReluDesc d = table ? table[blockIdx.z] : one;
-  const int m = d.m;
+  const int m = (flags & kRankCountOnDevice) ? d.counts[0] : d.m;
   const int tid = threadIdx.x;
   const int n_in = d.ncols_in - 1;
   if (flags & kRankOldBounds) {
@@ -658,7 +660,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // With the reset pending, all that is left to write are the predicate bounds and the crossing
   // neurons' (lb, ub).  The one-block classification does that itself, into buffers sized for the worst
   // case (every neuron crossing), and the step is a single launch.
-  const bool fold_bounds = lazy_rows && N <= kOneBlockN;
+  // Larger sets with the reset pending: the multi-block classification leaves the counts on the device, and the
+  // kernel that ranks the crossing list is queued right behind it, sized for the longest possible list; the host
+  // reads the counts while it runs.
+  const bool early_rank = lazy_rows && sorted && N > kOneBlockN;
+  const bool fold_bounds = lazy_rows && (N <= kOneBlockN || early_rank);
   BufRef pred_buf, lbub_buf;
   std::vector<int64_t> pred_off(count), lbub_off(count);
   const int64_t ldr_max = round_up(N, kLdAlign);
@@ -729,7 +735,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // algorithmic bytes of the classification: lb and ub read, the per-row class and the two index lists
   // written (plus, when it also writes the predicate bounds, the copy of the input's)
   double cls_bytes = 0.0;
-  for (int64_t i = 0; i < count; ++i) cls_bytes += 24.0 * (double)N + (fold_bounds ? 32.0 * (double)in[i]->n : 0.0);
+  for (int64_t i = 0; i < count; ++i) cls_bytes += 24.0 * (double)N + (fold_bounds && !early_rank ? 32.0 * (double)in[i]->n : 0.0);
   const bool tk = ctx->kernel_timing;
   if (N <= kOneBlockN) {
     if (!sorted)
@@ -745,6 +751,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->kernel_timer_end(tk, 6, 0.5 * cls_bytes));
     NNV_LAUNCH(ctx, tk, relu_compact_kernel, grid, dim3(1024), 0, table, descs[0]);
     NNV_TRY(ctx->kernel_timer_end(tk, 6, 0.5 * cls_bytes));
+    if (early_rank)
+      hipLaunchKernelGGL(relu_rank_kernel, dim3((unsigned)ceil_div(N, kRankI), 1, (unsigned)count), dim3(256), 0, ctx->stream, table,
+                         descs[0], kRankNewBounds | kRankOldBounds | kRankCountOnDevice);
   }
   NNV_HIP_TRY(hipGetLastError());
 
@@ -882,7 +891,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->upload_table(descs.data(), sizeof(ReluDesc) * count, &tab));
     table = tab->as<ReluDesc>();
   }
-  if (sorted && sort_cap == 0 && max_m > 0 && max_m <= 1024) {
+  if (early_rank) {
+    // ranked already
+  } else if (sorted && sort_cap == 0 && max_m > 0 && max_m <= 1024) {
     // (with the reset pending the kernel also writes the predicate bounds, as the rank kernel below does)
     ranked_with_bounds = lazy_rows;
     const int flags = lazy_rows ? (kRankNewBounds | (fold_bounds ? 0 : kRankOldBounds)) : 0;
