@@ -469,6 +469,7 @@ struct StampSet {
   double* part;         // [chunks][4][ldout] range sums of these columns (as the estimateRanges pass leaves them)
   int32_t m;
   int32_t win_only;     // 1: only the rows inside a column's window (the positions whose taps span its pixel) are written
+  const int32_t* pixel_col;  // (by-row pass) input row -> its column here, -1: none
 };
 
 __global__ __launch_bounds__(512) void conv_stamp_kernel(const StampSet* __restrict__ table, StampSet one, ConvGeom g,
@@ -749,7 +750,8 @@ bool conv2d_in_windows(const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho
 
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
-                  const int32_t* pending_cls, const ColBox* out_box, int eh, int ew, const ColBox* in_box, bool leave_outside) {
+                  const int32_t* pending_cls, const ColBox* out_box, int eh, int ew, const ColBox* in_box, bool leave_outside,
+                  const uint32_t* pending_bits) {
   if (cv->Kp > kMaxTaps) NNV_FAIL(NNVHIP_ERR_SHAPE, "filters with more than %d taps (FH*FW*Cin) are not supported", kMaxTaps);
   if ((cv->FH - 1) * cv->dil[0] > 0xffff || (cv->FW - 1) * cv->dil[1] > 0xffff)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "dilated filter extent too large");
@@ -764,12 +766,16 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W
   if (pending_cls != nullptr) {
     if (!conv2d_can_mask(cv, H, W, Ho, Wo, ldin)) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: row mask too large for the convolution kernel");
     keep_words = (int)ceil_div(n_in, 32);
-    NNV_TRY(ctx->alloc(sizeof(uint32_t) * (size_t)keep_words, &bits));
-    // whole waves only, so that every word is written by a lane that exists
-    hipLaunchKernelGGL(keep_bits_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, ctx->stream, pending_cls, n_in,
-                       bits->as<uint32_t>(), keep_words);
-    NNV_HIP_TRY(hipGetLastError());
-    keep = bits->as<uint32_t>();
+    if (pending_bits != nullptr) {
+      keep = pending_bits;
+    } else {
+      NNV_TRY(ctx->alloc(sizeof(uint32_t) * (size_t)keep_words, &bits));
+      // whole waves only, so that every word is written by a lane that exists
+      hipLaunchKernelGGL(keep_bits_kernel, dim3((unsigned)ceil_div(n_in, 256)), dim3(256), 0, ctx->stream, pending_cls, n_in,
+                         bits->as<uint32_t>(), keep_words);
+      NNV_HIP_TRY(hipGetLastError());
+      keep = bits->as<uint32_t>();
+    }
   }
   // 128 positions x Cout tile, eight waves per block (two per SIMD keep the MFMA pipe fed while
   // the other wave gathers)
@@ -914,6 +920,18 @@ __global__ __launch_bounds__(256) void conv_stamp_rows_kernel(StampSet d, ConvGe
 }
 
 static bool conv_stamps_by_row(const nnvhip_conv2d* cv) { return cv->dil[0] == 1 && cv->dil[1] == 1; }
+bool conv_stamps_by_pixel(const nnvhip_conv2d* cv) { return conv_stamps_by_row(cv); }
+
+int launch_pixel_columns(nnvhip_ctx* ctx, const int32_t* idx, int64_t m, int64_t n_in, BufRef* inv) {
+  NNV_TRY(ctx->alloc(sizeof(int32_t) * (size_t)n_in, inv));
+  NNV_HIP_TRY(hipMemsetAsync((*inv)->ptr, 0xff, sizeof(int32_t) * (size_t)n_in, ctx->stream));
+  if (m > 0) {
+    hipLaunchKernelGGL(stamp_pixel_columns_kernel, dim3((unsigned)ceil_div(m, 256)), dim3(256), 0, ctx->stream, idx, (int)m,
+                       (*inv)->as<int32_t>());
+    NNV_HIP_TRY(hipGetLastError());
+  }
+  return NNVHIP_OK;
+}
 
 int64_t conv_stamp_chunks(const nnvhip_conv2d* cv, int64_t ldout, int64_t count, int64_t max_m) {
   if (conv_stamps_by_row(cv)) return 1;
@@ -945,18 +963,21 @@ int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int6
     if (chunks != 1) NNV_FAIL(NNVHIP_ERR_ARG, "internal: one chunk of range sums per set");
     if (g.K > kStampTapTable) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: more taps than the stamp kernel's table holds");
     const int64_t n_in = H * W * cv->Cin;
-    BufRef inv;
-    NNV_TRY(ctx->alloc(sizeof(int32_t) * (size_t)n_in * (size_t)count, &inv));
-    NNV_HIP_TRY(hipMemsetAsync(inv->ptr, 0xff, sizeof(int32_t) * (size_t)n_in * (size_t)count, ctx->stream));
+    std::vector<BufRef> made;  // tables of the sets that came without one
     NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
     for (int64_t i = 0; i < count; ++i) {
       if (sets[i].m == 0) continue;
       StampSet one;
       memcpy(&one, &sets[i], sizeof one);
-      int32_t* pc = inv->as<int32_t>() + n_in * i;
+      const int32_t* pc = one.pixel_col;
+      if (pc == nullptr) {
+        BufRef inv;
+        NNV_TRY(launch_pixel_columns(ctx, one.idx, one.m, n_in, &inv));
+        pc = inv->as<int32_t>();
+        made.push_back(inv);
+      }
       if (!one.win_only)  // whole columns: the zeros first
         NNV_HIP_TRY(hipMemsetAsync(one.out, 0, sizeof(double) * (size_t)ldout * (size_t)one.m, ctx->stream));
-      hipLaunchKernelGGL(stamp_pixel_columns_kernel, dim3((unsigned)ceil_div(one.m, 256)), dim3(256), 0, ctx->stream, one.idx, one.m, pc);
       if (g.K <= 32)
         NNV_LAUNCH(ctx, ctx->kernel_timing && i == 0, conv_stamp_rows_kernel<1>, dim3((unsigned)ceil_div(ldout, 256)), dim3(256), 0, one, g,
                    cv->W->as<double>(), pc, ldout);

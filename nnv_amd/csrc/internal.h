@@ -11,7 +11,6 @@
 #include <map>
 #include <memory>
 #include <string>
-#include <unordered_set>
 #include <vector>
 
 #include "nnvhip.h"
@@ -271,6 +270,7 @@ struct nnvhip_ctx {
   // counters for diagnosing a slow step: hipMalloc calls of the pool, waits for the stream because the pinned
   // staging ring wrapped or grew, mailbox waits that went through the slow path
   int64_t n_device_mallocs = 0, n_staging_waits = 0;
+  uint64_t visit_seq = 0;
   int64_t device_bytes = 0;  // memory of the device (the pool grows past a released array only below a share of it)
   // pinned staging ring for descriptor tables and small read-backs
   char* pinned = nullptr;
@@ -390,6 +390,7 @@ struct nnvhip_star {
   // runs the pending pass (it needs the per-row classification cls) into a buffer of the set's own.
   bool rows_pending = false;
   nnvhip::BufRef cls_buf;
+  const uint32_t* keep_bits = nullptr;  // with cls (in cls_buf): bit r & 31 of word r >> 5 is set where row r is kept
   const int32_t* cls = nullptr;
   nnvhip::BufRef pbuf;
   double* plb = nullptr;
@@ -413,6 +414,10 @@ struct nnvhip_star {
   const int32_t* oh_idx = nullptr;
   const double* oh_scale = nullptr;
   nnvhip::BufRef oh_idx_buf, oh_scale_buf;
+  // The inverse of oh_idx where somebody has made it: oh_inv[r] = t with oh_idx[t] = r, -1 for rows no column names
+  // (N entries).  The ReLU step leaves it for image sets; the convolution's stamp pass makes it otherwise and keeps it.
+  nnvhip::BufRef oh_inv_buf;
+  const int32_t* oh_inv = nullptr;
   // Second hint, set by the ReLU step: only the rows kept_idx[0..n_kept) (ascending; the list is padded
   // with -1 up to a multiple of 16 and at least 16 entries) of the columns before the one-hot block can
   // be non-zero -- every other row was reset.  n_kept < 0 = no such knowledge.
@@ -437,6 +442,7 @@ struct nnvhip_star {
   // the predicates of the unit-vector block all have lower bound 0 (the block was appended by a ReLU step:
   // new_pred_lb = [plb; zeros(m,1)], nn/funcs/PosLin.m:737): products with those bounds are zero
   bool oh_plb_zero = false;
+  uint64_t visit = 0;  // nnvhip_ctx::visit_seq of the last pass that listed this handle (passes over an array skip repeats)
   // The reference's Star carries an outer zonotope Z from Star(lb, ub) on (set/Star.m:220-237) and maps it along in
   // affineMap (:332-340, set/Zono.m:47-74) until the ReLU step returns a Star without one (nn/funcs/PosLin.m:740).
   // Z = Zono(V(:,1), V(:,2:end)) of the same set all the way -- Star(lb, ub) builds both from the same centre and
@@ -690,7 +696,9 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t
                   int eh = 0, int ew = 0,
                   const ColBox* in_box = nullptr /* windows of the input columns: taps outside them are not read (the input
                                                     may be in memory inside its windows only); needs conv2d_in_windows */,
-                  bool leave_outside = false /* do not write the zeros outside the output windows */);
+                  bool leave_outside = false /* do not write the zeros outside the output windows */,
+                  const uint32_t* pending_bits = nullptr /* with pending_cls: the same as one bit per row (1 = kept), where
+                                                            the step that classified the rows left them */);
 int launch_zero_pad_rows(nnvhip_ctx* ctx, double* V, int64_t ld, int64_t N, int64_t ncols);  // rows [N, ld) of ncols columns := 0
 // whether launch_conv2d computes the generator images of such a call inside their windows only
 bool conv2d_in_windows(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin, int64_t ncols,
@@ -715,14 +723,28 @@ struct ConvStampSet {
   double* part;         // this set's [chunks][4][ldout] range sums
   int32_t m;
   int32_t win_only;     // 1: write the rows inside each column's window only
+  const int32_t* pixel_col;  // input row -> its one-hot column (index into idx), -1: none; or null (made by the launch)
 };
+// Whether the stamp launch of this layer looks columns up by pixel (ConvStampSet::pixel_col), and that table for one
+// set: inv[idx[t]] = t, -1 elsewhere (n_in entries, allocated here).
+bool conv_stamps_by_pixel(const nnvhip_conv2d* conv);
+int launch_pixel_columns(nnvhip_ctx* ctx, const int32_t* idx, int64_t m, int64_t n_in, BufRef* inv);
 // Number of column chunks (= range-sum chunks per set) the stamp launch will use.
 int64_t conv_stamp_chunks(const nnvhip_conv2d* conv, int64_t ldout, int64_t count, int64_t max_m);
 int launch_conv_stamps(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                        int64_t ldout, int64_t count, const ConvStampSet* sets, int64_t chunks);
 
 // ranges.hip
-int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s);
+// counts != null: where the estimate of every set of the call ends in the kernel that combines partial sums, that
+// kernel also counts the crossing / inactive / kept neurons (among the first nrows rows) of every `gran` rows of a
+// set: three numbers per block at base + stride * (set's place in the call); gran == 0 afterwards: it did not.
+struct RangeCounts {
+  int32_t* base = nullptr;
+  int64_t stride = 0;  // at least 3 * ceil(ld / 64)
+  int32_t nrows = 0;
+  int32_t gran = 0;    // out: rows per triple (64 or 128), 0: nothing was counted
+};
+int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, RangeCounts* counts = nullptr);
 // the fixed device workspace: address look-up (once per context) and Star.estimateRanges into it
 int init_static_scratch(nnvhip_ctx* ctx);
 int ranges_into_static(nnvhip_ctx* ctx, const nnvhip_star* s, double* lb_dev, double* ub_dev);

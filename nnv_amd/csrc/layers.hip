@@ -131,12 +131,19 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
     stamps[i].pub = o->pub + (pl.dense - 1);
     stamps[i].part = nullptr;
     stamps[i].m = (int32_t)pl.m;
+    if (pl.m > 0 && in[i]->oh_inv == nullptr && conv_stamps_by_pixel(cv)) {
+      // (kept on the input: its columns do not change, and an input set is usually mapped again)
+      st = launch_pixel_columns(c, in[i]->oh_idx, pl.m, in[i]->N, &in[i]->oh_inv_buf);
+      if (st != NNVHIP_OK) break;
+      in[i]->oh_inv = in[i]->oh_inv_buf->as<int32_t>();
+    }
+    stamps[i].pixel_col = in[i]->oh_inv;
     stamps[i].win_only = (lazy && pl.m > 0) ? 1 : 0;
     any_stamps = any_stamps || pl.m > 0;
     max_m = std::max<int64_t>(max_m, pl.m);
     st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, o->V, o->ld, pl.dense,
                        in[i]->rows_pending ? in[i]->cls : nullptr, pl.compact ? ob : nullptr, pl.dense_eh, pl.dense_ew,
-                       pl.compact ? in[i]->box : nullptr, pl.compact && lazy);
+                       pl.compact ? in[i]->box : nullptr, pl.compact && lazy, in[i]->rows_pending ? in[i]->keep_bits : nullptr);
     // (launch_conv2d zeroes the padding rows of the columns it writes; the stamp kernel only writes them when
     // it writes whole columns)
     if (st == NNVHIP_OK && stamps[i].win_only && o->ld != Nout) st = launch_zero_pad_rows(c, stamps[i].out, o->ld, Nout, pl.m);

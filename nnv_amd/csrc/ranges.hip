@@ -36,6 +36,10 @@ struct RangeDesc {
   // bH x bW positions per channel), or null: a row outside a column's window is not loaded
   const ColBox* box;
   int32_t bH, bW;
+  // not null: the kernel that combines the partial sums also counts, per block of its rows, the neurons a ReLU step
+  // will find crossing (lb < 0 < ub), inactive (ub <= 0) and kept among the first nrows rows: three numbers per block
+  int32_t* blk3;
+  int32_t nrows;
 };
 
 constexpr int kRowsPerWave = 128;  // 64 lanes x 2 rows
@@ -328,10 +332,39 @@ __device__ __forceinline__ void load_rows(const double* __restrict__ p, double (
 template <int R>
 __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __restrict__ table, RangeDesc one) {
   const RangeDesc d = table ? table[blockIdx.z] : one;
-  if (d.chunks == 1 && d.chunks2 == 0 && d.part3 == nullptr && d.cols_per_chunk != 0) return;  // the column pass wrote lb/ub itself
   const int lane = threadIdx.x & 63;
   const int q = threadIdx.x >> 6;
   const int64_t r = ((int64_t)blockIdx.x * 64 + lane) * R;
+  // the classes of the block's rows for the ReLU step that follows (RangeDesc::blk3), by the wave that has lb / ub
+  auto count_classes = [&](const double (&l)[R], const double (&u)[R]) {
+    int nc = 0, ni = 0, nk = 0;
+#pragma unroll
+    for (int e = 0; e < R; ++e) {
+      const bool valid = r + e < d.nrows;
+      const bool inactive = valid && (u[e] <= 0.0);
+      const bool crossing = valid && (l[e] < 0.0) && (u[e] > 0.0);
+      nc += __popcll(__ballot(crossing));
+      ni += __popcll(__ballot(inactive));
+      nk += __popcll(__ballot(valid && !inactive && !crossing));
+    }
+    if (lane == 0) {
+      d.blk3[3 * blockIdx.x] = nc;
+      d.blk3[3 * blockIdx.x + 1] = ni;
+      d.blk3[3 * blockIdx.x + 2] = nk;
+    }
+  };
+  if (d.chunks == 1 && d.chunks2 == 0 && d.part3 == nullptr && d.cols_per_chunk != 0) {  // the column pass wrote lb/ub itself
+    if (d.blk3 != nullptr && q == 0) {
+      double l[R], u[R];
+#pragma unroll
+      for (int e = 0; e < R; ++e) {
+        l[e] = r + e < d.ld ? d.lb[r + e] : 0.0;
+        u[e] = r + e < d.ld ? d.ub[r + e] : 0.0;
+      }
+      count_classes(l, u);
+    }
+    return;
+  }
   __shared__ double sums[4][64 * R];
   __shared__ double cen[64 * R];
   if (q == 4) {  // a wave of its own (the launch that has a centre to form brings five)
@@ -424,13 +457,21 @@ __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __re
 #pragma unroll
   for (int e = 0; e < R; ++e) sums[q][lane * R + e] = s[e];
   __syncthreads();
-  if (q == 0 && r < d.ld) {
+  if (q == 0) {
+    double l[R], u[R];
 #pragma unroll
-    for (int e = 0; e < R; ++e) {
-      const double c0 = d.cchunks > 0 ? cen[lane * R + e] : d.V[r + e];
-      d.lb[r + e] = (c0 + sums[0][lane * R + e]) + sums[1][lane * R + e];
-      d.ub[r + e] = (c0 + sums[2][lane * R + e]) + sums[3][lane * R + e];
+    for (int e = 0; e < R; ++e) l[e] = u[e] = 0.0;
+    if (r < d.ld) {
+#pragma unroll
+      for (int e = 0; e < R; ++e) {
+        const double c0 = d.cchunks > 0 ? cen[lane * R + e] : d.V[r + e];
+        l[e] = (c0 + sums[0][lane * R + e]) + sums[1][lane * R + e];
+        u[e] = (c0 + sums[2][lane * R + e]) + sums[3][lane * R + e];
+        d.lb[r + e] = l[e];
+        d.ub[r + e] = u[e];
+      }
     }
+    if (d.blk3 != nullptr) count_classes(l, u);
   }
 }
 
@@ -1029,12 +1070,16 @@ static bool scan_in_windows(const nnvhip_star* t) {
   return 2 * (int64_t)t->box_eh * t->box_ew <= P;
 }
 
-int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
+int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, RangeCounts* counts) {
   // sets that already carry ranges are skipped
   std::vector<nnvhip_star*> todo;
-  std::unordered_set<nnvhip_star*> seen;
+  todo.reserve((size_t)count);
+  const uint64_t visit = ++ctx->visit_seq;  // (a handle may be listed twice)
   for (int64_t i = 0; i < count; ++i)
-    if (!s[i]->lb && seen.insert(s[i]).second) todo.push_back(s[i]);
+    if (!s[i]->lb && s[i]->visit != visit) {
+      s[i]->visit = visit;
+      todo.push_back(s[i]);
+    }
   if (todo.empty()) return NNVHIP_OK;
   // Sets whose generator images are in memory inside their windows only are scanned inside the windows (all
   // sets of the call, or none: one launch serves them all; the same sums to the bit either way).
@@ -1109,6 +1154,8 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
     d.cout = nullptr;
     d.box = nullptr;
     d.bH = d.bW = 0;
+    d.blk3 = nullptr;
+    d.nrows = 0;
     if (in_windows) {
       d.box = t->box;
       d.bH = t->box_H;
@@ -1131,6 +1178,22 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   for (int64_t i = 0; i < nset; ++i) scan = scan || !(descs[i].n == 0 && (descs[i].chunks2 > 0 || descs[i].part3 != nullptr));
   if (!scan)
     for (int64_t i = 0; i < nset; ++i) descs[i].chunks = 0;
+  // an array of sets has blocks to spare for the last step: two rows per lane, read 16 bytes at a time
+  bool wide_final = ceil_div(ld, 64) * nset >= 4096;
+  {
+    auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    for (int64_t i = 0; i < nset && wide_final; ++i)
+      wide_final = aligned16(descs[i].part) && aligned16(descs[i].part2) && aligned16(descs[i].part3) && aligned16(descs[i].V) &&
+                   aligned16(descs[i].lb);
+  }
+  if (counts != nullptr && counts->base != nullptr && (chunks > 1 || any_pending) && nset == count) {
+    // (every set of the call is in the table, in the caller's order)
+    for (int64_t i = 0; i < nset; ++i) {
+      descs[i].blk3 = counts->base + counts->stride * i;
+      descs[i].nrows = counts->nrows;
+    }
+    counts->gran = wide_final ? 128 : 64;
+  }
   const RangeDesc* table = nullptr;
   BufRef tab;
   if (nset > 1) {
@@ -1166,13 +1229,7 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s) {
   if (chunks > 1 || any_pending) {
     double fbytes = 0.0;  // every chunk's four sums read, lb and ub written
     for (int64_t i = 0; i < nset; ++i) fbytes += 8.0 * (double)ld * (4.0 * (double)(descs[i].chunks + descs[i].chunks2) + 3.0);
-    // an array of sets has blocks to spare: two rows per lane, read 16 bytes at a time
-    bool wide = ceil_div(ld, 64) * nset >= 4096;
-    auto aligned16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-    for (int64_t i = 0; i < nset && wide; ++i)
-      wide = aligned16(descs[i].part) && aligned16(descs[i].part2) && aligned16(descs[i].part3) && aligned16(descs[i].V) &&
-             aligned16(descs[i].lb);
-    if (wide)
+    if (wide_final)
       NNV_LAUNCH(ctx, ctx->kernel_timing, ranges_final_kernel<2>, dim3((unsigned)ceil_div(ld, 128), 1, (unsigned)nset), dim3(256), 0,
                  table, descs[0]);
     else

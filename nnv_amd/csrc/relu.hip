@@ -75,6 +75,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
       wcross[wave] = __popcll(bc);
       winact[wave] = __popcll(bi);
       wkeep[wave] = __popcll(bk);
+      if (d.keep_bits != nullptr) *reinterpret_cast<uint2*>(d.keep_bits + ((r0 >> 5) + 2 * wave)) = make_uint2((uint32_t)bk, (uint32_t)(bk >> 32));
     }
     __syncthreads();
     int woff = 0, tot = 0, itot = 0, koff = 0, ktot = 0;
@@ -95,6 +96,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
       d.cls[r] = pos;
       if (d.order == NNVHIP_ORDER_INDEX) {
         idx_out[pos] = r;
+        if (d.col_of != nullptr) d.col_of[r] = pos;
       } else {
         // areas = 0.5*(abs(ub).*abs(lb))  |  ub - lb.  Lists of up to kSortInBlock entries are sorted
         // below, straight from LDS; a set with more neurons than that may have a longer list, which the
@@ -112,6 +114,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
       }
     } else if (valid) {
       d.cls[r] = inactive ? kZero : kKeep;
+      if (d.col_of != nullptr) d.col_of[r] = -1;
     }
     base += tot;
     inact_total += itot;
@@ -135,6 +138,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   int mine = 0;  // entry tid of the sorted list
   if (sort_here)  // the staged doubles are read back as their bit patterns
     mine = sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
+  if (sort_here && d.col_of != nullptr && tid < m) d.col_of[mine] = tid;
   if (d.write_bounds && sort_here) {
     // the output buffers were sized for the worst case: finish the set here.  New predicate tid belongs to the
     // neuron this thread holds: new_pred_lb = [plb; zeros(m,1)], new_pred_ub = [pub; ub(index)]
@@ -206,6 +210,7 @@ __global__ __launch_bounds__(1024) void relu_sort_small_kernel(const ReluDesc* _
   }
   __syncthreads();
   const int mine = sort_small_desc(reinterpret_cast<long long*>(skey), sidx, m, tid, d.cross_idx);
+  if (d.col_of != nullptr && tid < m) d.col_of[mine] = tid;
   if ((flags & kRankNewBounds) && tid < m) {
     const double ub = d.ub[mine];
     d.plb_out[n_in + tid] = 0.0;
@@ -255,12 +260,14 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
   __shared__ int sbase, stot, sinact, skbase;
   if (wave == 0) {  // offset of this block = crossing (kept) counts of the blocks before it
     int before = 0, tot = 0, inact = 0, kbefore = 0;
-    for (int b = lane; b < (int)gridDim.x; b += 64) {
+    const int nent = d.blk_gran == 1024 ? (int)gridDim.x : (int)((d.ld + d.blk_gran - 1) / d.blk_gran);
+    const int mine = (int)blockIdx.x * (1024 / d.blk_gran);  // first entry of this block's rows
+    for (int b = lane; b < nent; b += 64) {
       const int c = d.blk_counts[3 * b];
-      before += b < (int)blockIdx.x ? c : 0;
+      before += b < mine ? c : 0;
       tot += c;
       inact += d.blk_counts[3 * b + 1];
-      kbefore += b < (int)blockIdx.x ? d.blk_counts[3 * b + 2] : 0;
+      kbefore += b < mine ? d.blk_counts[3 * b + 2] : 0;
     }
     for (int off = 32; off > 0; off >>= 1) {
       before += __shfl_xor(before, off);
@@ -287,6 +294,8 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
   if (lane == 0) {
     wcross[wave] = __popcll(bc);
     wkeep[wave] = __popcll(bk);
+    if (d.keep_bits != nullptr)
+      *reinterpret_cast<uint2*>(d.keep_bits + (blockIdx.x * 32 + 2 * wave)) = make_uint2((uint32_t)bk, (uint32_t)(bk >> 32));
   }
   __syncthreads();
   int woff = 0, koff = 0;
@@ -301,11 +310,13 @@ __global__ __launch_bounds__(1024) void relu_compact_kernel(const ReluDesc* __re
     const int pos = sbase + woff + __popcll(bc & ((1ull << lane) - 1ull));
     idx_out[pos] = r;
     d.cls[r] = pos;
+    if (d.order == NNVHIP_ORDER_INDEX && d.col_of != nullptr) d.col_of[r] = pos;
     if (d.order != NNVHIP_ORDER_INDEX) {
       d.key[pos] = d.order == NNVHIP_ORDER_AREA ? 0.5 * (fabs(u) * fabs(l)) : d.order == NNVHIP_ORDER_RANGE ? u - l : d.given_key[r];
     }
   } else if (valid) {
     d.cls[r] = inactive ? kZero : kKeep;
+    if (d.col_of != nullptr) d.col_of[r] = -1;
   }
   if (blockIdx.x == gridDim.x - 1) {
     for (int64_t p = d.N + tid; p < d.ld; p += 1024) d.cls[p] = kKeep;  // padding rows stay zero
@@ -371,6 +382,7 @@ __global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restri
   for (int q = 0; q < 16; ++q) r += part[q][il];
   const int neuron = d.asc_idx[i];
   d.cross_idx[r] = neuron;
+  if (d.col_of != nullptr) d.col_of[neuron] = r;
   if (flags & kRankNewBounds) {
     const double ub = d.ub[neuron];
     d.plb_out[n_in + r] = 0.0;
@@ -550,11 +562,14 @@ int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets,
   }
   // sets with a pending row reset: one arena and one apply launch per leading dimension
   std::vector<nnvhip_star*> pend;
-  std::unordered_set<nnvhip_star*> seen;
+  const uint64_t visit = ++ctx->visit_seq;  // (a handle may be listed twice)
   for (int64_t i = 0; i < count; ++i) {
     nnvhip_star* s = sets[i];
     if (s->rows_pending) {
-      if (seen.insert(s).second) pend.push_back(s);
+      if (s->visit != visit) {
+        s->visit = visit;
+        pend.push_back(s);
+      }
     } else if (need_tail && s->stored_cols() != s->n + 1) {
       NNV_TRY(write_tail_columns(ctx, s));
     }
@@ -601,6 +616,7 @@ int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets,
       s->rows_pending = false;
       s->cls_buf.reset();
       s->cls = nullptr;
+      s->keep_bits = nullptr;
       // The rows that were kept still hold the gathered weight columns, which is all a later packing of kept rows
       // asks of this description; nothing of it is pending any more (the apply pass read whole columns).
       s->cs.pending = false;
@@ -635,19 +651,33 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const bool lazy_rows = !eager_tail && !ctx->eager_rows;
   // (with the reset left pending nothing here reads the inputs' columns: those not written yet stay so)
   NNV_TRY(ensure_dense_batch(ctx, count, in, true, !lazy_rows));
-  if (given == nullptr) NNV_TRY(compute_ranges(ctx, count, in));
   const int64_t N = in[0]->N;
   const int64_t ld = in[0]->ld;
   const int64_t kOneBlockN = one_block_limit();
+  // Larger sets are classified by several blocks, which need the class counts of the blocks before them: the kernel
+  // that finishes the range estimate counts as it writes lb / ub where it is the one that runs; a counting launch
+  // otherwise.
+  BufRef blk_buf;
+  const int64_t nblk = ceil_div(N, 1024);
+  const int64_t blk_stride = 3 * std::max<int64_t>(nblk, ceil_div(ld, 64));
+  RangeCounts rc;
+  if (N > kOneBlockN) {
+    NNV_TRY(ctx->alloc(sizeof(int32_t) * blk_stride * count, &blk_buf));
+    rc.base = blk_buf->as<int32_t>();
+    rc.stride = blk_stride;
+    rc.nrows = (int32_t)std::min<int64_t>(N, INT32_MAX);
+  }
+  if (given == nullptr) NNV_TRY(compute_ranges(ctx, count, in, &rc));
   if (N >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "set dimension too large");
   const bool sorted = order != NNVHIP_ORDER_INDEX;
 
   // scratch shared by all sets: cls | counts ; cross_idx is kept (it becomes the node's index list)
-  BufRef cls_buf, cnt_buf, asc_buf, key_buf, blk_buf;
-  const int64_t nblk = ceil_div(N, 1024);
-  NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &cls_buf));
+  BufRef cls_buf, cnt_buf, asc_buf, key_buf;
+  // (behind the classes: one bit per row, 1 = kept, in whole 1024-row blocks per set -- what a convolution that
+  // applies the pending reset as it loads wants)
+  const int64_t bit_words = ceil_div(N, 1024) * 32;
+  NNV_TRY(ctx->alloc(sizeof(int32_t) * (ld + bit_words) * count, &cls_buf));
   NNV_TRY(ctx->alloc(sizeof(int32_t) * 2 * count, &cnt_buf));
-  if (N > kOneBlockN) NNV_TRY(ctx->alloc(sizeof(int32_t) * 3 * nblk * count, &blk_buf));
   // kept-row lists of all sets in one buffer; the classification pads each list with -1 up to a whole
   // K-tile (at least one), which is what the GEMM's row map expects
   const int64_t keep_ld = round_up(N, kLdAlign) + kLdAlign;
@@ -681,6 +711,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // crossing lists of all sets in one buffer (they become the constraint nodes' index lists)
   BufRef idx_buf;
   NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &idx_buf));
+  // image sets (they carry windows): a convolution is likely to follow, whose stamp pass looks up the column of a
+  // pixel; the kernels that settle the crossing list's order leave that inverse behind
+  const bool want_inv = in[0]->box != nullptr && given == nullptr;
+  BufRef inv_buf;
+  if (want_inv) NNV_TRY(ctx->alloc(sizeof(int32_t) * ld * count, &inv_buf));
   std::vector<ReluDesc> descs(count);
   for (int64_t i = 0; i < count; ++i) {
     ReluDesc& d = descs[i];
@@ -699,11 +734,14 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     d.plb_in = in[i]->plb;
     d.pub_in = in[i]->pub;
     d.cls = cls_buf->as<int32_t>() + ld * i;
+    d.col_of = inv_buf ? inv_buf->as<int32_t>() + ld * i : nullptr;
+    d.keep_bits = lazy_rows ? cls_buf->as<uint32_t>() + ld * count + bit_words * i : nullptr;
     d.cross_idx = idx_buf->as<int32_t>() + ld * i;
     d.asc_idx = sorted ? asc_buf->as<int32_t>() + ld * i : nullptr;
     d.key = sorted ? key_buf->as<double>() + ld * i : nullptr;
     d.counts = cnt_buf->as<int32_t>() + 2 * i;
-    d.blk_counts = blk_buf ? blk_buf->as<int32_t>() + 3 * nblk * i : nullptr;
+    d.blk_counts = blk_buf ? blk_buf->as<int32_t>() + blk_stride * i : nullptr;
+    d.blk_gran = rc.gran > 0 ? rc.gran : 1024;
     d.keep_idx = keep_buf->as<int32_t>() + keep_ld * i;
     d.mailbox = nullptr;
     d.ld = ld;
@@ -747,8 +785,10 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     NNV_TRY(ctx->kernel_timer_end(tk, 6, cls_bytes));
   } else {
     const dim3 grid((unsigned)ceil_div(N, 1024), 1, (unsigned)count);
-    NNV_LAUNCH(ctx, tk, relu_count_kernel, grid, dim3(1024), 0, table, descs[0]);
-    NNV_TRY(ctx->kernel_timer_end(tk, 6, 0.5 * cls_bytes));
+    if (rc.gran == 0) {
+      NNV_LAUNCH(ctx, tk, relu_count_kernel, grid, dim3(1024), 0, table, descs[0]);
+      NNV_TRY(ctx->kernel_timer_end(tk, 6, 0.5 * cls_bytes));
+    }
     NNV_LAUNCH(ctx, tk, relu_compact_kernel, grid, dim3(1024), 0, table, descs[0]);
     NNV_TRY(ctx->kernel_timer_end(tk, 6, 0.5 * cls_bytes));
     if (early_rank)
@@ -769,6 +809,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->rows_pending = true;
       o->cls_buf = cls_buf;
       o->cls = cls_buf->as<int32_t>() + ld * i;
+      o->keep_bits = cls_buf->as<uint32_t>() + ld * count + bit_words * i;
       // ... and what is known about where its columns came from (and whether they are in memory yet)
       // holds for the rows that are kept
       o->cs = in[i]->cs;
@@ -955,6 +996,10 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->oh_plb_zero = true;
       o->oh_idx_buf = idx_buf;
       o->oh_idx = idx_buf->as<int32_t>() + ld * i;
+      if (inv_buf) {
+        o->oh_inv_buf = inv_buf;
+        o->oh_inv = inv_buf->as<int32_t>() + ld * i;
+      }
       if (!eager_tail) o->vcols = in[i]->n + 1;  // ... and exist only as that list
     }
     // rows of the leading columns that were not reset

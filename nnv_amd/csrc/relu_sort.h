@@ -23,10 +23,13 @@ struct ReluDesc {
   const double* given_key;  // order kOrderGiven: the key of every row is handed in (callers with an explicit list)
   int32_t* counts;     // [0] = m (crossing), [1] = inactive
   int32_t* keep_idx;   // rows left untouched (active neurons), ascending, then -1 up to a multiple of 16
-  int32_t* blk_counts; // multi-block classification: per 1024-row block {crossing, inactive, kept}
+  int32_t* blk_counts; // multi-block classification: {crossing, inactive, kept} per block of blk_gran rows (1024, or the
+                       // 64 / 128 rows of a block of the kernel that finished the range estimate and counted as it went)
+  int32_t* col_of;     // per row: the crossing neuron's place in new-predicate order, -1 for the other rows; or null
+  uint32_t* keep_bits; // one bit per row, 1 = kept (word w: rows 32w .. 32w+31), for whole 1024-row blocks; or null
   int32_t* mailbox;    // host-pinned {m, inactive, seq}; null = counts are fetched by a copy instead
   int32_t mailbox_seq;
-  int32_t pad2_;
+  int32_t blk_gran;
   double* lbub;        // lb then ub (offset ld_lbub) of the crossing neurons, new-predicate order
   int64_t ld;
   int64_t ld_lbub;
