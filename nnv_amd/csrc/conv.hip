@@ -267,28 +267,57 @@ __global__ void conv_weights_kmajor_kernel(const double* __restrict__ W, double*
   Wk[idx] = co < Cout ? W[k + (int64_t)co * Kp] : 0.0;
 }
 
+struct ConvFastArgs {
+  const double* in;
+  int64_t ldin;
+  double* out;
+  int64_t ldout;
+  const double* Wk;
+  int coutp;
+  const double* bias;
+  ConvGeom g;
+  int64_t total_rows;
+  int tiles_c;
+  const FastTap* taps;
+  const uint32_t* keep;
+  int keep_words;
+  ConvRows cr;
+};
+
+// LDS of a block of the kernel below: the weight tiles [2][k][channel] first (their transfers want 1 KiB alignment),
+// then the position tiles [2][k][position]; the row mask (MASK only) sits in the dynamic part behind them.
+constexpr size_t conv_fast_lds_bytes(int tc) { return sizeof(double) * 2 * kKt * (128 + (size_t)tc); }
+
 template <int TC, int WR, int WC, bool MASK, bool COMPACT>
-__global__ __launch_bounds__(512) void conv2d_fast_kernel(const double* __restrict__ in, int64_t ldin, double* __restrict__ out,
-                                                          int64_t ldout, const double* __restrict__ Wk, int coutp,
-                                                          const double* __restrict__ bias, ConvGeom g, int64_t total_rows,
-                                                          int tiles_c, const FastTap* __restrict__ taps,
-                                                          const uint32_t* __restrict__ keep, int keep_words, ConvRows cr) {
+__device__ __forceinline__ void conv2d_fast_block(const ConvFastArgs& a, int64_t bid, double* __restrict__ lds, uint32_t* keep_s) {
   constexpr int TP = 128, NT = 512;
   static_assert(WR * WC == 8, "eight waves");
   constexpr int FM = TP / WR / 16;
   constexpr int FN = TC / WC / 16;
   constexpr int kWLoads = kKt * TC / 128;  // 1 KiB wave transfers per K-tile of weights
   constexpr int kRowsPerLoad = 128 / TC;   // rows of Wk per transfer
-  __shared__ double Ps[2][kKt * TP];                                      // [k][position]
-  __shared__ __attribute__((aligned(1024))) double Wts[2][kKt * TC];     // [k][channel]
-  extern __shared__ uint32_t keep_s[];                                    // row mask (MASK only)
+  double(*Wts)[kKt * TC] = reinterpret_cast<double(*)[kKt * TC]>(lds);                // [k][channel]
+  double(*Ps)[kKt * TP] = reinterpret_cast<double(*)[kKt * TP]>(lds + 2 * kKt * TC);  // [k][position]
+  const double* __restrict__ in = a.in;
+  const int64_t ldin = a.ldin;
+  double* __restrict__ out = a.out;
+  const int64_t ldout = a.ldout;
+  const double* __restrict__ Wk = a.Wk;
+  const int coutp = a.coutp;
+  const double* __restrict__ bias = a.bias;
+  const ConvGeom& g = a.g;
+  const int64_t total_rows = a.total_rows;
+  const int tiles_c = a.tiles_c;
+  const FastTap* __restrict__ taps = a.taps;
+  const uint32_t* __restrict__ keep = a.keep;
+  const int keep_words = a.keep_words;
+  const ConvRows& cr = a.cr;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wr = wave % WR;
   const int wc = wave / WR;
-  const int64_t bid = blockIdx.x;
   const int c0 = (int)(bid % tiles_c) * TC;
   const int64_t R0 = (bid / tiles_c) * TP;
 
@@ -412,6 +441,13 @@ __global__ __launch_bounds__(512) void conv2d_fast_kernel(const double* __restri
     if (kt + 1 < nk) step(kt + 1, std::integral_constant<int, 1>());
   }
   conv_store_tile<TP, TC, WR, WC, FM, FN, COMPACT>(acc, out, ldout, bias, g, total_rows, R0, c0, wr, wc, lane, cr);
+}
+
+template <int TC, int WR, int WC, bool MASK, bool COMPACT>
+__global__ __launch_bounds__(512) void conv2d_fast_kernel(ConvFastArgs a) {
+  __shared__ __attribute__((aligned(1024))) double lds[2 * kKt * (128 + TC)];
+  extern __shared__ uint32_t keep_s[];  // row mask (MASK only)
+  conv2d_fast_block<TC, WR, WC, MASK, COMPACT>(a, blockIdx.x, lds, keep_s);
 }
 
 // Windows of the output columns of a convolution (see launch_conv_boxes in internal.h).
@@ -600,6 +636,128 @@ __global__ __launch_bounds__(256) void keep_bits_kernel(const int32_t* __restric
   if ((lane & 31) == 0 && w < words) bits[w] = (uint32_t)(b >> lane);
 }
 
+// ---- the stamps by output row (undilated filters) ---------------------------------------------------
+// Row r = (ho, wo, co) of the output meets the stamps of the pixels under its filter window, one per tap: for
+// tap k = (fh, fw, ci) the pixel (ho*sh - pt + fh, wo*sw - pl + fw, ci), whose unit-vector column t (pixel_col,
+// -1: none) gets out(r, t) = 0 + W(k, co) * scale.  One thread per row writes those elements - exactly the
+// non-zero candidates, i.e. the rows inside every column's window - and adds up the row's four range sums tap
+// by tap.  Everything else in the columns is zero and is written by the caller (or left for later).
+__global__ void stamp_pixel_columns_kernel(const int32_t* __restrict__ idx, int m, int32_t* __restrict__ pixel_col) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t < m) pixel_col[idx[t]] = t;
+}
+
+// S lanes share a row, lane s taking the taps k = s, s + S, ...; their sums are combined by a butterfly (a fixed
+// order).  S = 1 for filters with few taps, 16 otherwise (a row's taps are then walked by 16 lanes at once).
+// A block first decodes the taps once into LDS (filter position and the tap's offset from the pixel under the
+// filter's corner), so that the walk has no division in it, and looks up four taps' pixels before it handles them.
+constexpr int kStampTapTable = kMaxTaps;  // taps per output (FH * FW * Cin): no layer has more
+// Block `blk` of NT threads; taps: LDS for g.K entries.
+template <int S, int NT>
+__device__ __forceinline__ void conv_stamp_rows_block(int64_t blk, int2* taps, const StampSet& d, const ConvGeom& g,
+                                                      const double* __restrict__ Wt, const int32_t* __restrict__ pixel_col,
+                                                      int64_t ldout) {
+  for (int k = threadIdx.x; k < g.K; k += NT) {
+    const int fh = k % g.FH;
+    const int q = k / g.FH;
+    const int fw = q % g.FW;
+    const int ci = q / g.FW;
+    taps[k] = make_int2(fh | (fw << 16), fh + g.H * (fw + g.W * ci));  // x: fh | fw << 16, y: fh + H * (fw + W * ci)
+  }
+  __syncthreads();
+  const int64_t gt = blk * (int64_t)NT + threadIdx.x;
+  const int64_t r = gt / S;
+  const int s = (int)(gt % S);
+  const bool row = r < ldout;
+  const int64_t Nout = (int64_t)g.P * g.Cout;
+  double x1 = 0.0, x2 = 0.0, y1 = 0.0, y2 = 0.0;
+  if (row && r < Nout) {
+    const int co = (int)(r / g.P);
+    const int p = (int)(r - (int64_t)co * g.P);
+    const int wo = p / g.Ho, ho = p - wo * g.Ho;
+    const int hb = ho * g.sh - g.pt, wb = wo * g.sw - g.pl;
+    const int pbase = hb + g.H * wb;  // the pixel under the filter's corner (may lie outside the image)
+    const double* wcol = Wt + (int64_t)co * g.Kp;
+    for (int k0 = s; k0 < g.K; k0 += 4 * S) {
+      int t[4], pix[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + u * S;
+        t[u] = -1;
+        pix[u] = 0;
+        if (k < g.K) {
+          const int2 tp = taps[k];
+          const int h = hb + (tp.x & 0xffff), w = wb + (tp.x >> 16);
+          if ((unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W) {
+            pix[u] = pbase + tp.y;
+            t[u] = pixel_col[pix[u]];
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (t[u] < 0) continue;
+        const int k = k0 + u * S;
+        const double sc = d.scale != nullptr ? d.scale[pix[u]] : 1.0;
+        const double v = __dadd_rn(0.0, __dmul_rn(wcol[k], sc));
+        d.out[r + (int64_t)t[u] * ldout] = v;
+        const double pl = d.plb[t[u]], pu = d.pub[t[u]];
+        const double vp = fmax(v, 0.0), vn = fmin(v, 0.0);
+        x1 = fma(vp, pl, x1);  // xmin1
+        x2 = fma(vn, pu, x2);  // xmin2
+        y1 = fma(vp, pu, y1);  // xmax1
+        y2 = fma(vn, pl, y2);  // xmax2
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 1; off < S; off <<= 1) {
+    x1 += __shfl_xor(x1, off);
+    x2 += __shfl_xor(x2, off);
+    y1 += __shfl_xor(y1, off);
+    y2 += __shfl_xor(y2, off);
+  }
+  if (row && s == 0) {
+    d.part[r] = x1;
+    d.part[ldout + r] = x2;
+    d.part[2 * ldout + r] = y1;
+    d.part[3 * ldout + r] = y2;
+  }
+}
+
+template <int S>
+__global__ __launch_bounds__(256) void conv_stamp_rows_kernel(StampSet d, ConvGeom g, const double* __restrict__ Wt,
+                                                              const int32_t* __restrict__ pixel_col, int64_t ldout) {
+  __shared__ int2 taps[kStampTapTable];
+  conv_stamp_rows_block<S, 256>(blockIdx.x, taps, d, g, Wt, pixel_col, ldout);
+}
+
+// The dense images' convolution and the stamps of the unit-vector columns of the same layer in one launch: the two
+// write different columns of the output and read nothing of each other, the first is bound by the matrix pipe and the
+// second by scattered stores, so their blocks are dealt to the chip in turn (every stride-th block of the grid is a
+// stamp block, until there are no more) and run side by side on a compute unit.
+struct ConvStampArgs {
+  StampSet d;
+  const double* Wt;
+  const int32_t* pixel_col;
+  int32_t blocks;  // stamp blocks in the grid
+  int32_t stride;  // grid position p is stamp block (p + 1) / stride - 1 where (p + 1) % stride == 0 (and that is < blocks)
+};
+
+template <int TC, int WR, int WC, bool MASK, bool COMPACT, int S>
+__global__ __launch_bounds__(512) void conv2d_fast_stamps_kernel(ConvFastArgs a, ConvStampArgs st) {
+  static_assert(sizeof(int2) * kStampTapTable <= conv_fast_lds_bytes(TC), "the stamp blocks' tap table fits the tiles' LDS");
+  __shared__ __attribute__((aligned(1024))) double lds[2 * kKt * (128 + TC)];
+  extern __shared__ uint32_t keep_s[];  // row mask (MASK only)
+  const int p = blockIdx.x;
+  const int k = (p + 1) / st.stride;
+  if ((p + 1) % st.stride == 0 && k <= st.blocks) {
+    conv_stamp_rows_block<S, 512>(k - 1, reinterpret_cast<int2*>(lds), st.d, a.g, st.Wt, st.pixel_col, a.ldout);
+    return;
+  }
+  conv2d_fast_block<TC, WR, WC, MASK, COMPACT>(a, p - min(st.blocks, p / st.stride), lds, keep_s);
+}
+
 // LDS of the convolution kernel beside its tap table and row mask: the two double-buffered operand tiles
 template <int TP, int TC>
 constexpr size_t conv_static_lds() {
@@ -686,23 +844,56 @@ static int conv_fast_taps(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGe
   return NNVHIP_OK;
 }
 
+// stamp != null (a set's unit-vector columns, pixel_col and part filled in, filters undilated): their stamps go into
+// the same launch.
 template <int TC, int WR, int WC>
 static int launch_conv_fast(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const ConvGeom& g, const double* in, int64_t ldin, double* out,
-                            int64_t ldout, int64_t ncols, const uint32_t* keep, int keep_words, const ConvRows& cr) {
+                            int64_t ldout, int64_t ncols, const uint32_t* keep, int keep_words, const ConvRows& cr,
+                            const StampSet* stamp) {
   const bool compact = cr.box != nullptr;
   const int64_t total_rows = compact ? (int64_t)g.P + (ncols - 1) * cr.area : (int64_t)g.P * ncols;
   const int64_t tiles_c = ceil_div(g.Cout, TC);
   const int64_t blocks = ceil_div(total_rows, 128) * tiles_c;
-  if (blocks >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
   const size_t dyn = keep ? sizeof(uint32_t) * (size_t)keep_words : 0;
   if (conv_fast_static_lds(TC) + dyn > kConvLdsLimit) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: row mask too large for the convolution kernel");
-  const FastTap* taps = nullptr;
-  NNV_TRY(conv_fast_taps(ctx, cv, g, &taps));
-  const double* bias = cv->bias ? cv->bias->as<double>() : nullptr;
+  ConvFastArgs a{};
+  NNV_TRY(conv_fast_taps(ctx, cv, g, &a.taps));
+  a.in = in;
+  a.ldin = ldin;
+  a.out = out;
+  a.ldout = ldout;
+  a.Wk = cv->Wk->as<double>();
+  a.coutp = (int)cv->coutp;
+  a.bias = cv->bias ? cv->bias->as<double>() : nullptr;
+  a.g = g;
+  a.total_rows = total_rows;
+  a.tiles_c = (int)tiles_c;
+  a.keep = keep;
+  a.keep_words = keep_words;
+  a.cr = cr;
+  const bool wide_stamps = g.K > 32;  // lanes per output row of the stamp pass: 16, else 1
+  ConvStampArgs sa{};
+  if (stamp != nullptr) {
+    sa.d = *stamp;
+    sa.Wt = cv->W->as<double>();
+    sa.pixel_col = stamp->pixel_col;
+    sa.blocks = (int32_t)ceil_div(ldout * (wide_stamps ? 16 : 1), 512);
+    sa.stride = (int32_t)std::max<int64_t>(1, (blocks + sa.blocks) / sa.blocks);
+  }
+  const int64_t grid = blocks + sa.blocks;
+  if (grid >= (int64_t(1) << 31)) NNV_FAIL(NNVHIP_ERR_SHAPE, "convolution too large for one launch");
   NNV_TRY(ctx->kernel_timer_begin(ctx->kernel_timing));
-#define NNV_CONV_FAST(MASK, COMPACT)                                                                                              \
-  NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, MASK, COMPACT>), dim3((unsigned)blocks), dim3(512), dyn, in, \
-             ldin, out, ldout, cv->Wk->as<double>(), (int)cv->coutp, bias, g, total_rows, (int)tiles_c, taps, keep, keep_words, cr)
+#define NNV_CONV_FAST(MASK, COMPACT)                                                                                                    \
+  do {                                                                                                                                  \
+    if (stamp == nullptr)                                                                                                               \
+      NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, MASK, COMPACT>), dim3((unsigned)grid), dim3(512), dyn, a);    \
+    else if (wide_stamps)                                                                                                               \
+      NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_stamps_kernel<TC, WR, WC, MASK, COMPACT, 16>), dim3((unsigned)grid), dim3(512), \
+                 dyn, a, sa);                                                                                                           \
+    else                                                                                                                                \
+      NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_stamps_kernel<TC, WR, WC, MASK, COMPACT, 1>), dim3((unsigned)grid), dim3(512),  \
+                 dyn, a, sa);                                                                                                           \
+  } while (0)
   if (keep && compact)
     NNV_CONV_FAST(true, true);
   else if (keep)
@@ -751,7 +942,8 @@ bool conv2d_in_windows(const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
                   const int32_t* pending_cls, const ColBox* out_box, int eh, int ew, const ColBox* in_box, bool leave_outside,
-                  const uint32_t* pending_bits) {
+                  const uint32_t* pending_bits, const ConvStampSet* stamp, bool* stamped) {
+  if (stamped != nullptr) *stamped = false;
   if (cv->Kp > kMaxTaps) NNV_FAIL(NNVHIP_ERR_SHAPE, "filters with more than %d taps (FH*FW*Cin) are not supported", kMaxTaps);
   if ((cv->FH - 1) * cv->dil[0] > 0xffff || (cv->FW - 1) * cv->dil[1] > 0xffff)
     NNV_FAIL(NNVHIP_ERR_SHAPE, "dilated filter extent too large");
@@ -789,12 +981,25 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, int64_t H, int64_t W
   if (cr.box != nullptr && !leave_outside)  // everything outside the windows
     NNV_HIP_TRY(hipMemsetAsync(out + ldout, 0, sizeof(double) * (size_t)ldout * (size_t)(ncols - 1), ctx->stream));
   if (cr.box != nullptr || conv_fast_ok(cv, g, ldin)) {
+    // the stamps of the set's unit-vector columns ride along where they are made row by row and come with their
+    // pixel table and a place for their range sums
+    static_assert(sizeof(ConvStampSet) == sizeof(StampSet), "same layout");
+    StampSet one;
+    const StampSet* merge = nullptr;
+    if (stamp != nullptr && stamped != nullptr && stamp->m > 0 && stamp->pixel_col != nullptr && stamp->part != nullptr &&
+        cv->dil[0] == 1 && cv->dil[1] == 1 && g.K <= kStampTapTable) {
+      memcpy(&one, stamp, sizeof one);
+      merge = &one;
+      if (!one.win_only)  // whole columns: the zeros first
+        NNV_HIP_TRY(hipMemsetAsync(one.out, 0, sizeof(double) * (size_t)ldout * (size_t)one.m, ctx->stream));
+      *stamped = true;
+    }
     if (cv->Cout <= 16)
-      st = launch_conv_fast<16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr);
+      st = launch_conv_fast<16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr, merge);
     else if (cv->Cout <= 32)
-      st = launch_conv_fast<32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr);
+      st = launch_conv_fast<32, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr, merge);
     else
-      st = launch_conv_fast<64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr);
+      st = launch_conv_fast<64, 4, 2>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words, cr, merge);
   } else if (cv->Cout <= 16) {
     st = launch_conv_cfg<128, 16, 8, 1>(ctx, cv, g, in, ldin, out, ldout, ncols, keep, keep_words);
   } else if (cv->Cout <= 32) {
@@ -829,94 +1034,6 @@ static void fill_geom(ConvGeom& g, const nnvhip_conv2d* cv, int64_t H, int64_t W
   g.Kp = (int)cv->Kp;
   g.P = (int)(Ho * Wo);
   g.HW = (int)(H * W);
-}
-
-// ---- the stamps by output row (undilated filters) ---------------------------------------------------
-// Row r = (ho, wo, co) of the output meets the stamps of the pixels under its filter window, one per tap: for
-// tap k = (fh, fw, ci) the pixel (ho*sh - pt + fh, wo*sw - pl + fw, ci), whose unit-vector column t (pixel_col,
-// -1: none) gets out(r, t) = 0 + W(k, co) * scale.  One thread per row writes those elements - exactly the
-// non-zero candidates, i.e. the rows inside every column's window - and adds up the row's four range sums tap
-// by tap.  Everything else in the columns is zero and is written by the caller (or left for later).
-__global__ void stamp_pixel_columns_kernel(const int32_t* __restrict__ idx, int m, int32_t* __restrict__ pixel_col) {
-  const int t = blockIdx.x * 256 + threadIdx.x;
-  if (t < m) pixel_col[idx[t]] = t;
-}
-
-// S lanes share a row, lane s taking the taps k = s, s + S, ...; their sums are combined by a butterfly (a fixed
-// order).  S = 1 for filters with few taps, 16 otherwise (a row's taps are then walked by 16 lanes at once).
-// A block first decodes the taps once into LDS (filter position and the tap's offset from the pixel under the
-// filter's corner), so that the walk has no division in it, and looks up four taps' pixels before it handles them.
-constexpr int kStampTapTable = kMaxTaps;  // taps per output (FH * FW * Cin): no layer has more
-template <int S>
-__global__ __launch_bounds__(256) void conv_stamp_rows_kernel(StampSet d, ConvGeom g, const double* __restrict__ Wt,
-                                                              const int32_t* __restrict__ pixel_col, int64_t ldout) {
-  __shared__ int2 taps[kStampTapTable];  // x: fh | fw << 16, y: fh + H * (fw + W * ci)
-  for (int k = threadIdx.x; k < g.K; k += 256) {
-    const int fh = k % g.FH;
-    const int q = k / g.FH;
-    const int fw = q % g.FW;
-    const int ci = q / g.FW;
-    taps[k] = make_int2(fh | (fw << 16), fh + g.H * (fw + g.W * ci));
-  }
-  __syncthreads();
-  const int64_t gt = blockIdx.x * (int64_t)256 + threadIdx.x;
-  const int64_t r = gt / S;
-  const int s = (int)(gt % S);
-  const bool row = r < ldout;
-  const int64_t Nout = (int64_t)g.P * g.Cout;
-  double x1 = 0.0, x2 = 0.0, y1 = 0.0, y2 = 0.0;
-  if (row && r < Nout) {
-    const int co = (int)(r / g.P);
-    const int p = (int)(r - (int64_t)co * g.P);
-    const int wo = p / g.Ho, ho = p - wo * g.Ho;
-    const int hb = ho * g.sh - g.pt, wb = wo * g.sw - g.pl;
-    const int pbase = hb + g.H * wb;  // the pixel under the filter's corner (may lie outside the image)
-    const double* wcol = Wt + (int64_t)co * g.Kp;
-    for (int k0 = s; k0 < g.K; k0 += 4 * S) {
-      int t[4], pix[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int k = k0 + u * S;
-        t[u] = -1;
-        pix[u] = 0;
-        if (k < g.K) {
-          const int2 tp = taps[k];
-          const int h = hb + (tp.x & 0xffff), w = wb + (tp.x >> 16);
-          if ((unsigned)h < (unsigned)g.H && (unsigned)w < (unsigned)g.W) {
-            pix[u] = pbase + tp.y;
-            t[u] = pixel_col[pix[u]];
-          }
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (t[u] < 0) continue;
-        const int k = k0 + u * S;
-        const double sc = d.scale != nullptr ? d.scale[pix[u]] : 1.0;
-        const double v = __dadd_rn(0.0, __dmul_rn(wcol[k], sc));
-        d.out[r + (int64_t)t[u] * ldout] = v;
-        const double pl = d.plb[t[u]], pu = d.pub[t[u]];
-        const double vp = fmax(v, 0.0), vn = fmin(v, 0.0);
-        x1 = fma(vp, pl, x1);  // xmin1
-        x2 = fma(vn, pu, x2);  // xmin2
-        y1 = fma(vp, pu, y1);  // xmax1
-        y2 = fma(vn, pl, y2);  // xmax2
-      }
-    }
-  }
-#pragma unroll
-  for (int off = 1; off < S; off <<= 1) {
-    x1 += __shfl_xor(x1, off);
-    x2 += __shfl_xor(x2, off);
-    y1 += __shfl_xor(y1, off);
-    y2 += __shfl_xor(y2, off);
-  }
-  if (row && s == 0) {
-    d.part[r] = x1;
-    d.part[ldout + r] = x2;
-    d.part[2 * ldout + r] = y1;
-    d.part[3 * ldout + r] = y2;
-  }
 }
 
 static bool conv_stamps_by_row(const nnvhip_conv2d* cv) { return cv->dil[0] == 1 && cv->dil[1] == 1; }

@@ -688,6 +688,18 @@ int launch_bias_columns(nnvhip_ctx* ctx, double* const* centre_cols_dev, int64_t
                         int64_t Mp);
 
 // conv.hip
+// Convolution of the one-hot generator columns of every set ("stamps" of the filter), conv.hip.
+struct ConvStampSet {
+  const int32_t* idx;   // input row of every one-hot column
+  const double* scale;  // by input row, or null
+  double* out;          // first of these columns in the output set
+  const double* plb;    // predicate bounds of these columns
+  const double* pub;
+  double* part;         // this set's [chunks][4][ldout] range sums
+  int32_t m;
+  int32_t win_only;     // 1: write the rows inside each column's window only
+  const int32_t* pixel_col;  // input row -> its one-hot column (index into idx), -1: none; or null (made by the launch)
+};
 int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                   const double* in, int64_t ldin, double* out, int64_t ldout, int64_t ncols,
                   const int32_t* pending_cls /* per input row, or null: rows whose class is not kKeep read as zero */,
@@ -698,7 +710,10 @@ int launch_conv2d(nnvhip_ctx* ctx, const nnvhip_conv2d* conv, int64_t H, int64_t
                                                     may be in memory inside its windows only); needs conv2d_in_windows */,
                   bool leave_outside = false /* do not write the zeros outside the output windows */,
                   const uint32_t* pending_bits = nullptr /* with pending_cls: the same as one bit per row (1 = kept), where
-                                                            the step that classified the rows left them */);
+                                                            the step that classified the rows left them */,
+                  const ConvStampSet* stamp = nullptr /* the set's unit-vector columns: their stamps go into the same
+                                                                 launch where that is possible ... */,
+                  bool* stamped = nullptr /* ... which this reports (launch_conv_stamps is then not needed for the set) */);
 int launch_zero_pad_rows(nnvhip_ctx* ctx, double* V, int64_t ld, int64_t N, int64_t ncols);  // rows [N, ld) of ncols columns := 0
 // whether launch_conv2d computes the generator images of such a call inside their windows only
 bool conv2d_in_windows(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin, int64_t ncols,
@@ -713,18 +728,6 @@ int64_t conv_box_extent(const nnvhip_conv2d* conv, int dim, int64_t e, int64_t o
 bool conv2d_can_mask(const nnvhip_conv2d* conv, int64_t H, int64_t W, int64_t Ho, int64_t Wo, int64_t ldin);
 int conv2d_prepare_weights(nnvhip_ctx* ctx, nnvhip_conv2d* conv);  // builds conv->Wk from conv->W (at creation)
 
-// Convolution of the one-hot generator columns of every set ("stamps" of the filter), conv.hip.
-struct ConvStampSet {
-  const int32_t* idx;   // input row of every one-hot column
-  const double* scale;  // by input row, or null
-  double* out;          // first of these columns in the output set
-  const double* plb;    // predicate bounds of these columns
-  const double* pub;
-  double* part;         // this set's [chunks][4][ldout] range sums
-  int32_t m;
-  int32_t win_only;     // 1: write the rows inside each column's window only
-  const int32_t* pixel_col;  // input row -> its one-hot column (index into idx), -1: none; or null (made by the launch)
-};
 // Whether the stamp launch of this layer looks columns up by pixel (ConvStampSet::pixel_col), and that table for one
 // set: inv[idx[t]] = t, -1 elsewhere (n_in entries, allocated here).
 bool conv_stamps_by_pixel(const nnvhip_conv2d* conv);

@@ -85,6 +85,15 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
     if (st == NNVHIP_OK && !full.empty()) st = ensure_dense_batch(c, (int64_t)full.size(), full.data());
     if (st == NNVHIP_OK && !prefix.empty()) st = ensure_dense_batch(c, (int64_t)prefix.size(), prefix.data(), false);
   }
+  // range sums of the stamped columns, left on the output handles: one buffer for the call
+  for (int64_t i = 0; i < count; ++i) {
+    any_stamps = any_stamps || plan[i].m > 0;
+    max_m = std::max<int64_t>(max_m, plan[i].m);
+  }
+  const int64_t sch = any_stamps && st == NNVHIP_OK ? conv_stamp_chunks(cv, outs[0]->ld, count, max_m) : 0;
+  BufRef sums;
+  if (sch > 0) st = c->alloc(sizeof(double) * 4 * outs[0]->ld * sch * count, &sums);
+  std::vector<char> stamped((size_t)count, 0);
   for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i) {
     const Plan& pl = plan[i];
     nnvhip_star* o = outs[i];
@@ -129,7 +138,7 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
     stamps[i].out = o->V + pl.dense * o->ld;
     stamps[i].plb = o->plb + (pl.dense - 1);
     stamps[i].pub = o->pub + (pl.dense - 1);
-    stamps[i].part = nullptr;
+    stamps[i].part = sums ? sums->as<double>() + 4 * outs[0]->ld * sch * i : nullptr;
     stamps[i].m = (int32_t)pl.m;
     if (pl.m > 0 && in[i]->oh_inv == nullptr && conv_stamps_by_pixel(cv)) {
       // (kept on the input: its columns do not change, and an input set is usually mapped again)
@@ -139,24 +148,26 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
     }
     stamps[i].pixel_col = in[i]->oh_inv;
     stamps[i].win_only = (lazy && pl.m > 0) ? 1 : 0;
-    any_stamps = any_stamps || pl.m > 0;
-    max_m = std::max<int64_t>(max_m, pl.m);
+    bool done = false;
     st = launch_conv2d(c, cv, H, W, Ho, Wo, in[i]->V, in[i]->ld, o->V, o->ld, pl.dense,
                        in[i]->rows_pending ? in[i]->cls : nullptr, pl.compact ? ob : nullptr, pl.dense_eh, pl.dense_ew,
-                       pl.compact ? in[i]->box : nullptr, pl.compact && lazy, in[i]->rows_pending ? in[i]->keep_bits : nullptr);
+                       pl.compact ? in[i]->box : nullptr, pl.compact && lazy, in[i]->rows_pending ? in[i]->keep_bits : nullptr,
+                       sch == 1 ? &stamps[i] : nullptr, &done);
+    stamped[(size_t)i] = done ? 1 : 0;
     // (launch_conv2d zeroes the padding rows of the columns it writes; the stamp kernel only writes them when
     // it writes whole columns)
     if (st == NNVHIP_OK && stamps[i].win_only && o->ld != Nout) st = launch_zero_pad_rows(c, stamps[i].out, o->ld, Nout, pl.m);
   }
   if (st == NNVHIP_OK && any_stamps) {
-    // the stamp pass also leaves the range sums of its columns on the output handles
-    const int64_t sch = conv_stamp_chunks(cv, outs[0]->ld, count, max_m);
-    BufRef sums;
-    st = c->alloc(sizeof(double) * 4 * outs[0]->ld * sch * count, &sums);
-    if (st == NNVHIP_OK) {
-      for (int64_t i = 0; i < count; ++i) stamps[i].part = sums->as<double>() + 4 * outs[0]->ld * sch * i;
-      st = launch_conv_stamps(c, cv, H, W, Ho, Wo, outs[0]->ld, count, stamps.data(), sch);
+    // the stamp pass also leaves the range sums of its columns on the output handles; sets whose stamps went into
+    // their convolution's launch are done
+    std::vector<ConvStampSet> rest = stamps;
+    bool any_left = false;
+    for (int64_t i = 0; i < count; ++i) {
+      if (stamped[(size_t)i]) rest[(size_t)i].m = 0;
+      any_left = any_left || rest[(size_t)i].m > 0;
     }
+    if (any_left) st = launch_conv_stamps(c, cv, H, W, Ho, Wo, outs[0]->ld, count, rest.data(), sch);
     for (int64_t i = 0; i < count && st == NNVHIP_OK; ++i)
       if (stamps[i].m > 0) {
         outs[i]->rng_buf = sums;
