@@ -57,11 +57,30 @@ int enter_ctx(nnvhip_ctx* ctx) {
   return NNVHIP_OK;
 }
 
+// Handles come from (and go back to) a list of released ones kept by the context: an array of a thousand sets makes
+// and lets go of a thousand handles per layer, on the host's critical path.
 nnvhip_star* new_star(nnvhip_ctx* ctx) {
-  nnvhip_star* s = new nnvhip_star();
+  nnvhip_star* s;
+  if (!ctx->free_stars.empty()) {
+    void* mem = ctx->free_stars.back();
+    ctx->free_stars.pop_back();
+    s = new (mem) nnvhip_star();
+  } else {
+    s = new (::operator new(sizeof(nnvhip_star))) nnvhip_star();
+  }
   s->ctx = ctx;
   ctx->live_handles++;
   return s;
+}
+
+void delete_star(nnvhip_star* s) {
+  nnvhip_ctx* c = s->ctx;
+  s->~nnvhip_star();
+  if (c->free_stars.size() < nnvhip_ctx::kMaxFreeStars)
+    c->free_stars.push_back(s);
+  else
+    ::operator delete(static_cast<void*>(s));
+  c->live_handles--;
 }
 
 }  // namespace nnvhip
@@ -254,6 +273,8 @@ int nnvhip_destroy(nnvhip_ctx* c) {
     NNV_FAIL(NNVHIP_ERR_ARG, "context still has %lld live handles", (long long)c->live_handles);
   NNV_TRY(nnvhip::enter_ctx(c));
   c->trim();
+  for (void* mem : c->free_stars) ::operator delete(mem);
+  c->free_stars.clear();
   if (c->pinned) (void)hipHostFree(c->pinned);
   if (c->mailbox) (void)hipHostFree((void*)c->mailbox);
   for (char* r : c->retired_rings) (void)hipHostFree(r);

@@ -271,6 +271,9 @@ struct nnvhip_ctx {
   // staging ring wrapped or grew, mailbox waits that went through the slow path
   int64_t n_device_mallocs = 0, n_staging_waits = 0;
   uint64_t visit_seq = 0;
+  // memory of released handles, reused by new_star (at most kMaxFreeStars of them are kept)
+  static constexpr size_t kMaxFreeStars = 32768;
+  std::vector<void*> free_stars;
   int64_t device_bytes = 0;  // memory of the device (the pool grows past a released array only below a share of it)
   // pinned staging ring for descriptor tables and small read-backs
   char* pinned = nullptr;
@@ -499,6 +502,7 @@ struct nnvhip_conv2d {
 namespace nnvhip {
 
 nnvhip_star* new_star(nnvhip_ctx* ctx);
+void delete_star(nnvhip_star* s);  // the last reference is gone
 
 // Shared set-up of the affine layers (ctx.hip): validates the handle array; allocates one output arena
 // with the sets back to back and creates output handles that share constraints and predicate bounds

@@ -351,9 +351,7 @@ int nnvhip_star_retain(nnvhip_star* s) {
 int nnvhip_star_release(nnvhip_star* s) {
   if (!s) return NNVHIP_OK;
   if (s->refs.fetch_sub(1) == 1) {
-    nnvhip_ctx* c = s->ctx;
-    delete s;
-    c->live_handles--;
+    delete_star(s);
   }
   return NNVHIP_OK;
 }
