@@ -49,7 +49,7 @@ MIN_WARM_SECONDS = 0.3
 GROUP_KERNELS = {
     "gemm_f64_kernel": ("gemm_f64_kernel",),
     "gemm_seg_kernel": ("gemm_seg_kernel",),
-    "conv2d_fast_kernel": ("conv2d_fast_kernel", "conv2d_f64_kernel"),
+    "conv2d_fast_kernel": ("conv2d_fast_kernel", "conv2d_fast_stamps_kernel", "conv2d_f64_kernel"),
     "gather_columns_kernel": ("gather_columns_kernel", "gather_skinny_kernel", "fc_rowsum_kernel", "conv_stamp_kernel", "conv_stamp_rows_kernel"),
     "ranges_partial_kernel": ("ranges_partial_kernel", "ranges_window_kernel"),
     "relu_classify_kernel": ("relu_classify_kernel", "relu_count_kernel", "relu_compact_kernel"),
@@ -328,7 +328,12 @@ def measure(k, args, ctx, exact_steps, extras):
         groups.append((gemm_ms, mfma_roofline("gemm_f64_kernel", gemm_work, gemm_flop if gemm_ms > seg_ms or not seg_launches else 0.0,
                                               gemm_ms, gemm_launches)))
     if conv_launches:
-        groups.append((conv_ms, mfma_roofline("conv2d_fast_kernel", conv_work, conv_flop, conv_ms, conv_launches)))
+        g = mfma_roofline("conv2d_fast_kernel", conv_work, conv_flop, conv_ms, conv_launches)
+        if not ctx.switch_is_on("eager_cols", "dense_affine"):
+            # conv2d_fast_stamps_kernel: a layer's launch also writes the filter stamps of its unit-vector columns (blocks
+            # dealt in between the tile blocks); the flop count is that of the tiles, the duration that of the whole launch
+            g["stamp_blocks_in_the_same_launch"] = True
+        groups.append((conv_ms, g))
     if rng_launches:
         groups.append((rng_ms, hbm_roofline("ranges_partial_kernel", rng_ms, rng_launches, rng_bytes)))
     if app_launches:
