@@ -791,3 +791,41 @@ def test_chains_of_convolutions_keep_generator_images_inside_their_windows(nnv, 
     cfg = {"name": "conv chain %dx%dx%d" % shape, "kind": "image", "image_shape": shape, "layers": layers,
            "lb": x - 0.05, "ub": x + 0.05}
     run_cfg(cfg, method)
+
+
+def test_an_input_image_set_is_mapped_again_and_again(nnv, oracle):
+    """The stamp pass of a convolution looks the column of a pixel up in a table; for a box ImageStar that table is
+    made by the first convolution that maps the set and kept on the set's handle.  The same input set through two
+    networks with different first layers, twice each: every reach must give the same sets as the first one, and
+    the first one the oracle's."""
+    rs = np.random.RandomState(4242)
+    H, W, C = 11, 9, 2
+    x = rs.rand(H, W, C)
+    lb, ub = x - 0.03, x + 0.03
+    lb[3, 4, 1] = ub[3, 4, 1] = x[3, 4, 1]          # a pixel without a generator
+    dev_in = nnv.ImageStar(lb, ub)
+    ora_in = oracle.image_star_from_bounds(lb, ub)
+
+    def net_layers(fh, fw, co, st):
+        c1 = {"type": "conv", "W": rs.randn(fh, fw, C, co) * np.sqrt(2.0 / (fh * fw * C)), "b": 0.1 * rs.randn(co),
+              "padding": [1, 1, 1, 1], "stride": [st, st], "dilation": [1, 1]}
+        h, w = oracle.conv2d_output_size(H, W, fh, fw, [1, 1, 1, 1], [st, st], [1, 1])
+        c2 = {"type": "conv", "W": rs.randn(3, 3, co, 5) * np.sqrt(2.0 / (9 * co)), "b": 0.1 * rs.randn(5),
+              "padding": [0, 0, 0, 0], "stride": [1, 1], "dilation": [1, 1]}
+        h2, w2 = oracle.conv2d_output_size(h, w, 3, 3, [0, 0, 0, 0], [1, 1], [1, 1])
+        return [c1, {"type": "relu"}, c2, {"type": "relu"}, {"type": "fc", "W": rs.randn(4, h2 * w2 * 5) / 10.0, "b": rs.randn(4)}]
+
+    opts = {"reachMethod": "relax-star-area", "relaxFactor": 1}
+    for spec in ((3, 3, 6, 1), (2, 3, 4, 2)):
+        layers = net_layers(*spec)
+        net = nnv.NN.from_config(layers, "same input, %dx%d filters" % spec[:2])
+        ora_out, _ = oracle.nn_reach(layers, ora_in, "relax-star-area", 1.0, keep=True)
+        first = None
+        for _ in range(3):
+            out = net.reach(dev_in, opts)
+            V = flat_V(out).copy()
+            if first is None:
+                first = V
+                assert_close(V, flat_V(ora_out), "output set of the first reach")
+            else:
+                assert np.array_equal(V, first)
