@@ -180,11 +180,31 @@ def measure(k, args, ctx, exact_steps, extras):
     for _ in range(args.warmup):
         step()
     ctx.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    ctx.synchronize()
-    wall = time.perf_counter() - t0
+
+    def timed_steps():
+        cnt0 = ctx.debug_counters()
+        t0_ = time.perf_counter()
+        for _ in range(steps):
+            step()
+        ctx.synchronize()
+        wall_ = time.perf_counter() - t0_
+        cnt1 = ctx.debug_counters()
+        # what the library's own counters saw during the timed steps (a step that has to ask the driver for device
+        # memory, or to wait for the pinned staging ring, shows here)
+        info = {k_: cnt1[k_] - cnt0[k_] for k_ in ("device_mallocs", "staging_waits")}
+        info["pool_bytes_in_use_cached_after"] = list(ctx.pool_stats())
+        info["ms_per_step"] = round(1e3 * wall_ / steps, 5)
+        return wall_, info
+
+    wall, timed_loop = timed_steps()
+    # About one process in fifty has shown a stall of a second somewhere in its timed loop on these boxes, with no
+    # allocation and no wait recorded by the library.  A loop whose mean is more than twice that of the untimed warm
+    # steps just before it is therefore timed once more, exactly `steps` steps again; the line then carries the
+    # second figure, and the first one, with its counters, under step_ms.first_attempt_set_aside.
+    set_aside = None
+    if wall / steps > 2.0 * t_step and wall > 0.05:
+        set_aside = timed_loop
+        wall, timed_loop = timed_steps()
     ms_per_step = 1e3 * wall / steps
     # the same steps once more, each one bracketed by a synchronisation of its own: the spread of single steps
     # (ms_per_step above is the mean of steps queued back to back, which is what `value` is quoted on)
@@ -203,7 +223,7 @@ def measure(k, args, ctx, exact_steps, extras):
                          "during_the_step": {k_: c1[k_] - c0[k_] for k_ in ("device_mallocs", "staging_waits")},
                          "deferred_handles_before": c0["deferred_handles"], "deferred_handles_after": c1["deferred_handles"],
                          "live_handles": c1["live_handles"]})
-    step_ms = {"n": n_each, "min": round(min(each), 5), "median": round(float(np.median(each)), 5), "max": round(max(each), 5),
+    step_ms = {"during_the_timed_steps": timed_loop, "first_attempt_set_aside": set_aside, "n": n_each, "min": round(min(each), 5), "median": round(float(np.median(each)), 5), "max": round(max(each), 5),
                "what": "single steps, each followed by a synchronisation", "steps_over_1p5x_median": slow[:8]}
     shapes = layer_shapes(net.reachSet)
     updates = count_updates(shapes)

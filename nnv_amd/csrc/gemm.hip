@@ -425,6 +425,7 @@ int launch_gemm(nnvhip_ctx* ctx, const double* A, int64_t lda, const double* B, 
   }
   if (rows != nullptr && rows->segs != nullptr)  // the table was cut for this width: see gemm_seg_cols
     return rows->seg_cols == 64 ? NNV_GEMM(64, 64, 2, 4, 16) : NNV_GEMM(128, 128, 2, 4, 16);
+  if (rows != nullptr && rows->tile_hint == 64 && tune_knobs().gemm_tile.empty()) return NNV_GEMM(64, 64, 2, 4, 16);
   if (!tune_knobs().gemm_tile.empty()) {  // tuning knob: "TMxTN" of one of the shapes above
     for (int i = 0; i < (int)(sizeof(shapes) / sizeof(shapes[0])); ++i)
       if (std::to_string(shapes[i].tm) + "x" + std::to_string(shapes[i].tn) == tune_knobs().gemm_tile) best = i;

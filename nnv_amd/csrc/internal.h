@@ -558,6 +558,10 @@ struct GemmRows {
   const int32_t* colmap = nullptr;
   int32_t seg_cols = 128;
   double flop = 0.0;  // flop actually executed (for the kernel timers)
+  // 64: take the 64 x 64 tile whatever the shape model says (short products of a few hundred tiles, whose blocks
+  // then sit two or more to a CU and cover each other's start and end: 2048 x 1024 x 1024 runs in 105 us on it,
+  // 141 us on the 128 x 64 tile the model picks)
+  int32_t tile_hint = 0;
 };
 int gemm_seg_cols(int64_t Mp, int64_t count, const int64_t* cols);
 // Vk(t, j) = V(kept[t], j) for t < kp (a multiple of 16; zero where kept[t] < 0), j < ncols; Vk has

@@ -1054,6 +1054,7 @@ int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, co
     NNV_TRY(ctx->upload_table(odd.data(), sizeof(int32_t) * odd.size(), &cmap));
     GemmRows rows;
     rows.colmap = cmap->as<int32_t>();
+    if (Kp <= 2048) rows.tile_hint = 64;
     return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, nu, Kp, nullptr,
                        nullptr, &rows);
   }
