@@ -871,13 +871,15 @@ static int launch_conv_fast(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const Conv
   a.keep = keep;
   a.keep_words = keep_words;
   a.cr = cr;
-  const bool wide_stamps = g.K > 32;  // lanes per output row of the stamp pass: 16, else 1
+  // lanes per output row of the stamp blocks: 8 for filters with many taps (beside the tile blocks that measured best:
+  // config 4 0.747 ms against 0.752 with 16 lanes, 0.756 with 4, 0.782 with 32), else 1
+  const bool wide_stamps = g.K > 32;
   ConvStampArgs sa{};
   if (stamp != nullptr) {
     sa.d = *stamp;
     sa.Wt = cv->W->as<double>();
     sa.pixel_col = stamp->pixel_col;
-    sa.blocks = (int32_t)ceil_div(ldout * (wide_stamps ? 16 : 1), 512);
+    sa.blocks = (int32_t)ceil_div(ldout * (wide_stamps ? 8 : 1), 512);
     sa.stride = (int32_t)std::max<int64_t>(1, (blocks + sa.blocks) / sa.blocks);
   }
   const int64_t grid = blocks + sa.blocks;
@@ -888,7 +890,7 @@ static int launch_conv_fast(nnvhip_ctx* ctx, const nnvhip_conv2d* cv, const Conv
     if (stamp == nullptr)                                                                                                               \
       NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_kernel<TC, WR, WC, MASK, COMPACT>), dim3((unsigned)grid), dim3(512), dyn, a);    \
     else if (wide_stamps)                                                                                                               \
-      NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_stamps_kernel<TC, WR, WC, MASK, COMPACT, 16>), dim3((unsigned)grid), dim3(512), \
+      NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_stamps_kernel<TC, WR, WC, MASK, COMPACT, 8>), dim3((unsigned)grid), dim3(512), \
                  dyn, a, sa);                                                                                                           \
     else                                                                                                                                \
       NNV_LAUNCH(ctx, ctx->kernel_timing, (conv2d_fast_stamps_kernel<TC, WR, WC, MASK, COMPACT, 1>), dim3((unsigned)grid), dim3(512),  \
