@@ -176,6 +176,10 @@ struct ColSource {
   int64_t from = 0;
   int64_t cols = 0;
   bool pending = false;  // the columns [from, from + cols) are not in memory yet
+  // Rows of the matrix have been reset (zeroed in memory) since the columns were gathered: the description then holds
+  // for the rows on the handle's own kept-row list only, and does not pass on to a set that lists its rows anew
+  // (a ReLU step on top may keep a row the earlier reset zeroed: one that crossed and now carries a unit vector).
+  bool rows_reset = false;
   int64_t zero_to = 0;   // > 1: the columns [1, zero_to) are +0 and not in memory yet
   // Generator images of a convolution's output that are in memory inside their windows only (win_box[j], an
   // image of win_H x win_W positions per channel): columns [win_from, win_to); the rows outside the windows,

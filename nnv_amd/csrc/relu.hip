@@ -622,6 +622,7 @@ int ensure_dense_batch(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* sets,
       s->cs.pending = false;
       s->cs.zero_to = 0;
       s->cs.win_from = s->cs.win_to = 0;
+      s->cs.rows_reset = true;
       if (need_tail) s->vcols = -1;
     }
     pend.swap(rest);
@@ -811,8 +812,9 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->cls = cls_buf->as<int32_t>() + ld * i;
       o->keep_bits = cls_buf->as<uint32_t>() + ld * count + bit_words * i;
       // ... and what is known about where its columns came from (and whether they are in memory yet)
-      // holds for the rows that are kept
-      o->cs = in[i]->cs;
+      // holds for the rows that are kept -- unless rows of the input's matrix were reset in memory after the gather
+      // (this step may keep such a row)
+      o->cs = in[i]->cs.rows_reset ? ColSource() : in[i]->cs;
     }
     {
       // resetting rows leaves every generator image inside its window (the columns the step appends come
@@ -977,10 +979,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->V = d.Vout;
       // where the input's columns were gathered from: still true of the rows this step keeps (a later packing of
       // kept rows reads the cache-resident weights instead of this matrix); everything is in memory
-      o->cs = in[i]->cs;
+      o->cs = in[i]->cs.rows_reset ? ColSource() : in[i]->cs;
       o->cs.pending = false;
       o->cs.zero_to = 0;
       o->cs.win_from = o->cs.win_to = 0;
+      o->cs.rows_reset = true;
     }
     o->pbuf = pred_buf;
     o->plb = d.plb_out;

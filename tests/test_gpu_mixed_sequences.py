@@ -268,3 +268,25 @@ def test_neighbouring_boxes_share_the_product_over_their_common_rows(nnv, oracle
     _, launches = _shared_product_launches(ctx, lambda: _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area"))
     if expect is not None and not ctx.switch_is_on("no_row_deltas", "dense_affine", "eager_tail"):
         assert (launches > 0) == expect, "spread %g: %d launches of the shared-product pass" % (spread, launches)
+
+
+@pytest.mark.parametrize("count,half_width", [(1, 0.02), (1, 3.0), (5, 0.3)])
+def test_a_relu_on_top_of_a_relu_lists_its_rows_anew(nnv, oracle, count, half_width):
+    """ReLU, ReLU, FC: the second step keeps the rows whose neurons crossed in the first (their range is now
+    [0, ub]), rows the first step's reset zeroed -- whatever is remembered about where the kept rows' columns came
+    from does not hold for them, and the FC layer behind must read them as they are in memory.  From narrow boxes
+    (few neurons cross) to wide ones (nearly all do), one set and an array, with a second pair further down."""
+    rs = np.random.RandomState(1700 + count)
+    n_in = 90
+    layers = [_fc(rs, 300, n_in, 2.0), {"type": "relu"}, {"type": "relu"}, _fc(rs, 150, 300, 2.0), {"type": "relu"},
+              {"type": "relu"}, {"type": "relu"}, _fc(rs, 7, 150)]
+    centre = rs.rand(n_in, count)
+    half = np.abs(rs.randn(n_in, count)) * half_width
+    lbs, ubs = centre - half, centre + half
+    if count == 1:
+        dev_in, ora_in = nnv.Star(lbs[:, 0], ubs[:, 0]), oracle.star_from_box(lbs[:, 0], ubs[:, 0])
+    else:
+        dev_in = nnv.Star.from_boxes(lbs, ubs)
+        ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
+    for method in ("relax-star-area", "relax-star-random"):
+        _compare(nnv, oracle, layers, dev_in, ora_in, method)

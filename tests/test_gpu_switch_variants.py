@@ -82,6 +82,11 @@ def test_neighbouring_boxes_share_the_product_over_their_common_rows(route, nnv,
     seqs.test_neighbouring_boxes_share_the_product_over_their_common_rows(nnv, oracle, spread, shapes, None)
 
 
+@pytest.mark.parametrize("count,half_width", [(1, 3.0), (5, 0.3)])
+def test_a_relu_on_top_of_a_relu_lists_its_rows_anew(route, nnv, oracle, count, half_width):
+    seqs.test_a_relu_on_top_of_a_relu_lists_its_rows_anew(nnv, oracle, count, half_width)
+
+
 def test_one_wide_set_through_the_tile_kernel(route, nnv, oracle):
     seqs.test_one_wide_set_through_the_tile_kernel(nnv, oracle, "relax-star-area")
 
