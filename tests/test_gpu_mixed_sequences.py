@@ -290,3 +290,27 @@ def test_a_relu_on_top_of_a_relu_lists_its_rows_anew(nnv, oracle, count, half_wi
         ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
     for method in ("relax-star-area", "relax-star-random"):
         _compare(nnv, oracle, layers, dev_in, ora_in, method)
+
+
+@pytest.mark.parametrize("seed", [318, 456, 620, 690, 717, 720, 800, 843, 855, 892])
+def test_random_fc_sequences_that_once_failed(nnv, oracle, seed):
+    """Random FC / ReLU / batch-normalisation sequences over one, two or five boxes of widths from 0.005 to 3, the
+    six relax-star methods in turn: the seeds of a longer run of this generator on which an earlier build of the
+    library gave wrong sets (all of them hold a ReLU step directly on top of another one)."""
+    rs = np.random.RandomState(seed)
+    n_in = int(rs.choice([5, 12, 40, 90]))
+    layers = _random_fc_sequence(rs, n_in)
+    count = int(rs.choice([1, 2, 5]))
+    centre = rs.rand(n_in, count)
+    half = np.abs(rs.randn(n_in, count)) * rs.choice([0.005, 0.02, 0.3, 3.0], size=(1, count))
+    if rs.rand() < 0.5:
+        half[rs.randint(n_in), :] = 0.0
+    lbs, ubs = centre - half, centre + half
+    method = ["relax-star-area", "relax-star-range", "relax-star-static", "relax-star-random", "relax-star-bound",
+              "relax-star-ub"][seed % 6]
+    if count == 1:
+        dev_in, ora_in = nnv.Star(lbs[:, 0], ubs[:, 0]), oracle.star_from_box(lbs[:, 0], ubs[:, 0])
+    else:
+        dev_in = nnv.Star.from_boxes(lbs, ubs)
+        ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
+    _compare(nnv, oracle, layers, dev_in, ora_in, method)
