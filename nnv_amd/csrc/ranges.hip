@@ -1022,12 +1022,15 @@ int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, co
   }
   // Sets that gather the same columns with the same scales under the same bounds (the boxes of one shape,
   // nnvhip_star_from_box) have the same sums: one pair of columns serves them all.  Only runs of a few distinct
-  // descriptions are looked for (a set is compared with the last 16 new ones).
+  // descriptions are looked for (a set is compared with the last 16 new ones; the columns a ReLU step appended --
+  // no scales -- are a set's own list, and only the last description is looked at).
   std::vector<GatherSet> uniq;
+  uniq.reserve((size_t)count);
   slot->assign((size_t)count, 0);
   for (int64_t i = 0; i < count; ++i) {
     int64_t found = -1;
-    for (int64_t k = (int64_t)uniq.size() - 1; k >= 0 && k >= (int64_t)uniq.size() - 16 && found < 0; --k) {
+    const int64_t back = sets[i].scale != nullptr ? 16 : 1;
+    for (int64_t k = (int64_t)uniq.size() - 1; k >= 0 && k >= (int64_t)uniq.size() - back && found < 0; --k) {
       const GatherSet& u = uniq[(size_t)k];
       if (u.idx == sets[i].idx && u.scale == sets[i].scale && u.plb == sets[i].plb && u.pub == sets[i].pub && u.m == sets[i].m) found = k;
     }
