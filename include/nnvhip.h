@@ -326,6 +326,15 @@ NNVHIP_API int nnvhip_set_small_chain(nnvhip_ctx* ctx, int enabled);
  * A switch applies to the layer calls made
  * after it; sets produced before keep what they recorded.  Unknown name: NNVHIP_ERR_ARG. */
 NNVHIP_API int nnvhip_set_switch(nnvhip_ctx* ctx, const char* name, int enabled);
+/* A hint, with no counterpart in the reference (whose layer loop, nn/NN.m:1542-1547, calls one layer after the
+ * other): the FC layer that the caller will apply to the output of its NEXT nnvhip_relu_relax call on this context.
+ * For an array of at least 64 sets that ReLU step then queues, right behind its classification, the part of the FC
+ * layer's range estimate that needs nothing but the classes (the sums over the columns the step appends), so that
+ * the device works on it while the host reads the step's counts and sets the FC call up; nnvhip_affine_fc finds it
+ * on the sets and does not form it again.  Results are the same to the bit with and without the hint; a hint that
+ * does not come true (another layer follows, other sets are passed) costs the product and nothing else.  The hint
+ * is consumed by the next nnvhip_relu_relax call; fc == NULL withdraws it. */
+NNVHIP_API int nnvhip_hint_next_fc(nnvhip_ctx* ctx, const nnvhip_fc* fc);
 enum { NNVHIP_LAYER_FC = 0, NNVHIP_LAYER_CONV2D = 1, NNVHIP_LAYER_RELU = 2 };
 NNVHIP_API int nnvhip_reach_layers(nnvhip_ctx* ctx, int64_t n_layers, const int32_t* kind, const void* const* layer,
                         const int64_t* hw, int order, double relax_factor, int64_t count, nnvhip_star* const* in,

@@ -29,7 +29,7 @@ SYMBOLS = [
     "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists", "nnvhip_probe_mfma_peak",
     "nnvhip_estimate_ranges_static", "nnvhip_debug_mailbox_pack", "nnvhip_debug_mailbox_unpack",
     "nnvhip_debug_set_relu_call_number", "nnvhip_reach_layers", "nnvhip_relu_reduce_mem",
-    "nnvhip_set_switch", "nnvhip_debug_counters", "nnvhip_weight_cache_stats", "nnvhip_weight_cache_release", "nnvhip_debug_weak_weight_hash",
+    "nnvhip_set_switch", "nnvhip_hint_next_fc", "nnvhip_debug_counters", "nnvhip_weight_cache_stats", "nnvhip_weight_cache_release", "nnvhip_debug_weak_weight_hash",
 ]
 
 
@@ -122,6 +122,7 @@ def load():
         "nnvhip_reach_layers": [p, i64, p, p, p, C.c_int, dbl, i64, pp, pp],
         "nnvhip_relu_reduce_mem": [p, p, i64, i64, i64, pp, p, p],
         "nnvhip_set_switch": [p, C.c_char_p, C.c_int],
+        "nnvhip_hint_next_fc": [p, p],
         "nnvhip_debug_counters": [p, pi64, pi64, pi64, pi64],
         "nnvhip_weight_cache_stats": [p, pi64, pi64, pi64],
         "nnvhip_weight_cache_release": [p, pi64],
@@ -258,6 +259,10 @@ class Context:
         v = [C.c_int64() for _ in range(4)]
         check(self.lib.nnvhip_debug_counters(self.handle, *[C.byref(x) for x in v]))
         return dict(zip(("device_mallocs", "staging_waits", "deferred_handles", "live_handles"), (x.value for x in v)))
+
+    def hint_next_fc(self, weights):
+        """nnvhip_hint_next_fc: the FC layer (its device weights, or None) that will follow the next ReLU step."""
+        check(self.lib.nnvhip_hint_next_fc(self.handle, weights.h if weights is not None else None))
 
     def set_switch(self, name: str, on: bool):
         """One of the route switches a context otherwise reads from the environment (nnvhip_set_switch)."""

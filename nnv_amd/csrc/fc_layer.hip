@@ -113,7 +113,18 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       any = any || g.m > 0;
       mm_plb_zero = mm_plb_zero && (g.m == 0 || in[i]->oh_plb_zero);
     }
-    if (ok && any) st = launch_range_sums_mm(c, fc, count, es.data(), &mm_early, &mm_slot, mm_plb_zero);
+    // (the ReLU step that made the sets may have queued this very product already: nnvhip_hint_next_fc)
+    bool ahead = ok && any && mm_plb_zero;
+    for (int64_t i = 0; i < count && ahead; ++i)
+      ahead = in[i]->ahead_mm_buf && in[i]->ahead_mm_uid == fc->uid && in[i]->ahead_mm_buf == in[0]->ahead_mm_buf &&
+              in[i]->oh_scale == nullptr;
+    if (ahead) {
+      mm_early = in[0]->ahead_mm_buf;
+      mm_slot.resize((size_t)count);
+      for (int64_t i = 0; i < count; ++i) mm_slot[(size_t)i] = in[i]->ahead_mm_slot;
+    } else if (ok && any) {
+      st = launch_range_sums_mm(c, fc, count, es.data(), &mm_early, &mm_slot, mm_plb_zero);
+    }
   }
   if (st == NNVHIP_OK) st = make_affine_outputs(c, count, in, fc->M, &outs, &contig, &cols);
   if (st == NNVHIP_OK) {

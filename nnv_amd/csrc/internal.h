@@ -275,6 +275,9 @@ struct nnvhip_ctx {
   // staging ring wrapped or grew, mailbox waits that went through the slow path
   int64_t n_device_mallocs = 0, n_staging_waits = 0;
   uint64_t visit_seq = 0;
+  uint64_t next_layer_uid = 0;
+  // nnvhip_hint_next_fc: the FC layer the caller will apply to the output of its next ReLU step (consumed by that step)
+  const nnvhip_fc* next_fc = nullptr;
   // memory of released handles, reused by new_star (at most kMaxFreeStars of them are kept)
   static constexpr size_t kMaxFreeStars = 32768;
   std::vector<void*> free_stars;
@@ -443,6 +446,13 @@ struct nnvhip_star {
   // cover columns from rng_first_col on, like the chunks above, and are added after them.
   nnvhip::BufRef rng_mm_buf;
   const double* rng_mm = nullptr;
+  // A ReLU output of an array whose caller had said which FC layer comes next (nnvhip_hint_next_fc): the range sums
+  // of the columns that layer will gather for the columns this step appended, as launch_range_sums_mm leaves them
+  // (slot ahead_mm_slot of the product), queued behind the classification so that the device forms them while the
+  // host reads the counts and sets the layer call up.  For the layer with uid ahead_mm_uid only.
+  nnvhip::BufRef ahead_mm_buf;
+  uint64_t ahead_mm_uid = 0;
+  int64_t ahead_mm_slot = 0;
   bool has_producer_sums() const { return (rng_part != nullptr && rng_chunks > 0) || rng_mm != nullptr; }
   // some scale of the unit-vector block is negative (a box with ub < lb): sign-split products do not apply
   bool oh_scale_neg = false;
@@ -474,6 +484,7 @@ struct nnvhip_fc {
   std::atomic<int> refs{1};
   nnvhip_ctx* ctx = nullptr;
   int64_t M = 0, K = 0, Mp = 0, Kp = 0;
+  uint64_t uid = 0;     // of this context's layers, never reused (a set remembers which layer a product made ahead is for)
   nnvhip::BufRef W;     // Mp x Kp, zero padded, ld = Mp
   nnvhip::BufRef bias;  // Mp entries (zero padded) or null
   // [max(W, 0); min(W, 0)], 2*Mp x Kp with ld = 2*Mp: made on first use by launch_range_sums_mm
@@ -802,6 +813,14 @@ int launch_gather_columns(nnvhip_ctx* ctx, const double* W, int64_t ldw, int64_t
 // with a = scatter(sc * plb), b = scatter(sc * pub) per set, [max(W,0); min(W,0)] * [a b] holds
 // [xmin1; xmax2] and [xmax1; xmin2].  One fp64 MFMA product over all sets instead of a pass over the
 // cache-resident weights per set.  out: 2*Mp x 2*count, ld = 2*Mp, columns 2i and 2i+1 belong to set i.
+// The same product (every column's lower predicate bound zero, no scales) for the columns a ReLU step is about to
+// append, from the step's per-row classes and the input's upper bounds instead of the lists the host does not have
+// yet: x_s(r) = ub_s(r) where neuron r crosses (cls_s(r) >= 0), 0 elsewhere.  Set i's sums are slot i of *out.
+struct AheadSet {
+  const int32_t* cls;
+  const double* ub;
+};
+int launch_range_sums_mm_ahead(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const AheadSet* sets, int64_t N, BufRef* out);
 int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out,
                          std::vector<int64_t>* slot,  // slot[i]: which pair of columns of `out` holds set i's sums
                          bool plb_zero = false);      // every lower bound involved is 0: the first column of every pair is

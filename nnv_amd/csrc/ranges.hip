@@ -1009,17 +1009,59 @@ __global__ __launch_bounds__(256) void sum_vectors_kernel(const GatherSet* __res
   }
 }
 
+static int ensure_split_weights(nnvhip_ctx* ctx, const nnvhip_fc* fc) {
+  if (fc->Wpn) return NNVHIP_OK;
+  const int64_t Mp = fc->Mp, Kp = fc->Kp;
+  BufRef w;
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * Kp, &w));
+  hipLaunchKernelGGL(split_sign_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(Mp * Kp, 256), 4096)), dim3(256), 0, ctx->stream,
+                     fc->W->as<double>(), w->as<double>(), Mp, Kp);
+  NNV_HIP_TRY(hipGetLastError());
+  fc->Wpn = w;
+  return NNVHIP_OK;
+}
+
+// [W+; W-] * (the odd columns of X) into the odd column pairs of *out, whose even ones ([xmin1; xmax2], products with
+// a zero vector) are +0: what the product leaves when every gathered column has lower predicate bound zero.
+static int range_sums_upper_half(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t nu, const BufRef& X, BufRef* out) {
+  const int64_t Mp = fc->Mp, Kp = fc->Kp;
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * nu, out));
+  NNV_HIP_TRY(hipMemsetAsync((*out)->ptr, 0, sizeof(double) * 2 * Mp * 2 * nu, ctx->stream));
+  std::vector<int32_t> odd((size_t)nu);
+  for (int64_t k = 0; k < nu; ++k) odd[(size_t)k] = (int32_t)(2 * k + 1);
+  BufRef cmap;
+  NNV_TRY(ctx->upload_table(odd.data(), sizeof(int32_t) * odd.size(), &cmap));
+  GemmRows rows;
+  rows.colmap = cmap->as<int32_t>();
+  if (Kp <= 2048) rows.tile_hint = 64;
+  return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, nu, Kp, nullptr,
+                     nullptr, &rows);
+}
+
+// Column 2i+1 of X (Kp rows): ub where the neuron crosses, zero elsewhere (column 2i is not read).
+__global__ __launch_bounds__(256) void crossing_ub_vectors_kernel(const AheadSet* __restrict__ table, double* __restrict__ X, int Kp, int N) {
+  const AheadSet d = table[blockIdx.x];
+  double* xb = X + ((int64_t)2 * blockIdx.x + 1) * Kp;
+  for (int r = threadIdx.x; r < Kp; r += 256) xb[r] = (r < N && d.cls[r] >= 0) ? d.ub[r] : 0.0;
+}
+
+int launch_range_sums_mm_ahead(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const AheadSet* sets, int64_t N, BufRef* out) {
+  const int64_t Kp = fc->Kp;
+  if (count >= (int64_t(1) << 30) || N > Kp) NNV_FAIL(NNVHIP_ERR_ARG, "internal: range sums ahead of their layer out of range");
+  NNV_TRY(ensure_split_weights(ctx, fc));
+  BufRef X, tab;
+  NNV_TRY(ctx->alloc(sizeof(double) * Kp * 2 * count, &X));
+  NNV_TRY(ctx->upload(sets, sizeof(AheadSet) * count, &tab));
+  hipLaunchKernelGGL(crossing_ub_vectors_kernel, dim3((unsigned)count), dim3(256), 0, ctx->stream, tab->as<AheadSet>(), X->as<double>(),
+                     (int)Kp, (int)N);
+  NNV_HIP_TRY(hipGetLastError());
+  return range_sums_upper_half(ctx, fc, count, X, out);
+}
+
 int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out,
                          std::vector<int64_t>* slot, bool plb_zero) {
   const int64_t Mp = fc->Mp, Kp = fc->Kp;
-  if (!fc->Wpn) {
-    BufRef w;
-    NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * Kp, &w));
-    hipLaunchKernelGGL(split_sign_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(Mp * Kp, 256), 4096)), dim3(256), 0, ctx->stream,
-                       fc->W->as<double>(), w->as<double>(), Mp, Kp);
-    NNV_HIP_TRY(hipGetLastError());
-    fc->Wpn = w;
-  }
+  NNV_TRY(ensure_split_weights(ctx, fc));
   // Sets that gather the same columns with the same scales under the same bounds (the boxes of one shape,
   // nnvhip_star_from_box) have the same sums: one pair of columns serves them all.  Only runs of a few distinct
   // descriptions are looked for (a set is compared with the last 16 new ones; the columns a ReLU step appended --
@@ -1046,21 +1088,10 @@ int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, co
   NNV_TRY(ctx->upload(uniq.data(), sizeof(GatherSet) * nu, &tab));
   hipLaunchKernelGGL(sum_vectors_kernel, dim3((unsigned)nu), dim3(256), 0, ctx->stream, tab->as<GatherSet>(), X->as<double>(), (int)Kp);
   NNV_HIP_TRY(hipGetLastError());
+  // a = scatter(sc * plb) is zero for every set: its products [xmin1; xmax2] are +0 (a fill), and only the columns
+  // of b = scatter(sc * pub) go through the matrix cores
+  if (plb_zero && nu < (int64_t(1) << 30)) return range_sums_upper_half(ctx, fc, nu, X, out);
   NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * nu, out));
-  if (plb_zero && nu < (int64_t(1) << 30)) {
-    // a = scatter(sc * plb) is zero for every set: its products [xmin1; xmax2] are +0 (a fill), and only the columns
-    // of b = scatter(sc * pub) go through the matrix cores
-    NNV_HIP_TRY(hipMemsetAsync((*out)->ptr, 0, sizeof(double) * 2 * Mp * 2 * nu, ctx->stream));
-    std::vector<int32_t> odd((size_t)nu);
-    for (int64_t k = 0; k < nu; ++k) odd[(size_t)k] = (int32_t)(2 * k + 1);
-    BufRef cmap;
-    NNV_TRY(ctx->upload_table(odd.data(), sizeof(int32_t) * odd.size(), &cmap));
-    GemmRows rows;
-    rows.colmap = cmap->as<int32_t>();
-    if (Kp <= 2048) rows.tile_hint = 64;
-    return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, nu, Kp, nullptr,
-                       nullptr, &rows);
-  }
   return launch_gemm(ctx, fc->Wpn->as<double>(), 2 * Mp, X->as<double>(), Kp, (*out)->as<double>(), 2 * Mp, 2 * Mp, 2 * nu, Kp,
                      nullptr);
 }

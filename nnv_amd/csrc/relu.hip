@@ -644,6 +644,9 @@ static int64_t one_block_limit() {
 }
 
 int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in, nnvhip_star** out, const ReluGiven* given) {
+  // (a hint about the layer that follows is for this step, whatever becomes of it)
+  const nnvhip_fc* const next_fc = ctx->next_fc;
+  ctx->next_fc = nullptr;
   if (count > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "at most 65535 sets per call");
   if ((order == kOrderGiven) != (given != nullptr)) NNV_FAIL(NNVHIP_ERR_ARG, "internal: explicit lists and their order go together");
   // the appended unit-vector columns are stored only on request or when the FC / conv maps are told to
@@ -797,6 +800,17 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
                          descs[0], kRankNewBounds | kRankOldBounds | kRankCountOnDevice);
   }
   NNV_HIP_TRY(hipGetLastError());
+
+  // An array whose caller has said which FC layer comes next: that layer's range sums of the columns this step
+  // appends need only the per-row classes and the input's upper bounds, both on the device by now, and no count.
+  // Queued here, the product runs while the host reads the counts, makes the handles and sets the layer call up.
+  BufRef ahead_mm;
+  if (next_fc != nullptr && given == nullptr && lazy_rows && count >= 64 && !ctx->eager_cols && !ctx->dense_affine &&
+      next_fc->K == N && next_fc->ctx == ctx) {
+    std::vector<AheadSet> as((size_t)count);
+    for (int64_t i = 0; i < count; ++i) as[(size_t)i] = AheadSet{descs[i].cls, descs[i].ub};
+    NNV_TRY(launch_range_sums_mm_ahead(ctx, next_fc, count, as.data(), N, &ahead_mm));
+  }
 
   // Output handles: whatever does not depend on the counts is set up while the kernel runs (with the
   // row reset pending and the bounds written by the kernel, that is nearly everything).
@@ -993,6 +1007,11 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     if (given == nullptr) {  // the input's estimated upper bounds, by neuron
       o->pre_ub_buf = in[i]->rbuf;
       o->pre_ub = in[i]->ub;
+    }
+    if (ahead_mm) {
+      o->ahead_mm_buf = ahead_mm;
+      o->ahead_mm_uid = next_fc->uid;
+      o->ahead_mm_slot = i;
     }
     if (d.m > 0) {  // the appended columns are the unit vectors of the crossing neurons
       o->oh_from = in[i]->n + 1;

@@ -171,6 +171,7 @@ int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M,
   }
   std::unique_ptr<nnvhip_fc> fc(new nnvhip_fc());
   fc->ctx = c;
+  fc->uid = ++c->next_layer_uid;
   fc->M = M;
   fc->K = K;
   fc->Mp = round_up(M, kLdAlign);
@@ -210,8 +211,18 @@ int nnvhip_fc_create(nnvhip_ctx* c, const double* W, const double* b, int64_t M,
 int nnvhip_fc_destroy(nnvhip_fc* fc) {
   if (!fc) return NNVHIP_OK;
   nnvhip_ctx* c = fc->ctx;
-  if (fc->refs.fetch_sub(1) == 1) delete fc;
+  if (fc->refs.fetch_sub(1) == 1) {
+    if (c->next_fc == fc) c->next_fc = nullptr;
+    delete fc;
+  }
   c->live_handles--;
+  return NNVHIP_OK;
+}
+
+int nnvhip_hint_next_fc(nnvhip_ctx* c, const nnvhip_fc* fc) {
+  CHECK_CTX(c);
+  if (fc != nullptr && fc->ctx != c) NNV_FAIL(NNVHIP_ERR_ARG, "layer of another context");
+  c->next_fc = fc;
   return NNVHIP_OK;
 }
 

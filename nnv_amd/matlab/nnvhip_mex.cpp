@@ -194,6 +194,9 @@ void mexFunction(int nlhs, mxArray* plhs[], int nrhs, const mxArray* prhs[]) {
     std::vector<nnvhip_star*> in = handles_of(prhs[2]), out(in.size());
     check(nnvhip_affine_fc(ctx(), handle_of<nnvhip_fc>(prhs[1]), (int64_t)in.size(), in.data(), out.data()));
     plhs[0] = to_mx(out);
+  } else if (cmd == "hint_next_fc") {  // (layer | [])      the FC layer that will follow the next ReLU step (an array of sets)
+    need(nrhs, 1, "hint_next_fc");
+    check(nnvhip_hint_next_fc(ctx(), mxIsEmpty(prhs[1]) ? nullptr : handle_of<nnvhip_fc>(prhs[1])));
   } else if (cmd == "affine_conv2d") {  // (layer, H, W, handles) -> handles      Conv2DLayer.reach
     need(nrhs, 4, "affine_conv2d");
     std::vector<nnvhip_star*> in = handles_of(prhs[4]), out(in.size());

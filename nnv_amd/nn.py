@@ -113,6 +113,11 @@ class NN:
             eager = i == last and not ctx.eager_columns
             if eager:
                 ctx.set_eager_columns(True)
+            # an array of sets in front of a ReLU step that an FC layer follows: the library is told, and queues
+            # the part of that layer's range estimate that needs only the step's classes behind the classification
+            if (isinstance(layer, ReluLayer) and i < last and isinstance(self.Layers[i + 1], FullyConnectedLayer)
+                    and isinstance(rs, (list, tuple, SetArray)) and len(rs) >= 64):
+                ctx.hint_next_fc(self.Layers[i + 1]._weights(ctx))
             try:
                 rs = layer.reach(rs, self.reachMethod, self.reachOption, self.relaxFactor, self.dis_opt, self.lp_solver)
             finally:

@@ -314,3 +314,55 @@ def test_random_fc_sequences_that_once_failed(nnv, oracle, seed):
         dev_in = nnv.Star.from_boxes(lbs, ubs)
         ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
     _compare(nnv, oracle, layers, dev_in, ora_in, method)
+
+
+@pytest.mark.parametrize("count", [64, 100, 40])
+def test_a_hint_about_the_next_fc_layer_changes_no_bit(nnv, oracle, count):
+    """NN.reach tells the library which FC layer follows a ReLU step over an array of at least 64 sets; the step then
+    queues that layer's range-sum product of the columns it appends behind its classification, and the FC call
+    takes it from the sets instead of forming it.  With the hint, without it (the layers called one by one), with a
+    hint that does not come true (another FC layer of the same shape is applied), and for an array too small for
+    it: the same sets and the same bounds to the bit, and the oracle's to tolerance; where the hint is taken the FC
+    call launches one matrix product less."""
+    rs = np.random.RandomState(2100 + count)
+    n_in, hidden = 60, 320
+    half = rs.randint(1, 64, size=(n_in, count)) / 1024.0
+    centre = rs.randint(0, 1024, size=(n_in, count)) / 1024.0
+    lbs, ubs = centre - half, centre + half
+    layers = [_fc(rs, hidden, n_in, 2.0), {"type": "relu"}, _fc(rs, 290, hidden, 2.0), {"type": "relu"}, _fc(rs, 6, 290)]
+    other = nnv.NN.from_config([_fc(rs, 290, hidden, 2.0)], "another layer of the same shape").Layers[0]
+    ctx = nnv.default_context()
+    net = nnv.NN.from_config(layers, "hint")
+    L = net.Layers
+    opts = ("relax-star-area", [], 1, None, "linprog")
+
+    def run(hint, second=None):
+        s = nnv.Star.from_boxes(lbs, ubs)
+        s = L[0].reach(s, *opts)
+        if hint is not None:
+            ctx.hint_next_fc(hint._weights(ctx))
+        s = L[1].reach(s, *opts)
+        ctx.kernel_time(0)
+        ctx.set_timing(2)
+        try:
+            t = (second or L[2]).reach(s, *opts)
+        finally:
+            ctx.set_timing(0)
+        gemms = ctx.kernel_time(0)[1]
+        u = L[3].reach(t, *opts)
+        bounds = [tuple(np.asarray(x).copy() for x in a.estimateRanges()) for a in t]
+        return gemms, bounds, [np.asarray(a.V).copy() for a in u]
+
+    g0, b0, v0 = run(None)
+    g1, b1, v1 = run(L[2])
+    g2, b2, v2 = run(other, second=L[2])         # hinted at a layer that is not the one applied
+    for (l0, u0), (l1, u1), (l2, u2) in zip(b0, b1, b2):
+        assert np.array_equal(l0, l1) and np.array_equal(u0, u1) and np.array_equal(l0, l2) and np.array_equal(u0, u2)
+    for a, b, c_ in zip(v0, v1, v2):
+        assert np.array_equal(a, b) and np.array_equal(a, c_)
+    if not ctx.switch_is_on("eager_cols", "dense_affine", "eager_rows", "eager_tail"):
+        assert g1 == (g0 - 1 if count >= 64 else g0), (g0, g1)
+        assert g2 == g0
+    # NN.reach gives the hint itself; against the oracle
+    _compare(nnv, oracle, layers, nnv.Star.from_boxes(lbs, ubs), [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)],
+             "relax-star-area")

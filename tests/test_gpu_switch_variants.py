@@ -87,6 +87,10 @@ def test_a_relu_on_top_of_a_relu_lists_its_rows_anew(route, nnv, oracle, count, 
     seqs.test_a_relu_on_top_of_a_relu_lists_its_rows_anew(nnv, oracle, count, half_width)
 
 
+def test_a_hint_about_the_next_fc_layer_changes_no_bit(route, nnv, oracle):
+    seqs.test_a_hint_about_the_next_fc_layer_changes_no_bit(nnv, oracle, 64)
+
+
 def test_one_wide_set_through_the_tile_kernel(route, nnv, oracle):
     seqs.test_one_wide_set_through_the_tile_kernel(nnv, oracle, "relax-star-area")
 
