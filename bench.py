@@ -379,6 +379,15 @@ def measure(k, args, ctx, exact_steps, extras):
         g["what"] = ("FC layer over an array of sets of one shape: the product over the rows most sets keep is formed once per "
                      "shape, every set's tiles start from it and contract over the rows in which the set differs; bytes = the "
                      "output matrices written")
+        if not ctx.eager_columns and not args.dense and not args.written:
+            # nobody on the way to the next layer reads these matrices (the ReLU step takes the range sums): the pass forms
+            # and sums every piece and stores the centre columns and the partial sums only - what it then moves is a small
+            # part of what it computes, and the vector ALUs bound it, not HBM (the fraction of the HBM peak says so)
+            g["matrices_left_unwritten"] = True
+            g["what"] = ("FC layer over an array of sets of one shape: the product over the rows most sets keep is formed once per "
+                         "shape; every set's pieces start from it, add the rows in which the set differs and are summed into the "
+                         "set's range sums without being stored (written by the same pass on first read); bytes = centre columns "
+                         "and partial sums written; bound by the vector ALUs, not by HBM")
         g["dense_equivalent_flop_per_step"] = gemm_flop
         g["dense_equivalent_achieved_TFLOPs"] = round(gemm_flop * reps / (dlt_ms * 1e-3) / 1e12, 1)
         groups.append((dlt_ms, g))
@@ -530,8 +539,9 @@ def measure(k, args, ctx, exact_steps, extras):
                    "intermediate_sets": "dense" if args.dense else
                    "every layer writes its whole output matrix in the call, as the reference's reachSet{i} holds it" if args.written else
                    "every layer's set is written in full by the one launch that reaches the whole network" if chain_launches else
-                   "the sets between layers record a ReLU's row reset / appended columns and the columns an FC layer "
-                   "gathers from its weights and write them on first read; the returned set and its bounds are written",
+                   "the sets between layers record a ReLU's row reset / appended columns, the columns an FC layer "
+                   "gathers from its weights and the matrices an FC layer forms from a product its sets share, and write "
+                   "them on first read; the returned set and its bounds are written",
                    "predicates_per_layer": [n for (_, n) in shapes][:len(cfg["layers"])] if single else None},
         "roofline": roofline, "cpu_baseline": cpu, "spec_check": spec, "host_to_host": host_to_host,
         "all_sets_written": all_written, "layers": layer_report,

@@ -184,6 +184,14 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
       for (int64_t i = 1; i < count; ++i)
         if (in[i]->ld != in[0]->ld || in[i]->V != in[i - 1]->V + in[i - 1]->stored_cols() * in[i - 1]->ld) contig = false;
     }
+    // Matrices a shared-product call left unwritten (ColSource::delta) are written before rows of them are read; a set
+    // that keeps no row reads none.
+    {
+      std::vector<nnvhip_star*> need;
+      for (int64_t i = 0; i < count; ++i)
+        if (in[i]->cs.delta_pending() && !(in[i]->rows_pending && in[i]->n_kept == 0)) need.push_back(in[i]);
+      if (!need.empty() && st == NNVHIP_OK) st = write_pending_columns(c, (int64_t)need.size(), need.data());
+    }
     // Rows of the dense columns that the ReLU step reset to zero need no contraction either: the
     // GEMM then runs over the kept rows only (used when that at least halves K).
     // *pack: gather the listed rows into a matrix of their own first (several row tiles of W would each
@@ -675,8 +683,44 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                     dbytes += 8.0 * (double)Mp * (double)dense[i];
                     max_cols = std::max<int64_t>(max_cols, dense[i]);
                   }
-                if (st == NNVHIP_OK && !douts.empty())
-                  st = launch_delta_tiles(c, Wd, Mp, Mp, bias, ldo, (int64_t)douts.size(), douts.data(), dgroup.data(), max_cols, dbytes);
+                // Nothing on the way to the next layers reads these matrices where the layer's caller reads bounds only
+                // (the ReLU step takes the range sums, the next FC layer the rows the step keeps - often none): unless
+                // every column is to be in memory after the call, the pass forms and sums the pieces without storing
+                // them, and the description stays on the handles (ColSource::delta) for whoever reads them first.
+                const bool defer = lazy_ok && !douts.empty();
+                if (st == NNVHIP_OK && !douts.empty()) {
+                  double sums_only = 0.0;  // what the pass then writes: centre columns and partial sums
+                  for (const DeltaOut& d : douts) sums_only += 8.0 * (double)Mp + 32.0 * (double)ldo * (double)delta_tile_chunks(d.ncols);
+                  st = launch_delta_tiles(c, Wd, Mp, Mp, bias, ldo, (int64_t)douts.size(), douts.data(), dgroup.data(), max_cols,
+                                          defer ? sums_only : dbytes, !defer);
+                }
+                if (st == NNVHIP_OK && defer) {
+                  Ref<DeltaCall> call = make_ref<DeltaCall>();
+                  call->W = fc->W;
+                  call->bias = fc->bias;
+                  call->base = basebuf;
+                  call->S = shared_rows;
+                  call->cprod = cprod;
+                  call->lists = delta;
+                  call->arena = outs[0]->Vbuf;
+                  call->A = Wd;
+                  call->bias_ptr = bias;
+                  call->lda = Mp;
+                  call->Mp = Mp;
+                  call->ldo = ldo;
+                  call->max_cols = max_cols;
+                  call->bytes = dbytes;
+                  call->outs = douts;
+                  for (DeltaOut& d : call->outs) d.rpart = nullptr;
+                  call->group = dgroup;
+                  for (int64_t a = 0; a < nact; ++a) {
+                    nnvhip_star* o = outs[act[(size_t)a]];
+                    o->cs.delta = call;
+                    if (c->poison_pending && dense[act[(size_t)a]] > 1 &&  // debugging aid: NaNs where nothing was written
+                        hipMemsetAsync(o->V + o->ld, 0xff, sizeof(double) * o->ld * (dense[act[(size_t)a]] - 1), c->stream) != hipSuccess)
+                      st = NNVHIP_ERR_HIP;
+                  }
+                }
                 delta_done = true;
                 bias_in_kernel = true;
               }

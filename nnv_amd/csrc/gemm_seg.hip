@@ -552,11 +552,37 @@ constexpr int kDeltaCols = 64;  // columns of a block's piece = columns per chun
 struct DeltaBatch {
   int32_t first, nsets;  // sets [first, first + nsets) of the table, all of one group
 };
-__global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaOut* __restrict__ sets, const DeltaBatch* __restrict__ batches,
+// Entry `src_lane` (wave-uniform) of a value that the lanes of a wave hold one each.
+__device__ __forceinline__ double readlane_f64(double v, int src_lane) {
+  const int lo = __builtin_amdgcn_readlane(__double2loint(v), src_lane);
+  const int hi = __builtin_amdgcn_readlane(__double2hiint(v), src_lane);
+  return __hiloint2double(hi, lo);
+}
+
+// A set's description with the first four entries of its difference list beside it: one trip to memory tells a block
+// everything it needs to ask for the set's operands.
+struct DeltaRec {
+  DeltaOut d;
+  int32_t e4[4];  // -1: no such entry
+};
+__global__ __launch_bounds__(256) void delta_recs_kernel(const DeltaOut* __restrict__ sets, DeltaRec* __restrict__ recs, int count) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  DeltaRec r;
+  r.d = sets[i];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) r.e4[t] = t < r.d.dlen ? r.d.delta[t] : -1;
+  recs[i] = r;
+}
+
+// STORE == false: the pieces are formed and summed, and only the centre column is written (a call whose matrices
+// nobody may ever read; whoever does has them written by a second pass with STORE == true and no sums).
+template <bool STORE>
+__global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaRec* __restrict__ recs, const DeltaBatch* __restrict__ batches,
                                                           const double* __restrict__ A, int64_t lda, int Mp,
                                                           const double* __restrict__ bias, int64_t ldo) {
   const DeltaBatch bt = batches[blockIdx.z];
-  const DeltaOut d0 = sets[bt.first];
+  const DeltaOut d0 = recs[bt.first].d;
   const int cc = blockIdx.x, rb = blockIdx.y;
   const int j0 = cc * kDeltaCols;
   if (j0 >= d0.ncols) return;  // (the sets of a group have the same columns)
@@ -573,23 +599,54 @@ __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaOut* __rest
     if (active && u < nj) base[u] = *reinterpret_cast<const double2_t*>(d0.base + (int64_t)(jw + u) * Mp + r0);
   }
   __shared__ double2_t red[2][3][4][64];  // the sums of waves 1-3 of a set, two sets in flight
-  for (int s = 0; s < bt.nsets; ++s) {
-    const DeltaOut d = sets[bt.first + s];
-    double2_t x1 = {0.0, 0.0}, x2 = {0.0, 0.0}, y1 = {0.0, 0.0}, y2 = {0.0, 0.0};
-    // the set's row differences (usually a handful): the first four are looked up once per set - entry, weight column
-    // entries of the lane's rows, row of the shared operand - and any more go through the loop per column
-    int e4[4];
+  // What a set brings besides the shared piece.  Its row differences (usually a handful): the first four come with
+  // the set's record, and the weight column entries of the lane's rows and the rows of the shared operand they name
+  // are looked up once per set; any more go through the loop per column.  What the wave's sixteen columns need of
+  // those rows and the columns' predicate bounds is read by lane u (mod 16) for column u and handed round by lane
+  // reads: one load each instead of a scalar load per column and value.  The look-ups run ahead of the arithmetic:
+  // while set s is worked on, the operands of set s + 1 are in flight and the record of set s + 2 is on its way, so
+  // that no set waits for its two dependent trips to memory (the storing pass: 1.49 -> 1.39 ms for config 5's
+  // 6.7 GB; the pass that stores nothing is bound by its instruction count - 420 vector and 270 scalar instructions
+  // per set and wave, the vector unit busy half of the time - and gains nothing from it: 0.58 ms either way).
+  struct SetOps {
     double2_t w4[4];
-    const double* s4[4];
+    double sv4[4];
+    double pl16, pu16;
+  };
+  const int lcol = lane & 15;
+  const bool lcol_in = lcol < nj;
+  auto operands = [&](const DeltaRec& q, SetOps& o) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      e4[t] = t < d.dlen ? d.delta[t] : -1;
-      const int r = max(e4[t], 0) & (kSegSubtract - 1);
-      w4[t] = double2_t{0.0, 0.0};
-      if (e4[t] >= 0 && active) w4[t] = *reinterpret_cast<const double2_t*>(A + (int64_t)r * lda + r0);
-      if (e4[t] >= 0 && (e4[t] & kSegSubtract)) w4[t] = -w4[t];  // the row is taken away: -(w * s) = (-w) * s
-      s4[t] = d.S + (int64_t)r * d.lds;
+      const int r = max(q.e4[t], 0) & (kSegSubtract - 1);
+      o.w4[t] = double2_t{0.0, 0.0};
+      if (q.e4[t] >= 0 && active) o.w4[t] = *reinterpret_cast<const double2_t*>(A + (int64_t)r * lda + r0);
+      if (q.e4[t] >= 0 && (q.e4[t] & kSegSubtract)) o.w4[t] = -o.w4[t];  // the row is taken away: -(w * s) = (-w) * s
+      o.sv4[t] = (q.e4[t] >= 0 && lcol_in) ? q.d.S[(int64_t)r * q.d.lds + jw + lcol] : 0.0;
     }
+    o.pl16 = o.pu16 = 0.0;
+    if (q.d.rpart != nullptr && lcol_in && jw + lcol >= 1) {
+      o.pl16 = q.d.plb[jw + lcol - 1];
+      o.pu16 = q.d.pub[jw + lcol - 1];
+    }
+  };
+  DeltaRec rec = recs[bt.first];                                     // set s
+  DeltaRec rec1 = recs[bt.first + min(1, bt.nsets - 1)];             // set s + 1
+  SetOps cur, nxt;
+  operands(rec, cur);
+  for (int s = 0; s < bt.nsets; ++s) {
+    if (s + 1 < bt.nsets) operands(rec1, nxt);                       // (its record arrived an iteration ago)
+    const DeltaRec rec2 = recs[bt.first + min(s + 2, bt.nsets - 1)];  // asked for now, read at the top of the next round
+    const DeltaOut& d = rec.d;
+    const int(&e4)[4] = rec.e4;
+    const double2_t(&w4)[4] = cur.w4;
+    const double(&sv4)[4] = cur.sv4;
+    const double pl16 = cur.pl16, pu16 = cur.pu16;
+    double2_t x1 = {0.0, 0.0}, x2 = {0.0, 0.0}, y1 = {0.0, 0.0}, y2 = {0.0, 0.0};
+    // Columns whose predicate bounds mirror each other (plb = -pub: every generator of a box star) make xmin1 the
+    // mirror image of xmax1 and xmax2 that of xmin2, rounding included (fl(a * (-p) + (-s)) = -fl(a * p + s)): half
+    // of the products are then left out and the two sums negated at the end.
+    const bool mirrored = d.rpart != nullptr && __all(pl16 == -pu16);
     if (active && nj > 0) {
 #pragma unroll
       for (int u = 0; u < 16; ++u) {
@@ -599,7 +656,7 @@ __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaOut* __rest
 #pragma unroll
           for (int t = 0; t < 4; ++t)
             if (e4[t] >= 0) {
-              const double sv = s4[t][j];
+              const double sv = readlane_f64(sv4[t], u);
               o[0] = fma(w4[t][0], sv, o[0]);
               o[1] = fma(w4[t][1], sv, o[1]);
             }
@@ -619,23 +676,35 @@ __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaOut* __rest
               o[1] = o[1] + bias[r0 + 1];
             }
           } else if (d.rpart != nullptr) {
-            const double pl = d.plb[j - 1], pu = d.pub[j - 1];
+            const double pl = readlane_f64(pl16, u), pu = readlane_f64(pu16, u);
             const double px = fmax(o[0], 0.0), nx = fmin(o[0], 0.0), py = fmax(o[1], 0.0), ny = fmin(o[1], 0.0);
-            x1[0] = fma(px, pl, x1[0]);
-            x1[1] = fma(py, pl, x1[1]);
             x2[0] = fma(nx, pu, x2[0]);
             x2[1] = fma(ny, pu, x2[1]);
             y1[0] = fma(px, pu, y1[0]);
             y1[1] = fma(py, pu, y1[1]);
-            y2[0] = fma(nx, pl, y2[0]);
-            y2[1] = fma(ny, pl, y2[1]);
+            if (!mirrored) {
+              x1[0] = fma(px, pl, x1[0]);
+              x1[1] = fma(py, pl, x1[1]);
+              y2[0] = fma(nx, pl, y2[0]);
+              y2[1] = fma(ny, pl, y2[1]);
+            }
           }
           // (streaming store: the output is not read again here)
-          __builtin_nontemporal_store(o, reinterpret_cast<double2_t*>(d.out + (int64_t)j * ldo + r0));
+          if (STORE || j == 0) __builtin_nontemporal_store(o, reinterpret_cast<double2_t*>(d.out + (int64_t)j * ldo + r0));
         }
       }
     }
-    if (d.rpart == nullptr) continue;  // (all sets of a call agree on this)
+    if (d.rpart == nullptr) {  // (all sets of a call agree on this)
+      rec = rec1;
+      rec1 = rec2;
+      cur = nxt;
+      continue;
+    }
+    if (mirrored) {  // (0 - s: a sum that is still +0 stays +0, as the left-out additions of -0 would have left it)
+      x1 = double2_t{0.0 - y1[0], 0.0 - y1[1]};
+      y2 = double2_t{0.0 - x2[0], 0.0 - x2[1]};
+    }
+
     const int par = s & 1;
     if (wave > 0) {
       red[par][wave - 1][0][lane] = x1;
@@ -660,6 +729,9 @@ __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaOut* __rest
       *reinterpret_cast<double2_t*>(dst + 2 * ldo) = y1;  // xmax1 = sum max(v,0)*pub
       *reinterpret_cast<double2_t*>(dst + 3 * ldo) = y2;  // xmax2 = sum min(v,0)*plb
     }
+    rec = rec1;
+    rec1 = rec2;
+    cur = nxt;
   }
 }
 
@@ -706,7 +778,7 @@ int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev,
 int delta_tile_chunks(int64_t ncols) { return (int)ceil_div(ncols, kDeltaCols); }
 
 int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp, const double* bias, int64_t ldo, int64_t count,
-                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes) {
+                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes, bool store) {
   if (count <= 0 || max_cols <= 0) return NNVHIP_OK;
   if (Mp % 16 || Mp > ldo || count >= (int64_t(1) << 24)) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: shared-product tiles out of range");
   // batches of neighbouring sets of one group: long enough to make the read of the shared piece small next to the
@@ -722,12 +794,19 @@ int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp
     a = b;
   }
   if (batches.size() > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "array too large for one launch");
-  BufRef tab, btab;
+  BufRef tab, btab, rtab;
   NNV_TRY(ctx->upload_table(sets, sizeof(DeltaOut) * count, &tab));
   NNV_TRY(ctx->upload_table(batches.data(), sizeof(DeltaBatch) * batches.size(), &btab));
+  NNV_TRY(ctx->alloc(sizeof(DeltaRec) * (size_t)count, &rtab));
+  hipLaunchKernelGGL(delta_recs_kernel, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, ctx->stream, tab->as<DeltaOut>(),
+                     rtab->as<DeltaRec>(), (int)count);
   const bool timed = ctx->kernel_timing;
-  NNV_LAUNCH(ctx, timed, delta_tiles_kernel, dim3((unsigned)col_chunks, (unsigned)row_blocks, (unsigned)batches.size()), dim3(256), 0,
-             tab->as<DeltaOut>(), btab->as<DeltaBatch>(), A, lda, (int)Mp, bias, ldo);
+  if (store)
+    NNV_LAUNCH(ctx, timed, delta_tiles_kernel<true>, dim3((unsigned)col_chunks, (unsigned)row_blocks, (unsigned)batches.size()), dim3(256), 0,
+               rtab->as<DeltaRec>(), btab->as<DeltaBatch>(), A, lda, (int)Mp, bias, ldo);
+  else
+    NNV_LAUNCH(ctx, timed, delta_tiles_kernel<false>, dim3((unsigned)col_chunks, (unsigned)row_blocks, (unsigned)batches.size()), dim3(256),
+               0, rtab->as<DeltaRec>(), btab->as<DeltaBatch>(), A, lda, (int)Mp, bias, ldo);
   NNV_TRY(ctx->kernel_timer_end(timed, 10, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;

@@ -157,6 +157,37 @@ struct ColBox {
   int16_t h0, h1, w0, w1;
 };
 
+// One set of launch_delta_tiles (declared further down): its output is its group's shared product (base) plus the
+// row differences of (+/-) A(:, r) * S(r, j), the centre column replaced by cprod (+ bias).
+struct DeltaOut {
+  const int32_t* delta;  // dlen entries: r or r | kSegSubtract
+  const double* base;    // Mp x ncols, leading dimension Mp
+  const double* S;       // the group's scaled rows, row-major: S(r, j) at S[r * lds + j]
+  int64_t lds;
+  const double* cprod;   // Mp entries
+  double* out;           // the set's column 0 (leading dimension ldo)
+  const double* plb;     // the set's predicate bounds, by generator column
+  const double* pub;
+  double* rpart;
+  int32_t dlen;
+  int32_t ncols;
+};
+// A call of the shared-product route of an FC layer over an array whose output matrices have not been written: the
+// range sums and the centre columns are in place, the dense columns are what `outs` says and are written - for all
+// sets of the call at once - when somebody first reads any of them (write_pending_columns).  The buffers the
+// description points into are kept alive here.
+struct DeltaCall {
+  int64_t ref_count = 0;
+  BufRef W, bias, base, S, cprod, lists, arena;
+  const double* A = nullptr;
+  const double* bias_ptr = nullptr;
+  int64_t lda = 0, Mp = 0, ldo = 0, max_cols = 0;
+  double bytes = 0.0;
+  std::vector<DeltaOut> outs;  // rpart == null: the sums were delivered with the call
+  std::vector<int32_t> group;
+  bool written = false;
+};
+
 // Where an FC map gathered stored columns of a set from, and whether they are in memory yet.  Column
 // from + t holds 0 + W(:, r) * scale[r] with r = idx[t] (scale == null: 1).  A later packing of kept rows
 // reads the cache-resident weight matrix instead of the set's own matrix in HBM; and the FC map may leave
@@ -191,7 +222,11 @@ struct ColSource {
   int64_t win_rows = 0;  // rows of the image (H * W * channels)
   int32_t win_H = 0, win_W = 0;
   bool win_pending() const { return win_to > win_from; }
-  bool any_pending() const { return pending || zero_to > 1 || win_pending(); }
+  // The leading (contracted) columns 1 .. of the matrix are the output of a shared-product call that has not written
+  // them yet (column 0, the centre, is in memory).
+  Ref<DeltaCall> delta;
+  bool delta_pending() const { return delta && !delta->written; }
+  bool any_pending() const { return pending || zero_to > 1 || win_pending() || delta_pending(); }
 };
 
 // One node per ReLU layer of the structured constraint store.  The dense NNV matrix
@@ -656,23 +691,12 @@ int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev,
 // row differences of (+/-) A(:, r) * S(r, j) for j < ncols, the centre column (j = 0) replaced by cprod (+ bias), and
 // the four Star.estimateRanges partial sums of every piece of delta_tile_chunks' columns in rpart ([piece][4][ldo]).  A streaming
 // pass (gemm_seg.hip, delta_tiles_kernel): bound by the bytes it writes.
-struct DeltaOut {
-  const int32_t* delta;  // dlen entries: r or r | kSegSubtract
-  const double* base;    // Mp x ncols, leading dimension Mp
-  const double* S;       // the group's scaled rows, row-major: S(r, j) at S[r * lds + j]
-  int64_t lds;
-  const double* cprod;   // Mp entries
-  double* out;           // the set's column 0 (leading dimension ldo)
-  const double* plb;     // the set's predicate bounds, by generator column
-  const double* pub;
-  double* rpart;
-  int32_t dlen;
-  int32_t ncols;
-};
 // (sets: host table, neighbours of one group next to one another; group_of[i]: group of set i of the table; the
 // pass leaves delta_tile_chunks(ncols) chunks of range sums per set)
+// store == false: only the centre columns and the range sums are written (the matrices are left to a later call with
+// store == true and no rpart).
 int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp, const double* bias, int64_t ldo, int64_t count,
-                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes);
+                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes, bool store = true);
 int delta_tile_chunks(int64_t ncols);
 // Cm(r, s) = centre of set s at row r if the set keeps row r, else +0: Cm is Kp x count (ld = Kp), zeroed here.
 struct CentreSet {

@@ -78,7 +78,7 @@ int nnvhip_affine_conv2d(nnvhip_ctx* c, const nnvhip_conv2d* cv, int64_t H, int6
       const ColSource& cs = in[i]->cs;
       if (plan[i].dense > in[i]->stored_cols())
         full.push_back(in[i]);
-      else if (cs.pending || cs.zero_to > 1 || (cs.win_pending() && !plan[i].compact) ||
+      else if (cs.pending || cs.zero_to > 1 || cs.delta_pending() || (cs.win_pending() && !plan[i].compact) ||
                (in[i]->rows_pending && !mask_on_load(in[i])))
         prefix.push_back(in[i]);
     }

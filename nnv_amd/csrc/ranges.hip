@@ -1135,7 +1135,9 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, RangeC
       const int64_t scan_end = (t->has_producer_sums() && t->rng_first_col >= 1) ? t->rng_first_col : t->n + 1;
       // (columns that are in memory inside their windows only are fine for a scan that stays inside the windows)
       const bool win = t->cs.win_pending() && scan_end > t->cs.win_from && !in_windows;
-      if ((t->cs.pending && scan_end > t->cs.from) || (t->cs.zero_to > 1 && scan_end > 1) || win) cols.push_back(t);
+      if ((t->cs.pending && scan_end > t->cs.from) || (t->cs.zero_to > 1 && scan_end > 1) || win ||
+          (t->cs.delta_pending() && scan_end > 1))
+        cols.push_back(t);
     }
     if (!cols.empty()) NNV_TRY(write_pending_columns(ctx, (int64_t)cols.size(), cols.data()));
   }
@@ -1462,6 +1464,14 @@ static int write_window_zeros(nnvhip_ctx* ctx, double* V, int64_t ld, ColSource*
 
 // One gather launch per run of sets that share the weight matrix and the leading dimension.
 int write_cols(nnvhip_ctx* ctx, std::vector<PendingCols>& todo) {
+  // matrices a shared-product call described and did not store: all sets of such a call in one pass
+  for (auto& t : todo)
+    if (t.cs->delta_pending()) {
+      DeltaCall& dc = *t.cs->delta;
+      NNV_TRY(launch_delta_tiles(ctx, dc.A, dc.lda, dc.Mp, dc.bias_ptr, dc.ldo, (int64_t)dc.outs.size(), dc.outs.data(), dc.group.data(),
+                                 dc.max_cols, dc.bytes, true));
+      dc.written = true;
+    }
   {  // columns written inside their windows only: the zeros around them
     std::vector<PendingCols> rest;
     for (auto& t : todo) {

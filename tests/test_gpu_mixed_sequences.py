@@ -67,15 +67,18 @@ def _compare(nnv, oracle, layers, dev_in, ora_in, method, tol=1e-9):
         assert_close(np.asarray(ub).reshape(-1, order="F"), np.asarray(eub).reshape(-1, order="F"), "ub", tol)
     # every intermediate set too, read after the whole reach has run (so the reads meet sets whose
     # row reset or appended columns were never needed by the next layer)
+    # (of an array: its first, middle and last set - one read may write the matrices of many sets at once)
     for i, (rset, eset) in enumerate(zip(net.reachSet, exp_sets)):
-        r0 = rset[0] if isinstance(rset, (list, nnv.SetArray)) else rset
-        e0 = eset[0] if isinstance(eset, list) else eset
-        RV, EV = np.asarray(r0.V), e0.V
-        if EV.ndim == 4:
-            EV = EV.reshape(-1, EV.shape[-1], order="F")
-            RV = RV.reshape(-1, RV.shape[-1], order="F")
-        assert_close(RV, EV, "layer %d V" % (i + 1), tol)
-        assert np.array_equal(RV == 0, EV == 0), "layer %d zero pattern" % (i + 1)
+        many = isinstance(rset, (list, nnv.SetArray))
+        for k in (sorted({0, len(rset) // 2, len(rset) - 1}) if many else [None]):
+            r0 = rset[k] if many else rset
+            e0 = eset[k if many else 0] if isinstance(eset, list) else eset
+            RV, EV = np.asarray(r0.V), e0.V
+            if EV.ndim == 4:
+                EV = EV.reshape(-1, EV.shape[-1], order="F")
+                RV = RV.reshape(-1, RV.shape[-1], order="F")
+            assert_close(RV, EV, "layer %d set %s V" % (i + 1, k), tol)
+            assert np.array_equal(RV == 0, EV == 0), "layer %d set %s zero pattern" % (i + 1, k)
 
 
 @pytest.mark.parametrize("seed", range(10))
@@ -268,6 +271,93 @@ def test_neighbouring_boxes_share_the_product_over_their_common_rows(nnv, oracle
     _, launches = _shared_product_launches(ctx, lambda: _compare(nnv, oracle, layers, dev_in, ora_in, "relax-star-area"))
     if expect is not None and not ctx.switch_is_on("no_row_deltas", "dense_affine", "eager_tail"):
         assert (launches > 0) == expect, "spread %g: %d launches of the shared-product pass" % (spread, launches)
+
+
+@pytest.mark.parametrize("then", ["relu", "fc", "batchnorm", "relu_relu"])
+def test_matrices_a_layer_leaves_unwritten_read_the_same_later(nnv, oracle, then):
+    """An FC layer over neighbouring boxes that forms its outputs as shared product plus row differences stores, by
+    default, only their centres and range sums: the ReLU step behind it needs no more, and the next FC layer reads
+    only rows that step keeps.  Whoever does read the matrices first (a fetch, a layer that is not a ReLU step, an
+    FC layer behind two ReLU steps) has all sets of the call written by the same pass.  Against the "every column
+    written at once" mode: every matrix of the layer is the same to the bit, whether read early, late or only after
+    the next layers ran, and when it is read changes no bit of the bounds or of the sets two layers on; the pass
+    runs once inside the layer and once more at the first read, not again at the second."""
+    rs = np.random.RandomState(2300)
+    n_in, count, hidden = 200, 96, 400
+    widths = rs.randint(1, 64, size=(n_in, 2)) / 8192.0
+    half = widths[:, np.arange(count) % 2]
+    c0 = rs.randint(256, 768, size=(n_in, 1)) / 1024.0
+    centre = c0 + np.round(rs.randn(n_in, count) * 2e-3 * 1024.0) / 1024.0
+    lbs, ubs = centre - half, centre + half
+    fc1, fc2, fc3 = _fc(rs, hidden, n_in, 2.0), _fc(rs, 260, hidden, 2.0), _fc(rs, 9, 260)
+    tails = {"relu": [{"type": "relu"}, fc3], "fc": [fc3, {"type": "relu"}],
+             "batchnorm": [_bn(rs, 260), {"type": "relu"}, fc3],
+             "relu_relu": [{"type": "relu"}, {"type": "relu"}, fc3]}
+    layers = [fc1, {"type": "relu"}, fc2] + tails[then]
+    ctx = nnv.default_context()
+    L = nnv.NN.from_config(layers, "unwritten matrices").Layers
+    opts = ("relax-star-area", [], 1, None, "linprog")
+
+    def passes():
+        return ctx.kernel_time(10)[1]
+
+    def run(read_first):
+        s = nnv.Star.from_boxes(lbs, ubs)
+        for layer in L[:2]:
+            s = layer.reach(s, *opts)
+        ctx.set_timing(2)
+        try:
+            passes()
+            t = L[2].reach(s, *opts)
+            n_layer = passes()
+            early = [np.asarray(a.V).copy() for a in t] if read_first else None
+            n_early = passes()
+            u = t
+            for layer in L[3:]:
+                u = layer.reach(u, *opts)
+            n_next = passes()
+            outs = [np.asarray(a.V).copy() for a in u]
+            bounds = [tuple(np.asarray(x).copy() for x in a.estimateRanges()) for a in t]
+            n_rest = passes()
+            late = [np.asarray(t[k].V).copy() for k in (count - 1, 0, count // 2)]
+            n_late = passes()
+            again = np.asarray(t[3].V).copy()
+            n_again = passes()
+        finally:
+            ctx.set_timing(0)
+        return dict(early=early, outs=outs, bounds=bounds, late=late, again=again, n=(n_layer, n_early, n_next, n_rest, n_late, n_again))
+
+    a = run(False)
+    b = run(True)
+    was = ctx.switches.get("eager_cols", False)
+    ctx.set_switch("eager_cols", True)
+    try:
+        e = run(True)
+    finally:
+        ctx.set_switch("eager_cols", was)
+    for p, q in zip(a["outs"], b["outs"]):                               # read early or late: nothing else changes
+        assert np.array_equal(p, q)
+    for (l0, u0), (l1, u1) in zip(a["bounds"], b["bounds"]):
+        assert np.array_equal(l0, l1) and np.array_equal(u0, u1)
+    for x in (a, b):                                                     # the matrices themselves, whenever written
+        for p, q in zip(x["late"], e["late"]):
+            assert np.array_equal(p, q)
+        assert np.array_equal(x["again"], e["again"])
+        # (the other mode sums the bounds of these matrices in another order: equal to rounding, not to the bit)
+        for (l0, u0), (l1, u1) in zip(x["bounds"], e["bounds"]):
+            assert_close(l0, l1, "lb", 1e-11)
+            assert_close(u0, u1, "ub", 1e-11)
+    for p, q in zip(b["early"], e["early"]):
+        assert np.array_equal(p, q)
+    for k, idx in enumerate((count - 1, 0, count // 2)):
+        assert np.array_equal(b["late"][k], b["early"][idx])
+    if not ctx.switch_is_on("eager_cols", "dense_affine", "eager_tail", "no_row_deltas", "eager_rows"):
+        assert e["n"][0] == 1 and sum(e["n"][1:]) == 0, e["n"]           # everything written inside the layer
+        assert b["n"][:2] == (1, 1) and sum(b["n"][2:]) == 0, b["n"]     # ... at the first read
+        assert a["n"][:2] == (1, 0) and sum(a["n"][2:]) == 1 and a["n"][5] == 0, a["n"]   # ... by whoever reads first
+    # and against the oracle, all layers
+    _compare(nnv, oracle, layers, nnv.Star.from_boxes(lbs, ubs), [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)],
+             "relax-star-area")
 
 
 @pytest.mark.parametrize("count,half_width", [(1, 0.02), (1, 3.0), (5, 0.3)])

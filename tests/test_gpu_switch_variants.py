@@ -91,6 +91,11 @@ def test_a_hint_about_the_next_fc_layer_changes_no_bit(route, nnv, oracle):
     seqs.test_a_hint_about_the_next_fc_layer_changes_no_bit(nnv, oracle, 64)
 
 
+@pytest.mark.parametrize("then", ["relu", "batchnorm"])
+def test_matrices_a_layer_leaves_unwritten_read_the_same_later(route, nnv, oracle, then):
+    seqs.test_matrices_a_layer_leaves_unwritten_read_the_same_later(nnv, oracle, then)
+
+
 def test_one_wide_set_through_the_tile_kernel(route, nnv, oracle):
     seqs.test_one_wide_set_through_the_tile_kernel(nnv, oracle, "relax-star-area")
 
