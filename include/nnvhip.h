@@ -322,7 +322,10 @@ NNVHIP_API int nnvhip_set_small_chain(nnvhip_ctx* ctx, int enabled);
  * (NNVHIP_POISON_PENDING: whatever a layer leaves unwritten until first read is filled with NaNs),
  * "no_small_chain", "no_conv_mask", "no_conv_boxes" (NNVHIP_NO_*), "no_row_deltas" (NNVHIP_NO_ROW_DELTAS: an FC
  * layer over an array of sets of one shape contracts every set over its whole kept-row list instead of forming
- * the product over the rows most sets keep once and contracting each set over its differences from that list).
+ * the product over the rows most sets keep once and contracting each set over its differences from that list),
+ * "no_sum_shortcuts" (NNVHIP_NO_SUM_SHORTCUTS: where that layer sums its sets' pieces without storing them, every
+ * set is summed in full and with both bounds of every predicate - not once per run of sets that agree in list and
+ * bounds, and not with one bound where the bounds mirror each other; the sums are the same to the bit).
  * A switch applies to the layer calls made
  * after it; sets produced before keep what they recorded.  Unknown name: NNVHIP_ERR_ARG. */
 NNVHIP_API int nnvhip_set_switch(nnvhip_ctx* ctx, const char* name, int enabled);

@@ -37,7 +37,8 @@ SYMBOLS = [
 SWITCH_ENV = {"dense_affine": "NNVHIP_DENSE_AFFINE", "eager_rows": "NNVHIP_EAGER_ROWS", "eager_tail": "NNVHIP_EAGER_TAIL",
               "eager_cols": "NNVHIP_EAGER_COLS", "poison_pending": "NNVHIP_POISON_PENDING",
               "no_small_chain": "NNVHIP_NO_SMALL_CHAIN", "no_conv_mask": "NNVHIP_NO_CONV_MASK",
-              "no_conv_boxes": "NNVHIP_NO_CONV_BOXES", "no_row_deltas": "NNVHIP_NO_ROW_DELTAS"}
+              "no_conv_boxes": "NNVHIP_NO_CONV_BOXES", "no_row_deltas": "NNVHIP_NO_ROW_DELTAS",
+              "no_sum_shortcuts": "NNVHIP_NO_SUM_SHORTCUTS"}
 
 
 class NNVHipError(RuntimeError):

@@ -252,6 +252,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   c->no_conv_mask = getenv("NNVHIP_NO_CONV_MASK") != nullptr;
   c->no_conv_boxes = getenv("NNVHIP_NO_CONV_BOXES") != nullptr;
   c->no_row_deltas = getenv("NNVHIP_NO_ROW_DELTAS") != nullptr;
+  c->no_sum_shortcuts = getenv("NNVHIP_NO_SUM_SHORTCUTS") != nullptr;
   if (const char* e = getenv("NNVHIP_WEIGHT_CACHE_MB")) c->weight_cache_budget = (int64_t)atoll(e) << 20;
   NNV_HIP_TRY(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   NNV_HIP_TRY(hipEventCreate(&c->ev0));
@@ -341,7 +342,7 @@ int nnvhip_set_switch(nnvhip_ctx* c, const char* name, int enabled) {
       {"eager_tail", &c->eager_tail, false},       {"eager_cols", &c->eager_cols, false},
       {"poison_pending", &c->poison_pending, false}, {"no_small_chain", &c->small_chain, true},
       {"no_conv_mask", &c->no_conv_mask, false},   {"no_conv_boxes", &c->no_conv_boxes, false},
-      {"no_row_deltas", &c->no_row_deltas, false},
+      {"no_row_deltas", &c->no_row_deltas, false}, {"no_sum_shortcuts", &c->no_sum_shortcuts, false},
   };
   for (const auto& t : table)
     if (strcmp(t.name, name) == 0) {

@@ -571,17 +571,23 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                 st = launch_delta_lists(c, nact, dtab->as<DeltaSet>(), groups, gtab->as<int32_t>(), rowsK, rows_pad, kDeltaCap,
                                         votes->as<int32_t>(), common->as<int32_t>(), lens->as<int32_t>(), delta->as<int32_t>(),
                                         lens->as<int32_t>() + groups);
-              std::vector<int32_t> hl((size_t)(groups + nact));
+              // the lengths of the lists come back, and with them the first four entries of each (what the sets are
+              // put in order by further down)
+              std::vector<int32_t> hl((size_t)(groups + nact)), head((size_t)(4 * nact));
               if (st == NNVHIP_OK) {
                 void* hp = nullptr;
-                st = c->stage(sizeof(int32_t) * hl.size(), &hp);
+                st = c->stage(sizeof(int32_t) * (hl.size() + head.size()), &hp);
                 if (st == NNVHIP_OK) {
+                  int32_t* hh = static_cast<int32_t*>(hp) + hl.size();
                   if (hipMemcpyAsync(hp, lens->ptr, sizeof(int32_t) * hl.size(), hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+                      hipMemcpy2DAsync(hh, sizeof(int32_t) * 4, delta->ptr, sizeof(int32_t) * kDeltaCap, sizeof(int32_t) * 4, (size_t)nact,
+                                       hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
                       hipStreamSynchronize(c->stream) != hipSuccess) {
                     set_error("HIP error reading the row-difference lists back");
                     st = NNVHIP_ERR_HIP;
                   } else {
                     memcpy(hl.data(), hp, sizeof(int32_t) * hl.size());
+                    memcpy(head.data(), hh, sizeof(int32_t) * head.size());
                   }
                 }
               }
@@ -661,28 +667,45 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                 std::vector<int32_t> dgroup;
                 double dbytes = 0.0;
                 int64_t max_cols = 0;
-                for (int g = 0; g < groups && st == NNVHIP_OK; ++g)
-                  for (int64_t a = 0; a < nact; ++a) {
-                    const int64_t i = act[(size_t)a];
-                    if (shape_of[i] != g) continue;
-                    const RowShape& r = shapes[(size_t)g];
-                    DeltaOut d{};
-                    d.delta = delta->as<int32_t>() + a * kDeltaCap;
-                    d.base = basebuf->as<double>() + base_off[(size_t)g] * Mp;
-                    d.S = shared_rows->as<double>() + r.off;
-                    d.lds = r.ldws;
-                    d.cprod = cprod->as<double>() + a * Mp;
-                    d.out = outs[0]->V + col_off[(size_t)i] * ldo;
-                    d.plb = outs[i]->plb;
-                    d.pub = outs[i]->pub;
-                    d.rpart = sums->as<double>() + 4 * ldo * chunk_off[i];
-                    d.dlen = hl[(size_t)(groups + a)];
-                    d.ncols = (int32_t)dense[i];
-                    douts.push_back(d);
-                    dgroup.push_back((int32_t)g);
-                    dbytes += 8.0 * (double)Mp * (double)dense[i];
-                    max_cols = std::max<int64_t>(max_cols, dense[i]);
-                  }
+                // (within a group by the length of their lists and by the lists' first entries: sets with the same list -
+                // those without differences, whose pieces are the shared product itself, above all - then stand next to
+                // one another, and the pass that stores nothing sums a piece once for a run of sets that agree in list
+                // and bounds)
+                std::vector<int64_t> order;
+                for (int g = 0; g < groups; ++g) {
+                  const size_t from = order.size();
+                  for (int64_t a = 0; a < nact; ++a)
+                    if (shape_of[act[(size_t)a]] == g) order.push_back(a);
+                  std::stable_sort(order.begin() + (int64_t)from, order.end(), [&](int64_t x, int64_t y) {
+                    const int32_t lx = hl[(size_t)(groups + x)], ly = hl[(size_t)(groups + y)];
+                    if (lx != ly) return lx < ly;
+                    for (int t = 0; t < std::min(lx, 4); ++t)
+                      if (head[(size_t)(4 * x + t)] != head[(size_t)(4 * y + t)]) return head[(size_t)(4 * x + t)] < head[(size_t)(4 * y + t)];
+                    return false;
+                  });
+                }
+                for (size_t k = 0; k < order.size() && st == NNVHIP_OK; ++k) {
+                  const int64_t a = order[k];
+                  const int64_t i = act[(size_t)a];
+                  const int g = shape_of[i];
+                  const RowShape& r = shapes[(size_t)g];
+                  DeltaOut d{};
+                  d.delta = delta->as<int32_t>() + a * kDeltaCap;
+                  d.base = basebuf->as<double>() + base_off[(size_t)g] * Mp;
+                  d.S = shared_rows->as<double>() + r.off;
+                  d.lds = r.ldws;
+                  d.cprod = cprod->as<double>() + a * Mp;
+                  d.out = outs[0]->V + col_off[(size_t)i] * ldo;
+                  d.plb = outs[i]->plb;
+                  d.pub = outs[i]->pub;
+                  d.rpart = sums->as<double>() + 4 * ldo * chunk_off[i];
+                  d.dlen = hl[(size_t)(groups + a)];
+                  d.ncols = (int32_t)dense[i];
+                  douts.push_back(d);
+                  dgroup.push_back((int32_t)g);
+                  dbytes += 8.0 * (double)Mp * (double)dense[i];
+                  max_cols = std::max<int64_t>(max_cols, dense[i]);
+                }
                 // Nothing on the way to the next layers reads these matrices where the layer's caller reads bounds only
                 // (the ReLU step takes the range sums, the next FC layer the rows the step keeps - often none): unless
                 // every column is to be in memory after the call, the pass forms and sums the pieces without storing

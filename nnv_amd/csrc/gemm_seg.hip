@@ -575,9 +575,6 @@ __global__ __launch_bounds__(256) void delta_recs_kernel(const DeltaOut* __restr
   recs[i] = r;
 }
 
-// STORE == false: the pieces are formed and summed, and only the centre column is written (a call whose matrices
-// nobody may ever read; whoever does has them written by a second pass with STORE == true and no sums).
-template <bool STORE>
 __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaRec* __restrict__ recs, const DeltaBatch* __restrict__ batches,
                                                           const double* __restrict__ A, int64_t lda, int Mp,
                                                           const double* __restrict__ bias, int64_t ldo) {
@@ -690,7 +687,7 @@ __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaRec* __rest
             }
           }
           // (streaming store: the output is not read again here)
-          if (STORE || j == 0) __builtin_nontemporal_store(o, reinterpret_cast<double2_t*>(d.out + (int64_t)j * ldo + r0));
+          __builtin_nontemporal_store(o, reinterpret_cast<double2_t*>(d.out + (int64_t)j * ldo + r0));
         }
       }
     }
@@ -733,6 +730,280 @@ __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaRec* __rest
     rec1 = rec2;
     cur = nxt;
   }
+}
+
+// The pass that stores no matrix.  What a set adds to the shared piece is a product of rank four or less - (its
+// rows' weight entries) x (those rows of the shared operand) - which is one 16x16x4 MFMA per 16 x 16 outputs with
+// the shared piece as the accumulator going in (none for a set without differences, further ones for lists of more
+// than four entries).  fp64 MFMA runs at the rate of the vector unit's fp64 FMAs and shares it: the instruction
+// saves no time for the product itself but takes its operands per lane as they come from memory, where the
+// vector form (the pass above) hands every operand round by lane reads: 421 vector + 266 scalar instructions per
+// set and wave there, about 230 + 80 here.  A wave owns 32 rows x 64 columns (2 x 4 such tiles, held in registers
+// for the batch of sets as above); the instruction's "a" operand carries columns and its "b" operand rows, so that
+// result register r of lane l is O[row l % 16][column l / 16 + 4r]: a lane multiplies its four outputs by the
+// bounds of its own four columns, the sums over all of the wave's columns are left in four lane groups, and two
+// lane exchanges finish them - no LDS, no barrier.  Four waves of a block cover the 128 rows of the other pass's
+// block, and a block's columns are one chunk of range sums there as here.
+//
+// What the pass reads of a set ahead of its turn (SumRec) and at its turn (SumTail).
+struct SumRec {
+  const double* pub;
+  int32_t e4[4];  // the first four entries of the set's list; -1: no such entry
+  int32_t dlen;
+  int32_t flags;  // kSumMirrored, kSumSameAsLast
+};
+constexpr int32_t kSumMirrored = 1;    // every predicate of the set has plb = -pub (the sums then need one of the two)
+constexpr int32_t kSumSameAsLast = 2;  // group, list and bounds are those of the set before it in the table: so are its sums
+struct SumTail {
+  const double* plb;
+  double* rpart;
+  const double* cprod;
+  double* out;
+  const int32_t* delta;
+};
+// One wave per set.
+__global__ __launch_bounds__(64) void delta_sum_recs_kernel(const DeltaOut* __restrict__ sets, SumRec* __restrict__ recs,
+                                                            SumTail* __restrict__ tails, int shortcuts) {
+  const int i = blockIdx.x;
+  const int lane = threadIdx.x;
+  const DeltaOut d = sets[i];
+  bool mine = true;
+  for (int j = lane; j < d.ncols - 1; j += 64) mine = mine && d.plb[j] == -d.pub[j];
+  const bool mirrored = __all(mine);
+  bool same = i > 0;
+  if (same) {
+    const DeltaOut p = sets[i - 1];
+    same = p.base == d.base && p.S == d.S && p.ncols == d.ncols && p.dlen == d.dlen;
+    if (same) {
+      bool eq = true;
+      for (int t = lane; t < d.dlen; t += 64) eq = eq && p.delta[t] == d.delta[t];
+      for (int j = lane; j < d.ncols - 1; j += 64)  // (to the bit: a zero's sign shows in the sums)
+        eq = eq && __double_as_longlong(p.plb[j]) == __double_as_longlong(d.plb[j]) &&
+             __double_as_longlong(p.pub[j]) == __double_as_longlong(d.pub[j]);
+      same = __all(eq);
+    }
+  }
+  if (lane == 0) {
+    SumRec r;
+    r.pub = d.pub;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) r.e4[t] = t < d.dlen ? d.delta[t] : -1;
+    r.dlen = d.dlen;
+    r.flags = shortcuts ? (mirrored ? kSumMirrored : 0) | (same ? kSumSameAsLast : 0) : 0;
+    recs[i] = r;
+    tails[i] = SumTail{d.plb, d.rpart, d.cprod, d.out, d.delta};
+  }
+}
+
+typedef const double __attribute__((address_space(1)))* gdouble_t;  // (a pointer known to be to device memory)
+__device__ __forceinline__ gdouble_t in_global(const double* p) { return (gdouble_t)p; }
+__device__ __forceinline__ double max0(double v) {  // (fmax / fmin without the pass that quiets signalling NaNs first)
+  double r;
+  asm("v_max_f64 %0, %1, 0" : "=v"(r) : "v"(v));
+  return r;
+}
+__device__ __forceinline__ double min0(double v) {
+  double r;
+  asm("v_min_f64 %0, %1, 0" : "=v"(r) : "v"(v));
+  return r;
+}
+
+// EDGE: the block's columns include column 0 (the centre, which is the set's own and enters no sum) or columns past
+// the last; their entries of the shared piece and of the shared operand are made zero, so that they add nothing.
+template <bool EDGE, int RT>
+__device__ __forceinline__ void delta_sums_body(const SumRec* __restrict__ recs, const SumTail* __restrict__ tails, const DeltaBatch bt,
+                                                const double* __restrict__ basep, const double* __restrict__ S, int64_t lds, int ncols,
+                                                const double* __restrict__ A, int64_t lda, int Mp, const double* __restrict__ bias,
+                                                int64_t ldo, int cc, int row0, bool two) {
+  const int lane = threadIdx.x & 63;
+  const int l16 = lane & 15, g4 = lane >> 4;
+  const int j0 = cc * kDeltaCols;
+  int rows[RT];  // (a wave without a second row tile does the first twice)
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) rows[rt] = (rt == 0 || two ? row0 + 16 * rt : row0) + l16;
+  const int nct = EDGE ? min(4, (ncols - j0 + 15) / 16) : 4;
+  double4_t base[RT][4];
+#pragma unroll
+  for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int col = j0 + 16 * ct + g4 + 4 * r;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        base[rt][ct][r] = 0.0;
+        if (!EDGE || (col >= 1 && col < ncols)) base[rt][ct][r] = basep[(int64_t)col * Mp + rows[rt]];
+      }
+    }
+  // A set's operands.  "a": entry l / 16 of its list, column l % 16 of column tile ct of the shared operand; "b":
+  // the same entry, row l % 16 of row tile rt of the weights; the upper predicate bounds of the lane's sixteen
+  // columns.  Each is asked for again - for the next set - right after its last use for this one, so that a whole
+  // set's arithmetic lies between the request and the use and no second copy of the registers is needed.
+  double sv[4], w[RT], pu[4][4];
+  // (an entry that is not there reads row 0 of both operands and makes the weight entries zero)
+  auto entry_of = [&](const SumRec& q) { return g4 == 0 ? q.e4[0] : g4 == 1 ? q.e4[1] : g4 == 2 ? q.e4[2] : q.e4[3]; };
+  auto column_operand = [&](int e, int ct) {
+    const int r = max(e, 0) & (kSegSubtract - 1);
+    double v = (in_global(S) + ((int64_t)r * lds + j0 + l16))[16 * ct];  // (rows of S are padded past the last column)
+    if (EDGE) {
+      const int col = j0 + 16 * ct + l16;
+      if (col < 1 || col >= ncols) v = 0.0;
+    }
+    return v;
+  };
+  auto row_operand = [&](int e, int row) {
+    const int r = max(e, 0) & (kSegSubtract - 1);
+    double v = (in_global(A) + (int64_t)r * lda)[row];
+    if (e & kSegSubtract) v = -v;  // the row is taken away: -(w * s) = (-w) * s
+    if (e < 0) v = 0.0;
+    return v;
+  };
+  auto bounds_of = [&](const double* bounds, int ct, double (&out)[4]) {
+    const gdouble_t b = in_global(bounds);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int col = j0 + 16 * ct + g4 + 4 * r;
+      // (past the edges: some bound of the set; what it multiplies is zero)
+      out[r] = EDGE ? b[min(max(col, 1), ncols - 1) - 1] : (b + (j0 + g4 - 1))[16 * ct + 4 * r];
+    }
+  };
+  SumRec rec = recs[bt.first];                          // set s
+  SumRec rec1 = recs[bt.first + min(1, bt.nsets - 1)];  // set s + 1
+  {
+    const int e = entry_of(rec);
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+      sv[ct] = column_operand(e, ct);
+      bounds_of(rec.pub, ct, pu[ct]);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) w[rt] = row_operand(e, rows[rt]);
+  }
+  // A set that agrees with the one before it in list and bounds (a run of sub-boxes that differ from their
+  // group's list in nothing, say) has the same pieces and the same sums: they are written again from `last`.
+  double last[RT] = {};
+  for (int s = 0; s < bt.nsets; ++s) {
+    const SumRec rec2 = recs[bt.first + min(s + 2, bt.nsets - 1)];  // asked for now, read at the top of the next round
+    const SumTail tl = tails[bt.first + s];                         // (needed at the end of the round)
+    const bool again = s > 0 && (rec.flags & kSumSameAsLast) != 0;
+    const bool ask = (rec1.flags & kSumSameAsLast) == 0;  // the next set needs its operands (the last set's "next" is itself)
+    const int e1 = entry_of(rec1);
+    if (!again) {
+      double x1[RT] = {}, x2[RT] = {}, y1[RT] = {}, y2[RT] = {};
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        if (ct < nct) {
+          double4_t o[RT];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) o[rt] = base[rt][ct];
+          if (rec.dlen > 0) {  // (a set without differences: the shared piece as it is)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) o[rt] = __builtin_amdgcn_mfma_f64_16x16x4f64(sv[ct], w[rt], o[rt], 0, 0, 0);
+          }
+          for (int g = 1; 4 * g < rec.dlen; ++g) {  // (the list is padded with -1 to a multiple of 8)
+            asm volatile("" ::: "memory");  // (keeps the branch a branch: the rare path is not to be run under an empty mask)
+            const int e = tl.delta[4 * g + g4];
+            const double sve = column_operand(e, ct);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) o[rt] = __builtin_amdgcn_mfma_f64_16x16x4f64(sve, row_operand(e, rows[rt]), o[rt], 0, 0, 0);
+          }
+          // Columns whose predicate bounds mirror each other (plb = -pub: every generator of a box star) make xmin1
+          // the mirror image of xmax1 and xmax2 that of xmin2, rounding included (fl(a * (-p) + (-s)) =
+          // -fl(a * p + s)): half of the products are then left out and the two sums negated at the end.
+          if ((rec.flags & kSumMirrored) != 0) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const double v = o[rt][r];
+                x2[rt] = fma(min0(v), pu[ct][r], x2[rt]);
+                y1[rt] = fma(max0(v), pu[ct][r], y1[rt]);
+              }
+          } else {
+            asm volatile("" ::: "memory");
+            double pl[4];
+            bounds_of(tl.plb, ct, pl);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const double v = o[rt][r];
+                const double p = max0(v), q = min0(v);
+                x1[rt] = fma(p, pl[r], x1[rt]);
+                x2[rt] = fma(q, pu[ct][r], x2[rt]);
+                y1[rt] = fma(p, pu[ct][r], y1[rt]);
+                y2[rt] = fma(q, pl[r], y2[rt]);
+              }
+          }
+          if (ask) {
+            sv[ct] = column_operand(e1, ct);
+            bounds_of(rec1.pub, ct, pu[ct]);
+          }
+        }
+      }
+      if (ask) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) w[rt] = row_operand(e1, rows[rt]);
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        // the four lane groups hold different columns of the same rows
+        x2[rt] += __shfl_xor(x2[rt], 16);
+        y1[rt] += __shfl_xor(y1[rt], 16);
+        x2[rt] += __shfl_xor(x2[rt], 32);
+        y1[rt] += __shfl_xor(y1[rt], 32);
+        if ((rec.flags & kSumMirrored) != 0) {  // (0 - s: a sum that is still +0 stays +0, as the left-out additions of -0 would have left it)
+          x1[rt] = 0.0 - y1[rt];
+          y2[rt] = 0.0 - x2[rt];
+        } else {
+          asm volatile("" ::: "memory");
+          x1[rt] += __shfl_xor(x1[rt], 16);
+          y2[rt] += __shfl_xor(y2[rt], 16);
+          x1[rt] += __shfl_xor(x1[rt], 32);
+          y2[rt] += __shfl_xor(y2[rt], 32);
+        }
+        last[rt] = g4 == 0 ? x1[rt] : g4 == 1 ? x2[rt] : g4 == 2 ? y1[rt] : y2[rt];
+      }
+    } else if (ask) {
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        sv[ct] = column_operand(e1, ct);
+        bounds_of(rec1.pub, ct, pu[ct]);
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) w[rt] = row_operand(e1, rows[rt]);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)  // lane group g writes sum g of its sixteen rows
+      if (rt == 0 || two) tl.rpart[(int64_t)cc * 4 * ldo + (int64_t)g4 * ldo + rows[rt]] = last[rt];
+    if (cc == 0 && lane < 16 * RT && (lane < 16 || two)) {  // the centre is the set's own product, bias last
+      double c = tl.cprod[row0 + lane];
+      if (bias != nullptr) c = c + bias[row0 + lane];
+      __builtin_nontemporal_store(c, tl.out + row0 + lane);
+    }
+    rec = rec1;
+    rec1 = rec2;
+  }
+}
+
+template <int RT>
+__global__ __launch_bounds__(256, 2) void delta_sums_kernel(const SumRec* __restrict__ recs, const SumTail* __restrict__ tails,
+                                                            const DeltaBatch* __restrict__ batches, const DeltaOut* __restrict__ sets,
+                                                            const double* __restrict__ A, int64_t lda, int Mp,
+                                                            const double* __restrict__ bias, int64_t ldo) {
+  const DeltaBatch bt = batches[blockIdx.z];
+  const DeltaOut d0 = sets[bt.first];  // (the sets of a batch are of one group: same shared piece, operand and columns)
+  const int cc = blockIdx.x, rb = blockIdx.y;
+  const int j0 = cc * kDeltaCols;
+  if (j0 >= d0.ncols) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int row0 = rb * (64 * RT) + wave * (16 * RT);
+  if (row0 >= Mp) return;           // (no barrier in this kernel)
+  const bool two = RT == 2 && row0 + 16 < Mp;  // the wave's second row tile exists (Mp is a multiple of 16)
+  if (cc == 0 || j0 + kDeltaCols > d0.ncols)
+    delta_sums_body<true, RT>(recs, tails, bt, d0.base, d0.S, d0.lds, d0.ncols, A, lda, Mp, bias, ldo, cc, row0, two);
+  else
+    delta_sums_body<false, RT>(recs, tails, bt, d0.base, d0.S, d0.lds, d0.ncols, A, lda, Mp, bias, ldo, cc, row0, two);
 }
 
 __global__ __launch_bounds__(256) void masked_centres_kernel(const CentreSet* __restrict__ sets, double* __restrict__ Cm, int64_t Kp) {
@@ -794,19 +1065,26 @@ int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp
     a = b;
   }
   if (batches.size() > 65535) NNV_FAIL(NNVHIP_ERR_SHAPE, "array too large for one launch");
-  BufRef tab, btab, rtab;
+  BufRef tab, btab, rtab, ttab;
   NNV_TRY(ctx->upload_table(sets, sizeof(DeltaOut) * count, &tab));
   NNV_TRY(ctx->upload_table(batches.data(), sizeof(DeltaBatch) * batches.size(), &btab));
-  NNV_TRY(ctx->alloc(sizeof(DeltaRec) * (size_t)count, &rtab));
-  hipLaunchKernelGGL(delta_recs_kernel, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, ctx->stream, tab->as<DeltaOut>(),
-                     rtab->as<DeltaRec>(), (int)count);
   const bool timed = ctx->kernel_timing;
-  if (store)
-    NNV_LAUNCH(ctx, timed, delta_tiles_kernel<true>, dim3((unsigned)col_chunks, (unsigned)row_blocks, (unsigned)batches.size()), dim3(256), 0,
-               rtab->as<DeltaRec>(), btab->as<DeltaBatch>(), A, lda, (int)Mp, bias, ldo);
-  else
-    NNV_LAUNCH(ctx, timed, delta_tiles_kernel<false>, dim3((unsigned)col_chunks, (unsigned)row_blocks, (unsigned)batches.size()), dim3(256),
-               0, rtab->as<DeltaRec>(), btab->as<DeltaBatch>(), A, lda, (int)Mp, bias, ldo);
+  const dim3 grid((unsigned)col_chunks, (unsigned)row_blocks, (unsigned)batches.size());
+  if (store) {
+    NNV_TRY(ctx->alloc(sizeof(DeltaRec) * (size_t)count, &rtab));
+    hipLaunchKernelGGL(delta_recs_kernel, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, ctx->stream, tab->as<DeltaOut>(),
+                       rtab->as<DeltaRec>(), (int)count);
+    NNV_LAUNCH(ctx, timed, delta_tiles_kernel, grid, dim3(256), 0, rtab->as<DeltaRec>(), btab->as<DeltaBatch>(), A, lda, (int)Mp, bias, ldo);
+  } else {
+    for (int64_t i = 0; i < count; ++i)
+      if (sets[i].rpart == nullptr || sets[i].ncols < 2) NNV_FAIL(NNVHIP_ERR_ARG, "internal: the pass that stores no matrix is for range sums");
+    NNV_TRY(ctx->alloc(sizeof(SumRec) * (size_t)count, &rtab));
+    NNV_TRY(ctx->alloc(sizeof(SumTail) * (size_t)count, &ttab));
+    hipLaunchKernelGGL(delta_sum_recs_kernel, dim3((unsigned)count), dim3(64), 0, ctx->stream, tab->as<DeltaOut>(), rtab->as<SumRec>(),
+                       ttab->as<SumTail>(), ctx->no_sum_shortcuts ? 0 : 1);
+    NNV_LAUNCH(ctx, timed, delta_sums_kernel<2>, grid, dim3(256), 0, rtab->as<SumRec>(), ttab->as<SumTail>(), btab->as<DeltaBatch>(),
+               tab->as<DeltaOut>(), A, lda, (int)Mp, bias, ldo);
+  }
   NNV_TRY(ctx->kernel_timer_end(timed, 10, bytes));
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;

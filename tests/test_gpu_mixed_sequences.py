@@ -360,6 +360,59 @@ def test_matrices_a_layer_leaves_unwritten_read_the_same_later(nnv, oracle, then
              "relax-star-area")
 
 
+@pytest.mark.parametrize("spread,shapes", [(0.0, 1), (2e-3, 2), (2e-2, 3)])
+def test_shortcuts_of_the_pass_that_sums_unwritten_pieces_change_no_bit(nnv, oracle, spread, shapes):
+    """The pass that sums the pieces of an FC layer's outputs without storing them sums a piece once for a run of sets
+    that agree in their row differences and predicate bounds (at spread 0 all 96 sets do; further out, the sets of
+    one shape that differ from their group's list in nothing or in the same rows), and leaves out half of the
+    products where every predicate's bounds mirror each other (boxes: always).  With the shortcuts switched off -
+    every set summed in full, with both bounds - the layer's bounds and the sets two layers on are the same to
+    the bit."""
+    rs = np.random.RandomState(2400 + shapes)
+    n_in, count, hidden = 200, 96, 400
+    widths = rs.randint(1, 64, size=(n_in, shapes)) / 8192.0
+    half = widths[:, np.arange(count) % shapes]
+    c0 = rs.randint(256, 768, size=(n_in, 1)) / 1024.0
+    centre = c0 + np.round(rs.randn(n_in, count) * spread * 1024.0) / 1024.0
+    lbs, ubs = centre - half, centre + half
+    layers = [_fc(rs, hidden, n_in, 2.0), {"type": "relu"}, _fc(rs, 260, hidden, 2.0), {"type": "relu"}, _fc(rs, 6, 260)]
+    ctx = nnv.default_context()
+    L = nnv.NN.from_config(layers, "shortcuts").Layers
+    opts = ("relax-star-area", [], 1, None, "linprog")
+
+    def run():
+        s = nnv.Star.from_boxes(lbs, ubs)
+        for layer in L[:2]:
+            s = layer.reach(s, *opts)
+        ctx.set_timing(2)
+        try:
+            ctx.kernel_time(10)
+            t = L[2].reach(s, *opts)
+            passes = ctx.kernel_time(10)[1]
+        finally:
+            ctx.set_timing(0)
+        bounds = [tuple(np.asarray(x).copy() for x in a.estimateRanges()) for a in t]
+        u = L[4].reach(L[3].reach(t, *opts), *opts)
+        return passes, bounds, [np.asarray(a.V).copy() for a in u]
+
+    was = ctx.switches.get("no_sum_shortcuts", False)
+    ctx.set_switch("no_sum_shortcuts", False)
+    try:
+        p0, b0, v0 = run()
+        ctx.set_switch("no_sum_shortcuts", True)
+        p1, b1, v1 = run()
+    finally:
+        ctx.set_switch("no_sum_shortcuts", was)
+    for (l0, u0), (l1, u1) in zip(b0, b1):
+        assert np.array_equal(l0, l1) and np.array_equal(u0, u1)
+    for a, b in zip(v0, v1):
+        assert np.array_equal(a, b)
+    if not ctx.switch_is_on("no_row_deltas", "dense_affine", "eager_tail"):
+        assert p0 == 1 and p1 == 1, (p0, p1)
+    _compare(nnv, oracle, layers, nnv.Star.from_boxes(lbs, ubs), [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)],
+             "relax-star-area")
+
+
 @pytest.mark.parametrize("count,half_width", [(1, 0.02), (1, 3.0), (5, 0.3)])
 def test_a_relu_on_top_of_a_relu_lists_its_rows_anew(nnv, oracle, count, half_width):
     """ReLU, ReLU, FC: the second step keeps the rows whose neurons crossed in the first (their range is now

@@ -25,6 +25,7 @@ VARIANTS = {
     "poison_without_conv_boxes": ("poison_pending", "no_conv_boxes"),
     "dense_affine": ("dense_affine",),
     "no_row_deltas": ("no_row_deltas",),
+    "no_sum_shortcuts": ("no_sum_shortcuts",),
 }
 
 
