@@ -387,7 +387,9 @@ def measure(k, args, ctx, exact_steps, extras):
             g["what"] = ("FC layer over an array of sets of one shape: the product over the rows most sets keep is formed once per "
                          "shape; every set's pieces start from it, add the rows in which the set differs and are summed into the "
                          "set's range sums without being stored (written by the same pass on first read); bytes = centre columns "
-                         "and partial sums written; bound by the vector ALUs, not by HBM")
+                         "and partial sums of every set (a set whose row differences and bounds equal its neighbour's is sent "
+                         "to the neighbour's sums, which are then neither formed nor written again); bound by the vector "
+                         "ALUs, not by HBM")
         g["dense_equivalent_flop_per_step"] = gemm_flop
         g["dense_equivalent_achieved_TFLOPs"] = round(gemm_flop * reps / (dlt_ms * 1e-3) / 1e12, 1)
         groups.append((dlt_ms, g))

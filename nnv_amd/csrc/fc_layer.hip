@@ -664,6 +664,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                 }
                 // the sets by group, so that neighbours in the table read the same shared product
                 std::vector<DeltaOut> douts;
+                std::vector<int64_t> dset;  // the set each entry of the table is
                 std::vector<int32_t> dgroup;
                 double dbytes = 0.0;
                 int64_t max_cols = 0;
@@ -702,6 +703,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                   d.dlen = hl[(size_t)(groups + a)];
                   d.ncols = (int32_t)dense[i];
                   douts.push_back(d);
+                  dset.push_back(i);
                   dgroup.push_back((int32_t)g);
                   dbytes += 8.0 * (double)Mp * (double)dense[i];
                   max_cols = std::max<int64_t>(max_cols, dense[i]);
@@ -714,8 +716,15 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                 if (st == NNVHIP_OK && !douts.empty()) {
                   double sums_only = 0.0;  // what the pass then writes: centre columns and partial sums
                   for (const DeltaOut& d : douts) sums_only += 8.0 * (double)Mp + 32.0 * (double)ldo * (double)delta_tile_chunks(d.ncols);
+                  BufRef sums_at;
                   st = launch_delta_tiles(c, Wd, Mp, Mp, bias, ldo, (int64_t)douts.size(), douts.data(), dgroup.data(), max_cols,
-                                          defer ? sums_only : dbytes, !defer);
+                                          defer ? sums_only : dbytes, !defer, &sums_at);
+                  for (size_t k = 0; k < dset.size() && st == NNVHIP_OK && sums_at; ++k) {
+                    nnvhip_star* o = outs[dset[k]];
+                    o->rng_at_buf = sums_at;
+                    o->rng_part_at = sums_at->as<const double*>() + k;
+                    o->rng_chunks_at = tiles_of[dset[k]];
+                  }
                 }
                 if (st == NNVHIP_OK && defer) {
                   Ref<DeltaCall> call = make_ref<DeltaCall>();

@@ -761,29 +761,26 @@ struct SumTail {
   double* out;
   const int32_t* delta;
 };
-// One wave per set.
-__global__ __launch_bounds__(64) void delta_sum_recs_kernel(const DeltaOut* __restrict__ sets, SumRec* __restrict__ recs,
-                                                            SumTail* __restrict__ tails, int shortcuts) {
+// One block per set.
+__global__ __launch_bounds__(256) void delta_sum_recs_kernel(const DeltaOut* __restrict__ sets, SumRec* __restrict__ recs,
+                                                             SumTail* __restrict__ tails, int shortcuts) {
   const int i = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x;
   const DeltaOut d = sets[i];
-  bool mine = true;
-  for (int j = lane; j < d.ncols - 1; j += 64) mine = mine && d.plb[j] == -d.pub[j];
-  const bool mirrored = __all(mine);
-  bool same = i > 0;
-  if (same) {
-    const DeltaOut p = sets[i - 1];
-    same = p.base == d.base && p.S == d.S && p.ncols == d.ncols && p.dlen == d.dlen;
-    if (same) {
-      bool eq = true;
-      for (int t = lane; t < d.dlen; t += 64) eq = eq && p.delta[t] == d.delta[t];
-      for (int j = lane; j < d.ncols - 1; j += 64)  // (to the bit: a zero's sign shows in the sums)
-        eq = eq && __double_as_longlong(p.plb[j]) == __double_as_longlong(d.plb[j]) &&
-             __double_as_longlong(p.pub[j]) == __double_as_longlong(d.pub[j]);
-      same = __all(eq);
-    }
+  const DeltaOut p = sets[max(i - 1, 0)];
+  const bool alike = i > 0 && p.base == d.base && p.S == d.S && p.ncols == d.ncols && p.dlen == d.dlen;  // (the same for all threads)
+  bool mine = true, eq = alike;
+  for (int j = tid; j < d.ncols - 1; j += 256) {
+    const double lo = d.plb[j], hi = d.pub[j];
+    mine = mine && lo == -hi;
+    if (alike)  // (to the bit: a zero's sign shows in the sums)
+      eq = eq && __double_as_longlong(p.plb[j]) == __double_as_longlong(lo) && __double_as_longlong(p.pub[j]) == __double_as_longlong(hi);
   }
-  if (lane == 0) {
+  if (alike)
+    for (int t = tid; t < d.dlen; t += 256) eq = eq && p.delta[t] == d.delta[t];
+  const bool mirrored = __syncthreads_and(mine) != 0;
+  const bool same = __syncthreads_and(eq) != 0;
+  if (tid == 0) {
     SumRec r;
     r.pub = d.pub;
 #pragma unroll
@@ -793,6 +790,18 @@ __global__ __launch_bounds__(64) void delta_sum_recs_kernel(const DeltaOut* __re
     recs[i] = r;
     tails[i] = SumTail{d.plb, d.rpart, d.cprod, d.out, d.delta};
   }
+}
+
+// Where the sums of set i of the table are: its own chunks, or - for a set the pass finds equal to the one before it
+// in its batch - those of the set the run started with (the pass writes them once).
+__global__ __launch_bounds__(256) void delta_sum_alias_kernel(const SumRec* __restrict__ recs, const DeltaOut* __restrict__ sets,
+                                                              const int32_t* __restrict__ batch_first, const double** __restrict__ at,
+                                                              int count) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  int k = i;
+  while (k > batch_first[i] && (recs[k].flags & kSumSameAsLast) != 0) --k;
+  at[i] = sets[k].rpart;
 }
 
 typedef const double __attribute__((address_space(1)))* gdouble_t;  // (a pointer known to be to device memory)
@@ -879,7 +888,8 @@ __device__ __forceinline__ void delta_sums_body(const SumRec* __restrict__ recs,
     for (int rt = 0; rt < RT; ++rt) w[rt] = row_operand(e, rows[rt]);
   }
   // A set that agrees with the one before it in list and bounds (a run of sub-boxes that differ from their
-  // group's list in nothing, say) has the same pieces and the same sums: they are written again from `last`.
+  // group's list in nothing, say) has the same pieces and the same sums: nothing is summed or written for it, and
+  // whoever reads its sums is sent to those of the run's first set (delta_sum_alias_kernel).
   double last[RT] = {};
   for (int s = 0; s < bt.nsets; ++s) {
     const SumRec rec2 = recs[bt.first + min(s + 2, bt.nsets - 1)];  // asked for now, read at the top of the next round
@@ -973,9 +983,11 @@ __device__ __forceinline__ void delta_sums_body(const SumRec* __restrict__ recs,
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) w[rt] = row_operand(e1, rows[rt]);
     }
+    if (!again) {
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)  // lane group g writes sum g of its sixteen rows
-      if (rt == 0 || two) tl.rpart[(int64_t)cc * 4 * ldo + (int64_t)g4 * ldo + rows[rt]] = last[rt];
+      for (int rt = 0; rt < RT; ++rt)  // lane group g writes sum g of its sixteen rows
+        if (rt == 0 || two) tl.rpart[(int64_t)cc * 4 * ldo + (int64_t)g4 * ldo + rows[rt]] = last[rt];
+    }
     if (cc == 0 && lane < 16 * RT && (lane < 16 || two)) {  // the centre is the set's own product, bias last
       double c = tl.cprod[row0 + lane];
       if (bias != nullptr) c = c + bias[row0 + lane];
@@ -1049,7 +1061,8 @@ int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev,
 int delta_tile_chunks(int64_t ncols) { return (int)ceil_div(ncols, kDeltaCols); }
 
 int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp, const double* bias, int64_t ldo, int64_t count,
-                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes, bool store) {
+                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes, bool store, BufRef* sums_at) {
+  if (sums_at) sums_at->reset();
   if (count <= 0 || max_cols <= 0) return NNVHIP_OK;
   if (Mp % 16 || Mp > ldo || count >= (int64_t(1) << 24)) NNV_FAIL(NNVHIP_ERR_SHAPE, "internal: shared-product tiles out of range");
   // batches of neighbouring sets of one group: long enough to make the read of the shared piece small next to the
@@ -1080,8 +1093,17 @@ int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp
       if (sets[i].rpart == nullptr || sets[i].ncols < 2) NNV_FAIL(NNVHIP_ERR_ARG, "internal: the pass that stores no matrix is for range sums");
     NNV_TRY(ctx->alloc(sizeof(SumRec) * (size_t)count, &rtab));
     NNV_TRY(ctx->alloc(sizeof(SumTail) * (size_t)count, &ttab));
-    hipLaunchKernelGGL(delta_sum_recs_kernel, dim3((unsigned)count), dim3(64), 0, ctx->stream, tab->as<DeltaOut>(), rtab->as<SumRec>(),
+    if (sums_at == nullptr) NNV_FAIL(NNVHIP_ERR_ARG, "internal: the pass that stores no matrix says where its sums are");
+    std::vector<int32_t> first((size_t)count);
+    for (const DeltaBatch& b : batches)
+      for (int32_t k = 0; k < b.nsets; ++k) first[(size_t)(b.first + k)] = b.first;
+    BufRef ftab;
+    NNV_TRY(ctx->upload_table(first.data(), sizeof(int32_t) * first.size(), &ftab));
+    NNV_TRY(ctx->alloc(sizeof(const double*) * (size_t)count, sums_at));
+    hipLaunchKernelGGL(delta_sum_recs_kernel, dim3((unsigned)count), dim3(256), 0, ctx->stream, tab->as<DeltaOut>(), rtab->as<SumRec>(),
                        ttab->as<SumTail>(), ctx->no_sum_shortcuts ? 0 : 1);
+    hipLaunchKernelGGL(delta_sum_alias_kernel, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, ctx->stream, rtab->as<SumRec>(),
+                       tab->as<DeltaOut>(), ftab->as<int32_t>(), (*sums_at)->as<const double*>(), (int)count);
     NNV_LAUNCH(ctx, timed, delta_sums_kernel<2>, grid, dim3(256), 0, rtab->as<SumRec>(), ttab->as<SumTail>(), btab->as<DeltaBatch>(),
                tab->as<DeltaOut>(), A, lda, (int)Mp, bias, ldo);
   }

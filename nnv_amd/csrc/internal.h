@@ -477,6 +477,11 @@ struct nnvhip_star {
   const double* rng_part = nullptr;
   int64_t rng_chunks = 0;
   int64_t rng_first_col = 0;
+  // The first rng_chunks_at of those chunks were not written here: they equal another set's, whose address the
+  // device holds at *rng_part_at (the producer found that out on the device; it may be this set's own).
+  nnvhip::BufRef rng_at_buf;
+  const double* const* rng_part_at = nullptr;
+  int64_t rng_chunks_at = 0;
   // The same four sums for the gathered columns of a set in an array, as one matrix product left them
   // (launch_range_sums_mm): two vectors of 2 * ld entries, [xmin1; xmax2] and then [xmax1; xmin2].  They
   // cover columns from rng_first_col on, like the chunks above, and are added after them.
@@ -695,9 +700,11 @@ int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev,
 // (sets: host table, neighbours of one group next to one another; group_of[i]: group of set i of the table; the
 // pass leaves delta_tile_chunks(ncols) chunks of range sums per set)
 // store == false: only the centre columns and the range sums are written (the matrices are left to a later call with
-// store == true and no rpart).
+// store == true and no rpart), and not for every set: sums_at receives a device array with, per set of the table,
+// the address of the chunks that hold its sums - its own rpart, or that of an earlier set with the same sums.
 int launch_delta_tiles(nnvhip_ctx* ctx, const double* A, int64_t lda, int64_t Mp, const double* bias, int64_t ldo, int64_t count,
-                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes, bool store = true);
+                       const DeltaOut* sets, const int32_t* group_of, int64_t max_cols, double bytes, bool store = true,
+                       BufRef* sums_at = nullptr);
 int delta_tile_chunks(int64_t ncols);
 // Cm(r, s) = centre of set s at row r if the set keeps row r, else +0: Cm is Kp x count (ld = Kp), zeroed here.
 struct CentreSet {

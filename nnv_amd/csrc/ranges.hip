@@ -21,6 +21,8 @@ struct RangeDesc {
   const double* part2;  // further chunks2 chunks left by the producer of the trailing columns, or null
   const double* part3;  // sums of gathered columns from the matrix product: [xmin1; xmax2], [xmax1; xmin2] (2*ld each), or null
   int32_t chunks2;
+  int32_t chunks2_at;   // the first chunks2_at of those chunks are read at *part2_at instead (another set's, which are the same)
+  const double* const* part2_at;
   int32_t cchunks;      // > 0: the centre is the sum of cchunks vectors at cpart (ld apart) plus cbias (or
   const double* cpart;  // null), written to cout before it enters lb / ub
   const double* cbias;
@@ -430,13 +432,14 @@ __global__ __launch_bounds__(320) void ranges_final_kernel(const RangeDesc* __re
     }
     if (d.chunks2 > 0) {
       const double* p2 = d.part2 + (int64_t)q * d.ld + r;
+      const double* p2at = d.chunks2_at > 0 ? *d.part2_at + (int64_t)q * d.ld + r : p2;
       for (int c2 = 0; c2 < d.chunks2; c2 += 8) {
         double v[8][R];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
 #pragma unroll
           for (int e = 0; e < R; ++e) v[u][e] = 0.0;
-          if (c2 + u < d.chunks2) load_rows<R>(p2 + (int64_t)(c2 + u) * 4 * d.ld, v[u]);
+          if (c2 + u < d.chunks2) load_rows<R>((c2 + u < d.chunks2_at ? p2at : p2) + (int64_t)(c2 + u) * 4 * d.ld, v[u]);
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u)
@@ -1185,6 +1188,8 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, RangeC
     d.part2 = nullptr;
     d.part3 = nullptr;
     d.chunks2 = 0;
+    d.chunks2_at = 0;
+    d.part2_at = nullptr;
     d.cchunks = 0;
     d.cpart = nullptr;
     d.cbias = nullptr;
@@ -1202,6 +1207,10 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, RangeC
       // the producer of the trailing columns left their sums: scan only the columns before them
       d.part2 = t->rng_chunks > 0 ? t->rng_part : nullptr;
       d.chunks2 = d.part2 ? (int32_t)t->rng_chunks : 0;
+      if (d.part2 && t->rng_part_at != nullptr) {
+        d.part2_at = t->rng_part_at;
+        d.chunks2_at = (int32_t)std::min(t->rng_chunks_at, t->rng_chunks);
+      }
       d.part3 = t->rng_mm;
       d.n = (int32_t)(t->rng_first_col - 1);
       ch = std::max<int64_t>(1, std::min<int64_t>(chunks, ceil_div(std::max<int64_t>(d.n, 1), 64)));
@@ -1282,6 +1291,9 @@ int compute_ranges(nnvhip_ctx* ctx, int64_t count, nnvhip_star* const* s, RangeC
     todo[i]->rng_buf.reset();  // the sums are folded in
     todo[i]->rng_part = nullptr;
     todo[i]->rng_chunks = 0;
+    todo[i]->rng_at_buf.reset();
+    todo[i]->rng_part_at = nullptr;
+    todo[i]->rng_chunks_at = 0;
     todo[i]->rng_mm_buf.reset();
     todo[i]->rng_mm = nullptr;
   }
