@@ -261,6 +261,7 @@ int nnvhip_create(int device, nnvhip_ctx** out) {
   memset((void*)c->mailbox, 0xff, sizeof(int64_t) * nnvhip_ctx::kMailboxSets);  // kMailboxEmpty everywhere
   NNV_HIP_TRY(hipEventCreate(&c->kev0));
   NNV_HIP_TRY(hipEventCreate(&c->kev1));
+  NNV_HIP_TRY(hipEventCreateWithFlags(&c->read_ev, hipEventDisableTiming));
   NNV_TRY(init_static_scratch(c));
   *out = c;
   return NNVHIP_OK;
@@ -283,6 +284,7 @@ int nnvhip_destroy(nnvhip_ctx* c) {
   (void)hipEventDestroy(c->ev1);
   (void)hipEventDestroy(c->kev0);
   (void)hipEventDestroy(c->kev1);
+  if (c->read_ev) (void)hipEventDestroy(c->read_ev);
   (void)hipStreamDestroy(c->stream);
   delete c;
   return NNVHIP_OK;

@@ -573,7 +573,15 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                                         lens->as<int32_t>() + groups);
               // the lengths of the lists come back, and with them the first four entries of each (what the sets are
               // put in order by further down)
+              // While they travel and the host sets the tiles up, the device forms what does not depend on them: the
+              // centres, which are the sets' own - W * (centre masked to the kept rows), all sets in one product
+              // (wasted where the lists turn out too long for this route, next to the much longer work that follows
+              // then).
               std::vector<int32_t> hl((size_t)(groups + nact)), head((size_t)(4 * nact));
+              BufRef cm, cprod;
+              if (st == NNVHIP_OK) st = c->upload_table(csets.data(), sizeof(CentreSet) * csets.size(), &ctab);
+              if (st == NNVHIP_OK) st = c->alloc(sizeof(double) * fc->Kp * nact, &cm);
+              if (st == NNVHIP_OK) st = c->alloc(sizeof(double) * fc->Mp * nact, &cprod);
               if (st == NNVHIP_OK) {
                 void* hp = nullptr;
                 st = c->stage(sizeof(int32_t) * (hl.size() + head.size()), &hp);
@@ -582,10 +590,18 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                   if (hipMemcpyAsync(hp, lens->ptr, sizeof(int32_t) * hl.size(), hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
                       hipMemcpy2DAsync(hh, sizeof(int32_t) * 4, delta->ptr, sizeof(int32_t) * kDeltaCap, sizeof(int32_t) * 4, (size_t)nact,
                                        hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-                      hipStreamSynchronize(c->stream) != hipSuccess) {
+                      hipEventRecord(c->read_ev, c->stream) != hipSuccess) {
                     set_error("HIP error reading the row-difference lists back");
                     st = NNVHIP_ERR_HIP;
-                  } else {
+                  }
+                  if (st == NNVHIP_OK) st = launch_masked_centres(c, nact, ctab->as<CentreSet>(), cm->as<double>(), fc->Kp);
+                  if (st == NNVHIP_OK)
+                    st = launch_gemm(c, Wd, fc->Mp, cm->as<double>(), fc->Kp, cprod->as<double>(), fc->Mp, fc->Mp, nact, fc->Kp, nullptr);
+                  if (st == NNVHIP_OK && hipEventSynchronize(c->read_ev) != hipSuccess) {
+                    set_error("HIP error reading the row-difference lists back");
+                    st = NNVHIP_ERR_HIP;
+                  }
+                  if (st == NNVHIP_OK) {
                     memcpy(hl.data(), hp, sizeof(int32_t) * hl.size());
                     memcpy(head.data(), hh, sizeof(int32_t) * head.size());
                   }
@@ -610,7 +626,7 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                   base_off[(size_t)g] = base_cols;
                   base_cols += shapes[(size_t)g].ldws;
                 }
-                BufRef basebuf, cm, cprod;
+                BufRef basebuf;
                 st = c->alloc(sizeof(double) * Mp * base_cols, &basebuf);
                 std::vector<SegTile> bt_tiles;
                 double base_flop = 0.0;
@@ -640,13 +656,6 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                     st = launch_gemm_seg(c, Wd, Mp, basebuf->as<double>(), Mp, Mp, nullptr, 128, dt->as<SegTile>(), (int64_t)bt_tiles.size(),
                                          base_flop, true);
                 }
-                // the centres, which are the sets' own: W * (centre masked to the kept rows), all sets in one product
-                if (st == NNVHIP_OK) st = c->upload_table(csets.data(), sizeof(CentreSet) * csets.size(), &ctab);
-                if (st == NNVHIP_OK) st = c->alloc(sizeof(double) * fc->Kp * nact, &cm);
-                if (st == NNVHIP_OK) st = c->alloc(sizeof(double) * Mp * nact, &cprod);
-                if (st == NNVHIP_OK) st = launch_masked_centres(c, nact, ctab->as<CentreSet>(), cm->as<double>(), fc->Kp);
-                if (st == NNVHIP_OK)
-                  st = launch_gemm(c, Wd, Mp, cm->as<double>(), fc->Kp, cprod->as<double>(), Mp, Mp, nact, fc->Kp, nullptr);
                 // the sets' tiles, by column tile and group so that tiles that read the same piece of a shared product
                 // run next to one another
                 for (int64_t i = 0; i < count; ++i) {

@@ -377,6 +377,7 @@ struct nnvhip_ctx {
   double last_ms = 0.0;
   // timing of the dominant kernel alone (events directly around its launch), per instantiation group
   hipEvent_t kev0 = nullptr, kev1 = nullptr;
+  hipEvent_t read_ev = nullptr;  // marks a read-back in the stream whose arrival the host waits for while later work runs
   // [0] dense MFMA GEMM (tiles of at least 64 rows), [1] implicit-GEMM convolution (work = flop),
   // [2] estimateRanges column pass, [3] ReLU apply pass, [4] row-wise affine layers (batch
   // normalisation, input normalisation, average pooling, flatten), [5] gather of W's columns for the
