@@ -375,15 +375,21 @@ def measure(k, args, ctx, exact_steps, extras):
         # outputs that start from a product shared by the sets of a group and add only the rows in which a set differs
         # from the group's list: a block reads its piece of the shared product (from cache), adds a few rank-one
         # terms and writes itself out - bound by the bytes of output it writes
-        g = hbm_roofline("delta_tiles_kernel", dlt_ms, dlt_launches, dlt_bytes)
+        unwritten = not ctx.eager_columns and not args.dense and not args.written   # (the pass is then another kernel)
+        g = hbm_roofline("delta_sums_kernel" if unwritten else "delta_tiles_kernel", dlt_ms, dlt_launches, dlt_bytes)
         g["what"] = ("FC layer over an array of sets of one shape: the product over the rows most sets keep is formed once per "
                      "shape, every set's tiles start from it and contract over the rows in which the set differs; bytes = the "
                      "output matrices written")
-        if not ctx.eager_columns and not args.dense and not args.written:
+        if unwritten:
             # nobody on the way to the next layer reads these matrices (the ReLU step takes the range sums): the pass forms
-            # and sums every piece and stores the centre columns and the partial sums only - what it then moves is a small
-            # part of what it computes, and the vector ALUs bound it, not HBM (the fraction of the HBM peak says so)
+            # and sums every piece (one fp64 MFMA per 16 x 16 outputs, which runs at the vector unit's fp64 rate) and stores
+            # the centre columns and the partial sums only - what it then moves is a small part of what it computes, and
+            # the fp64 units bound it, not HBM (the fraction of the HBM peak says so)
             g["matrices_left_unwritten"] = True
+            # the library counts the sums of every set; a set equal to its neighbour in row differences and bounds is
+            # neither summed nor written again (decided on the device), so fewer bytes move - the counter table in
+            # profiles/ has the figure
+            g["bytes_are_an_upper_bound"] = True
             g["what"] = ("FC layer over an array of sets of one shape: the product over the rows most sets keep is formed once per "
                          "shape; every set's pieces start from it, add the rows in which the set differs and are summed into the "
                          "set's range sums without being stored (written by the same pass on first read); bytes = centre columns "
