@@ -1026,10 +1026,13 @@ static int ensure_split_weights(nnvhip_ctx* ctx, const nnvhip_fc* fc) {
 
 // [W+; W-] * (the odd columns of X) into the odd column pairs of *out, whose even ones ([xmin1; xmax2], products with
 // a zero vector) are +0: what the product leaves when every gathered column has lower predicate bound zero.
-static int range_sums_upper_half(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t nu, const BufRef& X, BufRef* out) {
+// (zeroed: the caller's own kernel has already filled the even column pairs of *out, which it allocated)
+static int range_sums_upper_half(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t nu, const BufRef& X, BufRef* out, bool zeroed = false) {
   const int64_t Mp = fc->Mp, Kp = fc->Kp;
-  NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * nu, out));
-  NNV_HIP_TRY(hipMemsetAsync((*out)->ptr, 0, sizeof(double) * 2 * Mp * 2 * nu, ctx->stream));
+  if (!zeroed) {
+    NNV_TRY(ctx->alloc(sizeof(double) * 2 * Mp * 2 * nu, out));
+    NNV_HIP_TRY(hipMemsetAsync((*out)->ptr, 0, sizeof(double) * 2 * Mp * 2 * nu, ctx->stream));
+  }
   std::vector<int32_t> odd((size_t)nu);
   for (int64_t k = 0; k < nu; ++k) odd[(size_t)k] = (int32_t)(2 * k + 1);
   BufRef cmap;
@@ -1041,11 +1044,15 @@ static int range_sums_upper_half(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t n
                      nullptr, &rows);
 }
 
-// Column 2i+1 of X (Kp rows): ub where the neuron crosses, zero elsewhere (column 2i is not read).
-__global__ __launch_bounds__(256) void crossing_ub_vectors_kernel(const AheadSet* __restrict__ table, double* __restrict__ X, int Kp, int N) {
+// Column 2i+1 of X (Kp rows): ub where the neuron crosses, zero elsewhere (column 2i is not read).  And column pair
+// 2i of the product to come (2 * Mp2 entries, Mp2 = the product's rows), which no tile of it writes: +0.
+__global__ __launch_bounds__(256) void crossing_ub_vectors_kernel(const AheadSet* __restrict__ table, double* __restrict__ X, int Kp, int N,
+                                                                  double* __restrict__ prod, int64_t Mp2) {
   const AheadSet d = table[blockIdx.x];
   double* xb = X + ((int64_t)2 * blockIdx.x + 1) * Kp;
   for (int r = threadIdx.x; r < Kp; r += 256) xb[r] = (r < N && d.cls[r] >= 0) ? d.ub[r] : 0.0;
+  double2* z = reinterpret_cast<double2*>(prod + (int64_t)2 * blockIdx.x * Mp2);  // (Mp2 is even, the buffer 256-byte aligned)
+  for (int64_t r = threadIdx.x; r < Mp2 / 2; r += 256) z[r] = make_double2(0.0, 0.0);
 }
 
 int launch_range_sums_mm_ahead(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const AheadSet* sets, int64_t N, BufRef* out) {
@@ -1054,11 +1061,12 @@ int launch_range_sums_mm_ahead(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t cou
   NNV_TRY(ensure_split_weights(ctx, fc));
   BufRef X, tab;
   NNV_TRY(ctx->alloc(sizeof(double) * Kp * 2 * count, &X));
-  NNV_TRY(ctx->upload(sets, sizeof(AheadSet) * count, &tab));
+  NNV_TRY(ctx->alloc(sizeof(double) * 2 * fc->Mp * 2 * count, out));
+  NNV_TRY(ctx->upload_table(sets, sizeof(AheadSet) * count, &tab));
   hipLaunchKernelGGL(crossing_ub_vectors_kernel, dim3((unsigned)count), dim3(256), 0, ctx->stream, tab->as<AheadSet>(), X->as<double>(),
-                     (int)Kp, (int)N);
+                     (int)Kp, (int)N, (*out)->as<double>(), 2 * fc->Mp);
   NNV_HIP_TRY(hipGetLastError());
-  return range_sums_upper_half(ctx, fc, count, X, out);
+  return range_sums_upper_half(ctx, fc, count, X, out, true);
 }
 
 int launch_range_sums_mm(nnvhip_ctx* ctx, const nnvhip_fc* fc, int64_t count, const GatherSet* sets, BufRef* out,
