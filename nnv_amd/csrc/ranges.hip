@@ -581,7 +581,10 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
         double2 o;
         o.x = __dadd_rn(0.0, __dmul_rn(v[u].x, sc[u]));
         o.y = __dadd_rn(0.0, __dmul_rn(v[u].y, sc[u]));
-        if (!d.lazy) *reinterpret_cast<double2*>(d.out + r0 + (int64_t)j * a.ldout) = o;
+        if (!d.lazy) {  // (streaming store: nothing here reads the column again)
+          typedef double dd2 __attribute__((ext_vector_type(2)));
+          __builtin_nontemporal_store(dd2{o.x, o.y}, reinterpret_cast<dd2*>(d.out + r0 + (int64_t)j * a.ldout));
+        }
         if (part != nullptr) {
           const double pl = d.plb[j], pu = d.pub[j];
           const double px = fmax(o.x, 0.0), nx = fmin(o.x, 0.0);

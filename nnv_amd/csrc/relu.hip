@@ -454,11 +454,13 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
   // each wave takes 4 consecutive columns per step; the 4 loads are issued before any is used
   for (int jb = j0 + 4 * wcol; jb < j1; jb += 4 * col_waves) {
     double2 v[4];
+    int hot[4];  // the neuron of an appended column (asked for together, ahead of the stores)
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = jb + u;
       v[u] = make_double2(0.0, 0.0);
       if (need && j < j1 && j < d.ncols_in) v[u] = *reinterpret_cast<const double2*>(d.Vin + r0 + (int64_t)j * d.ld);
+      hot[u] = (j >= d.ncols_in && j < j1) ? d.cross_idx[j - d.ncols_in] : -1;
     }
     if (!active) continue;
 #pragma unroll
@@ -470,11 +472,12 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
         o.x = cx == kKeep ? v[u].x : 0.0;  // V1(map,:) = 0
         o.y = cy == kKeep ? v[u].y : 0.0;
       } else {
-        const int neuron = d.cross_idx[j - d.ncols_in];
+        const int neuron = hot[u];
         o.x = r0 == neuron ? 1.0 : 0.0;  // V2(index(i), i) = 1
         o.y = r0 + 1 == neuron ? 1.0 : 0.0;
       }
-      *reinterpret_cast<double2*>(d.Vout + r0 + (int64_t)j * d.ld) = o;
+      typedef double dd2 __attribute__((ext_vector_type(2)));  // (streaming store: the pass does not read its output)
+      __builtin_nontemporal_store(dd2{o.x, o.y}, reinterpret_cast<dd2*>(d.Vout + r0 + (int64_t)j * d.ld));
     }
   }
 }
