@@ -145,6 +145,56 @@ def test_config5_full_batched_equals_single(nnv):
     del big
 
 
+def test_config5_full_shortcuts_of_the_summing_pass_change_no_bit(nnv):
+    """Config 5 at full size (batches of sixteen sets per block of the pass that sums the second FC layer's unwritten
+    pieces, runs of equal sets across and inside batches) with the pass's shortcuts on and off, and a second time
+    with them on: every ReLU step's counts and crossing lists, all output matrices and all output bounds are the same
+    to the bit; and the layer's matrices, written when first read after the reach, equal those of the mode that
+    writes them inside the call."""
+    cfg = make_config(5)
+    stars, _ = input_sets(cfg)
+    opts = {"reachMethod": "relax-star-area", "relaxFactor": 1}
+    ctx = nnv.default_context()
+    from nnv_amd import _lib
+    import ctypes as C
+
+    def run(read=()):
+        net = nnv.NN.from_config(cfg["layers"], cfg["name"])
+        outs = net.reach(stars, opts)
+        N = outs[0].dim
+        lb, ub = np.empty((N, 1024), order="F"), np.empty((N, 1024), order="F")
+        arr = (C.c_void_p * 1024)(*[s._h.h for s in outs])
+        _lib.check(ctx.lib.nnvhip_estimate_ranges_batch(ctx.handle, 1024, arr, _lib.ptr(lb), _lib.ptr(ub)))
+        infos = [[net.reachSet[li][i].relu_info() for i in (0, 255, 256, 700, 1023)]
+                 for li, L in enumerate(cfg["layers"]) if L["type"] == "relu"]
+        Vs = [np.asarray(outs[i].V).copy() for i in (0, 15, 16, 511, 1023)]
+        mats = [np.asarray(net.reachSet[2][i].V).copy() for i in read]   # the second FC layer's sets
+        return lb, ub, infos, Vs, mats
+
+    was = {nm: ctx.switches.get(nm, False) for nm in ("no_sum_shortcuts", "eager_cols")}
+    try:
+        ctx.set_switch("no_sum_shortcuts", False)
+        a = run(read=(1023, 0, 300))
+        ctx.set_switch("no_sum_shortcuts", True)
+        b = run()
+        ctx.set_switch("no_sum_shortcuts", False)
+        c = run()
+        ctx.set_switch("eager_cols", True)
+        e = run(read=(1023, 0, 300))
+    finally:
+        for nm, v in was.items():
+            ctx.set_switch(nm, v)
+    for x in (b, c):
+        assert np.array_equal(a[0], x[0]) and np.array_equal(a[1], x[1])
+        for ia, ix in zip(a[2], x[2]):
+            for p, q in zip(ia, ix):
+                assert p[0] == q[0] and np.array_equal(p[1], q[1])
+        for p, q in zip(a[3], x[3]):
+            assert np.array_equal(p, q)
+    for p, q in zip(a[4], e[4]):
+        assert np.array_equal(p, q)
+
+
 def test_reach_is_deterministic(nnv):
     cfg = make_config(2)
     net = nnv.NN.from_config(cfg["layers"])
