@@ -565,12 +565,12 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
               if (st == NNVHIP_OK) st = c->upload_table(gsize.data(), sizeof(int32_t) * gsize.size(), &gtab);
               if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * groups * rowsK, &votes);
               if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * groups * rows_pad, &common);
-              if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * (groups + nact), &lens);  // ncommon, then dlen
+              if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * (groups + 5 * nact), &lens);  // ncommon, dlen, first entries
               if (st == NNVHIP_OK) st = c->alloc(sizeof(int32_t) * nact * kDeltaCap, &delta);
               if (st == NNVHIP_OK)
                 st = launch_delta_lists(c, nact, dtab->as<DeltaSet>(), groups, gtab->as<int32_t>(), rowsK, rows_pad, kDeltaCap,
                                         votes->as<int32_t>(), common->as<int32_t>(), lens->as<int32_t>(), delta->as<int32_t>(),
-                                        lens->as<int32_t>() + groups);
+                                        lens->as<int32_t>() + groups, lens->as<int32_t>() + groups + nact);
               // the lengths of the lists come back, and with them the first four entries of each (what the sets are
               // put in order by further down)
               // While they travel and the host sets the tiles up, the device forms what does not depend on them: the
@@ -587,9 +587,8 @@ int nnvhip_affine_fc(nnvhip_ctx* c, const nnvhip_fc* fc, int64_t count, nnvhip_s
                 st = c->stage(sizeof(int32_t) * (hl.size() + head.size()), &hp);
                 if (st == NNVHIP_OK) {
                   int32_t* hh = static_cast<int32_t*>(hp) + hl.size();
-                  if (hipMemcpyAsync(hp, lens->ptr, sizeof(int32_t) * hl.size(), hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
-                      hipMemcpy2DAsync(hh, sizeof(int32_t) * 4, delta->ptr, sizeof(int32_t) * kDeltaCap, sizeof(int32_t) * 4, (size_t)nact,
-                                       hipMemcpyDeviceToHost, c->stream) != hipSuccess ||
+                  if (hipMemcpyAsync(hp, lens->ptr, sizeof(int32_t) * (hl.size() + head.size()), hipMemcpyDeviceToHost, c->stream) !=
+                          hipSuccess ||
                       hipEventRecord(c->read_ev, c->stream) != hipSuccess) {
                     set_error("HIP error reading the row-difference lists back");
                     st = NNVHIP_ERR_HIP;

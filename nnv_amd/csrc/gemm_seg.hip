@@ -491,7 +491,8 @@ __global__ __launch_bounds__(1024) void common_rows_kernel(const int32_t* __rest
 // one block per set: the rows in which the set's list differs from its group's majority list
 __global__ __launch_bounds__(1024) void delta_rows_kernel(const DeltaSet* __restrict__ sets, const int32_t* __restrict__ votes,
                                                           const int32_t* __restrict__ group_size, int rows, int cap,
-                                                          int32_t* __restrict__ delta, int32_t* __restrict__ dlen) {
+                                                          int32_t* __restrict__ delta, int32_t* __restrict__ dlen,
+                                                          int32_t* __restrict__ head) {
   extern __shared__ unsigned keptbits[];  // one bit per row
   const DeltaSet d = sets[blockIdx.x];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -541,6 +542,8 @@ __global__ __launch_bounds__(1024) void delta_rows_kernel(const DeltaSet* __rest
   const int npad = (n + kSegKS - 1) / kSegKS * kSegKS;
   for (int t = n + tid; t < npad; t += 1024) out[t] = -1;
   if (tid == 0) dlen[blockIdx.x] = n;
+  // the first four entries once more, next to the lengths: what the host reads back with them
+  if (tid < 4) head[4 * blockIdx.x + tid] = tid < n ? out[tid] : -1;
 }
 
 // Sets that start from their group's shared product (DeltaOut).  A block takes 128 rows x 64 columns of that product
@@ -1042,7 +1045,7 @@ int launch_scaled_rows(nnvhip_ctx* ctx, const ScaledRows& a) {
 
 int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev, int groups, const int32_t* group_size_dev,
                        int64_t rows, int64_t rows_pad, int cap, int32_t* votes, int32_t* common, int32_t* ncommon, int32_t* delta,
-                       int32_t* dlen) {
+                       int32_t* dlen, int32_t* head) {
   if (count <= 0 || groups <= 0 || rows <= 0 || rows >= (int64_t(1) << 30) || cap % kSegKS != 0 || rows_pad % 16 != 0 ||
       rows_pad < rows)
     NNV_FAIL(NNVHIP_ERR_ARG, "internal: row-difference lists out of range");
@@ -1053,7 +1056,7 @@ int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev,
   hipLaunchKernelGGL(common_rows_kernel, dim3((unsigned)groups), dim3(1024), 0, ctx->stream, votes, group_size_dev, (int)rows,
                      (int)rows_pad, common, ncommon);
   hipLaunchKernelGGL(delta_rows_kernel, dim3((unsigned)count), dim3(1024), bits, ctx->stream, sets_dev, votes, group_size_dev, (int)rows,
-                     cap, delta, dlen);
+                     cap, delta, dlen, head);
   NNV_HIP_TRY(hipGetLastError());
   return NNVHIP_OK;
 }

@@ -693,7 +693,8 @@ struct DeltaSet {
 };
 int launch_delta_lists(nnvhip_ctx* ctx, int64_t count, const DeltaSet* sets_dev, int groups, const int32_t* group_size_dev,
                        int64_t rows, int64_t rows_pad, int cap, int32_t* votes /* groups x rows, scratch */, int32_t* common /* groups x rows_pad */,
-                       int32_t* ncommon, int32_t* delta /* count x cap */, int32_t* dlen);
+                       int32_t* ncommon, int32_t* delta /* count x cap */, int32_t* dlen,
+                       int32_t* head /* count x 4: the first entries of every list, -1 where there is none */);
 // The output of one set that starts from its group's shared product: out(:, j) = base(:, j) + sum over the set's
 // row differences of (+/-) A(:, r) * S(r, j) for j < ncols, the centre column (j = 0) replaced by cprod (+ bias), and
 // the four Star.estimateRanges partial sums of every piece of delta_tile_chunks' columns in rpart ([piece][4][ldo]).  A streaming
