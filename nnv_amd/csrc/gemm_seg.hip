@@ -605,9 +605,9 @@ __global__ __launch_bounds__(256) void delta_tiles_kernel(const DeltaRec* __rest
   // those rows and the columns' predicate bounds is read by lane u (mod 16) for column u and handed round by lane
   // reads: one load each instead of a scalar load per column and value.  The look-ups run ahead of the arithmetic:
   // while set s is worked on, the operands of set s + 1 are in flight and the record of set s + 2 is on its way, so
-  // that no set waits for its two dependent trips to memory (the storing pass: 1.49 -> 1.39 ms for config 5's
-  // 6.7 GB; the pass that stores nothing is bound by its instruction count - 420 vector and 270 scalar instructions
-  // per set and wave, the vector unit busy half of the time - and gains nothing from it: 0.58 ms either way).
+  // that no set waits for its two dependent trips to memory (1.49 -> 1.22-1.39 ms for 6.7 GB of output; with the
+  // stores left out the same loop is bound by its instruction count - 420 vector and 270 scalar instructions per
+  // set and wave - which is why the pass that stores nothing is a kernel of its own, further down).
   struct SetOps {
     double2_t w4[4];
     double sv4[4];
