@@ -642,6 +642,7 @@ __global__ __launch_bounds__(64 * kRangeWaves) void gather_columns_kernel(const 
 template <int HL>
 __global__ __launch_bounds__(256) void gather_skinny_kernel(const GatherSet* __restrict__ table, GatherSet one, GatherArgs a) {
   constexpr int CPW = 64 / HL;  // columns per wave and step
+  typedef double dd2 __attribute__((ext_vector_type(2)));  // (streaming stores: nothing here reads a column again)
   const GatherSet d = table ? table[blockIdx.z] : one;
   const int chunk = blockIdx.y;
   const int j0 = chunk * a.cols_per_chunk;
@@ -661,7 +662,7 @@ __global__ __launch_bounds__(256) void gather_skinny_kernel(const GatherSet* __r
         o.x = __dadd_rn(0.0, d.bias[r0]);
         o.y = __dadd_rn(0.0, d.bias[r0 + 1]);
       }
-      *reinterpret_cast<double2*>(d.fill + r0 + (int64_t)j * a.ldout) = o;
+      __builtin_nontemporal_store(dd2{o.x, o.y}, reinterpret_cast<dd2*>(d.fill + r0 + (int64_t)j * a.ldout));
     }
   }
   double2 xmin1 = {0, 0}, xmin2 = {0, 0}, xmax1 = {0, 0}, xmax2 = {0, 0};
@@ -686,7 +687,7 @@ __global__ __launch_bounds__(256) void gather_skinny_kernel(const GatherSet* __r
       double2 o;
       o.x = __dadd_rn(0.0, __dmul_rn(v[u].x, sc[u]));
       o.y = __dadd_rn(0.0, __dmul_rn(v[u].y, sc[u]));
-      *reinterpret_cast<double2*>(d.out + r0 + (int64_t)j * a.ldout) = o;
+      __builtin_nontemporal_store(dd2{o.x, o.y}, reinterpret_cast<dd2*>(d.out + r0 + (int64_t)j * a.ldout));
       if (part != nullptr) {
         const double pl = d.plb[j], pu = d.pub[j];
         const double px = fmax(o.x, 0.0), nx = fmin(o.x, 0.0);
