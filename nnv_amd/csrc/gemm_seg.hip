@@ -820,6 +820,19 @@ __device__ __forceinline__ double min0(double v) {
   return r;
 }
 
+// Two sums over the halves of a wave at once: lanes 0-31 get a(l) + a(l + 32), lanes 32-63 get b(l - 32) + b(l).
+__device__ __forceinline__ double fold32(double a, double b) {
+  const auto lo = __builtin_amdgcn_permlane32_swap((unsigned)__double2loint(a), (unsigned)__double2loint(b), false, false);
+  const auto hi = __builtin_amdgcn_permlane32_swap((unsigned)__double2hiint(a), (unsigned)__double2hiint(b), false, false);
+  return __hiloint2double((int)hi[0], (int)lo[0]) + __hiloint2double((int)hi[1], (int)lo[1]);
+}
+// ... and over neighbouring 16-lane rows: rows 0 and 2 get c.row0 + c.row1 and c.row2 + c.row3, rows 1 and 3 the same of d.
+__device__ __forceinline__ double fold16(double c, double d) {
+  const auto lo = __builtin_amdgcn_permlane16_swap((unsigned)__double2loint(c), (unsigned)__double2loint(d), false, false);
+  const auto hi = __builtin_amdgcn_permlane16_swap((unsigned)__double2hiint(c), (unsigned)__double2hiint(d), false, false);
+  return __hiloint2double((int)hi[0], (int)lo[0]) + __hiloint2double((int)hi[1], (int)lo[1]);
+}
+
 // EDGE: the block's columns include column 0 (the centre, which is the set's own and enters no sum) or columns past
 // the last; their entries of the shared piece and of the shared operand are made zero, so that they add nothing.
 template <bool EDGE, int RT>
@@ -893,7 +906,6 @@ __device__ __forceinline__ void delta_sums_body(const SumRec* __restrict__ recs,
   // A set that agrees with the one before it in list and bounds (a run of sub-boxes that differ from their
   // group's list in nothing, say) has the same pieces and the same sums: nothing is summed or written for it, and
   // whoever reads its sums is sent to those of the run's first set (delta_sum_alias_kernel).
-  double last[RT] = {};
   for (int s = 0; s < bt.nsets; ++s) {
     const SumRec rec2 = recs[bt.first + min(s + 2, bt.nsets - 1)];  // asked for now, read at the top of the next round
     const SumTail tl = tails[bt.first + s];                         // (needed at the end of the round)
@@ -957,24 +969,29 @@ __device__ __forceinline__ void delta_sums_body(const SumRec* __restrict__ recs,
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) w[rt] = row_operand(e1, rows[rt]);
       }
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        // the four lane groups hold different columns of the same rows
-        x2[rt] += __shfl_xor(x2[rt], 16);
-        y1[rt] += __shfl_xor(y1[rt], 16);
-        x2[rt] += __shfl_xor(x2[rt], 32);
-        y1[rt] += __shfl_xor(y1[rt], 32);
-        if ((rec.flags & kSumMirrored) != 0) {  // (0 - s: a sum that is still +0 stays +0, as the left-out additions of -0 would have left it)
-          x1[rt] = 0.0 - y1[rt];
-          y2[rt] = 0.0 - x2[rt];
-        } else {
-          asm volatile("" ::: "memory");
-          x1[rt] += __shfl_xor(x1[rt], 16);
-          y2[rt] += __shfl_xor(y2[rt], 16);
-          x1[rt] += __shfl_xor(x1[rt], 32);
-          y2[rt] += __shfl_xor(y2[rt], 32);
+      // The four lane groups hold different columns of the same rows.  Two lane swaps add them up, two sums at a
+      // time: fold32 leaves a(l) + a(l + 32) in the lower half of the wave and the same of b in the upper half,
+      // fold16 then adds neighbouring 16-lane rows of two such values - lane row 0 and 1 end up with the finished
+      // first sum of row tile 0 and 1, lane row 2 and 3 with the second sum (every sum as (g0 + g2) + (g1 + g3)).
+      static_assert(RT == 2, "the lane rows of the finished sums are dealt to two row tiles");
+      const int tile = g4 & 1, second = g4 >> 1;
+      double* const dst = tl.rpart + (int64_t)cc * 4 * ldo + rows[tile];
+      if ((rec.flags & kSumMirrored) != 0) {
+        // lane rows 0, 1: xmin2; 2, 3: xmax1; the mirror images go out beside them (0 - s: a sum that is still +0
+        // stays +0, as the left-out additions of -0 would have left it)
+        const double v = fold16(fold32(x2[0], y1[0]), fold32(x2[1], y1[1]));
+        if (tile == 0 || two) {
+          dst[(second ? 2 : 1) * ldo] = v;
+          dst[(second ? 0 : 3) * ldo] = 0.0 - v;
         }
-        last[rt] = g4 == 0 ? x1[rt] : g4 == 1 ? x2[rt] : g4 == 2 ? y1[rt] : y2[rt];
+      } else {
+        asm volatile("" ::: "memory");
+        const double va = fold16(fold32(x1[0], x2[0]), fold32(x1[1], x2[1]));  // lane rows 0, 1: xmin1; 2, 3: xmin2
+        const double vb = fold16(fold32(y1[0], y2[0]), fold32(y1[1], y2[1]));  // xmax1; xmax2
+        if (tile == 0 || two) {
+          dst[(second ? 1 : 0) * ldo] = va;
+          dst[(second ? 3 : 2) * ldo] = vb;
+        }
       }
     } else if (ask) {
       asm volatile("" ::: "memory");
@@ -985,11 +1002,6 @@ __device__ __forceinline__ void delta_sums_body(const SumRec* __restrict__ recs,
       }
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) w[rt] = row_operand(e1, rows[rt]);
-    }
-    if (!again) {
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)  // lane group g writes sum g of its sixteen rows
-        if (rt == 0 || two) tl.rpart[(int64_t)cc * 4 * ldo + (int64_t)g4 * ldo + rows[rt]] = last[rt];
     }
     if (cc == 0 && lane < 16 * RT && (lane < 16 || two)) {  // the centre is the set's own product, bias last
       double c = tl.cprod[row0 + lane];
