@@ -665,6 +665,9 @@ int reach_small_chain(nnvhip_ctx* c, int64_t n_layers, const int32_t* kind, cons
         o->pbuf = prev->pbuf;
         o->plb = prev->plb;
         o->pub = prev->pub;
+        o->ptails = prev->ptails;
+        o->pslot = prev->pslot;
+        o->pcap = prev->pcap;
         o->cons = prev->cons;
         o->has_zono = prev->has_zono;
         o->rbuf = arena;

@@ -55,6 +55,9 @@ int nnvhip::make_affine_outputs(nnvhip_ctx* c, int64_t count, nnvhip_star* const
     o->pbuf = in[i]->pbuf;
     o->plb = in[i]->plb;
     o->pub = in[i]->pub;
+    o->ptails = in[i]->ptails;
+    o->pslot = in[i]->pslot;
+    o->pcap = in[i]->pcap;
     o->cons = in[i]->cons;
     off += in[i]->n + 1;
     outs->push_back(o);

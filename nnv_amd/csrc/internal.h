@@ -172,6 +172,14 @@ struct DeltaOut {
   int32_t dlen;
   int32_t ncols;
 };
+// Predicate-bound arrays with room behind their last entry (one record per ReLU call that allocated such arrays,
+// shared by the handles that point into them).  used[slot] = entries of the slot's arrays that are taken: a ReLU step
+// whose input ends exactly there, and whose worst case fits the room, appends its new predicates' bounds in place
+// instead of copying the old ones into arrays of its own (the input keeps reading its first n entries).
+struct PredTails {
+  int64_t ref_count = 0;
+  std::vector<int64_t> used;
+};
 // A call of the shared-product route of an FC layer over an array whose output matrices have not been written: the
 // range sums and the centre columns are in place, the dense columns are what `outs` says and are written - for all
 // sets of the call at once - when somebody first reads any of them (write_pending_columns).  The buffers the
@@ -442,6 +450,8 @@ struct nnvhip_star {
   nnvhip::BufRef pbuf;
   double* plb = nullptr;
   double* pub = nullptr;
+  nnvhip::Ref<nnvhip::PredTails> ptails;  // not null: plb / pub have room for pcap entries each (see PredTails)
+  int64_t pslot = 0, pcap = 0;
   nnvhip::ConsRef cons;
   // cached estimateRanges result
   nnvhip::BufRef rbuf;

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(1024) void relu_classify_kernel(const ReluDesc* __r
   const double u_first = tid < d.N ? d.ub[tid] : 1.0;
   // ... and while they travel, the bounds of the predicates the set already has are copied (new_pred_lb =
   // [plb; ...], new_pred_ub = [pub; ...]): nothing of that depends on the classification
-  if (d.write_bounds) {
+  if (d.write_bounds && d.plb_out != d.plb_in) {  // (in place: the old bounds are where they belong)
     const int n_in = d.ncols_in - 1;
     for (int jb = tid; jb < n_in; jb += 4096) {
       double a[4], b[4];
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(1024) void relu_sort_small_kernel(const ReluDesc* _
   const int m = d.m;
   const int tid = threadIdx.x;
   const int n_in = d.ncols_in - 1;
-  if (flags & kRankOldBounds) {
+  if ((flags & kRankOldBounds) && d.plb_out != d.plb_in) {
     for (int j = tid; j < n_in; j += 1024) {
       d.plb_out[j] = d.plb_in[j];
       d.pub_out[j] = d.pub_in[j];
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(256) void relu_rank_kernel(const ReluDesc* __restri
   const int m = (flags & kRankCountOnDevice) ? d.counts[0] : d.m;
   const int tid = threadIdx.x;
   const int n_in = d.ncols_in - 1;
-  if (flags & kRankOldBounds) {
+  if ((flags & kRankOldBounds) && d.plb_out != d.plb_in) {
     for (int j = blockIdx.x * 256 + tid; j < n_in; j += gridDim.x * 256) {
       d.plb_out[j] = d.plb_in[j];
       d.pub_out[j] = d.pub_in[j];
@@ -426,7 +426,7 @@ __global__ __launch_bounds__(64 * kApplyWaves) void relu_apply_kernel(const Relu
   if (blockIdx.x == 0 && d.write_bounds) {
     for (int j = j0 + (int)threadIdx.x; j < j1; j += 64 * kApplyWaves) {
       if (j < d.ncols_in) {
-        if (j >= 1) {
+        if (j >= 1 && d.plb_out != d.plb_in) {
           d.plb_out[j - 1] = d.plb_in[j - 1];
           d.pub_out[j - 1] = d.pub_in[j - 1];
         }
@@ -703,16 +703,28 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   const bool early_rank = lazy_rows && sorted && N > kOneBlockN;
   const bool fold_bounds = lazy_rows && (N <= kOneBlockN || early_rank);
   BufRef pred_buf, lbub_buf;
-  std::vector<int64_t> pred_off(count), lbub_off(count);
+  std::vector<int64_t> pred_off(count), lbub_off(count), pred_cap(count, 0);
+  // (sets whose predicate-bound arrays end where the set ends and have room for this step's worst case: the new
+  // bounds go behind the old ones, in place; the others get arrays of their own, with room for the steps to come)
+  std::vector<char> in_place(count, 0);
+  Ref<PredTails> tails;
   const int64_t ldr_max = round_up(N, kLdAlign);
   if (fold_bounds) {
     int64_t total_pred = 0;
     for (int64_t i = 0; i < count; ++i) {
-      pred_off[i] = total_pred;
+      const nnvhip_star* s = in[i];
       lbub_off[i] = 2 * ldr_max * i;
-      total_pred += 2 * round_up(in[i]->n + N, kLdAlign);
+      in_place[i] = s->ptails && s->ptails->used[(size_t)s->pslot] == s->n && s->n + N <= s->pcap;
+      if (in_place[i]) continue;
+      pred_off[i] = total_pred;
+      pred_cap[i] = round_up(s->n + 4 * N, kLdAlign);
+      total_pred += 2 * pred_cap[i];
     }
-    NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
+    if (total_pred > 0) {
+      NNV_TRY(ctx->alloc(sizeof(double) * total_pred, &pred_buf));
+      tails = make_ref<PredTails>();
+      tails->used.assign((size_t)count, -1);
+    }
     NNV_TRY(ctx->alloc(sizeof(double) * 2 * ldr_max * count, &lbub_buf));
   }
   // crossing lists of all sets in one buffer (they become the constraint nodes' index lists)
@@ -728,8 +740,8 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
     ReluDesc& d = descs[i];
     d = ReluDesc{};
     if (fold_bounds) {
-      d.plb_out = pred_buf->as<double>() + pred_off[i];
-      d.pub_out = d.plb_out + round_up(in[i]->n + N, kLdAlign);
+      d.plb_out = in_place[i] ? in[i]->plb : pred_buf->as<double>() + pred_off[i];
+      d.pub_out = in_place[i] ? in[i]->pub : d.plb_out + pred_cap[i];
       d.lbub = lbub_buf->as<double>() + lbub_off[i];
       d.ld_lbub = ldr_max;
       d.write_bounds = 1;
@@ -780,7 +792,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
   // algorithmic bytes of the classification: lb and ub read, the per-row class and the two index lists
   // written (plus, when it also writes the predicate bounds, the copy of the input's)
   double cls_bytes = 0.0;
-  for (int64_t i = 0; i < count; ++i) cls_bytes += 24.0 * (double)N + (fold_bounds && !early_rank ? 32.0 * (double)in[i]->n : 0.0);
+  for (int64_t i = 0; i < count; ++i) cls_bytes += 24.0 * (double)N + (fold_bounds && !early_rank && !in_place[i] ? 32.0 * (double)in[i]->n : 0.0);
   const bool tk = ctx->kernel_timing;
   if (N <= kOneBlockN) {
     if (!sorted)
@@ -1002,7 +1014,21 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->cs.win_from = o->cs.win_to = 0;
       o->cs.rows_reset = true;
     }
-    o->pbuf = pred_buf;
+    if (fold_bounds && in_place[i]) {
+      o->pbuf = in[i]->pbuf;
+      o->ptails = in[i]->ptails;
+      o->pslot = in[i]->pslot;
+      o->pcap = in[i]->pcap;
+      o->ptails->used[(size_t)o->pslot] = o->n;
+    } else {
+      o->pbuf = pred_buf;
+      if (fold_bounds) {
+        o->ptails = tails;
+        o->pslot = i;
+        o->pcap = pred_cap[i];
+        tails->used[(size_t)i] = o->n;
+      }
+    }
     o->plb = d.plb_out;
     o->pub = d.pub_out;
     o->n_inactive = counts[2 * i + 1];

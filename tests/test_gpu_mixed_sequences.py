@@ -435,6 +435,58 @@ def test_a_relu_on_top_of_a_relu_lists_its_rows_anew(nnv, oracle, count, half_wi
         _compare(nnv, oracle, layers, dev_in, ora_in, method)
 
 
+@pytest.mark.parametrize("count", [1, 40])
+def test_relu_steps_that_append_their_predicate_bounds_in_place(nnv, oracle, count):
+    """A ReLU step leaves room behind the predicate bounds it writes, and a later step whose input ends exactly
+    there appends its own in place instead of copying the old ones.  Seven ReLU steps in a row behind FC layers of
+    different widths (the room runs out on the way and a step copies again), every set of every layer against the
+    oracle; then two different steps applied to one and the same set, in both orders, and a third to the set before
+    it: nobody sees what another step appended behind the entries that are his."""
+    rs = np.random.RandomState(2500 + count)
+    n_in = 30
+    widths = [64, 64, 96, 64, 48, 200, 64]
+    layers, prev = [], n_in
+    for wd in widths:
+        layers += [_fc(rs, wd, prev, 2.5), {"type": "relu"}]
+        prev = wd
+    layers.append(_fc(rs, 5, prev))
+    centre = rs.rand(n_in, count)
+    half = np.abs(rs.randn(n_in, count)) * 0.4
+    lbs, ubs = centre - half, centre + half
+    if count == 1:
+        dev_in, ora_in = nnv.Star(lbs[:, 0], ubs[:, 0]), oracle.star_from_box(lbs[:, 0], ubs[:, 0])
+    else:
+        dev_in = nnv.Star.from_boxes(lbs, ubs)
+        ora_in = [oracle.star_from_box(lbs[:, i], ubs[:, i]) for i in range(count)]
+    for method in ("relax-star-area", "relax-star-static"):
+        _compare(nnv, oracle, layers, dev_in, ora_in, method)
+    # one set, several steps
+    L = nnv.NN.from_config(layers, "in place").Layers
+    opts = ("relax-star-area", [], 1, None, "linprog")
+
+    def bounds(sets):
+        sets = sets if isinstance(sets, (list, nnv.SetArray)) else [sets]
+        return [(np.asarray(t.predicate_lb).copy(), np.asarray(t.predicate_ub).copy()) for t in sets]
+
+    s1 = L[1].reach(L[0].reach(dev_in, *opts), *opts)        # the first step's output: room behind its bounds
+    f2 = L[2].reach(s1, *opts)
+    b_s1, b_f2 = bounds(s1), bounds(f2)
+    a = L[3].reach(f2, *opts)                                # appends in place
+    b_a = bounds(a)
+    b = L[3].reach(f2, "relax-star-range", [], 1, None, "linprog")   # the same input again: the room is taken
+    other = L[3].reach(L[2].reach(s1, *opts), *opts)        # ... and for an equal input made afresh from the set before
+    for (l0, u0), (l1, u1) in zip(b_s1, bounds(s1)):
+        assert np.array_equal(l0, l1) and np.array_equal(u0, u1)
+    for (l0, u0), (l1, u1) in zip(b_f2, bounds(f2)):
+        assert np.array_equal(l0, l1) and np.array_equal(u0, u1)
+    for (l0, u0), (l1, u1) in zip(b_a, bounds(a)):
+        assert np.array_equal(l0, l1) and np.array_equal(u0, u1)
+    for (l0, u0), (l1, u1), (l2, u2) in zip(b_a, bounds(b), bounds(other)):
+        # the same crossing neurons in another order: the same multiset of new bounds behind the same old ones
+        assert len(l0) == len(l1) and np.array_equal(np.sort(u0), np.sort(u1))
+        assert np.array_equal(l0, l2) and np.array_equal(u0, u2)      # the same step on an equal input: the same bounds
+
+
 @pytest.mark.parametrize("seed", [318, 456, 620, 690, 717, 720, 800, 843, 855, 892])
 def test_random_fc_sequences_that_once_failed(nnv, oracle, seed):
     """Random FC / ReLU / batch-normalisation sequences over one, two or five boxes of widths from 0.005 to 3, the

@@ -97,6 +97,11 @@ def test_matrices_a_layer_leaves_unwritten_read_the_same_later(route, nnv, oracl
     seqs.test_matrices_a_layer_leaves_unwritten_read_the_same_later(nnv, oracle, then)
 
 
+@pytest.mark.parametrize("count", [1, 40])
+def test_relu_steps_that_append_their_predicate_bounds_in_place(route, nnv, oracle, count):
+    seqs.test_relu_steps_that_append_their_predicate_bounds_in_place(nnv, oracle, count)
+
+
 def test_one_wide_set_through_the_tile_kernel(route, nnv, oracle):
     seqs.test_one_wide_set_through_the_tile_kernel(nnv, oracle, "relax-star-area")
 
