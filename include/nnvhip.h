@@ -144,6 +144,11 @@ NNVHIP_API int nnvhip_pool_stats(nnvhip_ctx* ctx, int64_t* bytes_in_use, int64_t
  * be NULL.  A benchmark reads them around a step that took unusually long. */
 NNVHIP_API int nnvhip_debug_counters(nnvhip_ctx* ctx, int64_t* device_mallocs, int64_t* staging_waits, int64_t* deferred_handles,
                           int64_t* live_handles);
+/* Test hook (no counterpart in the reference): how many sets, since the context was created, went through a ReLU
+ * step that wrote the bounds of its new predicates behind the input's in the arrays the input already had, and how
+ * many through one that copied the input's bounds into arrays of its own (new_pred_lb = [predicate_lb; zeros(m,1)],
+ * nn/funcs/PosLin.m:737-738, either way).  Either pointer may be NULL. */
+NNVHIP_API int nnvhip_debug_relu_bounds(nnvhip_ctx* ctx, int64_t* appended_in_place, int64_t* copied);
 /* Host-to-device traffic of the context since it was created (no counterpart in the reference, whose arrays
  * never leave the host): the number of layers whose weights were uploaded (nnvhip_fc_create /
  * nnvhip_conv2d_create calls that did not find their arrays resident), the bytes of those uploads, and all

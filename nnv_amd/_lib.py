@@ -29,7 +29,7 @@ SYMBOLS = [
     "nnvhip_star_fetch_rows", "nnvhip_relu_apply_lists", "nnvhip_probe_mfma_peak",
     "nnvhip_estimate_ranges_static", "nnvhip_debug_mailbox_pack", "nnvhip_debug_mailbox_unpack",
     "nnvhip_debug_set_relu_call_number", "nnvhip_reach_layers", "nnvhip_relu_reduce_mem",
-    "nnvhip_set_switch", "nnvhip_hint_next_fc", "nnvhip_debug_counters", "nnvhip_weight_cache_stats", "nnvhip_weight_cache_release", "nnvhip_debug_weak_weight_hash",
+    "nnvhip_set_switch", "nnvhip_hint_next_fc", "nnvhip_debug_counters", "nnvhip_debug_relu_bounds", "nnvhip_weight_cache_stats", "nnvhip_weight_cache_release", "nnvhip_debug_weak_weight_hash",
 ]
 
 
@@ -125,6 +125,7 @@ def load():
         "nnvhip_set_switch": [p, C.c_char_p, C.c_int],
         "nnvhip_hint_next_fc": [p, p],
         "nnvhip_debug_counters": [p, pi64, pi64, pi64, pi64],
+        "nnvhip_debug_relu_bounds": [p, pi64, pi64],
         "nnvhip_weight_cache_stats": [p, pi64, pi64, pi64],
         "nnvhip_weight_cache_release": [p, pi64],
         "nnvhip_debug_weak_weight_hash": [C.c_int],
@@ -260,6 +261,12 @@ class Context:
         v = [C.c_int64() for _ in range(4)]
         check(self.lib.nnvhip_debug_counters(self.handle, *[C.byref(x) for x in v]))
         return dict(zip(("device_mallocs", "staging_waits", "deferred_handles", "live_handles"), (x.value for x in v)))
+
+    def relu_bounds_counts(self):
+        """(sets whose ReLU step appended its predicate bounds in place, sets whose step copied the old ones)."""
+        a, b = C.c_int64(), C.c_int64()
+        check(self.lib.nnvhip_debug_relu_bounds(self.handle, C.byref(a), C.byref(b)))
+        return a.value, b.value
 
     def hint_next_fc(self, weights):
         """nnvhip_hint_next_fc: the FC layer (its device weights, or None) that will follow the next ReLU step."""

@@ -486,6 +486,13 @@ int nnvhip_debug_counters(nnvhip_ctx* c, int64_t* device_mallocs, int64_t* stagi
   return NNVHIP_OK;
 }
 
+int nnvhip_debug_relu_bounds(nnvhip_ctx* c, int64_t* appended_in_place, int64_t* copied) {
+  if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
+  if (appended_in_place) *appended_in_place = c->n_bounds_in_place;
+  if (copied) *copied = c->n_bounds_copied;
+  return NNVHIP_OK;
+}
+
 int nnvhip_pool_stats(nnvhip_ctx* c, int64_t* in_use, int64_t* cached) {
   if (!c) NNV_FAIL(NNVHIP_ERR_ARG, "null context");
   c->drain_deferred();

@@ -375,6 +375,7 @@ struct nnvhip_ctx {
   // arrays of sets of one shape always contract over their whole kept-row lists instead of starting from their
   // group's shared product and contracting over the rows in which they differ (environment NNVHIP_NO_ROW_DELTAS)
   bool no_row_deltas = false;
+  int64_t n_bounds_in_place = 0, n_bounds_copied = 0;  // sets through ReLU steps, by where their predicate bounds went
   bool no_sum_shortcuts = false;  // the pass that sums unwritten pieces: every set in full, with both bounds of every predicate
   // debugging aid (environment NNVHIP_POISON_PENDING): columns left unwritten are filled with NaNs
   bool poison_pending = false;

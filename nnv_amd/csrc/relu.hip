@@ -1014,6 +1014,7 @@ int relu_relax(nnvhip_ctx* ctx, int order, int64_t count, nnvhip_star* const* in
       o->cs.win_from = o->cs.win_to = 0;
       o->cs.rows_reset = true;
     }
+    (fold_bounds && in_place[i] ? ctx->n_bounds_in_place : ctx->n_bounds_copied)++;
     if (fold_bounds && in_place[i]) {
       o->pbuf = in[i]->pbuf;
       o->ptails = in[i]->ptails;

@@ -468,13 +468,22 @@ def test_relu_steps_that_append_their_predicate_bounds_in_place(nnv, oracle, cou
         sets = sets if isinstance(sets, (list, nnv.SetArray)) else [sets]
         return [(np.asarray(t.predicate_lb).copy(), np.asarray(t.predicate_ub).copy()) for t in sets]
 
+    ctx = nnv.default_context()
+    lazy = not ctx.switch_is_on("eager_rows", "eager_tail", "dense_affine")  # (a step that writes rows or columns at once sizes its arrays exactly)
+    c0 = ctx.relu_bounds_counts()
     s1 = L[1].reach(L[0].reach(dev_in, *opts), *opts)        # the first step's output: room behind its bounds
     f2 = L[2].reach(s1, *opts)
     b_s1, b_f2 = bounds(s1), bounds(f2)
+    c1 = ctx.relu_bounds_counts()
     a = L[3].reach(f2, *opts)                                # appends in place
+    c2 = ctx.relu_bounds_counts()
     b_a = bounds(a)
     b = L[3].reach(f2, "relax-star-range", [], 1, None, "linprog")   # the same input again: the room is taken
     other = L[3].reach(L[2].reach(s1, *opts), *opts)        # ... and for an equal input made afresh from the set before
+    c3 = ctx.relu_bounds_counts()
+    assert (c1[0] - c0[0], c1[1] - c0[1]) == (0, count)
+    if lazy:
+        assert (c2[0] - c1[0], c2[1] - c1[1]) == (count, 0) and (c3[0] - c2[0], c3[1] - c2[1]) == (0, 2 * count)
     for (l0, u0), (l1, u1) in zip(b_s1, bounds(s1)):
         assert np.array_equal(l0, l1) and np.array_equal(u0, u1)
     for (l0, u0), (l1, u1) in zip(b_f2, bounds(f2)):
